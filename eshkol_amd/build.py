@@ -1,0 +1,82 @@
+"""Build libeshkol_gpu_hip.so for gfx950 with hipcc (cross-compiles without a GPU).
+
+    python -m eshkol_amd.build            # build into eshkol_amd/lib/
+    python -m eshkol_amd.build --force    # rebuild even if up to date
+
+Each source is compiled to an object under eshkol_amd/lib/obj/ and linked into
+one shared library whose exported symbols are the C ABI declared in
+include/eshkol/backend/gpu/gpu_memory.h and gpu_hip_tiers.h.
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+LIBDIR = os.path.join(PKG, "lib")
+OBJDIR = os.path.join(LIBDIR, "obj")
+LIB = os.path.join(LIBDIR, "libeshkol_gpu_hip.so")
+
+SOURCES = [
+    "gpu_memory_hip.cpp",
+    "dgemm_f64.hip",
+    "igemm_i8.hip",
+    "hgemm_16.hip",
+    "ozaki_crt.hip",
+    "ozaki_int8.hip",
+    "elementwise.hip",
+]
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+# -ffp-contract=off: every fused multiply-add the arithmetic relies on is
+# written as fma(); the compiler must not add or remove any.
+# packed-fp32-ops is switched off for all device code in this library.
+COMMON = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+    "-I", os.path.join(ROOT, "include"), "-I", CSRC,
+]
+
+
+def _newer(target, deps):
+    if not os.path.exists(target):
+        return False
+    t = os.path.getmtime(target)
+    return all(os.path.getmtime(d) <= t for d in deps)
+
+
+def _compile(src, force):
+    path = os.path.join(CSRC, src)
+    obj = os.path.join(OBJDIR, os.path.splitext(src)[0] + ".o")
+    headers = [os.path.join(CSRC, h) for h in os.listdir(CSRC) if h.endswith(".h")]
+    headers += [os.path.join(ROOT, "include", "eshkol", "backend", "gpu", h)
+                for h in ("gpu_memory.h", "gpu_hip_tiers.h")]
+    if not force and _newer(obj, [path] + headers):
+        return obj
+    cmd = [HIPCC] + COMMON + ["-x", "hip", "-c", path, "-o", obj]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, res.stdout, res.stderr))
+    return obj
+
+
+def build(force=False, verbose=False):
+    os.makedirs(OBJDIR, exist_ok=True)
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
+        objs = list(pool.map(lambda s: _compile(s, force), SOURCES))
+    if force or not _newer(LIB, objs):
+        cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs + ["-ldl", "-lpthread"]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError("link failed:\n%s\n%s" % (res.stdout, res.stderr))
+    if verbose:
+        print("built", LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    build(force="--force" in sys.argv, verbose=True)

@@ -1,0 +1,205 @@
+/*
+ * Streaming (HBM-bound) kernels shared by the tiers: transpose, per-row
+ * absolute maximum, the elementwise family, the dense-layer epilogue, and the
+ * single-precision GEMM of eshkol_gpu_matmul_f32.
+ */
+#include "hip_common.h"
+#include "kernels.h"
+
+namespace {
+
+/* 64x64 tile through LDS, 256 threads; reads and writes are both 512-byte
+ * contiguous per wave row. (+1 pad: conflict-free column reads.) */
+__global__ __launch_bounds__(256)
+void transpose_f64_kernel(const double* __restrict__ in, double* __restrict__ out,
+                          uint64_t rows, uint64_t cols) {
+    __shared__ double tile[64][65];
+    const uint64_t r0 = (uint64_t)blockIdx.y * 64, c0 = (uint64_t)blockIdx.x * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const uint64_t r = r0 + ty + 4 * i, c = c0 + tx;
+        if (r < rows && c < cols) tile[ty + 4 * i][tx] = in[r * cols + c];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const uint64_t c = c0 + ty + 4 * i, r = r0 + tx;
+        if (r < rows && c < cols) out[c * rows + r] = tile[tx][ty + 4 * i];
+    }
+}
+
+/* One wave per row: lanes stride the row 16 bytes at a time, then a butterfly
+ * max across the wave. A NaN or infinity anywhere in the row makes the result
+ * +inf, which the tiers read as "not representable, use the native GEMM". */
+__device__ __forceinline__ void absmax_step(double v, double* m) {
+    const double a = fabs(v);
+    if (!(a <= 1.7976931348623157e308)) *m = __builtin_inf();
+    else if (a > *m) *m = a;
+}
+
+__global__ __launch_bounds__(256)
+void rowabsmax_f64_kernel(const double* __restrict__ A, uint64_t M, uint64_t K,
+                          double zero_value, double* __restrict__ rmax) {
+    const int lane = threadIdx.x & 63;
+    const uint64_t row = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= M) return;
+    const double* p = A + row * K;
+    double m = 0.0;
+    const bool vec = ((K & 1) == 0) && (((uintptr_t)A & 15) == 0);
+    if (vec) {
+        typedef double d2_t __attribute__((ext_vector_type(2)));
+        const d2_t* p2 = (const d2_t*)p;
+        const uint64_t n2 = K >> 1;
+        for (uint64_t k = lane; k < n2; k += 64) {
+            d2_t v = p2[k];
+            absmax_step(v.x, &m);
+            absmax_step(v.y, &m);
+        }
+    } else {
+        for (uint64_t k = lane; k < K; k += 64) absmax_step(p[k], &m);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        double o = __shfl_xor(m, off, 64);
+        if (o > m) m = o;
+    }
+    if (lane == 0) rmax[row] = (m > 0.0) ? m : zero_value;
+}
+
+__device__ __forceinline__ double apply_op(int op, double a, double b, bool has_b) {
+    switch (op) {
+        case 0:  return a + (has_b ? b : 0.0);
+        case 1:  return a - (has_b ? b : 0.0);
+        case 2:  return a * (has_b ? b : 1.0);
+        case 3:  return a / (has_b ? b : 1.0);
+        case 4:  return -a;
+        case 5:  return fabs(a);
+        case 6:  return exp(a);
+        case 7:  return log(a);
+        case 8:  return sin(a);
+        case 9:  return cos(a);
+        case 10: return tanh(a);
+        case 11: return a > 0.0 ? a : 0.0;
+        case 12: return 1.0 / (1.0 + exp(-a));
+        case 13: return sqrt(a);
+        default: return 1.0 / a;
+    }
+}
+
+__global__ __launch_bounds__(256)
+void elementwise_f64_kernel(const double* __restrict__ a, const double* __restrict__ b,
+                            double* __restrict__ out, uint64_t n, int op) {
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        out[i] = apply_op(op, a[i], b ? b[i] : 0.0, b != nullptr);
+}
+
+__global__ __launch_bounds__(256)
+void bias_act_f64_kernel(double* __restrict__ Y, const double* __restrict__ bias,
+                         uint64_t rows, uint64_t cols, int act) {
+    const uint64_t n = rows * cols;
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+        double v = Y[i];
+        if (bias) v += bias[i % cols];
+        if (act == 1) v = tanh(v);
+        Y[i] = v;
+    }
+}
+
+/* Plain LDS-tiled fp32 GEMM (64x64 tile, 4x4 outputs per thread). This entry
+ * has no caller on the language side; it is kept correct, not tuned. */
+__global__ __launch_bounds__(256)
+void sgemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C,
+                      int M, int N, int K) {
+    __shared__ float As[16][64 + 1];
+    __shared__ float Bs[16][64 + 1];
+    const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < K; k0 += 16) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int idx = threadIdx.x + 256 * r;
+            const int am = idx >> 4, ak = idx & 15;
+            As[ak][am] = (m0 + am < M && k0 + ak < K) ? A[(size_t)(m0 + am) * K + k0 + ak] : 0.0f;
+            const int bk = idx >> 6, bn = idx & 63;
+            Bs[bk][bn] = (k0 + bk < K && n0 + bn < N) ? B[(size_t)(k0 + bk) * N + n0 + bn] : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            float a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) { a[i] = As[k][ty * 4 + i]; b[i] = Bs[k][tx * 4 + i]; }
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int r = m0 + ty * 4 + i, c = n0 + tx * 4 + j;
+            if (r < M && c < N) C[(size_t)r * N + c] = acc[i][j];
+        }
+}
+
+inline unsigned grid_1d(uint64_t n, unsigned block, unsigned cap) {
+    uint64_t g = (n + block - 1) / block;
+    if (g > cap) g = cap;
+    if (g < 1) g = 1;
+    return (unsigned)g;
+}
+
+}  // namespace
+
+extern "C" int hip_transpose_f64(const double* in, double* out, uint64_t rows, uint64_t cols, void* stream) {
+    if (!in || !out || rows == 0 || cols == 0) return -1;
+    const uint64_t gx = (cols + 63) / 64, gy = (rows + 63) / 64;
+    if (gx > 0x7fffffffULL || gy > 65535ULL) return -1;
+    hipLaunchKernelGGL(transpose_f64_kernel, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0,
+                       (hipStream_t)stream, in, out, rows, cols);
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
+extern "C" int hip_rowabsmax_f64(const double* A, uint64_t M, uint64_t K, double zero_value,
+                                 double* rmax, void* stream) {
+    if (!A || !rmax || M == 0 || K == 0) return -1;
+    const uint64_t g = (M + 3) / 4;
+    if (g > 0x7fffffffULL) return -1;
+    hipLaunchKernelGGL(rowabsmax_f64_kernel, dim3((unsigned)g), dim3(256), 0, (hipStream_t)stream,
+                       A, M, K, zero_value, rmax);
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
+extern "C" int hip_elementwise_f64(const double* a, const double* b, double* out, uint64_t n, int op,
+                                   void* stream) {
+    if (!a || !out || n == 0 || op < 0 || op > 14) return -1;
+    hipLaunchKernelGGL(elementwise_f64_kernel, dim3(grid_1d(n, 256, 256 * 32)), dim3(256), 0,
+                       (hipStream_t)stream, a, b, out, n, op);
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
+extern "C" int hip_bias_act_f64(double* Y, const double* bias, uint64_t rows, uint64_t cols, int act,
+                                void* stream) {
+    if (!Y || rows == 0 || cols == 0 || act < 0 || act > 1) return -1;
+    hipLaunchKernelGGL(bias_act_f64_kernel, dim3(grid_1d(rows * cols, 256, 256 * 32)), dim3(256), 0,
+                       (hipStream_t)stream, Y, bias, rows, cols, act);
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
+extern "C" int hip_sgemm_f32(const float* A, const float* B, float* C,
+                             uint64_t M, uint64_t K, uint64_t N, void* stream) {
+    if (!A || !B || !C || M == 0 || K == 0 || N == 0) return -1;
+    if (M > 0x7fffffffULL || K > 0x7fffffffULL || N > 0x7fffffffULL) return -1;
+    const uint64_t gx = (N + 63) / 64, gy = (M + 63) / 64;
+    if (gy > 65535) return -1;
+    hipLaunchKernelGGL(sgemm_f32_kernel, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0,
+                       (hipStream_t)stream, A, B, C, (int)M, (int)N, (int)K);
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}

@@ -1,0 +1,308 @@
+/*
+ * Reduced-precision tier: f16 or bf16 operands, fp32 accumulation on the gfx950
+ * matrix cores (v_mfma_f32_32x32x16_f16 / _bf16). Takes the place of
+ * cuda_matmul_f16_from_f64 (lib/backend/gpu/gpu_memory_cuda.cpp:678-728): there
+ * the f64 -> half conversion and back run on the host around cublasGemmEx; here
+ * they are device kernels and the operands never leave HBM.
+ *
+ * The narrowing is the reference's two-step one: f64 -> f32 (round to nearest
+ * even), then f32 -> 16-bit (round to nearest even), as in reduce_precision
+ * (lib/core/runtime_tensor_dtype.cpp:37-109) and in the CUDA path's
+ * __float2half((float)x). dtype 3 multiplies true bf16 operands; the reference's
+ * CUDA unit sends bf16 tensors through half (gpu_memory_cuda.cpp:1125), which
+ * overflows for |x| > 65504.
+ *
+ * The contraction has the same shape as the int8 one: K-contiguous operands
+ * (B is transposed once in fp64), 64-byte k-blocks double-buffered in LDS with
+ * a 16-byte row pad, 2x2 waves of 4x4 (or 2x2) MFMA tiles, B fragment as the
+ * first MFMA operand so a lane owns 4 consecutive output columns.
+ */
+#include "hip_common.h"
+#include "kernels.h"
+
+#include <cstring>
+
+typedef int v4i_t __attribute__((ext_vector_type(4)));
+typedef float v4f_t __attribute__((ext_vector_type(4)));
+typedef float v16f_t __attribute__((ext_vector_type(16)));
+typedef _Float16 v8h_t __attribute__((ext_vector_type(8)));
+typedef __bf16 v8b_t __attribute__((ext_vector_type(8)));
+typedef double d2_t __attribute__((ext_vector_type(2)));
+
+namespace {
+
+constexpr int BKB = 64;            /* bytes of K per block = 32 elements */
+constexpr int LDS_PITCH = BKB + 16;
+
+/* runtime_tensor_dtype.cpp:97-109, NaN kept quiet instead of truncated */
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+    uint32_t bits = __float_as_uint(f);
+    if (((bits >> 23) & 0xffu) == 0xffu) {
+        uint16_t h = (uint16_t)(bits >> 16);
+        if (bits & 0x7fffffu) h |= 0x0040u;
+        return h;
+    }
+    bits += 0x7fffu + ((bits >> 16) & 1u);
+    return (uint16_t)(bits >> 16);
+}
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
+    _Float16 h = (_Float16)f;                 /* v_cvt_f16_f32: round to nearest even */
+    uint16_t u;
+    __builtin_memcpy(&u, &h, 2);
+    return u;
+}
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t u) {
+    _Float16 h;
+    __builtin_memcpy(&h, &u, 2);
+    return (float)h;
+}
+
+template <bool BF16>
+__global__ __launch_bounds__(256)
+void convert_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
+                    uint16_t* __restrict__ out, uint64_t rows_padded, uint64_t ld) {
+    const uint32_t cpr = (uint32_t)((ld / 2 + 255) / 256);
+    const uint64_t row = blockIdx.x / cpr;
+    const uint64_t k = ((uint64_t)(blockIdx.x % cpr) * 256 + threadIdx.x) * 2;
+    if (k >= ld) return;
+    double x0 = 0.0, x1 = 0.0;
+    if (row < rows) {
+        const double* p = X + row * K + k;
+        if (k + 1 < K) {
+            if ((K & 1) == 0 && (((uintptr_t)X & 15) == 0)) { d2_t v = *(const d2_t*)p; x0 = v.x; x1 = v.y; }
+            else { x0 = p[0]; x1 = p[1]; }
+        } else if (k < K) {
+            x0 = p[0];
+        }
+    }
+    const uint16_t h0 = BF16 ? f32_to_bf16_bits((float)x0) : f32_to_f16_bits((float)x0);
+    const uint16_t h1 = BF16 ? f32_to_bf16_bits((float)x1) : f32_to_f16_bits((float)x1);
+    *(uint32_t*)(out + row * ld + k) = (uint32_t)h0 | ((uint32_t)h1 << 16);
+}
+
+template <int TM, int TN> struct Cfg {
+    static constexpr int NT = 256;
+    static constexpr int BM = 2 * TM * 32;
+    static constexpr int BN = 2 * TN * 32;
+    static constexpr int A_TILE = BM * LDS_PITCH;
+    static constexpr int B_TILE = BN * LDS_PITCH;
+    static constexpr int SMEM_BYTES = 2 * (A_TILE + B_TILE);
+    static constexpr int A_CHUNKS = BM * BKB / 16 / NT;
+    static constexpr int B_CHUNKS = BN * BKB / 16 / NT;
+};
+
+/* out_mode 0: fp32 C; 1: f64 C; 2: f64 C after rounding to the 16-bit type */
+template <bool BF16, int TM, int TN>
+__global__ __launch_bounds__(256)
+void hgemm_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ Bt,
+                  int M, int N, int ld_bytes, int out_mode, void* __restrict__ Cout,
+                  int tiles_m, int tiles_n) {
+    using C = Cfg<TM, TN>;
+    extern __shared__ __align__(16) int8_t smem_h[];
+    int8_t* As = smem_h;
+    int8_t* Bs = smem_h + 2 * C::A_TILE;
+
+    int tm, tn;
+    {
+        const int nwg = gridDim.x, wg = blockIdx.x;
+        const int q = nwg >> 3, r = nwg & 7;
+        const int xcd = wg & 7, seq = wg >> 3;
+        const int L = xcd * q + (xcd < r ? xcd : r) + seq;
+        const int GM = 8;
+        const int width = GM * tiles_n;
+        const int group = L / width;
+        const int first_m = group * GM;
+        const int gsize = (tiles_m - first_m < GM) ? tiles_m - first_m : GM;
+        const int in_group = L - group * width;
+        tm = first_m + in_group % gsize;
+        tn = in_group / gsize;
+    }
+    const int m0 = tm * C::BM, n0 = tn * C::BN;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int li = lane & 31, lh = lane >> 5;
+
+    const int8_t* Ap = (const int8_t*)A + (size_t)m0 * ld_bytes;
+    const int8_t* Bp = (const int8_t*)Bt + (size_t)n0 * ld_bytes;
+    const int nkb = ld_bytes / BKB;
+
+    v4i_t ra[C::A_CHUNKS], rb[C::B_CHUNKS];
+    auto gload = [&](int kb) {
+        const int k0 = kb * BKB;
+#pragma unroll
+        for (int r = 0; r < C::A_CHUNKS; r++) {
+            const int c = tid + C::NT * r;
+            ra[r] = *(const v4i_t*)(Ap + (size_t)(c >> 2) * ld_bytes + k0 + (c & 3) * 16);
+        }
+#pragma unroll
+        for (int r = 0; r < C::B_CHUNKS; r++) {
+            const int c = tid + C::NT * r;
+            rb[r] = *(const v4i_t*)(Bp + (size_t)(c >> 2) * ld_bytes + k0 + (c & 3) * 16);
+        }
+    };
+    auto sstore = [&](int buf) {
+#pragma unroll
+        for (int r = 0; r < C::A_CHUNKS; r++) {
+            const int c = tid + C::NT * r;
+            *(v4i_t*)(As + buf * C::A_TILE + (c >> 2) * LDS_PITCH + (c & 3) * 16) = ra[r];
+        }
+#pragma unroll
+        for (int r = 0; r < C::B_CHUNKS; r++) {
+            const int c = tid + C::NT * r;
+            *(v4i_t*)(Bs + buf * C::B_TILE + (c >> 2) * LDS_PITCH + (c & 3) * 16) = rb[r];
+        }
+    };
+
+    v16f_t acc[TM][TN];
+#pragma unroll
+    for (int t = 0; t < TM; t++)
+#pragma unroll
+        for (int u = 0; u < TN; u++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[t][u][r] = 0.0f;
+
+    gload(0);
+    sstore(0);
+    __syncthreads();
+
+    int cur = 0;
+    for (int kb = 0; kb < nkb; kb++) {
+        const bool more = (kb + 1 < nkb);
+        if (more) gload(kb + 1);
+        const int8_t* a_base = As + cur * C::A_TILE + (wm * TM * 32 + li) * LDS_PITCH + lh * 16;
+        const int8_t* b_base = Bs + cur * C::B_TILE + (wn * TN * 32 + li) * LDS_PITCH + lh * 16;
+#pragma unroll
+        for (int ks = 0; ks < BKB / 32; ks++) {
+            v4i_t a[TM], b[TN];
+#pragma unroll
+            for (int t = 0; t < TM; t++) a[t] = *(const v4i_t*)(a_base + t * 32 * LDS_PITCH + ks * 32);
+#pragma unroll
+            for (int u = 0; u < TN; u++) b[u] = *(const v4i_t*)(b_base + u * 32 * LDS_PITCH + ks * 32);
+#pragma unroll
+            for (int t = 0; t < TM; t++)
+#pragma unroll
+                for (int u = 0; u < TN; u++) {
+                    if (BF16)
+                        acc[t][u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(v8b_t, b[u]), __builtin_bit_cast(v8b_t, a[t]), acc[t][u], 0, 0, 0);
+                    else
+                        acc[t][u] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                            __builtin_bit_cast(v8h_t, b[u]), __builtin_bit_cast(v8h_t, a[t]), acc[t][u], 0, 0, 0);
+                }
+        }
+        if (more) sstore(cur ^ 1);
+        __syncthreads();
+        cur ^= 1;
+    }
+
+    /* lane column is the output row; registers 4v..4v+3 are output columns
+     * 8v + 4*(lane/32) + 0..3 of the 32x32 tile */
+#pragma unroll
+    for (int t = 0; t < TM; t++) {
+        const int row = m0 + wm * TM * 32 + t * 32 + li;
+        if (row >= M) continue;
+#pragma unroll
+        for (int u = 0; u < TN; u++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int col = n0 + wn * TN * 32 + u * 32 + 8 * v + 4 * lh;
+                float f[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    float x = acc[t][u][4 * v + e];
+                    if (out_mode == 2)
+                        x = BF16 ? bf16_bits_to_f32(f32_to_bf16_bits(x)) : f16_bits_to_f32(f32_to_f16_bits(x));
+                    f[e] = x;
+                }
+                if (out_mode == 0) {
+                    float* p = (float*)Cout + (size_t)row * N + col;
+                    if ((N & 3) == 0 && col + 3 < N) *(v4f_t*)p = (v4f_t){f[0], f[1], f[2], f[3]};
+                    else for (int e = 0; e < 4; e++) if (col + e < N) p[e] = f[e];
+                } else {
+                    double* p = (double*)Cout + (size_t)row * N + col;
+                    if ((N & 1) == 0 && col + 3 < N) {
+                        *(d2_t*)p = (d2_t){(double)f[0], (double)f[1]};
+                        *(d2_t*)(p + 2) = (d2_t){(double)f[2], (double)f[3]};
+                    } else {
+                        for (int e = 0; e < 4; e++) if (col + e < N) p[e] = (double)f[e];
+                    }
+                }
+            }
+    }
+}
+
+template <bool BF16, int TM, int TN>
+int launch(const uint16_t* A, const uint16_t* Bt, int M, int N, int ld_bytes, int out_mode, void* C,
+           hipStream_t st) {
+    using Cf = Cfg<TM, TN>;
+    static bool attr_set = false;
+    auto kern = hgemm_kernel<BF16, TM, TN>;
+    if (!attr_set) {
+        if (!ESHKOL_HIP_OK(hipFuncSetAttribute((const void*)kern,
+                hipFuncAttributeMaxDynamicSharedMemorySize, Cf::SMEM_BYTES))) return -1;
+        attr_set = true;
+    }
+    const int tiles_m = (M + Cf::BM - 1) / Cf::BM, tiles_n = (N + Cf::BN - 1) / Cf::BN;
+    const long long nwg = (long long)tiles_m * tiles_n;
+    if (nwg > 0x7fffffffLL) return -1;
+    hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(256), Cf::SMEM_BYTES, st,
+                       A, Bt, M, N, ld_bytes, out_mode, C, tiles_m, tiles_n);
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
+int hgemm_any(const uint16_t* A, const uint16_t* Bt, uint64_t M, uint64_t K, uint64_t N, uint64_t ld,
+              int is_bf16, int out_mode, void* C, hipStream_t st) {
+    if (!A || !Bt || !C || M == 0 || K == 0 || N == 0) return -1;
+    if (M > 0x7fffffffULL || N > 0x7fffffffULL || ld < K || ld % 64 != 0 || ld * 2 > 0x7fffffffULL) return -1;
+    if (((uintptr_t)A & 15) || ((uintptr_t)Bt & 15)) return -1;
+    const int m = (int)M, n = (int)N, ldb = (int)(ld * 2);
+    const long long big = (long long)((M + 255) / 256) * ((N + 255) / 256);
+    if (big >= 256)
+        return is_bf16 ? launch<true, 4, 4>(A, Bt, m, n, ldb, out_mode, C, st)
+                       : launch<false, 4, 4>(A, Bt, m, n, ldb, out_mode, C, st);
+    return is_bf16 ? launch<true, 2, 2>(A, Bt, m, n, ldb, out_mode, C, st)
+                   : launch<false, 2, 2>(A, Bt, m, n, ldb, out_mode, C, st);
+}
+
+}  // namespace
+
+extern "C" int hip_convert_f64_to_16(const double* in, uint16_t* out, uint64_t rows, uint64_t cols,
+                                     uint64_t rows_padded, uint64_t ld, int is_bf16, void* stream) {
+    if (!in || !out || rows == 0 || cols == 0 || rows_padded < rows || ld < cols || (ld & 1)) return -1;
+    const uint64_t nblk = ((ld / 2 + 255) / 256) * rows_padded;
+    if (nblk > 0x7fffffffULL) return -1;
+    if (is_bf16)
+        hipLaunchKernelGGL(convert_kernel<true>, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
+                           in, rows, cols, out, rows_padded, ld);
+    else
+        hipLaunchKernelGGL(convert_kernel<false>, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
+                           in, rows, cols, out, rows_padded, ld);
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
+extern "C" int hip_hgemm_16(const uint16_t* A, const uint16_t* Bt, uint64_t M, uint64_t K, uint64_t N,
+                            uint64_t ld, int is_bf16, float* C, void* stream) {
+    return hgemm_any(A, Bt, M, K, N, ld, is_bf16, 0, C, (hipStream_t)stream);
+}
+
+extern "C" int hip_matmul_reduced_f64(const double* A, const double* B, double* C,
+                                      uint64_t M, uint64_t K, uint64_t N,
+                                      int dtype, int round_output, void* stream) {
+    if (!A || !B || !C || M == 0 || K == 0 || N == 0) return -1;
+    if (dtype != 2 && dtype != 3) return -1;
+    if (M > 0x7fffffffULL || K > 0x3fffffffULL || N > 0x7fffffffULL) return -1;
+    hipStream_t st = (hipStream_t)stream;
+    const int is_bf16 = (dtype == 3);
+    const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ld = round_up_sz(K, 64);
+    double* Bt = (double*)eshkol_hip_workspace(WS_BT, K * N * sizeof(double));
+    uint16_t* A16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_A, Mp * ld * 2);
+    uint16_t* B16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_B, Np * ld * 2);
+    if (!Bt || !A16 || !B16) return -1;
+    if (hip_transpose_f64(B, Bt, K, N, st) != 0) return -1;
+    if (hip_convert_f64_to_16(A, A16, M, K, Mp, ld, is_bf16, st) != 0) return -1;
+    if (hip_convert_f64_to_16(Bt, B16, N, K, Np, ld, is_bf16, st) != 0) return -1;
+    return hgemm_any(A16, B16, M, K, N, ld, is_bf16, round_output ? 2 : 1, C, st);
+}

@@ -1,0 +1,46 @@
+/*
+ * Internal declarations shared by the translation units of libeshkol_gpu_hip.so.
+ * Nothing here is part of the public ABI.
+ */
+#ifndef ESHKOL_HIP_COMMON_H
+#define ESHKOL_HIP_COMMON_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+#include <stdio.h>
+
+#define ESHKOL_HIP_OK(call) ((call) == hipSuccess)
+
+/* Log to stderr with the reference's "[GPU] " prefix when ESHKOL_GPU_VERBOSE is
+ * set (reference gpu_memory_cuda.cpp:25-38). */
+int eshkol_hip_verbose(void);
+#define GPU_LOG(fmt, ...) \
+    do { if (eshkol_hip_verbose()) fprintf(stderr, "[GPU] " fmt "\n", ##__VA_ARGS__); } while (0)
+
+/* The one stream every kernel of the library is launched on. */
+hipStream_t eshkol_hip_stream(void);
+
+/* Grow-only device workspace slots, kept for the life of the process so a
+ * matmul does not pay hipMalloc/hipFree per call. Returns NULL on failure. */
+enum {
+    WS_BT = 0,      /* transposed fp64 copy of B                          */
+    WS_APLANES,     /* int8 planes of A                                   */
+    WS_BPLANES,     /* int8 planes of B (transposed, K contiguous)        */
+    WS_PRODUCTS,    /* int8 residue products / int32 diagonal buffers     */
+    WS_ROWSCALE,    /* per-row fp64 scale or max, then int shifts         */
+    WS_COLSCALE,    /* per-column fp64 scale or max, then int shifts      */
+    WS_ROWSHIFT,
+    WS_COLSHIFT,
+    WS_HALF_A,      /* 16-bit copies of A, B and fp32 C for the reduced tier */
+    WS_HALF_B,
+    WS_F32_C,
+    WS_MISC,
+    WS_COUNT
+};
+void* eshkol_hip_workspace(int slot, size_t bytes);
+void  eshkol_hip_workspace_release(void);
+
+static inline size_t round_up_sz(size_t v, size_t m) { return (v + m - 1) / m * m; }
+
+#endif

@@ -1,0 +1,423 @@
+/*
+ * Ozaki-II CRT exact tier: C = A*B in fp64 recovered from int8 matrix-core
+ * products modulo up to 16 pairwise-coprime moduli. Follows ozaki_ii_dispatch
+ * of the reference (lib/backend/gpu/gpu_memory.mm:2474-2665), whose scaling,
+ * residue and reconstruction steps run on the CPU; here every O(MK+KN+MN) pass
+ * is a device kernel and only the O(M+N) scalar bookkeeping (log2 of the row
+ * and column maxima, the exponent E, the shifts) stays on the host, where it
+ * uses the same libm as the reference's host code.
+ *
+ * Pipeline (all on the library stream):
+ *   Bt = B^T                                  (fp64 transpose, so both operands
+ *                                              are split along contiguous K)
+ *   amax[i], bmax[j]                          one wave per row
+ *   -> host: frac bounds, E, mu[i], nu[j]     gpu_memory.mm:376-420, 2510-2532
+ *   A planes, B planes                        trunc(x*2^shift) mod p_l as int8
+ *   W_l = (A_l * B_l^T) mod p_l               int8 MFMA, int32 accumulate
+ *   C = CRT(W) * 2^-mu * 2^-nu                gpu_memory.mm:2626-2655, verbatim
+ *
+ * Residues are taken with exact integer arithmetic on the bit pattern of the
+ * input (the reference's float formula x - p*rint(x/p) loses exactness at the
+ * top of the range); the representative lies in [-p/2, p/2), so 128 mod 256 is
+ * stored as -128. Both choices are invisible modulo p.
+ */
+#include "hip_common.h"
+#include "kernels.h"
+
+#include <cmath>
+#include <cstring>
+#include <mutex>
+
+typedef double d2_t __attribute__((ext_vector_type(2)));
+
+namespace {
+
+/* gpu_memory.mm:227-233 (first 16 of 49; 16 is the most whose product fits
+ * a signed 128-bit integer, gpu_memory.mm:246-255) */
+#define OZAKI_MODULI_16 256, 255, 253, 251, 247, 241, 239, 233, 229, 227, 223, 217, 211, 199, 197, 193
+constexpr int MAX_MODULI = 16;
+const int H_MODULI[MAX_MODULI] = { OZAKI_MODULI_16 };
+
+struct ModuliTable { int p[MAX_MODULI]; int c18[MAX_MODULI]; int c36[MAX_MODULI]; };
+constexpr ModuliTable make_table() {
+    ModuliTable t{};
+    const int m[MAX_MODULI] = { OZAKI_MODULI_16 };
+    for (int l = 0; l < MAX_MODULI; l++) {
+        t.p[l] = m[l];
+        t.c18[l] = (int)((1ull << 18) % (unsigned)m[l]);
+        t.c36[l] = (int)((1ull << 36) % (unsigned)m[l]);
+    }
+    return t;
+}
+constexpr ModuliTable TBL = make_table();
+
+/* |trunc(x * 2^sh)| as an integer (< 2^53 by construction of sh) and its sign,
+ * read straight off the bit pattern: the right shift is the truncation. */
+__device__ __forceinline__ uint64_t scaled_magnitude(double x, int sh, bool* neg) {
+    const uint64_t bits = __double_as_longlong(x);
+    *neg = (bits >> 63) != 0;
+    const int e = (int)((bits >> 52) & 0x7ff);
+    uint64_t mant = bits & 0xfffffffffffffull;
+    int e_eff = 1;
+    if (e != 0) { mant |= 1ull << 52; e_eff = e; }
+    const int rs = 1075 - e_eff - sh;          /* value = mant * 2^-rs */
+    if (rs >= 64) return 0;
+    if (rs <= 0) return mant;                  /* excluded by the host's range check */
+    return mant >> rs;
+}
+
+template <int L>
+__device__ __forceinline__ int residue(uint64_t t, bool neg) {
+    constexpr int p = TBL.p[L];
+    const uint32_t lo = (uint32_t)(t & 0x3ffff);
+    const uint32_t mid = (uint32_t)((t >> 18) & 0x3ffff);
+    const uint32_t hi = (uint32_t)(t >> 36);
+    uint32_t r = (hi * (uint32_t)TBL.c36[L] + mid * (uint32_t)TBL.c18[L] + lo) % (uint32_t)p;
+    int s = (int)r;
+    if (neg && s != 0) s = p - s;
+    if (2 * s >= p) s -= p;
+    return s;
+}
+
+/* One thread: two consecutive k of one row -> one 16-bit store per plane. */
+template <int NMOD>
+__global__ __launch_bounds__(256)
+void crt_split_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
+                      const int32_t* __restrict__ shift, int8_t* __restrict__ planes,
+                      uint64_t rows_padded, uint64_t ldk) {
+    const uint32_t cpr = (uint32_t)((ldk / 2 + 255) / 256);      /* blocks per row */
+    const uint64_t row = blockIdx.x / cpr;
+    const uint64_t k = ((uint64_t)(blockIdx.x % cpr) * 256 + threadIdx.x) * 2;
+    if (k >= ldk) return;
+    double x0 = 0.0, x1 = 0.0;
+    int sh = 0;
+    if (row < rows) {
+        sh = shift[row];
+        const double* p = X + row * K + k;
+        if (k + 1 < K) {
+            if ((K & 1) == 0 && (((uintptr_t)X & 15) == 0)) { d2_t v = *(const d2_t*)p; x0 = v.x; x1 = v.y; }
+            else { x0 = p[0]; x1 = p[1]; }
+        } else if (k < K) {
+            x0 = p[0];
+        }
+    }
+    bool n0, n1;
+    const uint64_t t0 = scaled_magnitude(x0, sh, &n0);
+    const uint64_t t1 = scaled_magnitude(x1, sh, &n1);
+    const uint64_t plane_stride = rows_padded * ldk;
+    int8_t* out = planes + row * ldk + k;
+#define ESHKOL_SPLIT_ONE(L)                                                           \
+    if (L < NMOD) {                                                                   \
+        const int r0 = residue<L>(t0, n0), r1 = residue<L>(t1, n1);                   \
+        *(uint16_t*)(out + (uint64_t)L * plane_stride) =                              \
+            (uint16_t)((uint8_t)(int8_t)r0 | ((uint16_t)(uint8_t)(int8_t)r1 << 8));   \
+    }
+    ESHKOL_SPLIT_ONE(0)  ESHKOL_SPLIT_ONE(1)  ESHKOL_SPLIT_ONE(2)  ESHKOL_SPLIT_ONE(3)
+    ESHKOL_SPLIT_ONE(4)  ESHKOL_SPLIT_ONE(5)  ESHKOL_SPLIT_ONE(6)  ESHKOL_SPLIT_ONE(7)
+    ESHKOL_SPLIT_ONE(8)  ESHKOL_SPLIT_ONE(9)  ESHKOL_SPLIT_ONE(10) ESHKOL_SPLIT_ONE(11)
+    ESHKOL_SPLIT_ONE(12) ESHKOL_SPLIT_ONE(13) ESHKOL_SPLIT_ONE(14) ESHKOL_SPLIT_ONE(15)
+#undef ESHKOL_SPLIT_ONE
+}
+
+struct CrtConsts {
+    double sl1[MAX_MODULI], sl2[MAX_MODULI];
+    double P1, P2, Pinv;
+    int n;
+};
+
+/* One thread: four consecutive columns of one row. The arithmetic is the
+ * reference's, operation for operation: S1 = fma(sl1_l, w, S1), S2 likewise,
+ * l ascending; s = S1 + S2; Q = round(s*Pinv); c' = fma(-P1,Q,S1) + fma(-P2,Q,S2);
+ * C = (c' * 2^-mu) * 2^-nu. */
+__global__ __launch_bounds__(256)
+void crt_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t N, CrtConsts cc,
+                            const int32_t* __restrict__ mu, const int32_t* __restrict__ nu,
+                            const double* __restrict__ bias, int act, double* __restrict__ C) {
+    const uint32_t cpr = (uint32_t)(((N + 3) / 4 + 255) / 256);   /* blocks per row */
+    const uint64_t row = blockIdx.x / cpr;
+    const uint64_t col = ((uint64_t)(blockIdx.x % cpr) * 256 + threadIdx.x) * 4;
+    if (col >= N) return;
+    const uint64_t tot = M * N, idx = row * N + col;
+    const int nvalid = (N - col < 4) ? (int)(N - col) : 4;
+    const bool vec = (nvalid == 4) && ((N & 3) == 0) && (((uintptr_t)W & 3) == 0);
+    double S1[4] = {0, 0, 0, 0}, S2[4] = {0, 0, 0, 0};
+    for (int l = 0; l < cc.n; l++) {
+        const int8_t* w = W + (uint64_t)l * tot + idx;
+        int8_t v[4] = {0, 0, 0, 0};
+        if (vec) {
+            const uint32_t u = *(const uint32_t*)w;
+            v[0] = (int8_t)(u & 0xff); v[1] = (int8_t)((u >> 8) & 0xff);
+            v[2] = (int8_t)((u >> 16) & 0xff); v[3] = (int8_t)(u >> 24);
+        } else {
+            for (int e = 0; e < nvalid; e++) v[e] = w[e];
+        }
+        const double a = cc.sl1[l], b = cc.sl2[l];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const double wd = (double)v[e];
+            S1[e] = fma(a, wd, S1[e]);
+            S2[e] = fma(b, wd, S2[e]);
+        }
+    }
+    const double mu_inv = ldexp(1.0, -mu[row]);
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        if (e >= nvalid) break;
+        const double s = S1[e] + S2[e];
+        const double Q = round(s * cc.Pinv);
+        const double h1 = fma(-cc.P1, Q, S1[e]);
+        const double h2 = fma(-cc.P2, Q, S2[e]);
+        const double cp = h1 + h2;
+        double v = (cp * mu_inv) * ldexp(1.0, -nu[col + e]);
+        if (bias) v = v + bias[col + e];
+        if (act == 1) v = tanh(v);
+        C[idx + e] = v;
+    }
+}
+
+/* ---- host bookkeeping ------------------------------------------------------ */
+
+struct HostCrt { double P1, P2, Pinv, log2P; double sl1[MAX_MODULI], sl2[MAX_MODULI]; int q[MAX_MODULI]; bool ready; };
+HostCrt g_crt[MAX_MODULI + 1];
+std::mutex g_crt_mutex;
+
+int64_t ext_gcd(int64_t a, int64_t b, int64_t* x, int64_t* y) {
+    if (a == 0) { *x = 0; *y = 1; return b; }
+    int64_t x1, y1;
+    int64_t g = ext_gcd(b % a, a, &x1, &y1);
+    *x = y1 - (b / a) * x1;
+    *y = x1;
+    return g;
+}
+int mod_inverse(int64_t a, int64_t m) {
+    int64_t x, y;
+    ext_gcd(a % m, m, &x, &y);
+    return (int)((x % m + m) % m);
+}
+
+/* precompute_ozaki_constants, gpu_memory.mm:301-341. The volatile temporaries
+ * keep the Dekker split free of fused contraction. */
+const HostCrt& crt_constants(int n) {
+    std::lock_guard<std::mutex> lk(g_crt_mutex);
+    HostCrt& c = g_crt[n];
+    if (c.ready) return c;
+    __int128 P = 1;
+    for (int l = 0; l < n; l++) P *= H_MODULI[l];
+    c.P1 = (double)P;
+    c.P2 = (double)(P - (__int128)c.P1);
+    c.Pinv = 1.0 / (double)P;
+    c.log2P = log2((double)P);
+    for (int l = 0; l < n; l++) {
+        const int p = H_MODULI[l];
+        const __int128 Pp = P / p;
+        c.q[l] = mod_inverse((int64_t)(Pp % p), p);
+        const __int128 s = Pp * (__int128)c.q[l];
+        const int bits_to_remove = 8 + (int)ceil(log2((double)n));
+        const double s_d = (double)s;
+        const double factor = (double)(1LL << (bits_to_remove + 1)) + 1.0;
+        volatile double t = factor * s_d;
+        volatile double hi = t - s_d;
+        c.sl1[l] = t - hi;
+        c.sl2[l] = (double)(s - (__int128)c.sl1[l]);
+    }
+    c.ready = true;
+    return c;
+}
+
+double g_log2_cumul[MAX_MODULI + 1];
+std::once_flag g_cumul_once;
+
+/* pinned host staging for the maxima and shifts */
+void* g_pinned = nullptr;
+size_t g_pinned_bytes = 0;
+void* pinned(size_t bytes) {
+    if (g_pinned_bytes >= bytes) return g_pinned;
+    if (g_pinned) hipHostFree(g_pinned);
+    g_pinned = nullptr; g_pinned_bytes = 0;
+    if (!ESHKOL_HIP_OK(hipHostMalloc(&g_pinned, bytes, hipHostMallocDefault))) return nullptr;
+    g_pinned_bytes = bytes;
+    return g_pinned;
+}
+
+/* device-resident constant tables for the contraction: identity pair lists and moduli */
+int32_t* g_tables = nullptr;   /* [0..16] pair_first, [17..32] pair index, [33..48] moduli */
+int ensure_tables(hipStream_t st) {
+    if (g_tables) return 0;
+    int32_t h[17 + 16 + 16];
+    for (int i = 0; i <= 16; i++) h[i] = i;
+    for (int i = 0; i < 16; i++) { h[17 + i] = i; h[33 + i] = H_MODULI[i]; }
+    if (!ESHKOL_HIP_OK(hipMalloc((void**)&g_tables, sizeof h))) { g_tables = nullptr; return -1; }
+    if (!ESHKOL_HIP_OK(hipMemcpyAsync(g_tables, h, sizeof h, hipMemcpyHostToDevice, st)) ||
+        !ESHKOL_HIP_OK(hipStreamSynchronize(st))) { hipFree(g_tables); g_tables = nullptr; return -1; }
+    return 0;
+}
+
+HipOzakiCrtStages g_last = {};
+
+template <int NMOD>
+void launch_split(const double* X, uint64_t rows, uint64_t K, const int32_t* shift, int8_t* planes,
+                  uint64_t rows_padded, uint64_t ldk, hipStream_t st) {
+    dim3 grid((unsigned)(((ldk / 2 + 255) / 256) * rows_padded));
+    hipLaunchKernelGGL(crt_split_kernel<NMOD>, grid, dim3(256), 0, st, X, rows, K, shift, planes,
+                       rows_padded, ldk);
+}
+
+}  // namespace
+
+extern "C" int hip_ozaki_crt_split_f64(const double* X, uint64_t rows, uint64_t K,
+                                       const int32_t* shift, int num_moduli,
+                                       int8_t* planes, uint64_t rows_padded, uint64_t ldk, void* stream) {
+    if (!X || !shift || !planes || rows == 0 || K == 0) return -1;
+    if (num_moduli < 2 || num_moduli > MAX_MODULI) return -1;
+    if (rows_padded < rows || ldk < K || (ldk & 1)) return -1;
+    if (((ldk / 2 + 255) / 256) * rows_padded > 0x7fffffffULL) return -1;
+    hipStream_t st = (hipStream_t)stream;
+    switch (num_moduli) {
+#define CASE(n) case n: launch_split<n>(X, rows, K, shift, planes, rows_padded, ldk, st); break;
+        CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8) CASE(9)
+        CASE(10) CASE(11) CASE(12) CASE(13) CASE(14) CASE(15) CASE(16)
+#undef CASE
+    }
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
+extern "C" int hip_ozaki_crt_reconstruct_f64(const int8_t* w_planes, uint64_t M, uint64_t N, int num_moduli,
+                                             const double* sl1, const double* sl2,
+                                             double P1, double P2, double Pinv,
+                                             const int32_t* mu, const int32_t* nu,
+                                             const double* bias, int act,
+                                             double* C, void* stream) {
+    if (!w_planes || !sl1 || !sl2 || !mu || !nu || !C || M == 0 || N == 0) return -1;
+    if (num_moduli < 2 || num_moduli > MAX_MODULI || act < 0 || act > 1) return -1;
+    if ((((N + 3) / 4 + 255) / 256) * M > 0x7fffffffULL) return -1;
+    CrtConsts cc;
+    memset(&cc, 0, sizeof cc);
+    for (int l = 0; l < num_moduli; l++) { cc.sl1[l] = sl1[l]; cc.sl2[l] = sl2[l]; }
+    cc.P1 = P1; cc.P2 = P2; cc.Pinv = Pinv; cc.n = num_moduli;
+    dim3 grid((unsigned)((((N + 3) / 4 + 255) / 256) * M));
+    hipLaunchKernelGGL(crt_reconstruct_kernel, grid, dim3(256), 0, (hipStream_t)stream,
+                       w_planes, M, N, cc, mu, nu, bias, act, C);
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
+extern "C" int hip_ozaki_crt_last_stages(HipOzakiCrtStages* out) {
+    if (!out || !g_last.a_planes) return -1;
+    *out = g_last;
+    return 0;
+}
+
+extern "C" int hip_matmul_ozaki_crt_f64(const double* A, const double* B, double* C,
+                                        uint64_t M, uint64_t K, uint64_t N,
+                                        int num_moduli, int adaptive,
+                                        const double* bias, int act, void* stream) {
+    if (!A || !B || !C || M == 0 || K == 0 || N == 0) return -1;
+    if (M > 0x7fffffffULL || N > 0x7fffffffULL) return -1;
+    /* int32 accumulation of |a*b| <= 128*128 is exact while K*16384 < 2^31 */
+    if (K > 131071) {
+        static bool warned = false;
+        if (!warned) {
+            warned = true;
+            fprintf(stderr, "[GPU] Ozaki-II: K=%llu exceeds the int32-exact bound 131071; "
+                            "falling back to the native fp64 GEMM\n", (unsigned long long)K);
+        }
+        return -1;
+    }
+    if (num_moduli < 2) num_moduli = 2;
+    if (num_moduli > MAX_MODULI) {
+        fprintf(stderr, "[GPU] Ozaki-II: requested N=%d exceeds max %d (would overflow "
+                        "__int128 P); clamping to %d\n", num_moduli, MAX_MODULI, MAX_MODULI);
+        num_moduli = MAX_MODULI;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    if (ensure_tables(st) != 0) return -1;
+
+    const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ldk = round_up_sz(K, 128);
+    double* Bt   = (double*)eshkol_hip_workspace(WS_BT, K * N * sizeof(double));
+    double* amax = (double*)eshkol_hip_workspace(WS_ROWSCALE, M * sizeof(double));
+    double* bmax = (double*)eshkol_hip_workspace(WS_COLSCALE, N * sizeof(double));
+    int32_t* dmu = (int32_t*)eshkol_hip_workspace(WS_ROWSHIFT, M * sizeof(int32_t));
+    int32_t* dnu = (int32_t*)eshkol_hip_workspace(WS_COLSHIFT, N * sizeof(int32_t));
+    if (!Bt || !amax || !bmax || !dmu || !dnu) return -1;
+    char* host = (char*)pinned((M + N) * (sizeof(double) + sizeof(int32_t)));
+    if (!host) return -1;
+    double* h_amax = (double*)host;
+    double* h_bmax = h_amax + M;
+    int32_t* h_mu = (int32_t*)(h_bmax + N);
+    int32_t* h_nu = h_mu + M;
+
+    if (hip_transpose_f64(B, Bt, K, N, st) != 0) return -1;
+    if (hip_rowabsmax_f64(A, M, K, 0.0, amax, st) != 0) return -1;
+    if (hip_rowabsmax_f64(Bt, N, K, 0.0, bmax, st) != 0) return -1;
+    if (!ESHKOL_HIP_OK(hipMemcpyAsync(h_amax, amax, M * sizeof(double), hipMemcpyDeviceToHost, st))) return -1;
+    if (!ESHKOL_HIP_OK(hipMemcpyAsync(h_bmax, bmax, N * sizeof(double), hipMemcpyDeviceToHost, st))) return -1;
+    if (!ESHKOL_HIP_OK(hipStreamSynchronize(st))) return -1;
+
+    /* frac bounds (gpu_memory.mm:403-417); a non-finite maximum marks NaN/Inf input */
+    double frac_A = 0.0, frac_B = 0.0;
+    for (uint64_t i = 0; i < M; i++) {
+        const double m = h_amax[i];
+        if (!std::isfinite(m)) return -1;
+        if (m > 0.0) { double lg = log2(m); double f = lg - floor(lg); if (f > frac_A) frac_A = f; }
+    }
+    for (uint64_t j = 0; j < N; j++) {
+        const double m = h_bmax[j];
+        if (!std::isfinite(m)) return -1;
+        if (m > 0.0) { double lg = log2(m); double f = lg - floor(lg); if (f > frac_B) frac_B = f; }
+    }
+    const double log2K = log2((double)K);
+    if (adaptive) {                                   /* gpu_memory.mm:433-453 */
+        std::call_once(g_cumul_once, [] {
+            g_log2_cumul[0] = 0.0;
+            for (int i = 0; i < MAX_MODULI; i++) g_log2_cumul[i + 1] = g_log2_cumul[i] + log2((double)H_MODULI[i]);
+        });
+        int chosen = num_moduli;
+        for (int n = 2; n <= num_moduli; n++) {
+            double emax = floor((g_log2_cumul[n] - 1.0 - log2K - frac_A - frac_B) / 2.0);
+            if (emax >= 52.0) { chosen = n; break; }
+        }
+        num_moduli = chosen;
+    }
+    const HostCrt& crt = crt_constants(num_moduli);
+    fprintf(stderr, "[GPU] Ozaki-II: N=%d%s, log2(P)=%.1f\n", num_moduli,
+            adaptive ? " (adaptive)" : "", crt.log2P);       /* gpu_memory.mm:2503 */
+
+    int E = (int)floor((crt.log2P - 1.0 - log2K - frac_A - frac_B) / 2.0);   /* gpu_memory.mm:2510-2512 */
+    if (E > 52) E = 52;
+    if (E < 0) E = 0;
+    for (uint64_t i = 0; i < M; i++) {
+        h_mu[i] = (h_amax[i] == 0.0) ? 0 : E - (int)floor(log2(h_amax[i]));
+        if (h_mu[i] > 1023 || h_mu[i] < -1022) return -1;
+    }
+    for (uint64_t j = 0; j < N; j++) {
+        h_nu[j] = (h_bmax[j] == 0.0) ? 0 : E - (int)floor(log2(h_bmax[j]));
+        if (h_nu[j] > 1023 || h_nu[j] < -1022) return -1;
+    }
+    if (!ESHKOL_HIP_OK(hipMemcpyAsync(dmu, h_mu, M * sizeof(int32_t), hipMemcpyHostToDevice, st))) return -1;
+    if (!ESHKOL_HIP_OK(hipMemcpyAsync(dnu, h_nu, N * sizeof(int32_t), hipMemcpyHostToDevice, st))) return -1;
+
+    int8_t* Ap = (int8_t*)eshkol_hip_workspace(WS_APLANES, (size_t)num_moduli * Mp * ldk);
+    int8_t* Bp = (int8_t*)eshkol_hip_workspace(WS_BPLANES, (size_t)num_moduli * Np * ldk);
+    int8_t* Wp = (int8_t*)eshkol_hip_workspace(WS_PRODUCTS, (size_t)num_moduli * M * N);
+    if (!Ap || !Bp || !Wp) return -1;
+
+    if (hip_ozaki_crt_split_f64(A, M, K, dmu, num_moduli, Ap, Mp, ldk, st) != 0) return -1;
+    if (hip_ozaki_crt_split_f64(Bt, N, K, dnu, num_moduli, Bp, Np, ldk, st) != 0) return -1;
+
+    HipIgemmArgs ga;
+    memset(&ga, 0, sizeof ga);
+    ga.a_planes = Ap; ga.b_planes = Bp;
+    ga.a_plane_stride = Mp * ldk; ga.b_plane_stride = Np * ldk;
+    ga.ldk = (uint32_t)ldk; ga.M = (uint32_t)M; ga.N = (uint32_t)N; ga.n_out = (uint32_t)num_moduli;
+    ga.pair_first = g_tables; ga.pair_a = g_tables + 17; ga.pair_b = g_tables + 17;
+    ga.mode = 1; ga.modulus = g_tables + 33; ga.out_i8 = Wp;
+    if (hip_igemm_i8(&ga, st) != 0) return -1;
+
+    if (hip_ozaki_crt_reconstruct_f64(Wp, M, N, num_moduli, crt.sl1, crt.sl2, crt.P1, crt.P2, crt.Pinv,
+                                      dmu, dnu, bias, act, C, st) != 0) return -1;
+
+    g_last.a_planes = Ap; g_last.b_planes = Bp; g_last.w_planes = Wp;
+    g_last.mu = dmu; g_last.nu = dnu;
+    g_last.rows_a_padded = Mp; g_last.rows_b_padded = Np; g_last.ldk = ldk;
+    g_last.num_moduli = num_moduli; g_last.E = E;
+    return 0;
+}

@@ -1,0 +1,218 @@
+/*
+ * INT8 slice tier (Ootomo-Ozaki-Yokota base-128 slicing): C = A*B in fp64 from
+ * int8 matrix-core products of per-row / per-column scaled slices. Follows
+ * cuda_matmul_ozaki_int8_f64 (lib/backend/gpu/gpu_memory_cuda.cpp:339-452) and
+ * its kernels (lib/backend/gpu/gpu_cuda_kernels.cu:663-741):
+ *
+ *   r_i = max_k |A[i,k]| (0 -> 1), c_j = max_k |B[k,j]| (0 -> 1)
+ *   res = x / scale; s times: res *= 128; a = rint(res); clamp +-127; store; res -= a
+ *   G_b = sum over the buffer's (p,q) pairs of A_p * B_q          exact int32
+ *   C[i,j] = ((sum_b w_b * G_b[i,j]) * r_i) * c_j, b ascending, w_b = 2^(-7(d+2))
+ *
+ * Differences from the reference's execution, none of them arithmetic: B is
+ * transposed once in fp64 so both operands are sliced along contiguous K by the
+ * same kernel (the reference's B kernel scatters transposed bytes); the row
+ * maximum is a wave-wide reduction; all pairs of a buffer are summed inside one
+ * matrix-core launch instead of beta=1 accumulation across cuBLAS calls.
+ */
+#include "hip_common.h"
+#include "kernels.h"
+
+#include <cmath>
+#include <cstring>
+
+typedef double d2_t __attribute__((ext_vector_type(2)));
+
+namespace {
+
+/* gpu_cuda_kernels.cu:694-701 for two consecutive k of one row. */
+__global__ __launch_bounds__(256)
+void slice_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
+                  const double* __restrict__ scale, int s, int8_t* __restrict__ planes,
+                  uint64_t rows_padded, uint64_t ldk) {
+    const uint32_t cpr = (uint32_t)((ldk / 2 + 255) / 256);
+    const uint64_t row = blockIdx.x / cpr;
+    const uint64_t k = ((uint64_t)(blockIdx.x % cpr) * 256 + threadIdx.x) * 2;
+    if (k >= ldk) return;
+    double x0 = 0.0, x1 = 0.0, sc = 1.0;
+    if (row < rows) {
+        sc = scale[row];
+        const double* p = X + row * K + k;
+        if (k + 1 < K) {
+            if ((K & 1) == 0 && (((uintptr_t)X & 15) == 0)) { d2_t v = *(const d2_t*)p; x0 = v.x; x1 = v.y; }
+            else { x0 = p[0]; x1 = p[1]; }
+        } else if (k < K) {
+            x0 = p[0];
+        }
+    }
+    double r0 = x0 / sc, r1 = x1 / sc;
+    const uint64_t plane_stride = rows_padded * ldk;
+    int8_t* out = planes + row * ldk + k;
+    for (int p = 0; p < s; p++) {
+        r0 *= 128.0; r1 *= 128.0;
+        double a0 = rint(r0), a1 = rint(r1);
+        if (a0 > 127.0) a0 = 127.0; else if (a0 < -127.0) a0 = -127.0;
+        if (a1 > 127.0) a1 = 127.0; else if (a1 < -127.0) a1 = -127.0;
+        const int i0 = (int)a0, i1 = (int)a1;
+        *(uint16_t*)(out + (uint64_t)p * plane_stride) =
+            (uint16_t)((uint8_t)(int8_t)i0 | ((uint16_t)(uint8_t)(int8_t)i1 << 8));
+        r0 -= a0; r1 -= a1;
+    }
+}
+
+/* gpu_cuda_kernels.cu:728-741, two columns per thread. */
+__global__ __launch_bounds__(256)
+void reconstruct_kernel(double* __restrict__ C, const int32_t* __restrict__ Gall,
+                        const double* __restrict__ weights, int nbuf,
+                        const double* __restrict__ rmax, const double* __restrict__ cmax,
+                        uint64_t M, uint64_t N) {
+    const uint32_t cpr = (uint32_t)(((N + 1) / 2 + 255) / 256);
+    const uint64_t row = blockIdx.x / cpr;
+    const uint64_t col = ((uint64_t)(blockIdx.x % cpr) * 256 + threadIdx.x) * 2;
+    if (col >= N) return;
+    const uint64_t tot = M * N, idx = row * N + col;
+    const bool two = (col + 1 < N);
+    const bool vec = two && ((N & 1) == 0);
+    double acc0 = 0.0, acc1 = 0.0;
+    for (int b = 0; b < nbuf; b++) {
+        const int32_t* g = Gall + (uint64_t)b * tot + idx;
+        int32_t g0, g1 = 0;
+        if (vec) { const int2 v = *(const int2*)g; g0 = v.x; g1 = v.y; }
+        else { g0 = g[0]; if (two) g1 = g[1]; }
+        const double w = weights[b];
+        acc0 = acc0 + w * (double)g0;
+        acc1 = acc1 + w * (double)g1;
+    }
+    const double r = rmax[row];
+    C[idx] = (acc0 * r) * cmax[col];
+    if (two) C[idx + 1] = (acc1 * r) * cmax[col + 1];
+}
+
+void* g_pinned = nullptr;
+size_t g_pinned_bytes = 0;
+void* pinned(size_t bytes) {
+    if (g_pinned_bytes >= bytes) return g_pinned;
+    if (g_pinned) hipHostFree(g_pinned);
+    g_pinned = nullptr; g_pinned_bytes = 0;
+    if (!ESHKOL_HIP_OK(hipHostMalloc(&g_pinned, bytes, hipHostMallocDefault))) return nullptr;
+    g_pinned_bytes = bytes;
+    return g_pinned;
+}
+
+HipOzakiInt8Stages g_last = {};
+
+constexpr int MAX_BUF = 128, MAX_PAIRS = 128;
+
+}  // namespace
+
+extern "C" int hip_ozaki_slice_f64(const double* X, uint64_t rows, uint64_t K, const double* scale, int s,
+                                   int8_t* planes, uint64_t rows_padded, uint64_t ldk, void* stream) {
+    if (!X || !scale || !planes || rows == 0 || K == 0 || s < 1 || s > 16) return -1;
+    if (rows_padded < rows || ldk < K || (ldk & 1)) return -1;
+    const uint64_t nblk = ((ldk / 2 + 255) / 256) * rows_padded;
+    if (nblk > 0x7fffffffULL) return -1;
+    hipLaunchKernelGGL(slice_kernel, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
+                       X, rows, K, scale, s, planes, rows_padded, ldk);
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
+extern "C" int hip_ozaki_reconstruct_f64(double* C, const int32_t* Gall, const double* d_weights, int nbuf,
+                                         const double* rmax, const double* cmax,
+                                         uint64_t M, uint64_t N, void* stream) {
+    if (!C || !Gall || !d_weights || !rmax || !cmax || nbuf < 1 || M == 0 || N == 0) return -1;
+    const uint64_t nblk = (((N + 1) / 2 + 255) / 256) * M;
+    if (nblk > 0x7fffffffULL) return -1;
+    hipLaunchKernelGGL(reconstruct_kernel, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
+                       C, Gall, d_weights, nbuf, rmax, cmax, M, N);
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
+extern "C" int hip_ozaki_int8_last_stages(HipOzakiInt8Stages* out) {
+    if (!out || !g_last.a_slices) return -1;
+    *out = g_last;
+    return 0;
+}
+
+extern "C" int hip_matmul_ozaki_int8_f64(const double* A, const double* B, double* C,
+                                         uint64_t M, uint64_t K, uint64_t N, int T, void* stream) {
+    if (!A || !B || !C || M == 0 || K == 0 || N == 0) return -1;
+    if (M > 0x7fffffffULL || K > 0x7fffffffULL || N > 0x7fffffffULL) return -1;
+    if (T < 1 || T > 8) return -1;
+    /* gpu_memory_cuda.cpp:351-361: int32-exact bound on K, loud once */
+    if (K > 133000) {
+        static bool warned = false;
+        if (!warned) {
+            warned = true;
+            fprintf(stderr, "[GPU] INT8-Ozaki: K=%llu exceeds the int32-exact bound 133000; falling back to "
+                            "the native fp64 GEMM for this and future GEMMs at this K\n", (unsigned long long)K);
+        }
+        return -1;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    const int s = T + 1;
+
+    /* buffer plan, gpu_memory_cuda.cpp:367-389 */
+    long long cap = (long long)(2147483647.0 / ((double)K * 16129.0));
+    if (cap < 1) return -1;
+    struct Plan { double w[MAX_BUF]; int32_t first[MAX_BUF + 1]; int32_t pa[MAX_PAIRS]; int32_t pb[MAX_PAIRS]; };
+    Plan* plan = (Plan*)pinned(sizeof(Plan) + (M + N) * sizeof(double));
+    if (!plan) return -1;
+    double* h_max = (double*)(plan + 1);
+    int nbuf = 0, npairs = 0;
+    for (int d = 0; d <= T; d++) {
+        int pp[16], pq[16], n = 0;
+        for (int p = 0; p < s; p++) { int q = d - p; if (q >= 0 && q < s) { pp[n] = p; pq[n] = q; n++; } }
+        const double w = pow(2.0, -7.0 * (d + 2));
+        for (long long off = 0; off < n; off += cap) {
+            if (nbuf >= MAX_BUF) return -1;
+            plan->w[nbuf] = w;
+            plan->first[nbuf] = npairs;
+            for (long long t = off; t < n && t < off + cap; t++) {
+                if (npairs >= MAX_PAIRS) return -1;
+                plan->pa[npairs] = pp[t]; plan->pb[npairs] = pq[t]; npairs++;
+            }
+            nbuf++;
+        }
+    }
+    plan->first[nbuf] = npairs;
+
+    const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ldk = round_up_sz(K, 128);
+    double* Bt   = (double*)eshkol_hip_workspace(WS_BT, K * N * sizeof(double));
+    double* rmax = (double*)eshkol_hip_workspace(WS_ROWSCALE, M * sizeof(double));
+    double* cmax = (double*)eshkol_hip_workspace(WS_COLSCALE, N * sizeof(double));
+    Plan* dplan  = (Plan*)eshkol_hip_workspace(WS_MISC, sizeof(Plan));
+    int8_t* As   = (int8_t*)eshkol_hip_workspace(WS_APLANES, (size_t)s * Mp * ldk);
+    int8_t* Bs   = (int8_t*)eshkol_hip_workspace(WS_BPLANES, (size_t)s * Np * ldk);
+    int32_t* G   = (int32_t*)eshkol_hip_workspace(WS_PRODUCTS, (size_t)nbuf * M * N * sizeof(int32_t));
+    if (!Bt || !rmax || !cmax || !dplan || !As || !Bs || !G) return -1;
+
+    if (!ESHKOL_HIP_OK(hipMemcpyAsync(dplan, plan, sizeof(Plan), hipMemcpyHostToDevice, st))) return -1;
+    if (hip_transpose_f64(B, Bt, K, N, st) != 0) return -1;
+    if (hip_rowabsmax_f64(A, M, K, 1.0, rmax, st) != 0) return -1;
+    if (hip_rowabsmax_f64(Bt, N, K, 1.0, cmax, st) != 0) return -1;
+    /* NaN/Inf input is unspecified in the reference; here it is detected through
+     * the maxima and reported as failure so the caller uses the native GEMM. */
+    if (!ESHKOL_HIP_OK(hipMemcpyAsync(h_max, rmax, M * sizeof(double), hipMemcpyDeviceToHost, st))) return -1;
+    if (!ESHKOL_HIP_OK(hipMemcpyAsync(h_max + M, cmax, N * sizeof(double), hipMemcpyDeviceToHost, st))) return -1;
+    if (hip_ozaki_slice_f64(A, M, K, rmax, s, As, Mp, ldk, st) != 0) return -1;
+    if (hip_ozaki_slice_f64(Bt, N, K, cmax, s, Bs, Np, ldk, st) != 0) return -1;
+
+    HipIgemmArgs ga;
+    memset(&ga, 0, sizeof ga);
+    ga.a_planes = As; ga.b_planes = Bs;
+    ga.a_plane_stride = Mp * ldk; ga.b_plane_stride = Np * ldk;
+    ga.ldk = (uint32_t)ldk; ga.M = (uint32_t)M; ga.N = (uint32_t)N; ga.n_out = (uint32_t)nbuf;
+    ga.pair_first = dplan->first; ga.pair_a = dplan->pa; ga.pair_b = dplan->pb;
+    ga.mode = 0; ga.out_i32 = G;
+    if (hip_igemm_i8(&ga, st) != 0) return -1;
+    if (hip_ozaki_reconstruct_f64(C, G, dplan->w, nbuf, rmax, cmax, M, N, st) != 0) return -1;
+
+    if (!ESHKOL_HIP_OK(hipStreamSynchronize(st))) return -1;
+    for (uint64_t i = 0; i < M + N; i++) if (!std::isfinite(h_max[i])) return -1;
+
+    g_last.a_slices = As; g_last.b_slices = Bs; g_last.products = G;
+    g_last.rmax = rmax; g_last.cmax = cmax;
+    g_last.rows_a_padded = Mp; g_last.rows_b_padded = Np; g_last.ldk = ldk;
+    g_last.s = s; g_last.nbuf = nbuf;
+    return 0;
+}

@@ -1,0 +1,186 @@
+/*
+ * Per-tier and per-stage entry points of libeshkol_gpu_hip.so.
+ *
+ * These are the AMD counterparts of the launchers the reference's CUDA
+ * translation unit binds from its kernel file
+ * (lib/backend/gpu/gpu_memory_cuda.cpp:52-100: cuda_launch_*_f64,
+ * cuda_ozaki_split_a_f64, cuda_ozaki_split_b_f64, cuda_ozaki_reconstruct_f64)
+ * and of its static tier functions (cuda_matmul_ozaki_int8_f64 :339-452,
+ * cuda_matmul_f16_from_f64 :678-728, ozaki_ii_dispatch gpu_memory.mm:2474-2771).
+ * The runtime reaches them through eshkol_gpu_matmul_f64 /
+ * eshkol_matmul_dispatch; they are exported so that each stage can be checked
+ * on its own against the reference arithmetic.
+ *
+ * Conventions: plain C, device pointers, sizes as uint64_t in (M, K, N) order,
+ * `stream` is a hipStream_t passed as void* (NULL = the null stream). Return 0
+ * on success, -1 on a bad argument, an unsupported shape or a launch failure.
+ * Launchers do not synchronise. Tier pipelines (hip_matmul_*) may synchronise
+ * internally and use the library's cached device workspace, so calls into them
+ * must not overlap; eshkol_gpu_init() must have succeeded first.
+ */
+#ifndef ESHKOL_GPU_HIP_TIERS_H
+#define ESHKOL_GPU_HIP_TIERS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* The stream all library work is issued on (hipStream_t), for callers that
+ * bracket calls with their own events. NULL before eshkol_gpu_init(). */
+void* eshkol_hip_get_stream(void);
+
+/* ---- native fp64 tier ------------------------------------------------------
+ * C = A*B on the fp64 matrix cores; replaces the cublasDgemm call at
+ * gpu_memory_cuda.cpp:633-640 (alpha 1, beta 0, row-major, no leading dims). */
+int hip_dgemm_f64(const double* A, const double* B, double* C,
+                  uint64_t M, uint64_t K, uint64_t N, void* stream);
+
+/* Single precision, replaces cublasSgemm at gpu_memory_cuda.cpp:658-665. */
+int hip_sgemm_f32(const float* A, const float* B, float* C,
+                  uint64_t M, uint64_t K, uint64_t N, void* stream);
+
+/* ---- shared streaming kernels --------------------------------------------- */
+
+/* out[cols x rows] = in[rows x cols]^T; cuda_launch_transpose_f64,
+ * gpu_cuda_kernels.cu:189-213. */
+int hip_transpose_f64(const double* in, double* out, uint64_t rows, uint64_t cols, void* stream);
+
+/* rmax[i] = max_k |A[i,k]|, with zero_value substituted for an all-zero row:
+ * 1.0 gives ozaki_rowmax_f64_kernel (gpu_cuda_kernels.cu:664-673), 0.0 gives
+ * the row maxima of ozaki_ii_dispatch (gpu_memory.mm:2517-2524). One wave per
+ * row instead of the reference's one thread per row. */
+int hip_rowabsmax_f64(const double* A, uint64_t M, uint64_t K, double zero_value,
+                      double* rmax, void* stream);
+
+/* The 15 operations of EshkolElementwiseOp; cuda_launch_elementwise_f64,
+ * gpu_cuda_kernels.cu:21-43. b may be NULL (identity operand). */
+int hip_elementwise_f64(const double* a, const double* b, double* out, uint64_t n, int op, void* stream);
+
+/* In place Y[i,j] = act(Y[i,j] + bias[j]); act 0 none, 1 tanh. bias may be
+ * NULL. The dense-layer epilogue (broadcast add runtime_tensor_math.cpp:672-740,
+ * tanh lib/core/model_io.cpp:709) for tiers that do not fuse it. */
+int hip_bias_act_f64(double* Y, const double* bias, uint64_t rows, uint64_t cols, int act, void* stream);
+
+/* ---- int8 matrix-core contraction ------------------------------------------
+ * Replaces the cublasGemmEx(int8 x int8 -> int32) loop at
+ * gpu_memory_cuda.cpp:415-434 and the modular GEMM matmul_ozaki_gemm
+ * (metal_softfloat.h:3907-4100). Operand planes are K-contiguous int8 with a
+ * row pitch of ldk bytes (multiple of 128, zero padded beyond K) and row counts
+ * padded with zero rows to multiples of 256. */
+typedef struct {
+    const int8_t* a_planes;   /* [n_a_planes][rows_a_padded][ldk]                */
+    const int8_t* b_planes;   /* [n_b_planes][rows_b_padded][ldk]                */
+    uint64_t a_plane_stride;  /* bytes between consecutive A planes              */
+    uint64_t b_plane_stride;
+    uint32_t ldk;
+    uint32_t M, N;            /* logical output size                             */
+    uint32_t n_out;           /* number of output planes                         */
+    /* Output plane o is the int32 sum of the products pair_first[o] ..
+     * pair_first[o+1]-1; product t multiplies A plane pair_a[t] by B plane
+     * pair_b[t]. The three arrays live in device memory.                        */
+    const int32_t* pair_first;
+    const int32_t* pair_a;
+    const int32_t* pair_b;
+    /* mode 0: out_i32[o][M][N] = the int32 sums
+     * mode 1: out_i8[o][M][N]  = the sum modulo modulus[o], representative in
+     *         [-p/2, p/2); modulus[] in device memory                           */
+    int32_t mode;
+    const int32_t* modulus;
+    int32_t* out_i32;
+    int8_t*  out_i8;
+} HipIgemmArgs;
+int hip_igemm_i8(const HipIgemmArgs* args, void* stream);
+
+/* ---- Ozaki-II CRT exact tier ------------------------------------------------
+ * Residue planes of trunc(X[i,k] * 2^shift[i]) modulo the first num_moduli
+ * entries of the reference's modulus table (gpu_memory.mm:227-233, 2538-2583):
+ * planes[l][i][k], representative in [-p/2, p/2), pitch ldk, rows_padded rows
+ * per plane (padding written as zeros). Used for A directly and for B through
+ * its transpose, so both operands come out K-contiguous. */
+int hip_ozaki_crt_split_f64(const double* X, uint64_t rows, uint64_t K,
+                            const int32_t* shift, int num_moduli,
+                            int8_t* planes, uint64_t rows_padded, uint64_t ldk, void* stream);
+
+/* CRT accumulation, reconstruction and inverse scaling (gpu_memory.mm:2626-2655)
+ * from the int8 residue products w_planes[l][M][N]; optional fused dense-layer
+ * epilogue C = act(C + bias[j]) (act 0 none, 1 tanh; bias may be NULL). */
+int hip_ozaki_crt_reconstruct_f64(const int8_t* w_planes, uint64_t M, uint64_t N, int num_moduli,
+                                  const double* sl1, const double* sl2,
+                                  double P1, double P2, double Pinv,
+                                  const int32_t* mu, const int32_t* nu,
+                                  const double* bias, int act,
+                                  double* C, void* stream);
+
+/* Whole tier: ozaki_ii_dispatch (gpu_memory.mm:2474-2665). num_moduli in
+ * [2,16]; adaptive != 0 picks the count as ESHKOL_OZAKI_ADAPTIVE=1 does.
+ * Returns -1 (caller falls back to the native tier) for K > 131071, non-finite
+ * input, or scale factors outside the double range. */
+int hip_matmul_ozaki_crt_f64(const double* A, const double* B, double* C,
+                             uint64_t M, uint64_t K, uint64_t N,
+                             int num_moduli, int adaptive,
+                             const double* bias, int act, void* stream);
+
+/* Stage outputs of the last hip_matmul_ozaki_crt_f64 call, for parity checks:
+ * device pointers into the library workspace (valid until the next call). */
+typedef struct {
+    const int8_t* a_planes; const int8_t* b_planes; const int8_t* w_planes;
+    const int32_t* mu; const int32_t* nu;
+    uint64_t rows_a_padded, rows_b_padded, ldk;
+    int32_t num_moduli, E;
+} HipOzakiCrtStages;
+int hip_ozaki_crt_last_stages(HipOzakiCrtStages* out);
+
+/* ---- INT8 slice tier ----------------------------------------------------------
+ * s base-128 slices of X[i,k] / scale[i] (gpu_cuda_kernels.cu:688-723):
+ * planes[p][i][k], pitch ldk, rows_padded rows per plane, padding zero. With
+ * rows_padded == rows and ldk == K this is the reference's layout for A, and
+ * for B when X is B transposed. */
+int hip_ozaki_slice_f64(const double* X, uint64_t rows, uint64_t K, const double* scale, int s,
+                        int8_t* planes, uint64_t rows_padded, uint64_t ldk, void* stream);
+
+/* cuda_ozaki_reconstruct_f64 (gpu_cuda_kernels.cu:728-741, 779-798), weights
+ * already in device memory. */
+int hip_ozaki_reconstruct_f64(double* C, const int32_t* Gall, const double* d_weights, int nbuf,
+                              const double* rmax, const double* cmax,
+                              uint64_t M, uint64_t N, void* stream);
+
+/* Whole tier: cuda_matmul_ozaki_int8_f64 (gpu_memory_cuda.cpp:339-452), T in [1,8]. */
+int hip_matmul_ozaki_int8_f64(const double* A, const double* B, double* C,
+                              uint64_t M, uint64_t K, uint64_t N, int T, void* stream);
+
+typedef struct {
+    const int8_t* a_slices; const int8_t* b_slices; const int32_t* products;
+    const double* rmax; const double* cmax;
+    uint64_t rows_a_padded, rows_b_padded, ldk;
+    int32_t s, nbuf;
+} HipOzakiInt8Stages;
+int hip_ozaki_int8_last_stages(HipOzakiInt8Stages* out);
+
+/* ---- reduced-precision tier ----------------------------------------------------
+ * cuda_matmul_f16_from_f64 (gpu_memory_cuda.cpp:678-728) with the conversions
+ * on the device: operands in f64 storage are narrowed to dtype 2 (f16) or 3
+ * (bf16), multiplied on the matrix cores with fp32 accumulation, and written
+ * back as f64. round_output != 0 rounds the fp32 result to the 16-bit type
+ * first, as the reference's 16F output does. */
+int hip_matmul_reduced_f64(const double* A, const double* B, double* C,
+                           uint64_t M, uint64_t K, uint64_t N,
+                           int dtype, int round_output, void* stream);
+
+/* 16-bit operands already in device memory (A [M][K], Bt [N][K], pitch ld
+ * elements, multiple of 64, rows padded to multiples of 256 with zeros), fp32
+ * result C[M][N]: the contraction alone (BASELINE configuration 4). */
+int hip_hgemm_16(const uint16_t* A, const uint16_t* Bt, uint64_t M, uint64_t K, uint64_t N,
+                 uint64_t ld, int is_bf16, float* C, void* stream);
+
+/* RNE narrowing of f64 storage to f16/bf16 (runtime_tensor_dtype.cpp:37-109),
+ * out[i][k] with pitch ld and rows_padded rows, padding zero. */
+int hip_convert_f64_to_16(const double* in, uint16_t* out, uint64_t rows, uint64_t cols,
+                          uint64_t rows_padded, uint64_t ld, int is_bf16, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
