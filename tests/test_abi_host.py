@@ -1,0 +1,198 @@
+"""Host-side checks that need no GPU: the library loads, exports every symbol
+the public headers declare, keeps the reference's struct layout and return
+conventions, parses its environment loudly, and hands work it cannot run to the
+host runtime's CPU matmul. No compute kernel is launched here."""
+import ctypes as C
+import os
+import re
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+import eshkol_amd as ea
+import oracle
+from conftest import ROOT
+
+INC = os.path.join(ROOT, "include", "eshkol", "backend", "gpu")
+HAVE_GPU = os.path.exists("/dev/kfd")
+
+
+def declared_functions(header):
+    text = open(os.path.join(INC, header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = re.findall(r"\b([a-z_0-9]+)\s*\(", text)
+    return sorted({n for n in names if n.startswith(("eshkol_", "hip_"))})
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ea.load()
+    declared = declared_functions("gpu_memory.h") + declared_functions("gpu_hip_tiers.h")
+    assert len(declared) >= 45
+    for name in declared:
+        assert hasattr(lib, name), name
+        assert name in ea.SIGNATURES, "binding table is missing %s" % name
+    assert C.c_size_t.in_dll(lib, "g_gpu_threshold").value in (100000, int(os.environ.get("ESHKOL_GPU_THRESHOLD", 100000)))
+
+
+def test_reference_header_symbols_are_all_present():
+    # the 30 functions + 1 global of the reference's gpu_memory.h:90-474
+    expected = """eshkol_gpu_init eshkol_gpu_shutdown eshkol_gpu_get_backend eshkol_gpu_backend_name
+    eshkol_gpu_backend_available eshkol_gpu_supports_f64 eshkol_gpu_has_fp64 eshkol_gpu_alloc
+    eshkol_gpu_alloc_aligned eshkol_gpu_free eshkol_gpu_wrap_host eshkol_gpu_sync eshkol_gpu_sync_async
+    eshkol_gpu_wait eshkol_gpu_matmul_f64 eshkol_gpu_matmul_f32 eshkol_gpu_set_threshold
+    eshkol_gpu_get_threshold eshkol_gpu_should_use eshkol_gpu_elementwise_f64 eshkol_gpu_reduce_f64
+    eshkol_gpu_reduce_axis_f64 eshkol_gpu_transpose_f64 eshkol_gpu_softmax_f64 eshkol_gpu_normalize_f64
+    eshkol_gpu_conv2d_backward_input_f64 eshkol_gpu_conv2d_backward_kernel_f64
+    eshkol_gpu_batchnorm_backward_f64 eshkol_gpu_layernorm_backward_f64 eshkol_matmul_dispatch
+    eshkol_batch_matmul_dispatch""".split()
+    assert len(expected) == 31
+    lib = ea.load()
+    for name in expected:
+        assert hasattr(lib, name), name
+
+
+def test_buffer_struct_layout_matches_reference():
+    # vm_gpu_dispatch.h:60 mirrors this layout by hand: 2 pointers, size_t, 2 enums, u32, pointer
+    assert C.sizeof(ea.EshkolGPUBuffer) == 48
+    assert ea.EshkolGPUBuffer.size_bytes.offset == 16
+    assert ea.EshkolGPUBuffer.mem_type.offset == 24
+    assert ea.EshkolGPUBuffer.flags.offset == 32
+    assert ea.EshkolGPUBuffer.backend_data.offset == 40
+
+
+def test_backend_names_and_enum():
+    lib = ea.load()
+    assert lib.eshkol_gpu_backend_name(ea.GPU_HIP) == b"AMD HIP (gfx950)"
+    assert lib.eshkol_gpu_backend_name(ea.GPU_NONE) == b"CPU (no GPU)"
+    assert lib.eshkol_gpu_backend_name(99) == b"Unknown"
+
+
+def test_threshold_api():
+    lib = ea.load()
+    old = lib.eshkol_gpu_get_threshold()
+    lib.eshkol_gpu_set_threshold(12345)
+    assert lib.eshkol_gpu_get_threshold() == 12345
+    assert C.c_size_t.in_dll(lib, "g_gpu_threshold").value == 12345
+    lib.eshkol_gpu_set_threshold(old)
+
+
+def test_argument_validation_needs_no_device():
+    lib = ea.load()
+    buf = ea.EshkolGPUBuffer()
+    assert lib.eshkol_gpu_alloc(0, ea.MEM_DEVICE, C.byref(buf)) == -1
+    assert lib.eshkol_gpu_alloc(16, ea.MEM_DEVICE, None) == -1
+    assert lib.eshkol_gpu_wrap_host(None, 16, C.byref(buf)) == -1
+    assert lib.eshkol_gpu_sync(None, ea.SYNC_DEVICE_TO_HOST) == -1
+    assert lib.eshkol_gpu_matmul_f64(None, None, None, 1, 1, 1) == -1
+    assert lib.eshkol_gpu_alloc_aligned(100, 3, ea.MEM_DEVICE, C.byref(buf)) == -1   # not a power of two
+    assert lib.hip_dgemm_f64(None, None, None, 4, 4, 4, None) == -1
+    assert lib.hip_matmul_ozaki_int8_f64(None, None, None, 4, 4, 4, 6, None) == -1
+    assert lib.eshkol_gpu_reduce_f64(None, None, 4, 0) == -1
+    assert lib.eshkol_gpu_conv2d_backward_input_f64(None, None, None, *([1] * 11)) == -1
+    lib.eshkol_gpu_free(None)
+
+
+# ---- behaviour without a GPU, in a child process so state does not leak ----------
+
+CHILD = r"""
+import ctypes as C, os, sys
+import numpy as np
+sys.path.insert(0, %(root)r)
+import oracle, eshkol_amd as ea
+rt = C.CDLL(oracle.HOSTRT_PATH, mode=C.RTLD_GLOBAL)       # plays the host runtime's CPU side
+rt.oracle_hostrt_matmul_calls.restype = C.c_long
+rt.oracle_hostrt_batch_calls.restype = C.c_long
+lib = ea.load()
+%(body)s
+"""
+
+
+def run_child(body, env=None):
+    e = dict(os.environ)
+    e["HIP_VISIBLE_DEVICES"] = "-1"
+    e["ROCR_VISIBLE_DEVICES"] = "-1"
+    if env:
+        e.update(env)
+    code = CHILD % {"root": ROOT, "body": body}
+    return subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=e, timeout=300)
+
+
+def test_init_without_device_reports_cpu_only_and_host_buffers_work():
+    body = r"""
+r = lib.eshkol_gpu_init()
+assert r == 0 and lib.eshkol_gpu_init() == 0, r          # boolean, idempotent
+assert lib.eshkol_gpu_get_backend() == ea.GPU_NONE
+assert lib.eshkol_gpu_supports_f64() == 0 and lib.eshkol_gpu_has_fp64() == 0
+assert lib.eshkol_gpu_backend_available(ea.GPU_HIP) == 0 and lib.eshkol_gpu_backend_available(ea.GPU_NONE) == 1
+assert lib.eshkol_gpu_should_use(10**9) == 0
+b = ea.EshkolGPUBuffer()
+assert lib.eshkol_gpu_alloc(1024, ea.MEM_UNIFIED, C.byref(b)) == 0
+assert b.backend == ea.GPU_NONE and b.mem_type == ea.MEM_HOST and b.host_ptr == b.device_ptr and b.size_bytes == 1024
+lib.eshkol_gpu_free(C.byref(b)); assert not b.host_ptr and b.size_bytes == 0
+x = np.arange(8.0)
+assert lib.eshkol_gpu_wrap_host(x.ctypes.data, x.nbytes, C.byref(b)) == 0
+assert b.host_ptr == x.ctypes.data and (b.flags & 1)
+assert lib.eshkol_gpu_sync(C.byref(b), ea.SYNC_DEVICE_TO_HOST) == 0
+lib.eshkol_gpu_free(C.byref(b)); assert x[3] == 3.0      # wrapped memory is never freed
+lib.eshkol_gpu_shutdown(); assert lib.eshkol_gpu_init() == 0
+print("OK")
+"""
+    r = run_child(body)
+    assert r.returncode == 0 and "OK" in r.stdout, r.stderr + r.stdout
+
+
+def test_dispatch_falls_back_to_host_runtime_without_device():
+    body = r"""
+rng = np.random.default_rng(0)
+A = rng.standard_normal((40, 30)); B = rng.standard_normal((30, 50))
+got = ea.matmul_dispatch(A, B)
+assert rt.oracle_hostrt_matmul_calls() == 1
+assert np.array_equal(got, oracle.matmul_f64(A, B))
+got = ea.matmul_dispatch(A, B, ea.DTYPE_BF16)               # dtype is ignored without a GPU
+assert rt.oracle_hostrt_matmul_calls() == 2 and np.array_equal(got, oracle.matmul_f64(A, B))
+# eshkol_gpu_matmul_f64 on host buffers runs the runtime's CPU matmul too
+ba, bb, bc = ea.EshkolGPUBuffer(), ea.EshkolGPUBuffer(), ea.EshkolGPUBuffer()
+out = np.zeros((40, 50))
+for arr, b in ((A, ba), (B, bb), (out, bc)):
+    assert lib.eshkol_gpu_wrap_host(arr.ctypes.data, arr.nbytes, C.byref(b)) == 0
+assert lib.eshkol_gpu_matmul_f64(C.byref(ba), C.byref(bb), C.byref(bc), 40, 30, 50) == 0
+assert np.array_equal(out, oracle.matmul_f64(A, B)) and rt.oracle_hostrt_matmul_calls() == 3
+a = rng.standard_normal((3, 5, 7)); b = rng.standard_normal((3, 7, 4)); c = np.empty((3, 5, 4))
+lib.eshkol_batch_matmul_dispatch(a.ctypes.data, b.ctypes.data, c.ctypes.data, 3, 5, 7, 4, 0)
+assert rt.oracle_hostrt_batch_calls() == 1 and np.array_equal(c, oracle.batch_matmul_f64(a, b))
+print("OK")
+"""
+    r = run_child(body)
+    assert r.returncode == 0 and "OK" in r.stdout, r.stderr + r.stdout
+
+
+def test_missing_host_runtime_is_fatal_not_silent():
+    code = r"""
+import sys
+sys.path.insert(0, %r)
+import numpy as np, eshkol_amd as ea
+A = np.ones((4, 4)); ea.matmul_dispatch(A, A)
+print("SURVIVED")
+""" % ROOT
+    e = dict(os.environ, HIP_VISIBLE_DEVICES="-1", ROCR_VISIBLE_DEVICES="-1")
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=e, timeout=300)
+    assert r.returncode != 0 and "SURVIVED" not in r.stdout
+    assert "FATAL" in r.stderr and "eshkol_matmul_f64" in r.stderr
+
+
+def test_out_of_range_knobs_are_loud():
+    # cuda_ozaki_correctness_gate.sh:120-125 greps for "out of range"
+    body = 'lib.eshkol_gpu_init(); print("OK")'
+    r = run_child(body, {"ESHKOL_OZAKI_CUDA_T": "99"})
+    assert r.returncode == 0 and "ESHKOL_OZAKI_CUDA_T=99 out of range" in r.stderr
+    r = run_child(body, {"ESHKOL_OZAKI_NUM_MODULI": "32"})
+    assert r.returncode == 0 and "ESHKOL_OZAKI_NUM_MODULI=32 out of range" in r.stderr
+    r = run_child(body, {"ESHKOL_OZAKI_CUDA_T": "4", "ESHKOL_OZAKI_NUM_MODULI": "12"})
+    assert r.returncode == 0 and "out of range" not in r.stderr
+
+
+def test_threshold_env_is_read_at_init():
+    r = run_child('lib.eshkol_gpu_init(); print(lib.eshkol_gpu_get_threshold())', {"ESHKOL_GPU_THRESHOLD": "777"})
+    assert r.returncode == 0 and r.stdout.strip().endswith("777")

@@ -1,0 +1,231 @@
+"""The drop-in boundary on a GPU: buffer lifecycle, eshkol_gpu_matmul_f64 and
+its environment-driven tier selection, eshkol_matmul_dispatch with its threshold
+and fallback ladder, the batched entry, elementwise and transpose. Environment
+variables are parsed once per process, so each configuration runs in a child
+process that calls the library through the same ctypes binding."""
+import ctypes as C
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+import eshkol_amd as ea
+import oracle
+from eshkol_amd import synth
+from conftest import ROOT
+from gpu_util import normwise
+
+pytestmark = pytest.mark.gpu
+
+CHILD = r"""
+import ctypes as C, os, sys
+import numpy as np
+sys.path.insert(0, %(root)r); sys.path.insert(0, os.path.join(%(root)r, "tests"))
+import oracle, eshkol_amd as ea
+from eshkol_amd import synth
+from gpu_util import normwise, ulp_distance
+rt = C.CDLL(oracle.HOSTRT_PATH, mode=C.RTLD_GLOBAL)
+rt.oracle_hostrt_matmul_calls.restype = C.c_long
+rt.oracle_hostrt_batch_calls.restype = C.c_long
+lib = ea.load()
+%(body)s
+print("CHILD-OK")
+"""
+
+
+def run_child(body, env=None):
+    e = dict(os.environ)
+    for k in list(e):
+        if k.startswith("ESHKOL_"):
+            del e[k]
+    if env:
+        e.update(env)
+    r = subprocess.run([sys.executable, "-u", "-c", CHILD % {"root": ROOT, "body": body}],
+                       capture_output=True, text=True, env=e, timeout=600)
+    assert r.returncode == 0 and "CHILD-OK" in r.stdout, "stdout:\n%s\nstderr:\n%s" % (r.stdout, r.stderr)
+    return r
+
+
+def test_buffer_lifecycle(gpu):
+    lib = ea.load()
+    b = ea.EshkolGPUBuffer()
+    assert lib.eshkol_gpu_get_backend() == ea.GPU_HIP and lib.eshkol_gpu_init() == 1
+    assert lib.eshkol_gpu_supports_f64() == 1 and lib.eshkol_gpu_has_fp64() == 1
+    assert lib.eshkol_gpu_backend_available(ea.GPU_HIP) == 1 and lib.eshkol_gpu_backend_available(ea.GPU_CUDA) == 0
+    assert lib.eshkol_gpu_alloc(4096, ea.MEM_DEVICE, C.byref(b)) == 0
+    assert b.host_ptr is None and b.device_ptr and b.mem_type == ea.MEM_DEVICE and b.backend == ea.GPU_HIP
+    lib.eshkol_gpu_free(C.byref(b)); assert not b.device_ptr and b.size_bytes == 0
+    assert lib.eshkol_gpu_alloc(4096, ea.MEM_UNIFIED, C.byref(b)) == 0
+    assert b.host_ptr == b.device_ptr and b.host_ptr
+    lib.eshkol_gpu_free(C.byref(b))
+    assert lib.eshkol_gpu_alloc(4096, ea.MEM_HOST_PINNED, C.byref(b)) == 0
+    assert b.host_ptr and b.device_ptr is None
+    lib.eshkol_gpu_free(C.byref(b))
+    assert lib.eshkol_gpu_alloc_aligned(1000, 256, ea.MEM_DEVICE, C.byref(b)) == 0 and b.size_bytes == 1024
+    lib.eshkol_gpu_free(C.byref(b))
+    # wrap: device copy, sync D2H lands in the caller's memory, free never frees it
+    x = np.arange(1024.0); y = np.zeros(1024)
+    bx, by = ea.EshkolGPUBuffer(), ea.EshkolGPUBuffer()
+    assert lib.eshkol_gpu_wrap_host(x.ctypes.data, x.nbytes, C.byref(bx)) == 0 and (bx.flags & 1)
+    assert lib.eshkol_gpu_wrap_host(y.ctypes.data, y.nbytes, C.byref(by)) == 0
+    assert lib.eshkol_gpu_elementwise_f64(C.byref(bx), C.byref(bx), C.byref(by), 1024, 0) == 0   # y = x + x
+    assert lib.eshkol_gpu_sync(C.byref(by), ea.SYNC_DEVICE_TO_HOST) == 0
+    assert np.array_equal(y, 2 * x)
+    assert lib.eshkol_gpu_elementwise_f64(C.byref(by), None, C.byref(by), 1024, 4) == 0          # y = -y
+    lib.eshkol_gpu_free(C.byref(by))                       # copy-back on free
+    assert np.array_equal(y, -2 * x)
+    lib.eshkol_gpu_free(C.byref(bx)); assert x[5] == 5.0
+    lib.eshkol_gpu_wait(None)
+
+
+def test_gpu_matmul_f64_on_device_buffers(gpu):
+    lib = ea.load()
+    M, K, N = 300, 200, 260
+    A, B = synth.normal(1, (M, K)), synth.normal(2, (K, N))
+    dA, dB, dC = ea.DeviceArray.from_host(A), ea.DeviceArray.from_host(B), ea.DeviceArray((M, N))
+    assert lib.eshkol_gpu_matmul_f64(C.byref(dA.buf), C.byref(dB.buf), C.byref(dC.buf), M, K, N) == 0
+    assert normwise(dC.download(), oracle.matmul_f64(A, B), A, B) <= 1e-14
+    small = ea.DeviceArray((4, 4))
+    assert lib.eshkol_gpu_matmul_f64(C.byref(dA.buf), C.byref(dB.buf), C.byref(small.buf), M, K, N) == -1
+    host = ea.EshkolGPUBuffer()
+    assert lib.eshkol_gpu_matmul_f64(C.byref(host), C.byref(dB.buf), C.byref(dC.buf), M, K, N) == -1
+    # single precision entry
+    Af, Bf = A.astype(np.float32), B.astype(np.float32)
+    fa, fb, fc = ea.DeviceArray.from_host(Af), ea.DeviceArray.from_host(Bf), ea.DeviceArray((M, N), np.float32)
+    assert lib.eshkol_gpu_matmul_f32(C.byref(fa.buf), C.byref(fb.buf), C.byref(fc.buf), M, K, N) == 0
+    assert normwise(fc.download(), Af.astype(np.float64) @ Bf.astype(np.float64), Af, Bf) <= 1e-6
+
+
+def test_elementwise_family_and_transpose(gpu):
+    lib = ea.load()
+    n = 5000
+    a = synth.uniform(3, (n,), 0.1, 3.0); b = synth.uniform(4, (n,), 0.5, 2.0)
+    da, db, do = ea.DeviceArray.from_host(a), ea.DeviceArray.from_host(b), ea.DeviceArray((n,))
+    expect = [a + b, a - b, a * b, a / b, -a, np.abs(a), np.exp(a), np.log(a), np.sin(a), np.cos(a),
+              np.tanh(a), np.maximum(a, 0), 1 / (1 + np.exp(-a)), np.sqrt(a), 1 / a]
+    for op, want in enumerate(expect):
+        bb = C.byref(db.buf) if op < 4 else None
+        assert lib.eshkol_gpu_elementwise_f64(C.byref(da.buf), bb, C.byref(do.buf), n, op) == 0
+        got = do.download()
+        if op in (0, 1, 2, 3, 4, 5, 11, 13, 14):
+            assert np.array_equal(got, want), op          # correctly rounded operations
+        else:
+            assert np.abs(got - want).max() <= 4e-16 * max(1.0, np.abs(want).max()), op
+    assert lib.eshkol_gpu_elementwise_f64(C.byref(da.buf), None, C.byref(do.buf), n, 15) == -1
+    X = synth.normal(5, (130, 70))
+    dx, dt = ea.DeviceArray.from_host(X), ea.DeviceArray((70, 130))
+    assert lib.eshkol_gpu_transpose_f64(C.byref(dx.buf), C.byref(dt.buf), 130, 70) == 0
+    assert np.array_equal(dt.download(), X.T)
+    # the operations left to the caller's CPU rules report failure
+    assert lib.eshkol_gpu_reduce_f64(C.byref(da.buf), C.byref(do.buf), n, 0) == -1
+    assert lib.eshkol_gpu_softmax_f64(C.byref(da.buf), C.byref(do.buf), 10, 500) == -1
+
+
+def test_dispatch_threshold_and_fallback_ladder(gpu):
+    body = r"""
+A = synth.normal(1, (200, 150)); B = synth.normal(2, (150, 300))
+ref = oracle.matmul_f64(A, B)
+# default threshold 100000: 200*300 = 60000 outputs stay on the runtime's CPU path
+got = ea.matmul_dispatch(A, B)
+assert rt.oracle_hostrt_matmul_calls() == 1 and np.array_equal(got, ref)
+lib.eshkol_gpu_set_threshold(1)
+got = ea.matmul_dispatch(A, B)
+assert rt.oracle_hostrt_matmul_calls() == 1               # GPU took it
+assert normwise(got, ref, A, B) <= 1e-14
+assert lib.eshkol_gpu_should_use(1) == 1
+# known answers through the dispatcher (tests/gpu/matmul_correctness_test.esk)
+assert np.array_equal(ea.matmul_dispatch(np.array([[1., 2.], [3., 4.]]), np.array([[5., 6.], [7., 8.]])), [[19, 22], [43, 50]])
+# tests/gpu/gpu_scale_correctness_test.esk:14-80
+n = 4096
+Cc = ea.matmul_dispatch(np.ones((n, n)), np.ones((n, n)))
+assert np.all(Cc == 4096.0)
+R = np.repeat(np.arange(1., n + 1)[:, None], n, axis=1)
+Cc = ea.matmul_dispatch(R, np.ones((n, n)))
+assert np.array_equal(Cc[:, 0], 4096.0 * np.arange(1, n + 1))
+# f16 / bf16 dtype codes take the reduced tier
+A = synth.normal(3, (256, 512), 1 / np.sqrt(512)); B = synth.normal(4, (512, 128), 1 / np.sqrt(512))
+for d in (2, 3):
+    got = ea.matmul_dispatch(A, B, d)
+    Ar, Br = oracle.reduce_precision(A, d), oracle.reduce_precision(B, d)
+    assert normwise(got, oracle.matmul_f64(Ar, Br), Ar, Br) <= 1e-2
+    ok = np.abs(got) >= 2.0 ** -14                                   # away from the reference's f16 subnormal quirk
+    assert np.array_equal(got[ok], oracle.reduce_precision(got, d)[ok])   # result carries the 16-bit rounding
+assert rt.oracle_hostrt_matmul_calls() == 1
+# batched entry: dtype 3 on the GPU, dtype 0 on the runtime's CPU path
+a = synth.normal(5, (4, 96, 160), 0.1); b = synth.normal(6, (4, 160, 64), 0.1); c = np.empty((4, 96, 64))
+lib.eshkol_batch_matmul_dispatch(a.ctypes.data, b.ctypes.data, c.ctypes.data, 4, 96, 160, 64, 3)
+assert rt.oracle_hostrt_batch_calls() == 0
+for i in range(4):
+    Ar, Br = oracle.reduce_precision(a[i], 3), oracle.reduce_precision(b[i], 3)
+    assert normwise(c[i], oracle.matmul_f64(Ar, Br), Ar, Br) <= 1e-2
+lib.eshkol_batch_matmul_dispatch(a.ctypes.data, b.ctypes.data, c.ctypes.data, 4, 96, 160, 64, 0)
+assert rt.oracle_hostrt_batch_calls() == 1 and np.array_equal(c, oracle.batch_matmul_f64(a, b))
+"""
+    r = run_child(body, {"ESHKOL_GPU_VERBOSE": "1"})
+    assert "native fp64 MFMA" in r.stderr and "reduced tier" in r.stderr
+
+
+def test_threshold_env_forces_gpu(gpu):
+    body = r"""
+A = synth.normal(1, (8, 8)); B = np.eye(8)
+got = ea.matmul_dispatch(A, B)                 # tests/gpu/cuda_host_sync_regression_test.esk:14-39
+assert np.array_equal(got, A) and rt.oracle_hostrt_matmul_calls() == 0
+"""
+    r = run_child(body, {"ESHKOL_GPU_THRESHOLD": "1", "ESHKOL_GPU_VERBOSE": "1"})
+    assert "[GPU] matmul 8x8 @ 8x8 -> native fp64 MFMA" in r.stderr
+
+
+def test_tier_override_crt(gpu):
+    body = r"""
+n = 512
+A = synth.wide_range(1, (n, n)); B = synth.wide_range(2, (n, n))
+got = ea.matmul_dispatch(A, B)
+assert ulp_distance(got, oracle.matmul_ozaki_crt(A, B)).max() <= 2
+small = ea.matmul_dispatch(A[:256, :256], B[:256, :256])     # below 512: native tier
+assert normwise(small, oracle.matmul_f64(A[:256, :256], B[:256, :256]), A[:256, :256], B[:256, :256]) <= 1e-14
+"""
+    for env in ({"ESHKOL_HIP_F64_KERNEL": "ozaki-crt"}, {"ESHKOL_SF64_KERNEL": "ozaki"}):
+        env = dict(env, ESHKOL_GPU_THRESHOLD="1", ESHKOL_GPU_VERBOSE="1", ESHKOL_OZAKI_PROFILE="1")
+        r = run_child(body, env)
+        assert r.stderr.count("[GPU] Ozaki-II: N=16, log2(P)=125.4") == 1      # one marker per dispatch
+        assert "Ozaki-II CRT exact" in r.stderr and "[OZAKI_PROFILE] exact M=512" in r.stderr
+        assert "native fp64 MFMA" in r.stderr
+    r = run_child(body, {"ESHKOL_HIP_F64_KERNEL": "ozaki-crt", "ESHKOL_GPU_THRESHOLD": "1",
+                         "ESHKOL_OZAKI_NUM_MODULI": "32"})
+    assert "out of range" in r.stderr                                          # loud clamp, still correct
+
+
+def test_tier_override_int8_and_budget_selector(gpu):
+    body = r"""
+n = 1024
+A = synth.normal(1, (n, n)); B = synth.normal(2, (n, n))
+T = int(os.environ.get("EXPECT_T", "6"))
+got = ea.matmul_dispatch(A, B)
+assert ulp_distance(got, oracle.matmul_ozaki_int8(A, B, T)).max() <= 2
+"""
+    r = run_child(body, {"ESHKOL_CUDA_F64_KERNEL": "ozaki-int8", "ESHKOL_GPU_THRESHOLD": "1", "ESHKOL_GPU_VERBOSE": "1"})
+    assert "INT8-Ozaki T=6" in r.stderr
+    r = run_child(body, {"ESHKOL_HIP_F64_KERNEL": "ozaki-int8", "ESHKOL_OZAKI_CUDA_T": "4", "EXPECT_T": "4",
+                         "ESHKOL_GPU_THRESHOLD": "1", "ESHKOL_GPU_VERBOSE": "1"})
+    assert "INT8-Ozaki T=4" in r.stderr
+    r = run_child(body, {"ESHKOL_CUDA_F64_KERNEL": "ozaki-int8", "ESHKOL_OZAKI_CUDA_T": "99",
+                         "ESHKOL_GPU_THRESHOLD": "1"})
+    assert "out of range" in r.stderr
+    # accuracy budget: a loose budget picks a small T, a strict one stays native
+    body2 = r"""
+n = 4096
+A = synth.normal(1, (n, n)); B = synth.normal(2, (n, n))
+got = ea.matmul_dispatch(A, B)
+rows = list(range(0, n, 587))
+ref = A[rows].astype(np.longdouble) @ B.astype(np.longdouble)
+err = normwise(got[rows], ref, A[rows], B)
+assert err <= float(os.environ["EXPECT_ERR"]), err
+"""
+    r = run_child(body2, {"ESHKOL_MATMUL_ACCURACY": "fast", "EXPECT_ERR": "1e-3", "ESHKOL_GPU_THRESHOLD": "1",
+                          "ESHKOL_GPU_VERBOSE": "1"})
+    assert "INT8-Ozaki T=1 (accuracy-budget selector" in r.stderr
+    r = run_child(body2, {"ESHKOL_MATMUL_ACCURACY": "exact", "EXPECT_ERR": "1e-14", "ESHKOL_GPU_THRESHOLD": "1",
+                          "ESHKOL_GPU_VERBOSE": "1"})
+    assert "native fp64 MFMA (budget met cheapest by native fp64)" in r.stderr

@@ -1,0 +1,86 @@
+"""Native fp64 tier on the GPU (hip_dgemm_f64, through the C ABI) against the
+oracle's restatement of the reference CPU matmul. Bar (BASELINE.json):
+||C - C_ref||_F / (||A||_F ||B||_F) <= 1e-14."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from eshkol_amd import synth
+from conftest import GOLDEN
+from gpu_util import normwise, run_dgemm
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-14
+
+SHAPES = [(1, 1, 1), (2, 2, 2), (1, 100, 1), (3, 5, 4), (5, 7, 3), (16, 16, 16), (64, 64, 64),
+          (65, 67, 66), (37, 130, 9), (128, 128, 128), (129, 257, 131), (256, 256, 256),
+          (300, 17, 500), (512, 1000, 64), (1000, 33, 1000), (1024, 1024, 1024)]
+
+
+@pytest.mark.parametrize("M,K,N", SHAPES)
+def test_dgemm_matches_reference_cpu_statement(gpu, M, K, N):
+    print("dgemm", M, K, N, flush=True)
+    A, B = synth.uniform(100 + M, (M, K)), synth.uniform(200 + N, (K, N))
+    Cg = run_dgemm(A, B)
+    assert normwise(Cg, oracle.matmul_f64(A, B), A, B) <= TOL
+
+
+def test_dgemm_against_golden_vectors(gpu):
+    g = np.load(os.path.join(GOLDEN, "fp64_matmul.npz"))
+    for ci in range(8):
+        M, K, N = (int(v) for v in g["case%d_shape" % ci])
+        sa, sb = (int(v) for v in g["case%d_seeds" % ci])
+        A, B = synth.uniform(sa, (M, K)), synth.uniform(sb, (K, N))
+        assert normwise(run_dgemm(A, B), g["case%d_avx" % ci], A, B) <= TOL
+    A, B = synth.uniform(42, (256, 256)), synth.uniform(43, (256, 256))      # configuration 1
+    Cg = run_dgemm(A, B)
+    assert np.abs(Cg[17] - g["c1_avx_row17"]).max() <= 1e-13
+    assert abs(float(np.sum(Cg.astype(np.longdouble))) - float(g["c1_avx_sum"][0])) <= 1e-9
+
+
+def test_known_answers_are_exact(gpu):
+    a = np.array([[1., 2.], [3., 4.]]); b = np.array([[5., 6.], [7., 8.]])
+    assert np.array_equal(run_dgemm(a, b), [[19, 22], [43, 50]])
+    assert np.array_equal(run_dgemm(np.eye(2), a), a)
+    a23 = np.array([[1., 2., 3.], [4., 5., 6.]]); b32 = np.array([[7., 8.], [9., 10.], [11., 12.]])
+    assert np.array_equal(run_dgemm(a23, b32), [[58, 64], [139, 154]])
+    assert np.array_equal(run_dgemm(run_dgemm(a, b), a), [[85, 126], [193, 286]])
+    assert np.array_equal(run_dgemm(np.arange(6.).reshape(2, 3), np.arange(6.).reshape(3, 2)), [[10, 13], [28, 40]])
+    assert run_dgemm(np.ones((1, 100)), np.arange(100.).reshape(100, 1))[0, 0] == 4950.0
+    for n in (4, 8, 10, 16, 32, 46, 47, 49, 50, 51, 53, 64, 100, 192):
+        assert np.all(run_dgemm(np.ones((n, n)), np.ones((n, n))) == float(n)), n
+    S = np.arange(2500.).reshape(50, 50)
+    assert np.array_equal(run_dgemm(S, np.eye(50)), S)
+    R = np.repeat(np.arange(1., 51.)[:, None], 50, axis=1)
+    assert np.array_equal(run_dgemm(R, np.ones((50, 50)))[:, 0], 50.0 * np.arange(1, 51))
+
+
+def test_nonsquare_tile_edges_config2b_reduced(gpu):
+    # configuration 2b is M=8192, N=1024, K=8192; same aspect at a size the oracle finishes
+    A, B = synth.normal(7, (1024, 1024)), synth.normal(8, (1024, 128))
+    assert normwise(run_dgemm(A, B), oracle.matmul_f64(A, B), A, B) <= TOL
+
+
+@pytest.mark.parametrize("M,K,N", [(8192, 8192, 8192), (8192, 8192, 1024)])
+def test_full_size_properties(gpu, M, K, N):
+    """Configuration 2 at full size: exact integer identities that hold for any
+    summation order, plus sampled rows and columns against the oracle."""
+    print("dgemm full", M, K, N, flush=True)
+    i = np.arange(M * K, dtype=np.int64).reshape(M, K)
+    j = np.arange(K * N, dtype=np.int64).reshape(K, N)
+    A = ((i * 7 + i // K) % 7 - 3).astype(np.float64)
+    B = ((j * 5 + j // N) % 5 - 2).astype(np.float64)
+    Cg = run_dgemm(A, B)
+    # checksum of checksums: all quantities are integers far below 2^53
+    assert np.array_equal(Cg.sum(axis=1), A @ B.sum(axis=1))
+    assert np.array_equal(Cg.sum(axis=0), A.sum(axis=0) @ B)
+    rows = [0, 1, 127, 128, 4095, M - 129, M - 1]
+    cols = [0, 1, 127, 128, 777, N - 129, N - 1]
+    assert np.array_equal(Cg[rows][:, cols], A[rows] @ B[:, cols])
+    # real-valued inputs of the configuration, sampled block against the oracle
+    A, B = synth.normal(11, (M, K)), synth.normal(12, (K, N))
+    Cg = run_dgemm(A, B)
+    ref = oracle.matmul_f64(A[rows], B[:, cols])
+    assert normwise(Cg[rows][:, cols], ref, A[rows], B[:, cols]) <= TOL

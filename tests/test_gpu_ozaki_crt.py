@@ -1,0 +1,138 @@
+"""Ozaki-II CRT exact tier on the GPU, stage by stage against the oracle.
+Bars (BASELINE.json): int8 residue planes and residue products bit-exact;
+C within 2 ulp per element of the reference statement of the tier."""
+import numpy as np
+import pytest
+
+import oracle
+from eshkol_amd import synth
+from gpu_util import run_crt, ulp_distance
+from test_oracle_ozaki import regimes
+
+pytestmark = pytest.mark.gpu
+MAX_ULP = 2
+
+
+def check_all_stages(A, B, num_moduli=16, adaptive=False):
+    rc, Cg, st = run_crt(A, B, num_moduli, adaptive)
+    assert rc == 0
+    so = oracle.ozaki_crt_stages(A, B, num_moduli, adaptive)
+    assert st["num_moduli"] == so["num_moduli"] and st["E"] == so["E"]
+    assert np.array_equal(st["mu"], so["mu"]) and np.array_equal(st["nu"], so["nu"])
+    assert np.array_equal(st["a_planes"], so["a_planes"])          # bit-exact residues
+    assert np.array_equal(st["b_planes"], so["b_planes"])
+    assert st["a_pad_clear"] and st["b_pad_clear"]
+    assert np.array_equal(st["w_planes"], so["w_planes"])          # bit-exact residue products
+    assert ulp_distance(Cg, so["C"]).max() <= MAX_ULP
+    return Cg, so
+
+
+SHAPES = [(1, 1, 1), (5, 3, 4), (64, 128, 64), (100, 200, 90), (257, 129, 255), (300, 1000, 17),
+          (512, 512, 512), (33, 2049, 65), (768, 640, 1024)]
+
+
+@pytest.mark.parametrize("M,K,N", SHAPES)
+def test_wide_range_inputs_all_stages(gpu, M, K, N):
+    print("crt", M, K, N, flush=True)
+    A = synth.wide_range(300 + M, (M, K))          # configuration 3's input law
+    B = synth.wide_range(400 + N, (K, N))
+    check_all_stages(A, B)
+
+
+def test_zero_rows_columns_and_negative_zero(gpu):
+    A = synth.normal(1, (70, 90)); B = synth.normal(2, (90, 50))
+    A[3, :] = 0.0; A[10, :] = -0.0; B[:, 7] = 0.0; A[20, 5] = 0.0; B[4, 4] = -0.0
+    A[30, :] = 2.0 ** -600; B[:, 9] = 2.0 ** 500       # extreme but representable scales
+    Cg, so = check_all_stages(A, B)
+    assert np.all(Cg[3] == 0.0) and np.all(Cg[:, 7] == 0.0)
+
+
+@pytest.mark.parametrize("n", [2, 3, 7, 12, 15, 16])
+def test_moduli_counts(gpu, n):
+    A, B = synth.normal(3, (96, 160)), synth.normal(4, (160, 80))
+    check_all_stages(A, B, num_moduli=n)
+
+
+def test_adaptive_moduli_selection(gpu):
+    A = 1.0 + synth.uniform(40, (64, 8), 0.0, 0.4)
+    B = 1.0 + synth.uniform(41, (8, 64), 0.0, 0.4)
+    _, so = check_all_stages(A, B, adaptive=True)
+    assert so["num_moduli"] < 16
+
+
+def test_reference_gate_regimes(gpu):
+    # tests/gpu/ozaki_correctness_test.esk:33-90: four regimes, per-element rel < 1e-9 on a 5x5 grid
+    for n in (512, 1024):
+        for A, B in regimes(n):
+            rc, Cg, _ = run_crt(A, B, want_stages=False)
+            assert rc == 0
+            grid = [int(p * (n - 1) / 4) for p in range(5)]
+            ref = A[grid].astype(np.longdouble) @ B[:, grid].astype(np.longdouble)
+            got = Cg[grid][:, grid]
+            denom = np.where(np.abs(ref) > 1e-9, np.abs(ref), 1.0)     # the reference test's denominator
+            assert np.all(np.abs(got - ref) / denom < 1e-9)
+
+
+def test_certification_witness(gpu):
+    # tests/gpu/ozaki_certification_test.esk:14-106
+    n = 512
+    r = np.arange(n, dtype=np.int64)[:, None]
+    c = np.arange(n, dtype=np.int64)[None, :]
+    a = (16777216 + ((97 * r + 53 * c) % 257)) * np.where((131 * r + 13 * c) % 2 == 0, 1, -1)
+    b = (16777216 + ((71 * r + 29 * c + r * c) % 257)) * np.where((73 * r + 23 * c) % 2 == 0, 1, -1)
+    exact = a @ b
+    Cg, _ = check_all_stages(a.astype(np.float64), b.astype(np.float64))
+    pts = [0, 128, 256, 384, 511]
+    for i in pts:
+        for j in pts:
+            assert Cg[i, j] == float(int(exact[i, j]))
+
+
+def test_rejects_what_the_tier_cannot_represent(gpu):
+    A = np.ones((8, 8)); B = np.ones((8, 8))
+    for bad in (np.nan, np.inf, -np.inf):
+        A2 = A.copy(); A2[2, 3] = bad
+        assert run_crt(A2, B)[0] == -1
+        B2 = B.copy(); B2[5, 1] = bad
+        assert run_crt(A, B2)[0] == -1
+    assert run_crt(A * 1e-300, B)[0] == -1                      # 2^mu outside the double range
+    A3 = A.copy(); A3[4, :] = 5e-324                            # subnormal row: same
+    assert run_crt(A3, B)[0] == -1
+    assert run_crt(np.ones((2, 131072)), np.ones((131072, 2)))[0] == -1   # int32-exact bound on K
+
+
+def test_fused_bias_tanh_epilogue(gpu):
+    X = synth.normal(50, (96, 200)); W = synth.xavier_uniform(51, 200, 72)
+    b = synth.uniform(52, (72,), -0.1, 0.1)
+    rc, Y, _ = run_crt(X, W, bias=b, act=1, want_stages=False)
+    assert rc == 0
+    expect = oracle.mlp_layer(X, W, b)
+    assert np.abs(Y - expect).max() <= 4 * np.finfo(np.float64).eps    # device tanh vs glibc tanh
+    rc, Y0, _ = run_crt(X, W, bias=b, act=0, want_stages=False)
+    assert np.array_equal(Y0, oracle.matmul_ozaki_crt(X, W) + b[None, :])
+
+
+def test_full_size_config3_sampled(gpu):
+    """Configuration 3 at 8192^3: sampled residue products recomputed from the
+    device's own planes with exact integers, and a sampled block of C against the
+    oracle run on the same rows and columns (mu, nu depend only on the row or
+    column; E is clamped to 52 at this K for both)."""
+    n = 8192
+    print("crt full", n, flush=True)
+    A = synth.wide_range(31, (n, n)); B = synth.wide_range(32, (n, n))
+    rc, Cg, st = run_crt(A, B)
+    assert rc == 0 and st["E"] == 52 and st["num_moduli"] == 16
+    rows = [0, 1, 255, 256, 4097, n - 257, n - 1]
+    cols = [0, 3, 255, 256, 5000, n - 256, n - 1]
+    so = oracle.ozaki_crt_stages(A[rows], B[:, cols])
+    assert so["E"] == 52
+    assert np.array_equal(st["mu"][rows], so["mu"]) and np.array_equal(st["nu"][cols], so["nu"])
+    assert np.array_equal(st["a_planes"][:, rows, :], so["a_planes"])
+    assert np.array_equal(st["b_planes"][:, cols, :], so["b_planes"])
+    for l, p in enumerate(oracle.MODULI):
+        acc = st["a_planes"][l][rows].astype(np.int64) @ st["b_planes"][l][cols].astype(np.int64).T
+        w = st["w_planes"][l][rows][:, cols].astype(np.int64)
+        assert np.all((acc - w) % p == 0) and w.min() >= -(p // 2) and w.max() <= (p - 1) // 2
+    assert np.array_equal(st["w_planes"][:, rows][:, :, cols], so["w_planes"])
+    assert ulp_distance(Cg[rows][:, cols], so["C"]).max() <= MAX_ULP
+    assert st["a_pad_clear"] and st["b_pad_clear"]

@@ -1,0 +1,96 @@
+"""Reduced-precision tier on the GPU. Bar (BASELINE.json): normwise error
+<= 1e-2 against the reference's reduced tier, whose CPU statement is the f64
+GEMM over operands already rounded to the 16-bit type."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import eshkol_amd as ea
+import oracle
+from eshkol_amd import synth
+from gpu_util import normwise, run_reduced, stream
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+@pytest.mark.parametrize("dtype", [2, 3])
+@pytest.mark.parametrize("M,K,N", [(1, 1, 1), (5, 3, 4), (64, 128, 64), (100, 200, 90), (257, 129, 255),
+                                   (512, 512, 512), (33, 2049, 65), (1024, 768, 640)])
+def test_reduced_matches_reference_statement(gpu, M, K, N, dtype):
+    print("reduced", M, K, N, dtype, flush=True)
+    A = synth.normal(700 + M, (M, K), 1.0 / np.sqrt(K))      # configuration 4's input law
+    B = synth.normal(800 + N, (K, N), 1.0 / np.sqrt(K))
+    # The runtime hands this tier tensors whose f64 storage was already rounded to the
+    # 16-bit type when they were created (runtime_tensor_dtype.cpp:194-229).
+    Ar, Br = oracle.reduce_precision(A, dtype), oracle.reduce_precision(B, dtype)
+    ref = oracle.matmul_f64(Ar, Br)
+    assert np.array_equal(ref, oracle.matmul_reduced(A, B, dtype))
+    wide = run_reduced(Ar, Br, dtype, round_output=False)
+    assert normwise(wide, ref, Ar, Br) <= 1e-6               # fp32 accumulation only
+    narrow = run_reduced(Ar, Br, dtype, round_output=True)   # what the reference's 16F output does
+    assert normwise(narrow, ref, Ar, Br) <= TOL
+    ok = (np.abs(wide) >= 2.0 ** -14) | (wide == 0)         # outside the reference's f16 subnormal quirk
+    assert np.array_equal(narrow[ok], oracle.reduce_precision(wide, dtype)[ok])
+    if dtype == 3:
+        # fp32 accumulation order is unspecified; the sum is close to a k-ascending one
+        assert normwise(wide, oracle.matmul_reduced_f32acc(A, B, dtype, False), Ar, Br) <= 1e-6
+
+
+@pytest.mark.parametrize("is_bf16", [0, 1])
+def test_device_narrowing_is_round_to_nearest_even(gpu, is_bf16):
+    lib = ea.load()
+    rows, cols, rp, ld = 37, 150, 256, 192
+    x = np.concatenate([synth.normal(1, (3000,)), synth.normal(2, (1500,)) * 300.0,
+                        synth.normal(3, (1000,)) * 1e-3, np.array([0.0, -0.0, 1.0009765625, 65504.0, 65520.0, 1e6])])
+    x = np.resize(x, rows * cols).reshape(rows, cols)
+    d_in = ea.DeviceArray.from_host(x)
+    d_out = ea.DeviceArray((rp, ld), np.uint16)
+    assert lib.hip_convert_f64_to_16(d_in.ptr, d_out.ptr, rows, cols, rp, ld, is_bf16, stream()) == 0
+    ea.synchronize()
+    got = d_out.download()
+    assert not got[rows:].any() and not got[:, cols:].any()
+    bits = got[:rows, :cols]
+    if is_bf16:
+        val = (bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    else:
+        val = bits.view(np.float16).astype(np.float64)
+    normal_range = (np.abs(x) >= 2.0 ** -14) | (x == 0)
+    expect = oracle.reduce_precision(x, 3 if is_bf16 else 2)
+    assert np.array_equal(val[normal_range], expect[normal_range])
+    assert np.array_equal(np.signbit(val), np.signbit(expect))
+
+
+def test_hgemm_fp32_output_config4_reduced_size(gpu):
+    """The contraction alone, bf16 in / fp32 out (configuration 4 at 1024^3)."""
+    lib = ea.load()
+    n = 1024
+    A = synth.normal(4, (n, n), 1.0 / np.sqrt(n)); B = synth.normal(5, (n, n), 1.0 / np.sqrt(n))
+    dA, dBt = ea.DeviceArray.from_host(A), ea.DeviceArray.from_host(np.ascontiguousarray(B.T))
+    a16, b16 = ea.DeviceArray((n, n), np.uint16), ea.DeviceArray((n, n), np.uint16)
+    assert lib.hip_convert_f64_to_16(dA.ptr, a16.ptr, n, n, n, n, 1, stream()) == 0
+    assert lib.hip_convert_f64_to_16(dBt.ptr, b16.ptr, n, n, n, n, 1, stream()) == 0
+    dC = ea.DeviceArray((n, n), np.float32)
+    assert lib.hip_hgemm_16(a16.ptr, b16.ptr, n, n, n, n, 1, dC.ptr, stream()) == 0
+    ea.synchronize()
+    Cg = dC.download().astype(np.float64)
+    Ar, Br = oracle.reduce_precision(A, 3), oracle.reduce_precision(B, 3)
+    assert normwise(Cg, oracle.matmul_f64(Ar, Br), Ar, Br) <= 1e-6
+
+
+def test_full_size_config4_sampled(gpu):
+    n = 8192
+    print("reduced full", n, flush=True)
+    A = synth.normal(61, (n, n), 1.0 / np.sqrt(n)); B = synth.normal(62, (n, n), 1.0 / np.sqrt(n))
+    Cg = run_reduced(A, B, 3, round_output=False)
+    rows = [0, 1, 255, 256, 4097, n - 257, n - 1]
+    cols = [0, 3, 255, 256, 5000, n - 256, n - 1]
+    Ar, Br = oracle.reduce_precision(A[rows], 3), oracle.reduce_precision(B[:, cols], 3)
+    assert normwise(Cg[rows][:, cols], oracle.matmul_f64(Ar, Br), Ar, Br) <= TOL
+    # linearity in exact arithmetic: small integers are exact in bf16 and in fp32 sums
+    i = np.arange(n * n, dtype=np.int64).reshape(n, n)
+    Ai = ((i * 7 + i // n) % 7 - 3).astype(np.float64); Bi = ((i * 5 + i // n) % 5 - 2).astype(np.float64)
+    Ci = run_reduced(Ai, Bi, 3, round_output=False)
+    assert np.array_equal(Ci.sum(axis=1), Ai @ Bi.sum(axis=1))
+    assert np.array_equal(Ci[rows][:, cols], Ai[rows] @ Bi[:, cols])
