@@ -1,0 +1,250 @@
+#!/usr/bin/env python3
+"""Benchmark of the tensor-matmul GPU hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--size 8192] [--no-cpu] [--no-stages]
+
+Prints ONE JSON line. A step is one GEMM C = A*B with operands resident in HBM;
+work is counted as 2*M*N*K flop whatever the tier does internally (the
+reference's convention, benchmarks/gpu_matmul_bench.sh:147-148).
+
+  value      native fp64 tier (hip_dgemm_f64) at M=N=K=8192, N(0,1) inputs:
+             BASELINE.json configuration 2, the one its metric is quoted on
+  roofline   that kernel against the fp64 matrix-core peak; the duration is
+             measured here with HIP events on the library's stream
+  tiers      the other tiers of the metric at the same size, each with its own
+             configuration's input law, plus the HBM-bound stages of the exact
+             tier against the HBM peak
+  cpu_baseline  the reference's CPU matmul (compiled from its sources into
+             oracle/_ref when available, else the oracle's port) on one host
+             core, on a bounded sample
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK = {"fp64_mfma": 78.6e12, "int8_mfma": 5.0e15, "bf16_mfma": 2.5e15, "hbm": 8.0e12}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def read_traffic(name):
+    """HBM bytes per launch from the committed rocprofv3 --pmc summary, if any."""
+    path = os.path.join(ROOT, "profiles", name)
+    if not os.path.exists(path):
+        return None
+    vals = {}
+    for line in open(path):
+        if "=" in line and not line.lstrip().startswith("#"):
+            k, v = line.split("=", 1)
+            try:
+                vals[k.strip()] = float(v.split()[0])
+            except ValueError:
+                pass
+    if "HBM_BYTES_PER_LAUNCH" in vals:
+        return vals["HBM_BYTES_PER_LAUNCH"]
+    return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--size", type=int, default=8192)
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-stages", action="store_true")
+    ap.add_argument("--only", default="", help="comma list of tiers to time besides native: crt,int8,reduced")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this build measures one GPU only (the path shards by rows of A with no "
+                 "exchange; see DESIGN.md). Run with --gpus 1.")
+
+    import eshkol_amd as ea
+    from eshkol_amd import synth
+    lib = ea.init()
+    hip = ea.hip_runtime()
+    st = lib.eshkol_hip_get_stream()
+    n = args.size
+    M = K = N = n
+    flops = 2.0 * M * N * K
+    steps, warm = args.steps, args.warmup
+    timer = ea.Timer()
+    want = set(args.only.split(",")) if args.only else {"crt", "int8", "reduced"}
+
+    def timed(fn, k=steps, w=warm):
+        """w untimed calls, then k calls bracketed by device syncs and HIP events
+        on the library stream. Returns (ms per call by events, ms per call by wall clock)."""
+        for _ in range(w):
+            rc = fn()
+            assert rc == 0, rc
+        hip.hipDeviceSynchronize()
+        t0 = time.perf_counter()
+        timer.start()
+        for _ in range(k):
+            fn()
+        ev_ms = timer.stop()
+        hip.hipDeviceSynchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3
+        return ev_ms / k, wall_ms / k
+
+    # ---- native fp64 tier: configuration 2 ------------------------------------
+    log("generating N(0,1) operands %dx%d" % (n, n))
+    A = synth.normal(11, (M, K))
+    B = synth.normal(12, (K, N))
+    dA, dB, dC = ea.DeviceArray.from_host(A), ea.DeviceArray.from_host(B), ea.DeviceArray((M, N))
+    ev_ms, wall_ms = timed(lambda: lib.hip_dgemm_f64(dA.ptr, dB.ptr, dC.ptr, M, K, N, st))
+    native_gflops = flops / (wall_ms * 1e-3) / 1e9
+    achieved = flops / (ev_ms * 1e-3)
+    log("native fp64: %.3f ms/step (events %.3f ms) %.1f GFLOP/s" % (wall_ms, ev_ms, native_gflops))
+    roofline = {"bound": "mfma", "kernel": "dgemm_mfma_kernel<128,128>",
+                "achieved": achieved / 1e12, "peak": PEAK["fp64_mfma"] / 1e12, "unit": "TFLOP/s",
+                "frac": achieved / PEAK["fp64_mfma"], "launch_ms": ev_ms,
+                "traffic": read_traffic("dgemm_mfma_8192_hbm_traffic.txt")}
+    tiers = {"native_fp64": {"ms": wall_ms, "gflops": native_gflops, "frac_of_peak": achieved / PEAK["fp64_mfma"],
+                             "peak": "fp64 MFMA 78.6 TFLOP/s"}}
+
+    # non-square case of configuration 2 (tile edges)
+    N2 = max(n // 8, 1)
+    dB2, dC2 = ea.DeviceArray.from_host(np.ascontiguousarray(B[:, :N2])), ea.DeviceArray((M, N2))
+    e2, w2 = timed(lambda: lib.hip_dgemm_f64(dA.ptr, dB2.ptr, dC2.ptr, M, K, N2, st))
+    tiers["native_fp64_%dx%dx%d" % (M, N2, K)] = {"ms": w2, "gflops": 2.0 * M * N2 * K / (w2 * 1e-3) / 1e9,
+                                                   "frac_of_peak": 2.0 * M * N2 * K / (e2 * 1e-3) / PEAK["fp64_mfma"]}
+    dB2.free(); dC2.free()
+
+    # ---- Ozaki-II CRT exact tier: configuration 3 --------------------------------
+    if "crt" in want:
+        log("generating wide-range operands")
+        Aw = synth.wide_range(31, (M, K))
+        Bw = synth.wide_range(32, (K, N))
+        dA.upload(Aw); dB.upload(Bw)
+        devnull = os.open(os.devnull, os.O_WRONLY)
+        saved = os.dup(2)
+        os.dup2(devnull, 2)                 # the tier prints one marker line per call
+        try:
+            e3, w3 = timed(lambda: lib.hip_matmul_ozaki_crt_f64(dA.ptr, dB.ptr, dC.ptr, M, K, N, 16, 0, None, 0, st))
+        finally:
+            os.dup2(saved, 2)
+        tiers["ozaki_crt_exact_16_moduli"] = {
+            "ms": w3, "gflops_fp64_equiv": flops / (w3 * 1e-3) / 1e9,
+            "vs_native": (flops / (w3 * 1e-3) / 1e9) / native_gflops}
+        log("ozaki crt: %.3f ms/step %.1f GFLOP/s-eq" % (w3, flops / (w3 * 1e-3) / 1e9))
+
+        if not args.no_stages:
+            nmod = 16
+            Mp, ldk = (M + 255) // 256 * 256, (K + 255) // 256 * 256
+            sg = ea.HipOzakiCrtStages()
+            assert lib.hip_ozaki_crt_last_stages(C.byref(sg)) == 0
+            # split: 8*M*K read + nmod*M*K written
+            e, _ = timed(lambda: lib.hip_ozaki_crt_split_f64(dA.ptr, M, K, sg.mu, nmod, sg.a_planes, Mp, ldk, st))
+            split_bytes = 8.0 * M * K + nmod * M * K
+            # contraction: nmod int8 GEMMs
+            ga = ea.HipIgemmArgs()
+            tables = np.concatenate([np.arange(17), np.arange(16), np.array([256, 255, 253, 251, 247, 241, 239, 233,
+                                     229, 227, 223, 217, 211, 199, 197, 193])]).astype(np.int32)
+            dT = ea.DeviceArray.from_host(tables)
+            ga.a_planes, ga.b_planes = sg.a_planes, sg.b_planes
+            ga.a_plane_stride, ga.b_plane_stride = Mp * ldk, sg.rows_b_padded * ldk
+            ga.ldk, ga.M, ga.N, ga.n_out = ldk, M, N, nmod
+            ga.pair_first, ga.pair_a, ga.pair_b = dT.ptr, dT.ptr + 17 * 4, dT.ptr + 17 * 4
+            ga.mode, ga.modulus, ga.out_i8 = 1, dT.ptr + 33 * 4, sg.w_planes
+            ga.max_pairs = 1
+            eg, _ = timed(lambda: lib.hip_igemm_i8(C.byref(ga), st))
+            # reconstruct: nmod*M*N read + 8*M*N written
+            ones = (C.c_double * 16)(*([1.0] * 16))
+            er, _ = timed(lambda: lib.hip_ozaki_crt_reconstruct_f64(sg.w_planes, M, N, nmod, ones, ones, 1.0, 0.0, 1.0,
+                                                                     sg.mu, sg.nu, None, 0, dC.ptr, st))
+            rec_bytes = float(nmod) * M * N + 8.0 * M * N
+            tiers["ozaki_crt_exact_16_moduli"]["stages"] = {
+                "split_A": {"ms": e, "GBps": split_bytes / (e * 1e-3) / 1e9, "frac_of_hbm": split_bytes / (e * 1e-3) / PEAK["hbm"],
+                            "algorithmic_bytes": split_bytes},
+                "int8_contraction": {"ms": eg, "TOPs": nmod * flops / (eg * 1e-3) / 1e12,
+                                     "frac_of_int8_peak": nmod * flops / (eg * 1e-3) / PEAK["int8_mfma"]},
+                "reconstruct": {"ms": er, "GBps": rec_bytes / (er * 1e-3) / 1e9, "frac_of_hbm": rec_bytes / (er * 1e-3) / PEAK["hbm"],
+                                "algorithmic_bytes": rec_bytes}}
+            dT.free()
+        del Aw, Bw
+
+    # ---- INT8 slice tier, T = 6 -----------------------------------------------------
+    if "int8" in want:
+        dA.upload(A); dB.upload(B)
+        e4, w4 = timed(lambda: lib.hip_matmul_ozaki_int8_f64(dA.ptr, dB.ptr, dC.ptr, M, K, N, 6, st),
+                       k=max(3, steps // 2), w=2)
+        tiers["ozaki_int8_slices_T6"] = {"ms": w4, "gflops_fp64_equiv": flops / (w4 * 1e-3) / 1e9,
+                                         "vs_native": (flops / (w4 * 1e-3) / 1e9) / native_gflops,
+                                         "int8_TOPs": 28 * flops / (e4 * 1e-3) / 1e12}
+        log("ozaki int8 T=6: %.3f ms/step %.1f GFLOP/s-eq" % (w4, flops / (w4 * 1e-3) / 1e9))
+
+    # ---- reduced tier: configuration 4 ---------------------------------------------------
+    if "reduced" in want:
+        log("generating N(0,1/sqrt(K)) operands")
+        Ar = synth.normal(61, (M, K), 1.0 / np.sqrt(K))
+        Br = synth.normal(62, (K, N), 1.0 / np.sqrt(K))
+        dA.upload(Ar); dB.upload(Br)
+        e5, w5 = timed(lambda: lib.hip_matmul_reduced_f64(dA.ptr, dB.ptr, dC.ptr, M, K, N, 3, 0, st))
+        # the contraction alone on bf16 operands already in HBM, fp32 output
+        ld = (K + 63) // 64 * 64
+        Mp, Np = (M + 255) // 256 * 256, (N + 255) // 256 * 256
+        a16, b16 = ea.DeviceArray((Mp, ld), np.uint16), ea.DeviceArray((Np, ld), np.uint16)
+        dBt = ea.DeviceArray((N, K))
+        assert lib.hip_transpose_f64(dB.ptr, dBt.ptr, K, N, st) == 0
+        assert lib.hip_convert_f64_to_16(dA.ptr, a16.ptr, M, K, Mp, ld, 1, st) == 0
+        assert lib.hip_convert_f64_to_16(dBt.ptr, b16.ptr, N, K, Np, ld, 1, st) == 0
+        dC32 = ea.DeviceArray((M, N), np.float32)
+        e6, w6 = timed(lambda: lib.hip_hgemm_16(a16.ptr, b16.ptr, M, K, N, ld, 1, dC32.ptr, st))
+        tiers["reduced_bf16_fp32acc"] = {
+            "f64_storage_in_out": {"ms": w5, "gflops": flops / (w5 * 1e-3) / 1e9},
+            "bf16_in_fp32_out": {"ms": w6, "gflops": flops / (w6 * 1e-3) / 1e9,
+                                 "frac_of_bf16_peak": flops / (e6 * 1e-3) / PEAK["bf16_mfma"]}}
+        log("reduced bf16: %.3f ms (f64 storage), %.3f ms (bf16 operands)" % (w5, w6))
+        for d in (a16, b16, dBt, dC32):
+            d.free()
+        del Ar, Br
+
+    # ---- CPU baseline on one host core ---------------------------------------------------------
+    cpu = None
+    if not args.no_cpu:
+        import oracle
+        dp = C.POINTER(C.c_double)
+        if os.path.exists(oracle.REF_PATH):
+            ref = C.CDLL(oracle.REF_PATH)
+            ref.eshkol_matmul_f64.argtypes = [dp, dp, dp, C.c_uint64, C.c_uint64, C.c_uint64]
+            m = min(4096, n)
+            kind, call = "reference", lambda a, b, c: ref.eshkol_matmul_f64(a, b, c, m, m, m)
+        else:
+            L = oracle.lib()
+            L.oracle_matmul_f64.argtypes = [dp, dp, dp, C.c_uint64, C.c_uint64, C.c_uint64]
+            m = min(2048, n)
+            kind, call = "port", lambda a, b, c: L.oracle_matmul_f64(a, b, c, m, m, m)
+        As = np.ascontiguousarray(A[:m, :m]); Bs = np.ascontiguousarray(B[:m, :m]); Cs = np.empty((m, m))
+        log("cpu baseline (%s), %d^3 on one core" % (kind, m))
+        t0 = time.perf_counter()
+        call(As.ctypes.data_as(dp), Bs.ctypes.data_as(dp), Cs.ctypes.data_as(dp))
+        dt = time.perf_counter() - t0
+        cpu = {"value": 2.0 * m ** 3 / dt / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": kind,
+               "sample": "eshkol_matmul_f64 (AVX2+FMA 4x8 kernel, 64^3 blocking), top-left %d^3 block of the "
+                         "same operands, one run, %.1f s" % (m, dt)}
+
+    out = {
+        "metric": "fp64-equiv GFLOP/s per GEMM tier at 8192^3 on 1 MI355X; % of MFMA peak",
+        "value": native_gflops, "unit": "GFLOP/s", "n_gpus": 1, "steps": steps, "warmup": warm,
+        "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f64", "data": "synthetic",
+        "config": {"workload": "native fp64 tier, C=A*B, M=N=K=%d, A,B ~ N(0,1) from seed, row-major dense, "
+                               "operands resident in HBM" % n},
+        "roofline": roofline, "cpu_baseline": cpu, "tiers": tiers,
+    }
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

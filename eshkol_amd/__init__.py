@@ -36,7 +36,7 @@ class HipIgemmArgs(C.Structure):
     _fields_ = [("a_planes", vp), ("b_planes", vp), ("a_plane_stride", u64), ("b_plane_stride", u64),
                 ("ldk", u32), ("M", u32), ("N", u32), ("n_out", u32),
                 ("pair_first", vp), ("pair_a", vp), ("pair_b", vp),
-                ("mode", i32), ("modulus", vp), ("out_i32", vp), ("out_i8", vp)]
+                ("mode", i32), ("max_pairs", i32), ("modulus", vp), ("out_i32", vp), ("out_i8", vp)]
 
 
 class HipOzakiCrtStages(C.Structure):

@@ -10,158 +10,74 @@
  * MFMA operands are 16-byte LDS reads along K; which k each lane feeds does not
  * matter as long as both operands agree, because the int32 sum is exact.
  *
- * Work decomposition
- *   workgroup  WGM x WGN waves, block tile (WGM*TM*32) x (WGN*TN*32), BK = 64 bytes
- *   wave       TM x TN MFMA tiles of 32x32, int32 accumulators in registers
- *   LDS        double-buffered [rows][64(+16)] bytes per operand; the 16-byte pad
- *              spreads the 16-byte reads of 16 consecutive rows over all banks
- *   operands   the B fragment is passed as the MFMA's first operand, so a lane
- *              ends up with 4 consecutive columns of one output row and can
- *              store them as one word (int8) or one 16-byte vector (int32)
- *   epilogue   mode 1 reduces modulo p in fp64 (exact: |sum| < 2^31), stages
- *              the int8 tile through LDS and writes whole 16-byte chunks
+ * Two kernels share the tile mapping and the epilogue:
+ *   pipelined  256x256 tile, 128-byte k-blocks, register-ring prefetch
+ *              (gemm_pipe.h); used when the launch fills the chip and the row
+ *              pitch is a multiple of 256 bytes
+ *   simple     128x128 tile, 64-byte k-blocks, one block in flight; small or
+ *              oddly padded problems
  *
- * One launch covers every output plane: the flattened workgroup id is remapped
- * so each XCD works through whole planes, 8 tile-rows at a time, and the
- * workgroups resident together share operand rows in that XCD's L2.
+ * The B fragment is passed as the MFMA's first operand, so a lane ends up with
+ * 4 consecutive columns of one output row and stores them as one word (int8)
+ * or one 16-byte vector (int32). Mode 1 reduces modulo p in fp64 (exact:
+ * |sum| < 2^31), stages the int8 tile through LDS and writes 16-byte chunks.
+ *
+ * One launch covers every output plane. Workgroup ids congruent mod 8 run on
+ * the same XCD; the id is remapped so that XCD x owns the x-th eighth of every
+ * plane's tiles (8 tile-rows at a time inside it). All XCDs then carry the same
+ * work whatever the per-plane cost, and the workgroups resident together on an
+ * XCD share operand rows in its L2.
  */
 #include "hip_common.h"
 #include "kernels.h"
+#include "gemm_pipe.h"
 
 typedef int v4i_t __attribute__((ext_vector_type(4)));
 typedef int v16i_t __attribute__((ext_vector_type(16)));
 
 namespace {
 
-constexpr int BKB = 64;            /* bytes of K per block */
-constexpr int LDS_PITCH = BKB + 16;
-
-template <int WGM, int WGN, int TM, int TN> struct Cfg {
-    static constexpr int NT = 64 * WGM * WGN;
-    static constexpr int BM = WGM * TM * 32;
-    static constexpr int BN = WGN * TN * 32;
-    static constexpr int A_TILE = BM * LDS_PITCH;
-    static constexpr int B_TILE = BN * LDS_PITCH;
-    static constexpr int SMEM_MAIN = 2 * (A_TILE + B_TILE);
-    static constexpr int SMEM_EPI = BM * (BN + 16);
-    static constexpr int SMEM_BYTES = SMEM_MAIN > SMEM_EPI ? SMEM_MAIN : SMEM_EPI;
-    static constexpr int A_CHUNKS = BM * BKB / 16 / NT;
-    static constexpr int B_CHUNKS = BN * BKB / 16 / NT;
-    static_assert(BM * BKB / 16 % NT == 0 && BN * BKB / 16 % NT == 0, "tile/thread mismatch");
+struct I8Op {
+    typedef v16i_t acc_t;
+    static __device__ __forceinline__ void mfma(const v4i_t& first, const v4i_t& second, v16i_t& acc) {
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(first, second, acc, 0, 0, 0);
+    }
 };
 
-template <int WGM, int WGN, int TM, int TN>
-__global__ __launch_bounds__(64 * WGM * WGN)
-void igemm_i8_kernel(HipIgemmArgs g, int tiles_m, int tiles_n) {
-    using C = Cfg<WGM, WGN, TM, TN>;
-    extern __shared__ __align__(16) int8_t smem_i8[];
-    int8_t* As = smem_i8;
-    int8_t* Bs = smem_i8 + 2 * C::A_TILE;
+/* workgroup -> (output plane, tile); false for the padding workgroups of an XCD */
+__device__ __forceinline__ bool map_workgroup(int tiles_m, int tiles_n, int n_out, int chunk,
+                                              int* o, int* tm, int* tn) {
+    const int wg = blockIdx.x;
+    const int xcd = wg & 7, seq = wg >> 3;
+    const int per_plane = tiles_m * tiles_n;
+    /* planes from last to first: in the slice tier later planes sum more products */
+    *o = n_out - 1 - seq / chunk;
+    const int in_plane = xcd * chunk + seq % chunk;
+    if (in_plane >= per_plane) return false;
+    const int GM = 8;
+    const int width = GM * tiles_n;
+    const int group = in_plane / width;
+    const int first_m = group * GM;
+    const int gsize = (tiles_m - first_m < GM) ? tiles_m - first_m : GM;
+    const int in_group = in_plane - group * width;
+    *tm = first_m + in_group % gsize;
+    *tn = in_group / gsize;
+    return true;
+}
 
-    /* workgroup -> (output plane, tile) */
-    int o, tm, tn;
-    {
-        const int nwg = gridDim.x, wg = blockIdx.x;
-        const int q = nwg >> 3, r = nwg & 7;
-        const int xcd = wg & 7, seq = wg >> 3;
-        const int L = xcd * q + (xcd < r ? xcd : r) + seq;
-        const int per_plane = tiles_m * tiles_n;
-        o = L / per_plane;
-        const int in_plane = L - o * per_plane;
-        const int GM = 8;
-        const int width = GM * tiles_n;
-        const int group = in_plane / width;
-        const int first_m = group * GM;
-        const int gsize = (tiles_m - first_m < GM) ? tiles_m - first_m : GM;
-        const int in_group = in_plane - group * width;
-        tm = first_m + in_group % gsize;
-        tn = in_group / gsize;
-    }
-    const int m0 = tm * C::BM, n0 = tn * C::BN;
-
+/* The accumulator is the transposed tile (B was the first operand): lane
+ * column (lane%32) is the output row, registers 4v..4v+3 are output columns
+ * 8v + 4*(lane/32) + 0..3. `stage` is LDS of at least BM*(BN+16) bytes that no
+ * wave is still reading. */
+template <int TM, int TN>
+__device__ __forceinline__ void epilogue(const HipIgemmArgs& g, int o, int m0, int n0,
+                                         v16i_t (&acc)[TM][TN], int8_t* stage) {
+    constexpr int BM = 2 * TM * 32, BN = 2 * TN * 32, NT = 256;
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WGN, wn = wave % WGN;
+    const int wm = wave >> 1, wn = wave & 1;
     const int li = lane & 31, lh = lane >> 5;
 
-    const int pair_lo = g.pair_first[o], pair_hi = g.pair_first[o + 1];
-    const int nkb_per = (int)(g.ldk / BKB);
-    const int nkb = (pair_hi - pair_lo) * nkb_per;
-
-    v4i_t ra[C::A_CHUNKS], rb[C::B_CHUNKS];
-
-    auto gload = [&](int kb) {
-        const int t = pair_lo + kb / nkb_per;
-        const int k0 = (kb % nkb_per) * BKB;
-        const int8_t* Ap = g.a_planes + (size_t)g.pair_a[t] * g.a_plane_stride + (size_t)m0 * g.ldk + k0;
-        const int8_t* Bp = g.b_planes + (size_t)g.pair_b[t] * g.b_plane_stride + (size_t)n0 * g.ldk + k0;
-#pragma unroll
-        for (int r = 0; r < C::A_CHUNKS; r++) {
-            const int c = tid + C::NT * r;
-            ra[r] = *(const v4i_t*)(Ap + (size_t)(c >> 2) * g.ldk + (c & 3) * 16);
-        }
-#pragma unroll
-        for (int r = 0; r < C::B_CHUNKS; r++) {
-            const int c = tid + C::NT * r;
-            rb[r] = *(const v4i_t*)(Bp + (size_t)(c >> 2) * g.ldk + (c & 3) * 16);
-        }
-    };
-    auto sstore = [&](int buf) {
-#pragma unroll
-        for (int r = 0; r < C::A_CHUNKS; r++) {
-            const int c = tid + C::NT * r;
-            *(v4i_t*)(As + buf * C::A_TILE + (c >> 2) * LDS_PITCH + (c & 3) * 16) = ra[r];
-        }
-#pragma unroll
-        for (int r = 0; r < C::B_CHUNKS; r++) {
-            const int c = tid + C::NT * r;
-            *(v4i_t*)(Bs + buf * C::B_TILE + (c >> 2) * LDS_PITCH + (c & 3) * 16) = rb[r];
-        }
-    };
-
-    v16i_t acc[TM][TN];
-#pragma unroll
-    for (int t = 0; t < TM; t++)
-#pragma unroll
-        for (int u = 0; u < TN; u++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[t][u][r] = 0;
-
-    if (nkb > 0) {
-        gload(0);
-        sstore(0);
-    }
-    __syncthreads();
-
-    int cur = 0;
-    for (int kb = 0; kb < nkb; kb++) {
-        const bool more = (kb + 1 < nkb);
-        if (more) gload(kb + 1);
-
-        const int8_t* a_base = As + cur * C::A_TILE + (wm * TM * 32 + li) * LDS_PITCH + lh * 16;
-        const int8_t* b_base = Bs + cur * C::B_TILE + (wn * TN * 32 + li) * LDS_PITCH + lh * 16;
-#pragma unroll
-        for (int ks = 0; ks < BKB / 32; ks++) {
-            v4i_t a[TM], b[TN];
-#pragma unroll
-            for (int t = 0; t < TM; t++) a[t] = *(const v4i_t*)(a_base + t * 32 * LDS_PITCH + ks * 32);
-#pragma unroll
-            for (int u = 0; u < TN; u++) b[u] = *(const v4i_t*)(b_base + u * 32 * LDS_PITCH + ks * 32);
-#pragma unroll
-            for (int t = 0; t < TM; t++)
-#pragma unroll
-                for (int u = 0; u < TN; u++)
-                    acc[t][u] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[u], a[t], acc[t][u], 0, 0, 0);
-        }
-
-        if (more) sstore(cur ^ 1);
-        __syncthreads();
-        cur ^= 1;
-    }
-
-    /* With B as the first operand the accumulator is the transposed tile:
-     * lane column (lane%32) is the output row, and registers 4v..4v+3 are the
-     * output columns 8v + 4*(lane/32) + 0..3. */
     if (g.mode == 0) {
         int32_t* out = g.out_i32 + (size_t)o * g.M * g.N;
         const bool vec_ok = (g.N % 4 == 0);
@@ -193,8 +109,7 @@ void igemm_i8_kernel(HipIgemmArgs g, int tiles_m, int tiles_n) {
     /* mode 1: residues modulo p, staged through LDS */
     const int p = g.modulus[o];
     const double pinv = 1.0 / (double)p;
-    constexpr int EPITCH = C::BN + 16;
-    int8_t* stage = smem_i8;     /* the main loop's last barrier has passed */
+    constexpr int EPITCH = BN + 16;
 #pragma unroll
     for (int t = 0; t < TM; t++) {
         const int lrow = wm * TM * 32 + t * 32 + li;
@@ -217,44 +132,186 @@ void igemm_i8_kernel(HipIgemmArgs g, int tiles_m, int tiles_n) {
             }
     }
     __syncthreads();
-    {
-        int8_t* out = g.out_i8 + (size_t)o * g.M * g.N;
-        const bool vec_ok = (g.N % 16 == 0) && (((uintptr_t)out & 15) == 0);
-        constexpr int CHUNKS_PER_ROW = C::BN / 16;
-        constexpr int TOTAL = C::BM * CHUNKS_PER_ROW;
-        for (int c = tid; c < TOTAL; c += C::NT) {
-            const int lrow = c / CHUNKS_PER_ROW, lc = (c % CHUNKS_PER_ROW) * 16;
-            const int row = m0 + lrow, col = n0 + lc;
-            if (row >= (int)g.M || col >= (int)g.N) continue;
-            const int8_t* src = stage + lrow * EPITCH + lc;
-            int8_t* dst = out + (size_t)row * g.N + col;
-            if (vec_ok && col + 15 < (int)g.N) {
-                *(v4i_t*)dst = *(const v4i_t*)src;
-            } else {
-                for (int e = 0; e < 16 && col + e < (int)g.N; e++) dst[e] = src[e];
-            }
+    int8_t* out = g.out_i8 + (size_t)o * g.M * g.N;
+    const bool vec_ok = (g.N % 16 == 0) && (((uintptr_t)out & 15) == 0);
+    constexpr int CHUNKS_PER_ROW = BN / 16;
+    constexpr int TOTAL = BM * CHUNKS_PER_ROW;
+    for (int c = tid; c < TOTAL; c += NT) {
+        const int lrow = c / CHUNKS_PER_ROW, lc = (c % CHUNKS_PER_ROW) * 16;
+        const int row = m0 + lrow, col = n0 + lc;
+        if (row >= (int)g.M || col >= (int)g.N) continue;
+        const int8_t* src = stage + lrow * EPITCH + lc;
+        int8_t* dst = out + (size_t)row * g.N + col;
+        if (vec_ok && col + 15 < (int)g.N) {
+            *(v4i_t*)dst = *(const v4i_t*)src;
+        } else {
+            for (int e = 0; e < 16 && col + e < (int)g.N; e++) dst[e] = src[e];
         }
     }
 }
 
-template <int WGM, int WGN, int TM, int TN>
-int launch(const HipIgemmArgs& a, hipStream_t st) {
-    using C = Cfg<WGM, WGN, TM, TN>;
-    static bool attr_set = false;
-    auto kern = igemm_i8_kernel<WGM, WGN, TM, TN>;
-    if (!attr_set) {
-        if (!ESHKOL_HIP_OK(hipFuncSetAttribute((const void*)kern,
-                hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM_BYTES))) return -1;
-        attr_set = true;
+/* ---- pipelined kernel ------------------------------------------------------ */
+
+template <int TM, int TN, int PF>
+__global__ __launch_bounds__(256, 1)
+void igemm_i8_pipe_kernel(HipIgemmArgs g, int tiles_m, int tiles_n, int chunk) {
+    extern __shared__ __align__(16) int8_t smem_i8[];
+    int o, tm, tn;
+    if (!map_workgroup(tiles_m, tiles_n, (int)g.n_out, chunk, &o, &tm, &tn)) return;
+    constexpr int BM = 2 * TM * 32, BN = 2 * TN * 32;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const int pair_lo = g.pair_first[o];
+    pipe::Source src;
+    src.a_planes = g.a_planes; src.b_planes = g.b_planes;
+    src.a_plane_stride = g.a_plane_stride; src.b_plane_stride = g.b_plane_stride;
+    src.a_idx = g.pair_a + pair_lo; src.b_idx = g.pair_b + pair_lo;
+    src.npairs = g.pair_first[o + 1] - pair_lo;
+    src.ld = (int)g.ldk;
+
+    v16i_t acc[TM][TN];
+#pragma unroll
+    for (int t = 0; t < TM; t++)
+#pragma unroll
+        for (int u = 0; u < TN; u++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[t][u][r] = 0;
+
+    if (src.npairs > 0) pipe::run<I8Op, TM, TN, PF>(smem_i8, src, m0, n0, acc);
+    epilogue<TM, TN>(g, o, m0, n0, acc, smem_i8);
+}
+
+/* ---- simple kernel --------------------------------------------------------- */
+
+constexpr int SBK = 64;
+constexpr int SPITCH = SBK + 16;
+
+template <int TM, int TN>
+__global__ __launch_bounds__(256, 2)
+void igemm_i8_simple_kernel(HipIgemmArgs g, int tiles_m, int tiles_n, int chunk) {
+    constexpr int BM = 2 * TM * 32, BN = 2 * TN * 32, NT = 256;
+    constexpr int A_TILE = BM * SPITCH, B_TILE = BN * SPITCH;
+    constexpr int A_CH = BM * SBK / 16 / NT, B_CH = BN * SBK / 16 / NT;
+    extern __shared__ __align__(16) int8_t smem_i8[];
+    int8_t* As = smem_i8;
+    int8_t* Bs = smem_i8 + 2 * A_TILE;
+
+    int o, tm, tn;
+    if (!map_workgroup(tiles_m, tiles_n, (int)g.n_out, chunk, &o, &tm, &tn)) return;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int li = lane & 31, lh = lane >> 5;
+
+    const int pair_lo = g.pair_first[o], pair_hi = g.pair_first[o + 1];
+    const int nkb_per = (int)(g.ldk / SBK);
+    const int nkb = (pair_hi - pair_lo) * nkb_per;
+
+    v4i_t ra[A_CH], rb[B_CH];
+    auto gload = [&](int kb) {
+        const int t = pair_lo + kb / nkb_per;
+        const int k0 = (kb % nkb_per) * SBK;
+        const int8_t* Ap = g.a_planes + (size_t)g.pair_a[t] * g.a_plane_stride + (size_t)m0 * g.ldk + k0;
+        const int8_t* Bp = g.b_planes + (size_t)g.pair_b[t] * g.b_plane_stride + (size_t)n0 * g.ldk + k0;
+#pragma unroll
+        for (int r = 0; r < A_CH; r++) {
+            const int c = tid + NT * r;
+            ra[r] = *(const v4i_t*)(Ap + (size_t)(c >> 2) * g.ldk + (c & 3) * 16);
+        }
+#pragma unroll
+        for (int r = 0; r < B_CH; r++) {
+            const int c = tid + NT * r;
+            rb[r] = *(const v4i_t*)(Bp + (size_t)(c >> 2) * g.ldk + (c & 3) * 16);
+        }
+    };
+    auto sstore = [&](int buf) {
+#pragma unroll
+        for (int r = 0; r < A_CH; r++) {
+            const int c = tid + NT * r;
+            *(v4i_t*)(As + buf * A_TILE + (c >> 2) * SPITCH + (c & 3) * 16) = ra[r];
+        }
+#pragma unroll
+        for (int r = 0; r < B_CH; r++) {
+            const int c = tid + NT * r;
+            *(v4i_t*)(Bs + buf * B_TILE + (c >> 2) * SPITCH + (c & 3) * 16) = rb[r];
+        }
+    };
+
+    v16i_t acc[TM][TN];
+#pragma unroll
+    for (int t = 0; t < TM; t++)
+#pragma unroll
+        for (int u = 0; u < TN; u++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[t][u][r] = 0;
+
+    if (nkb > 0) { gload(0); sstore(0); }
+    __syncthreads();
+    int cur = 0;
+    for (int kb = 0; kb < nkb; kb++) {
+        const bool more = (kb + 1 < nkb);
+        if (more) gload(kb + 1);
+        const int8_t* a_base = As + cur * A_TILE + (wm * TM * 32 + li) * SPITCH + lh * 16;
+        const int8_t* b_base = Bs + cur * B_TILE + (wn * TN * 32 + li) * SPITCH + lh * 16;
+#pragma unroll
+        for (int ks = 0; ks < SBK / 32; ks++) {
+            v4i_t a[TM], b[TN];
+#pragma unroll
+            for (int t = 0; t < TM; t++) a[t] = *(const v4i_t*)(a_base + t * 32 * SPITCH + ks * 32);
+#pragma unroll
+            for (int u = 0; u < TN; u++) b[u] = *(const v4i_t*)(b_base + u * 32 * SPITCH + ks * 32);
+#pragma unroll
+            for (int t = 0; t < TM; t++)
+#pragma unroll
+                for (int u = 0; u < TN; u++) I8Op::mfma(b[u], a[t], acc[t][u]);
+        }
+        if (more) sstore(cur ^ 1);
+        __syncthreads();
+        cur ^= 1;
     }
-    const int tiles_m = (int)((a.M + C::BM - 1) / C::BM), tiles_n = (int)((a.N + C::BN - 1) / C::BN);
-    const long long nwg = (long long)tiles_m * tiles_n * a.n_out;
+    epilogue<TM, TN>(g, o, m0, n0, acc, smem_i8);
+}
+
+int g_prefetch = 2;     /* blocks in flight in the pipelined kernel */
+
+template <class K>
+int launch_kernel(K kern, int smem, bool* attr_set, const HipIgemmArgs& a, int BM, int BN, hipStream_t st) {
+    if (!*attr_set) {
+        if (!ESHKOL_HIP_OK(hipFuncSetAttribute((const void*)kern,
+                hipFuncAttributeMaxDynamicSharedMemorySize, smem))) return -1;
+        *attr_set = true;
+    }
+    const int tiles_m = (int)((a.M + BM - 1) / BM), tiles_n = (int)((a.N + BN - 1) / BN);
+    const int chunk = (tiles_m * tiles_n + 7) / 8;
+    const long long nwg = 8LL * chunk * a.n_out;
     if (nwg > 0x7fffffffLL || nwg <= 0) return -1;
-    hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(C::NT), C::SMEM_BYTES, st, a, tiles_m, tiles_n);
+    hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(256), smem, st, a, tiles_m, tiles_n, chunk);
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 
+template <int PF>
+int launch_pipe(const HipIgemmArgs& a, hipStream_t st) {
+    using C = pipe::Cfg<4, 4>;
+    constexpr int EPI = C::BM * (C::BN + 16);
+    constexpr int SMEM = C::SMEM_MAIN > EPI ? C::SMEM_MAIN : EPI;
+    static bool attr_set = false;
+    return launch_kernel(igemm_i8_pipe_kernel<4, 4, PF>, SMEM, &attr_set, a, C::BM, C::BN, st);
+}
+
+int launch_simple(const HipIgemmArgs& a, hipStream_t st) {
+    constexpr int BM = 128, BN = 128;
+    constexpr int MAIN = 2 * (BM + BN) * SPITCH, EPI = BM * (BN + 16);
+    constexpr int SMEM = MAIN > EPI ? MAIN : EPI;
+    static bool attr_set = false;
+    return launch_kernel(igemm_i8_simple_kernel<2, 2>, SMEM, &attr_set, a, BM, BN, st);
+}
+
 }  // namespace
+
+/* Tuning hook: k-blocks in flight in the pipelined kernel (1..3), 0 = simple kernel only. */
+extern "C" void hip_igemm_set_prefetch(int pf) { if (pf >= 0 && pf <= 3) g_prefetch = pf; }
 
 extern "C" int hip_igemm_i8(const HipIgemmArgs* args, void* stream) {
     if (!args || !args->a_planes || !args->b_planes || !args->pair_first || !args->pair_a || !args->pair_b)
@@ -268,9 +325,18 @@ extern "C" int hip_igemm_i8(const HipIgemmArgs* args, void* stream) {
     else if (a.mode == 1) { if (!a.out_i8 || !a.modulus) return -1; }
     else return -1;
     hipStream_t st = (hipStream_t)stream;
-    /* 256x256 tiles when they fill the chip, else 128x128. Operand planes are
-     * padded to multiples of 256 rows, so either tiling reads in bounds. */
+    /* Operand planes are padded to multiples of 256 rows, so either tiling reads
+     * in bounds. The pipelined kernel needs whole groups of prefetched blocks
+     * per product and at most 64 products per output plane. */
     const long long big = (long long)((a.M + 255) / 256) * ((a.N + 255) / 256) * a.n_out;
-    if (big >= 256) return launch<2, 2, 4, 4>(a, st);
-    return launch<2, 2, 2, 2>(a, st);
+    int pf = g_prefetch;
+    while (pf > 0 && a.ldk % (128u * pf) != 0) pf--;
+    if (pf > 0 && big >= 128 && a.max_pairs >= 1 && a.max_pairs <= pipe::MAX_PAIRS) {
+        switch (pf) {
+            case 1: return launch_pipe<1>(a, st);
+            case 2: return launch_pipe<2>(a, st);
+            default: return launch_pipe<3>(a, st);
+        }
+    }
+    return launch_simple(a, st);
 }

@@ -331,7 +331,7 @@ extern "C" int hip_matmul_ozaki_crt_f64(const double* A, const double* B, double
     hipStream_t st = (hipStream_t)stream;
     if (ensure_tables(st) != 0) return -1;
 
-    const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ldk = round_up_sz(K, 128);
+    const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ldk = round_up_sz(K, 256);
     double* Bt   = (double*)eshkol_hip_workspace(WS_BT, K * N * sizeof(double));
     double* amax = (double*)eshkol_hip_workspace(WS_ROWSCALE, M * sizeof(double));
     double* bmax = (double*)eshkol_hip_workspace(WS_COLSCALE, N * sizeof(double));
@@ -409,7 +409,7 @@ extern "C" int hip_matmul_ozaki_crt_f64(const double* A, const double* B, double
     ga.a_plane_stride = Mp * ldk; ga.b_plane_stride = Np * ldk;
     ga.ldk = (uint32_t)ldk; ga.M = (uint32_t)M; ga.N = (uint32_t)N; ga.n_out = (uint32_t)num_moduli;
     ga.pair_first = g_tables; ga.pair_a = g_tables + 17; ga.pair_b = g_tables + 17;
-    ga.mode = 1; ga.modulus = g_tables + 33; ga.out_i8 = Wp;
+    ga.mode = 1; ga.max_pairs = 1; ga.modulus = g_tables + 33; ga.out_i8 = Wp;
     if (hip_igemm_i8(&ga, st) != 0) return -1;
 
     if (hip_ozaki_crt_reconstruct_f64(Wp, M, N, num_moduli, crt.sl1, crt.sl2, crt.P1, crt.P2, crt.Pinv,

@@ -176,7 +176,7 @@ extern "C" int hip_matmul_ozaki_int8_f64(const double* A, const double* B, doubl
     }
     plan->first[nbuf] = npairs;
 
-    const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ldk = round_up_sz(K, 128);
+    const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ldk = round_up_sz(K, 256);
     double* Bt   = (double*)eshkol_hip_workspace(WS_BT, K * N * sizeof(double));
     double* rmax = (double*)eshkol_hip_workspace(WS_ROWSCALE, M * sizeof(double));
     double* cmax = (double*)eshkol_hip_workspace(WS_COLSCALE, N * sizeof(double));
@@ -203,7 +203,7 @@ extern "C" int hip_matmul_ozaki_int8_f64(const double* A, const double* B, doubl
     ga.a_plane_stride = Mp * ldk; ga.b_plane_stride = Np * ldk;
     ga.ldk = (uint32_t)ldk; ga.M = (uint32_t)M; ga.N = (uint32_t)N; ga.n_out = (uint32_t)nbuf;
     ga.pair_first = dplan->first; ga.pair_a = dplan->pa; ga.pair_b = dplan->pb;
-    ga.mode = 0; ga.out_i32 = G;
+    ga.mode = 0; ga.max_pairs = s; ga.out_i32 = G;
     if (hip_igemm_i8(&ga, st) != 0) return -1;
     if (hip_ozaki_reconstruct_f64(C, G, dplan->w, nbuf, rmax, cmax, M, N, st) != 0) return -1;
 

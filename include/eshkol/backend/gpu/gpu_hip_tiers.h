@@ -88,6 +88,7 @@ typedef struct {
      * mode 1: out_i8[o][M][N]  = the sum modulo modulus[o], representative in
      *         [-p/2, p/2); modulus[] in device memory                           */
     int32_t mode;
+    int32_t max_pairs;        /* upper bound on products per output plane (host knows the plan) */
     const int32_t* modulus;
     int32_t* out_i32;
     int8_t*  out_i8;
