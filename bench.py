@@ -64,6 +64,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-stages", action="store_true")
     ap.add_argument("--only", default="", help="comma list of tiers to time besides native: crt,int8,reduced")
+    ap.add_argument("--pmc-probe", default="", choices=["", "dgemm", "crt", "int8", "reduced"],
+                    help="run a calibration copy and three launches of one tier, for rocprofv3 --pmc")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build measures one GPU only (the path shards by rows of A with no "
@@ -80,6 +82,24 @@ def main():
     steps, warm = args.steps, args.warmup
     timer = ea.Timer()
     want = set(args.only.split(",")) if args.only else {"crt", "int8", "reduced"}
+
+    if args.pmc_probe:
+        # Short program for `rocprofv3 --pmc ...` runs: a 512 MiB device copy of known size
+        # (calibrates FETCH_SIZE / WRITE_SIZE), then three launches of one tier. No timing.
+        src, dst, out = ea.DeviceArray((M, K)), ea.DeviceArray((K, N)), ea.DeviceArray((M, N))
+        src.upload(synth.normal(11, (M, K)))
+        hip.hipMemcpy(dst.ptr, src.ptr, min(src.nbytes, 512 << 20), ea.D2D)
+        hip.hipDeviceSynchronize()
+        dst.upload(synth.normal(12, (K, N)))
+        calls = {"dgemm": lambda: lib.hip_dgemm_f64(src.ptr, dst.ptr, out.ptr, M, K, N, st),
+                 "crt": lambda: lib.hip_matmul_ozaki_crt_f64(src.ptr, dst.ptr, out.ptr, M, K, N, 16, 0, None, 0, st),
+                 "int8": lambda: lib.hip_matmul_ozaki_int8_f64(src.ptr, dst.ptr, out.ptr, M, K, N, 6, st),
+                 "reduced": lambda: lib.hip_matmul_reduced_f64(src.ptr, dst.ptr, out.ptr, M, K, N, 3, 0, st)}
+        for _ in range(3):
+            assert calls[args.pmc_probe]() == 0
+        hip.hipDeviceSynchronize()
+        print(json.dumps({"pmc_probe": args.pmc_probe, "size": n}))
+        return
 
     def timed(fn, k=steps, w=warm):
         """w untimed calls, then k calls bracketed by device syncs and HIP events
@@ -106,10 +126,23 @@ def main():
     native_gflops = flops / (wall_ms * 1e-3) / 1e9
     achieved = flops / (ev_ms * 1e-3)
     log("native fp64: %.3f ms/step (events %.3f ms) %.1f GFLOP/s" % (wall_ms, ev_ms, native_gflops))
+    # what the device itself sustains on a register-only MFMA loop / a large copy
+    sustained = {}
+    for name, kind, rnd in (("fp64_mfma_constant_operands", 0, 0), ("fp64_mfma_random_operands", 0, 1),
+                            ("int8_mfma_constant_operands", 1, 0), ("int8_mfma_random_operands", 1, 1),
+                            ("bf16_mfma_constant_operands", 2, 0), ("bf16_mfma_random_operands", 2, 1),
+                            ("hbm_copy_read_plus_write", 3, 0)):
+        rate = C.c_double()
+        if lib.hip_probe_peak(kind, rnd, C.byref(rate), st) == 0:
+            sustained[name] = rate.value / 1e12
+    log("device sustains (T/s):", json.dumps(sustained))
     roofline = {"bound": "mfma", "kernel": "dgemm_mfma_kernel<128,128>",
                 "achieved": achieved / 1e12, "peak": PEAK["fp64_mfma"] / 1e12, "unit": "TFLOP/s",
                 "frac": achieved / PEAK["fp64_mfma"], "launch_ms": ev_ms,
-                "traffic": read_traffic("dgemm_mfma_8192_hbm_traffic.txt")}
+                "traffic": read_traffic("dgemm_mfma_8192_hbm_traffic.txt"),
+                "sustained_peak_random_operands": sustained.get("fp64_mfma_random_operands"),
+                "frac_of_sustained": (achieved / 1e12 / sustained["fp64_mfma_random_operands"])
+                if sustained.get("fp64_mfma_random_operands") else None}
     tiers = {"native_fp64": {"ms": wall_ms, "gflops": native_gflops, "frac_of_peak": achieved / PEAK["fp64_mfma"],
                              "peak": "fp64 MFMA 78.6 TFLOP/s"}}
 
@@ -242,6 +275,7 @@ def main():
         "config": {"workload": "native fp64 tier, C=A*B, M=N=K=%d, A,B ~ N(0,1) from seed, row-major dense, "
                                "operands resident in HBM" % n},
         "roofline": roofline, "cpu_baseline": cpu, "tiers": tiers,
+        "device_sustains_T_per_s": sustained,
     }
     print(json.dumps(out), flush=True)
 

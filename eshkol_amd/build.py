@@ -27,6 +27,7 @@ SOURCES = [
     "ozaki_crt.hip",
     "ozaki_int8.hip",
     "elementwise.hip",
+    "peak_probe.hip",
 ]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -34,7 +35,8 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # On gfx950 the fp64 MFMA runs at half rate when its accumulator lives in the
 # AGPR half of the register file (measured: 36 vs 78 TFLOP/s on a register-only
 # loop); the int8 and 16-bit MFMAs do not care. Keep fp64 accumulators in VGPRs.
-EXTRA = {"dgemm_f64.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+EXTRA = {"dgemm_f64.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+         "peak_probe.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 # -ffp-contract=off: every fused multiply-add the arithmetic relies on is
 # written as fma(); the compiler must not add or remove any.

@@ -19,6 +19,7 @@
  */
 #include "hip_common.h"
 #include "kernels.h"
+#include "gemm_pipe.h"
 
 #include <cstring>
 
@@ -234,6 +235,122 @@ void hgemm_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
     }
 }
 
+/* ---- pipelined kernel (gemm_pipe.h): 256x256 tile, 128-byte k-blocks ------- */
+
+template <bool BF16> struct H16Op {
+    typedef v16f_t acc_t;
+    static __device__ __forceinline__ void mfma(const v4i_t& first, const v4i_t& second, v16f_t& acc) {
+        if (BF16)
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8b_t, first),
+                                                          __builtin_bit_cast(v8b_t, second), acc, 0, 0, 0);
+        else
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h_t, first),
+                                                         __builtin_bit_cast(v8h_t, second), acc, 0, 0, 0);
+    }
+};
+
+template <bool BF16>
+__device__ __forceinline__ float round16(float x) {
+    return BF16 ? bf16_bits_to_f32(f32_to_bf16_bits(x)) : f16_bits_to_f32(f32_to_f16_bits(x));
+}
+
+/* lane column is the output row; registers 4v..4v+3 are output columns
+ * 8v + 4*(lane/32) + 0..3 of the 32x32 tile */
+template <bool BF16, int TM, int TN>
+__device__ __forceinline__ void store_tile(v16f_t (&acc)[TM][TN], int m0, int n0, int M, int N,
+                                           int out_mode, void* Cout) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int li = lane & 31, lh = lane >> 5;
+#pragma unroll
+    for (int t = 0; t < TM; t++) {
+        const int row = m0 + wm * TM * 32 + t * 32 + li;
+        if (row >= M) continue;
+#pragma unroll
+        for (int u = 0; u < TN; u++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int col = n0 + wn * TN * 32 + u * 32 + 8 * v + 4 * lh;
+                float f[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    float x = acc[t][u][4 * v + e];
+                    if (out_mode == 2) x = round16<BF16>(x);
+                    f[e] = x;
+                }
+                if (out_mode == 0) {
+                    float* p = (float*)Cout + (size_t)row * N + col;
+                    if ((N & 3) == 0 && col + 3 < N) *(v4f_t*)p = (v4f_t){f[0], f[1], f[2], f[3]};
+                    else for (int e = 0; e < 4; e++) if (col + e < N) p[e] = f[e];
+                } else {
+                    double* p = (double*)Cout + (size_t)row * N + col;
+                    if ((N & 1) == 0 && col + 3 < N) {
+                        *(d2_t*)p = (d2_t){(double)f[0], (double)f[1]};
+                        *(d2_t*)(p + 2) = (d2_t){(double)f[2], (double)f[3]};
+                    } else {
+                        for (int e = 0; e < 4; e++) if (col + e < N) p[e] = (double)f[e];
+                    }
+                }
+            }
+    }
+}
+
+template <bool BF16, int PF>
+__global__ __launch_bounds__(256, 1)
+void hgemm_pipe_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ Bt,
+                       int M, int N, int ld_bytes, int out_mode, void* __restrict__ Cout,
+                       int tiles_m, int tiles_n) {
+    extern __shared__ __align__(16) int8_t smem_h[];
+    int tm, tn;
+    {
+        const int nwg = gridDim.x, wg = blockIdx.x;
+        const int q = nwg >> 3, r = nwg & 7;
+        const int xcd = wg & 7, seq = wg >> 3;
+        const int L = xcd * q + (xcd < r ? xcd : r) + seq;
+        const int GM = 8;
+        const int width = GM * tiles_n;
+        const int group = L / width;
+        const int first_m = group * GM;
+        const int gsize = (tiles_m - first_m < GM) ? tiles_m - first_m : GM;
+        const int in_group = L - group * width;
+        tm = first_m + in_group % gsize;
+        tn = in_group / gsize;
+    }
+    const int m0 = tm * 256, n0 = tn * 256;
+    pipe::Source src;
+    src.a_planes = (const int8_t*)A; src.b_planes = (const int8_t*)Bt;
+    src.a_plane_stride = 0; src.b_plane_stride = 0;
+    src.a_idx = nullptr; src.b_idx = nullptr;
+    src.npairs = 1;
+    src.ld = ld_bytes;
+    v16f_t acc[4][4];
+#pragma unroll
+    for (int t = 0; t < 4; t++)
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[t][u][r] = 0.0f;
+    pipe::run<H16Op<BF16>, 4, 4, PF>(smem_h, src, m0, n0, acc);
+    store_tile<BF16, 4, 4>(acc, m0, n0, M, N, out_mode, Cout);
+}
+
+template <bool BF16>
+int launch_pipe(const uint16_t* A, const uint16_t* Bt, int M, int N, int ld_bytes, int out_mode, void* C,
+                hipStream_t st) {
+    using Cf = pipe::Cfg<4, 4>;
+    static bool attr_set = false;
+    auto kern = hgemm_pipe_kernel<BF16, 2>;
+    if (!attr_set) {
+        if (!ESHKOL_HIP_OK(hipFuncSetAttribute((const void*)kern,
+                hipFuncAttributeMaxDynamicSharedMemorySize, Cf::SMEM_MAIN))) return -1;
+        attr_set = true;
+    }
+    const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(256), Cf::SMEM_MAIN, st,
+                       A, Bt, M, N, ld_bytes, out_mode, C, tiles_m, tiles_n);
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
 template <bool BF16, int TM, int TN>
 int launch(const uint16_t* A, const uint16_t* Bt, int M, int N, int ld_bytes, int out_mode, void* C,
            hipStream_t st) {
@@ -260,6 +377,9 @@ int hgemm_any(const uint16_t* A, const uint16_t* Bt, uint64_t M, uint64_t K, uin
     if (((uintptr_t)A & 15) || ((uintptr_t)Bt & 15)) return -1;
     const int m = (int)M, n = (int)N, ldb = (int)(ld * 2);
     const long long big = (long long)((M + 255) / 256) * ((N + 255) / 256);
+    if (big >= 128 && ldb % 256 == 0)
+        return is_bf16 ? launch_pipe<true>(A, Bt, m, n, ldb, out_mode, C, st)
+                       : launch_pipe<false>(A, Bt, m, n, ldb, out_mode, C, st);
     if (big >= 256)
         return is_bf16 ? launch<true, 4, 4>(A, Bt, m, n, ldb, out_mode, C, st)
                        : launch<false, 4, 4>(A, Bt, m, n, ldb, out_mode, C, st);
@@ -296,7 +416,7 @@ extern "C" int hip_matmul_reduced_f64(const double* A, const double* B, double* 
     if (M > 0x7fffffffULL || K > 0x3fffffffULL || N > 0x7fffffffULL) return -1;
     hipStream_t st = (hipStream_t)stream;
     const int is_bf16 = (dtype == 3);
-    const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ld = round_up_sz(K, 64);
+    const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ld = round_up_sz(K, 128);
     double* Bt = (double*)eshkol_hip_workspace(WS_BT, K * N * sizeof(double));
     uint16_t* A16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_A, Mp * ld * 2);
     uint16_t* B16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_B, Np * ld * 2);

@@ -1,0 +1,161 @@
+/*
+ * What the device sustains, measured in place, so that every throughput figure
+ * can be quoted against both the published peak and the rate the silicon holds
+ * under the same kind of data.
+ *
+ * The matrix-core probes run a register-only MFMA loop (no memory traffic, every
+ * SIMD occupied by several waves). With constant operands they reach the
+ * published rates; with random operand bits the chip lowers its clock to hold
+ * its power limit and sustains markedly less (about 63 of 78.6 TFLOP/s for fp64,
+ * 3.0 of 5.0 POP/s for int8, 1.7 of 2.5 PFLOP/s for bf16 were measured). A GEMM
+ * on real data cannot beat the random-operand figure.
+ *
+ * The memory probe is a plain 16-byte-per-lane copy of a buffer much larger
+ * than the caches: the read+write rate HBM sustains.
+ */
+#include "hip_common.h"
+#include "kernels.h"
+
+typedef int v4i_t __attribute__((ext_vector_type(4)));
+typedef int v16i_t __attribute__((ext_vector_type(16)));
+typedef float v16f_t __attribute__((ext_vector_type(16)));
+typedef double d4_t __attribute__((ext_vector_type(4)));
+typedef __bf16 v8b_t __attribute__((ext_vector_type(8)));
+
+namespace {
+
+__device__ __forceinline__ unsigned mix(unsigned x) {
+    x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+    return x;
+}
+
+__global__ __launch_bounds__(256)
+void probe_f64(int iters, int random, int* sink) {
+    d4_t acc[8];
+    double a[8], b[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        acc[i] = (d4_t){0.0, 0.0, 0.0, 0.0};
+        const unsigned h1 = mix(threadIdx.x * 64 + i + blockIdx.x * 7919), h2 = mix(h1 + 1);
+        a[i] = random ? ((double)h1 / 4294967296.0 - 0.5) * 1.37 : 1.0;
+        b[i] = random ? ((double)h2 / 4294967296.0 - 0.5) * 0.73 : 0.5;
+    }
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+            acc[i] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[i], b[(i + it) & 7], acc[i], 0, 0, 0);
+    }
+    double s = 0.0;
+    for (int i = 0; i < 8; i++) for (int r = 0; r < 4; r++) s += acc[i][r];
+    if (s == 12345.678) sink[0] = 1;
+}
+
+__global__ __launch_bounds__(256)
+void probe_i8(int iters, int random, int* sink) {
+    v16i_t acc[8];
+    v4i_t a[8], b[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[i][r] = 0;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const unsigned h1 = mix(threadIdx.x * 64 + i * 8 + c + blockIdx.x * 7919), h2 = mix(h1 + 12345);
+            a[i][c] = random ? (int)h1 : 0x01010101;
+            b[i][c] = random ? (int)h2 : 0x02020202;
+        }
+    }
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+            acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[(i + it) & 7], acc[i], 0, 0, 0);
+    }
+    int s = 0;
+    for (int i = 0; i < 8; i++) for (int r = 0; r < 16; r++) s += acc[i][r];
+    if (s == 123456789) sink[0] = s;
+}
+
+__global__ __launch_bounds__(256)
+void probe_bf16(int iters, int random, int* sink) {
+    v16f_t acc[8];
+    v4i_t a[8], b[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[i][r] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const unsigned h1 = mix(threadIdx.x * 64 + i * 8 + c + blockIdx.x * 7919), h2 = mix(h1 + 12345);
+            /* random sign and mantissa, exponent near 1.0 so nothing overflows */
+            a[i][c] = random ? (int)((h1 & 0x807f807fu) | 0x3c003c00u) : 0x3f803f80;
+            b[i][c] = random ? (int)((h2 & 0x807f807fu) | 0x3c003c00u) : 0x3f803f80;
+        }
+    }
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+            acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8b_t, a[i]),
+                                                             __builtin_bit_cast(v8b_t, b[(i + it) & 7]),
+                                                             acc[i], 0, 0, 0);
+    }
+    float s = 0.0f;
+    for (int i = 0; i < 8; i++) for (int r = 0; r < 16; r++) s += acc[i][r];
+    if (s == 12345.678f) sink[0] = 1;
+}
+
+__global__ __launch_bounds__(256)
+void probe_copy(const v4i_t* __restrict__ src, v4i_t* __restrict__ dst, size_t n16) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}
+
+}  // namespace
+
+/* kind 0: fp64 MFMA flop/s, 1: int8 MFMA op/s, 2: bf16 MFMA flop/s, 3: HBM copy
+ * bytes/s (read + written). random_operands selects random operand bits for the
+ * matrix-core kinds. Synchronises the stream. */
+extern "C" int hip_probe_peak(int kind, int random_operands, double* rate, void* stream) {
+    if (!rate || kind < 0 || kind > 3) return -1;
+    hipStream_t st = (hipStream_t)stream;
+    hipEvent_t e0, e1;
+    if (!ESHKOL_HIP_OK(hipEventCreate(&e0)) || !ESHKOL_HIP_OK(hipEventCreate(&e1))) return -1;
+    int rc = -1;
+    float ms = 0.0f;
+    if (kind == 3) {
+        const size_t bytes = (size_t)1 << 30;
+        char* buf = (char*)eshkol_hip_workspace(WS_MISC, 2 * bytes);
+        if (buf) {
+            for (int rep = 0; rep < 2; rep++) {
+                if (rep == 1) (void)hipEventRecord(e0, st);
+                hipLaunchKernelGGL(probe_copy, dim3(256 * 16), dim3(256), 0, st,
+                                   (const v4i_t*)buf, (v4i_t*)(buf + bytes), bytes / 16);
+            }
+            (void)hipEventRecord(e1, st);
+            if (ESHKOL_HIP_OK(hipEventSynchronize(e1)) && ESHKOL_HIP_OK(hipEventElapsedTime(&ms, e0, e1)) && ms > 0) {
+                *rate = 2.0 * (double)bytes / (ms * 1e-3);
+                rc = 0;
+            }
+        }
+    } else {
+        int* sink = (int*)eshkol_hip_workspace(WS_MISC, 256);
+        const int wgs = 1024;
+        const int iters = (kind == 0) ? 20000 : 40000;
+        const double per_mfma = (kind == 0) ? 2048.0 : (kind == 1) ? 65536.0 : 32768.0;
+        if (sink) {
+            for (int rep = 0; rep < 2; rep++) {
+                if (rep == 1) (void)hipEventRecord(e0, st);
+                if (kind == 0) hipLaunchKernelGGL(probe_f64, dim3(wgs), dim3(256), 0, st, iters, random_operands, sink);
+                else if (kind == 1) hipLaunchKernelGGL(probe_i8, dim3(wgs), dim3(256), 0, st, iters, random_operands, sink);
+                else hipLaunchKernelGGL(probe_bf16, dim3(wgs), dim3(256), 0, st, iters, random_operands, sink);
+            }
+            (void)hipEventRecord(e1, st);
+            if (ESHKOL_HIP_OK(hipEventSynchronize(e1)) && ESHKOL_HIP_OK(hipEventElapsedTime(&ms, e0, e1)) && ms > 0) {
+                *rate = (double)wgs * 4.0 * iters * 8.0 * per_mfma / (ms * 1e-3);
+                rc = 0;
+            }
+        }
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return rc;
+}

@@ -181,6 +181,18 @@ int hip_hgemm_16(const uint16_t* A, const uint16_t* Bt, uint64_t M, uint64_t K, 
 int hip_convert_f64_to_16(const double* in, uint16_t* out, uint64_t rows, uint64_t cols,
                           uint64_t rows_padded, uint64_t ld, int is_bf16, void* stream);
 
+/* ---- measurement support ----------------------------------------------------
+ * Rate the device sustains on a register-only MFMA loop (kind 0 fp64 flop/s,
+ * 1 int8 op/s, 2 bf16 flop/s; random_operands != 0 uses random operand bits,
+ * under which the chip clocks down to hold its power limit) or on a large copy
+ * (kind 3, bytes/s read+written). The counterpart of the reference's
+ * self-calibrating peak model (gpu_memory_cuda.cpp:499-522), measured rather
+ * than seeded. Synchronises the stream. */
+int hip_probe_peak(int kind, int random_operands, double* rate, void* stream);
+
+/* k-blocks kept in flight by the pipelined int8 kernel (1..3; 0 = simple kernel only). */
+void hip_igemm_set_prefetch(int pf);
+
 #ifdef __cplusplus
 }
 #endif
