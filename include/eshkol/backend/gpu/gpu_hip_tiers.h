@@ -69,7 +69,9 @@ int hip_bias_act_f64(double* Y, const double* bias, uint64_t rows, uint64_t cols
  * gpu_memory_cuda.cpp:415-434 and the modular GEMM matmul_ozaki_gemm
  * (metal_softfloat.h:3907-4100). Operand planes are K-contiguous int8 with a
  * row pitch of ldk bytes (multiple of 128, zero padded beyond K) and row counts
- * padded with zero rows to multiples of 256. */
+ * padded with zero rows to multiples of 256. The pipelined kernel needs ldk to
+ * be a multiple of 256 and 1 <= max_pairs <= 64; other plans take the simple
+ * kernel. */
 typedef struct {
     const int8_t* a_planes;   /* [n_a_planes][rows_a_padded][ldk]                */
     const int8_t* b_planes;   /* [n_b_planes][rows_b_padded][ldk]                */
