@@ -72,6 +72,7 @@ SIGNATURES = {
     "eshkol_gpu_wait": (None, [BUF]),
     "eshkol_gpu_matmul_f64": (C.c_int, [BUF, BUF, BUF, u64, u64, u64]),
     "eshkol_gpu_matmul_f32": (C.c_int, [BUF, BUF, BUF, u64, u64, u64]),
+    "eshkol_gpu_matmul_backward_f64": (C.c_int, [BUF, BUF, BUF, BUF, BUF, u64, u64, u64]),
     "eshkol_gpu_set_threshold": (None, [C.c_size_t]),
     "eshkol_gpu_get_threshold": (C.c_size_t, []),
     "eshkol_gpu_should_use": (C.c_int, [C.c_size_t]),
@@ -90,6 +91,7 @@ SIGNATURES = {
     # gpu_hip_tiers.h
     "eshkol_hip_get_stream": (vp, []),
     "hip_dgemm_f64": (C.c_int, [vp, vp, vp, u64, u64, u64, vp]),
+    "hip_dgemm_f64_ex": (C.c_int, [vp, vp, vp, u64, u64, u64, C.c_int, C.c_int, vp]),
     "hip_sgemm_f32": (C.c_int, [vp, vp, vp, u64, u64, u64, vp]),
     "hip_transpose_f64": (C.c_int, [vp, vp, u64, u64, vp]),
     "hip_rowabsmax_f64": (C.c_int, [vp, u64, u64, C.c_double, vp, vp]),
@@ -106,6 +108,11 @@ SIGNATURES = {
     "hip_matmul_ozaki_int8_f64": (C.c_int, [vp, vp, vp, u64, u64, u64, C.c_int, vp]),
     "hip_ozaki_int8_last_stages": (C.c_int, [C.POINTER(HipOzakiInt8Stages)]),
     "hip_matmul_reduced_f64": (C.c_int, [vp, vp, vp, u64, u64, u64, C.c_int, C.c_int, vp]),
+    "hip_matmul_ozaki_crt_f64_ex": (C.c_int, [vp, vp, vp, u64, u64, u64, C.c_int, C.c_int, C.c_int, C.c_int,
+                                              vp, C.c_int, vp]),
+    "hip_matmul_ozaki_int8_f64_ex": (C.c_int, [vp, vp, vp, u64, u64, u64, C.c_int, C.c_int, C.c_int, vp]),
+    "hip_matmul_reduced_f64_ex": (C.c_int, [vp, vp, vp, u64, u64, u64, C.c_int, C.c_int, C.c_int, C.c_int, vp]),
+    "hip_matmul_backward_f64": (C.c_int, [vp, vp, vp, vp, vp, u64, u64, u64, C.c_int, C.c_int, vp]),
     "hip_hgemm_16": (C.c_int, [vp, vp, u64, u64, u64, u64, C.c_int, vp, vp]),
     "hip_convert_f64_to_16": (C.c_int, [vp, vp, u64, u64, u64, u64, C.c_int, vp]),
     "hip_probe_peak": (C.c_int, [C.c_int, C.c_int, dp, vp]),

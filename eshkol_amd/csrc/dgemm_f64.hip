@@ -9,7 +9,9 @@
  *              in registers
  *   LDS        double-buffered: A tile [BM][16(+2)] k-contiguous, B tile
  *              [16][BN(+4)] n-contiguous; the pads make every ds_read hit
- *              distinct banks
+ *              distinct banks. An operand the caller holds transposed (the
+ *              backward products G*B^T and A^T*G) takes the other operand's
+ *              tile form, so no transposed copy is ever made
  *   pipeline   global loads of block kb+1 are issued before the MFMAs of block
  *              kb and written to the other LDS buffer after them: one barrier
  *              per k-block
@@ -32,17 +34,87 @@ typedef double d2_t __attribute__((ext_vector_type(2)));
 namespace {
 
 constexpr int BK = 16;
-constexpr int LDA_S = BK + 2;      /* doubles per A row in LDS: 144 B */
 
-template <int BM, int BN> struct Tile {
-    static constexpr int LDB_S = BN + 4;              /* doubles per B row in LDS */
-    static constexpr int A_TILE = BM * LDA_S;
-    static constexpr int B_TILE = BK * LDB_S;
-    static constexpr int SMEM_BYTES = 2 * (A_TILE + B_TILE) * (int)sizeof(double);
-    static constexpr int TM = BM / 32;                /* 16x16 tiles per wave, rows */
-    static constexpr int TN = BN / 32;
-    static constexpr int A_CHUNKS = BM * BK / 2 / 256; /* 16-byte chunks per thread */
-    static constexpr int B_CHUNKS = BK * BN / 2 / 256;
+/* One operand of a block tile: R rows (the m or the n extent) by BK k-values.
+ * KMAJ = false: the matrix is stored row by row with k contiguous (A as given,
+ *   B when the caller holds its transpose); LDS tile [R][BK+2], a lane reads
+ *   its four k-values as two 16-byte loads.
+ * KMAJ = true:  the matrix is stored k by k with the row index contiguous (B
+ *   as given, A when the caller holds its transpose); LDS tile [BK][R+4], a
+ *   lane reads one 8-byte value per MFMA step.
+ * The pads make every LDS read of a wave hit distinct banks. Both forms hand
+ * the MFMA the value at (row li + 16 t, k = 4 lg + s), so they are
+ * interchangeable on either side of the instruction. */
+template <int R, bool KMAJ, bool VEC> struct Operand {
+    static constexpr int LD_S = KMAJ ? R + 4 : BK + 2;
+    static constexpr int TILE = KMAJ ? BK * LD_S : R * LD_S;
+    static constexpr int CHUNKS = R * BK / 2 / 256;   /* 16-byte chunks per thread */
+    static constexpr int T = R / 32;                  /* 16-row tiles per wave */
+    d2_t reg[CHUNKS];
+    d2_t lo[KMAJ ? 1 : T], hi[KMAJ ? 1 : T];
+    const double* base;
+
+    /* rows = row count of the whole matrix, K = its k extent */
+    __device__ __forceinline__ void gload(const double* __restrict__ P, int rows, int K,
+                                          int r0, int k0, int tid) {
+#pragma unroll
+        for (int r = 0; r < CHUNKS; r++) {
+            const int c = tid + 256 * r;
+            d2_t v = {0.0, 0.0};
+            if (KMAJ) {
+                const int kr = c / (R / 2), rc = c % (R / 2);
+                const int gk = k0 + kr, gr = r0 + 2 * rc;
+                const double* p = P + (size_t)gk * rows + gr;
+                if (VEC) {
+                    if (gk < K && gr < rows) v = *(const d2_t*)p;
+                } else {
+                    if (gk < K && gr < rows) v.x = p[0];
+                    if (gk < K && gr + 1 < rows) v.y = p[1];
+                }
+            } else {
+                const int row = c >> 3, kc = c & 7;
+                const int gr = r0 + row, gk = k0 + 2 * kc;
+                const double* p = P + (size_t)gr * K + gk;
+                if (VEC) {
+                    if (gr < rows && gk < K) v = *(const d2_t*)p;
+                } else {
+                    if (gr < rows && gk < K) v.x = p[0];
+                    if (gr < rows && gk + 1 < K) v.y = p[1];
+                }
+            }
+            reg[r] = v;
+        }
+    }
+    __device__ __forceinline__ void sstore(double* S, int tid) const {
+#pragma unroll
+        for (int r = 0; r < CHUNKS; r++) {
+            const int c = tid + 256 * r;
+            if (KMAJ) {
+                const int kr = c / (R / 2), rc = c % (R / 2);
+                *(d2_t*)(S + kr * LD_S + 2 * rc) = reg[r];
+            } else {
+                const int row = c >> 3, kc = c & 7;
+                *(d2_t*)(S + row * LD_S + 2 * kc) = reg[r];
+            }
+        }
+    }
+    /* woff = first row of this wave inside the block tile */
+    __device__ __forceinline__ void frag_begin(const double* S, int woff, int li, int lg) {
+        if (KMAJ) {
+            base = S + (4 * lg) * LD_S + woff + li;
+        } else {
+            base = S + (woff + li) * LD_S + 4 * lg;
+#pragma unroll
+            for (int t = 0; t < T; t++) {
+                lo[t] = *(const d2_t*)(base + t * 16 * LD_S);
+                hi[t] = *(const d2_t*)(base + t * 16 * LD_S + 2);
+            }
+        }
+    }
+    __device__ __forceinline__ double frag(int s, int t) const {
+        if (KMAJ) return base[s * LD_S + t * 16];
+        return (s == 0) ? lo[t].x : (s == 1) ? lo[t].y : (s == 2) ? hi[t].x : hi[t].y;
+    }
 };
 
 __device__ __forceinline__ void tile_of_workgroup(int tiles_m, int tiles_n, int* tm, int* tn) {
@@ -60,16 +132,19 @@ __device__ __forceinline__ void tile_of_workgroup(int tiles_m, int tiles_n, int*
     *tn = in_group / gsize;
 }
 
-/* VEC: K and N even and A, B 16-byte aligned, so operands move as 16-byte pairs. */
-template <int BM, int BN, bool VEC>
+/* C[MxN] = op(A) * op(B). TA: A is stored as its transpose [K][M]; TB: B is
+ * stored as its transpose [N][K]. VEC: every row pitch is even and both bases
+ * are 16-byte aligned, so operands move as 16-byte pairs. */
+template <int BM, int BN, bool VEC, bool TA, bool TB>
 __global__ __launch_bounds__(256)
 void dgemm_mfma_kernel(const double* __restrict__ A, const double* __restrict__ B,
                        double* __restrict__ C, int M, int N, int K,
                        int tiles_m, int tiles_n) {
-    using T = Tile<BM, BN>;
+    using OpA = Operand<BM, TA, VEC>;
+    using OpB = Operand<BN, !TB, VEC>;
     extern __shared__ __align__(16) double smem[];
     double* As = smem;
-    double* Bs = smem + 2 * T::A_TILE;
+    double* Bs = smem + 2 * OpA::TILE;
 
     int tm, tn;
     tile_of_workgroup(tiles_m, tiles_n, &tm, &tn);
@@ -80,106 +155,59 @@ void dgemm_mfma_kernel(const double* __restrict__ A, const double* __restrict__ 
     const int wm = wave >> 1, wn = wave & 1;
     const int li = lane & 15, lg = lane >> 4;
 
-    d2_t ra[T::A_CHUNKS], rb[T::B_CHUNKS];
+    OpA a;
+    OpB b;
 
-    auto gload = [&](int kb) {
-        const int k0 = kb * BK;
+    d4_t acc[OpA::T][OpB::T];
 #pragma unroll
-        for (int r = 0; r < T::A_CHUNKS; r++) {
-            const int c = tid + 256 * r;
-            const int row = c >> 3, kc = c & 7;
-            const int gr = m0 + row, gk = k0 + 2 * kc;
-            const double* p = A + (size_t)gr * K + gk;
-            d2_t v = {0.0, 0.0};
-            if (VEC) {
-                if (gr < M && gk < K) v = *(const d2_t*)p;
-            } else {
-                if (gr < M && gk < K) v.x = p[0];
-                if (gr < M && gk + 1 < K) v.y = p[1];
-            }
-            ra[r] = v;
-        }
+    for (int t = 0; t < OpA::T; t++)
 #pragma unroll
-        for (int r = 0; r < T::B_CHUNKS; r++) {
-            const int c = tid + 256 * r;
-            const int kr = c / (BN / 2), nc = c % (BN / 2);
-            const int gk = k0 + kr, gn = n0 + 2 * nc;
-            const double* p = B + (size_t)gk * N + gn;
-            d2_t v = {0.0, 0.0};
-            if (VEC) {
-                if (gk < K && gn < N) v = *(const d2_t*)p;
-            } else {
-                if (gk < K && gn < N) v.x = p[0];
-                if (gk < K && gn + 1 < N) v.y = p[1];
-            }
-            rb[r] = v;
-        }
-    };
-    auto sstore = [&](int buf) {
-#pragma unroll
-        for (int r = 0; r < T::A_CHUNKS; r++) {
-            const int c = tid + 256 * r;
-            const int row = c >> 3, kc = c & 7;
-            *(d2_t*)(As + buf * T::A_TILE + row * LDA_S + 2 * kc) = ra[r];
-        }
-#pragma unroll
-        for (int r = 0; r < T::B_CHUNKS; r++) {
-            const int c = tid + 256 * r;
-            const int kr = c / (BN / 2), nc = c % (BN / 2);
-            *(d2_t*)(Bs + buf * T::B_TILE + kr * T::LDB_S + 2 * nc) = rb[r];
-        }
-    };
-
-    d4_t acc[T::TM][T::TN];
-#pragma unroll
-    for (int t = 0; t < T::TM; t++)
-#pragma unroll
-        for (int u = 0; u < T::TN; u++) acc[t][u] = (d4_t){0.0, 0.0, 0.0, 0.0};
+        for (int u = 0; u < OpB::T; u++) acc[t][u] = (d4_t){0.0, 0.0, 0.0, 0.0};
 
     const int nkb = (K + BK - 1) / BK;
-    gload(0);
-    sstore(0);
+    a.gload(A, M, K, m0, 0, tid);
+    b.gload(B, N, K, n0, 0, tid);
+    a.sstore(As, tid);
+    b.sstore(Bs, tid);
     __syncthreads();
 
     int cur = 0;
     for (int kb = 0; kb < nkb; kb++) {
         const bool more = (kb + 1 < nkb);
-        if (more) gload(kb + 1);
-
-        const double* a_base = As + cur * T::A_TILE + (wm * (BM / 2) + li) * LDA_S + 4 * lg;
-        const double* b_base = Bs + cur * T::B_TILE + (4 * lg) * T::LDB_S + wn * (BN / 2) + li;
-
-        d2_t a_lo[T::TM], a_hi[T::TM];
-#pragma unroll
-        for (int t = 0; t < T::TM; t++) {
-            a_lo[t] = *(const d2_t*)(a_base + t * 16 * LDA_S);
-            a_hi[t] = *(const d2_t*)(a_base + t * 16 * LDA_S + 2);
+        if (more) {
+            a.gload(A, M, K, m0, (kb + 1) * BK, tid);
+            b.gload(B, N, K, n0, (kb + 1) * BK, tid);
         }
+
+        a.frag_begin(As + cur * OpA::TILE, wm * (BM / 2), li, lg);
+        b.frag_begin(Bs + cur * OpB::TILE, wn * (BN / 2), li, lg);
 #pragma unroll
         for (int s = 0; s < 4; s++) {
-            double b[T::TN];
+            double av[OpA::T], bv[OpB::T];
 #pragma unroll
-            for (int u = 0; u < T::TN; u++) b[u] = b_base[s * T::LDB_S + u * 16];
+            for (int t = 0; t < OpA::T; t++) av[t] = a.frag(s, t);
 #pragma unroll
-            for (int t = 0; t < T::TM; t++) {
-                const double a = (s == 0) ? a_lo[t].x : (s == 1) ? a_lo[t].y
-                               : (s == 2) ? a_hi[t].x : a_hi[t].y;
+            for (int u = 0; u < OpB::T; u++) bv[u] = b.frag(s, u);
 #pragma unroll
-                for (int u = 0; u < T::TN; u++)
-                    acc[t][u] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, b[u], acc[t][u], 0, 0, 0);
-            }
+            for (int t = 0; t < OpA::T; t++)
+#pragma unroll
+                for (int u = 0; u < OpB::T; u++)
+                    acc[t][u] = __builtin_amdgcn_mfma_f64_16x16x4f64(av[t], bv[u], acc[t][u], 0, 0, 0);
         }
 
-        if (more) sstore(cur ^ 1);
+        if (more) {
+            a.sstore(As + (cur ^ 1) * OpA::TILE, tid);
+            b.sstore(Bs + (cur ^ 1) * OpB::TILE, tid);
+        }
         __syncthreads();
         cur ^= 1;
     }
 
     /* accumulator layout: register r of the lane is row 4*r + lane/16, column lane%16 */
 #pragma unroll
-    for (int t = 0; t < T::TM; t++)
+    for (int t = 0; t < OpA::T; t++)
 #pragma unroll
-        for (int u = 0; u < T::TN; u++) {
+        for (int u = 0; u < OpB::T; u++) {
             const int col = n0 + wn * (BN / 2) + u * 16 + li;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
@@ -189,40 +217,57 @@ void dgemm_mfma_kernel(const double* __restrict__ A, const double* __restrict__ 
         }
 }
 
-template <int BM, int BN, bool VEC>
+template <int BM, int BN, bool VEC, bool TA, bool TB>
 int launch(const double* A, const double* B, double* C, int M, int N, int K, hipStream_t st) {
-    using T = Tile<BM, BN>;
+    constexpr int SMEM_BYTES = 2 * (Operand<BM, TA, VEC>::TILE + Operand<BN, !TB, VEC>::TILE)
+                               * (int)sizeof(double);
     static bool attr_set = false;
-    auto kern = dgemm_mfma_kernel<BM, BN, VEC>;
+    auto kern = dgemm_mfma_kernel<BM, BN, VEC, TA, TB>;
     if (!attr_set) {
         if (!ESHKOL_HIP_OK(hipFuncSetAttribute((const void*)kern,
-                hipFuncAttributeMaxDynamicSharedMemorySize, T::SMEM_BYTES))) return -1;
+                hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES))) return -1;
         attr_set = true;
     }
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const long long nwg = (long long)tiles_m * tiles_n;
     if (nwg > 0x7fffffffLL) return -1;
-    hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(256), T::SMEM_BYTES, st,
+    hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(256), SMEM_BYTES, st,
                        A, B, C, M, N, K, tiles_m, tiles_n);
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 
+template <bool TA, bool TB>
+int launch_shape(const double* A, const double* B, double* C, int m, int n, int k, bool vec, hipStream_t st) {
+    /* Small outputs cannot fill 256 CUs with 128x128 tiles: use 64x64 there. */
+    const long long big_tiles = (long long)((m + 127) / 128) * (long long)((n + 127) / 128);
+    if (big_tiles >= 256) {
+        return vec ? launch<128, 128, true, TA, TB>(A, B, C, m, n, k, st)
+                   : launch<128, 128, false, TA, TB>(A, B, C, m, n, k, st);
+    }
+    return vec ? launch<64, 64, true, TA, TB>(A, B, C, m, n, k, st)
+               : launch<64, 64, false, TA, TB>(A, B, C, m, n, k, st);
+}
+
 }  // namespace
+
+extern "C" int hip_dgemm_f64_ex(const double* A, const double* B, double* C,
+                                uint64_t M, uint64_t K, uint64_t N,
+                                int trans_a, int trans_b, void* stream) {
+    if (!A || !B || !C || M == 0 || K == 0 || N == 0) return -1;
+    if (M > 0x7fffffffULL || K > 0x7fffffffULL || N > 0x7fffffffULL) return -1;
+    if (trans_a && trans_b) return -1;   /* no caller needs it: (B*A)^T, transpose the result instead */
+    hipStream_t st = (hipStream_t)stream;
+    /* row pitches: A is [M][K] or [K][M]; B is [K][N] or [N][K] */
+    const uint64_t pitch_a = trans_a ? M : K, pitch_b = trans_b ? K : N;
+    const bool vec = (pitch_a % 2 == 0) && (pitch_b % 2 == 0) &&
+                     ((uintptr_t)A % 16 == 0) && ((uintptr_t)B % 16 == 0);
+    const int m = (int)M, n = (int)N, k = (int)K;
+    if (trans_a) return launch_shape<true, false>(A, B, C, m, n, k, vec, st);
+    if (trans_b) return launch_shape<false, true>(A, B, C, m, n, k, vec, st);
+    return launch_shape<false, false>(A, B, C, m, n, k, vec, st);
+}
 
 extern "C" int hip_dgemm_f64(const double* A, const double* B, double* C,
                              uint64_t M, uint64_t K, uint64_t N, void* stream) {
-    if (!A || !B || !C || M == 0 || K == 0 || N == 0) return -1;
-    if (M > 0x7fffffffULL || K > 0x7fffffffULL || N > 0x7fffffffULL) return -1;
-    hipStream_t st = (hipStream_t)stream;
-    const bool vec = (K % 2 == 0) && (N % 2 == 0) &&
-                     ((uintptr_t)A % 16 == 0) && ((uintptr_t)B % 16 == 0);
-    const int m = (int)M, n = (int)N, k = (int)K;
-    /* Small outputs cannot fill 256 CUs with 128x128 tiles: use 64x64 there. */
-    const long long big_tiles = (long long)((M + 127) / 128) * (long long)((N + 127) / 128);
-    if (big_tiles >= 256) {
-        return vec ? launch<128, 128, true>(A, B, C, m, n, k, st)
-                   : launch<128, 128, false>(A, B, C, m, n, k, st);
-    }
-    return vec ? launch<64, 64, true>(A, B, C, m, n, k, st)
-               : launch<64, 64, false>(A, B, C, m, n, k, st);
+    return hip_dgemm_f64_ex(A, B, C, M, K, N, 0, 0, stream);
 }

@@ -135,15 +135,17 @@ const TierEnv& tier_env(void) { std::call_once(g_env_once, parse_env); return g_
 /* ---- cost model of the accuracy-budget selector --------------------------
  * Same shape as the reference's (gpu_memory_cuda.cpp:485-566): per kernel
  * t_ns = overhead + work/peak, peak self-calibrates upward from measured calls.
- * Seeds are MI355X measurements of this library at 8192^3 and 1024^3. */
+ * Seeds are MI355X measurements of this library: the line through the times
+ * at 4096^3 and 8192^3 for the slice tiers (T1 2.54 ms ... T8 24.0 ms at
+ * 8192^3), 1024^3 and 8192^3 for the native kernel (0.059 ms, 17.5 ms). */
 const double OZAKI_TOL[9] = { 1.0, 1e-3, 1e-5, 1e-7, 1e-9, 1e-11, 1e-13, 1e-14, 1e-14 };
 struct GemmModel { double overhead_ns; double peak_gflops; };
 GemmModel g_model[9] = {
-    /* native */ {  30000.0,  55000.0 },
-    /* T1 */ { 250000.0, 400000.0 }, /* T2 */ { 270000.0, 230000.0 },
-    /* T3 */ { 300000.0, 150000.0 }, /* T4 */ { 330000.0, 105000.0 },
-    /* T5 */ { 360000.0,  78000.0 }, /* T6 */ { 400000.0,  60000.0 },
-    /* T7 */ { 440000.0,  47000.0 }, /* T8 */ { 480000.0,  38000.0 } };
+    /* native */ {  25000.0,  63000.0 },
+    /* T1 */ { 250000.0, 479000.0 }, /* T2 */ { 290000.0, 282000.0 },
+    /* T3 */ { 360000.0, 183000.0 }, /* T4 */ { 290000.0, 126000.0 },
+    /* T5 */ { 290000.0,  93000.0 }, /* T6 */ { 320000.0,  71800.0 },
+    /* T7 */ { 360000.0,  57000.0 }, /* T8 */ { 400000.0,  46500.0 } };
 const double OZAKI_SAFETY = 1.15;
 std::mutex g_model_mutex;
 
@@ -255,8 +257,10 @@ bool is_hip_buffer(const EshkolGPUBuffer* b) { return b && b->backend == ESHKOL_
 
 /* ---- matmul tiers -------------------------------------------------------- */
 
+/* C[MxN] = op(A)*op(B) on the tier the environment selects; ta/tb mark an
+ * operand the caller holds transposed (A as [K][M], B as [N][K]). */
 int hip_matmul_f64(EshkolGPUBuffer* A, EshkolGPUBuffer* B, EshkolGPUBuffer* C,
-                   uint64_t M, uint64_t K, uint64_t N) {
+                   uint64_t M, uint64_t K, uint64_t N, int ta = 0, int tb = 0) {
     const TierEnv& env = tier_env();
     const double* dA = (const double*)A->device_ptr;
     const double* dB = (const double*)B->device_ptr;
@@ -285,13 +289,13 @@ int hip_matmul_f64(EshkolGPUBuffer* A, EshkolGPUBuffer* B, EshkolGPUBuffer* C,
             GPU_LOG("matmul %llux%llu @ %llux%llu -> Ozaki-II CRT exact (%s)",
                     (unsigned long long)M, (unsigned long long)K, (unsigned long long)K,
                     (unsigned long long)N, why);
-            rc = hip_matmul_ozaki_crt_f64(dA, dB, dC, M, K, N, env.num_moduli, env.adaptive ? 1 : 0,
-                                          nullptr, 0, g_stream);
+            rc = hip_matmul_ozaki_crt_f64_ex(dA, dB, dC, M, K, N, ta, tb, env.num_moduli,
+                                             env.adaptive ? 1 : 0, nullptr, 0, g_stream);
         } else {
             GPU_LOG("matmul %llux%llu @ %llux%llu -> INT8-Ozaki T=%d (%s, ~%.2fx vs native)",
                     (unsigned long long)M, (unsigned long long)K, (unsigned long long)K,
                     (unsigned long long)N, ozT, why, pred);
-            rc = hip_matmul_ozaki_int8_f64(dA, dB, dC, M, K, N, ozT, g_stream);
+            rc = hip_matmul_ozaki_int8_f64_ex(dA, dB, dC, M, K, N, ta, tb, ozT, g_stream);
         }
         if (rc == 0 && ESHKOL_HIP_OK(hipStreamSynchronize(g_stream))) {
             double ns = std::chrono::duration<double, std::nano>(std::chrono::steady_clock::now() - t0).count();
@@ -312,7 +316,7 @@ int hip_matmul_f64(EshkolGPUBuffer* A, EshkolGPUBuffer* B, EshkolGPUBuffer* C,
     }
 
     auto t0 = std::chrono::steady_clock::now();
-    if (hip_dgemm_f64(dA, dB, dC, M, K, N, g_stream) != 0) return -1;
+    if (hip_dgemm_f64_ex(dA, dB, dC, M, K, N, ta, tb, g_stream) != 0) return -1;
     if (!ESHKOL_HIP_OK(hipStreamSynchronize(g_stream))) return -1;
     double ns = std::chrono::duration<double, std::nano>(std::chrono::steady_clock::now() - t0).count();
     calibrate(0, work, ns);
@@ -521,6 +525,45 @@ int eshkol_gpu_matmul_f64(EshkolGPUBuffer* A, EshkolGPUBuffer* B, EshkolGPUBuffe
     matmul_fn f = host_matmul();
     if (!f || !A->host_ptr || !B->host_ptr || !C->host_ptr) return -1;
     f((const double*)A->host_ptr, (const double*)B->host_ptr, (double*)C->host_ptr, M, K, N);
+    return 0;
+}
+
+/* Gradients of C = A*B for device-resident buffers: grad_A[MxK] = grad_out *
+ * B^T, grad_B[KxN] = A^T * grad_out, each through the tier the environment
+ * selects for a forward product of that shape. Takes the place of the GPU
+ * branch of eshkol_matmul_backward_f64 (reference lib/backend/blas_backend.cpp:
+ * 968-1003: two host transposes, six wraps, two eshkol_gpu_matmul_f64 calls). */
+int eshkol_gpu_matmul_backward_f64(EshkolGPUBuffer* grad_out, EshkolGPUBuffer* A, EshkolGPUBuffer* B,
+                                   EshkolGPUBuffer* grad_A, EshkolGPUBuffer* grad_B,
+                                   uint64_t M, uint64_t K, uint64_t N) {
+    if (!grad_out || !A || !B || (!grad_A && !grad_B)) return -1;
+    if (g_backend != ESHKOL_GPU_HIP) return -1;
+    if (!is_hip_buffer(grad_out) || !is_hip_buffer(A) || !is_hip_buffer(B)) return -1;
+    if ((grad_A && !is_hip_buffer(grad_A)) || (grad_B && !is_hip_buffer(grad_B))) return -1;
+    std::lock_guard<std::recursive_mutex> g(g_gpu_mutex);
+    /* grad_A: rows M, contraction N, columns K; B[KxN] is the second operand held transposed */
+    if (grad_A && hip_matmul_f64(grad_out, B, grad_A, M, N, K, 0, 1) != 0) return -1;
+    /* grad_B: rows K, contraction M, columns N; A[MxK] is the first operand held transposed */
+    if (grad_B && hip_matmul_f64(A, grad_out, grad_B, K, M, N, 1, 0) != 0) return -1;
+    return 0;
+}
+
+int hip_matmul_backward_f64(const double* grad_out, const double* A, const double* B,
+                            double* grad_A, double* grad_B,
+                            uint64_t M, uint64_t K, uint64_t N,
+                            int tier, int T, void* stream) {
+    if (!grad_out || !A || !B || (!grad_A && !grad_B)) return -1;
+    auto one = [&](const double* X, const double* Y, double* Z, uint64_t m, uint64_t k, uint64_t n,
+                   int ta, int tb) -> int {
+        switch (tier) {
+            case 0: return hip_dgemm_f64_ex(X, Y, Z, m, k, n, ta, tb, stream);
+            case 1: return hip_matmul_ozaki_int8_f64_ex(X, Y, Z, m, k, n, ta, tb, T, stream);
+            case 2: return hip_matmul_ozaki_crt_f64_ex(X, Y, Z, m, k, n, ta, tb, 16, 0, nullptr, 0, stream);
+        }
+        return -1;
+    };
+    if (grad_A && one(grad_out, B, grad_A, M, N, K, 0, 1) != 0) return -1;
+    if (grad_B && one(A, grad_out, grad_B, K, M, N, 1, 0) != 0) return -1;
     return 0;
 }
 

@@ -408,21 +408,37 @@ extern "C" int hip_hgemm_16(const uint16_t* A, const uint16_t* Bt, uint64_t M, u
     return hgemm_any(A, Bt, M, K, N, ld, is_bf16, 0, C, (hipStream_t)stream);
 }
 
-extern "C" int hip_matmul_reduced_f64(const double* A, const double* B, double* C,
-                                      uint64_t M, uint64_t K, uint64_t N,
-                                      int dtype, int round_output, void* stream) {
+extern "C" int hip_matmul_reduced_f64_ex(const double* A, const double* B, double* C,
+                                         uint64_t M, uint64_t K, uint64_t N,
+                                         int trans_a, int trans_b,
+                                         int dtype, int round_output, void* stream) {
     if (!A || !B || !C || M == 0 || K == 0 || N == 0) return -1;
     if (dtype != 2 && dtype != 3) return -1;
     if (M > 0x7fffffffULL || K > 0x3fffffffULL || N > 0x7fffffffULL) return -1;
     hipStream_t st = (hipStream_t)stream;
     const int is_bf16 = (dtype == 3);
     const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ld = round_up_sz(K, 128);
-    double* Bt = (double*)eshkol_hip_workspace(WS_BT, K * N * sizeof(double));
+    const double* Bt = B;
+    if (!trans_b) {
+        double* t = (double*)eshkol_hip_workspace(WS_BT, K * N * sizeof(double));
+        if (!t || hip_transpose_f64(B, t, K, N, st) != 0) return -1;
+        Bt = t;
+    }
+    if (trans_a) {
+        double* t = (double*)eshkol_hip_workspace(WS_AT, M * K * sizeof(double));
+        if (!t || hip_transpose_f64(A, t, K, M, st) != 0) return -1;
+        A = t;
+    }
     uint16_t* A16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_A, Mp * ld * 2);
     uint16_t* B16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_B, Np * ld * 2);
-    if (!Bt || !A16 || !B16) return -1;
-    if (hip_transpose_f64(B, Bt, K, N, st) != 0) return -1;
+    if (!A16 || !B16) return -1;
     if (hip_convert_f64_to_16(A, A16, M, K, Mp, ld, is_bf16, st) != 0) return -1;
     if (hip_convert_f64_to_16(Bt, B16, N, K, Np, ld, is_bf16, st) != 0) return -1;
     return hgemm_any(A16, B16, M, K, N, ld, is_bf16, round_output ? 2 : 1, C, st);
+}
+
+extern "C" int hip_matmul_reduced_f64(const double* A, const double* B, double* C,
+                                      uint64_t M, uint64_t K, uint64_t N,
+                                      int dtype, int round_output, void* stream) {
+    return hip_matmul_reduced_f64_ex(A, B, C, M, K, N, 0, 0, dtype, round_output, stream);
 }

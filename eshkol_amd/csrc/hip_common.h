@@ -25,6 +25,7 @@ hipStream_t eshkol_hip_stream(void);
  * matmul does not pay hipMalloc/hipFree per call. Returns NULL on failure. */
 enum {
     WS_BT = 0,      /* transposed fp64 copy of B                          */
+    WS_AT,          /* row-major fp64 copy of an A the caller holds transposed */
     WS_APLANES,     /* int8 planes of A                                   */
     WS_BPLANES,     /* int8 planes of B (transposed, K contiguous)        */
     WS_PRODUCTS,    /* int8 residue products / int32 diagonal buffers     */

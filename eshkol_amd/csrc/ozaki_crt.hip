@@ -306,10 +306,11 @@ extern "C" int hip_ozaki_crt_last_stages(HipOzakiCrtStages* out) {
     return 0;
 }
 
-extern "C" int hip_matmul_ozaki_crt_f64(const double* A, const double* B, double* C,
-                                        uint64_t M, uint64_t K, uint64_t N,
-                                        int num_moduli, int adaptive,
-                                        const double* bias, int act, void* stream) {
+extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, double* C,
+                                           uint64_t M, uint64_t K, uint64_t N,
+                                           int trans_a, int trans_b,
+                                           int num_moduli, int adaptive,
+                                           const double* bias, int act, void* stream) {
     if (!A || !B || !C || M == 0 || K == 0 || N == 0) return -1;
     if (M > 0x7fffffffULL || N > 0x7fffffffULL) return -1;
     /* int32 accumulation of |a*b| <= 128*128 is exact while K*16384 < 2^31 */
@@ -332,12 +333,25 @@ extern "C" int hip_matmul_ozaki_crt_f64(const double* A, const double* B, double
     if (ensure_tables(st) != 0) return -1;
 
     const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ldk = round_up_sz(K, 256);
-    double* Bt   = (double*)eshkol_hip_workspace(WS_BT, K * N * sizeof(double));
+    /* Both operands are split along rows with k contiguous: B goes through its
+     * transpose unless the caller already holds it, A only if the caller holds
+     * A transposed. */
+    const double* Bt = B;
+    if (!trans_b) {
+        double* t = (double*)eshkol_hip_workspace(WS_BT, K * N * sizeof(double));
+        if (!t || hip_transpose_f64(B, t, K, N, (hipStream_t)stream) != 0) return -1;
+        Bt = t;
+    }
+    if (trans_a) {
+        double* t = (double*)eshkol_hip_workspace(WS_AT, M * K * sizeof(double));
+        if (!t || hip_transpose_f64(A, t, K, M, (hipStream_t)stream) != 0) return -1;
+        A = t;
+    }
     double* amax = (double*)eshkol_hip_workspace(WS_ROWSCALE, M * sizeof(double));
     double* bmax = (double*)eshkol_hip_workspace(WS_COLSCALE, N * sizeof(double));
     int32_t* dmu = (int32_t*)eshkol_hip_workspace(WS_ROWSHIFT, M * sizeof(int32_t));
     int32_t* dnu = (int32_t*)eshkol_hip_workspace(WS_COLSHIFT, N * sizeof(int32_t));
-    if (!Bt || !amax || !bmax || !dmu || !dnu) return -1;
+    if (!amax || !bmax || !dmu || !dnu) return -1;
     char* host = (char*)pinned((M + N) * (sizeof(double) + sizeof(int32_t)));
     if (!host) return -1;
     double* h_amax = (double*)host;
@@ -345,7 +359,6 @@ extern "C" int hip_matmul_ozaki_crt_f64(const double* A, const double* B, double
     int32_t* h_mu = (int32_t*)(h_bmax + N);
     int32_t* h_nu = h_mu + M;
 
-    if (hip_transpose_f64(B, Bt, K, N, st) != 0) return -1;
     if (hip_rowabsmax_f64(A, M, K, 0.0, amax, st) != 0) return -1;
     if (hip_rowabsmax_f64(Bt, N, K, 0.0, bmax, st) != 0) return -1;
     if (!ESHKOL_HIP_OK(hipMemcpyAsync(h_amax, amax, M * sizeof(double), hipMemcpyDeviceToHost, st))) return -1;
@@ -420,4 +433,11 @@ extern "C" int hip_matmul_ozaki_crt_f64(const double* A, const double* B, double
     g_last.rows_a_padded = Mp; g_last.rows_b_padded = Np; g_last.ldk = ldk;
     g_last.num_moduli = num_moduli; g_last.E = E;
     return 0;
+}
+
+extern "C" int hip_matmul_ozaki_crt_f64(const double* A, const double* B, double* C,
+                                        uint64_t M, uint64_t K, uint64_t N,
+                                        int num_moduli, int adaptive,
+                                        const double* bias, int act, void* stream) {
+    return hip_matmul_ozaki_crt_f64_ex(A, B, C, M, K, N, 0, 0, num_moduli, adaptive, bias, act, stream);
 }

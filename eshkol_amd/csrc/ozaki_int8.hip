@@ -133,8 +133,9 @@ extern "C" int hip_ozaki_int8_last_stages(HipOzakiInt8Stages* out) {
     return 0;
 }
 
-extern "C" int hip_matmul_ozaki_int8_f64(const double* A, const double* B, double* C,
-                                         uint64_t M, uint64_t K, uint64_t N, int T, void* stream) {
+extern "C" int hip_matmul_ozaki_int8_f64_ex(const double* A, const double* B, double* C,
+                                            uint64_t M, uint64_t K, uint64_t N,
+                                            int trans_a, int trans_b, int T, void* stream) {
     if (!A || !B || !C || M == 0 || K == 0 || N == 0) return -1;
     if (M > 0x7fffffffULL || K > 0x7fffffffULL || N > 0x7fffffffULL) return -1;
     if (T < 1 || T > 8) return -1;
@@ -177,17 +178,29 @@ extern "C" int hip_matmul_ozaki_int8_f64(const double* A, const double* B, doubl
     plan->first[nbuf] = npairs;
 
     const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ldk = round_up_sz(K, 256);
-    double* Bt   = (double*)eshkol_hip_workspace(WS_BT, K * N * sizeof(double));
+    /* Both operands are sliced along rows with k contiguous: B goes through its
+     * transpose unless the caller already holds it, A only if the caller holds
+     * A transposed. */
+    const double* Bt = B;
+    if (!trans_b) {
+        double* t = (double*)eshkol_hip_workspace(WS_BT, K * N * sizeof(double));
+        if (!t || hip_transpose_f64(B, t, K, N, st) != 0) return -1;
+        Bt = t;
+    }
+    if (trans_a) {
+        double* t = (double*)eshkol_hip_workspace(WS_AT, M * K * sizeof(double));
+        if (!t || hip_transpose_f64(A, t, K, M, st) != 0) return -1;
+        A = t;
+    }
     double* rmax = (double*)eshkol_hip_workspace(WS_ROWSCALE, M * sizeof(double));
     double* cmax = (double*)eshkol_hip_workspace(WS_COLSCALE, N * sizeof(double));
     Plan* dplan  = (Plan*)eshkol_hip_workspace(WS_MISC, sizeof(Plan));
     int8_t* As   = (int8_t*)eshkol_hip_workspace(WS_APLANES, (size_t)s * Mp * ldk);
     int8_t* Bs   = (int8_t*)eshkol_hip_workspace(WS_BPLANES, (size_t)s * Np * ldk);
     int32_t* G   = (int32_t*)eshkol_hip_workspace(WS_PRODUCTS, (size_t)nbuf * M * N * sizeof(int32_t));
-    if (!Bt || !rmax || !cmax || !dplan || !As || !Bs || !G) return -1;
+    if (!rmax || !cmax || !dplan || !As || !Bs || !G) return -1;
 
     if (!ESHKOL_HIP_OK(hipMemcpyAsync(dplan, plan, sizeof(Plan), hipMemcpyHostToDevice, st))) return -1;
-    if (hip_transpose_f64(B, Bt, K, N, st) != 0) return -1;
     if (hip_rowabsmax_f64(A, M, K, 1.0, rmax, st) != 0) return -1;
     if (hip_rowabsmax_f64(Bt, N, K, 1.0, cmax, st) != 0) return -1;
     /* NaN/Inf input is unspecified in the reference; here it is detected through
@@ -215,4 +228,9 @@ extern "C" int hip_matmul_ozaki_int8_f64(const double* A, const double* B, doubl
     g_last.rows_a_padded = Mp; g_last.rows_b_padded = Np; g_last.ldk = ldk;
     g_last.s = s; g_last.nbuf = nbuf;
     return 0;
+}
+
+extern "C" int hip_matmul_ozaki_int8_f64(const double* A, const double* B, double* C,
+                                         uint64_t M, uint64_t K, uint64_t N, int T, void* stream) {
+    return hip_matmul_ozaki_int8_f64_ex(A, B, C, M, K, N, 0, 0, T, stream);
 }

@@ -38,6 +38,15 @@ void* eshkol_hip_get_stream(void);
 int hip_dgemm_f64(const double* A, const double* B, double* C,
                   uint64_t M, uint64_t K, uint64_t N, void* stream);
 
+/* C[MxN] = op(A)*op(B) with an operand held transposed: trans_a != 0 means A
+ * points at A^T stored [K][M]; trans_b != 0 means B points at B^T stored
+ * [N][K] (not both). What cblas_dgemm's CblasTrans flags give the reference's
+ * backward pass (lib/backend/blas_backend.cpp:1013-1024); its GPU branch makes
+ * transposed host copies instead (:969-977). */
+int hip_dgemm_f64_ex(const double* A, const double* B, double* C,
+                     uint64_t M, uint64_t K, uint64_t N,
+                     int trans_a, int trans_b, void* stream);
+
 /* Single precision, replaces cublasSgemm at gpu_memory_cuda.cpp:658-665. */
 int hip_sgemm_f32(const float* A, const float* B, float* C,
                   uint64_t M, uint64_t K, uint64_t N, void* stream);
@@ -182,6 +191,34 @@ int hip_hgemm_16(const uint16_t* A, const uint16_t* Bt, uint64_t M, uint64_t K, 
  * out[i][k] with pitch ld and rows_padded rows, padding zero. */
 int hip_convert_f64_to_16(const double* in, uint16_t* out, uint64_t rows, uint64_t cols,
                           uint64_t rows_padded, uint64_t ld, int is_bf16, void* stream);
+
+/* ---- operands held transposed, and the backward pass ---------------------------
+ * The tier pipelines with the trans_a / trans_b meaning of hip_dgemm_f64_ex.
+ * The Ozaki and reduced tiers split both operands along rows with k
+ * contiguous, so a B the caller holds transposed saves them their transpose
+ * pass, and an A held transposed costs one. */
+int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, double* C,
+                                uint64_t M, uint64_t K, uint64_t N,
+                                int trans_a, int trans_b, int num_moduli, int adaptive,
+                                const double* bias, int act, void* stream);
+int hip_matmul_ozaki_int8_f64_ex(const double* A, const double* B, double* C,
+                                 uint64_t M, uint64_t K, uint64_t N,
+                                 int trans_a, int trans_b, int T, void* stream);
+int hip_matmul_reduced_f64_ex(const double* A, const double* B, double* C,
+                              uint64_t M, uint64_t K, uint64_t N,
+                              int trans_a, int trans_b,
+                              int dtype, int round_output, void* stream);
+
+/* Gradients of C = A*B (eshkol_matmul_backward_f64, lib/backend/blas_backend.cpp:
+ * 924-1039): grad_A[MxK] = grad_out[MxN] * B^T and grad_B[KxN] = A^T * grad_out,
+ * straight from the saved row-major A[MxK] and B[KxN] with no transposed
+ * copies (the reference's GPU branch transposes both on the host, :969-977).
+ * tier: 0 native fp64, 1 INT8 slices with T, 2 Ozaki-II CRT (16 moduli).
+ * Either gradient pointer may be NULL to skip it. */
+int hip_matmul_backward_f64(const double* grad_out, const double* A, const double* B,
+                            double* grad_A, double* grad_B,
+                            uint64_t M, uint64_t K, uint64_t N,
+                            int tier, int T, void* stream);
 
 /* ---- measurement support ----------------------------------------------------
  * Rate the device sustains on a register-only MFMA loop (kind 0 fp64 flop/s,

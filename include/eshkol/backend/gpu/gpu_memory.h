@@ -92,6 +92,16 @@ int eshkol_gpu_matmul_f64(EshkolGPUBuffer* A, EshkolGPUBuffer* B, EshkolGPUBuffe
 int eshkol_gpu_matmul_f32(EshkolGPUBuffer* A, EshkolGPUBuffer* B, EshkolGPUBuffer* C,
                           uint64_t M, uint64_t K, uint64_t N);
 
+/* Gradients of C = A*B: grad_A[MxK] = grad_out[MxN] * B^T and grad_B[KxN] =
+ * A^T * grad_out from the saved row-major operands, same tier selection as
+ * the forward product. An addition to the reference header: it replaces the
+ * GPU branch inside eshkol_matmul_backward_f64 (lib/backend/blas_backend.cpp:
+ * 968-1003), which transposes both operands on the host and calls
+ * eshkol_gpu_matmul_f64 twice. Either gradient buffer may be NULL. */
+int eshkol_gpu_matmul_backward_f64(EshkolGPUBuffer* grad_out, EshkolGPUBuffer* A, EshkolGPUBuffer* B,
+                                   EshkolGPUBuffer* grad_A, EshkolGPUBuffer* grad_B,
+                                   uint64_t M, uint64_t K, uint64_t N);
+
 /* ---- thresholds: reference gpu_memory.h:261-280 -------------------------- */
 extern size_t g_gpu_threshold;
 void eshkol_gpu_set_threshold(size_t threshold);

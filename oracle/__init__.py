@@ -69,6 +69,20 @@ def matmul_f64(A, B, fused=True):
     return out
 
 
+def matmul_backward_f64(G, A, B, fused=True):
+    """(grad_A, grad_B) for C = A @ B given grad_out G."""
+    G, A, B = _f64(G), _f64(A), _f64(B)
+    M, K = A.shape
+    N = B.shape[1]
+    assert G.shape == (M, N) and B.shape[0] == K
+    gA, gB = np.empty((M, K)), np.empty((K, N))
+    L = lib()
+    L.oracle_matmul_set_fused(1 if fused else 0)
+    L.oracle_matmul_backward_f64(_d(G), _d(A), _d(B), _d(gA), _d(gB), u64(M), u64(K), u64(N))
+    L.oracle_matmul_set_fused(1)
+    return gA, gB
+
+
 def batch_matmul_f64(a, b):
     a, b = _f64(a), _f64(b)
     batch, M, K = a.shape

@@ -60,6 +60,13 @@ void oracle_matmul_f64(const double* A, const double* B, double* C,
 void oracle_batch_matmul_f64(const double* a, const double* b, double* c,
                              int64_t batch, int64_t M, int64_t K, int64_t N);
 
+/* eshkol_matmul_backward_f64, blas_backend.cpp:924-1039 (the scalar loops of a
+ * non-BLAS, non-GPU build): grad_A[MxK] = grad_out[MxN] * B^T, grad_B[KxN] =
+ * A^T * grad_out, each output accumulated in ascending contraction order. */
+void oracle_matmul_backward_f64(const double* grad_out, const double* saved_A, const double* saved_B,
+                                double* grad_A, double* grad_B,
+                                uint64_t M, uint64_t K, uint64_t N);
+
 /* ---- reduced-precision tier (lib/core/runtime_tensor_dtype.cpp) ---------- */
 
 /* reduce_precision, runtime_tensor_dtype.cpp:37-145. dtype codes: 0 f64,

@@ -92,6 +92,25 @@ void oracle_batch_matmul_f64(const double* a, const double* b, double* c,
     }
 }
 
+/* eshkol_matmul_backward_f64, blas_backend.cpp:924-1039, non-BLAS non-GPU
+ * build: both the tiny-matrix branch (941-954) and the scalar fallback
+ * (1029-1038) are the same two accumulation loops, n ascending for grad_A and
+ * i ascending for grad_B, `+=` contracting to fma with -mfma. */
+void oracle_matmul_backward_f64(const double* grad_out, const double* saved_A, const double* saved_B,
+                                double* grad_A, double* grad_B,
+                                uint64_t M, uint64_t K, uint64_t N) {
+    memset(grad_A, 0, (size_t)(M * K) * sizeof(double));
+    for (uint64_t i = 0; i < M; i++)
+        for (uint64_t j = 0; j < K; j++)
+            for (uint64_t n = 0; n < N; n++)
+                grad_A[i * K + j] = madd(grad_out[i * N + n], saved_B[j * N + n], grad_A[i * K + j]);
+    memset(grad_B, 0, (size_t)(K * N) * sizeof(double));
+    for (uint64_t j = 0; j < K; j++)
+        for (uint64_t n = 0; n < N; n++)
+            for (uint64_t i = 0; i < M; i++)
+                grad_B[j * N + n] = madd(saved_A[i * K + j], grad_out[i * N + n], grad_B[j * N + n]);
+}
+
 /* ---- reduced precision --------------------------------------------------- */
 
 /* runtime_tensor_dtype.cpp:37-93 */

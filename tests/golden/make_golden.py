@@ -6,7 +6,7 @@ oracle/_ref/libeshkol_ref.so (AVX2+FMA build) and libeshkol_ref_sse2.so
     make -C oracle ref && python tests/golden/make_golden.py
 
 Outputs (committed): tests/golden/fp64_matmul.npz, fp64_batch.npz,
-reduce_precision.npz. Inputs come from eshkol_amd.synth (seeded), small cases
+fp64_backward.npz, reduce_precision.npz. Inputs come from eshkol_amd.synth (seeded), small cases
 are stored whole, the 256^3 case as a checksum plus sampled entries.
 """
 import ctypes as C
@@ -28,6 +28,7 @@ def ref(path):
     lib = C.CDLL(path)
     lib.eshkol_matmul_f64.argtypes = [dp, dp, dp, u64, u64, u64]
     lib.eshkol_batch_matmul_f64.argtypes = [dp, dp, dp, i64, i64, i64, i64]
+    lib.eshkol_matmul_backward_f64.argtypes = [dp, dp, dp, dp, dp, u64, u64, u64]
     lib.eshkol_tensor_reduce_precision_value.argtypes = [C.c_double, i64]
     lib.eshkol_tensor_reduce_precision_value.restype = C.c_double
     return lib
@@ -38,6 +39,7 @@ def P(a):
 
 
 CASES = [(2, 2, 2), (4, 4, 4), (3, 5, 4), (5, 7, 3), (1, 100, 1), (64, 64, 64), (65, 67, 66), (37, 130, 9)]
+BACKWARD_CASES = [(2, 2, 2), (4, 4, 4), (3, 5, 4), (17, 23, 11), (64, 48, 80), (1, 33, 1)]
 SAMPLES_256 = [(0, 0), (0, 255), (255, 0), (255, 255), (128, 128), (17, 201), (64, 63), (63, 64), (100, 3)]
 
 
@@ -74,6 +76,20 @@ def main():
         lib.eshkol_batch_matmul_f64(P(a), P(b), P(c), 3, 17, 23, 11)
         bo[tag] = c
     np.savez(os.path.join(HERE, "fp64_batch.npz"), **bo)
+
+    # matmul backward (eshkol_matmul_backward_f64): grad_A, grad_B for seeded G, A, B
+    wo = {}
+    for ci, (M, K, N) in enumerate(BACKWARD_CASES):
+        G = synth.normal(300 + ci, (M, N))
+        A = synth.normal(400 + ci, (M, K))
+        B = synth.normal(500 + ci, (K, N))
+        for tag, lib in (("avx", avx), ("sse2", sse)):
+            gA, gB = np.empty((M, K)), np.empty((K, N))
+            lib.eshkol_matmul_backward_f64(P(G), P(A), P(B), P(gA), P(gB), M, K, N)
+            wo["case%d_%s_gradA" % (ci, tag)] = gA
+            wo["case%d_%s_gradB" % (ci, tag)] = gB
+        wo["case%d_shape" % ci] = np.array([M, K, N])
+    np.savez(os.path.join(HERE, "fp64_backward.npz"), **wo)
 
     vals = np.concatenate([
         synth.normal(11, (3000,)), synth.normal(12, (2000,)) * 1e-6, synth.normal(13, (1000,)) * 1e5,

@@ -1,0 +1,187 @@
+"""Matmul backward on the GPU through the C ABI: the transposed-operand forms
+of the native fp64 kernel, the tier pipelines fed operands the caller holds
+transposed, hip_matmul_backward_f64 and eshkol_gpu_matmul_backward_f64,
+against the oracle's restatement of eshkol_matmul_backward_f64
+(lib/backend/blas_backend.cpp:924-1039).
+
+Bars: native fp64 normwise <= 1e-14; Ozaki tiers bit-identical to the same
+tier on explicit transposed copies (the pipelines see the same k-contiguous
+operands either way) and to the oracle of that tier; integer cases exact."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import eshkol_amd as ea
+import oracle
+from eshkol_amd import synth
+from gpu_util import normwise, run_crt, run_int8, stream
+from test_gpu_dispatch import run_child
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-14
+
+SHAPES = [(1, 1, 1), (2, 3, 4), (5, 7, 3), (16, 16, 16), (64, 64, 64), (65, 67, 66), (37, 130, 9),
+          (129, 257, 131), (256, 256, 256), (300, 17, 500), (512, 1000, 64), (1000, 33, 1000),
+          (1024, 1024, 1024), (2050, 130, 2046)]
+
+
+def dev(x):
+    return ea.DeviceArray.from_host(np.ascontiguousarray(x, dtype=np.float64))
+
+
+def dgemm_ex(X, Y, m, k, n, ta, tb):
+    """C[m x n] = op(X) op(Y) with X, Y as the caller holds them."""
+    dX, dY, dZ = dev(X), dev(Y), ea.DeviceArray((m, n))
+    assert ea.load().hip_dgemm_f64_ex(dX.ptr, dY.ptr, dZ.ptr, m, k, n, ta, tb, stream()) == 0
+    ea.synchronize()
+    return dZ.download()
+
+
+def backward(G, A, B, tier, T=0):
+    M, K = A.shape
+    N = B.shape[1]
+    dG, dA, dB = dev(G), dev(A), dev(B)
+    gA, gB = ea.DeviceArray((M, K)), ea.DeviceArray((K, N))
+    rc = ea.load().hip_matmul_backward_f64(dG.ptr, dA.ptr, dB.ptr, gA.ptr, gB.ptr, M, K, N, tier, T, stream())
+    assert rc == 0
+    ea.synchronize()
+    return gA.download(), gB.download()
+
+
+@pytest.mark.parametrize("M,K,N", SHAPES)
+def test_native_transposed_operands_match_oracle(gpu, M, K, N):
+    print("dgemm_ex", M, K, N, flush=True)
+    A, B = synth.uniform(100 + M, (M, K)), synth.uniform(200 + N, (K, N))
+    ref = oracle.matmul_f64(A, B)
+    At, Bt = np.ascontiguousarray(A.T), np.ascontiguousarray(B.T)
+    assert normwise(dgemm_ex(A, Bt, M, K, N, 0, 1), ref, A, B) <= TOL
+    assert normwise(dgemm_ex(At, B, M, K, N, 1, 0), ref, A, B) <= TOL
+
+
+def test_native_rejects_both_transposed(gpu):
+    dX, dZ = dev(np.ones((4, 4))), ea.DeviceArray((4, 4))
+    assert ea.load().hip_dgemm_f64_ex(dX.ptr, dX.ptr, dZ.ptr, 4, 4, 4, 1, 1, stream()) == -1
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 1, 1), (2, 3, 4), (31, 33, 29), (130, 64, 258), (257, 300, 129)])
+def test_native_backward_integers_exact(gpu, M, K, N):
+    rng = np.random.default_rng(M * 7 + N)
+    G = rng.integers(-9, 10, (M, N)).astype(np.float64)
+    A = rng.integers(-9, 10, (M, K)).astype(np.float64)
+    B = rng.integers(-9, 10, (K, N)).astype(np.float64)
+    gA, gB = backward(G, A, B, 0)
+    assert np.array_equal(gA, G @ B.T) and np.array_equal(gB, A.T @ G)
+
+
+@pytest.mark.parametrize("M,K,N", [(64, 48, 80), (17, 23, 11), (300, 513, 130), (1024, 768, 512)])
+def test_native_backward_matches_oracle(gpu, M, K, N):
+    G, A, B = synth.normal(1 + M, (M, N)), synth.normal(2 + K, (M, K)), synth.normal(3 + N, (K, N))
+    gA, gB = backward(G, A, B, 0)
+    oA, oB = oracle.matmul_backward_f64(G, A, B)
+    assert normwise(gA, oA, G, B) <= TOL
+    assert normwise(gB, oB, A, G) <= TOL
+
+
+def test_skipping_one_gradient(gpu):
+    G, A, B = synth.normal(1, (40, 24)), synth.normal(2, (40, 56)), synth.normal(3, (56, 24))
+    dG, dA, dB = dev(G), dev(A), dev(B)
+    gA = ea.DeviceArray.from_host(np.full((40, 56), 7.0))
+    gB = ea.DeviceArray.from_host(np.full((56, 24), 7.0))
+    lib = ea.load()
+    assert lib.hip_matmul_backward_f64(dG.ptr, dA.ptr, dB.ptr, gA.ptr, None, 40, 56, 24, 0, 0, stream()) == 0
+    ea.synchronize()
+    assert np.all(gB.download() == 7.0) and normwise(gA.download(), G @ B.T, G, B) <= TOL
+    assert lib.hip_matmul_backward_f64(dG.ptr, dA.ptr, dB.ptr, None, None, 40, 56, 24, 0, 0, stream()) == -1
+
+
+@pytest.mark.parametrize("M,K,N", [(512, 512, 512), (520, 777, 300)])
+def test_crt_tier_backward_is_bit_identical_to_forward_on_transposed_copies(gpu, M, K, N):
+    G, A, B = synth.normal(5, (M, N)), synth.wide_range(6, (M, K)), synth.normal(7, (K, N))
+    gA, gB = backward(G, A, B, 2)
+    # the same tier on explicit copies, and the oracle of the tier
+    rc, fA, _ = run_crt(G, np.ascontiguousarray(B.T), want_stages=False)
+    assert rc == 0 and np.array_equal(gA, fA)
+    rc, fB, _ = run_crt(np.ascontiguousarray(A.T), G, want_stages=False)
+    assert rc == 0 and np.array_equal(gB, fB)
+    assert np.array_equal(gA, oracle.matmul_ozaki_crt(G, np.ascontiguousarray(B.T)))
+    assert np.array_equal(gB, oracle.matmul_ozaki_crt(np.ascontiguousarray(A.T), G))
+
+
+@pytest.mark.parametrize("T", [1, 4, 6])
+def test_int8_tier_backward_is_bit_identical_to_forward_on_transposed_copies(gpu, T):
+    M, K, N = 384, 300, 260
+    G, A, B = synth.normal(8, (M, N)), synth.normal(9, (M, K)), synth.uniform(10, (K, N))
+    gA, gB = backward(G, A, B, 1, T)
+    rc, fA, _ = run_int8(G, np.ascontiguousarray(B.T), T, want_stages=False)
+    assert rc == 0 and np.array_equal(gA, fA)
+    rc, fB, _ = run_int8(np.ascontiguousarray(A.T), G, T, want_stages=False)
+    assert rc == 0 and np.array_equal(gB, fB)
+    assert np.array_equal(gA, oracle.matmul_ozaki_int8(G, np.ascontiguousarray(B.T), T))
+    assert np.array_equal(gB, oracle.matmul_ozaki_int8(np.ascontiguousarray(A.T), G, T))
+
+
+def test_reduced_tier_with_operands_held_transposed(gpu):
+    M, K, N = 200, 330, 140
+    A = oracle.reduce_precision(synth.normal(11, (M, K)), 3)
+    B = oracle.reduce_precision(synth.normal(12, (K, N)), 3)
+    lib = ea.load()
+    dA, dB, dAt, dBt = dev(A), dev(B), dev(A.T), dev(B.T)
+    outs = []
+    for (x, y, ta, tb) in ((dA, dB, 0, 0), (dA, dBt, 0, 1), (dAt, dB, 1, 0)):
+        dC = ea.DeviceArray((M, N))
+        assert lib.hip_matmul_reduced_f64_ex(x.ptr, y.ptr, dC.ptr, M, K, N, ta, tb, 3, 0, stream()) == 0
+        ea.synchronize()
+        outs.append(dC.download())
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+
+
+def test_buffer_entry_default_tier(gpu):
+    lib = ea.load()
+    M, K, N = 260, 140, 330
+    G, A, B = synth.normal(13, (M, N)), synth.normal(14, (M, K)), synth.normal(15, (K, N))
+    dG, dA, dB = dev(G), dev(A), dev(B)
+    gA, gB = ea.DeviceArray((M, K)), ea.DeviceArray((K, N))
+    rc = lib.eshkol_gpu_matmul_backward_f64(C.byref(dG.buf), C.byref(dA.buf), C.byref(dB.buf),
+                                            C.byref(gA.buf), C.byref(gB.buf), M, K, N)
+    assert rc == 0
+    oA, oB = oracle.matmul_backward_f64(G, A, B)
+    assert normwise(gA.download(), oA, G, B) <= TOL and normwise(gB.download(), oB, A, G) <= TOL
+    # a buffer too small for its shape is refused
+    small = ea.DeviceArray((M, K - 1))
+    assert lib.eshkol_gpu_matmul_backward_f64(C.byref(dG.buf), C.byref(dA.buf), C.byref(dB.buf),
+                                              C.byref(small.buf), C.byref(gB.buf), M, K, N) == -1
+
+
+def test_buffer_entry_follows_the_tier_override(gpu):
+    r = run_child(r"""
+assert lib.eshkol_gpu_init() == 1
+M, K, N = 640, 512, 576
+G, A, B = synth.normal(16, (M, N)), synth.normal(17, (M, K)), synth.normal(18, (K, N))
+dG, dA, dB = (ea.DeviceArray.from_host(x) for x in (G, A, B))
+gA, gB = ea.DeviceArray((M, K)), ea.DeviceArray((K, N))
+assert lib.eshkol_gpu_matmul_backward_f64(C.byref(dG.buf), C.byref(dA.buf), C.byref(dB.buf),
+                                          C.byref(gA.buf), C.byref(gB.buf), M, K, N) == 0
+assert np.array_equal(gA.download(), oracle.matmul_ozaki_crt(G, np.ascontiguousarray(B.T)))
+assert np.array_equal(gB.download(), oracle.matmul_ozaki_crt(np.ascontiguousarray(A.T), G))
+""", env={"ESHKOL_HIP_F64_KERNEL": "ozaki-crt", "ESHKOL_GPU_VERBOSE": "1"})
+    assert r.stderr.count("[GPU] Ozaki-II: N=16") == 2
+    assert r.stderr.count("Ozaki-II CRT exact") == 2
+
+
+def test_full_size_backward_properties(gpu):
+    """8192-wide gradients: integer identities that hold in any summation order."""
+    M, K, N = 8192, 2048, 4096
+    i = np.arange(M * N, dtype=np.int64).reshape(M, N)
+    G = ((i * 7 + i // N) % 7 - 3).astype(np.float64)
+    i = np.arange(M * K, dtype=np.int64).reshape(M, K)
+    A = ((i * 5 + i // K) % 5 - 2).astype(np.float64)
+    i = np.arange(K * N, dtype=np.int64).reshape(K, N)
+    B = ((i * 3 + i // N) % 11 - 5).astype(np.float64)
+    gA, gB = backward(G, A, B, 0)
+    assert np.array_equal(gA.sum(axis=1), G @ B.sum(axis=0))          # row sums of G B^T
+    assert np.array_equal(gB.sum(axis=1), A.T @ G.sum(axis=1))        # row sums of A^T G
+    rows = [0, 1, 127, 128, 4095, M - 1]
+    assert np.array_equal(gA[rows], G[rows] @ B.T)
+    cols = [0, 1, 127, 128, 777, N - 1]
+    assert np.array_equal(gB[:, cols], A.T @ G[:, cols])
