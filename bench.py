@@ -63,7 +63,7 @@ def main():
     ap.add_argument("--size", type=int, default=8192)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-stages", action="store_true")
-    ap.add_argument("--only", default="", help="comma list of tiers to time besides native: crt,int8,reduced")
+    ap.add_argument("--only", default="", help="comma list of what to time besides native: crt,int8,reduced,mlp,backward,host")
     ap.add_argument("--pmc-probe", default="", choices=["", "dgemm", "crt", "int8", "reduced"],
                     help="run a calibration copy and three launches of one tier, for rocprofv3 --pmc")
     args = ap.parse_args()
@@ -81,7 +81,7 @@ def main():
     flops = 2.0 * M * N * K
     steps, warm = args.steps, args.warmup
     timer = ea.Timer()
-    want = set(args.only.split(",")) if args.only else {"crt", "int8", "reduced"}
+    want = set(args.only.split(",")) if args.only else {"crt", "int8", "reduced", "mlp", "backward", "host"}
 
     if args.pmc_probe:
         # Short program for `rocprofv3 --pmc ...` runs: a 512 MiB device copy of known size
@@ -242,6 +242,67 @@ def main():
         for d in (a16, b16, dBt, dC32):
             d.free()
         del Ar, Br
+
+    # ---- batched MLP forward through the exact tier: configuration 5 ---------------------------
+    if "mlp" in want:
+        batch, dims = 4096, (1024, 4096, 4096, 1024)
+        X = ea.DeviceArray.from_host(synth.normal(71, (batch, dims[0])))
+        Ws = [ea.DeviceArray.from_host(synth.xavier_uniform(72 + i, dims[i], dims[i + 1])) for i in range(3)]
+        bs = [ea.DeviceArray.from_host(synth.uniform(82 + i, (dims[i + 1],), -0.1, 0.1)) for i in range(3)]
+        acts = [ea.DeviceArray((batch, dims[i + 1])) for i in range(3)]
+
+        def mlp_forward():
+            src = X
+            for i in range(3):
+                rc = lib.hip_matmul_ozaki_crt_f64(src.ptr, Ws[i].ptr, acts[i].ptr, batch, dims[i], dims[i + 1],
+                                                  16, 0, bs[i].ptr, 1, st)
+                if rc != 0:
+                    return rc
+                src = acts[i]
+            return 0
+
+        devnull = os.open(os.devnull, os.O_WRONLY)
+        saved = os.dup(2)
+        os.dup2(devnull, 2)
+        try:
+            e7, w7 = timed(mlp_forward)
+        finally:
+            os.dup2(saved, 2)
+        mlp_flops = 2.0 * batch * sum(dims[i] * dims[i + 1] for i in range(3))
+        tiers["mlp_forward_exact_tier_batch4096_1024_4096_4096_1024"] = {
+            "ms": w7, "gflops_fp64_equiv": mlp_flops / (w7 * 1e-3) / 1e9,
+            "note": "three GEMMs, bias add + tanh fused in the reconstruct epilogue"}
+        log("mlp forward (exact tier): %.3f ms %.1f GFLOP/s-eq" % (w7, mlp_flops / (w7 * 1e-3) / 1e9))
+        for d in [X] + Ws + bs + acts:
+            d.free()
+
+    # ---- matmul backward (both gradients, native tier) ------------------------------------------
+    if "backward" in want:
+        dA.upload(A); dB.upload(B)
+        dG, dGA, dGB = ea.DeviceArray((M, N)), ea.DeviceArray((M, K)), ea.DeviceArray((K, N))
+        hip.hipMemcpy(dG.ptr, dA.ptr, dG.nbytes, ea.D2D)
+        e8, w8 = timed(lambda: lib.hip_matmul_backward_f64(dG.ptr, dA.ptr, dB.ptr, dGA.ptr, dGB.ptr, M, K, N, 0, 0, st),
+                       k=max(3, steps // 2), w=2)
+        tiers["backward_native_fp64_both_gradients"] = {
+            "ms": w8, "gflops": 2 * flops / (w8 * 1e-3) / 1e9,
+            "frac_of_peak": 2 * flops / (e8 * 1e-3) / PEAK["fp64_mfma"],
+            "note": "grad_A = G*B^T and grad_B = A^T*G from the saved operands, no transposed copies"}
+        log("backward native: %.3f ms %.1f GFLOP/s" % (w8, 2 * flops / (w8 * 1e-3) / 1e9))
+        for d in (dG, dGA, dGB):
+            d.free()
+
+    # ---- host-buffer entry: eshkol_matmul_dispatch on pageable host memory (PCIe inclusive) -----
+    if "host" in want:
+        Ch = np.empty((M, N))
+        t0 = time.perf_counter()
+        lib.eshkol_matmul_dispatch(A.ctypes.data, B.ctypes.data, Ch.ctypes.data, M, K, N, 0)
+        dt = time.perf_counter() - t0
+        tiers["host_buffers_eshkol_matmul_dispatch"] = {
+            "ms": dt * 1e3, "gflops": flops / dt / 1e9,
+            "note": "one call, operands and result in pageable host memory: two uploads, one download, "
+                    "device allocations included; never the headline value"}
+        log("eshkol_matmul_dispatch from host memory: %.1f ms %.1f GFLOP/s" % (dt * 1e3, flops / dt / 1e9))
+        del Ch
 
     # ---- CPU baseline on one host core ---------------------------------------------------------
     cpu = None

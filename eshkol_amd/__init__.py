@@ -73,6 +73,10 @@ SIGNATURES = {
     "eshkol_gpu_matmul_f64": (C.c_int, [BUF, BUF, BUF, u64, u64, u64]),
     "eshkol_gpu_matmul_f32": (C.c_int, [BUF, BUF, BUF, u64, u64, u64]),
     "eshkol_gpu_matmul_backward_f64": (C.c_int, [BUF, BUF, BUF, BUF, BUF, u64, u64, u64]),
+    "eshkol_gpu_resident_pin": (C.c_int, [vp, C.c_size_t]),
+    "eshkol_gpu_resident_refresh": (C.c_int, [vp]),
+    "eshkol_gpu_resident_unpin": (None, [vp]),
+    "eshkol_gpu_resident_bytes": (C.c_size_t, []),
     "eshkol_gpu_set_threshold": (None, [C.c_size_t]),
     "eshkol_gpu_get_threshold": (C.c_size_t, []),
     "eshkol_gpu_should_use": (C.c_int, [C.c_size_t]),
@@ -92,6 +96,7 @@ SIGNATURES = {
     "eshkol_hip_get_stream": (vp, []),
     "hip_dgemm_f64": (C.c_int, [vp, vp, vp, u64, u64, u64, vp]),
     "hip_dgemm_f64_ex": (C.c_int, [vp, vp, vp, u64, u64, u64, C.c_int, C.c_int, vp]),
+    "hip_dgemm_f64_batched": (C.c_int, [vp, vp, vp, u64, u64, u64, u64, vp]),
     "hip_sgemm_f32": (C.c_int, [vp, vp, vp, u64, u64, u64, vp]),
     "hip_transpose_f64": (C.c_int, [vp, vp, u64, u64, vp]),
     "hip_rowabsmax_f64": (C.c_int, [vp, u64, u64, C.c_double, vp, vp]),

@@ -45,13 +45,17 @@ constexpr int BK = 16;
  * The pads make every LDS read of a wave hit distinct banks. Both forms hand
  * the MFMA the value at (row li + 16 t, k = 4 lg + s), so they are
  * interchangeable on either side of the instruction. */
-template <int R, bool KMAJ, bool VEC> struct Operand {
-    static constexpr int LD_S = KMAJ ? R + 4 : BK + 2;
-    static constexpr int TILE = KMAJ ? BK * LD_S : R * LD_S;
+template <int R, bool KMAJ, bool VEC, bool LK = KMAJ> struct Operand {
+    /* LK: the LDS tile is k-major. Always so for a k-major matrix; for a
+     * row-major one it means the pair a thread loaded is written as two 8-byte
+     * values one LDS row apart (a transpose on the way in). */
+    static_assert(LK || !KMAJ, "a k-major matrix keeps its form in LDS");
+    static constexpr int LD_S = LK ? R + 4 : BK + 2;
+    static constexpr int TILE = LK ? BK * LD_S : R * LD_S;
     static constexpr int CHUNKS = R * BK / 2 / 256;   /* 16-byte chunks per thread */
     static constexpr int T = R / 32;                  /* 16-row tiles per wave */
     d2_t reg[CHUNKS];
-    d2_t lo[KMAJ ? 1 : T], hi[KMAJ ? 1 : T];
+    d2_t lo[LK ? 1 : T], hi[LK ? 1 : T];
     const double* base;
 
     /* rows = row count of the whole matrix, K = its k extent */
@@ -92,6 +96,10 @@ template <int R, bool KMAJ, bool VEC> struct Operand {
             if (KMAJ) {
                 const int kr = c / (R / 2), rc = c % (R / 2);
                 *(d2_t*)(S + kr * LD_S + 2 * rc) = reg[r];
+            } else if (LK) {
+                const int row = c >> 3, kc = c & 7;
+                S[(2 * kc) * LD_S + row] = reg[r].x;
+                S[(2 * kc + 1) * LD_S + row] = reg[r].y;
             } else {
                 const int row = c >> 3, kc = c & 7;
                 *(d2_t*)(S + row * LD_S + 2 * kc) = reg[r];
@@ -100,7 +108,7 @@ template <int R, bool KMAJ, bool VEC> struct Operand {
     }
     /* woff = first row of this wave inside the block tile */
     __device__ __forceinline__ void frag_begin(const double* S, int woff, int li, int lg) {
-        if (KMAJ) {
+        if (LK) {
             base = S + (4 * lg) * LD_S + woff + li;
         } else {
             base = S + (woff + li) * LD_S + 4 * lg;
@@ -112,7 +120,7 @@ template <int R, bool KMAJ, bool VEC> struct Operand {
         }
     }
     __device__ __forceinline__ double frag(int s, int t) const {
-        if (KMAJ) return base[s * LD_S + t * 16];
+        if (LK) return base[s * LD_S + t * 16];
         return (s == 0) ? lo[t].x : (s == 1) ? lo[t].y : (s == 2) ? hi[t].x : hi[t].y;
     }
 };
@@ -135,16 +143,21 @@ __device__ __forceinline__ void tile_of_workgroup(int tiles_m, int tiles_n, int*
 /* C[MxN] = op(A) * op(B). TA: A is stored as its transpose [K][M]; TB: B is
  * stored as its transpose [N][K]. VEC: every row pitch is even and both bases
  * are 16-byte aligned, so operands move as 16-byte pairs. */
-template <int BM, int BN, bool VEC, bool TA, bool TB>
+template <int BM, int BN, bool VEC, bool TA, bool TB, bool ALK, bool BLK>
 __global__ __launch_bounds__(256)
 void dgemm_mfma_kernel(const double* __restrict__ A, const double* __restrict__ B,
                        double* __restrict__ C, int M, int N, int K,
                        int tiles_m, int tiles_n) {
-    using OpA = Operand<BM, TA, VEC>;
-    using OpB = Operand<BN, !TB, VEC>;
+    using OpA = Operand<BM, TA, VEC, ALK>;
+    using OpB = Operand<BN, !TB, VEC, BLK>;
     extern __shared__ __align__(16) double smem[];
     double* As = smem;
     double* Bs = smem + 2 * OpA::TILE;
+
+    /* blockIdx.y walks a batch of dense products stored back to back */
+    A += (size_t)blockIdx.y * M * K;
+    B += (size_t)blockIdx.y * K * N;
+    C += (size_t)blockIdx.y * M * N;
 
     int tm, tn;
     tile_of_workgroup(tiles_m, tiles_n, &tm, &tn);
@@ -217,12 +230,12 @@ void dgemm_mfma_kernel(const double* __restrict__ A, const double* __restrict__ 
         }
 }
 
-template <int BM, int BN, bool VEC, bool TA, bool TB>
-int launch(const double* A, const double* B, double* C, int M, int N, int K, hipStream_t st) {
-    constexpr int SMEM_BYTES = 2 * (Operand<BM, TA, VEC>::TILE + Operand<BN, !TB, VEC>::TILE)
+template <int BM, int BN, bool VEC, bool TA, bool TB, bool ALK, bool BLK>
+int launch(const double* A, const double* B, double* C, int M, int N, int K, int batch, hipStream_t st) {
+    constexpr int SMEM_BYTES = 2 * (Operand<BM, TA, VEC, ALK>::TILE + Operand<BN, !TB, VEC, BLK>::TILE)
                                * (int)sizeof(double);
     static bool attr_set = false;
-    auto kern = dgemm_mfma_kernel<BM, BN, VEC, TA, TB>;
+    auto kern = dgemm_mfma_kernel<BM, BN, VEC, TA, TB, ALK, BLK>;
     if (!attr_set) {
         if (!ESHKOL_HIP_OK(hipFuncSetAttribute((const void*)kern,
                 hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES))) return -1;
@@ -230,44 +243,74 @@ int launch(const double* A, const double* B, double* C, int M, int N, int K, hip
     }
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     const long long nwg = (long long)tiles_m * tiles_n;
-    if (nwg > 0x7fffffffLL) return -1;
-    hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(256), SMEM_BYTES, st,
+    if (nwg > 0x7fffffffLL || batch < 1 || batch > 65535) return -1;
+    hipLaunchKernelGGL(kern, dim3((unsigned)nwg, (unsigned)batch), dim3(256), SMEM_BYTES, st,
                        A, B, C, M, N, K, tiles_m, tiles_n);
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 
 template <bool TA, bool TB>
-int launch_shape(const double* A, const double* B, double* C, int m, int n, int k, bool vec, hipStream_t st) {
+int launch_shape(const double* A, const double* B, double* C, int m, int n, int k, int batch, bool vec,
+                 hipStream_t st) {
     /* Small outputs cannot fill 256 CUs with 128x128 tiles: use 64x64 there. */
-    const long long big_tiles = (long long)((m + 127) / 128) * (long long)((n + 127) / 128);
+    const long long big_tiles = (long long)((m + 127) / 128) * (long long)((n + 127) / 128) * batch;
+    /* Row-major A next to a k-major B: writing A's tile k-major into LDS (so both
+     * operands are read the same way) measured 1 % faster than keeping A's rows
+     * at 8192^3; with both operands row-major the natural forms are faster. */
+    constexpr bool ALK = TA || !TB;
     if (big_tiles >= 256) {
-        return vec ? launch<128, 128, true, TA, TB>(A, B, C, m, n, k, st)
-                   : launch<128, 128, false, TA, TB>(A, B, C, m, n, k, st);
+        return vec ? launch<128, 128, true, TA, TB, ALK, !TB>(A, B, C, m, n, k, batch, st)
+                   : launch<128, 128, false, TA, TB, TA, !TB>(A, B, C, m, n, k, batch, st);
     }
-    return vec ? launch<64, 64, true, TA, TB>(A, B, C, m, n, k, st)
-               : launch<64, 64, false, TA, TB>(A, B, C, m, n, k, st);
+    return vec ? launch<64, 64, true, TA, TB, TA, !TB>(A, B, C, m, n, k, batch, st)
+               : launch<64, 64, false, TA, TB, TA, !TB>(A, B, C, m, n, k, batch, st);
 }
 
+}  // namespace
+
+namespace {
+int dgemm_any(const double* A, const double* B, double* C, uint64_t M, uint64_t K, uint64_t N,
+              int trans_a, int trans_b, uint64_t batch, void* stream) {
+    if (!A || !B || !C || M == 0 || K == 0 || N == 0 || batch == 0) return -1;
+    if (M > 0x7fffffffULL || K > 0x7fffffffULL || N > 0x7fffffffULL) return -1;
+    if (trans_a && trans_b) return -1;   /* no caller needs it: (B*A)^T, transpose the result instead */
+    hipStream_t st = (hipStream_t)stream;
+    /* row pitches: A is [M][K] or [K][M]; B is [K][N] or [N][K]. In a batch every
+     * matrix must start on a 16-byte boundary as well. */
+    const uint64_t pitch_a = trans_a ? M : K, pitch_b = trans_b ? K : N;
+    const bool vec = (pitch_a % 2 == 0) && (pitch_b % 2 == 0) &&
+                     ((uintptr_t)A % 16 == 0) && ((uintptr_t)B % 16 == 0) &&
+                     (batch == 1 || ((M * K) % 2 == 0 && (K * N) % 2 == 0));
+    const int m = (int)M, n = (int)N, k = (int)K;
+    /* the grid's y extent is limited to 65535 */
+    for (uint64_t done = 0; done < batch; ) {
+        const int nb = (int)((batch - done < 65535) ? batch - done : 65535);
+        const double* a = A + done * M * K;
+        const double* b = B + done * K * N;
+        double* c = C + done * M * N;
+        int rc;
+        if (trans_a) rc = launch_shape<true, false>(a, b, c, m, n, k, nb, vec, st);
+        else if (trans_b) rc = launch_shape<false, true>(a, b, c, m, n, k, nb, vec, st);
+        else rc = launch_shape<false, false>(a, b, c, m, n, k, nb, vec, st);
+        if (rc != 0) return rc;
+        done += (uint64_t)nb;
+    }
+    return 0;
+}
 }  // namespace
 
 extern "C" int hip_dgemm_f64_ex(const double* A, const double* B, double* C,
                                 uint64_t M, uint64_t K, uint64_t N,
                                 int trans_a, int trans_b, void* stream) {
-    if (!A || !B || !C || M == 0 || K == 0 || N == 0) return -1;
-    if (M > 0x7fffffffULL || K > 0x7fffffffULL || N > 0x7fffffffULL) return -1;
-    if (trans_a && trans_b) return -1;   /* no caller needs it: (B*A)^T, transpose the result instead */
-    hipStream_t st = (hipStream_t)stream;
-    /* row pitches: A is [M][K] or [K][M]; B is [K][N] or [N][K] */
-    const uint64_t pitch_a = trans_a ? M : K, pitch_b = trans_b ? K : N;
-    const bool vec = (pitch_a % 2 == 0) && (pitch_b % 2 == 0) &&
-                     ((uintptr_t)A % 16 == 0) && ((uintptr_t)B % 16 == 0);
-    const int m = (int)M, n = (int)N, k = (int)K;
-    if (trans_a) return launch_shape<true, false>(A, B, C, m, n, k, vec, st);
-    if (trans_b) return launch_shape<false, true>(A, B, C, m, n, k, vec, st);
-    return launch_shape<false, false>(A, B, C, m, n, k, vec, st);
+    return dgemm_any(A, B, C, M, K, N, trans_a, trans_b, 1, stream);
 }
 
 extern "C" int hip_dgemm_f64(const double* A, const double* B, double* C,
                              uint64_t M, uint64_t K, uint64_t N, void* stream) {
-    return hip_dgemm_f64_ex(A, B, C, M, K, N, 0, 0, stream);
+    return dgemm_any(A, B, C, M, K, N, 0, 0, 1, stream);
+}
+
+extern "C" int hip_dgemm_f64_batched(const double* A, const double* B, double* C,
+                                     uint64_t batch, uint64_t M, uint64_t K, uint64_t N, void* stream) {
+    return dgemm_any(A, B, C, M, K, N, 0, 0, batch, stream);
 }

@@ -27,6 +27,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
+#include <vector>
 #include <dlfcn.h>
 
 extern "C" {
@@ -55,6 +56,7 @@ char g_arch[64] = "";
 constexpr uint32_t FLAG_WRAPPED_HOST = 1u << 0;   /* host memory is the caller's   */
 constexpr uint32_t FLAG_COPY_BACK    = 1u << 1;   /* device copy must reach host   */
 constexpr uint32_t FLAG_HOST_CURRENT = 1u << 3;   /* host already holds device data */
+constexpr uint32_t FLAG_RESIDENT     = 1u << 4;   /* device copy belongs to the resident table */
 
 struct Slot { void* ptr = nullptr; size_t bytes = 0; };
 Slot g_ws[WS_COUNT];
@@ -202,12 +204,94 @@ int hip_alloc(size_t size_bytes, EshkolMemoryType mem_type, EshkolGPUBuffer* out
 /* Staged wrap: device copy of caller-owned host memory. Registration of
  * existing host memory is not available on the target machines, so this is the
  * reference's fallback branch (gpu_memory_cuda.cpp:811-820). */
-int hip_wrap(void* host_ptr, size_t size_bytes, bool upload, bool copy_back, EshkolGPUBuffer* out) {
+/* ---- device copies of host tensors -------------------------------------------
+ * Staging pool: the device side of a wrapped host buffer comes from a small
+ * cache of earlier allocations, so a matmul on host memory does not pay
+ * hipMalloc/hipFree (each a device-wide synchronisation) per operand per call.
+ * Resident table: host tensors the runtime has declared stable
+ * (eshkol_gpu_resident_pin, typically weights) keep their device copy across
+ * calls, so wrapping them moves no bytes at all. Both are guarded by
+ * g_gpu_mutex. */
+struct Staged { void* ptr; size_t bytes; bool in_use; };
+std::vector<Staged> g_staging;
+constexpr size_t STAGING_KEEP = 8;        /* idle buffers kept for reuse */
+
+void* staging_get(size_t bytes) {
+    int best = -1;
+    for (size_t i = 0; i < g_staging.size(); i++) {
+        const Staged& s = g_staging[i];
+        if (!s.in_use && s.bytes >= bytes && s.bytes <= 2 * bytes + 4096 &&
+            (best < 0 || s.bytes < g_staging[best].bytes)) best = (int)i;
+    }
+    if (best >= 0) { g_staging[best].in_use = true; return g_staging[best].ptr; }
     void* d = nullptr;
-    if (!ESHKOL_HIP_OK(hipMalloc(&d, size_bytes))) return -1;
+    if (!ESHKOL_HIP_OK(hipMalloc(&d, bytes))) {
+        /* memory may be held by idle staging buffers: drop them and retry once */
+        (void)hipGetLastError();
+        for (size_t i = 0; i < g_staging.size();) {
+            if (!g_staging[i].in_use) { hipFree(g_staging[i].ptr); g_staging.erase(g_staging.begin() + i); }
+            else i++;
+        }
+        if (!ESHKOL_HIP_OK(hipMalloc(&d, bytes))) return nullptr;
+    }
+    g_staging.push_back({d, bytes, true});
+    return d;
+}
+
+void staging_put(void* d) {
+    size_t idle = 0;
+    for (Staged& s : g_staging) {
+        if (s.ptr == d) s.in_use = false;
+        if (!s.in_use) idle++;
+    }
+    /* keep the newest STAGING_KEEP idle buffers */
+    for (size_t i = 0; i < g_staging.size() && idle > STAGING_KEEP;) {
+        if (!g_staging[i].in_use) {
+            hipFree(g_staging[i].ptr);
+            g_staging.erase(g_staging.begin() + i);
+            idle--;
+        } else i++;
+    }
+}
+
+void staging_release_all(void) {
+    for (Staged& s : g_staging) hipFree(s.ptr);
+    g_staging.clear();
+}
+
+struct Resident { const void* host; size_t bytes; void* dev; };
+std::vector<Resident> g_resident;
+
+Resident* resident_find(const void* host) {
+    for (Resident& r : g_resident) if (r.host == host) return &r;
+    return nullptr;
+}
+
+void resident_release_all(void) {
+    for (Resident& r : g_resident) hipFree(r.dev);
+    g_resident.clear();
+}
+
+int hip_wrap(void* host_ptr, size_t size_bytes, bool upload, bool copy_back, EshkolGPUBuffer* out) {
+    /* a read-only operand that is resident needs no copy and owns no memory */
+    if (upload && !copy_back) {
+        Resident* r = resident_find(host_ptr);
+        if (r && r->bytes >= size_bytes) {
+            out->host_ptr = host_ptr;
+            out->device_ptr = r->dev;
+            out->size_bytes = size_bytes;
+            out->mem_type = ESHKOL_MEM_DEVICE;
+            out->backend = ESHKOL_GPU_HIP;
+            out->flags = FLAG_WRAPPED_HOST | FLAG_HOST_CURRENT | FLAG_RESIDENT;
+            out->backend_data = host_ptr;
+            return 0;
+        }
+    }
+    void* d = staging_get(size_bytes);
+    if (!d) return -1;
     if (upload) {
         if (!ESHKOL_HIP_OK(hipMemcpyAsync(d, host_ptr, size_bytes, hipMemcpyHostToDevice, g_stream)) ||
-            !ESHKOL_HIP_OK(hipStreamSynchronize(g_stream))) { hipFree(d); return -1; }
+            !ESHKOL_HIP_OK(hipStreamSynchronize(g_stream))) { staging_put(d); return -1; }
     }
     out->host_ptr = host_ptr;
     out->device_ptr = d;
@@ -239,10 +323,11 @@ int hip_sync(EshkolGPUBuffer* b, EshkolSyncDirection dir) {
 void hip_free(EshkolGPUBuffer* b) {
     hipStreamSynchronize(g_stream);
     if (b->flags & FLAG_WRAPPED_HOST) {
+        if (b->flags & FLAG_RESIDENT) return;
         if ((b->flags & FLAG_COPY_BACK) && !(b->flags & FLAG_HOST_CURRENT) &&
             b->backend_data && b->device_ptr)
             hipMemcpy(b->backend_data, b->device_ptr, b->size_bytes, hipMemcpyDeviceToHost);
-        if (b->device_ptr) hipFree(b->device_ptr);
+        if (b->device_ptr) staging_put(b->device_ptr);
         return;
     }
     switch (b->mem_type) {
@@ -408,6 +493,8 @@ void eshkol_gpu_shutdown(void) {
     if (g_backend == ESHKOL_GPU_HIP) {
         if (g_stream) hipStreamSynchronize(g_stream);
         eshkol_hip_workspace_release();
+        staging_release_all();
+        resident_release_all();
         if (g_stream) { hipStreamDestroy(g_stream); g_stream = nullptr; }
     }
     g_backend = ESHKOL_GPU_NONE;
@@ -583,6 +670,59 @@ int eshkol_gpu_matmul_f32(EshkolGPUBuffer* A, EshkolGPUBuffer* B, EshkolGPUBuffe
     return -1;
 }
 
+/* ---- resident host tensors (no counterpart in the reference, whose dispatch
+ * re-wraps and re-uploads every operand on every call, gpu_memory_cuda.cpp:
+ * 1136-1145) ------------------------------------------------------------------ */
+
+int eshkol_gpu_resident_pin(const void* host_ptr, size_t size_bytes) {
+    if (g_backend == ESHKOL_GPU_NONE) eshkol_gpu_init();
+    if (!host_ptr || size_bytes == 0 || g_backend != ESHKOL_GPU_HIP) return -1;
+    std::lock_guard<std::recursive_mutex> g(g_gpu_mutex);
+    Resident* r = resident_find(host_ptr);
+    if (r && r->bytes != size_bytes) {
+        hipStreamSynchronize(g_stream);
+        hipFree(r->dev);
+        g_resident.erase(g_resident.begin() + (r - g_resident.data()));
+        r = nullptr;
+    }
+    void* d = r ? r->dev : nullptr;
+    if (!d && !ESHKOL_HIP_OK(hipMalloc(&d, size_bytes))) return -1;
+    if (!ESHKOL_HIP_OK(hipMemcpyAsync(d, host_ptr, size_bytes, hipMemcpyHostToDevice, g_stream)) ||
+        !ESHKOL_HIP_OK(hipStreamSynchronize(g_stream))) {
+        if (!r) hipFree(d);
+        return -1;
+    }
+    if (!r) g_resident.push_back({host_ptr, size_bytes, d});
+    return 0;
+}
+
+int eshkol_gpu_resident_refresh(const void* host_ptr) {
+    if (g_backend != ESHKOL_GPU_HIP) return -1;
+    std::lock_guard<std::recursive_mutex> g(g_gpu_mutex);
+    Resident* r = resident_find(host_ptr);
+    if (!r) return -1;
+    if (!ESHKOL_HIP_OK(hipMemcpyAsync(r->dev, host_ptr, r->bytes, hipMemcpyHostToDevice, g_stream)) ||
+        !ESHKOL_HIP_OK(hipStreamSynchronize(g_stream))) return -1;
+    return 0;
+}
+
+void eshkol_gpu_resident_unpin(const void* host_ptr) {
+    if (g_backend != ESHKOL_GPU_HIP) return;
+    std::lock_guard<std::recursive_mutex> g(g_gpu_mutex);
+    Resident* r = resident_find(host_ptr);
+    if (!r) return;
+    hipStreamSynchronize(g_stream);
+    hipFree(r->dev);
+    g_resident.erase(g_resident.begin() + (r - g_resident.data()));
+}
+
+size_t eshkol_gpu_resident_bytes(void) {
+    std::lock_guard<std::recursive_mutex> g(g_gpu_mutex);
+    size_t total = 0;
+    for (const Resident& r : g_resident) total += r.bytes;
+    return total;
+}
+
 void eshkol_gpu_set_threshold(size_t threshold) { g_gpu_threshold = threshold; }
 size_t eshkol_gpu_get_threshold(void) { return g_gpu_threshold; }
 int eshkol_gpu_should_use(size_t num_elements) {
@@ -691,8 +831,13 @@ void eshkol_matmul_dispatch(const double* A, const double* B, double* C,
 void eshkol_batch_matmul_dispatch(const double* a, const double* b, double* c,
                                   int64_t batch, int64_t M, int64_t K, int64_t N, int32_t dtype) {
     if (g_backend == ESHKOL_GPU_NONE) eshkol_gpu_init();
-    if ((dtype == 2 || dtype == 3) && g_backend == ESHKOL_GPU_HIP &&
-        a && b && c && batch > 0 && M > 0 && K > 0 && N > 0) {
+    /* 16-bit tensors always take the GPU (as the reference's CUDA unit does);
+     * f64 batches take the native fp64 kernel, strided over the batch in one
+     * launch, once the whole output reaches the element threshold. */
+    const bool reduced = (dtype == 2 || dtype == 3);
+    const bool valid = a && b && c && batch > 0 && M > 0 && K > 0 && N > 0;
+    if (valid && g_backend == ESHKOL_GPU_HIP &&
+        (reduced || (size_t)batch * (size_t)M * (size_t)N >= g_gpu_threshold)) {
         std::lock_guard<std::recursive_mutex> g(g_gpu_mutex);
         const size_t na = (size_t)batch * M * K, nb = (size_t)batch * K * N, nc = (size_t)batch * M * N;
         EshkolGPUBuffer ba{}, bb{}, bc{};
@@ -702,11 +847,19 @@ void eshkol_batch_matmul_dispatch(const double* a, const double* b, double* c,
         bool done = false;
         if (wa && wb && wc) {
             int rc = 0;
-            for (int64_t i = 0; i < batch && rc == 0; i++)
-                rc = hip_matmul_reduced_f64((const double*)ba.device_ptr + (size_t)i * M * K,
-                                            (const double*)bb.device_ptr + (size_t)i * K * N,
-                                            (double*)bc.device_ptr + (size_t)i * M * N,
-                                            (uint64_t)M, (uint64_t)K, (uint64_t)N, dtype, 1, g_stream);
+            if (reduced) {
+                for (int64_t i = 0; i < batch && rc == 0; i++)
+                    rc = hip_matmul_reduced_f64((const double*)ba.device_ptr + (size_t)i * M * K,
+                                                (const double*)bb.device_ptr + (size_t)i * K * N,
+                                                (double*)bc.device_ptr + (size_t)i * M * N,
+                                                (uint64_t)M, (uint64_t)K, (uint64_t)N, dtype, 1, g_stream);
+            } else {
+                GPU_LOG("batch matmul %lld x (%lldx%lld @ %lldx%lld) -> native fp64 MFMA, one strided launch",
+                        (long long)batch, (long long)M, (long long)K, (long long)K, (long long)N);
+                rc = hip_dgemm_f64_batched((const double*)ba.device_ptr, (const double*)bb.device_ptr,
+                                           (double*)bc.device_ptr, (uint64_t)batch,
+                                           (uint64_t)M, (uint64_t)K, (uint64_t)N, g_stream);
+            }
             if (rc == 0) { mark_written(&bc); done = hip_sync(&bc, ESHKOL_SYNC_DEVICE_TO_HOST) == 0; }
         }
         if (!done) bc.flags &= ~FLAG_COPY_BACK;

@@ -47,6 +47,14 @@ int hip_dgemm_f64_ex(const double* A, const double* B, double* C,
                      uint64_t M, uint64_t K, uint64_t N,
                      int trans_a, int trans_b, void* stream);
 
+/* batch dense products stored back to back (A [batch][M][K], B [batch][K][N],
+ * C [batch][M][N]) in one launch, the batch index on the grid's second axis:
+ * the f64 counterpart of the strided-batched call the reference has for 16-bit
+ * tensors only (gpu_memory_cuda.cpp:763-771); its f64 batches run the CPU loop
+ * (lib/core/runtime_tensor_math.cpp:796-817). */
+int hip_dgemm_f64_batched(const double* A, const double* B, double* C,
+                          uint64_t batch, uint64_t M, uint64_t K, uint64_t N, void* stream);
+
 /* Single precision, replaces cublasSgemm at gpu_memory_cuda.cpp:658-665. */
 int hip_sgemm_f32(const float* A, const float* B, float* C,
                   uint64_t M, uint64_t K, uint64_t N, void* stream);

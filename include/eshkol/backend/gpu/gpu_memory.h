@@ -102,6 +102,24 @@ int eshkol_gpu_matmul_backward_f64(EshkolGPUBuffer* grad_out, EshkolGPUBuffer* A
                                    EshkolGPUBuffer* grad_A, EshkolGPUBuffer* grad_B,
                                    uint64_t M, uint64_t K, uint64_t N);
 
+/* ---- resident host tensors -------------------------------------------------
+ * An addition to the reference header. The reference's dispatchers wrap and
+ * upload every operand on every call (gpu_memory_cuda.cpp:1136-1145), so a
+ * weight matrix crosses the host link once per matmul. A tensor the runtime
+ * declares stable keeps a device copy: eshkol_matmul_dispatch and
+ * eshkol_batch_matmul_dispatch then use that copy for an input operand whose
+ * host pointer matches, moving no bytes.
+ *   pin      upload now (again if already pinned); 0 on success
+ *   refresh  the host contents changed: upload again; -1 if not pinned
+ *   unpin    drop the device copy
+ *   bytes    device memory currently held by pinned tensors
+ * The caller owns the contract that a pinned tensor is not modified on the
+ * host without a refresh. eshkol_gpu_shutdown drops every copy. */
+int eshkol_gpu_resident_pin(const void* host_ptr, size_t size_bytes);
+int eshkol_gpu_resident_refresh(const void* host_ptr);
+void eshkol_gpu_resident_unpin(const void* host_ptr);
+size_t eshkol_gpu_resident_bytes(void);
+
 /* ---- thresholds: reference gpu_memory.h:261-280 -------------------------- */
 extern size_t g_gpu_threshold;
 void eshkol_gpu_set_threshold(size_t threshold);

@@ -160,11 +160,85 @@ assert rt.oracle_hostrt_batch_calls() == 0
 for i in range(4):
     Ar, Br = oracle.reduce_precision(a[i], 3), oracle.reduce_precision(b[i], 3)
     assert normwise(c[i], oracle.matmul_f64(Ar, Br), Ar, Br) <= 1e-2
+# f64 batches: below the element threshold (4*96*64 outputs) the runtime's CPU loop, above it one strided launch
+lib.eshkol_gpu_set_threshold(100000)
 lib.eshkol_batch_matmul_dispatch(a.ctypes.data, b.ctypes.data, c.ctypes.data, 4, 96, 160, 64, 0)
 assert rt.oracle_hostrt_batch_calls() == 1 and np.array_equal(c, oracle.batch_matmul_f64(a, b))
+lib.eshkol_gpu_set_threshold(1)
+c[:] = 0
+lib.eshkol_batch_matmul_dispatch(a.ctypes.data, b.ctypes.data, c.ctypes.data, 4, 96, 160, 64, 0)
+assert rt.oracle_hostrt_batch_calls() == 1
+ref = oracle.batch_matmul_f64(a, b)
+for i in range(4):
+    assert normwise(c[i], ref[i], a[i], b[i]) <= 1e-14
 """
     r = run_child(body, {"ESHKOL_GPU_VERBOSE": "1"})
     assert "native fp64 MFMA" in r.stderr and "reduced tier" in r.stderr
+    assert "batch matmul 4 x (96x160 @ 160x64) -> native fp64 MFMA, one strided launch" in r.stderr
+
+
+def test_batched_native_kernel(gpu):
+    """hip_dgemm_f64_batched against the oracle's batch loop: even and odd shapes
+    (the odd ones leave matrices of the batch off 16-byte boundaries), integer
+    cases exact, a batch larger than one grid axis allows."""
+    lib = ea.load()
+    st = lib.eshkol_hip_get_stream()
+    for (bt, M, K, N) in [(1, 64, 64, 64), (3, 17, 23, 11), (5, 33, 7, 9), (8, 128, 96, 160), (2, 300, 257, 129),
+                          (16, 256, 256, 256)]:
+        a, b = synth.normal(bt + M, (bt, M, K)), synth.normal(bt + N, (bt, K, N))
+        da, db, dc = ea.DeviceArray.from_host(a), ea.DeviceArray.from_host(b), ea.DeviceArray((bt, M, N))
+        assert lib.hip_dgemm_f64_batched(da.ptr, db.ptr, dc.ptr, bt, M, K, N, st) == 0
+        ea.synchronize()
+        got, ref = dc.download(), oracle.batch_matmul_f64(a, b)
+        for i in range(bt):
+            assert normwise(got[i], ref[i], a[i], b[i]) <= 1e-14, (bt, M, K, N, i)
+    rng = np.random.default_rng(9)
+    bt, M, K, N = 70000, 4, 6, 2
+    a = rng.integers(-5, 6, (bt, M, K)).astype(np.float64)
+    b = rng.integers(-5, 6, (bt, K, N)).astype(np.float64)
+    da, db, dc = ea.DeviceArray.from_host(a), ea.DeviceArray.from_host(b), ea.DeviceArray((bt, M, N))
+    assert lib.hip_dgemm_f64_batched(da.ptr, db.ptr, dc.ptr, bt, M, K, N, st) == 0
+    ea.synchronize()
+    assert np.array_equal(dc.download(), np.einsum("bmk,bkn->bmn", a, b))
+    assert lib.hip_dgemm_f64_batched(da.ptr, db.ptr, dc.ptr, 0, M, K, N, st) == -1
+
+
+def test_resident_tensors_skip_the_upload(gpu):
+    body = r"""
+lib.eshkol_gpu_set_threshold(1)
+W = synth.normal(1, (300, 200)); X = synth.normal(2, (150, 300))
+assert lib.eshkol_gpu_resident_bytes() == 0
+assert lib.eshkol_gpu_resident_pin(W.ctypes.data, W.nbytes) == 0
+assert lib.eshkol_gpu_resident_bytes() == W.nbytes
+ref = oracle.matmul_f64(X, W)
+assert normwise(ea.matmul_dispatch(X, W), ref, X, W) <= 1e-14
+# the device copy is what the product reads: a host change is invisible until refresh
+keep = W.copy()
+W[:] = 0.0
+assert normwise(ea.matmul_dispatch(X, W), ref, X, keep) <= 1e-14
+assert lib.eshkol_gpu_resident_refresh(W.ctypes.data) == 0
+assert np.all(ea.matmul_dispatch(X, W) == 0.0)
+W[:] = keep
+assert lib.eshkol_gpu_resident_pin(W.ctypes.data, W.nbytes) == 0          # pin again = upload again
+assert normwise(ea.matmul_dispatch(X, W), ref, X, W) <= 1e-14
+# as the first operand too, and in the batched entry
+assert normwise(ea.matmul_dispatch(W.T.copy(), X.T.copy()), ref.T, X, W) <= 1e-14
+lib.eshkol_gpu_resident_unpin(W.ctypes.data)
+assert lib.eshkol_gpu_resident_bytes() == 0 and lib.eshkol_gpu_resident_refresh(W.ctypes.data) == -1
+W[:] = 1.0
+assert np.array_equal(ea.matmul_dispatch(np.ones((150, 300)), W), np.full((150, 200), 300.0))
+assert rt.oracle_hostrt_matmul_calls() == 0
+# staging buffers are reused: many calls, no growth in device memory in use
+free0, total = C.c_size_t(), C.c_size_t()
+ea.hip_runtime().hipMemGetInfo(C.byref(free0), C.byref(total))
+for _ in range(20):
+    ea.matmul_dispatch(X, W)
+free1 = C.c_size_t()
+ea.hip_runtime().hipMemGetInfo(C.byref(free1), C.byref(total))
+assert free0.value - free1.value <= (8 << 20)
+lib.eshkol_gpu_shutdown()
+"""
+    run_child(body)
 
 
 def test_threshold_env_forces_gpu(gpu):
