@@ -99,6 +99,10 @@ SIGNATURES = {
     "hip_dgemm_f64_batched": (C.c_int, [vp, vp, vp, u64, u64, u64, u64, vp]),
     "hip_sgemm_f32": (C.c_int, [vp, vp, vp, u64, u64, u64, vp]),
     "hip_transpose_f64": (C.c_int, [vp, vp, u64, u64, vp]),
+    "hip_colabsmax_f64": (C.c_int, [vp, u64, u64, C.c_double, vp, vp]),
+    "hip_ozaki_crt_split_kmajor_f64": (C.c_int, [vp, u64, u64, vp, C.c_int, vp, u64, u64, vp]),
+    "hip_ozaki_slice_kmajor_f64": (C.c_int, [vp, u64, u64, vp, C.c_int, vp, u64, u64, vp]),
+    "hip_convert_f64_to_16_kmajor": (C.c_int, [vp, vp, u64, u64, u64, u64, C.c_int, vp]),
     "hip_rowabsmax_f64": (C.c_int, [vp, u64, u64, C.c_double, vp, vp]),
     "hip_elementwise_f64": (C.c_int, [vp, vp, vp, u64, C.c_int, vp]),
     "hip_bias_act_f64": (C.c_int, [vp, vp, u64, u64, C.c_int, vp]),

@@ -67,6 +67,40 @@ void rowabsmax_f64_kernel(const double* __restrict__ A, uint64_t M, uint64_t K,
     if (lane == 0) rmax[row] = (m > 0.0) ? m : zero_value;
 }
 
+/* Column maxima of a row-major X[K][R] in two steps: a block takes 64 columns
+ * by one slice of the rows (a wave reads 512 contiguous bytes per row) and
+ * writes its partial maxima; the second kernel folds the slices. */
+constexpr int COLMAX_SLICES = 64;
+
+__global__ __launch_bounds__(256)
+void colabsmax_partial_kernel(const double* __restrict__ X, uint64_t K, uint64_t R,
+                              uint64_t rows_per_slice, double* __restrict__ partial) {
+    __shared__ double red[4][64];
+    const int c = threadIdx.x & 63, part = threadIdx.x >> 6;
+    const uint64_t col = (uint64_t)blockIdx.x * 64 + c;
+    const uint64_t k0 = (uint64_t)blockIdx.y * rows_per_slice;
+    const uint64_t k1 = (k0 + rows_per_slice < K) ? k0 + rows_per_slice : K;
+    double m = 0.0;
+    if (col < R)
+        for (uint64_t k = k0 + part; k < k1; k += 4) absmax_step(X[k * R + col], &m);
+    red[part][c] = m;
+    __syncthreads();
+    if (part == 0 && col < R) {
+        for (int p = 1; p < 4; p++) { const double o = red[p][c]; if (o > m) m = o; }
+        partial[(uint64_t)blockIdx.y * R + col] = m;
+    }
+}
+
+__global__ __launch_bounds__(256)
+void colabsmax_fold_kernel(const double* __restrict__ partial, uint64_t R, int slices,
+                           double zero_value, double* __restrict__ out) {
+    const uint64_t col = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (col >= R) return;
+    double m = 0.0;
+    for (int s = 0; s < slices; s++) { const double o = partial[(uint64_t)s * R + col]; if (o > m) m = o; }
+    out[col] = (m > 0.0) ? m : zero_value;
+}
+
 __device__ __forceinline__ double apply_op(int op, double a, double b, bool has_b) {
     switch (op) {
         case 0:  return a + (has_b ? b : 0.0);
@@ -174,6 +208,24 @@ extern "C" int hip_rowabsmax_f64(const double* A, uint64_t M, uint64_t K, double
     if (g > 0x7fffffffULL) return -1;
     hipLaunchKernelGGL(rowabsmax_f64_kernel, dim3((unsigned)g), dim3(256), 0, (hipStream_t)stream,
                        A, M, K, zero_value, rmax);
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
+extern "C" int hip_colabsmax_f64(const double* X, uint64_t K, uint64_t R, double zero_value,
+                                 double* cmax, void* stream) {
+    if (!X || !cmax || K == 0 || R == 0) return -1;
+    const uint64_t gx = (R + 63) / 64;
+    if (gx > 0x7fffffffULL) return -1;
+    int slices = (int)((K + 63) / 64);                 /* at least 64 rows per slice */
+    if (slices > COLMAX_SLICES) slices = COLMAX_SLICES;
+    const uint64_t rows_per_slice = (K + slices - 1) / slices;
+    slices = (int)((K + rows_per_slice - 1) / rows_per_slice);
+    double* partial = (double*)eshkol_hip_workspace(WS_COLPARTIAL, (size_t)slices * R * sizeof(double));
+    if (!partial) return -1;
+    hipLaunchKernelGGL(colabsmax_partial_kernel, dim3((unsigned)gx, (unsigned)slices), dim3(256), 0,
+                       (hipStream_t)stream, X, K, R, rows_per_slice, partial);
+    hipLaunchKernelGGL(colabsmax_fold_kernel, dim3((unsigned)((R + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, partial, R, slices, zero_value, cmax);
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 

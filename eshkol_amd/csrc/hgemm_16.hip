@@ -20,6 +20,7 @@
 #include "hip_common.h"
 #include "kernels.h"
 #include "gemm_pipe.h"
+#include "kmajor_tile.h"
 
 #include <cstring>
 
@@ -61,6 +62,14 @@ __device__ __forceinline__ float f16_bits_to_f32(uint16_t u) {
 }
 
 template <bool BF16>
+__device__ __forceinline__ uint32_t narrow_pair(double x0, double x1) {
+    const uint16_t h0 = BF16 ? f32_to_bf16_bits((float)x0) : f32_to_f16_bits((float)x0);
+    const uint16_t h1 = BF16 ? f32_to_bf16_bits((float)x1) : f32_to_f16_bits((float)x1);
+    return (uint32_t)h0 | ((uint32_t)h1 << 16);
+}
+
+/* Row-major X[rows][K]. One thread: two consecutive k of one row. */
+template <bool BF16>
 __global__ __launch_bounds__(256)
 void convert_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
                     uint16_t* __restrict__ out, uint64_t rows_padded, uint64_t ld) {
@@ -78,9 +87,19 @@ void convert_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
             x0 = p[0];
         }
     }
-    const uint16_t h0 = BF16 ? f32_to_bf16_bits((float)x0) : f32_to_f16_bits((float)x0);
-    const uint16_t h1 = BF16 ? f32_to_bf16_bits((float)x1) : f32_to_f16_bits((float)x1);
-    *(uint32_t*)(out + row * ld + k) = (uint32_t)h0 | ((uint32_t)h1 << 16);
+    *(uint32_t*)(out + row * ld + k) = narrow_pair<BF16>(x0, x1);
+}
+
+/* k-major X[K][rows] (B as the runtime stores it), same output. */
+template <bool BF16>
+__global__ __launch_bounds__(256)
+void convert_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
+                           uint16_t* __restrict__ out, uint64_t rows_padded, uint64_t ld) {
+    __shared__ __align__(16) double tile[kmaj::SMEM_DOUBLES];
+    kmaj::for_each_pair(X, rows, K, rows_padded, ld, tile,
+        [&](uint64_t row, uint64_t k, double x0, double x1) {
+            *(uint32_t*)(out + row * ld + k) = narrow_pair<BF16>(x0, x1);
+        });
 }
 
 template <int TM, int TN> struct Cfg {
@@ -389,18 +408,33 @@ int hgemm_any(const uint16_t* A, const uint16_t* Bt, uint64_t M, uint64_t K, uin
 
 }  // namespace
 
+namespace {
+int convert_any(const double* in, uint16_t* out, uint64_t rows, uint64_t cols,
+                uint64_t rows_padded, uint64_t ld, int is_bf16, bool kmajor, void* stream) {
+    if (!in || !out || rows == 0 || cols == 0 || rows_padded < rows || ld < cols || (ld & 1)) return -1;
+    const uint64_t nblk = kmajor ? kmaj::grid_blocks(rows_padded, ld) : ((ld / 2 + 255) / 256) * rows_padded;
+    if (nblk > 0x7fffffffULL) return -1;
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 grid((unsigned)nblk), block(256);
+    if (kmajor) {
+        if (is_bf16) hipLaunchKernelGGL(convert_kmajor_kernel<true>, grid, block, 0, st, in, rows, cols, out, rows_padded, ld);
+        else         hipLaunchKernelGGL(convert_kmajor_kernel<false>, grid, block, 0, st, in, rows, cols, out, rows_padded, ld);
+    } else {
+        if (is_bf16) hipLaunchKernelGGL(convert_kernel<true>, grid, block, 0, st, in, rows, cols, out, rows_padded, ld);
+        else         hipLaunchKernelGGL(convert_kernel<false>, grid, block, 0, st, in, rows, cols, out, rows_padded, ld);
+    }
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+}  // namespace
+
 extern "C" int hip_convert_f64_to_16(const double* in, uint16_t* out, uint64_t rows, uint64_t cols,
                                      uint64_t rows_padded, uint64_t ld, int is_bf16, void* stream) {
-    if (!in || !out || rows == 0 || cols == 0 || rows_padded < rows || ld < cols || (ld & 1)) return -1;
-    const uint64_t nblk = ((ld / 2 + 255) / 256) * rows_padded;
-    if (nblk > 0x7fffffffULL) return -1;
-    if (is_bf16)
-        hipLaunchKernelGGL(convert_kernel<true>, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
-                           in, rows, cols, out, rows_padded, ld);
-    else
-        hipLaunchKernelGGL(convert_kernel<false>, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
-                           in, rows, cols, out, rows_padded, ld);
-    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+    return convert_any(in, out, rows, cols, rows_padded, ld, is_bf16, false, stream);
+}
+
+extern "C" int hip_convert_f64_to_16_kmajor(const double* in, uint16_t* out, uint64_t rows, uint64_t cols,
+                                            uint64_t rows_padded, uint64_t ld, int is_bf16, void* stream) {
+    return convert_any(in, out, rows, cols, rows_padded, ld, is_bf16, true, stream);
 }
 
 extern "C" int hip_hgemm_16(const uint16_t* A, const uint16_t* Bt, uint64_t M, uint64_t K, uint64_t N,
@@ -418,22 +452,14 @@ extern "C" int hip_matmul_reduced_f64_ex(const double* A, const double* B, doubl
     hipStream_t st = (hipStream_t)stream;
     const int is_bf16 = (dtype == 3);
     const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ld = round_up_sz(K, 128);
-    const double* Bt = B;
-    if (!trans_b) {
-        double* t = (double*)eshkol_hip_workspace(WS_BT, K * N * sizeof(double));
-        if (!t || hip_transpose_f64(B, t, K, N, st) != 0) return -1;
-        Bt = t;
-    }
-    if (trans_a) {
-        double* t = (double*)eshkol_hip_workspace(WS_AT, M * K * sizeof(double));
-        if (!t || hip_transpose_f64(A, t, K, M, st) != 0) return -1;
-        A = t;
-    }
+    /* 16-bit copies [row][k] of both operands; one stored k-major (B as given, A
+     * when the caller holds A^T) is narrowed through LDS tiles, so no transposed
+     * fp64 copy is made. */
     uint16_t* A16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_A, Mp * ld * 2);
     uint16_t* B16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_B, Np * ld * 2);
     if (!A16 || !B16) return -1;
-    if (hip_convert_f64_to_16(A, A16, M, K, Mp, ld, is_bf16, st) != 0) return -1;
-    if (hip_convert_f64_to_16(Bt, B16, N, K, Np, ld, is_bf16, st) != 0) return -1;
+    if (convert_any(A, A16, M, K, Mp, ld, is_bf16, trans_a != 0, st) != 0) return -1;
+    if (convert_any(B, B16, N, K, Np, ld, is_bf16, trans_b == 0, st) != 0) return -1;
     return hgemm_any(A16, B16, M, K, N, ld, is_bf16, round_output ? 2 : 1, C, st);
 }
 

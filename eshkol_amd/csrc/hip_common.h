@@ -24,9 +24,7 @@ hipStream_t eshkol_hip_stream(void);
 /* Grow-only device workspace slots, kept for the life of the process so a
  * matmul does not pay hipMalloc/hipFree per call. Returns NULL on failure. */
 enum {
-    WS_BT = 0,      /* transposed fp64 copy of B                          */
-    WS_AT,          /* row-major fp64 copy of an A the caller holds transposed */
-    WS_APLANES,     /* int8 planes of A                                   */
+    WS_APLANES = 0, /* int8 planes of A                                   */
     WS_BPLANES,     /* int8 planes of B (transposed, K contiguous)        */
     WS_PRODUCTS,    /* int8 residue products / int32 diagonal buffers     */
     WS_ROWSCALE,    /* per-row fp64 scale or max, then int shifts         */
@@ -36,6 +34,7 @@ enum {
     WS_HALF_A,      /* 16-bit copies of A, B and fp32 C for the reduced tier */
     WS_HALF_B,
     WS_F32_C,
+    WS_COLPARTIAL,  /* per-slice partial column maxima                       */
     WS_MISC,
     WS_COUNT
 };

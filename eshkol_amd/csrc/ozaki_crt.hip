@@ -8,11 +8,11 @@
  * uses the same libm as the reference's host code.
  *
  * Pipeline (all on the library stream):
- *   Bt = B^T                                  (fp64 transpose, so both operands
- *                                              are split along contiguous K)
- *   amax[i], bmax[j]                          one wave per row
+ *   amax[i], bmax[j]                          row maxima of A, column maxima of B
  *   -> host: frac bounds, E, mu[i], nu[j]     gpu_memory.mm:376-420, 2510-2532
- *   A planes, B planes                        trunc(x*2^shift) mod p_l as int8
+ *   A planes, B planes                        trunc(x*2^shift) mod p_l as int8, both
+ *                                              [row][k]; B is read k-major through
+ *                                              LDS tiles, never transposed in HBM
  *   W_l = (A_l * B_l^T) mod p_l               int8 MFMA, int32 accumulate
  *   C = CRT(W) * 2^-mu * 2^-nu                gpu_memory.mm:2626-2655, verbatim
  *
@@ -23,6 +23,7 @@
  */
 #include "hip_common.h"
 #include "kernels.h"
+#include "kmajor_tile.h"
 
 #include <cmath>
 #include <cstring>
@@ -79,7 +80,26 @@ __device__ __forceinline__ int residue(uint64_t t, bool neg) {
     return s;
 }
 
-/* One thread: two consecutive k of one row -> one 16-bit store per plane. */
+/* Residues of two consecutive k of one row: one 16-bit store per plane. */
+template <int NMOD>
+__device__ __forceinline__ void split_pair(double x0, double x1, int sh, int8_t* out, uint64_t plane_stride) {
+    bool n0, n1;
+    const uint64_t t0 = scaled_magnitude(x0, sh, &n0);
+    const uint64_t t1 = scaled_magnitude(x1, sh, &n1);
+#define ESHKOL_SPLIT_ONE(L)                                                           \
+    if (L < NMOD) {                                                                   \
+        const int r0 = residue<L>(t0, n0), r1 = residue<L>(t1, n1);                   \
+        *(uint16_t*)(out + (uint64_t)L * plane_stride) =                              \
+            (uint16_t)((uint8_t)(int8_t)r0 | ((uint16_t)(uint8_t)(int8_t)r1 << 8));   \
+    }
+    ESHKOL_SPLIT_ONE(0)  ESHKOL_SPLIT_ONE(1)  ESHKOL_SPLIT_ONE(2)  ESHKOL_SPLIT_ONE(3)
+    ESHKOL_SPLIT_ONE(4)  ESHKOL_SPLIT_ONE(5)  ESHKOL_SPLIT_ONE(6)  ESHKOL_SPLIT_ONE(7)
+    ESHKOL_SPLIT_ONE(8)  ESHKOL_SPLIT_ONE(9)  ESHKOL_SPLIT_ONE(10) ESHKOL_SPLIT_ONE(11)
+    ESHKOL_SPLIT_ONE(12) ESHKOL_SPLIT_ONE(13) ESHKOL_SPLIT_ONE(14) ESHKOL_SPLIT_ONE(15)
+#undef ESHKOL_SPLIT_ONE
+}
+
+/* Row-major X[rows][K]. One thread: two consecutive k of one row. */
 template <int NMOD>
 __global__ __launch_bounds__(256)
 void crt_split_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
@@ -101,22 +121,22 @@ void crt_split_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
             x0 = p[0];
         }
     }
-    bool n0, n1;
-    const uint64_t t0 = scaled_magnitude(x0, sh, &n0);
-    const uint64_t t1 = scaled_magnitude(x1, sh, &n1);
+    split_pair<NMOD>(x0, x1, sh, planes + row * ldk + k, rows_padded * ldk);
+}
+
+/* k-major X[K][rows] (B as the runtime stores it), same output. */
+template <int NMOD>
+__global__ __launch_bounds__(256)
+void crt_split_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
+                             const int32_t* __restrict__ shift, int8_t* __restrict__ planes,
+                             uint64_t rows_padded, uint64_t ldk) {
+    __shared__ __align__(16) double tile[kmaj::SMEM_DOUBLES];
     const uint64_t plane_stride = rows_padded * ldk;
-    int8_t* out = planes + row * ldk + k;
-#define ESHKOL_SPLIT_ONE(L)                                                           \
-    if (L < NMOD) {                                                                   \
-        const int r0 = residue<L>(t0, n0), r1 = residue<L>(t1, n1);                   \
-        *(uint16_t*)(out + (uint64_t)L * plane_stride) =                              \
-            (uint16_t)((uint8_t)(int8_t)r0 | ((uint16_t)(uint8_t)(int8_t)r1 << 8));   \
-    }
-    ESHKOL_SPLIT_ONE(0)  ESHKOL_SPLIT_ONE(1)  ESHKOL_SPLIT_ONE(2)  ESHKOL_SPLIT_ONE(3)
-    ESHKOL_SPLIT_ONE(4)  ESHKOL_SPLIT_ONE(5)  ESHKOL_SPLIT_ONE(6)  ESHKOL_SPLIT_ONE(7)
-    ESHKOL_SPLIT_ONE(8)  ESHKOL_SPLIT_ONE(9)  ESHKOL_SPLIT_ONE(10) ESHKOL_SPLIT_ONE(11)
-    ESHKOL_SPLIT_ONE(12) ESHKOL_SPLIT_ONE(13) ESHKOL_SPLIT_ONE(14) ESHKOL_SPLIT_ONE(15)
-#undef ESHKOL_SPLIT_ONE
+    kmaj::for_each_pair(X, rows, K, rows_padded, ldk, tile,
+        [&](uint64_t row, uint64_t k, double x0, double x1) {
+            const int sh = (row < rows) ? shift[row] : 0;
+            split_pair<NMOD>(x0, x1, sh, planes + row * ldk + k, plane_stride);
+        });
 }
 
 struct CrtConsts {
@@ -256,7 +276,13 @@ HipOzakiCrtStages g_last = {};
 
 template <int NMOD>
 void launch_split(const double* X, uint64_t rows, uint64_t K, const int32_t* shift, int8_t* planes,
-                  uint64_t rows_padded, uint64_t ldk, hipStream_t st) {
+                  uint64_t rows_padded, uint64_t ldk, bool kmajor, hipStream_t st) {
+    if (kmajor) {
+        dim3 grid((unsigned)kmaj::grid_blocks(rows_padded, ldk));
+        hipLaunchKernelGGL(crt_split_kmajor_kernel<NMOD>, grid, dim3(256), 0, st, X, rows, K, shift, planes,
+                           rows_padded, ldk);
+        return;
+    }
     dim3 grid((unsigned)(((ldk / 2 + 255) / 256) * rows_padded));
     hipLaunchKernelGGL(crt_split_kernel<NMOD>, grid, dim3(256), 0, st, X, rows, K, shift, planes,
                        rows_padded, ldk);
@@ -264,21 +290,35 @@ void launch_split(const double* X, uint64_t rows, uint64_t K, const int32_t* shi
 
 }  // namespace
 
-extern "C" int hip_ozaki_crt_split_f64(const double* X, uint64_t rows, uint64_t K,
-                                       const int32_t* shift, int num_moduli,
-                                       int8_t* planes, uint64_t rows_padded, uint64_t ldk, void* stream) {
+namespace {
+int crt_split_any(const double* X, uint64_t rows, uint64_t K, const int32_t* shift, int num_moduli,
+                  int8_t* planes, uint64_t rows_padded, uint64_t ldk, bool kmajor, void* stream) {
     if (!X || !shift || !planes || rows == 0 || K == 0) return -1;
     if (num_moduli < 2 || num_moduli > MAX_MODULI) return -1;
     if (rows_padded < rows || ldk < K || (ldk & 1)) return -1;
     if (((ldk / 2 + 255) / 256) * rows_padded > 0x7fffffffULL) return -1;
+    if (kmaj::grid_blocks(rows_padded, ldk) > 0x7fffffffULL) return -1;
     hipStream_t st = (hipStream_t)stream;
     switch (num_moduli) {
-#define CASE(n) case n: launch_split<n>(X, rows, K, shift, planes, rows_padded, ldk, st); break;
+#define CASE(n) case n: launch_split<n>(X, rows, K, shift, planes, rows_padded, ldk, kmajor, st); break;
         CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8) CASE(9)
         CASE(10) CASE(11) CASE(12) CASE(13) CASE(14) CASE(15) CASE(16)
 #undef CASE
     }
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+}  // namespace
+
+extern "C" int hip_ozaki_crt_split_f64(const double* X, uint64_t rows, uint64_t K,
+                                       const int32_t* shift, int num_moduli,
+                                       int8_t* planes, uint64_t rows_padded, uint64_t ldk, void* stream) {
+    return crt_split_any(X, rows, K, shift, num_moduli, planes, rows_padded, ldk, false, stream);
+}
+
+extern "C" int hip_ozaki_crt_split_kmajor_f64(const double* X, uint64_t rows, uint64_t K,
+                                              const int32_t* shift, int num_moduli,
+                                              int8_t* planes, uint64_t rows_padded, uint64_t ldk, void* stream) {
+    return crt_split_any(X, rows, K, shift, num_moduli, planes, rows_padded, ldk, true, stream);
 }
 
 extern "C" int hip_ozaki_crt_reconstruct_f64(const int8_t* w_planes, uint64_t M, uint64_t N, int num_moduli,
@@ -333,20 +373,11 @@ extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, dou
     if (ensure_tables(st) != 0) return -1;
 
     const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ldk = round_up_sz(K, 256);
-    /* Both operands are split along rows with k contiguous: B goes through its
-     * transpose unless the caller already holds it, A only if the caller holds
-     * A transposed. */
-    const double* Bt = B;
-    if (!trans_b) {
-        double* t = (double*)eshkol_hip_workspace(WS_BT, K * N * sizeof(double));
-        if (!t || hip_transpose_f64(B, t, K, N, (hipStream_t)stream) != 0) return -1;
-        Bt = t;
-    }
-    if (trans_a) {
-        double* t = (double*)eshkol_hip_workspace(WS_AT, M * K * sizeof(double));
-        if (!t || hip_transpose_f64(A, t, K, M, (hipStream_t)stream) != 0) return -1;
-        A = t;
-    }
+    /* Both operands come out as planes [row][k]. An operand stored with k
+     * contiguous (A as given, B when the caller holds B^T) is read row by row;
+     * one stored k-major (B as given, A when the caller holds A^T) is read
+     * through LDS tiles: no transposed fp64 copy is made either way. */
+    const bool a_kmajor = trans_a != 0, b_kmajor = trans_b == 0;
     double* amax = (double*)eshkol_hip_workspace(WS_ROWSCALE, M * sizeof(double));
     double* bmax = (double*)eshkol_hip_workspace(WS_COLSCALE, N * sizeof(double));
     int32_t* dmu = (int32_t*)eshkol_hip_workspace(WS_ROWSHIFT, M * sizeof(int32_t));
@@ -359,23 +390,35 @@ extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, dou
     int32_t* h_mu = (int32_t*)(h_bmax + N);
     int32_t* h_nu = h_mu + M;
 
-    if (hip_rowabsmax_f64(A, M, K, 0.0, amax, st) != 0) return -1;
-    if (hip_rowabsmax_f64(Bt, N, K, 0.0, bmax, st) != 0) return -1;
+    if ((a_kmajor ? hip_colabsmax_f64(A, K, M, 0.0, amax, st) : hip_rowabsmax_f64(A, M, K, 0.0, amax, st)) != 0) return -1;
+    if ((b_kmajor ? hip_colabsmax_f64(B, K, N, 0.0, bmax, st) : hip_rowabsmax_f64(B, N, K, 0.0, bmax, st)) != 0) return -1;
     if (!ESHKOL_HIP_OK(hipMemcpyAsync(h_amax, amax, M * sizeof(double), hipMemcpyDeviceToHost, st))) return -1;
     if (!ESHKOL_HIP_OK(hipMemcpyAsync(h_bmax, bmax, N * sizeof(double), hipMemcpyDeviceToHost, st))) return -1;
     if (!ESHKOL_HIP_OK(hipStreamSynchronize(st))) return -1;
 
-    /* frac bounds (gpu_memory.mm:403-417); a non-finite maximum marks NaN/Inf input */
+    /* frac bounds (gpu_memory.mm:403-417); a non-finite maximum marks NaN/Inf input.
+     * floor(log2(max)) is needed again for the shifts below: it is kept in the
+     * shift arrays so each maximum costs one log2. */
     double frac_A = 0.0, frac_B = 0.0;
     for (uint64_t i = 0; i < M; i++) {
         const double m = h_amax[i];
         if (!std::isfinite(m)) return -1;
-        if (m > 0.0) { double lg = log2(m); double f = lg - floor(lg); if (f > frac_A) frac_A = f; }
+        h_mu[i] = 0;
+        if (m > 0.0) {
+            const double lg = log2(m), fl = floor(lg), f = lg - fl;
+            h_mu[i] = (int32_t)fl;
+            if (f > frac_A) frac_A = f;
+        }
     }
     for (uint64_t j = 0; j < N; j++) {
         const double m = h_bmax[j];
         if (!std::isfinite(m)) return -1;
-        if (m > 0.0) { double lg = log2(m); double f = lg - floor(lg); if (f > frac_B) frac_B = f; }
+        h_nu[j] = 0;
+        if (m > 0.0) {
+            const double lg = log2(m), fl = floor(lg), f = lg - fl;
+            h_nu[j] = (int32_t)fl;
+            if (f > frac_B) frac_B = f;
+        }
     }
     const double log2K = log2((double)K);
     if (adaptive) {                                   /* gpu_memory.mm:433-453 */
@@ -398,11 +441,11 @@ extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, dou
     if (E > 52) E = 52;
     if (E < 0) E = 0;
     for (uint64_t i = 0; i < M; i++) {
-        h_mu[i] = (h_amax[i] == 0.0) ? 0 : E - (int)floor(log2(h_amax[i]));
+        h_mu[i] = (h_amax[i] == 0.0) ? 0 : E - h_mu[i];
         if (h_mu[i] > 1023 || h_mu[i] < -1022) return -1;
     }
     for (uint64_t j = 0; j < N; j++) {
-        h_nu[j] = (h_bmax[j] == 0.0) ? 0 : E - (int)floor(log2(h_bmax[j]));
+        h_nu[j] = (h_bmax[j] == 0.0) ? 0 : E - h_nu[j];
         if (h_nu[j] > 1023 || h_nu[j] < -1022) return -1;
     }
     if (!ESHKOL_HIP_OK(hipMemcpyAsync(dmu, h_mu, M * sizeof(int32_t), hipMemcpyHostToDevice, st))) return -1;
@@ -413,8 +456,8 @@ extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, dou
     int8_t* Wp = (int8_t*)eshkol_hip_workspace(WS_PRODUCTS, (size_t)num_moduli * M * N);
     if (!Ap || !Bp || !Wp) return -1;
 
-    if (hip_ozaki_crt_split_f64(A, M, K, dmu, num_moduli, Ap, Mp, ldk, st) != 0) return -1;
-    if (hip_ozaki_crt_split_f64(Bt, N, K, dnu, num_moduli, Bp, Np, ldk, st) != 0) return -1;
+    if (crt_split_any(A, M, K, dmu, num_moduli, Ap, Mp, ldk, a_kmajor, st) != 0) return -1;
+    if (crt_split_any(B, N, K, dnu, num_moduli, Bp, Np, ldk, b_kmajor, st) != 0) return -1;
 
     HipIgemmArgs ga;
     memset(&ga, 0, sizeof ga);

@@ -72,6 +72,13 @@ int hip_transpose_f64(const double* in, double* out, uint64_t rows, uint64_t col
 int hip_rowabsmax_f64(const double* A, uint64_t M, uint64_t K, double zero_value,
                       double* rmax, void* stream);
 
+/* cmax[j] = max_k |X[k,j]| of a row-major X[K][R], same conventions as
+ * hip_rowabsmax_f64: the column maxima of B without transposing it
+ * (ozaki_colmax_f64_kernel, gpu_cuda_kernels.cu:675-685). Uses the library
+ * workspace. */
+int hip_colabsmax_f64(const double* X, uint64_t K, uint64_t R, double zero_value,
+                      double* cmax, void* stream);
+
 /* The 15 operations of EshkolElementwiseOp; cuda_launch_elementwise_f64,
  * gpu_cuda_kernels.cu:21-43. b may be NULL (identity operand). */
 int hip_elementwise_f64(const double* a, const double* b, double* out, uint64_t n, int op, void* stream);
@@ -124,6 +131,12 @@ int hip_ozaki_crt_split_f64(const double* X, uint64_t rows, uint64_t K,
                             const int32_t* shift, int num_moduli,
                             int8_t* planes, uint64_t rows_padded, uint64_t ldk, void* stream);
 
+/* The same planes from a k-major operand X[K][rows] (B as the runtime stores
+ * it): output identical to hip_ozaki_crt_split_f64 on X^T. */
+int hip_ozaki_crt_split_kmajor_f64(const double* X, uint64_t rows, uint64_t K,
+                                   const int32_t* shift, int num_moduli,
+                                   int8_t* planes, uint64_t rows_padded, uint64_t ldk, void* stream);
+
 /* CRT accumulation, reconstruction and inverse scaling (gpu_memory.mm:2626-2655)
  * from the int8 residue products w_planes[l][M][N]; optional fused dense-layer
  * epilogue C = act(C + bias[j]) (act 0 none, 1 tanh; bias may be NULL). */
@@ -160,6 +173,11 @@ int hip_ozaki_crt_last_stages(HipOzakiCrtStages* out);
  * for B when X is B transposed. */
 int hip_ozaki_slice_f64(const double* X, uint64_t rows, uint64_t K, const double* scale, int s,
                         int8_t* planes, uint64_t rows_padded, uint64_t ldk, void* stream);
+
+/* The same planes from a k-major operand X[K][rows]: the reference's B kernel
+ * (gpu_cuda_kernels.cu:706-723); output identical to hip_ozaki_slice_f64 on X^T. */
+int hip_ozaki_slice_kmajor_f64(const double* X, uint64_t rows, uint64_t K, const double* scale, int s,
+                               int8_t* planes, uint64_t rows_padded, uint64_t ldk, void* stream);
 
 /* cuda_ozaki_reconstruct_f64 (gpu_cuda_kernels.cu:728-741, 779-798), weights
  * already in device memory. */
@@ -200,11 +218,15 @@ int hip_hgemm_16(const uint16_t* A, const uint16_t* Bt, uint64_t M, uint64_t K, 
 int hip_convert_f64_to_16(const double* in, uint16_t* out, uint64_t rows, uint64_t cols,
                           uint64_t rows_padded, uint64_t ld, int is_bf16, void* stream);
 
+/* The same narrowing from a k-major operand in[cols][rows]: out[i][k] = in[k][i]. */
+int hip_convert_f64_to_16_kmajor(const double* in, uint16_t* out, uint64_t rows, uint64_t cols,
+                                 uint64_t rows_padded, uint64_t ld, int is_bf16, void* stream);
+
 /* ---- operands held transposed, and the backward pass ---------------------------
  * The tier pipelines with the trans_a / trans_b meaning of hip_dgemm_f64_ex.
- * The Ozaki and reduced tiers split both operands along rows with k
- * contiguous, so a B the caller holds transposed saves them their transpose
- * pass, and an A held transposed costs one. */
+ * The Ozaki and reduced tiers turn both operands into planes [row][k]; an
+ * operand stored k-major is read through LDS tiles, so neither form costs a
+ * transposed copy. */
 int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, double* C,
                                 uint64_t M, uint64_t K, uint64_t N,
                                 int trans_a, int trans_b, int num_moduli, int adaptive,

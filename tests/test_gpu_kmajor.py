@@ -1,0 +1,109 @@
+"""Operands read k-major (B as the runtime stores it) without a transposed copy:
+column maxima, CRT residue planes, INT8 slice planes and 16-bit narrowing must
+be bit-identical to the row-major kernels applied to an explicit transpose,
+padding included. The row-major kernels are themselves checked against the
+oracle in the tier tests, so equality here carries that parity over."""
+import numpy as np
+import pytest
+
+import eshkol_amd as ea
+from eshkol_amd import synth
+from gpu_util import stream
+
+pytestmark = pytest.mark.gpu
+
+# (K, R): k extent, number of rows of the transposed view (columns of the stored matrix)
+SHAPES = [(1, 1), (2, 3), (7, 5), (64, 64), (128, 32), (129, 33), (130, 257), (300, 70), (1000, 513),
+          (1024, 1024), (2049, 511)]
+
+
+def dev(x, dtype=np.float64):
+    return ea.DeviceArray.from_host(np.ascontiguousarray(x, dtype=dtype))
+
+
+def pad(n, m):
+    return (n + m - 1) // m * m
+
+
+@pytest.mark.parametrize("K,R", SHAPES)
+def test_column_maxima(gpu, K, R):
+    lib = ea.load()
+    X = synth.wide_range(K * 31 + R, (K, R))
+    X[:, R // 2] = 0.0                                   # an all-zero column takes zero_value
+    dX, dXt = dev(X), dev(X.T)
+    for zero_value in (0.0, 1.0):
+        a, b = ea.DeviceArray((R,)), ea.DeviceArray((R,))
+        assert lib.hip_colabsmax_f64(dX.ptr, K, R, zero_value, a.ptr, stream()) == 0
+        assert lib.hip_rowabsmax_f64(dXt.ptr, R, K, zero_value, b.ptr, stream()) == 0
+        ea.synchronize()
+        got = a.download()
+        assert np.array_equal(got, b.download())
+        want = np.abs(X).max(axis=0)
+        want[want == 0.0] = zero_value
+        assert np.array_equal(got, want)
+
+
+def test_column_maxima_flag_non_finite_input(gpu):
+    lib = ea.load()
+    X = synth.normal(3, (200, 70))
+    X[17, 5] = np.nan
+    X[199, 69] = -np.inf
+    out = ea.DeviceArray((70,))
+    assert lib.hip_colabsmax_f64(dev(X).ptr, 200, 70, 0.0, out.ptr, stream()) == 0
+    ea.synchronize()
+    got = out.download()
+    assert np.isposinf(got[5]) and np.isposinf(got[69]) and np.isfinite(np.delete(got, [5, 69])).all()
+
+
+@pytest.mark.parametrize("K,R", SHAPES)
+@pytest.mark.parametrize("nmod", [2, 9, 16])
+def test_crt_planes(gpu, K, R, nmod):
+    lib = ea.load()
+    X = synth.wide_range(K + 7 * R, (K, R), -8, 8)
+    shift = (20 - np.floor(np.log2(np.maximum(np.abs(X).max(axis=0), 1e-300)))).astype(np.int32)
+    Rp, ldk = pad(R, 256), pad(K, 256)
+    dX, dXt, dsh = dev(X), dev(X.T), dev(shift, np.int32)
+    pa = ea.DeviceArray.from_host(np.full((nmod, Rp, ldk), 77, np.int8))
+    pb = ea.DeviceArray.from_host(np.full((nmod, Rp, ldk), 78, np.int8))
+    assert lib.hip_ozaki_crt_split_kmajor_f64(dX.ptr, R, K, dsh.ptr, nmod, pa.ptr, Rp, ldk, stream()) == 0
+    assert lib.hip_ozaki_crt_split_f64(dXt.ptr, R, K, dsh.ptr, nmod, pb.ptr, Rp, ldk, stream()) == 0
+    ea.synchronize()
+    a = pa.download()
+    assert np.array_equal(a, pb.download())
+    assert not a[:, R:, :].any() and not a[:, :, K:].any()
+
+
+@pytest.mark.parametrize("K,R", SHAPES)
+def test_slice_planes(gpu, K, R):
+    lib = ea.load()
+    s = 7
+    X = synth.normal(K + 3 * R, (K, R))
+    scale = np.abs(X).max(axis=0)
+    scale[scale == 0.0] = 1.0
+    Rp, ldk = pad(R, 256), pad(K, 256)
+    dX, dXt, dsc = dev(X), dev(X.T), dev(scale)
+    pa = ea.DeviceArray.from_host(np.full((s, Rp, ldk), 77, np.int8))
+    pb = ea.DeviceArray.from_host(np.full((s, Rp, ldk), 78, np.int8))
+    assert lib.hip_ozaki_slice_kmajor_f64(dX.ptr, R, K, dsc.ptr, s, pa.ptr, Rp, ldk, stream()) == 0
+    assert lib.hip_ozaki_slice_f64(dXt.ptr, R, K, dsc.ptr, s, pb.ptr, Rp, ldk, stream()) == 0
+    ea.synchronize()
+    a = pa.download()
+    assert np.array_equal(a, pb.download())
+    assert not a[:, R:, :].any() and not a[:, :, K:].any()
+
+
+@pytest.mark.parametrize("K,R", SHAPES)
+@pytest.mark.parametrize("is_bf16", [0, 1])
+def test_narrowing(gpu, K, R, is_bf16):
+    lib = ea.load()
+    X = synth.normal(K + 5 * R, (K, R))
+    Rp, ld = pad(R, 256), pad(K, 128)
+    dX, dXt = dev(X), dev(X.T)
+    pa = ea.DeviceArray.from_host(np.full((Rp, ld), 0x7777, np.uint16))
+    pb = ea.DeviceArray.from_host(np.full((Rp, ld), 0x7878, np.uint16))
+    assert lib.hip_convert_f64_to_16_kmajor(dX.ptr, pa.ptr, R, K, Rp, ld, is_bf16, stream()) == 0
+    assert lib.hip_convert_f64_to_16(dXt.ptr, pb.ptr, R, K, Rp, ld, is_bf16, stream()) == 0
+    ea.synchronize()
+    a = pa.download()
+    assert np.array_equal(a, pb.download())
+    assert not a[R:, :].any() and not a[:, K:].any()
