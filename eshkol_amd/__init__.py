@@ -97,6 +97,7 @@ SIGNATURES = {
     "hip_dgemm_f64": (C.c_int, [vp, vp, vp, u64, u64, u64, vp]),
     "hip_dgemm_f64_ex": (C.c_int, [vp, vp, vp, u64, u64, u64, C.c_int, C.c_int, vp]),
     "hip_dgemm_f64_batched": (C.c_int, [vp, vp, vp, u64, u64, u64, u64, vp]),
+    "hip_dgemm_set_fast_path": (None, [C.c_int]),
     "hip_sgemm_f32": (C.c_int, [vp, vp, vp, u64, u64, u64, vp]),
     "hip_transpose_f64": (C.c_int, [vp, vp, u64, u64, vp]),
     "hip_colabsmax_f64": (C.c_int, [vp, u64, u64, C.c_double, vp, vp]),

@@ -92,11 +92,11 @@ void convert_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
 
 /* k-major X[K][rows] (B as the runtime stores it), same output. */
 template <bool BF16>
-__global__ __launch_bounds__(256)
+__global__ __launch_bounds__(256, 4)
 void convert_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
                            uint16_t* __restrict__ out, uint64_t rows_padded, uint64_t ld) {
     __shared__ __align__(16) double tile[kmaj::SMEM_DOUBLES];
-    kmaj::for_each_pair(X, rows, K, rows_padded, ld, tile,
+    kmaj::for_each_pair<false>(X, rows, K, rows_padded, ld, tile,
         [&](uint64_t row, uint64_t k, double x0, double x1) {
             *(uint32_t*)(out + row * ld + k) = narrow_pair<BF16>(x0, x1);
         });

@@ -19,8 +19,9 @@
  *
  * The B fragment is passed as the MFMA's first operand, so a lane ends up with
  * 4 consecutive columns of one output row and stores them as one word (int8)
- * or one 16-byte vector (int32). Mode 1 reduces modulo p in fp64 (exact:
- * |sum| < 2^31), stages the int8 tile through LDS and writes 16-byte chunks.
+ * or one 16-byte vector (int32). Mode 1 reduces modulo p exactly (two integer
+ * folds of 2^14, then a nearest-multiple step in fp32), stages the int8 tile
+ * through LDS and writes 16-byte chunks.
  *
  * One launch covers every output plane. Workgroup ids congruent mod 8 run on
  * the same XCD; the id is remapped so that XCD x owns the x-th eighth of every
@@ -106,9 +107,17 @@ __device__ __forceinline__ void epilogue(const HipIgemmArgs& g, int o, int m0, i
         return;
     }
 
-    /* mode 1: residues modulo p, staged through LDS */
+    /* mode 1: residues modulo p, staged through LDS.
+     * |sum| <= K * 128 * 128 < 2^31. Fold 2^14 into the modulus twice (the
+     * result is below 2^21 in magnitude, exact in fp32), then take the nearest
+     * multiple of p in fp32: x/p < 2^14 is known to within 1e-3 and, unless it is
+     * a tie, lies at least 1/(2p) >= 2e-3 from a half-integer, so q is the
+     * nearest integer and x - q p is exact and in [-p/2, p/2]; the tie (even p)
+     * is folded to -p/2. Every instruction is full rate, unlike the fp64
+     * conversions and the 32-bit multiply a direct reduction needs. */
     const int p = g.modulus[o];
-    const double pinv = 1.0 / (double)p;
+    const int c14 = 16384 % p;
+    const float pf = (float)p, pinv = 1.0f / (float)p;
     constexpr int EPITCH = BN + 16;
 #pragma unroll
     for (int t = 0; t < TM; t++) {
@@ -122,10 +131,12 @@ __device__ __forceinline__ void epilogue(const HipIgemmArgs& g, int o, int m0, i
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     const int s = acc[t][u][4 * v + e];
-                    const int qd = (int)rint((double)s * pinv);
-                    int r = s - qd * p;
+                    const int x1 = (s >> 14) * c14 + (s & 0x3fff);       /* |x1| < 2^26 */
+                    const int x2 = (x1 >> 14) * c14 + (x1 & 0x3fff);     /* |x2| < 2^21 */
+                    const float xf = (float)x2;
+                    const float q = rintf(xf * pinv);
+                    int r = (int)fmaf(-q, pf, xf);
                     if (2 * r >= p) r -= p;
-                    else if (2 * r < -p) r += p;
                     packed |= ((uint32_t)(uint8_t)(int8_t)r) << (8 * e);
                 }
                 *(uint32_t*)(stage + lrow * EPITCH + lcol) = packed;

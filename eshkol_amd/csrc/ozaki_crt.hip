@@ -73,9 +73,17 @@ __device__ __forceinline__ int residue(uint64_t t, bool neg) {
     const uint32_t lo = (uint32_t)(t & 0x3ffff);
     const uint32_t mid = (uint32_t)((t >> 18) & 0x3ffff);
     const uint32_t hi = (uint32_t)(t >> 36);
-    uint32_t r = (hi * (uint32_t)TBL.c36[L] + mid * (uint32_t)TBL.c18[L] + lo) % (uint32_t)p;
-    int s = (int)r;
-    if (neg && s != 0) s = p - s;
+    /* fold 2^36 and 2^18 into the modulus twice: t = r27 = x (mod p), x < 2^19 */
+    const uint32_t r27 = hi * (uint32_t)TBL.c36[L] + mid * (uint32_t)TBL.c18[L] + lo;   /* < 2^27 */
+    const uint32_t x = (r27 >> 18) * (uint32_t)TBL.c18[L] + (r27 & 0x3ffff);
+    /* nearest-multiple reduction in fp32, all full-rate instructions. x/p < 2^12
+     * is computed to within 4e-4 and, unless it is a tie, lies at least 1/(2p) >=
+     * 2e-3 from a half-integer, so q is the nearest integer to x/p and x - q p is
+     * exact and already in [-p/2, p/2]. The tie (p = 256, x = 128 mod 256) may
+     * come out as +128 and is folded to -128. */
+    const float xf = neg ? -(float)x : (float)x;
+    const float q = rintf(xf * (1.0f / (float)p));
+    int s = (int)fmaf(-q, (float)p, xf);
     if (2 * s >= p) s -= p;
     return s;
 }
@@ -126,13 +134,13 @@ void crt_split_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
 
 /* k-major X[K][rows] (B as the runtime stores it), same output. */
 template <int NMOD>
-__global__ __launch_bounds__(256)
+__global__ __launch_bounds__(256, 4)
 void crt_split_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
                              const int32_t* __restrict__ shift, int8_t* __restrict__ planes,
                              uint64_t rows_padded, uint64_t ldk) {
     __shared__ __align__(16) double tile[kmaj::SMEM_DOUBLES];
     const uint64_t plane_stride = rows_padded * ldk;
-    kmaj::for_each_pair(X, rows, K, rows_padded, ldk, tile,
+    kmaj::for_each_pair<true>(X, rows, K, rows_padded, ldk, tile,
         [&](uint64_t row, uint64_t k, double x0, double x1) {
             const int sh = (row < rows) ? shift[row] : 0;
             split_pair<NMOD>(x0, x1, sh, planes + row * ldk + k, plane_stride);

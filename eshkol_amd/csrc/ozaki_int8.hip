@@ -69,13 +69,13 @@ void slice_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
 /* k-major X[K][rows] (B as the runtime stores it), same output: the job of the
  * reference's B kernel (gpu_cuda_kernels.cu:706-723), which scatters transposed
  * bytes; here the transposition happens in LDS and the stores stay contiguous. */
-__global__ __launch_bounds__(256)
+__global__ __launch_bounds__(256, 4)
 void slice_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
                          const double* __restrict__ scale, int s, int8_t* __restrict__ planes,
                          uint64_t rows_padded, uint64_t ldk) {
     __shared__ __align__(16) double tile[kmaj::SMEM_DOUBLES];
     const uint64_t plane_stride = rows_padded * ldk;
-    kmaj::for_each_pair(X, rows, K, rows_padded, ldk, tile,
+    kmaj::for_each_pair<false>(X, rows, K, rows_padded, ldk, tile,
         [&](uint64_t row, uint64_t k, double x0, double x1) {
             const double sc = (row < rows) ? scale[row] : 1.0;
             slice_pair(x0, x1, sc, s, planes + row * ldk + k, plane_stride);

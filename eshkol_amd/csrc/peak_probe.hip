@@ -4,11 +4,12 @@
  * under the same kind of data.
  *
  * The matrix-core probes run a register-only MFMA loop (no memory traffic, every
- * SIMD occupied by several waves). With constant operands they reach the
- * published rates; with random operand bits the chip lowers its clock to hold
- * its power limit and sustains markedly less (about 63 of 78.6 TFLOP/s for fp64,
- * 3.0 of 5.0 POP/s for int8, 1.7 of 2.5 PFLOP/s for bf16 were measured). A GEMM
- * on real data cannot beat the random-operand figure.
+ * SIMD occupied by several waves, operand registers fixed at compile time). With
+ * constant operands the int8 and bf16 loops reach the published rates; with
+ * random operand bits the chip lowers its clock to hold its power limit and
+ * sustains markedly less (about 3.0 of 5.0 POP/s for int8 and 1.7 of 2.5 PFLOP/s
+ * for bf16 were measured). The figures are context for the GEMM numbers, not
+ * bounds: a GEMM also spends power on LDS and cache traffic.
  *
  * The memory probe is a plain 16-byte-per-lane copy of a buffer much larger
  * than the caches: the read+write rate HBM sustains.
@@ -43,7 +44,7 @@ void probe_f64(int iters, int random, int* sink) {
     for (int it = 0; it < iters; it++) {
 #pragma unroll
         for (int i = 0; i < 8; i++)
-            acc[i] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[i], b[(i + it) & 7], acc[i], 0, 0, 0);
+            acc[i] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[i], b[(i + 3) & 7], acc[i], 0, 0, 0);
     }
     double s = 0.0;
     for (int i = 0; i < 8; i++) for (int r = 0; r < 4; r++) s += acc[i][r];
@@ -68,7 +69,7 @@ void probe_i8(int iters, int random, int* sink) {
     for (int it = 0; it < iters; it++) {
 #pragma unroll
         for (int i = 0; i < 8; i++)
-            acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[(i + it) & 7], acc[i], 0, 0, 0);
+            acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[(i + 3) & 7], acc[i], 0, 0, 0);
     }
     int s = 0;
     for (int i = 0; i < 8; i++) for (int r = 0; r < 16; r++) s += acc[i][r];
@@ -95,7 +96,7 @@ void probe_bf16(int iters, int random, int* sink) {
 #pragma unroll
         for (int i = 0; i < 8; i++)
             acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8b_t, a[i]),
-                                                             __builtin_bit_cast(v8b_t, b[(i + it) & 7]),
+                                                             __builtin_bit_cast(v8b_t, b[(i + 3) & 7]),
                                                              acc[i], 0, 0, 0);
     }
     float s = 0.0f;

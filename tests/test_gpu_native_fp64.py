@@ -84,3 +84,44 @@ def test_full_size_properties(gpu, M, K, N):
     Cg = run_dgemm(A, B)
     ref = oracle.matmul_f64(A[rows], B[:, cols])
     assert normwise(Cg[rows][:, cols], ref, A[rows], B[:, cols]) <= TOL
+
+
+@pytest.mark.parametrize("M,K,N", [(2048, 16, 2048), (2048, 48, 2048), (2048, 1024, 2048), (4096, 2064, 1024), (1024, 512, 4096)])
+def test_straight_line_kernel_matches_bounds_checked_kernel_bitwise(gpu, M, K, N):
+    """Interior shapes take a kernel without bounds checks: same tiles, same
+    summation order, so the same bits, for all three operand forms."""
+    import eshkol_amd as ea
+    from gpu_util import stream
+    lib = ea.load()
+    A, B = synth.normal(M + K, (M, K)), synth.normal(K + N, (K, N))
+    ref = oracle.matmul_f64(A, B) if M * K * N <= 2 ** 32 else None
+    forms = [(A, B, 0, 0), (A, np.ascontiguousarray(B.T), 0, 1), (np.ascontiguousarray(A.T), B, 1, 0)]
+    for X, Y, ta, tb in forms:
+        dX, dY = ea.DeviceArray.from_host(X), ea.DeviceArray.from_host(Y)
+        outs = []
+        try:
+            for fast in (0, 1):
+                lib.hip_dgemm_set_fast_path(fast)
+                dC = ea.DeviceArray.from_host(np.full((M, N), np.nan))
+                assert lib.hip_dgemm_f64_ex(dX.ptr, dY.ptr, dC.ptr, M, K, N, ta, tb, stream()) == 0
+                ea.synchronize()
+                outs.append(dC.download())
+        finally:
+            lib.hip_dgemm_set_fast_path(1)
+        assert np.array_equal(outs[0], outs[1]), (ta, tb)
+        if ref is not None:
+            assert normwise(outs[1], ref, A, B) <= TOL
+
+
+def test_straight_line_kernel_in_a_batch(gpu):
+    import eshkol_amd as ea
+    from gpu_util import stream
+    lib = ea.load()
+    bt, M, K, N = 3, 2048, 64, 2048
+    a, b = synth.normal(5, (bt, M, K)), synth.normal(6, (bt, K, N))
+    da, db, dc = ea.DeviceArray.from_host(a), ea.DeviceArray.from_host(b), ea.DeviceArray((bt, M, N))
+    assert lib.hip_dgemm_f64_batched(da.ptr, db.ptr, dc.ptr, bt, M, K, N, stream()) == 0
+    ea.synchronize()
+    got = dc.download()
+    for i in range(bt):
+        assert normwise(got[i], oracle.matmul_f64(a[i], b[i]), a[i], b[i]) <= TOL
