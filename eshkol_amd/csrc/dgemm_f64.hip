@@ -232,10 +232,13 @@ void dgemm_mfma_kernel(const double* __restrict__ A, const double* __restrict__ 
         }
 }
 
-/* ---- interior fast path -------------------------------------------------------
- * M, N multiples of 128, K a multiple of 16, 16-byte aligned operands: no
- * bounds checks, so a k-block is one straight-line region and its memory
- * operations can be placed between the MFMAs instead of around them:
+/* ---- straight-line kernel -----------------------------------------------------
+ * For launches of at least 256 tiles whose operands move as 16-byte chunks
+ * (even row pitches, aligned bases). The loads carry no bounds checks: rows of
+ * an edge tile are clamped to the matrix (their outputs are never stored) and a
+ * k-tail is zeroed with selects in a variant of its own. A k-block is therefore
+ * one straight-line region and its memory operations can be placed between the
+ * MFMAs instead of around them:
  *
  *   step 0   MFMAs of k 0..3    | LDS reads of the step-1 fragments
  *   step 1   MFMAs of k 4..7    | LDS reads of step 2
@@ -258,7 +261,7 @@ __device__ __forceinline__ void lds_only_barrier() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-template <bool TA, bool TB>
+template <bool TA, bool TB, bool KTAIL>
 __global__ __launch_bounds__(256, 2)
 void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ B,
                        double* __restrict__ C, int M, int N, int K,
@@ -284,31 +287,62 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
     const int wm = wave >> 1, wn = wave & 1;
     const int li = lane & 15, lg = lane >> 4;
 
-    /* this thread's four 16-byte chunks of each operand tile: global pointers for k-block 0 */
+    /* This thread's four 16-byte chunks of each operand tile: global pointers
+     * for k-block 0. Rows beyond the matrix (edge tiles) are clamped to its last
+     * rows: they load valid memory and feed outputs that are never stored. */
     const double* pa[OpA::CHUNKS];
     const double* pb[OpB::CHUNKS];
+    int ka[OpA::CHUNKS], kbo[OpB::CHUNKS];       /* first k of the chunk inside a k-block */
 #pragma unroll
     for (int r = 0; r < OpA::CHUNKS; r++) {
         const int c = tid + 256 * r;
-        pa[r] = TA ? A + (size_t)(c / (BM / 2)) * M + m0 + 2 * (c % (BM / 2))
-                   : A + (size_t)(m0 + (c >> 3)) * K + 2 * (c & 7);
+        if (TA) {
+            int m = m0 + 2 * (c % (BM / 2));
+            m = (m < M - 2) ? m : M - 2;
+            ka[r] = c / (BM / 2);
+            pa[r] = A + (size_t)ka[r] * M + m;
+        } else {
+            int m = m0 + (c >> 3);
+            m = (m < M - 1) ? m : M - 1;
+            ka[r] = 2 * (c & 7);
+            pa[r] = A + (size_t)m * K + ka[r];
+        }
     }
 #pragma unroll
     for (int r = 0; r < OpB::CHUNKS; r++) {
         const int c = tid + 256 * r;
-        pb[r] = TB ? B + (size_t)(n0 + (c >> 3)) * K + 2 * (c & 7)
-                   : B + (size_t)(c / (BN / 2)) * N + n0 + 2 * (c % (BN / 2));
+        if (TB) {
+            int n = n0 + (c >> 3);
+            n = (n < N - 1) ? n : N - 1;
+            kbo[r] = 2 * (c & 7);
+            pb[r] = B + (size_t)n * K + kbo[r];
+        } else {
+            int n = n0 + 2 * (c % (BN / 2));
+            n = (n < N - 2) ? n : N - 2;
+            kbo[r] = c / (BN / 2);
+            pb[r] = B + (size_t)kbo[r] * N + n;
+        }
     }
     const size_t a_step = TA ? (size_t)BK * M : (size_t)BK;     /* doubles per k-block */
     const size_t b_step = TB ? (size_t)BK : (size_t)BK * N;
 
     OpA a;
     OpB b;
+    /* KTAIL: K is not a multiple of 16. A chunk whose k lies beyond K reads the
+     * same chunk of k-block 0 instead (valid memory, K >= 16) and is zeroed. */
     auto gload = [&](int kb) {
 #pragma unroll
-        for (int r = 0; r < OpA::CHUNKS; r++) a.reg[r] = *(const d2_t*)(pa[r] + (size_t)kb * a_step);
+        for (int r = 0; r < OpA::CHUNKS; r++) {
+            const bool ok = !KTAIL || (kb * BK + ka[r] < K);
+            const d2_t v = *(const d2_t*)(pa[r] + (size_t)(ok ? kb : 0) * a_step);
+            a.reg[r] = ok ? v : (d2_t){0.0, 0.0};
+        }
 #pragma unroll
-        for (int r = 0; r < OpB::CHUNKS; r++) b.reg[r] = *(const d2_t*)(pb[r] + (size_t)kb * b_step);
+        for (int r = 0; r < OpB::CHUNKS; r++) {
+            const bool ok = !KTAIL || (kb * BK + kbo[r] < K);
+            const d2_t v = *(const d2_t*)(pb[r] + (size_t)(ok ? kb : 0) * b_step);
+            b.reg[r] = ok ? v : (d2_t){0.0, 0.0};
+        }
     };
 
     d4_t acc[4][4];
@@ -338,7 +372,7 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
                 acc[t][u] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[W][t], bf[W][u], acc[t][u], 0, 0, 0);
     };
 
-    const int nkb = K / BK;
+    const int nkb = (K + BK - 1) / BK;
     gload(0);
     a.sstore(As, tid);
     b.sstore(Bs, tid);
@@ -402,28 +436,34 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 const int row = m0 + wm * 64 + t * 16 + 4 * r + lg;
-                C[(size_t)row * N + col] = acc[t][u][r];
+                if (row < M && col < N) C[(size_t)row * N + col] = acc[t][u][r];
             }
         }
 }
 
-template <bool TA, bool TB>
-int launch_fast(const double* A, const double* B, double* C, int M, int N, int K, int batch, hipStream_t st) {
+template <bool TA, bool TB, bool KTAIL>
+int launch_fast_k(const double* A, const double* B, double* C, int M, int N, int K, int batch, hipStream_t st) {
     constexpr int SMEM_BYTES = 2 * (Operand<128, TA, true, true>::TILE + Operand<128, !TB, true, true>::TILE)
                                * (int)sizeof(double);
     static bool attr_set = false;
-    auto kern = dgemm_fast_kernel<TA, TB>;
+    auto kern = dgemm_fast_kernel<TA, TB, KTAIL>;
     if (!attr_set) {
         if (!ESHKOL_HIP_OK(hipFuncSetAttribute((const void*)kern,
                 hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES))) return -1;
         attr_set = true;
     }
-    const int tiles_m = M / 128, tiles_n = N / 128;
+    const int tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
     const long long nwg = (long long)tiles_m * tiles_n;
     if (nwg > 0x7fffffffLL || batch < 1 || batch > 65535) return -1;
     hipLaunchKernelGGL(kern, dim3((unsigned)nwg, (unsigned)batch), dim3(256), SMEM_BYTES, st,
                        A, B, C, M, N, K, tiles_m, tiles_n);
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
+template <bool TA, bool TB>
+int launch_fast(const double* A, const double* B, double* C, int M, int N, int K, int batch, hipStream_t st) {
+    return (K % BK == 0) ? launch_fast_k<TA, TB, false>(A, B, C, M, N, K, batch, st)
+                         : launch_fast_k<TA, TB, true>(A, B, C, M, N, K, batch, st);
 }
 
 int g_fast_path = 1;
@@ -456,7 +496,8 @@ int launch_shape(const double* A, const double* B, double* C, int m, int n, int 
      * operands are read the same way) measured 1 % faster than keeping A's rows
      * at 8192^3; with both operands row-major the natural forms are faster. */
     constexpr bool ALK = TA || !TB;
-    if (g_fast_path && big_tiles >= 256 && vec && m % 128 == 0 && n % 128 == 0 && k % BK == 0)
+    /* 16-byte operand chunks (even pitches, aligned bases) and at least one whole k-block */
+    if (g_fast_path && big_tiles >= 256 && vec && m >= 2 && n >= 2 && k >= BK)
         return launch_fast<TA, TB>(A, B, C, m, n, k, batch, st);
     if (big_tiles >= 256) {
         return vec ? launch<128, 128, true, TA, TB, ALK, !TB>(A, B, C, m, n, k, batch, st)

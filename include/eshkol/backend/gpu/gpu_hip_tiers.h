@@ -260,8 +260,9 @@ int hip_matmul_backward_f64(const double* grad_out, const double* A, const doubl
 int hip_probe_peak(int kind, int random_operands, double* rate, void* stream);
 
 /* 0 sends every fp64 product through the bounds-checked kernel; 1 (default)
- * lets shapes with M, N multiples of 128 and K a multiple of 16 take the
- * straight-line kernel. Both give the same bits; the switch exists to compare them. */
+ * lets launches of at least 256 tiles with even row pitches, 16-byte aligned
+ * operands and K >= 16 take the straight-line kernel. Both give the same bits;
+ * the switch exists to compare them. */
 void hip_dgemm_set_fast_path(int on);
 
 /* k-blocks kept in flight by the pipelined int8 kernel (1..3; 0 = simple kernel only). */

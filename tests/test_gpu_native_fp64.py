@@ -86,10 +86,14 @@ def test_full_size_properties(gpu, M, K, N):
     assert normwise(Cg[rows][:, cols], ref, A[rows], B[:, cols]) <= TOL
 
 
-@pytest.mark.parametrize("M,K,N", [(2048, 16, 2048), (2048, 48, 2048), (2048, 1024, 2048), (4096, 2064, 1024), (1024, 512, 4096)])
+@pytest.mark.parametrize("M,K,N", [(2048, 16, 2048), (2048, 48, 2048), (2048, 1024, 2048), (4096, 2064, 1024),
+                                   (1024, 512, 4096), (2050, 130, 2046), (2049, 1000, 2050), (3000, 72, 1500),
+                                   (1922, 4098, 2174), (2048, 18, 2048), (2176, 30, 1930)])
 def test_straight_line_kernel_matches_bounds_checked_kernel_bitwise(gpu, M, K, N):
-    """Interior shapes take a kernel without bounds checks: same tiles, same
-    summation order, so the same bits, for all three operand forms."""
+    """Large launches take a kernel without bounds checks (edge rows clamped,
+    k-tail zeroed): same tiles, same summation order, so the same bits as the
+    bounds-checked kernel, for all three operand forms. The output buffer is
+    pre-filled with NaN and framed by guard rows to catch stray stores."""
     import eshkol_amd as ea
     from gpu_util import stream
     lib = ea.load()
@@ -102,10 +106,14 @@ def test_straight_line_kernel_matches_bounds_checked_kernel_bitwise(gpu, M, K, N
         try:
             for fast in (0, 1):
                 lib.hip_dgemm_set_fast_path(fast)
-                dC = ea.DeviceArray.from_host(np.full((M, N), np.nan))
-                assert lib.hip_dgemm_f64_ex(dX.ptr, dY.ptr, dC.ptr, M, K, N, ta, tb, stream()) == 0
+                guard = np.full((M + 2, N), np.nan)
+                guard[0] = guard[-1] = 12345.0
+                dC = ea.DeviceArray.from_host(guard)
+                assert lib.hip_dgemm_f64_ex(dX.ptr, dY.ptr, dC.ptr + N * 8, M, K, N, ta, tb, stream()) == 0
                 ea.synchronize()
-                outs.append(dC.download())
+                got = dC.download()
+                assert np.all(got[0] == 12345.0) and np.all(got[-1] == 12345.0)
+                outs.append(got[1:-1])
         finally:
             lib.hip_dgemm_set_fast_path(1)
         assert np.array_equal(outs[0], outs[1]), (ta, tb)
