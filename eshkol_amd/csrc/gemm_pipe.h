@@ -221,5 +221,203 @@ __device__ __forceinline__ void run(int8_t* smem, const Source& src, int m0, int
     __syncthreads();            /* LDS is free for the epilogue */
 }
 
+/* ---- several tiles per workgroup ------------------------------------------------
+ * The same main loop for a workgroup that walks a list of output tiles. The
+ * stream of k-blocks is continuous across tiles: when the request cursor runs
+ * past the last block of a tile it moves on to the first blocks of the next
+ * one, so those loads are in flight while the tile's epilogue runs and the
+ * next tile starts with its operands already in registers. What a workgroup
+ * launch costs (dispatch, cold first loads, a drained pipe) is paid once. */
+struct Tile {
+    int m0, n0;                 /* first row of the A planes / of the B planes */
+    int tag;                    /* caller's: output plane */
+    const int32_t* a_idx;       /* plane indices of the tile's products (device memory) */
+    const int32_t* b_idx;
+    int npairs;                 /* >= 1 */
+};
+
+template <int TM, int TN> struct TilesCfg {
+    static constexpr int SMEM_MAIN = Cfg<TM, TN>::SMEM_MAIN + Cfg<TM, TN>::TABLE_BYTES;   /* two index tables */
+};
+
+/* next_tile(Tile&) -> bool hands out this workgroup's tiles in order;
+ * epilogue(acc, tile) consumes a finished accumulator (LDS is free for it). */
+template <class Op, int TM, int TN, int PF, class Next, class Epi>
+__device__ __forceinline__ void run_tiles(int8_t* smem, const Source& cm, Next next_tile, Epi epilogue) {
+    using C = Cfg<TM, TN>;
+    int8_t* As = smem;
+    int8_t* Bs = smem + 2 * C::A_TILE;
+    int32_t* table = (int32_t*)(smem + 2 * (C::A_TILE + C::B_TILE));      /* [2][2 * MAX_PAIRS] */
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int li = lane & 31, lh = lane >> 5;
+
+    Tile cur, nxt;
+    if (!next_tile(cur)) return;
+    int tab = 0;                                   /* table half that describes `cur` */
+    if (tid < cur.npairs) {
+        table[tid] = cur.a_idx[tid];
+        table[MAX_PAIRS + tid] = cur.b_idx[tid];
+    }
+    __syncthreads();
+
+    const int nkb_per = cm.ld / BKB;
+    const size_t g_off = (size_t)(tid >> 3) * cm.ld + (tid & 7) * 16;
+    const int s_off = (tid >> 3) * PITCH + (tid & 7) * 16;
+
+    /* request cursor */
+    const int8_t* a_t = cm.a_planes + (size_t)cur.m0 * cm.ld + g_off;
+    const int8_t* b_t = cm.b_planes + (size_t)cur.n0 * cm.ld + g_off;
+    int gl_t = 0, gl_j = 0, gl_np = cur.npairs, gl_tab = 0;
+    int v_ia = table[0], v_ib = table[MAX_PAIRS];
+    /* where the cursor goes after the current tile */
+    const int8_t* nx_a = a_t;
+    const int8_t* nx_b = b_t;
+    int nx_np = 1;
+    bool nx_has = false;
+
+    v4i_t ra[PF][C::A_CH], rb[PF][C::B_CH];
+    auto gload = [&](auto slot) {
+        constexpr int S = decltype(slot)::value;
+        const int ia = __builtin_amdgcn_readfirstlane(v_ia);
+        const int ib = __builtin_amdgcn_readfirstlane(v_ib);
+        const int8_t* ap = a_t + (size_t)ia * cm.a_plane_stride + (size_t)gl_j * BKB;
+        const int8_t* bp = b_t + (size_t)ib * cm.b_plane_stride + (size_t)gl_j * BKB;
+#pragma unroll
+        for (int r = 0; r < C::A_CH; r++) ra[S][r] = *(const v4i_t*)(ap + (size_t)(32 * r) * cm.ld);
+#pragma unroll
+        for (int r = 0; r < C::B_CH; r++) rb[S][r] = *(const v4i_t*)(bp + (size_t)(32 * r) * cm.ld);
+        /* advance: next k-block, next product, next tile; with no next tile the
+         * cursor stays on the last block (those requests are never consumed) */
+        const int nj = gl_j + 1;
+        const bool wrap = (nj == nkb_per);
+        const bool last = wrap && (gl_t + 1 == gl_np);
+        const bool hop = last && nx_has;
+        gl_j = hop ? 0 : (last ? gl_j : (wrap ? 0 : nj));
+        gl_t = hop ? 0 : ((wrap && !last) ? gl_t + 1 : gl_t);
+        a_t = hop ? nx_a : a_t;
+        b_t = hop ? nx_b : b_t;
+        gl_np = hop ? nx_np : gl_np;
+        gl_tab = hop ? (gl_tab ^ 1) : gl_tab;
+        v_ia = table[gl_tab * 2 * MAX_PAIRS + gl_t];
+        v_ib = table[gl_tab * 2 * MAX_PAIRS + MAX_PAIRS + gl_t];
+    };
+    auto sstore = [&](int buf, auto slot) {
+        constexpr int S = decltype(slot)::value;
+        int8_t* ad = As + buf * C::A_TILE + s_off;
+        int8_t* bd = Bs + buf * C::B_TILE + s_off;
+#pragma unroll
+        for (int r = 0; r < C::A_CH; r++) *(v4i_t*)(ad + 32 * r * PITCH) = ra[S][r];
+#pragma unroll
+        for (int r = 0; r < C::B_CH; r++) *(v4i_t*)(bd + 32 * r * PITCH) = rb[S][r];
+    };
+
+    v4i_t fa[2][TM], fb[2][TN];
+    const int a_frag_off = (wm * TM * 32 + li) * PITCH + lh * 16;
+    const int b_frag_off = (wn * TN * 32 + li) * PITCH + lh * 16;
+    typename Op::acc_t acc[TM][TN];
+    auto ldfrag = [&](int buf, int ks, auto which) {
+        constexpr int W = decltype(which)::value;
+        const int8_t* ab = As + buf * C::A_TILE + a_frag_off + ks * 32;
+        const int8_t* bb = Bs + buf * C::B_TILE + b_frag_off + ks * 32;
+#pragma unroll
+        for (int t = 0; t < TM; t++) fa[W][t] = *(const v4i_t*)(ab + t * 32 * PITCH);
+#pragma unroll
+        for (int u = 0; u < TN; u++) fb[W][u] = *(const v4i_t*)(bb + u * 32 * PITCH);
+    };
+    auto mfma_all = [&](auto which) {
+        constexpr int W = decltype(which)::value;
+#pragma unroll
+        for (int t = 0; t < TM; t++)
+#pragma unroll
+            for (int u = 0; u < TN; u++) Op::mfma(fb[W][u], fa[W][t], acc[t][u]);
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    constexpr int NM = TM * TN, NF = TM + TN;
+
+    /* the first tile's first PF blocks; later tiles find theirs already requested */
+    static_for<PF>([&](auto s) { gload(s); });
+
+    for (;;) {
+        /* learn the next tile and park its index table in the other half */
+        nx_has = next_tile(nxt);
+        if (nx_has) {
+            if (tid < nxt.npairs) {
+                table[(tab ^ 1) * 2 * MAX_PAIRS + tid] = nxt.a_idx[tid];
+                table[(tab ^ 1) * 2 * MAX_PAIRS + MAX_PAIRS + tid] = nxt.b_idx[tid];
+            }
+            nx_a = cm.a_planes + (size_t)nxt.m0 * cm.ld + g_off;
+            nx_b = cm.b_planes + (size_t)nxt.n0 * cm.ld + g_off;
+            nx_np = nxt.npairs;
+        }
+#pragma unroll
+        for (int t = 0; t < TM; t++)
+#pragma unroll
+            for (int u = 0; u < TN; u++) Op::zero(acc[t][u]);
+
+        const int nkb = cur.npairs * nkb_per;      /* even: the row pitch is a multiple of 2 * BKB */
+        sstore(0, I0{});
+        lds_barrier();                             /* also publishes the parked table */
+        ldfrag(0, 0, I0{});
+
+        for (int g0 = 0; g0 < nkb; g0 += PF) {
+            static_for<PF>([&](auto s) {
+                constexpr int S = decltype(s)::value;
+                const int cb = (g0 + S) & 1;
+
+                ldfrag(cb, 1, I1{});
+                gload(s);
+                mfma_all(I0{});
+#pragma unroll
+                for (int i = 0; i < NM; i++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    if (i < NF) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    if (i < C::A_CH + C::B_CH) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+
+                ldfrag(cb, 2, I0{});
+                sstore(cb ^ 1, std::integral_constant<int, (S + 1) % PF>{});
+                mfma_all(I1{});
+#pragma unroll
+                for (int i = 0; i < NM; i++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    if (i < NF) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    if (i < C::A_CH + C::B_CH) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+
+                ldfrag(cb, 3, I1{});
+                mfma_all(I0{});
+#pragma unroll
+                for (int i = 0; i < NM; i++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    if (i < NF) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                lds_barrier();
+
+                ldfrag(cb ^ 1, 0, I0{});
+                mfma_all(I1{});
+#pragma unroll
+                for (int i = 0; i < NM; i++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    if (i < NF) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        }
+        lds_barrier();                 /* every wave is done with the LDS tiles */
+        epilogue(acc, cur);
+        if (!nx_has) break;
+        lds_barrier();                 /* the epilogue's LDS staging has been read */
+        cur = nxt;
+        tab ^= 1;
+    }
+}
+
 }  // namespace pipe
 #endif

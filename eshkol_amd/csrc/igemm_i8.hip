@@ -43,12 +43,15 @@ struct I8Op {
     static __device__ __forceinline__ void mfma(const v4i_t& first, const v4i_t& second, v16i_t& acc) {
         acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(first, second, acc, 0, 0, 0);
     }
+    static __device__ __forceinline__ void zero(v16i_t& acc) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = 0;
+    }
 };
 
 /* workgroup -> (output plane, tile); false for the padding workgroups of an XCD */
-__device__ __forceinline__ bool map_workgroup(int tiles_m, int tiles_n, int n_out, int chunk,
+__device__ __forceinline__ bool map_workgroup(int wg, int tiles_m, int tiles_n, int n_out, int chunk,
                                               int* o, int* tm, int* tn) {
-    const int wg = blockIdx.x;
     const int xcd = wg & 7, seq = wg >> 3;
     const int per_plane = tiles_m * tiles_n;
     /* planes from last to first: in the slice tier later planes sum more products */
@@ -86,7 +89,8 @@ __device__ __forceinline__ void epilogue(const HipIgemmArgs& g, int o, int m0, i
         for (int t = 0; t < TM; t++) {
             const int row = m0 + wm * TM * 32 + t * 32 + li;
 #pragma unroll
-            for (int u = 0; u < TN; u++)
+            for (int u = 0; u < TN; u++) {
+                asm volatile("" : "+a"(acc[t][u]));      /* see mode 1 */
 #pragma unroll
                 for (int v = 0; v < 4; v++) {
                     const int col = n0 + wn * TN * 32 + u * 32 + 8 * v + 4 * lh;
@@ -102,45 +106,57 @@ __device__ __forceinline__ void epilogue(const HipIgemmArgs& g, int o, int m0, i
                                 if (col + e < (int)g.N) p[e] = acc[t][u][4 * v + e];
                         }
                     }
+                    /* one 4-register group at a time: without the fence the
+                     * scheduler reads all 256 accumulators out first and spills */
+                    __builtin_amdgcn_sched_barrier(0);
                 }
+            }
         }
         return;
     }
 
     /* mode 1: residues modulo p, staged through LDS.
-     * |sum| <= K * 128 * 128 < 2^31. Fold 2^14 into the modulus twice (the
-     * result is below 2^21 in magnitude, exact in fp32), then take the nearest
-     * multiple of p in fp32: x/p < 2^14 is known to within 1e-3 and, unless it is
-     * a tie, lies at least 1/(2p) >= 2e-3 from a half-integer, so q is the
-     * nearest integer and x - q p is exact and in [-p/2, p/2]; the tie (even p)
-     * is folded to -p/2. Every instruction is full rate, unlike the fp64
-     * conversions and the 32-bit multiply a direct reduction needs. */
+     * |sum| <= K * 128 * 128 <= 2^31. One fold of 2^20 into the modulus
+     * (sum = hi 2^20 + lo, hi 2^20 = hi c20 mod p) leaves |x| < 2^21, exact in
+     * fp32; then the nearest multiple of p in fp32: x/p < 2^14 is known to
+     * within 1e-3 and, unless it is a tie, lies at least 1/(2p) >= 2e-3 from a
+     * half-integer, so q is the nearest integer and x - q p is exact and in
+     * [-p/2, p/2]. The tie (p = 256, +128) and -128 are the same int8 byte.
+     * About nine full-rate instructions per element: the epilogue is VALU
+     * time the matrix pipe sits idle for, so it is kept short. */
     const int p = g.modulus[o];
-    const int c14 = 16384 % p;
+    const int c20 = (1 << 20) % p;
     const float pf = (float)p, pinv = 1.0f / (float)p;
     constexpr int EPITCH = BN + 16;
 #pragma unroll
     for (int t = 0; t < TM; t++) {
         const int lrow = wm * TM * 32 + t * 32 + li;
 #pragma unroll
-        for (int u = 0; u < TN; u++)
+        for (int u = 0; u < TN; u++) {
+            /* Keep this 16-register tile in the accumulator file until here.
+             * Otherwise the allocator copies all 256 accumulators into vector
+             * registers on entry and spills what does not fit. */
+            asm volatile("" : "+a"(acc[t][u]));
 #pragma unroll
             for (int v = 0; v < 4; v++) {
                 const int lcol = wn * TN * 32 + u * 32 + 8 * v + 4 * lh;
-                uint32_t packed = 0;
+                int r[4];
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     const int s = acc[t][u][4 * v + e];
-                    const int x1 = (s >> 14) * c14 + (s & 0x3fff);       /* |x1| < 2^26 */
-                    const int x2 = (x1 >> 14) * c14 + (x1 & 0x3fff);     /* |x2| < 2^21 */
-                    const float xf = (float)x2;
+                    const int x = __mul24(s >> 20, c20) + (s & 0xfffff);
+                    const float xf = (float)x;
                     const float q = rintf(xf * pinv);
-                    int r = (int)fmaf(-q, pf, xf);
-                    if (2 * r >= p) r -= p;
-                    packed |= ((uint32_t)(uint8_t)(int8_t)r) << (8 * e);
+                    r[e] = (int)fmaf(-q, pf, xf);
                 }
+                /* low bytes of r[0..3] into one word */
+                const uint32_t lo2 = __builtin_amdgcn_perm((uint32_t)r[1], (uint32_t)r[0], 0x0c0c0400u);
+                const uint32_t hi2 = __builtin_amdgcn_perm((uint32_t)r[3], (uint32_t)r[2], 0x04000c0cu);
+                const uint32_t packed = lo2 | hi2;
                 *(uint32_t*)(stage + lrow * EPITCH + lcol) = packed;
+                __builtin_amdgcn_sched_barrier(0);
             }
+        }
     }
     __syncthreads();
     int8_t* out = g.out_i8 + (size_t)o * g.M * g.N;
@@ -168,7 +184,7 @@ __global__ __launch_bounds__(256, 1)
 void igemm_i8_pipe_kernel(HipIgemmArgs g, int tiles_m, int tiles_n, int chunk) {
     extern __shared__ __align__(16) int8_t smem_i8[];
     int o, tm, tn;
-    if (!map_workgroup(tiles_m, tiles_n, (int)g.n_out, chunk, &o, &tm, &tn)) return;
+    if (!map_workgroup((int)blockIdx.x, tiles_m, tiles_n, (int)g.n_out, chunk, &o, &tm, &tn)) return;
     constexpr int BM = 2 * TM * 32, BN = 2 * TN * 32;
     const int m0 = tm * BM, n0 = tn * BN;
 
@@ -192,6 +208,44 @@ void igemm_i8_pipe_kernel(HipIgemmArgs g, int tiles_m, int tiles_n, int chunk) {
     epilogue<TM, TN>(g, o, m0, n0, acc, smem_i8);
 }
 
+/* ---- persistent pipelined kernel ------------------------------------------------
+ * One workgroup per CU walks the tile ids blockIdx.x, blockIdx.x + gridDim.x, ...
+ * (gridDim.x is a multiple of 8, so an id keeps the XCD the tile mapping meant
+ * for it). The operand stream runs on across tile boundaries (pipe::run_tiles). */
+template <int TM, int TN, int PF>
+__global__ __launch_bounds__(256, 1)
+void igemm_i8_persistent_kernel(HipIgemmArgs g, int tiles_m, int tiles_n, int chunk, int n_ids) {
+    extern __shared__ __align__(16) int8_t smem_i8[];
+    constexpr int BM = 2 * TM * 32, BN = 2 * TN * 32;
+    pipe::Source cm;
+    cm.a_planes = g.a_planes; cm.b_planes = g.b_planes;
+    cm.a_plane_stride = g.a_plane_stride; cm.b_plane_stride = g.b_plane_stride;
+    cm.a_idx = nullptr; cm.b_idx = nullptr; cm.npairs = 0;
+    cm.ld = (int)g.ldk;
+
+    int next_id = (int)blockIdx.x;
+    auto next_tile = [&](pipe::Tile& t) -> bool {
+        while (next_id < n_ids) {
+            int o, tm, tn;
+            const bool real = map_workgroup(next_id, tiles_m, tiles_n, (int)g.n_out, chunk, &o, &tm, &tn);
+            next_id += (int)gridDim.x;
+            if (!real) continue;
+            const int pair_lo = g.pair_first[o];
+            t.m0 = tm * BM; t.n0 = tn * BN; t.tag = o;
+            t.a_idx = g.pair_a + pair_lo; t.b_idx = g.pair_b + pair_lo;
+            t.npairs = g.pair_first[o + 1] - pair_lo;
+            /* the caller promises every output plane at least one product
+             * (max_pairs >= 1 selects this kernel); an empty one is skipped */
+            if (t.npairs > 0) return true;
+        }
+        return false;
+    };
+    auto epi = [&](v16i_t (&acc)[TM][TN], const pipe::Tile& t) {
+        epilogue<TM, TN>(g, t.tag, t.m0, t.n0, acc, smem_i8);
+    };
+    pipe::run_tiles<I8Op, TM, TN, PF>(smem_i8, cm, next_tile, epi);
+}
+
 /* ---- simple kernel --------------------------------------------------------- */
 
 constexpr int SBK = 64;
@@ -208,7 +262,7 @@ void igemm_i8_simple_kernel(HipIgemmArgs g, int tiles_m, int tiles_n, int chunk)
     int8_t* Bs = smem_i8 + 2 * A_TILE;
 
     int o, tm, tn;
-    if (!map_workgroup(tiles_m, tiles_n, (int)g.n_out, chunk, &o, &tm, &tn)) return;
+    if (!map_workgroup((int)blockIdx.x, tiles_m, tiles_n, (int)g.n_out, chunk, &o, &tm, &tn)) return;
     const int m0 = tm * BM, n0 = tn * BN;
 
     const int tid = threadIdx.x;
@@ -286,6 +340,7 @@ void igemm_i8_simple_kernel(HipIgemmArgs g, int tiles_m, int tiles_n, int chunk)
 }
 
 int g_prefetch = 2;     /* blocks in flight in the pipelined kernel */
+int g_persistent = 1;   /* pipelined kernel as one workgroup per CU walking a tile list */
 
 template <class K>
 int launch_kernel(K kern, int smem, bool* attr_set, const HipIgemmArgs& a, int BM, int BN, hipStream_t st) {
@@ -311,6 +366,35 @@ int launch_pipe(const HipIgemmArgs& a, hipStream_t st) {
     return launch_kernel(igemm_i8_pipe_kernel<4, 4, PF>, SMEM, &attr_set, a, C::BM, C::BN, st);
 }
 
+template <int PF>
+int launch_persistent(const HipIgemmArgs& a, hipStream_t st) {
+    using C = pipe::Cfg<4, 4>;
+    constexpr int EPI = C::BM * (C::BN + 16);
+    constexpr int MAIN = pipe::TilesCfg<4, 4>::SMEM_MAIN;
+    constexpr int SMEM = MAIN > EPI ? MAIN : EPI;
+    static bool attr_set = false;
+    static int num_cus = 0;
+    auto kern = igemm_i8_persistent_kernel<4, 4, PF>;
+    if (!attr_set) {
+        if (!ESHKOL_HIP_OK(hipFuncSetAttribute((const void*)kern,
+                hipFuncAttributeMaxDynamicSharedMemorySize, SMEM))) return -1;
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (!ESHKOL_HIP_OK(hipGetDevice(&dev)) || !ESHKOL_HIP_OK(hipGetDeviceProperties(&prop, dev))) return -1;
+        num_cus = prop.multiProcessorCount;
+        attr_set = true;
+    }
+    const int tiles_m = (int)((a.M + C::BM - 1) / C::BM), tiles_n = (int)((a.N + C::BN - 1) / C::BN);
+    const int chunk = (tiles_m * tiles_n + 7) / 8;
+    const long long n_ids = 8LL * chunk * a.n_out;
+    if (n_ids > 0x7fffffffLL || n_ids <= 0) return -1;
+    long long grid = (num_cus / 8) * 8;             /* one workgroup per CU, a multiple of the XCD count */
+    if (grid < 8) grid = 8;
+    if (grid > n_ids) grid = n_ids;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), SMEM, st, a, tiles_m, tiles_n, chunk, (int)n_ids);
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
 int launch_simple(const HipIgemmArgs& a, hipStream_t st) {
     constexpr int BM = 128, BN = 128;
     constexpr int MAIN = 2 * (BM + BN) * SPITCH, EPI = BM * (BN + 16);
@@ -323,6 +407,9 @@ int launch_simple(const HipIgemmArgs& a, hipStream_t st) {
 
 /* Tuning hook: k-blocks in flight in the pipelined kernel (1..3), 0 = simple kernel only. */
 extern "C" void hip_igemm_set_prefetch(int pf) { if (pf >= 0 && pf <= 3) g_prefetch = pf; }
+/* Tuning hook: 1 (default) runs the pipelined kernel as one workgroup per CU
+ * walking a list of tiles, 0 as one workgroup per tile. Same results. */
+extern "C" void hip_igemm_set_persistent(int on) { g_persistent = on ? 1 : 0; }
 
 extern "C" int hip_igemm_i8(const HipIgemmArgs* args, void* stream) {
     if (!args || !args->a_planes || !args->b_planes || !args->pair_first || !args->pair_a || !args->pair_b)
@@ -343,6 +430,13 @@ extern "C" int hip_igemm_i8(const HipIgemmArgs* args, void* stream) {
     int pf = g_prefetch;
     while (pf > 0 && a.ldk % (128u * pf) != 0) pf--;
     if (pf > 0 && big >= 128 && a.max_pairs >= 1 && a.max_pairs <= pipe::MAX_PAIRS) {
+        if (g_persistent) {
+            switch (pf) {
+                case 1: return launch_persistent<1>(a, st);
+                case 2: return launch_persistent<2>(a, st);
+                default: return launch_persistent<3>(a, st);
+            }
+        }
         switch (pf) {
             case 1: return launch_pipe<1>(a, st);
             case 2: return launch_pipe<2>(a, st);

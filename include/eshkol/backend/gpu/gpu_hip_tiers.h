@@ -94,8 +94,9 @@ int hip_bias_act_f64(double* Y, const double* bias, uint64_t rows, uint64_t cols
  * (metal_softfloat.h:3907-4100). Operand planes are K-contiguous int8 with a
  * row pitch of ldk bytes (multiple of 128, zero padded beyond K) and row counts
  * padded with zero rows to multiples of 256. The pipelined kernel needs ldk to
- * be a multiple of 256 and 1 <= max_pairs <= 64; other plans take the simple
- * kernel. */
+ * be a multiple of 256, 1 <= max_pairs <= 64 and every output plane to have at
+ * least one product (pair_first strictly increasing); pass max_pairs = 0 for
+ * plans with empty planes: they take the simple kernel, which writes zeros. */
 typedef struct {
     const int8_t* a_planes;   /* [n_a_planes][rows_a_padded][ldk]                */
     const int8_t* b_planes;   /* [n_b_planes][rows_b_padded][ldk]                */
@@ -267,6 +268,11 @@ void hip_dgemm_set_fast_path(int on);
 
 /* k-blocks kept in flight by the pipelined int8 kernel (1..3; 0 = simple kernel only). */
 void hip_igemm_set_prefetch(int pf);
+
+/* 1 (default): the pipelined int8 kernel runs as one workgroup per CU walking a
+ * list of tiles, its operand stream continuous across tile boundaries; 0: one
+ * workgroup per tile. Same results; the switch exists to compare them. */
+void hip_igemm_set_persistent(int on);
 
 #ifdef __cplusplus
 }
