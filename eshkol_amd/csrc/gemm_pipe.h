@@ -227,7 +227,9 @@ __device__ __forceinline__ void run(int8_t* smem, const Source& src, int m0, int
  * past the last block of a tile it moves on to the first blocks of the next
  * one, so those loads are in flight while the tile's epilogue runs and the
  * next tile starts with its operands already in registers. What a workgroup
- * launch costs (dispatch, cold first loads, a drained pipe) is paid once. */
+ * launch costs (dispatch, cold first loads, a drained pipe) is paid once.
+ * Every tile must have at least 2 * PF k-blocks: the cursor runs PF blocks
+ * ahead and learns about the tile after the next only when it gets there. */
 struct Tile {
     int m0, n0;                 /* first row of the A planes / of the B planes */
     int tag;                    /* caller's: output plane */

@@ -430,7 +430,9 @@ extern "C" int hip_igemm_i8(const HipIgemmArgs* args, void* stream) {
     int pf = g_prefetch;
     while (pf > 0 && a.ldk % (128u * pf) != 0) pf--;
     if (pf > 0 && big >= 128 && a.max_pairs >= 1 && a.max_pairs <= pipe::MAX_PAIRS) {
-        if (g_persistent) {
+        /* the persistent kernel's request cursor may not reach the end of a tile
+         * before the tile after it is known: more than PF blocks per tile */
+        if (g_persistent && a.ldk >= 256u * pf) {
             switch (pf) {
                 case 1: return launch_persistent<1>(a, st);
                 case 2: return launch_persistent<2>(a, st);

@@ -1,0 +1,125 @@
+"""The int8 matrix-core contraction on its own (hip_igemm_i8), against exact
+integer arithmetic in numpy, for each of its kernels: the simple one, the
+pipelined one (a workgroup per tile) and the persistent one (a workgroup per
+CU walking a tile list). All three must give the same bits: int32 sums for
+the slice tier's plans, symmetric residues for the CRT tier's."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import eshkol_amd as ea
+from gpu_util import stream
+
+pytestmark = pytest.mark.gpu
+
+MODULI = [256, 255, 253, 251, 247, 241, 239, 233, 229, 227, 223, 217, 211, 199, 197, 193]
+KERNELS = {"simple": (0, 0), "pipelined": (2, 0), "persistent": (2, 1), "pipelined-1": (1, 0), "persistent-1": (1, 1)}
+
+
+def pad(n, m):
+    return (n + m - 1) // m * m
+
+
+def planes(rng, n_planes, rows, K, lo=-128, hi=128):
+    """[n_planes][rows padded to 256][K padded to 256] int8, padding zero."""
+    out = np.zeros((n_planes, pad(rows, 256), pad(K, 256)), np.int8)
+    out[:, :rows, :K] = rng.integers(lo, hi, (n_planes, rows, K), dtype=np.int8)
+    return out
+
+
+def run(a, b, M, N, plan, mode, kernel):
+    """plan: list of lists of (a_plane, b_plane) per output plane."""
+    lib = ea.load()
+    pf, pers = KERNELS[kernel]
+    first = np.cumsum([0] + [len(p) for p in plan]).astype(np.int32)
+    pa = np.array([t[0] for p in plan for t in p], np.int32)
+    pb = np.array([t[1] for p in plan for t in p], np.int32)
+    dA, dB = ea.DeviceArray.from_host(a), ea.DeviceArray.from_host(b)
+    dF, dPa, dPb = (ea.DeviceArray.from_host(x) for x in (first, pa, pb))
+    dMod = ea.DeviceArray.from_host(np.array(MODULI[:len(plan)] if mode == 1 else [1], np.int32))
+    n_out = len(plan)
+    out = ea.DeviceArray.from_host(np.full((n_out, M, N), 0x55, np.int8 if mode == 1 else np.int32))
+    g = ea.HipIgemmArgs()
+    g.a_planes, g.b_planes = dA.ptr, dB.ptr
+    g.a_plane_stride, g.b_plane_stride = a.shape[1] * a.shape[2], b.shape[1] * b.shape[2]
+    g.ldk, g.M, g.N, g.n_out = a.shape[2], M, N, n_out
+    g.pair_first, g.pair_a, g.pair_b = dF.ptr, dPa.ptr, dPb.ptr
+    g.mode, g.max_pairs, g.modulus = mode, max(len(p) for p in plan), dMod.ptr
+    if mode == 1:
+        g.out_i8 = out.ptr
+    else:
+        g.out_i32 = out.ptr
+    lib.hip_igemm_set_prefetch(pf)
+    lib.hip_igemm_set_persistent(pers)
+    try:
+        assert lib.hip_igemm_i8(C.byref(g), stream()) == 0
+        ea.synchronize()
+    finally:
+        lib.hip_igemm_set_prefetch(2)
+        lib.hip_igemm_set_persistent(1)
+    return out.download()
+
+
+def exact(a, b, M, N, K, plan):
+    """Sums of int8 products are integers far below 2^53: a float64 GEMM computes them exactly."""
+    af, bf = a[:, :M, :K].astype(np.float64), b[:, :N, :K].astype(np.float64)
+    return np.stack([sum(af[i] @ bf[j].T for i, j in p) for p in plan]).astype(np.int64)
+
+
+def symmetric(v, p):
+    r = np.mod(v, p)
+    return np.where(2 * r >= p, r - p, r)
+
+
+@pytest.mark.parametrize("kernel", list(KERNELS))
+@pytest.mark.parametrize("M,K,N", [(1024, 1024, 1024), (1000, 700, 1300), (2048, 256, 1024), (1536, 1000, 1792)])
+def test_residue_products(gpu, M, K, N, kernel):
+    rng = np.random.default_rng(M + K)
+    a, b = planes(rng, 16, M, K), planes(rng, 16, N, K)
+    plan = [[(l, l)] for l in range(16)]
+    got = run(a, b, M, N, plan, 1, kernel)
+    want = exact(a, b, M, N, K, plan)
+    for l, p in enumerate(MODULI):
+        assert np.array_equal(got[l].astype(np.int64), symmetric(want[l], p)), (l, p)
+
+
+@pytest.mark.parametrize("kernel", list(KERNELS))
+def test_residues_at_the_extremes_of_the_accumulator(gpu, kernel):
+    """All operands -128 (sums up to +K 2^14) and mixed signs (down to -K 127 128):
+    the reduction must stay exact at both ends of the int32 range it is specified for."""
+    M = N = 1024
+    for K in (8192, 131072 - 256):
+        a = np.full((16, M, pad(K, 256)), -128, np.int8)
+        b = np.full((16, N, pad(K, 256)), -128, np.int8)
+        a[:, :, K:] = 0
+        b[:, 1::2, :] = 127
+        b[:, :, K:] = 0
+        if K > 8192:                      # keep the large case cheap: eight planes still fill the chip
+            a, b = a[:8], b[:8]
+        plan = [[(l, l)] for l in range(a.shape[0])]
+        got = run(a, b, M, N, plan, 1, kernel)
+        for l in range(a.shape[0]):
+            p = MODULI[l]
+            even, odd = K * 128 * 128, -K * 128 * 127
+            assert np.all(got[l][:, 0::2] == symmetric(np.int64(even), p)), (K, l)
+            assert np.all(got[l][:, 1::2] == symmetric(np.int64(odd), p)), (K, l)
+
+
+@pytest.mark.parametrize("kernel", list(KERNELS))
+@pytest.mark.parametrize("M,K,N,s", [(1024, 512, 1024, 7), (900, 300, 1100, 5), (2048, 256, 2048, 3), (2048, 512, 2048, 5),
+                                     (1800, 1100, 2300, 7)])
+def test_slice_diagonal_sums(gpu, M, K, N, s, kernel):
+    """The slice tier's plan: output d sums the products (p, d - p); several products per output."""
+    rng = np.random.default_rng(s * M)
+    a, b = planes(rng, s, M, K, -127, 128), planes(rng, s, N, K, -127, 128)
+    plan = [[(p, d - p) for p in range(s) if 0 <= d - p < s] for d in range(s)]
+    got = run(a, b, M, N, plan, 0, kernel)
+    assert np.array_equal(got.astype(np.int64), exact(a, b, M, N, K, plan))
+
+
+def test_bad_arguments(gpu):
+    lib = ea.load()
+    g = ea.HipIgemmArgs()
+    assert lib.hip_igemm_i8(C.byref(g), stream()) == -1
+    assert lib.hip_igemm_i8(None, stream()) == -1
