@@ -225,7 +225,11 @@ void hgemm_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
         const int row = m0 + wm * TM * 32 + t * 32 + li;
         if (row >= M) continue;
 #pragma unroll
-        for (int u = 0; u < TN; u++)
+        for (int u = 0; u < TN; u++) {
+            /* With 256 accumulator registers, keep each 16-register tile in the
+             * accumulator file until it is stored: otherwise the allocator copies
+             * all of them into vector registers on entry and spills. */
+            if constexpr (TM * TN >= 16) asm volatile("" : "+a"(acc[t][u]));
 #pragma unroll
             for (int v = 0; v < 4; v++) {
                 const int col = n0 + wn * TN * 32 + u * 32 + 8 * v + 4 * lh;
@@ -251,6 +255,7 @@ void hgemm_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
                     }
                 }
             }
+        }
     }
 }
 
@@ -286,7 +291,11 @@ __device__ __forceinline__ void store_tile(v16f_t (&acc)[TM][TN], int m0, int n0
         const int row = m0 + wm * TM * 32 + t * 32 + li;
         if (row >= M) continue;
 #pragma unroll
-        for (int u = 0; u < TN; u++)
+        for (int u = 0; u < TN; u++) {
+            /* With 256 accumulator registers, keep each 16-register tile in the
+             * accumulator file until it is stored: otherwise the allocator copies
+             * all of them into vector registers on entry and spills. */
+            if constexpr (TM * TN >= 16) asm volatile("" : "+a"(acc[t][u]));
 #pragma unroll
             for (int v = 0; v < 4; v++) {
                 const int col = n0 + wn * TN * 32 + u * 32 + 8 * v + 4 * lh;
@@ -311,6 +320,7 @@ __device__ __forceinline__ void store_tile(v16f_t (&acc)[TM][TN], int m0, int n0
                     }
                 }
             }
+        }
     }
 }
 
