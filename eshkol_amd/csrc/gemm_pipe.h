@@ -21,8 +21,8 @@
  *              full __syncthreads would also wait for the prefetched global
  *              loads and undo the ring
  *
- * The loop body is branch-free (prefetches past the end are clamped to the last
- * block and never consumed), so it is one scheduling region.
+ * The loop body is branch-free (prefetches past the end of the last tile are
+ * clamped to its last block and never consumed), so it is one scheduling region.
  */
 #ifndef ESHKOL_HIP_GEMM_PIPE_H
 #define ESHKOL_HIP_GEMM_PIPE_H
@@ -64,162 +64,13 @@ __device__ __forceinline__ void lds_barrier() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-/* What one output tile multiplies: for product t of the tile, operand planes
- * a_idx[t], b_idx[t]; every plane is [rows][ld] bytes. */
+/* The operand planes a launch multiplies: every plane is [rows][ld] bytes. */
 struct Source {
     const int8_t* a_planes;
     const int8_t* b_planes;
     uint64_t a_plane_stride, b_plane_stride;
-    const int32_t* a_idx;       /* device arrays, npairs entries, or NULL for plane 0 */
-    const int32_t* b_idx;
-    int npairs;
     int ld;                     /* bytes per row, multiple of BKB*PF */
 };
-
-/* Op::acc_t accumulator of one 32x32 tile, Op::mfma(first, second, acc). */
-template <class Op, int TM, int TN, int PF>
-__device__ __forceinline__ void run(int8_t* smem, const Source& src, int m0, int n0,
-                                    typename Op::acc_t (&acc)[TM][TN]) {
-    using C = Cfg<TM, TN>;
-    int8_t* As = smem;
-    int8_t* Bs = smem + 2 * C::A_TILE;
-    int32_t* table = (int32_t*)(smem + 2 * (C::A_TILE + C::B_TILE));
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
-    const int li = lane & 31, lh = lane >> 5;
-
-    if (tid < src.npairs) {
-        table[tid] = src.a_idx ? src.a_idx[tid] : 0;
-        table[MAX_PAIRS + tid] = src.b_idx ? src.b_idx[tid] : 0;
-    }
-    __syncthreads();
-
-    const int nkb_per = src.ld / BKB;
-    const int nkb = src.npairs * nkb_per;
-
-    /* this thread's chunk: row tid/8 (+32 per chunk index), 16 bytes at (tid%8)*16 */
-    const size_t g_off = (size_t)(tid >> 3) * src.ld + (tid & 7) * 16;
-    const int s_off = (tid >> 3) * PITCH + (tid & 7) * 16;
-    const int8_t* a_tile0 = src.a_planes + (size_t)m0 * src.ld + g_off;
-    const int8_t* b_tile0 = src.b_planes + (size_t)n0 * src.ld + g_off;
-
-    v4i_t ra[PF][C::A_CH], rb[PF][C::B_CH];
-    int gl_t = 0, gl_j = 0;            /* next block to request: product gl_t, k-block gl_j */
-    int v_ia = table[0], v_ib = table[MAX_PAIRS];   /* its plane indices, read one block ahead */
-
-    auto gload = [&](auto slot) {
-        constexpr int S = decltype(slot)::value;
-        const int ia = __builtin_amdgcn_readfirstlane(v_ia);
-        const int ib = __builtin_amdgcn_readfirstlane(v_ib);
-        const int8_t* ap = a_tile0 + (size_t)ia * src.a_plane_stride + (size_t)gl_j * BKB;
-        const int8_t* bp = b_tile0 + (size_t)ib * src.b_plane_stride + (size_t)gl_j * BKB;
-#pragma unroll
-        for (int r = 0; r < C::A_CH; r++) ra[S][r] = *(const v4i_t*)(ap + (size_t)(32 * r) * src.ld);
-#pragma unroll
-        for (int r = 0; r < C::B_CH; r++) rb[S][r] = *(const v4i_t*)(bp + (size_t)(32 * r) * src.ld);
-        /* advance, clamped to the last block (requests past the end are never consumed) */
-        const int nj = gl_j + 1;
-        const bool wrap = (nj == nkb_per);
-        const bool last = wrap && (gl_t + 1 == src.npairs);
-        gl_j = last ? gl_j : (wrap ? 0 : nj);
-        gl_t = (wrap && !last) ? gl_t + 1 : gl_t;
-        v_ia = table[gl_t];
-        v_ib = table[MAX_PAIRS + gl_t];
-    };
-    auto sstore = [&](int buf, auto slot) {
-        constexpr int S = decltype(slot)::value;
-        int8_t* ad = As + buf * C::A_TILE + s_off;
-        int8_t* bd = Bs + buf * C::B_TILE + s_off;
-#pragma unroll
-        for (int r = 0; r < C::A_CH; r++) *(v4i_t*)(ad + 32 * r * PITCH) = ra[S][r];
-#pragma unroll
-        for (int r = 0; r < C::B_CH; r++) *(v4i_t*)(bd + 32 * r * PITCH) = rb[S][r];
-    };
-
-    v4i_t fa[2][TM], fb[2][TN];
-    const int a_frag_off = (wm * TM * 32 + li) * PITCH + lh * 16;
-    const int b_frag_off = (wn * TN * 32 + li) * PITCH + lh * 16;
-    auto ldfrag = [&](int buf, int ks, auto which) {
-        constexpr int W = decltype(which)::value;
-        const int8_t* ab = As + buf * C::A_TILE + a_frag_off + ks * 32;
-        const int8_t* bb = Bs + buf * C::B_TILE + b_frag_off + ks * 32;
-#pragma unroll
-        for (int t = 0; t < TM; t++) fa[W][t] = *(const v4i_t*)(ab + t * 32 * PITCH);
-#pragma unroll
-        for (int u = 0; u < TN; u++) fb[W][u] = *(const v4i_t*)(bb + u * 32 * PITCH);
-    };
-    auto mfma_all = [&](auto which) {
-        constexpr int W = decltype(which)::value;
-#pragma unroll
-        for (int t = 0; t < TM; t++)
-#pragma unroll
-            for (int u = 0; u < TN; u++) Op::mfma(fb[W][u], fa[W][t], acc[t][u]);
-    };
-    using I0 = std::integral_constant<int, 0>;
-    using I1 = std::integral_constant<int, 1>;
-    constexpr int NM = TM * TN, NF = TM + TN;
-
-    /* prologue: PF blocks requested, block 0 in LDS buffer 0, its first fragments loaded */
-    static_for<PF>([&](auto s) { gload(s); });
-    sstore(0, I0{});
-    lds_barrier();
-    ldfrag(0, 0, I0{});
-
-    for (int g0 = 0; g0 < nkb; g0 += PF) {
-        static_for<PF>([&](auto s) {
-            constexpr int S = decltype(s)::value;
-            const int cur = (g0 + S) & 1;
-
-            /* k-step 0: request block g+PF into the slot block g has vacated */
-            ldfrag(cur, 1, I1{});
-            gload(s);
-            mfma_all(I0{});
-#pragma unroll
-            for (int i = 0; i < NM; i++) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                if (i < NF) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                if (i < C::A_CH + C::B_CH) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-
-            /* k-step 1: block g+1 goes to the other LDS buffer */
-            ldfrag(cur, 2, I0{});
-            sstore(cur ^ 1, std::integral_constant<int, (S + 1) % PF>{});
-            mfma_all(I1{});
-#pragma unroll
-            for (int i = 0; i < NM; i++) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                if (i < NF) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                if (i < C::A_CH + C::B_CH) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-
-            /* k-step 2 */
-            ldfrag(cur, 3, I1{});
-            mfma_all(I0{});
-#pragma unroll
-            for (int i = 0; i < NM; i++) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                if (i < NF) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            lds_barrier();      /* block g+1 visible; every read of block g has completed */
-
-            /* k-step 3, with the first fragments of block g+1 */
-            ldfrag(cur ^ 1, 0, I0{});
-            mfma_all(I1{});
-#pragma unroll
-            for (int i = 0; i < NM; i++) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                if (i < NF) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        });
-    }
-    __syncthreads();            /* LDS is free for the epilogue */
-}
 
 /* ---- several tiles per workgroup ------------------------------------------------
  * The same main loop for a workgroup that walks a list of output tiles. The
@@ -233,7 +84,7 @@ __device__ __forceinline__ void run(int8_t* smem, const Source& src, int m0, int
 struct Tile {
     int m0, n0;                 /* first row of the A planes / of the B planes */
     int tag;                    /* caller's: output plane */
-    const int32_t* a_idx;       /* plane indices of the tile's products (device memory) */
+    const int32_t* a_idx;       /* plane indices of the tile's products (device memory), or NULL for plane 0 */
     const int32_t* b_idx;
     int npairs;                 /* >= 1 */
 };
@@ -260,8 +111,8 @@ __device__ __forceinline__ void run_tiles(int8_t* smem, const Source& cm, Next n
     if (!next_tile(cur)) return;
     int tab = 0;                                   /* table half that describes `cur` */
     if (tid < cur.npairs) {
-        table[tid] = cur.a_idx[tid];
-        table[MAX_PAIRS + tid] = cur.b_idx[tid];
+        table[tid] = cur.a_idx ? cur.a_idx[tid] : 0;
+        table[MAX_PAIRS + tid] = cur.b_idx ? cur.b_idx[tid] : 0;
     }
     __syncthreads();
 
@@ -348,8 +199,8 @@ __device__ __forceinline__ void run_tiles(int8_t* smem, const Source& cm, Next n
         nx_has = next_tile(nxt);
         if (nx_has) {
             if (tid < nxt.npairs) {
-                table[(tab ^ 1) * 2 * MAX_PAIRS + tid] = nxt.a_idx[tid];
-                table[(tab ^ 1) * 2 * MAX_PAIRS + MAX_PAIRS + tid] = nxt.b_idx[tid];
+                table[(tab ^ 1) * 2 * MAX_PAIRS + tid] = nxt.a_idx ? nxt.a_idx[tid] : 0;
+                table[(tab ^ 1) * 2 * MAX_PAIRS + MAX_PAIRS + tid] = nxt.b_idx ? nxt.b_idx[tid] : 0;
             }
             nx_a = cm.a_planes + (size_t)nxt.m0 * cm.ld + g_off;
             nx_b = cm.b_planes + (size_t)nxt.n0 * cm.ld + g_off;

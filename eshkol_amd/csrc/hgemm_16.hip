@@ -271,6 +271,10 @@ template <bool BF16> struct H16Op {
             acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h_t, first),
                                                          __builtin_bit_cast(v8h_t, second), acc, 0, 0, 0);
     }
+    static __device__ __forceinline__ void zero(v16f_t& acc) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+    }
 };
 
 template <bool BF16>
@@ -324,59 +328,73 @@ __device__ __forceinline__ void store_tile(v16f_t (&acc)[TM][TN], int m0, int n0
     }
 }
 
+/* One workgroup per CU walks the tile ids blockIdx.x, blockIdx.x + gridDim.x, ...
+ * (gridDim.x is a multiple of 8, so an id stays on its XCD); ids are laid out so
+ * that each XCD owns a contiguous run of tiles, 8 tile-rows at a time. The
+ * operand stream runs on across tile boundaries (pipe::run_tiles). */
 template <bool BF16, int PF>
 __global__ __launch_bounds__(256, 1)
 void hgemm_pipe_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ Bt,
                        int M, int N, int ld_bytes, int out_mode, void* __restrict__ Cout,
-                       int tiles_m, int tiles_n) {
+                       int tiles_m, int tiles_n, int n_ids) {
     extern __shared__ __align__(16) int8_t smem_h[];
-    int tm, tn;
-    {
-        const int nwg = gridDim.x, wg = blockIdx.x;
-        const int q = nwg >> 3, r = nwg & 7;
-        const int xcd = wg & 7, seq = wg >> 3;
-        const int L = xcd * q + (xcd < r ? xcd : r) + seq;
-        const int GM = 8;
-        const int width = GM * tiles_n;
-        const int group = L / width;
-        const int first_m = group * GM;
-        const int gsize = (tiles_m - first_m < GM) ? tiles_m - first_m : GM;
-        const int in_group = L - group * width;
-        tm = first_m + in_group % gsize;
-        tn = in_group / gsize;
-    }
-    const int m0 = tm * 256, n0 = tn * 256;
-    pipe::Source src;
-    src.a_planes = (const int8_t*)A; src.b_planes = (const int8_t*)Bt;
-    src.a_plane_stride = 0; src.b_plane_stride = 0;
-    src.a_idx = nullptr; src.b_idx = nullptr;
-    src.npairs = 1;
-    src.ld = ld_bytes;
-    v16f_t acc[4][4];
-#pragma unroll
-    for (int t = 0; t < 4; t++)
-#pragma unroll
-        for (int u = 0; u < 4; u++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[t][u][r] = 0.0f;
-    pipe::run<H16Op<BF16>, 4, 4, PF>(smem_h, src, m0, n0, acc);
-    store_tile<BF16, 4, 4>(acc, m0, n0, M, N, out_mode, Cout);
+    pipe::Source cm;
+    cm.a_planes = (const int8_t*)A; cm.b_planes = (const int8_t*)Bt;
+    cm.a_plane_stride = 0; cm.b_plane_stride = 0;
+    cm.ld = ld_bytes;
+
+    const int n_tiles = tiles_m * tiles_n;
+    int next_id = (int)blockIdx.x;
+    auto next_tile = [&](pipe::Tile& t) -> bool {
+        while (next_id < n_ids) {
+            const int id = next_id;
+            next_id += (int)gridDim.x;
+            /* XCD x owns tiles [x * per, (x + 1) * per) */
+            const int per = n_ids >> 3;
+            const int L = (id & 7) * per + (id >> 3);
+            if (L >= n_tiles) continue;
+            const int GM = 8;
+            const int width = GM * tiles_n;
+            const int group = L / width;
+            const int first_m = group * GM;
+            const int gsize = (tiles_m - first_m < GM) ? tiles_m - first_m : GM;
+            const int in_group = L - group * width;
+            t.m0 = (first_m + in_group % gsize) * 256;
+            t.n0 = (in_group / gsize) * 256;
+            t.tag = 0; t.a_idx = nullptr; t.b_idx = nullptr; t.npairs = 1;
+            return true;
+        }
+        return false;
+    };
+    auto epi = [&](v16f_t (&acc)[4][4], const pipe::Tile& t) {
+        store_tile<BF16, 4, 4>(acc, t.m0, t.n0, M, N, out_mode, Cout);
+    };
+    pipe::run_tiles<H16Op<BF16>, 4, 4, PF>(smem_h, cm, next_tile, epi);
 }
 
 template <bool BF16>
 int launch_pipe(const uint16_t* A, const uint16_t* Bt, int M, int N, int ld_bytes, int out_mode, void* C,
                 hipStream_t st) {
-    using Cf = pipe::Cfg<4, 4>;
+    constexpr int SMEM = pipe::TilesCfg<4, 4>::SMEM_MAIN;
     static bool attr_set = false;
+    static int num_cus = 0;
     auto kern = hgemm_pipe_kernel<BF16, 2>;
     if (!attr_set) {
         if (!ESHKOL_HIP_OK(hipFuncSetAttribute((const void*)kern,
-                hipFuncAttributeMaxDynamicSharedMemorySize, Cf::SMEM_MAIN))) return -1;
+                hipFuncAttributeMaxDynamicSharedMemorySize, SMEM))) return -1;
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (!ESHKOL_HIP_OK(hipGetDevice(&dev)) || !ESHKOL_HIP_OK(hipGetDeviceProperties(&prop, dev))) return -1;
+        num_cus = prop.multiProcessorCount;
         attr_set = true;
     }
     const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(256), Cf::SMEM_MAIN, st,
-                       A, Bt, M, N, ld_bytes, out_mode, C, tiles_m, tiles_n);
+    const int n_ids = (tiles_m * tiles_n + 7) / 8 * 8;      /* padded so every XCD owns the same count */
+    int grid = (num_cus / 8) * 8;
+    if (grid < 8) grid = 8;
+    if (grid > n_ids) grid = n_ids;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), SMEM, st,
+                       A, Bt, M, N, ld_bytes, out_mode, C, tiles_m, tiles_n, n_ids);
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 
@@ -406,7 +424,8 @@ int hgemm_any(const uint16_t* A, const uint16_t* Bt, uint64_t M, uint64_t K, uin
     if (((uintptr_t)A & 15) || ((uintptr_t)Bt & 15)) return -1;
     const int m = (int)M, n = (int)N, ldb = (int)(ld * 2);
     const long long big = (long long)((M + 255) / 256) * ((N + 255) / 256);
-    if (big >= 128 && ldb % 256 == 0)
+    /* the pipelined kernel wants whole pairs of 128-byte k-blocks and more than two per tile */
+    if (big >= 128 && ldb % 256 == 0 && ldb >= 512)
         return is_bf16 ? launch_pipe<true>(A, Bt, m, n, ldb, out_mode, C, st)
                        : launch_pipe<false>(A, Bt, m, n, ldb, out_mode, C, st);
     if (big >= 256)

@@ -179,6 +179,7 @@ __device__ __forceinline__ void epilogue(const HipIgemmArgs& g, int o, int m0, i
 
 /* ---- pipelined kernel ------------------------------------------------------ */
 
+/* One workgroup per tile: the same pipeline with a tile list of one. */
 template <int TM, int TN, int PF>
 __global__ __launch_bounds__(256, 1)
 void igemm_i8_pipe_kernel(HipIgemmArgs g, int tiles_m, int tiles_n, int chunk) {
@@ -186,26 +187,27 @@ void igemm_i8_pipe_kernel(HipIgemmArgs g, int tiles_m, int tiles_n, int chunk) {
     int o, tm, tn;
     if (!map_workgroup((int)blockIdx.x, tiles_m, tiles_n, (int)g.n_out, chunk, &o, &tm, &tn)) return;
     constexpr int BM = 2 * TM * 32, BN = 2 * TN * 32;
-    const int m0 = tm * BM, n0 = tn * BN;
+    pipe::Source cm;
+    cm.a_planes = g.a_planes; cm.b_planes = g.b_planes;
+    cm.a_plane_stride = g.a_plane_stride; cm.b_plane_stride = g.b_plane_stride;
+    cm.ld = (int)g.ldk;
 
     const int pair_lo = g.pair_first[o];
-    pipe::Source src;
-    src.a_planes = g.a_planes; src.b_planes = g.b_planes;
-    src.a_plane_stride = g.a_plane_stride; src.b_plane_stride = g.b_plane_stride;
-    src.a_idx = g.pair_a + pair_lo; src.b_idx = g.pair_b + pair_lo;
-    src.npairs = g.pair_first[o + 1] - pair_lo;
-    src.ld = (int)g.ldk;
-
-    v16i_t acc[TM][TN];
-#pragma unroll
-    for (int t = 0; t < TM; t++)
-#pragma unroll
-        for (int u = 0; u < TN; u++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[t][u][r] = 0;
-
-    if (src.npairs > 0) pipe::run<I8Op, TM, TN, PF>(smem_i8, src, m0, n0, acc);
-    epilogue<TM, TN>(g, o, m0, n0, acc, smem_i8);
+    const int npairs = g.pair_first[o + 1] - pair_lo;
+    if (npairs <= 0) return;             /* the caller promises every plane a product */
+    bool handed_out = false;
+    auto next_tile = [&](pipe::Tile& t) -> bool {
+        if (handed_out) return false;
+        handed_out = true;
+        t.m0 = tm * BM; t.n0 = tn * BN; t.tag = o;
+        t.a_idx = g.pair_a + pair_lo; t.b_idx = g.pair_b + pair_lo;
+        t.npairs = npairs;
+        return true;
+    };
+    auto epi = [&](v16i_t (&acc)[TM][TN], const pipe::Tile& t) {
+        epilogue<TM, TN>(g, t.tag, t.m0, t.n0, acc, smem_i8);
+    };
+    pipe::run_tiles<I8Op, TM, TN, PF>(smem_i8, cm, next_tile, epi);
 }
 
 /* ---- persistent pipelined kernel ------------------------------------------------
@@ -220,7 +222,6 @@ void igemm_i8_persistent_kernel(HipIgemmArgs g, int tiles_m, int tiles_n, int ch
     pipe::Source cm;
     cm.a_planes = g.a_planes; cm.b_planes = g.b_planes;
     cm.a_plane_stride = g.a_plane_stride; cm.b_plane_stride = g.b_plane_stride;
-    cm.a_idx = nullptr; cm.b_idx = nullptr; cm.npairs = 0;
     cm.ld = (int)g.ldk;
 
     int next_id = (int)blockIdx.x;
@@ -361,7 +362,8 @@ template <int PF>
 int launch_pipe(const HipIgemmArgs& a, hipStream_t st) {
     using C = pipe::Cfg<4, 4>;
     constexpr int EPI = C::BM * (C::BN + 16);
-    constexpr int SMEM = C::SMEM_MAIN > EPI ? C::SMEM_MAIN : EPI;
+    constexpr int MAIN = pipe::TilesCfg<4, 4>::SMEM_MAIN;
+    constexpr int SMEM = MAIN > EPI ? MAIN : EPI;
     static bool attr_set = false;
     return launch_kernel(igemm_i8_pipe_kernel<4, 4, PF>, SMEM, &attr_set, a, C::BM, C::BN, st);
 }
