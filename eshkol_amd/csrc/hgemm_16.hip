@@ -96,8 +96,9 @@ __global__ __launch_bounds__(256, 4)
 void convert_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
                            uint16_t* __restrict__ out, uint64_t rows_padded, uint64_t ld) {
     __shared__ __align__(16) double tile[kmaj::SMEM_DOUBLES];
-    kmaj::for_each_pair<false>(X, rows, K, rows_padded, ld, tile,
-        [&](uint64_t row, uint64_t k, double x0, double x1) {
+    kmaj::for_each_pair(X, rows, K, rows_padded, ld, 0xffffffffu, tile,
+        [](uint64_t) { return 0; },
+        [&](uint64_t row, uint64_t k, double x0, double x1, int) {
             *(uint32_t*)(out + row * ld + k) = narrow_pair<BF16>(x0, x1);
         });
 }
@@ -441,8 +442,8 @@ namespace {
 int convert_any(const double* in, uint16_t* out, uint64_t rows, uint64_t cols,
                 uint64_t rows_padded, uint64_t ld, int is_bf16, bool kmajor, void* stream) {
     if (!in || !out || rows == 0 || cols == 0 || rows_padded < rows || ld < cols || (ld & 1)) return -1;
-    const uint64_t nblk = kmajor ? kmaj::grid_blocks(rows_padded, ld) : ((ld / 2 + 255) / 256) * rows_padded;
-    if (nblk > 0x7fffffffULL) return -1;
+    const uint64_t nblk = kmajor ? kmaj::grid_blocks(rows_padded, ld, eshkol_hip_num_cus()) : ((ld / 2 + 255) / 256) * rows_padded;
+    if (nblk > 0x7fffffffULL || (kmajor && kmaj::tile_count(rows_padded, ld) > 0x7fffffffULL)) return -1;
     hipStream_t st = (hipStream_t)stream;
     const dim3 grid((unsigned)nblk), block(256);
     if (kmajor) {

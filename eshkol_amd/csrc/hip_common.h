@@ -41,6 +41,18 @@ enum {
 void* eshkol_hip_workspace(int slot, size_t bytes);
 void  eshkol_hip_workspace_release(void);
 
+/* compute units of the current device (256 if the query fails) */
+static inline int eshkol_hip_num_cus(void) {
+    static int cached = 0;
+    if (cached == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached = n;
+    }
+    return cached;
+}
+
 static inline size_t round_up_sz(size_t v, size_t m) { return (v + m - 1) / m * m; }
 
 #endif

@@ -30,6 +30,7 @@
 #include <mutex>
 
 typedef double d2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t v4u_t __attribute__((ext_vector_type(4)));
 
 namespace {
 
@@ -39,66 +40,93 @@ namespace {
 constexpr int MAX_MODULI = 16;
 const int H_MODULI[MAX_MODULI] = { OZAKI_MODULI_16 };
 
-struct ModuliTable { int p[MAX_MODULI]; int c18[MAX_MODULI]; int c36[MAX_MODULI]; };
+/* Byte weights of the moduli: 256^i mod p for the seven magnitude bytes, and
+ * -(256^7) mod p for the sign byte (see scaled_integer). */
+struct ModuliTable { int p[MAX_MODULI]; uint32_t wlo[MAX_MODULI]; uint32_t whi[MAX_MODULI]; };
 constexpr ModuliTable make_table() {
     ModuliTable t{};
     const int m[MAX_MODULI] = { OZAKI_MODULI_16 };
     for (int l = 0; l < MAX_MODULI; l++) {
+        const uint32_t p = (uint32_t)m[l];
         t.p[l] = m[l];
-        t.c18[l] = (int)((1ull << 18) % (unsigned)m[l]);
-        t.c36[l] = (int)((1ull << 36) % (unsigned)m[l]);
+        uint32_t c[8] = {}, pw = 1u % p;
+        for (int i = 0; i < 8; i++) { c[i] = pw; pw = pw * 256u % p; }
+        c[7] = (p - c[7]) % p;
+        t.wlo[l] = c[0] | c[1] << 8 | c[2] << 16 | c[3] << 24;
+        t.whi[l] = c[4] | c[5] << 8 | c[6] << 16 | c[7] << 24;
     }
     return t;
 }
 constexpr ModuliTable TBL = make_table();
 
-/* |trunc(x * 2^sh)| as an integer (< 2^53 by construction of sh) and its sign,
- * read straight off the bit pattern: the right shift is the truncation. */
-__device__ __forceinline__ uint64_t scaled_magnitude(double x, int sh, bool* neg) {
+/* trunc(x * 2^sh), an integer of magnitude below 2^53 by construction of sh, as
+ * eight bytes: the low seven of its 64-bit two's complement, and 1 or 0 in the
+ * eighth for negative or not. Its value is sum_{i<7} b_i 256^i - b_7 256^7. The
+ * magnitude is read straight off the bit pattern: the right shift is the
+ * truncation. */
+struct Scaled { uint32_t lo, hi; };
+__device__ __forceinline__ Scaled scaled_integer(double x, int sh) {
     const uint64_t bits = __double_as_longlong(x);
-    *neg = (bits >> 63) != 0;
     const int e = (int)((bits >> 52) & 0x7ff);
     uint64_t mant = bits & 0xfffffffffffffull;
     int e_eff = 1;
     if (e != 0) { mant |= 1ull << 52; e_eff = e; }
     const int rs = 1075 - e_eff - sh;          /* value = mant * 2^-rs */
-    if (rs >= 64) return 0;
-    if (rs <= 0) return mant;                  /* excluded by the host's range check */
-    return mant >> rs;
+    uint64_t t = mant;                         /* rs <= 0 is excluded by the host's range check */
+    if (rs >= 64) t = 0;
+    else if (rs > 0) t = mant >> rs;
+    const uint64_t m = (uint64_t)((int64_t)bits >> 63);
+    const uint64_t v = (t ^ m) - m;
+    return { (uint32_t)v, (uint32_t)(v >> 32) & 0x01ffffffu };
 }
 
+/* A word whose low byte is the int8 residue of s modulo p_L, the representative
+ * in [-p/2, p/2). Five full-rate instructions: two byte dot products give
+ * x = sum b_i w_i < 2^19, congruent to s; q = nearest integer to x/p comes out of
+ * one fma against 1.5 * 2^23 (x/p < 2^12 is off by at most 2e-4 in the product
+ * and, p being odd, at least 1/(2p) >= 2e-3 from a half-integer), left in the low
+ * bits of the float as 2^22 + q; x - (2^22 + q) p then differs from the residue by
+ * a multiple of 256. For p = 256 the residue is the low byte of s itself. */
 template <int L>
-__device__ __forceinline__ int residue(uint64_t t, bool neg) {
+__device__ __forceinline__ uint32_t residue_byte(Scaled s) {
     constexpr int p = TBL.p[L];
-    const uint32_t lo = (uint32_t)(t & 0x3ffff);
-    const uint32_t mid = (uint32_t)((t >> 18) & 0x3ffff);
-    const uint32_t hi = (uint32_t)(t >> 36);
-    /* fold 2^36 and 2^18 into the modulus twice: t = r27 = x (mod p), x < 2^19 */
-    const uint32_t r27 = hi * (uint32_t)TBL.c36[L] + mid * (uint32_t)TBL.c18[L] + lo;   /* < 2^27 */
-    const uint32_t x = (r27 >> 18) * (uint32_t)TBL.c18[L] + (r27 & 0x3ffff);
-    /* nearest-multiple reduction in fp32, all full-rate instructions. x/p < 2^12
-     * is computed to within 4e-4 and, unless it is a tie, lies at least 1/(2p) >=
-     * 2e-3 from a half-integer, so q is the nearest integer to x/p and x - q p is
-     * exact and already in [-p/2, p/2]. The tie (p = 256, x = 128 mod 256) may
-     * come out as +128 and is folded to -128. */
-    const float xf = neg ? -(float)x : (float)x;
-    const float q = rintf(xf * (1.0f / (float)p));
-    int s = (int)fmaf(-q, (float)p, xf);
-    if (2 * s >= p) s -= p;
-    return s;
+    if (p == 256) return s.lo;
+    const uint32_t x = __builtin_amdgcn_udot4(s.lo, TBL.wlo[L], __builtin_amdgcn_udot4(s.hi, TBL.whi[L], 0u, false), false);
+    const float qm = fmaf((float)x, 1.0f / (float)p, 12582912.0f);
+    return (uint32_t)(__mul24(__float_as_int(qm), -p) + (int)x);
 }
 
 /* Residues of two consecutive k of one row: one 16-bit store per plane. */
 template <int NMOD>
 __device__ __forceinline__ void split_pair(double x0, double x1, int sh, int8_t* out, uint64_t plane_stride) {
-    bool n0, n1;
-    const uint64_t t0 = scaled_magnitude(x0, sh, &n0);
-    const uint64_t t1 = scaled_magnitude(x1, sh, &n1);
+    const Scaled s0 = scaled_integer(x0, sh), s1 = scaled_integer(x1, sh);
+#define ESHKOL_SPLIT_ONE(L)                                                           \
+    if (L < NMOD)                                                                     \
+        *(uint16_t*)(out + (uint64_t)L * plane_stride) =                              \
+            (uint16_t)__builtin_amdgcn_perm(residue_byte<L>(s1), residue_byte<L>(s0), 0x0c0c0400u);
+    ESHKOL_SPLIT_ONE(0)  ESHKOL_SPLIT_ONE(1)  ESHKOL_SPLIT_ONE(2)  ESHKOL_SPLIT_ONE(3)
+    ESHKOL_SPLIT_ONE(4)  ESHKOL_SPLIT_ONE(5)  ESHKOL_SPLIT_ONE(6)  ESHKOL_SPLIT_ONE(7)
+    ESHKOL_SPLIT_ONE(8)  ESHKOL_SPLIT_ONE(9)  ESHKOL_SPLIT_ONE(10) ESHKOL_SPLIT_ONE(11)
+    ESHKOL_SPLIT_ONE(12) ESHKOL_SPLIT_ONE(13) ESHKOL_SPLIT_ONE(14) ESHKOL_SPLIT_ONE(15)
+#undef ESHKOL_SPLIT_ONE
+}
+
+/* Residues of sixteen consecutive k of one row: one 16-byte store per plane. */
+template <int NMOD>
+__device__ __forceinline__ void split_16(const double* x, int sh, int8_t* out, uint64_t plane_stride) {
+    Scaled s[16];
+#pragma unroll
+    for (int e = 0; e < 16; e++) s[e] = scaled_integer(x[e], sh);
 #define ESHKOL_SPLIT_ONE(L)                                                           \
     if (L < NMOD) {                                                                   \
-        const int r0 = residue<L>(t0, n0), r1 = residue<L>(t1, n1);                   \
-        *(uint16_t*)(out + (uint64_t)L * plane_stride) =                              \
-            (uint16_t)((uint8_t)(int8_t)r0 | ((uint16_t)(uint8_t)(int8_t)r1 << 8));   \
+        v4u_t w;                                                                      \
+        _Pragma("unroll")                                                             \
+        for (int g = 0; g < 4; g++) {                                                 \
+            const uint32_t w01 = __builtin_amdgcn_perm(residue_byte<L>(s[4 * g + 1]), residue_byte<L>(s[4 * g]), 0x0c0c0400u); \
+            const uint32_t w23 = __builtin_amdgcn_perm(residue_byte<L>(s[4 * g + 3]), residue_byte<L>(s[4 * g + 2]), 0x0c0c0400u); \
+            w[g] = __builtin_amdgcn_perm(w23, w01, 0x05040100u);                      \
+        }                                                                             \
+        *(v4u_t*)(out + (uint64_t)L * plane_stride) = w;                              \
     }
     ESHKOL_SPLIT_ONE(0)  ESHKOL_SPLIT_ONE(1)  ESHKOL_SPLIT_ONE(2)  ESHKOL_SPLIT_ONE(3)
     ESHKOL_SPLIT_ONE(4)  ESHKOL_SPLIT_ONE(5)  ESHKOL_SPLIT_ONE(6)  ESHKOL_SPLIT_ONE(7)
@@ -132,17 +160,80 @@ void crt_split_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
     split_pair<NMOD>(x0, x1, sh, planes + row * ldk + k, rows_padded * ldk);
 }
 
+/* Row-major X[rows][K], pitches that are multiples of 16 bytes. One thread: four
+ * consecutive k of one row. The residues of a block (1024 k of one row, all
+ * planes) are collected in LDS as one word per thread and plane, then leave as
+ * 16-byte stores: four store instructions per thread instead of a 2-byte store
+ * per plane and pair. */
+template <int NMOD>
+__global__ __launch_bounds__(256)
+void crt_split_staged_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
+                             const int32_t* __restrict__ shift, int8_t* __restrict__ planes,
+                             uint64_t rows_padded, uint64_t ldk) {
+    __shared__ __align__(16) uint32_t stage[NMOD][256];
+    const uint32_t cpr = (uint32_t)((ldk + 1023) / 1024);        /* blocks per row */
+    const uint64_t row = blockIdx.x / cpr;
+    const uint64_t kbase = (uint64_t)(blockIdx.x % cpr) * 1024;
+    const int tid = threadIdx.x;
+    const uint64_t k = kbase + 4 * (uint64_t)tid;
+    double x[4] = {0.0, 0.0, 0.0, 0.0};
+    int sh = 0;
+    if (row < rows && k < K) {
+        sh = shift[row];
+        const double* p = X + row * K + k;
+        if (k + 3 < K && (K & 1) == 0 && (((uintptr_t)X & 15) == 0)) {
+            const d2_t v0 = *(const d2_t*)p, v1 = *(const d2_t*)(p + 2);
+            x[0] = v0.x; x[1] = v0.y; x[2] = v1.x; x[3] = v1.y;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) if (k + e < K) x[e] = p[e];
+        }
+    }
+    Scaled t[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) t[e] = scaled_integer(x[e], sh);
+#define ESHKOL_SPLIT_ONE(L)                                                           \
+    if (L < NMOD) {                                                                   \
+        const uint32_t w01 = __builtin_amdgcn_perm(residue_byte<L>(t[1]), residue_byte<L>(t[0]), 0x0c0c0400u); \
+        const uint32_t w23 = __builtin_amdgcn_perm(residue_byte<L>(t[3]), residue_byte<L>(t[2]), 0x0c0c0400u); \
+        stage[L][tid] = __builtin_amdgcn_perm(w23, w01, 0x05040100u);                 \
+    }
+    ESHKOL_SPLIT_ONE(0)  ESHKOL_SPLIT_ONE(1)  ESHKOL_SPLIT_ONE(2)  ESHKOL_SPLIT_ONE(3)
+    ESHKOL_SPLIT_ONE(4)  ESHKOL_SPLIT_ONE(5)  ESHKOL_SPLIT_ONE(6)  ESHKOL_SPLIT_ONE(7)
+    ESHKOL_SPLIT_ONE(8)  ESHKOL_SPLIT_ONE(9)  ESHKOL_SPLIT_ONE(10) ESHKOL_SPLIT_ONE(11)
+    ESHKOL_SPLIT_ONE(12) ESHKOL_SPLIT_ONE(13) ESHKOL_SPLIT_ONE(14) ESHKOL_SPLIT_ONE(15)
+#undef ESHKOL_SPLIT_ONE
+    __syncthreads();
+    const uint64_t plane_stride = rows_padded * ldk;
+#pragma unroll
+    for (int j = 0; j < NMOD * 64 / 256 + (NMOD * 64 % 256 != 0); j++) {
+        const int c = tid + 256 * j;
+        const int plane = c >> 6, ch = c & 63;
+        const uint64_t kk = kbase + 16 * (uint64_t)ch;
+        if (plane < NMOD && kk < ldk)
+            *(v4u_t*)(planes + (uint64_t)plane * plane_stride + row * ldk + kk) = *(const v4u_t*)&stage[plane][4 * ch];
+    }
+}
+
 /* k-major X[K][rows] (B as the runtime stores it), same output. */
 template <int NMOD>
 __global__ __launch_bounds__(256, 4)
 void crt_split_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
                              const int32_t* __restrict__ shift, int8_t* __restrict__ planes,
-                             uint64_t rows_padded, uint64_t ldk) {
+                             uint64_t rows_padded, uint64_t ldk, uint32_t group) {
     __shared__ __align__(16) double tile[kmaj::SMEM_DOUBLES];
     const uint64_t plane_stride = rows_padded * ldk;
-    kmaj::for_each_pair<true>(X, rows, K, rows_padded, ldk, tile,
-        [&](uint64_t row, uint64_t k, double x0, double x1) {
-            const int sh = (row < rows) ? shift[row] : 0;
+    if ((ldk & 15) == 0 && (((uintptr_t)planes & 15) == 0)) {
+        kmaj::for_each_16(X, rows, K, rows_padded, ldk, group, tile,
+            [&](uint64_t row) { return (row < rows) ? shift[row] : 0; },
+            [&](uint64_t row, uint64_t k, const double* x, int sh) {
+                split_16<NMOD>(x, sh, planes + row * ldk + k, plane_stride);
+            });
+        return;
+    }
+    kmaj::for_each_pair(X, rows, K, rows_padded, ldk, group, tile,
+        [&](uint64_t row) { return (row < rows) ? shift[row] : 0; },
+        [&](uint64_t row, uint64_t k, double x0, double x1, int sh) {
             split_pair<NMOD>(x0, x1, sh, planes + row * ldk + k, plane_stride);
         });
 }
@@ -286,8 +377,14 @@ template <int NMOD>
 void launch_split(const double* X, uint64_t rows, uint64_t K, const int32_t* shift, int8_t* planes,
                   uint64_t rows_padded, uint64_t ldk, bool kmajor, hipStream_t st) {
     if (kmajor) {
-        dim3 grid((unsigned)kmaj::grid_blocks(rows_padded, ldk));
+        dim3 grid((unsigned)kmaj::grid_blocks(rows_padded, ldk, eshkol_hip_num_cus()));
         hipLaunchKernelGGL(crt_split_kmajor_kernel<NMOD>, grid, dim3(256), 0, st, X, rows, K, shift, planes,
+                           rows_padded, ldk, 0xffffffffu);
+        return;
+    }
+    if (ldk % 16 == 0 && ((uintptr_t)planes & 15) == 0) {
+        dim3 grid((unsigned)(((ldk + 1023) / 1024) * rows_padded));
+        hipLaunchKernelGGL(crt_split_staged_kernel<NMOD>, grid, dim3(256), 0, st, X, rows, K, shift, planes,
                            rows_padded, ldk);
         return;
     }
@@ -305,7 +402,7 @@ int crt_split_any(const double* X, uint64_t rows, uint64_t K, const int32_t* shi
     if (num_moduli < 2 || num_moduli > MAX_MODULI) return -1;
     if (rows_padded < rows || ldk < K || (ldk & 1)) return -1;
     if (((ldk / 2 + 255) / 256) * rows_padded > 0x7fffffffULL) return -1;
-    if (kmaj::grid_blocks(rows_padded, ldk) > 0x7fffffffULL) return -1;
+    if (kmaj::tile_count(rows_padded, ldk) > 0x7fffffffULL) return -1;
     hipStream_t st = (hipStream_t)stream;
     switch (num_moduli) {
 #define CASE(n) case n: launch_split<n>(X, rows, K, shift, planes, rows_padded, ldk, kmajor, st); break;

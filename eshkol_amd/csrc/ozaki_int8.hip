@@ -75,9 +75,9 @@ void slice_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K
                          uint64_t rows_padded, uint64_t ldk) {
     __shared__ __align__(16) double tile[kmaj::SMEM_DOUBLES];
     const uint64_t plane_stride = rows_padded * ldk;
-    kmaj::for_each_pair<false>(X, rows, K, rows_padded, ldk, tile,
-        [&](uint64_t row, uint64_t k, double x0, double x1) {
-            const double sc = (row < rows) ? scale[row] : 1.0;
+    kmaj::for_each_pair(X, rows, K, rows_padded, ldk, 0xffffffffu, tile,
+        [&](uint64_t row) { return (row < rows) ? scale[row] : 1.0; },
+        [&](uint64_t row, uint64_t k, double x0, double x1, double sc) {
             slice_pair(x0, x1, sc, s, planes + row * ldk + k, plane_stride);
         });
 }
@@ -132,8 +132,8 @@ int slice_any(const double* X, uint64_t rows, uint64_t K, const double* scale, i
               int8_t* planes, uint64_t rows_padded, uint64_t ldk, bool kmajor, void* stream) {
     if (!X || !scale || !planes || rows == 0 || K == 0 || s < 1 || s > 16) return -1;
     if (rows_padded < rows || ldk < K || (ldk & 1)) return -1;
-    const uint64_t nblk = kmajor ? kmaj::grid_blocks(rows_padded, ldk) : ((ldk / 2 + 255) / 256) * rows_padded;
-    if (nblk > 0x7fffffffULL) return -1;
+    const uint64_t nblk = kmajor ? kmaj::grid_blocks(rows_padded, ldk, eshkol_hip_num_cus()) : ((ldk / 2 + 255) / 256) * rows_padded;
+    if (nblk > 0x7fffffffULL || (kmajor && kmaj::tile_count(rows_padded, ldk) > 0x7fffffffULL)) return -1;
     if (kmajor)
         hipLaunchKernelGGL(slice_kmajor_kernel, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
                            X, rows, K, scale, s, planes, rows_padded, ldk);
