@@ -97,7 +97,15 @@ void colabsmax_fold_kernel(const double* __restrict__ partial, uint64_t R, int s
     const uint64_t col = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     if (col >= R) return;
     double m = 0.0;
-    for (int s = 0; s < slices; s++) { const double o = partial[(uint64_t)s * R + col]; if (o > m) m = o; }
+    int s = 0;
+    for (; s + 8 <= slices; s += 8) {           /* eight loads in flight, not one */
+        double o[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) o[u] = partial[(uint64_t)(s + u) * R + col];
+#pragma unroll
+        for (int u = 0; u < 8; u++) if (o[u] > m) m = o[u];
+    }
+    for (; s < slices; s++) { const double o = partial[(uint64_t)s * R + col]; if (o > m) m = o; }
     out[col] = (m > 0.0) ? m : zero_value;
 }
 

@@ -25,6 +25,7 @@
 #include "kernels.h"
 #include "kmajor_tile.h"
 
+#include <climits>
 #include <cmath>
 #include <cstring>
 #include <mutex>
@@ -247,11 +248,16 @@ struct CrtConsts {
 /* One thread: four consecutive columns of one row. The arithmetic is the
  * reference's, operation for operation: S1 = fma(sl1_l, w, S1), S2 likewise,
  * l ascending; s = S1 + S2; Q = round(s*Pinv); c' = fma(-P1,Q,S1) + fma(-P2,Q,S2);
- * C = (c' * 2^-mu) * 2^-nu. */
+ * C = (c' * 2^-mu) * 2^-nu. The number of planes is a compile-time constant so
+ * that a thread's loads of all planes are issued together, before the first
+ * use: the kernel moves 24 bytes per element and has to keep HBM busy. So is
+ * the tanh epilogue: its code would otherwise cost every launch three quarters
+ * of its occupancy in registers. */
+template <int NMOD, bool TANH>
 __global__ __launch_bounds__(256)
 void crt_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t N, CrtConsts cc,
                             const int32_t* __restrict__ mu, const int32_t* __restrict__ nu,
-                            const double* __restrict__ bias, int act, double* __restrict__ C) {
+                            const double* __restrict__ bias, double* __restrict__ C) {
     const uint32_t cpr = (uint32_t)(((N + 3) / 4 + 255) / 256);   /* blocks per row */
     const uint64_t row = blockIdx.x / cpr;
     const uint64_t col = ((uint64_t)(blockIdx.x % cpr) * 256 + threadIdx.x) * 4;
@@ -259,39 +265,210 @@ void crt_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t N
     const uint64_t tot = M * N, idx = row * N + col;
     const int nvalid = (N - col < 4) ? (int)(N - col) : 4;
     const bool vec = (nvalid == 4) && ((N & 3) == 0) && (((uintptr_t)W & 3) == 0);
-    double S1[4] = {0, 0, 0, 0}, S2[4] = {0, 0, 0, 0};
-    for (int l = 0; l < cc.n; l++) {
-        const int8_t* w = W + (uint64_t)l * tot + idx;
-        int8_t v[4] = {0, 0, 0, 0};
-        if (vec) {
-            const uint32_t u = *(const uint32_t*)w;
-            v[0] = (int8_t)(u & 0xff); v[1] = (int8_t)((u >> 8) & 0xff);
-            v[2] = (int8_t)((u >> 16) & 0xff); v[3] = (int8_t)(u >> 24);
-        } else {
-            for (int e = 0; e < nvalid; e++) v[e] = w[e];
+    uint32_t u[NMOD];
+    if (vec) {
+#pragma unroll
+        for (int l = 0; l < NMOD; l++) u[l] = *(const uint32_t*)(W + (uint64_t)l * tot + idx);
+    } else {
+#pragma unroll
+        for (int l = 0; l < NMOD; l++) {
+            const int8_t* w = W + (uint64_t)l * tot + idx;
+            u[l] = 0;
+#pragma unroll
+            for (int e = 0; e < 4; e++) if (e < nvalid) u[l] |= (uint32_t)(uint8_t)w[e] << (8 * e);
         }
+    }
+    int sh[4] = {0, 0, 0, 0};
+    double bv[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        if (e < nvalid) {
+            sh[e] = nu[col + e];
+            if (bias) bv[e] = bias[col + e];
+        }
+    }
+    const double mu_inv = ldexp(1.0, -mu[row]);
+    double S1[4] = {0, 0, 0, 0}, S2[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int l = 0; l < NMOD; l++) {
         const double a = cc.sl1[l], b = cc.sl2[l];
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            const double wd = (double)v[e];
+            const double wd = (double)(int8_t)(u[l] >> (8 * e));
             S1[e] = fma(a, wd, S1[e]);
             S2[e] = fma(b, wd, S2[e]);
         }
     }
-    const double mu_inv = ldexp(1.0, -mu[row]);
+    double out[4];
 #pragma unroll
     for (int e = 0; e < 4; e++) {
-        if (e >= nvalid) break;
         const double s = S1[e] + S2[e];
         const double Q = round(s * cc.Pinv);
         const double h1 = fma(-cc.P1, Q, S1[e]);
         const double h2 = fma(-cc.P2, Q, S2[e]);
         const double cp = h1 + h2;
-        double v = (cp * mu_inv) * ldexp(1.0, -nu[col + e]);
-        if (bias) v = v + bias[col + e];
-        if (act == 1) v = tanh(v);
-        C[idx + e] = v;
+        double v = (cp * mu_inv) * ldexp(1.0, -sh[e]);
+        if (bias) v = v + bv[e];
+        if (TANH) v = tanh(v);
+        out[e] = v;
     }
+    if (vec && (((uintptr_t)C & 15) == 0)) {
+        d2_t* o = (d2_t*)(C + idx);
+        d2_t lo, hi;
+        lo.x = out[0]; lo.y = out[1]; hi.x = out[2]; hi.y = out[3];
+        o[0] = lo; o[1] = hi;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) if (e < nvalid) C[idx + e] = out[e];
+    }
+}
+
+/* ---- shifts without a host pass over the maxima ---------------------------------
+ *
+ * The reference takes log2 of every row and column maximum on the host
+ * (gpu_memory.mm:376-420) for two things: floor(log2 m) per row, and the largest
+ * fractional part frac = log2 m - floor(log2 m) per operand. Both can be had
+ * without M + N libm calls. floor(log2 m) is the exponent of m unless its
+ * mantissa sits within 2^-40 of a power of two, where a libm result may round
+ * across the integer. And frac is within 2^-42 of log2 of the mantissa (a libm
+ * accurate to an ulp, results below 1024 in magnitude), so only maxima whose
+ * mantissa lies within 2^-40 of the largest one can carry the largest frac. The
+ * scan below leaves the exponents on the device and hands the host those few
+ * maxima; the host calls log2 on them exactly as the reference does. An operand
+ * with a mantissa next to a power of two, or with more than SCAN_CAND distinct
+ * candidates, takes the full host pass instead. */
+constexpr int SCAN_CAND = 64;
+constexpr int SCAN_THREADS = 1024;
+constexpr int32_t FL_ZERO = INT32_MIN;          /* marks a maximum of zero: shift 0 */
+constexpr unsigned long long MANT_ONE = 1ull << 52, MANT_WINDOW = 1ull << 12;
+
+struct CrtScan {
+    unsigned long long mant_max;
+    int32_t nonfinite, extreme, nonzero, e_min, e_max, ncand;
+    double cand[SCAN_CAND];
+};
+
+/* m > 0 finite -> exponent e = floor(log2 m) and mantissa n in [2^52, 2^53), m = n 2^(e-52) */
+__device__ __forceinline__ void decode_positive(double m, int* e, unsigned long long* n) {
+    const unsigned long long bits = (unsigned long long)__double_as_longlong(m);
+    const int ef = (int)(bits >> 52);
+    const unsigned long long mant = bits & (MANT_ONE - 1);
+    if (ef != 0) { *e = ef - 1023; *n = mant | MANT_ONE; }
+    else { const int p = 63 - __clzll((long long)mant); *e = p - 1074; *n = mant << (52 - p); }
+}
+
+/* block 0: the M row maxima of A; block 1: the N maxima of B */
+__global__ __launch_bounds__(SCAN_THREADS)
+void crt_scan_kernel(const double* __restrict__ amax, uint64_t M, const double* __restrict__ bmax, uint64_t N,
+                     int32_t* __restrict__ fl_a, int32_t* __restrict__ fl_b, CrtScan* __restrict__ out) {
+    __shared__ unsigned long long s_max, keys[256];
+    __shared__ int s_nonfinite, s_extreme, s_nonzero, s_emin, s_emax, s_ncand;
+    const double* x = blockIdx.x ? bmax : amax;
+    const uint64_t n_rows = blockIdx.x ? N : M;
+    int32_t* fl = blockIdx.x ? fl_b : fl_a;
+    CrtScan* o = out + blockIdx.x;
+    const int tid = threadIdx.x;
+    if (tid == 0) { s_max = 0; s_nonfinite = 0; s_extreme = 0; s_nonzero = 0; s_emin = INT32_MAX; s_emax = INT32_MIN; s_ncand = 0; }
+    if (tid < 256) keys[tid] = 0;
+    __syncthreads();
+    unsigned long long my_max = 0;
+    int my_nonfinite = 0, my_extreme = 0, my_nonzero = 0, my_emin = INT32_MAX, my_emax = INT32_MIN;
+    /* four loads in flight per thread: a single block must not crawl from one
+     * memory latency to the next */
+    for (uint64_t base = 0; base < n_rows; base += 4 * SCAN_THREADS) {
+        double v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const uint64_t i = base + (uint64_t)u * SCAN_THREADS + tid;
+            v[u] = (i < n_rows) ? x[i] : 0.0;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const uint64_t i = base + (uint64_t)u * SCAN_THREADS + tid;
+            if (i >= n_rows) continue;
+            const double m = v[u];
+            int32_t f = FL_ZERO;
+            if (!(m <= 1.79769313486231570815e308)) my_nonfinite = 1;   /* NaN or +Inf; maxima are >= 0 */
+            else if (m > 0.0) {
+                int e; unsigned long long n;
+                decode_positive(m, &e, &n);
+                f = e;
+                my_nonzero = 1;
+                if (n > my_max) my_max = n;
+                if (e < my_emin) my_emin = e;
+                if (e > my_emax) my_emax = e;
+                if ((n != MANT_ONE && n < MANT_ONE + MANT_WINDOW) || n >= 2 * MANT_ONE - MANT_WINDOW) my_extreme = 1;
+            }
+            fl[i] = f;
+        }
+    }
+    /* fold within the wave first: a thousand atomics on one LDS word would take
+     * longer than the scan itself */
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        const unsigned long long om = __shfl_xor(my_max, d);
+        const int on = __shfl_xor(my_emin, d), ox = __shfl_xor(my_emax, d);
+        const int flags = __shfl_xor(my_nonfinite | my_extreme << 1 | my_nonzero << 2, d);
+        if (om > my_max) my_max = om;
+        if (on < my_emin) my_emin = on;
+        if (ox > my_emax) my_emax = ox;
+        my_nonfinite |= flags & 1; my_extreme |= flags >> 1 & 1; my_nonzero |= flags >> 2 & 1;
+    }
+    if ((tid & 63) == 0) {
+        if (my_max) atomicMax(&s_max, my_max);
+        if (my_nonfinite) atomicOr(&s_nonfinite, 1);
+        if (my_extreme) atomicOr(&s_extreme, 1);
+        if (my_nonzero) { atomicOr(&s_nonzero, 1); atomicMin(&s_emin, my_emin); atomicMax(&s_emax, my_emax); }
+    }
+    __syncthreads();
+    /* second pass: the distinct maxima whose mantissa is within the window of the largest */
+    const unsigned long long floor_n = (s_max > MANT_ONE + MANT_WINDOW) ? s_max - MANT_WINDOW : MANT_ONE;
+    if (s_nonzero && !s_nonfinite) {
+        for (uint64_t base = 0; base < n_rows; base += 4 * SCAN_THREADS) {
+            double v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const uint64_t i = base + (uint64_t)u * SCAN_THREADS + tid;
+                v[u] = (i < n_rows) ? x[i] : 0.0;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const double m = v[u];
+                if (!(m > 0.0)) continue;
+                int e; unsigned long long n;
+                decode_positive(m, &e, &n);
+                if (n < floor_n) continue;
+                const unsigned long long bits = (unsigned long long)__double_as_longlong(m);
+                unsigned h = (unsigned)((bits * 0x9E3779B97F4A7C15ull) >> 56);
+                int probes = 0;
+                for (; probes < 256; probes++, h = (h + 1) & 255) {
+                    const unsigned long long old = atomicCAS(&keys[h], 0ull, bits);
+                    if (old == bits) break;
+                    if (old == 0ull) {
+                        const int slot = atomicAdd(&s_ncand, 1);
+                        if (slot < SCAN_CAND) o->cand[slot] = m;
+                        break;
+                    }
+                }
+                if (probes == 256) atomicAdd(&s_ncand, SCAN_CAND + 1);
+            }
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {
+        o->mant_max = s_max; o->nonfinite = s_nonfinite; o->extreme = s_extreme; o->nonzero = s_nonzero;
+        o->e_min = s_emin; o->e_max = s_emax; o->ncand = s_ncand;
+    }
+}
+
+/* shift = E - floor(log2 max), 0 for a maximum of zero (gpu_memory.mm:2524-2532), in place */
+__global__ __launch_bounds__(256)
+void crt_shift_kernel(int32_t* __restrict__ fl_a, uint64_t M, int32_t* __restrict__ fl_b, uint64_t N, int E) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= M + N) return;
+    int32_t* p = (i < M) ? fl_a + i : fl_b + (i - M);
+    const int32_t f = *p;
+    *p = (f == FL_ZERO) ? 0 : E - f;
 }
 
 /* ---- host bookkeeping ------------------------------------------------------ */
@@ -372,6 +549,7 @@ int ensure_tables(hipStream_t st) {
 }
 
 HipOzakiCrtStages g_last = {};
+bool g_force_host_pass = false;
 
 template <int NMOD>
 void launch_split(const double* X, uint64_t rows, uint64_t K, const int32_t* shift, int8_t* planes,
@@ -440,10 +618,22 @@ extern "C" int hip_ozaki_crt_reconstruct_f64(const int8_t* w_planes, uint64_t M,
     for (int l = 0; l < num_moduli; l++) { cc.sl1[l] = sl1[l]; cc.sl2[l] = sl2[l]; }
     cc.P1 = P1; cc.P2 = P2; cc.Pinv = Pinv; cc.n = num_moduli;
     dim3 grid((unsigned)((((N + 3) / 4 + 255) / 256) * M));
-    hipLaunchKernelGGL(crt_reconstruct_kernel, grid, dim3(256), 0, (hipStream_t)stream,
-                       w_planes, M, N, cc, mu, nu, bias, act, C);
+    switch (num_moduli) {
+#define CASE(n) case n:                                                                                   \
+        if (act == 1) hipLaunchKernelGGL((crt_reconstruct_kernel<n, true>), grid, dim3(256), 0, (hipStream_t)stream,  \
+                                         w_planes, M, N, cc, mu, nu, bias, C);                            \
+        else hipLaunchKernelGGL((crt_reconstruct_kernel<n, false>), grid, dim3(256), 0, (hipStream_t)stream,           \
+                                w_planes, M, N, cc, mu, nu, bias, C);                                     \
+        break;
+        CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8) CASE(9)
+        CASE(10) CASE(11) CASE(12) CASE(13) CASE(14) CASE(15) CASE(16)
+#undef CASE
+        default: return -1;
+    }
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
+
+extern "C" void hip_ozaki_crt_set_host_pass(int on) { g_force_host_pass = on != 0; }
 
 extern "C" int hip_ozaki_crt_last_stages(HipOzakiCrtStages* out) {
     if (!out || !g_last.a_planes) return -1;
@@ -488,43 +678,64 @@ extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, dou
     int32_t* dmu = (int32_t*)eshkol_hip_workspace(WS_ROWSHIFT, M * sizeof(int32_t));
     int32_t* dnu = (int32_t*)eshkol_hip_workspace(WS_COLSHIFT, N * sizeof(int32_t));
     if (!amax || !bmax || !dmu || !dnu) return -1;
-    char* host = (char*)pinned((M + N) * (sizeof(double) + sizeof(int32_t)));
-    if (!host) return -1;
-    double* h_amax = (double*)host;
+    CrtScan* dscan = (CrtScan*)eshkol_hip_workspace(WS_MISC, 2 * sizeof(CrtScan));
+    char* host = (char*)pinned(2 * sizeof(CrtScan) + (M + N) * (sizeof(double) + sizeof(int32_t)));
+    if (!dscan || !host) return -1;
+    CrtScan* h_scan = (CrtScan*)host;
+    double* h_amax = (double*)(h_scan + 2);
     double* h_bmax = h_amax + M;
     int32_t* h_mu = (int32_t*)(h_bmax + N);
     int32_t* h_nu = h_mu + M;
 
     if ((a_kmajor ? hip_colabsmax_f64(A, K, M, 0.0, amax, st) : hip_rowabsmax_f64(A, M, K, 0.0, amax, st)) != 0) return -1;
     if ((b_kmajor ? hip_colabsmax_f64(B, K, N, 0.0, bmax, st) : hip_rowabsmax_f64(B, N, K, 0.0, bmax, st)) != 0) return -1;
-    if (!ESHKOL_HIP_OK(hipMemcpyAsync(h_amax, amax, M * sizeof(double), hipMemcpyDeviceToHost, st))) return -1;
-    if (!ESHKOL_HIP_OK(hipMemcpyAsync(h_bmax, bmax, N * sizeof(double), hipMemcpyDeviceToHost, st))) return -1;
+    hipLaunchKernelGGL(crt_scan_kernel, dim3(2), dim3(SCAN_THREADS), 0, st, amax, M, bmax, N, dmu, dnu, dscan);
+    if (!ESHKOL_HIP_OK(hipMemcpyAsync(h_scan, dscan, 2 * sizeof(CrtScan), hipMemcpyDeviceToHost, st))) return -1;
     if (!ESHKOL_HIP_OK(hipStreamSynchronize(st))) return -1;
+    if (h_scan[0].nonfinite || h_scan[1].nonfinite) return -1;          /* NaN/Inf input */
 
-    /* frac bounds (gpu_memory.mm:403-417); a non-finite maximum marks NaN/Inf input.
-     * floor(log2(max)) is needed again for the shifts below: it is kept in the
-     * shift arrays so each maximum costs one log2. */
-    double frac_A = 0.0, frac_B = 0.0;
-    for (uint64_t i = 0; i < M; i++) {
-        const double m = h_amax[i];
-        if (!std::isfinite(m)) return -1;
-        h_mu[i] = 0;
-        if (m > 0.0) {
-            const double lg = log2(m), fl = floor(lg), f = lg - fl;
-            h_mu[i] = (int32_t)fl;
-            if (f > frac_A) frac_A = f;
+    /* frac bounds (gpu_memory.mm:403-417) and the range of floor(log2 max) per operand */
+    double frac[2] = {0.0, 0.0};
+    int e_min[2], e_max[2];
+    bool any[2];
+    const bool full_pass = g_force_host_pass || h_scan[0].extreme || h_scan[1].extreme ||
+                           h_scan[0].ncand > SCAN_CAND || h_scan[1].ncand > SCAN_CAND;
+    if (!full_pass) {
+        for (int o = 0; o < 2; o++) {
+            for (int c = 0; c < h_scan[o].ncand; c++) {
+                const double lg = log2(h_scan[o].cand[c]), f = lg - floor(lg);
+                if (f > frac[o]) frac[o] = f;
+            }
+            any[o] = h_scan[o].nonzero != 0; e_min[o] = h_scan[o].e_min; e_max[o] = h_scan[o].e_max;
         }
-    }
-    for (uint64_t j = 0; j < N; j++) {
-        const double m = h_bmax[j];
-        if (!std::isfinite(m)) return -1;
-        h_nu[j] = 0;
-        if (m > 0.0) {
-            const double lg = log2(m), fl = floor(lg), f = lg - fl;
-            h_nu[j] = (int32_t)fl;
-            if (f > frac_B) frac_B = f;
+    } else {
+        /* the reference's own pass: one log2 per maximum */
+        if (!ESHKOL_HIP_OK(hipMemcpyAsync(h_amax, amax, M * sizeof(double), hipMemcpyDeviceToHost, st))) return -1;
+        if (!ESHKOL_HIP_OK(hipMemcpyAsync(h_bmax, bmax, N * sizeof(double), hipMemcpyDeviceToHost, st))) return -1;
+        if (!ESHKOL_HIP_OK(hipStreamSynchronize(st))) return -1;
+        const double* h_max[2] = { h_amax, h_bmax };
+        int32_t* h_fl[2] = { h_mu, h_nu };
+        const uint64_t cnt[2] = { M, N };
+        for (int o = 0; o < 2; o++) {
+            any[o] = false; e_min[o] = INT32_MAX; e_max[o] = INT32_MIN;
+            for (uint64_t i = 0; i < cnt[o]; i++) {
+                const double m = h_max[o][i];
+                h_fl[o][i] = FL_ZERO;
+                if (m > 0.0) {
+                    const double lg = log2(m), fl = floor(lg), f = lg - fl;
+                    const int e = (int)fl;
+                    h_fl[o][i] = e;
+                    if (f > frac[o]) frac[o] = f;
+                    any[o] = true;
+                    if (e < e_min[o]) e_min[o] = e;
+                    if (e > e_max[o]) e_max[o] = e;
+                }
+            }
         }
+        if (!ESHKOL_HIP_OK(hipMemcpyAsync(dmu, h_mu, M * sizeof(int32_t), hipMemcpyHostToDevice, st))) return -1;
+        if (!ESHKOL_HIP_OK(hipMemcpyAsync(dnu, h_nu, N * sizeof(int32_t), hipMemcpyHostToDevice, st))) return -1;
     }
+    const double frac_A = frac[0], frac_B = frac[1];
     const double log2K = log2((double)K);
     if (adaptive) {                                   /* gpu_memory.mm:433-453 */
         std::call_once(g_cumul_once, [] {
@@ -545,16 +756,10 @@ extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, dou
     int E = (int)floor((crt.log2P - 1.0 - log2K - frac_A - frac_B) / 2.0);   /* gpu_memory.mm:2510-2512 */
     if (E > 52) E = 52;
     if (E < 0) E = 0;
-    for (uint64_t i = 0; i < M; i++) {
-        h_mu[i] = (h_amax[i] == 0.0) ? 0 : E - h_mu[i];
-        if (h_mu[i] > 1023 || h_mu[i] < -1022) return -1;
-    }
-    for (uint64_t j = 0; j < N; j++) {
-        h_nu[j] = (h_bmax[j] == 0.0) ? 0 : E - h_nu[j];
-        if (h_nu[j] > 1023 || h_nu[j] < -1022) return -1;
-    }
-    if (!ESHKOL_HIP_OK(hipMemcpyAsync(dmu, h_mu, M * sizeof(int32_t), hipMemcpyHostToDevice, st))) return -1;
-    if (!ESHKOL_HIP_OK(hipMemcpyAsync(dnu, h_nu, N * sizeof(int32_t), hipMemcpyHostToDevice, st))) return -1;
+    /* every shift E - floor(log2 max) must be an exponent ldexp can apply exactly */
+    for (int o = 0; o < 2; o++)
+        if (any[o] && (E - e_min[o] > 1023 || E - e_max[o] < -1022)) return -1;
+    hipLaunchKernelGGL(crt_shift_kernel, dim3((unsigned)((M + N + 255) / 256)), dim3(256), 0, st, dmu, M, dnu, N, E);
 
     int8_t* Ap = (int8_t*)eshkol_hip_workspace(WS_APLANES, (size_t)num_moduli * Mp * ldk);
     int8_t* Bp = (int8_t*)eshkol_hip_workspace(WS_BPLANES, (size_t)num_moduli * Np * ldk);

@@ -23,47 +23,67 @@
 #include <cstring>
 
 typedef double d2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t v4u_t __attribute__((ext_vector_type(4)));
 
 namespace {
 
-/* gpu_cuda_kernels.cu:694-701 for two consecutive k of one row: one 16-bit
- * store per slice plane. */
-__device__ __forceinline__ void slice_pair(double x0, double x1, double sc, int s,
-                                           int8_t* out, uint64_t plane_stride) {
-    double r0 = x0 / sc, r1 = x1 / sc;
+/* gpu_cuda_kernels.cu:694-701 for G (2, 4 or 16) consecutive k of one row: one
+ * G-byte store per slice plane. */
+template <int G>
+__device__ __forceinline__ void slice_group(const double* x, double sc, int s, int8_t* out, uint64_t plane_stride) {
+    double r[G];
+#pragma unroll
+    for (int e = 0; e < G; e++) r[e] = x[e] / sc;
     for (int p = 0; p < s; p++) {
-        r0 *= 128.0; r1 *= 128.0;
-        double a0 = rint(r0), a1 = rint(r1);
-        if (a0 > 127.0) a0 = 127.0; else if (a0 < -127.0) a0 = -127.0;
-        if (a1 > 127.0) a1 = 127.0; else if (a1 < -127.0) a1 = -127.0;
-        const int i0 = (int)a0, i1 = (int)a1;
-        *(uint16_t*)(out + (uint64_t)p * plane_stride) =
-            (uint16_t)((uint8_t)(int8_t)i0 | ((uint16_t)(uint8_t)(int8_t)i1 << 8));
-        r0 -= a0; r1 -= a1;
+        uint32_t w[(G + 3) / 4];
+#pragma unroll
+        for (int e = 0; e < (G + 3) / 4; e++) w[e] = 0;
+#pragma unroll
+        for (int e = 0; e < G; e++) {
+            r[e] *= 128.0;
+            double a = rint(r[e]);
+            if (a > 127.0) a = 127.0; else if (a < -127.0) a = -127.0;
+            w[e / 4] |= (uint32_t)(uint8_t)(int8_t)(int)a << (8 * (e % 4));
+            r[e] -= a;
+        }
+        int8_t* o = out + (uint64_t)p * plane_stride;
+        if (G == 2) *(uint16_t*)o = (uint16_t)w[0];
+        else if (G == 4) *(uint32_t*)o = w[0];
+        else {
+            v4u_t v;
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = w[e % ((G + 3) / 4)];
+            *(v4u_t*)o = v;
+        }
     }
 }
 
-/* Row-major X[rows][K]. */
+/* Row-major X[rows][K]. One thread: G (2 or 4) consecutive k of one row; the
+ * wider form needs a pitch that is a multiple of 4. */
+template <int G>
 __global__ __launch_bounds__(256)
 void slice_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
                   const double* __restrict__ scale, int s, int8_t* __restrict__ planes,
                   uint64_t rows_padded, uint64_t ldk) {
-    const uint32_t cpr = (uint32_t)((ldk / 2 + 255) / 256);
+    const uint32_t cpr = (uint32_t)((ldk / G + 255) / 256);
     const uint64_t row = blockIdx.x / cpr;
-    const uint64_t k = ((uint64_t)(blockIdx.x % cpr) * 256 + threadIdx.x) * 2;
+    const uint64_t k = ((uint64_t)(blockIdx.x % cpr) * 256 + threadIdx.x) * G;
     if (k >= ldk) return;
-    double x0 = 0.0, x1 = 0.0, sc = 1.0;
+    double x[G], sc = 1.0;
+#pragma unroll
+    for (int e = 0; e < G; e++) x[e] = 0.0;
     if (row < rows) {
         sc = scale[row];
         const double* p = X + row * K + k;
-        if (k + 1 < K) {
-            if ((K & 1) == 0 && (((uintptr_t)X & 15) == 0)) { d2_t v = *(const d2_t*)p; x0 = v.x; x1 = v.y; }
-            else { x0 = p[0]; x1 = p[1]; }
-        } else if (k < K) {
-            x0 = p[0];
+        if (k + G <= K && (K & 1) == 0 && (((uintptr_t)X & 15) == 0)) {
+#pragma unroll
+            for (int e = 0; e < G; e += 2) { const d2_t v = *(const d2_t*)(p + e); x[e] = v.x; x[e + 1] = v.y; }
+        } else {
+#pragma unroll
+            for (int e = 0; e < G; e++) if (k + e < K) x[e] = p[e];
         }
     }
-    slice_pair(x0, x1, sc, s, planes + row * ldk + k, rows_padded * ldk);
+    slice_group<G>(x, sc, s, planes + row * ldk + k, rows_padded * ldk);
 }
 
 /* k-major X[K][rows] (B as the runtime stores it), same output: the job of the
@@ -75,39 +95,62 @@ void slice_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K
                          uint64_t rows_padded, uint64_t ldk) {
     __shared__ __align__(16) double tile[kmaj::SMEM_DOUBLES];
     const uint64_t plane_stride = rows_padded * ldk;
+    if ((ldk & 15) == 0 && (((uintptr_t)planes & 15) == 0)) {
+        kmaj::for_each_16(X, rows, K, rows_padded, ldk, 0xffffffffu, tile,
+            [&](uint64_t row) { return (row < rows) ? scale[row] : 1.0; },
+            [&](uint64_t row, uint64_t k, const double* x, double sc) {
+                slice_group<16>(x, sc, s, planes + row * ldk + k, plane_stride);
+            });
+        return;
+    }
     kmaj::for_each_pair(X, rows, K, rows_padded, ldk, 0xffffffffu, tile,
         [&](uint64_t row) { return (row < rows) ? scale[row] : 1.0; },
         [&](uint64_t row, uint64_t k, double x0, double x1, double sc) {
-            slice_pair(x0, x1, sc, s, planes + row * ldk + k, plane_stride);
+            const double x[2] = {x0, x1};
+            slice_group<2>(x, sc, s, planes + row * ldk + k, plane_stride);
         });
 }
 
-/* gpu_cuda_kernels.cu:728-741, two columns per thread. */
+/* gpu_cuda_kernels.cu:728-741, COLS (2 or 4) consecutive columns per thread; the
+ * wider form needs N to be a multiple of 4. The buffers of one element are read
+ * four at a time so that a wave keeps several kilobytes of loads in flight. */
+template <int COLS>
 __global__ __launch_bounds__(256)
 void reconstruct_kernel(double* __restrict__ C, const int32_t* __restrict__ Gall,
                         const double* __restrict__ weights, int nbuf,
                         const double* __restrict__ rmax, const double* __restrict__ cmax,
                         uint64_t M, uint64_t N) {
-    const uint32_t cpr = (uint32_t)(((N + 1) / 2 + 255) / 256);
+    typedef int32_t vec_t __attribute__((ext_vector_type(COLS)));
+    const uint32_t cpr = (uint32_t)(((N + COLS - 1) / COLS + 255) / 256);
     const uint64_t row = blockIdx.x / cpr;
-    const uint64_t col = ((uint64_t)(blockIdx.x % cpr) * 256 + threadIdx.x) * 2;
+    const uint64_t col = ((uint64_t)(blockIdx.x % cpr) * 256 + threadIdx.x) * COLS;
     if (col >= N) return;
     const uint64_t tot = M * N, idx = row * N + col;
-    const bool two = (col + 1 < N);
-    const bool vec = two && ((N & 1) == 0);
-    double acc0 = 0.0, acc1 = 0.0;
+    const int nvalid = (N - col < COLS) ? (int)(N - col) : COLS;
+    const bool vec = (nvalid == COLS) && (N % COLS == 0);
+    double acc[COLS];
+#pragma unroll
+    for (int e = 0; e < COLS; e++) acc[e] = 0.0;
+#pragma unroll 4
     for (int b = 0; b < nbuf; b++) {
         const int32_t* g = Gall + (uint64_t)b * tot + idx;
-        int32_t g0, g1 = 0;
-        if (vec) { const int2 v = *(const int2*)g; g0 = v.x; g1 = v.y; }
-        else { g0 = g[0]; if (two) g1 = g[1]; }
+        int32_t gv[COLS];
+        if (vec) {
+            const vec_t v = *(const vec_t*)g;
+#pragma unroll
+            for (int e = 0; e < COLS; e++) gv[e] = v[e];
+        } else {
+#pragma unroll
+            for (int e = 0; e < COLS; e++) gv[e] = (e < nvalid) ? g[e] : 0;
+        }
         const double w = weights[b];
-        acc0 = acc0 + w * (double)g0;
-        acc1 = acc1 + w * (double)g1;
+#pragma unroll
+        for (int e = 0; e < COLS; e++) acc[e] = acc[e] + w * (double)gv[e];
     }
     const double r = rmax[row];
-    C[idx] = (acc0 * r) * cmax[col];
-    if (two) C[idx + 1] = (acc1 * r) * cmax[col + 1];
+#pragma unroll
+    for (int e = 0; e < COLS; e++)
+        if (e < nvalid) C[idx + e] = (acc[e] * r) * cmax[col + e];
 }
 
 void* g_pinned = nullptr;
@@ -132,13 +175,17 @@ int slice_any(const double* X, uint64_t rows, uint64_t K, const double* scale, i
               int8_t* planes, uint64_t rows_padded, uint64_t ldk, bool kmajor, void* stream) {
     if (!X || !scale || !planes || rows == 0 || K == 0 || s < 1 || s > 16) return -1;
     if (rows_padded < rows || ldk < K || (ldk & 1)) return -1;
-    const uint64_t nblk = kmajor ? kmaj::grid_blocks(rows_padded, ldk, eshkol_hip_num_cus()) : ((ldk / 2 + 255) / 256) * rows_padded;
+    const int g = (ldk % 4 == 0 && ((uintptr_t)planes & 3) == 0) ? 4 : 2;
+    const uint64_t nblk = kmajor ? kmaj::grid_blocks(rows_padded, ldk, eshkol_hip_num_cus()) : ((ldk / g + 255) / 256) * rows_padded;
     if (nblk > 0x7fffffffULL || (kmajor && kmaj::tile_count(rows_padded, ldk) > 0x7fffffffULL)) return -1;
     if (kmajor)
         hipLaunchKernelGGL(slice_kmajor_kernel, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
                            X, rows, K, scale, s, planes, rows_padded, ldk);
+    else if (g == 4)
+        hipLaunchKernelGGL(slice_kernel<4>, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
+                           X, rows, K, scale, s, planes, rows_padded, ldk);
     else
-        hipLaunchKernelGGL(slice_kernel, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
+        hipLaunchKernelGGL(slice_kernel<2>, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
                            X, rows, K, scale, s, planes, rows_padded, ldk);
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
@@ -158,10 +205,15 @@ extern "C" int hip_ozaki_reconstruct_f64(double* C, const int32_t* Gall, const d
                                          const double* rmax, const double* cmax,
                                          uint64_t M, uint64_t N, void* stream) {
     if (!C || !Gall || !d_weights || !rmax || !cmax || nbuf < 1 || M == 0 || N == 0) return -1;
-    const uint64_t nblk = (((N + 1) / 2 + 255) / 256) * M;
+    const int cols = (N % 4 == 0 && ((uintptr_t)Gall & 15) == 0) ? 4 : 2;
+    const uint64_t nblk = (((N + cols - 1) / cols + 255) / 256) * M;
     if (nblk > 0x7fffffffULL) return -1;
-    hipLaunchKernelGGL(reconstruct_kernel, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
-                       C, Gall, d_weights, nbuf, rmax, cmax, M, N);
+    if (cols == 4)
+        hipLaunchKernelGGL(reconstruct_kernel<4>, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
+                           C, Gall, d_weights, nbuf, rmax, cmax, M, N);
+    else
+        hipLaunchKernelGGL(reconstruct_kernel<2>, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
+                           C, Gall, d_weights, nbuf, rmax, cmax, M, N);
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 

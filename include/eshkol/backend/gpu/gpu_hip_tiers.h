@@ -274,6 +274,14 @@ void hip_igemm_set_prefetch(int pf);
  * workgroup per tile. Same results; the switch exists to compare them. */
 void hip_igemm_set_persistent(int on);
 
+/* 0 (default): the CRT tier finds floor(log2) of the row and column maxima and
+ * the few maxima that can carry the largest fractional part of log2 on the
+ * device, and the host calls log2 on those few only; 1: the host takes log2 of
+ * every maximum, as gpu_memory.mm:376-420 does. Same E, shifts and results (the
+ * first falls back to the second whenever a maximum lies within 2^-40 of a power
+ * of two); the switch exists to compare them. */
+void hip_ozaki_crt_set_host_pass(int on);
+
 #ifdef __cplusplus
 }
 #endif

@@ -115,6 +115,29 @@ def test_slice_planes(gpu, K, R):
     assert not a[:, R:, :].any() and not a[:, :, K:].any()
 
 
+@pytest.mark.parametrize("K,R", [(7, 5), (130, 257), (300, 70), (1000, 513)])
+def test_slice_planes_at_any_even_pitch(gpu, K, R):
+    lib = ea.load()
+    X = synth.wide_range(5 * K + R, (K, R), -8, 8)
+    scale = np.abs(X).max(axis=0)
+    scale[scale == 0.0] = 1.0
+    dX, dXt, dsc = dev(X), dev(X.T), dev(scale)
+    want = None
+    for Rp, ldk in [(pad(R, 256), pad(K, 256)), (R, K + (K & 1)), (R + 3, K + (K & 1) + 2), (R + 1, pad(K, 4) + 4),
+                    (R, pad(K, 16)), (R + 2, pad(K, 16) + 16)]:
+        pa = ea.DeviceArray.from_host(np.full((7, Rp, ldk), 77, np.int8))
+        pb = ea.DeviceArray.from_host(np.full((7, Rp, ldk), 78, np.int8))
+        assert lib.hip_ozaki_slice_kmajor_f64(dX.ptr, R, K, dsc.ptr, 7, pa.ptr, Rp, ldk, stream()) == 0
+        assert lib.hip_ozaki_slice_f64(dXt.ptr, R, K, dsc.ptr, 7, pb.ptr, Rp, ldk, stream()) == 0
+        ea.synchronize()
+        a, b = pa.download(), pb.download()
+        assert np.array_equal(a, b), (Rp, ldk)
+        assert not a[:, R:, :].any() and not a[:, :, K:].any(), (Rp, ldk)
+        if want is None:
+            want = a[:, :R, :K].copy()
+        assert np.array_equal(a[:, :R, :K], want), (Rp, ldk)
+
+
 @pytest.mark.parametrize("K,R", SHAPES)
 @pytest.mark.parametrize("is_bf16", [0, 1])
 def test_narrowing(gpu, K, R, is_bf16):

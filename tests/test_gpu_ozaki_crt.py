@@ -136,3 +136,58 @@ def test_full_size_config3_sampled(gpu):
     assert np.array_equal(st["w_planes"][:, rows][:, :, cols], so["w_planes"])
     assert ulp_distance(Cg[rows][:, cols], so["C"]).max() <= MAX_ULP
     assert st["a_pad_clear"] and st["b_pad_clear"]
+
+
+def both_bookkeeping_paths(A, B, **kw):
+    """The device scan with a handful of host log2 calls, and the host pass over every
+    maximum, must give the same E, shifts, planes and result; returns the first."""
+    import eshkol_amd as ea
+    lib = ea.load()
+    fast = check_all_stages(A, B, **kw)
+    lib.hip_ozaki_crt_set_host_pass(1)
+    try:
+        rc, Ch, sh = run_crt(A, B, kw.get("num_moduli", 16), kw.get("adaptive", False))
+    finally:
+        lib.hip_ozaki_crt_set_host_pass(0)
+    assert rc == 0
+    so = fast[1]
+    assert sh["E"] == so["E"] and np.array_equal(sh["mu"], so["mu"]) and np.array_equal(sh["nu"], so["nu"])
+    assert np.array_equal(Ch, fast[0])
+    return fast
+
+
+def test_shift_bookkeeping_structured_maxima(gpu):
+    """Maxima that are powers of two, equal in every row, subnormal, or spread over a
+    hundred binades with one mantissa (more distinct candidates than the scan keeps)."""
+    rng = np.random.default_rng(11)
+    A = rng.standard_normal((130, 70)); B = rng.standard_normal((70, 90))
+    both_bookkeeping_paths(np.ones((40, 30)), np.full((30, 50), 0.5))
+    both_bookkeeping_paths(np.eye(64), np.eye(64) * 3.0)
+    As = A.copy(); As[5, :] = 0.0; As[6, :] *= 2.0 ** -900           # a zero row and a tiny one
+    both_bookkeeping_paths(As, B)
+    As[6, :] *= 2.0 ** -140                                           # a subnormal maximum: no shift reaches it
+    import eshkol_amd as ea
+    for host_pass in (0, 1):
+        ea.load().hip_ozaki_crt_set_host_pass(host_pass)
+        try:
+            assert run_crt(As, B)[0] == -1
+        finally:
+            ea.load().hip_ozaki_crt_set_host_pass(0)
+    Aw = A / np.abs(A).max(axis=1, keepdims=True) * 1.75             # every row maximum 1.75 ...
+    Aw *= 2.0 ** np.arange(-65, 65)[:, None]                         # ... in 130 different binades
+    both_bookkeeping_paths(Aw, B)
+    Bw = B / np.abs(B).max(axis=0, keepdims=True) * (1.0 + 2.0 ** -30)
+    Bw *= 2.0 ** rng.integers(-3, 4, 90)[None, :]                    # seven binades: few candidates
+    both_bookkeeping_paths(A, Bw)
+
+
+def test_shift_bookkeeping_mantissas_next_to_a_power_of_two(gpu):
+    """Within 2^-40 of a power of two libm may round log2 across the integer: the scan
+    must notice and leave such operands to the host pass. Results equal the oracle's."""
+    rng = np.random.default_rng(12)
+    A = rng.standard_normal((50, 40)); B = rng.standard_normal((40, 60))
+    for val in (np.nextafter(2.0, 0.0), np.nextafter(1.0, 2.0), 4.0 - 2.0 ** -45, 8.0 * (1.0 + 2.0 ** -50)):
+        Ax = A / np.abs(A).max() * 0.9; Ax[7, 3] = val
+        Bx = B / np.abs(B).max() * 0.9; Bx[5, 9] = -val
+        both_bookkeeping_paths(Ax, B)
+        both_bookkeeping_paths(A, Bx)
