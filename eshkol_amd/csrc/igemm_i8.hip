@@ -118,15 +118,17 @@ __device__ __forceinline__ void epilogue(const HipIgemmArgs& g, int o, int m0, i
     /* mode 1: residues modulo p, staged through LDS.
      * |sum| <= K * 128 * 128 <= 2^31. One fold of 2^20 into the modulus
      * (sum = hi 2^20 + lo, hi 2^20 = hi c20 mod p) leaves |x| < 2^21, exact in
-     * fp32; then the nearest multiple of p in fp32: x/p < 2^14 is known to
-     * within 1e-3 and, unless it is a tie, lies at least 1/(2p) >= 2e-3 from a
-     * half-integer, so q is the nearest integer and x - q p is exact and in
-     * [-p/2, p/2]. The tie (p = 256, +128) and -128 are the same int8 byte.
-     * About nine full-rate instructions per element: the epilogue is VALU
-     * time the matrix pipe sits idle for, so it is kept short. */
+     * fp32. One fma against 1.5 * 2^23 then rounds x/p to the nearest integer
+     * q and leaves 2^22 + q in the low 24 bits of the float: x/p < 2^14 is off
+     * by at most 7e-4 in the product and, unless it is a tie, lies at least
+     * 1/(2p) >= 2e-3 from a half-integer. x - (2^22 + q) p differs from the
+     * residue x - q p in [-p/2, p/2] by a multiple of 256, so its low byte is the
+     * int8 residue; the tie (p = 256, +-128) is the same byte either way.
+     * Six full-rate instructions per element after the accumulator read: the
+     * epilogue is VALU time the matrix pipe sits idle for, so it is kept short. */
     const int p = g.modulus[o];
     const int c20 = (1 << 20) % p;
-    const float pf = (float)p, pinv = 1.0f / (float)p;
+    const float pinv = 1.0f / (float)p;
     constexpr int EPITCH = BN + 16;
 #pragma unroll
     for (int t = 0; t < TM; t++) {
@@ -145,9 +147,8 @@ __device__ __forceinline__ void epilogue(const HipIgemmArgs& g, int o, int m0, i
                 for (int e = 0; e < 4; e++) {
                     const int s = acc[t][u][4 * v + e];
                     const int x = __mul24(s >> 20, c20) + (s & 0xfffff);
-                    const float xf = (float)x;
-                    const float q = rintf(xf * pinv);
-                    r[e] = (int)fmaf(-q, pf, xf);
+                    const float qm = fmaf((float)x, pinv, 12582912.0f);
+                    r[e] = __mul24(__float_as_int(qm), -p) + x;
                 }
                 /* low bytes of r[0..3] into one word */
                 const uint32_t lo2 = __builtin_amdgcn_perm((uint32_t)r[1], (uint32_t)r[0], 0x0c0c0400u);
