@@ -7,12 +7,15 @@
  *   block      256 threads = 2x2 waves; wave tile (TM*32) x (TN*32); k-block of
  *              128 bytes = 4 k-steps, so every global row segment is a whole
  *              128-byte line
- *   global     a register ring of PF k-blocks in flight: block g+PF is
- *              requested while block g is multiplied. The ring, not occupancy,
- *              hides the ~1.3 us a miss takes: the accumulators leave room for
- *              one wave per SIMD only.
- *   LDS        two buffers of [rows][128(+16)] bytes per operand; block g+1 is
- *              written during the second k-step of block g
+ *   global     a register ring of PF k-blocks in flight: block g+1+PF is
+ *              requested during the last two k-steps of block g (A's rows in
+ *              the third, B's in the fourth: sixteen requests in one k-step
+ *              queue up behind the address unit), into the ring slot the
+ *              second k-step has just emptied. The ring, not occupancy, hides
+ *              the ~1.3 us a miss takes: the accumulators leave room for one
+ *              wave per SIMD only.
+ *   LDS        two buffers, each [A rows][128(+16)] then [B rows][128(+16)]
+ *              bytes; block g+1 is written during the second k-step of block g
  *   fragments  double-buffered: the 16-byte LDS reads of k-step s+1 are issued
  *              between the MFMAs of k-step s (sched_group_barrier pins that
  *              interleaving; left alone the scheduler sinks each read next to
@@ -52,6 +55,8 @@ template <int TM, int TN> struct Cfg {
     static constexpr int B_CH = BN * BKB / 16 / NT;
 };
 
+template <int V> using IC = std::integral_constant<int, V>;
+
 template <int N, typename F>
 __device__ __forceinline__ void static_for(F&& f) {
     if constexpr (N > 0) {
@@ -79,8 +84,12 @@ struct Source {
  * one, so those loads are in flight while the tile's epilogue runs and the
  * next tile starts with its operands already in registers. What a workgroup
  * launch costs (dispatch, cold first loads, a drained pipe) is paid once.
- * Every tile must have at least 2 * PF k-blocks: the cursor runs PF blocks
- * ahead and learns about the tile after the next only when it gets there. */
+ * The cursor runs PF + 1 blocks ahead and the tile after the current one is
+ * always known; every tile must have at least max(2 PF, PF + 2) k-blocks so
+ * that the cursor has left a tile's index table before the table of the tile
+ * after the next replaces it. A tile's first block reaches LDS buffer 0 during
+ * the last block of the tile before it, so an epilogue that needs LDS takes
+ * buffer 1 (epilogue_stage). */
 struct Tile {
     int m0, n0;                 /* first row of the A planes / of the B planes */
     int tag;                    /* caller's: output plane */
@@ -98,15 +107,20 @@ template <int TM, int TN> struct TilesCfg {
 template <class Op, int TM, int TN, int PF, class Next, class Epi>
 __device__ __forceinline__ void run_tiles(int8_t* smem, const Source& cm, Next next_tile, Epi epilogue) {
     using C = Cfg<TM, TN>;
-    int8_t* As = smem;
-    int8_t* Bs = smem + 2 * C::A_TILE;
-    int32_t* table = (int32_t*)(smem + 2 * (C::A_TILE + C::B_TILE));      /* [2][2 * MAX_PAIRS] */
+    constexpr int BUF = C::A_TILE + C::B_TILE;                            /* LDS: [A0][B0][A1][B1][tables] */
+    int32_t* table = (int32_t*)(smem + 2 * BUF);                          /* [2][2 * MAX_PAIRS] */
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int li = lane & 31, lh = lane >> 5;
 
+    const int nkb_per = cm.ld / BKB;
+    const size_t g_off = (size_t)(tid >> 3) * cm.ld + (tid & 7) * 16;
+    const int s_off = (tid >> 3) * PITCH + (tid & 7) * 16;
+
+    /* The current tile and the one after it: the request cursor may cross into the
+     * next tile at any time, so that tile is always known one tile ahead. */
     Tile cur, nxt;
     if (!next_tile(cur)) return;
     int tab = 0;                                   /* table half that describes `cur` */
@@ -114,32 +128,45 @@ __device__ __forceinline__ void run_tiles(int8_t* smem, const Source& cm, Next n
         table[tid] = cur.a_idx ? cur.a_idx[tid] : 0;
         table[MAX_PAIRS + tid] = cur.b_idx ? cur.b_idx[tid] : 0;
     }
+    const int8_t* nx_a = nullptr;
+    const int8_t* nx_b = nullptr;
+    int nx_np = 1;
+    bool nx_has = false;
+    auto learn_next = [&]() {
+        nx_has = next_tile(nxt);
+        if (nx_has) {
+            if (tid < nxt.npairs) {
+                table[(tab ^ 1) * 2 * MAX_PAIRS + tid] = nxt.a_idx ? nxt.a_idx[tid] : 0;
+                table[(tab ^ 1) * 2 * MAX_PAIRS + MAX_PAIRS + tid] = nxt.b_idx ? nxt.b_idx[tid] : 0;
+            }
+            nx_a = cm.a_planes + (size_t)nxt.m0 * cm.ld + g_off;
+            nx_b = cm.b_planes + (size_t)nxt.n0 * cm.ld + g_off;
+            nx_np = nxt.npairs;
+        }
+    };
+    learn_next();
     __syncthreads();
-
-    const int nkb_per = cm.ld / BKB;
-    const size_t g_off = (size_t)(tid >> 3) * cm.ld + (tid & 7) * 16;
-    const int s_off = (tid >> 3) * PITCH + (tid & 7) * 16;
 
     /* request cursor */
     const int8_t* a_t = cm.a_planes + (size_t)cur.m0 * cm.ld + g_off;
     const int8_t* b_t = cm.b_planes + (size_t)cur.n0 * cm.ld + g_off;
     int gl_t = 0, gl_j = 0, gl_np = cur.npairs, gl_tab = 0;
     int v_ia = table[0], v_ib = table[MAX_PAIRS];
-    /* where the cursor goes after the current tile */
-    const int8_t* nx_a = a_t;
-    const int8_t* nx_b = b_t;
-    int nx_np = 1;
-    bool nx_has = false;
 
     v4i_t ra[PF][C::A_CH], rb[PF][C::B_CH];
-    auto gload = [&](auto slot) {
+    /* One k-block is requested in two halves, A's rows and then B's, in two
+     * consecutive k-steps; the cursor moves on after the second. */
+    auto gload_a = [&](auto slot) {
         constexpr int S = decltype(slot)::value;
         const int ia = __builtin_amdgcn_readfirstlane(v_ia);
-        const int ib = __builtin_amdgcn_readfirstlane(v_ib);
         const int8_t* ap = a_t + (size_t)ia * cm.a_plane_stride + (size_t)gl_j * BKB;
-        const int8_t* bp = b_t + (size_t)ib * cm.b_plane_stride + (size_t)gl_j * BKB;
 #pragma unroll
         for (int r = 0; r < C::A_CH; r++) ra[S][r] = *(const v4i_t*)(ap + (size_t)(32 * r) * cm.ld);
+    };
+    auto gload_b = [&](auto slot) {
+        constexpr int S = decltype(slot)::value;
+        const int ib = __builtin_amdgcn_readfirstlane(v_ib);
+        const int8_t* bp = b_t + (size_t)ib * cm.b_plane_stride + (size_t)gl_j * BKB;
 #pragma unroll
         for (int r = 0; r < C::B_CH; r++) rb[S][r] = *(const v4i_t*)(bp + (size_t)(32 * r) * cm.ld);
         /* advance: next k-block, next product, next tile; with no next tile the
@@ -159,8 +186,8 @@ __device__ __forceinline__ void run_tiles(int8_t* smem, const Source& cm, Next n
     };
     auto sstore = [&](int buf, auto slot) {
         constexpr int S = decltype(slot)::value;
-        int8_t* ad = As + buf * C::A_TILE + s_off;
-        int8_t* bd = Bs + buf * C::B_TILE + s_off;
+        int8_t* ad = smem + buf * BUF + s_off;
+        int8_t* bd = ad + C::A_TILE;
 #pragma unroll
         for (int r = 0; r < C::A_CH; r++) *(v4i_t*)(ad + 32 * r * PITCH) = ra[S][r];
 #pragma unroll
@@ -169,12 +196,12 @@ __device__ __forceinline__ void run_tiles(int8_t* smem, const Source& cm, Next n
 
     v4i_t fa[2][TM], fb[2][TN];
     const int a_frag_off = (wm * TM * 32 + li) * PITCH + lh * 16;
-    const int b_frag_off = (wn * TN * 32 + li) * PITCH + lh * 16;
+    const int b_frag_off = C::A_TILE + (wn * TN * 32 + li) * PITCH + lh * 16;
     typename Op::acc_t acc[TM][TN];
     auto ldfrag = [&](int buf, int ks, auto which) {
         constexpr int W = decltype(which)::value;
-        const int8_t* ab = As + buf * C::A_TILE + a_frag_off + ks * 32;
-        const int8_t* bb = Bs + buf * C::B_TILE + b_frag_off + ks * 32;
+        const int8_t* ab = smem + buf * BUF + a_frag_off + ks * 32;
+        const int8_t* bb = smem + buf * BUF + b_frag_off + ks * 32;
 #pragma unroll
         for (int t = 0; t < TM; t++) fa[W][t] = *(const v4i_t*)(ab + t * 32 * PITCH);
 #pragma unroll
@@ -187,53 +214,45 @@ __device__ __forceinline__ void run_tiles(int8_t* smem, const Source& cm, Next n
 #pragma unroll
             for (int u = 0; u < TN; u++) Op::mfma(fb[W][u], fa[W][t], acc[t][u]);
     };
-    using I0 = std::integral_constant<int, 0>;
-    using I1 = std::integral_constant<int, 1>;
+    using I0 = IC<0>;
+    using I1 = IC<1>;
     constexpr int NM = TM * TN, NF = TM + TN;
 
-    /* the first tile's first PF blocks; later tiles find theirs already requested */
-    static_for<PF>([&](auto s) { gload(s); });
+    /* Start of the stream: block 0 into LDS buffer 0, blocks 1..PF into the ring
+     * (block j in slot j % PF). Every later tile finds the same state: its block
+     * 0 was written to buffer 0 during the last block of the tile before it. */
+    static_for<PF>([&](auto s) { gload_a(s); gload_b(s); });
+    sstore(0, I0{});
+    gload_a(I0{});
+    gload_b(I0{});
 
     for (;;) {
-        /* learn the next tile and park its index table in the other half */
-        nx_has = next_tile(nxt);
-        if (nx_has) {
-            if (tid < nxt.npairs) {
-                table[(tab ^ 1) * 2 * MAX_PAIRS + tid] = nxt.a_idx ? nxt.a_idx[tid] : 0;
-                table[(tab ^ 1) * 2 * MAX_PAIRS + MAX_PAIRS + tid] = nxt.b_idx ? nxt.b_idx[tid] : 0;
-            }
-            nx_a = cm.a_planes + (size_t)nxt.m0 * cm.ld + g_off;
-            nx_b = cm.b_planes + (size_t)nxt.n0 * cm.ld + g_off;
-            nx_np = nxt.npairs;
-        }
 #pragma unroll
         for (int t = 0; t < TM; t++)
 #pragma unroll
             for (int u = 0; u < TN; u++) Op::zero(acc[t][u]);
 
         const int nkb = cur.npairs * nkb_per;      /* even: the row pitch is a multiple of 2 * BKB */
-        sstore(0, I0{});
-        lds_barrier();                             /* also publishes the parked table */
+        lds_barrier();                             /* block 0 and the parked table are visible */
         ldfrag(0, 0, I0{});
 
         for (int g0 = 0; g0 < nkb; g0 += PF) {
             static_for<PF>([&](auto s) {
                 constexpr int S = decltype(s)::value;
+                using NextSlot = IC<(S + 1) % PF>;           /* holds block g+1, then block g+1+PF */
                 const int cb = (g0 + S) & 1;
 
                 ldfrag(cb, 1, I1{});
-                gload(s);
                 mfma_all(I0{});
 #pragma unroll
                 for (int i = 0; i < NM; i++) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                     if (i < NF) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                    if (i < C::A_CH + C::B_CH) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
 
                 ldfrag(cb, 2, I0{});
-                sstore(cb ^ 1, std::integral_constant<int, (S + 1) % PF>{});
+                sstore(cb ^ 1, NextSlot{});
                 mfma_all(I1{});
 #pragma unroll
                 for (int i = 0; i < NM; i++) {
@@ -244,33 +263,46 @@ __device__ __forceinline__ void run_tiles(int8_t* smem, const Source& cm, Next n
                 __builtin_amdgcn_sched_barrier(0);
 
                 ldfrag(cb, 3, I1{});
+                gload_a(NextSlot{});
                 mfma_all(I0{});
 #pragma unroll
                 for (int i = 0; i < NM; i++) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                     if (i < NF) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    if (i >= NF && i - NF < C::A_CH) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 lds_barrier();
 
                 ldfrag(cb ^ 1, 0, I0{});
+                gload_b(NextSlot{});
                 mfma_all(I1{});
 #pragma unroll
                 for (int i = 0; i < NM; i++) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                     if (i < NF) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    if (i >= NF && i - NF < C::B_CH) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             });
         }
-        lds_barrier();                 /* every wave is done with the LDS tiles */
-        epilogue(acc, cur);
+        lds_barrier();                 /* every wave is done with LDS buffer 1 */
+        epilogue(acc, cur);            /* may stage in buffer 1 (epilogue_stage): buffer 0 holds the next tile's block 0 */
         if (!nx_has) break;
-        lds_barrier();                 /* the epilogue's LDS staging has been read */
         cur = nxt;
         tab ^= 1;
+        learn_next();                  /* parks the table in the half the cursor has left behind */
     }
 }
+
+/* LDS an epilogue may use while the stream continues: the second operand buffer. */
+template <int TM, int TN>
+__device__ __forceinline__ int8_t* epilogue_stage(int8_t* smem) {
+    return smem + Cfg<TM, TN>::A_TILE + Cfg<TM, TN>::B_TILE;
+}
+template <int TM, int TN> struct StageCfg {
+    static constexpr int BYTES = Cfg<TM, TN>::A_TILE + Cfg<TM, TN>::B_TILE;
+};
 
 }  // namespace pipe
 #endif

@@ -206,7 +206,7 @@ void igemm_i8_pipe_kernel(HipIgemmArgs g, int tiles_m, int tiles_n, int chunk) {
         return true;
     };
     auto epi = [&](v16i_t (&acc)[TM][TN], const pipe::Tile& t) {
-        epilogue<TM, TN>(g, t.tag, t.m0, t.n0, acc, smem_i8);
+        epilogue<TM, TN>(g, t.tag, t.m0, t.n0, acc, pipe::epilogue_stage<TM, TN>(smem_i8));
     };
     pipe::run_tiles<I8Op, TM, TN, PF>(smem_i8, cm, next_tile, epi);
 }
@@ -243,7 +243,7 @@ void igemm_i8_persistent_kernel(HipIgemmArgs g, int tiles_m, int tiles_n, int ch
         return false;
     };
     auto epi = [&](v16i_t (&acc)[TM][TN], const pipe::Tile& t) {
-        epilogue<TM, TN>(g, t.tag, t.m0, t.n0, acc, smem_i8);
+        epilogue<TM, TN>(g, t.tag, t.m0, t.n0, acc, pipe::epilogue_stage<TM, TN>(smem_i8));
     };
     pipe::run_tiles<I8Op, TM, TN, PF>(smem_i8, cm, next_tile, epi);
 }
@@ -363,6 +363,7 @@ template <int PF>
 int launch_pipe(const HipIgemmArgs& a, hipStream_t st) {
     using C = pipe::Cfg<4, 4>;
     constexpr int EPI = C::BM * (C::BN + 16);
+    static_assert(EPI <= pipe::StageCfg<4, 4>::BYTES, "the epilogue stages its tile in one LDS operand buffer");
     constexpr int MAIN = pipe::TilesCfg<4, 4>::SMEM_MAIN;
     constexpr int SMEM = MAIN > EPI ? MAIN : EPI;
     static bool attr_set = false;
@@ -373,6 +374,7 @@ template <int PF>
 int launch_persistent(const HipIgemmArgs& a, hipStream_t st) {
     using C = pipe::Cfg<4, 4>;
     constexpr int EPI = C::BM * (C::BN + 16);
+    static_assert(EPI <= pipe::StageCfg<4, 4>::BYTES, "the epilogue stages its tile in one LDS operand buffer");
     constexpr int MAIN = pipe::TilesCfg<4, 4>::SMEM_MAIN;
     constexpr int SMEM = MAIN > EPI ? MAIN : EPI;
     static bool attr_set = false;
@@ -433,9 +435,9 @@ extern "C" int hip_igemm_i8(const HipIgemmArgs* args, void* stream) {
     int pf = g_prefetch;
     while (pf > 0 && a.ldk % (128u * pf) != 0) pf--;
     if (pf > 0 && big >= 128 && a.max_pairs >= 1 && a.max_pairs <= pipe::MAX_PAIRS) {
-        /* the persistent kernel's request cursor may not reach the end of a tile
-         * before the tile after it is known: more than PF blocks per tile */
-        if (g_persistent && a.ldk >= 256u * pf) {
+        /* the persistent kernel's request cursor must have left a tile before the
+         * tile after the next is announced: max(2 PF, PF + 2) blocks per tile */
+        if (g_persistent && a.ldk >= 128u * (unsigned)(2 * pf > pf + 2 ? 2 * pf : pf + 2)) {
             switch (pf) {
                 case 1: return launch_persistent<1>(a, st);
                 case 2: return launch_persistent<2>(a, st);
