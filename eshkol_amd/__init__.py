@@ -127,6 +127,7 @@ SIGNATURES = {
     "hip_convert_f64_to_16": (C.c_int, [vp, vp, u64, u64, u64, u64, C.c_int, vp]),
     "hip_probe_peak": (C.c_int, [C.c_int, C.c_int, dp, vp]),
     "hip_igemm_set_persistent": (None, [C.c_int]),
+    "hip_dgemm_set_tail_split": (None, [C.c_int]),
     "hip_ozaki_crt_set_host_pass": (None, [C.c_int]),
     "hip_igemm_set_prefetch": (None, [C.c_int]),
 }

@@ -127,11 +127,9 @@ template <int R, bool KMAJ, bool VEC, bool LK = KMAJ> struct Operand {
     }
 };
 
-__device__ __forceinline__ void tile_of_workgroup(int tiles_m, int tiles_n, int* tm, int* tn) {
-    const int nwg = gridDim.x, wg = blockIdx.x;
-    const int q = nwg >> 3, r = nwg & 7;
-    const int xcd = wg & 7, seq = wg >> 3;
-    const int L = xcd * q + (xcd < r ? xcd : r) + seq;
+/* Position L in the tile order -> tile: groups of eight tile rows, the row index
+ * running fastest inside a group. */
+__device__ __forceinline__ void tile_of_index(int L, int tiles_m, int tiles_n, int* tm, int* tn) {
     const int GM = 8;
     const int width = GM * tiles_n;
     const int group = L / width;
@@ -140,6 +138,16 @@ __device__ __forceinline__ void tile_of_workgroup(int tiles_m, int tiles_n, int*
     const int in_group = L - group * width;
     *tm = first_m + in_group % gsize;
     *tn = in_group / gsize;
+}
+
+/* Workgroup -> position in the tile order: XCD x (workgroups x, x+8, ...) takes
+ * the x-th eighth of the launch's positions, so neighbours in the order share an L2. */
+__device__ __forceinline__ void tile_of_workgroup(int tiles_m, int tiles_n, int* tm, int* tn) {
+    const int nwg = gridDim.x, wg = blockIdx.x;
+    const int q = nwg >> 3, r = nwg & 7;
+    const int xcd = wg & 7, seq = wg >> 3;
+    const int L = xcd * q + (xcd < r ? xcd : r) + seq;
+    tile_of_index(L, tiles_m, tiles_n, tm, tn);
 }
 
 /* C[MxN] = op(A) * op(B). TA: A is stored as its transpose [K][M]; TB: B is
@@ -261,11 +269,17 @@ __device__ __forceinline__ void lds_only_barrier() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-template <bool TA, bool TB, bool KTAIL>
+/* SPLIT: the launch covers the last `tail` tiles of the tile order, each cut
+ * along k into pieces of kb_per_piece k-blocks; workgroup piece * tail + i
+ * multiplies piece `piece` of tail tile i and leaves the whole 128 x 128 partial
+ * tile in `partial` (dgemm_fixup_kernel adds the pieces up in order). */
+struct SplitArgs { int first_tile, tail, kb_per_piece; double* partial; };
+
+template <bool TA, bool TB, bool KTAIL, bool SPLIT>
 __global__ __launch_bounds__(256, 2)
 void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ B,
                        double* __restrict__ C, int M, int N, int K,
-                       int tiles_m, int tiles_n) {
+                       int tiles_m, int tiles_n, SplitArgs sp) {
     constexpr int BM = 128, BN = 128;
     using OpA = Operand<BM, TA, true, true>;
     using OpB = Operand<BN, !TB, true, true>;
@@ -279,7 +293,8 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
     C += (size_t)blockIdx.y * M * N;
 
     int tm, tn;
-    tile_of_workgroup(tiles_m, tiles_n, &tm, &tn);
+    if (SPLIT) tile_of_index(sp.first_tile + (int)(blockIdx.x % (unsigned)sp.tail), tiles_m, tiles_n, &tm, &tn);
+    else tile_of_workgroup(tiles_m, tiles_n, &tm, &tn);
     const int m0 = tm * BM, n0 = tn * BN;
 
     const int tid = threadIdx.x;
@@ -372,18 +387,22 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
                 acc[t][u] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[W][t], bf[W][u], acc[t][u], 0, 0, 0);
     };
 
-    const int nkb = (K + BK - 1) / BK;
-    gload(0);
+    /* this workgroup's k-blocks [kb_lo, kb_hi): all of them unless the tile is split */
+    const int nkb_all = (K + BK - 1) / BK;
+    const int piece = SPLIT ? (int)(blockIdx.x / (unsigned)sp.tail) : 0;
+    const int kb_lo = SPLIT ? piece * sp.kb_per_piece : 0;
+    const int kb_hi = SPLIT ? ((kb_lo + sp.kb_per_piece < nkb_all) ? kb_lo + sp.kb_per_piece : nkb_all) : nkb_all;
+    gload(kb_lo);
     a.sstore(As, tid);
     b.sstore(Bs, tid);
-    gload(nkb > 1 ? 1 : 0);
+    gload(kb_hi - kb_lo > 1 ? kb_lo + 1 : kb_lo);
     __syncthreads();
     ldfrag(0, 0, I0{});
 
-    for (int kb = 0; kb < nkb; kb++) {
-        const int cur = kb & 1;
+    for (int kb = kb_lo; kb < kb_hi; kb++) {
+        const int cur = (kb - kb_lo) & 1;
         /* the block after next, clamped: requests past the end are never consumed */
-        const int kb2 = (kb + 2 < nkb) ? kb + 2 : nkb - 1;
+        const int kb2 = (kb + 2 < kb_hi) ? kb + 2 : kb_hi - 1;
 
         ldfrag(cur, 1, I1{});
         mfma_step(I0{});
@@ -428,6 +447,17 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
         __builtin_amdgcn_sched_barrier(0);
     }
 
+    if (SPLIT) {
+        double* out = sp.partial + (size_t)blockIdx.x * (BM * BN);
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    out[(wm * 64 + t * 16 + 4 * r + lg) * BN + wn * 64 + u * 16 + li] = acc[t][u][r];
+        return;
+    }
 #pragma unroll
     for (int t = 0; t < 4; t++)
 #pragma unroll
@@ -441,22 +471,86 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
         }
 }
 
+/* Adds up the partial tiles of dgemm_fast_kernel<..., SPLIT>: piece 0 first, so the
+ * result does not depend on which workgroup finished when. grid (tail, 16): a
+ * workgroup sums eight rows of one tile, a thread four consecutive columns. */
+__global__ __launch_bounds__(256)
+void dgemm_fixup_kernel(const double* __restrict__ partial, int tail, int pieces, int first_tile,
+                        int tiles_m, int tiles_n, double* __restrict__ C, int M, int N) {
+    int tm, tn;
+    tile_of_index(first_tile + (int)blockIdx.x, tiles_m, tiles_n, &tm, &tn);
+    const int lrow = (int)blockIdx.y * 8 + (threadIdx.x >> 5), lcol = 4 * (threadIdx.x & 31);
+    const double* p = partial + (size_t)blockIdx.x * (128 * 128) + lrow * 128 + lcol;
+    d2_t s0 = *(const d2_t*)p, s1 = *(const d2_t*)(p + 2);
+    for (int q = 1; q < pieces; q++) {
+        const double* pq = p + (size_t)q * tail * (128 * 128);
+        const d2_t v0 = *(const d2_t*)pq, v1 = *(const d2_t*)(pq + 2);
+        s0.x += v0.x; s0.y += v0.y; s1.x += v1.x; s1.y += v1.y;
+    }
+    const int row = tm * 128 + lrow, col = tn * 128 + lcol;
+    if (row >= M) return;
+    double* c = C + (size_t)row * N + col;
+    if (col < N) c[0] = s0.x;
+    if (col + 1 < N) c[1] = s0.y;
+    if (col + 2 < N) c[2] = s1.x;
+    if (col + 3 < N) c[3] = s1.y;
+}
+
+int g_tail_split = 1;
+
 template <bool TA, bool TB, bool KTAIL>
 int launch_fast_k(const double* A, const double* B, double* C, int M, int N, int K, int batch, hipStream_t st) {
     constexpr int SMEM_BYTES = 2 * (Operand<128, TA, true, true>::TILE + Operand<128, !TB, true, true>::TILE)
                                * (int)sizeof(double);
     static bool attr_set = false;
-    auto kern = dgemm_fast_kernel<TA, TB, KTAIL>;
+    auto kern = dgemm_fast_kernel<TA, TB, KTAIL, false>;
+    auto kern_split = dgemm_fast_kernel<TA, TB, KTAIL, true>;
     if (!attr_set) {
         if (!ESHKOL_HIP_OK(hipFuncSetAttribute((const void*)kern,
+                hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES))) return -1;
+        if (!ESHKOL_HIP_OK(hipFuncSetAttribute((const void*)kern_split,
                 hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES))) return -1;
         attr_set = true;
     }
     const int tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
     const long long nwg = (long long)tiles_m * tiles_n;
     if (nwg > 0x7fffffffLL || batch < 1 || batch > 65535) return -1;
+    SplitArgs sp = {0, 1, 0, nullptr};
+
+    /* Two workgroups fit on a CU, so a launch runs in rounds of `slots` tiles, and
+     * a last round of a few tiles takes as long as a full one. Its tiles are
+     * therefore cut along k into p pieces each: p * tail workgroups of 1/p the
+     * length, in ceil(p * tail / slots) short rounds (5000^3: 1600 tiles on 512
+     * slots, 4.4 -> 4.0 ms; 7680^3: 13.7 -> 12.5 ms). p minimises that time plus
+     * a small charge per piece for the extra prologues and the workspace traffic;
+     * the pieces go through a workspace and are added in a fixed order. */
+    const int slots = 2 * eshkol_hip_num_cus();
+    const int tail = (int)(nwg % slots), nkb = (K + BK - 1) / BK;
+    if (g_tail_split && batch == 1 && nwg > slots && tail > 0) {
+        int best_p = 1;
+        double best = 1.0;
+        for (int p = 2; p <= 32 && nkb / p >= 4; p++) {
+            const long long rounds = ((long long)p * tail + slots - 1) / slots;
+            const double cost = (double)rounds / p + 0.006 * p;
+            if (cost < best - 1e-9) { best = cost; best_p = p; }
+        }
+        const int kbpp = (nkb + best_p - 1) / best_p;
+        const int pieces = (nkb + kbpp - 1) / kbpp;
+        double* ws = (best < 0.9 && pieces >= 2) ? (double*)eshkol_hip_workspace(WS_DGEMM_PARTIAL,
+                                         (size_t)tail * pieces * 128 * 128 * sizeof(double)) : nullptr;
+        if (ws) {
+            sp.first_tile = (int)(nwg - tail); sp.tail = tail; sp.kb_per_piece = kbpp; sp.partial = ws;
+            hipLaunchKernelGGL(kern, dim3((unsigned)(nwg - tail), 1), dim3(256), SMEM_BYTES, st,
+                               A, B, C, M, N, K, tiles_m, tiles_n, sp);
+            hipLaunchKernelGGL(kern_split, dim3((unsigned)(tail * pieces), 1), dim3(256), SMEM_BYTES, st,
+                               A, B, C, M, N, K, tiles_m, tiles_n, sp);
+            hipLaunchKernelGGL(dgemm_fixup_kernel, dim3((unsigned)tail, 16), dim3(256), 0, st,
+                               ws, tail, pieces, sp.first_tile, tiles_m, tiles_n, C, M, N);
+            return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+        }
+    }
     hipLaunchKernelGGL(kern, dim3((unsigned)nwg, (unsigned)batch), dim3(256), SMEM_BYTES, st,
-                       A, B, C, M, N, K, tiles_m, tiles_n);
+                       A, B, C, M, N, K, tiles_m, tiles_n, sp);
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 
@@ -542,6 +636,8 @@ int dgemm_any(const double* A, const double* B, double* C, uint64_t M, uint64_t 
 
 /* 0 routes every shape through the bounds-checked kernel (for comparisons). */
 extern "C" void hip_dgemm_set_fast_path(int on) { g_fast_path = on ? 1 : 0; }
+/* 0 keeps every tile whole (results then equal the bounds-checked kernel's bit for bit). */
+extern "C" void hip_dgemm_set_tail_split(int on) { g_tail_split = on ? 1 : 0; }
 
 extern "C" int hip_dgemm_f64_ex(const double* A, const double* B, double* C,
                                 uint64_t M, uint64_t K, uint64_t N,

@@ -35,6 +35,7 @@ enum {
     WS_HALF_B,
     WS_F32_C,
     WS_COLPARTIAL,  /* per-slice partial column maxima                       */
+    WS_DGEMM_PARTIAL, /* partial tiles of a k-split last round of the fp64 GEMM */
     WS_MISC,
     WS_COUNT
 };

@@ -266,6 +266,13 @@ int hip_probe_peak(int kind, int random_operands, double* rate, void* stream);
  * the switch exists to compare them. */
 void hip_dgemm_set_fast_path(int on);
 
+/* 1 (default): when the last round of 128 x 128 tiles of a large product would
+ * leave more than half of the CUs idle, those tiles are cut along k, the pieces
+ * multiplied side by side and added in a fixed order (deterministic, but the
+ * summation order of those tiles differs from an unsplit launch); 0: every tile
+ * is multiplied whole. */
+void hip_dgemm_set_tail_split(int on);
+
 /* k-blocks kept in flight by the pipelined int8 kernel (1..3; 0 = simple kernel only). */
 void hip_igemm_set_prefetch(int pf);
 

@@ -106,6 +106,7 @@ def test_straight_line_kernel_matches_bounds_checked_kernel_bitwise(gpu, M, K, N
         try:
             for fast in (0, 1):
                 lib.hip_dgemm_set_fast_path(fast)
+                lib.hip_dgemm_set_tail_split(0)
                 guard = np.full((M + 2, N), np.nan)
                 guard[0] = guard[-1] = 12345.0
                 dC = ea.DeviceArray.from_host(guard)
@@ -116,6 +117,7 @@ def test_straight_line_kernel_matches_bounds_checked_kernel_bitwise(gpu, M, K, N
                 outs.append(got[1:-1])
         finally:
             lib.hip_dgemm_set_fast_path(1)
+            lib.hip_dgemm_set_tail_split(1)
         assert np.array_equal(outs[0], outs[1]), (ta, tb)
         if ref is not None:
             assert normwise(outs[1], ref, A, B) <= TOL
@@ -133,3 +135,44 @@ def test_straight_line_kernel_in_a_batch(gpu):
     got = dc.download()
     for i in range(bt):
         assert normwise(got[i], oracle.matmul_f64(a[i], b[i]), a[i], b[i]) <= TOL
+
+
+@pytest.mark.parametrize("M,K,N", [(3072, 256, 3072), (3072, 1000, 3072), (3000, 520, 3100), (3200, 160, 3072),
+                                   (2944, 4100, 3060)])
+def test_k_split_last_round(gpu, M, K, N):
+    """More than one round of tiles with a nearly empty last round: those tiles are cut
+    along k and the pieces added in a fixed order. Same result on every run, the tiles
+    of the full rounds bit-identical to an unsplit launch, everything within the tier's
+    bound, nothing stored outside C; for all three operand forms."""
+    import eshkol_amd as ea
+    from gpu_util import stream
+    lib = ea.load()
+    A, B = synth.normal(M + 3 * K, (M, K)), synth.normal(K + 3 * N, (K, N))
+    ref = oracle.matmul_f64(A, B) if M * K * N <= 2 ** 33 else None
+    forms = [(A, B, 0, 0), (A, np.ascontiguousarray(B.T), 0, 1), (np.ascontiguousarray(A.T), B, 1, 0)]
+    for X, Y, ta, tb in forms:
+        dX, dY = ea.DeviceArray.from_host(X), ea.DeviceArray.from_host(Y)
+        outs = []
+        try:
+            for split in (0, 1, 1):
+                lib.hip_dgemm_set_tail_split(split)
+                guard = np.full((M + 2, N), np.nan)
+                guard[0] = guard[-1] = 12345.0
+                dC = ea.DeviceArray.from_host(guard)
+                assert lib.hip_dgemm_f64_ex(dX.ptr, dY.ptr, dC.ptr + N * 8, M, K, N, ta, tb, stream()) == 0
+                ea.synchronize()
+                got = dC.download()
+                assert np.all(got[0] == 12345.0) and np.all(got[-1] == 12345.0)
+                outs.append(got[1:-1])
+        finally:
+            lib.hip_dgemm_set_tail_split(1)
+        whole, cut, again = outs
+        assert np.array_equal(cut, again), (ta, tb)
+        same = (whole == cut)
+        assert not same.all(), "the launch was expected to split its last round"
+        assert same.mean() > 0.5                      # the full rounds are untouched
+        assert np.isfinite(cut).all()
+        if ref is not None:
+            assert normwise(cut, ref, A, B) <= TOL, (ta, tb)
+        else:
+            assert np.abs(cut - whole).max() <= 1e-11 * np.sqrt(K)
