@@ -25,6 +25,8 @@
 #include "kernels.h"
 #include "kmajor_tile.h"
 
+#include <atomic>
+#include <chrono>
 #include <climits>
 #include <cmath>
 #include <cstring>
@@ -346,6 +348,8 @@ struct CrtScan {
     unsigned long long mant_max;
     int32_t nonfinite, extreme, nonzero, e_min, e_max, ncand;
     double cand[SCAN_CAND];
+    uint32_t ready;             /* the launch's ticket, written last */
+    uint32_t pad;
 };
 
 /* m > 0 finite -> exponent e = floor(log2 m) and mantissa n in [2^52, 2^53), m = n 2^(e-52) */
@@ -360,7 +364,7 @@ __device__ __forceinline__ void decode_positive(double m, int* e, unsigned long 
 /* block 0: the M row maxima of A; block 1: the N maxima of B */
 __global__ __launch_bounds__(SCAN_THREADS)
 void crt_scan_kernel(const double* __restrict__ amax, uint64_t M, const double* __restrict__ bmax, uint64_t N,
-                     int32_t* __restrict__ fl_a, int32_t* __restrict__ fl_b, CrtScan* __restrict__ out) {
+                     int32_t* __restrict__ fl_a, int32_t* __restrict__ fl_b, CrtScan* out, uint32_t ticket) {
     __shared__ unsigned long long s_max, keys[256];
     __shared__ int s_nonfinite, s_extreme, s_nonzero, s_emin, s_emax, s_ncand;
     const double* x = blockIdx.x ? bmax : amax;
@@ -454,10 +458,15 @@ void crt_scan_kernel(const double* __restrict__ amax, uint64_t M, const double* 
             }
         }
     }
+    /* `out` is host memory the CPU is polling: every thread's candidate stores must
+     * be out before the ticket that announces them */
+    __threadfence_system();
     __syncthreads();
     if (tid == 0) {
         o->mant_max = s_max; o->nonfinite = s_nonfinite; o->extreme = s_extreme; o->nonzero = s_nonzero;
         o->e_min = s_emin; o->e_max = s_emax; o->ncand = s_ncand;
+        __threadfence_system();
+        *(volatile uint32_t*)&o->ready = ticket;
     }
 }
 
@@ -533,6 +542,40 @@ void* pinned(size_t bytes) {
     if (!ESHKOL_HIP_OK(hipHostMalloc(&g_pinned, bytes, hipHostMallocDefault))) return nullptr;
     g_pinned_bytes = bytes;
     return g_pinned;
+}
+
+/* The scan's result goes straight into pinned host memory that the device can
+ * write (no copy command, no stream synchronisation: those cost 25 us of GPU idle
+ * time per call, a tenth of a small layer). The host polls the ticket the kernel
+ * writes last and falls back to a stream synchronisation if it does not show. */
+CrtScan* g_mailbox = nullptr;         /* host address; [2] */
+CrtScan* g_mailbox_dev = nullptr;     /* the same memory as the device sees it */
+uint32_t g_ticket = 0;
+bool ensure_mailbox() {
+    if (g_mailbox) return true;
+    void* h = nullptr;
+    void* d = nullptr;
+    if (!ESHKOL_HIP_OK(hipHostMalloc(&h, 2 * sizeof(CrtScan), hipHostMallocMapped))) return false;
+    if (!ESHKOL_HIP_OK(hipHostGetDevicePointer(&d, h, 0))) { (void)hipHostFree(h); return false; }
+    memset(h, 0, 2 * sizeof(CrtScan));
+    g_mailbox = (CrtScan*)h; g_mailbox_dev = (CrtScan*)d;
+    return true;
+}
+/* 0 when both halves carry `ticket` */
+int await_mailbox(uint32_t ticket, hipStream_t st) {
+    volatile uint32_t* r0 = &g_mailbox[0].ready;
+    volatile uint32_t* r1 = &g_mailbox[1].ready;
+    const auto t0 = std::chrono::steady_clock::now();
+    for (unsigned spin = 0; *r0 != ticket || *r1 != ticket; spin++) {
+        if ((spin & 1023) == 1023 &&
+            std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(20)) {
+            if (!ESHKOL_HIP_OK(hipStreamSynchronize(st))) return -1;
+            return (*r0 == ticket && *r1 == ticket) ? 0 : -1;
+        }
+        __builtin_ia32_pause();
+    }
+    std::atomic_thread_fence(std::memory_order_acquire);
+    return 0;
 }
 
 /* device-resident constant tables for the contraction: identity pair lists and moduli */
@@ -678,20 +721,20 @@ extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, dou
     int32_t* dmu = (int32_t*)eshkol_hip_workspace(WS_ROWSHIFT, M * sizeof(int32_t));
     int32_t* dnu = (int32_t*)eshkol_hip_workspace(WS_COLSHIFT, N * sizeof(int32_t));
     if (!amax || !bmax || !dmu || !dnu) return -1;
-    CrtScan* dscan = (CrtScan*)eshkol_hip_workspace(WS_MISC, 2 * sizeof(CrtScan));
-    char* host = (char*)pinned(2 * sizeof(CrtScan) + (M + N) * (sizeof(double) + sizeof(int32_t)));
-    if (!dscan || !host) return -1;
-    CrtScan* h_scan = (CrtScan*)host;
-    double* h_amax = (double*)(h_scan + 2);
+    char* host = (char*)pinned((M + N) * (sizeof(double) + sizeof(int32_t)));
+    if (!host || !ensure_mailbox()) return -1;
+    const CrtScan* h_scan = g_mailbox;
+    double* h_amax = (double*)host;
     double* h_bmax = h_amax + M;
     int32_t* h_mu = (int32_t*)(h_bmax + N);
     int32_t* h_nu = h_mu + M;
 
     if ((a_kmajor ? hip_colabsmax_f64(A, K, M, 0.0, amax, st) : hip_rowabsmax_f64(A, M, K, 0.0, amax, st)) != 0) return -1;
     if ((b_kmajor ? hip_colabsmax_f64(B, K, N, 0.0, bmax, st) : hip_rowabsmax_f64(B, N, K, 0.0, bmax, st)) != 0) return -1;
-    hipLaunchKernelGGL(crt_scan_kernel, dim3(2), dim3(SCAN_THREADS), 0, st, amax, M, bmax, N, dmu, dnu, dscan);
-    if (!ESHKOL_HIP_OK(hipMemcpyAsync(h_scan, dscan, 2 * sizeof(CrtScan), hipMemcpyDeviceToHost, st))) return -1;
-    if (!ESHKOL_HIP_OK(hipStreamSynchronize(st))) return -1;
+    const uint32_t ticket = ++g_ticket ? g_ticket : ++g_ticket;            /* never 0: the mailbox starts zeroed */
+    hipLaunchKernelGGL(crt_scan_kernel, dim3(2), dim3(SCAN_THREADS), 0, st, amax, M, bmax, N, dmu, dnu,
+                       g_mailbox_dev, ticket);
+    if (!ESHKOL_HIP_OK(hipGetLastError()) || await_mailbox(ticket, st) != 0) return -1;
     if (h_scan[0].nonfinite || h_scan[1].nonfinite) return -1;          /* NaN/Inf input */
 
     /* frac bounds (gpu_memory.mm:403-417) and the range of floor(log2 max) per operand */
