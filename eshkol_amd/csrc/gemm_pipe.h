@@ -65,6 +65,13 @@ __device__ __forceinline__ void static_for(F&& f) {
     }
 }
 
+/* Buffer descriptor of the 256 plane rows that start at `rows` (wave-uniform):
+ * untyped, no stride, so a load's address is rows + the lane's 32-bit offset +
+ * a scalar offset, and none of it is vector arithmetic. */
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t plane_rsrc(const int8_t* rows) {
+    return __builtin_amdgcn_make_buffer_rsrc((void*)rows, 0, 0x7fffffff, 0x00020000);
+}
+
 __device__ __forceinline__ void lds_barrier() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
@@ -116,7 +123,13 @@ __device__ __forceinline__ void run_tiles(int8_t* smem, const Source& cm, Next n
     const int li = lane & 31, lh = lane >> 5;
 
     const int nkb_per = cm.ld / BKB;
-    const size_t g_off = (size_t)(tid >> 3) * cm.ld + (tid & 7) * 16;
+    /* A thread's chunks of a k-block: rows tid/8 + 32 r, bytes 16 (tid%8) of the
+     * 128. Kept as 32-bit offsets from a wave-uniform block address, so the
+     * loads take their base from scalar registers and the cursor is scalar work. */
+    uint32_t voff[(C::A_CH > C::B_CH) ? C::A_CH : C::B_CH];
+#pragma unroll
+    for (int r = 0; r < ((C::A_CH > C::B_CH) ? C::A_CH : C::B_CH); r++)
+        voff[r] = (uint32_t)((tid >> 3) + 32 * r) * (uint32_t)cm.ld + (uint32_t)(tid & 7) * 16u;
     const int s_off = (tid >> 3) * PITCH + (tid & 7) * 16;
 
     /* The current tile and the one after it: the request cursor may cross into the
@@ -139,8 +152,8 @@ __device__ __forceinline__ void run_tiles(int8_t* smem, const Source& cm, Next n
                 table[(tab ^ 1) * 2 * MAX_PAIRS + tid] = nxt.a_idx ? nxt.a_idx[tid] : 0;
                 table[(tab ^ 1) * 2 * MAX_PAIRS + MAX_PAIRS + tid] = nxt.b_idx ? nxt.b_idx[tid] : 0;
             }
-            nx_a = cm.a_planes + (size_t)nxt.m0 * cm.ld + g_off;
-            nx_b = cm.b_planes + (size_t)nxt.n0 * cm.ld + g_off;
+            nx_a = cm.a_planes + (size_t)nxt.m0 * cm.ld;
+            nx_b = cm.b_planes + (size_t)nxt.n0 * cm.ld;
             nx_np = nxt.npairs;
         }
     };
@@ -148,8 +161,8 @@ __device__ __forceinline__ void run_tiles(int8_t* smem, const Source& cm, Next n
     __syncthreads();
 
     /* request cursor */
-    const int8_t* a_t = cm.a_planes + (size_t)cur.m0 * cm.ld + g_off;
-    const int8_t* b_t = cm.b_planes + (size_t)cur.n0 * cm.ld + g_off;
+    const int8_t* a_t = cm.a_planes + (size_t)cur.m0 * cm.ld;
+    const int8_t* b_t = cm.b_planes + (size_t)cur.n0 * cm.ld;
     int gl_t = 0, gl_j = 0, gl_np = cur.npairs, gl_tab = 0;
     int v_ia = table[0], v_ib = table[MAX_PAIRS];
 
@@ -159,16 +172,18 @@ __device__ __forceinline__ void run_tiles(int8_t* smem, const Source& cm, Next n
     auto gload_a = [&](auto slot) {
         constexpr int S = decltype(slot)::value;
         const int ia = __builtin_amdgcn_readfirstlane(v_ia);
-        const int8_t* ap = a_t + (size_t)ia * cm.a_plane_stride + (size_t)gl_j * BKB;
+        const __amdgpu_buffer_rsrc_t rs = plane_rsrc(a_t + (size_t)ia * cm.a_plane_stride);
+        const int soff = gl_j * BKB;
 #pragma unroll
-        for (int r = 0; r < C::A_CH; r++) ra[S][r] = *(const v4i_t*)(ap + (size_t)(32 * r) * cm.ld);
+        for (int r = 0; r < C::A_CH; r++) ra[S][r] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff[r], soff, 0);
     };
     auto gload_b = [&](auto slot) {
         constexpr int S = decltype(slot)::value;
         const int ib = __builtin_amdgcn_readfirstlane(v_ib);
-        const int8_t* bp = b_t + (size_t)ib * cm.b_plane_stride + (size_t)gl_j * BKB;
+        const __amdgpu_buffer_rsrc_t rs = plane_rsrc(b_t + (size_t)ib * cm.b_plane_stride);
+        const int soff = gl_j * BKB;
 #pragma unroll
-        for (int r = 0; r < C::B_CH; r++) rb[S][r] = *(const v4i_t*)(bp + (size_t)(32 * r) * cm.ld);
+        for (int r = 0; r < C::B_CH; r++) rb[S][r] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff[r], soff, 0);
         /* advance: next k-block, next product, next tile; with no next tile the
          * cursor stays on the last block (those requests are never consumed) */
         const int nj = gl_j + 1;
