@@ -5,6 +5,7 @@
  */
 #include "hip_common.h"
 #include "kernels.h"
+#include "tanh_f64.h"
 
 namespace {
 
@@ -121,7 +122,7 @@ __device__ __forceinline__ double apply_op(int op, double a, double b, bool has_
         case 7:  return log(a);
         case 8:  return sin(a);
         case 9:  return cos(a);
-        case 10: return tanh(a);
+        case 10: return eshkol_tanh_f64(a);
         case 11: return a > 0.0 ? a : 0.0;
         case 12: return 1.0 / (1.0 + exp(-a));
         case 13: return sqrt(a);
@@ -145,7 +146,7 @@ void bias_act_f64_kernel(double* __restrict__ Y, const double* __restrict__ bias
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
         double v = Y[i];
         if (bias) v += bias[i % cols];
-        if (act == 1) v = tanh(v);
+        if (act == 1) v = eshkol_tanh_f64(v);
         Y[i] = v;
     }
 }

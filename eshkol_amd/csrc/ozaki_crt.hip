@@ -23,6 +23,7 @@
  */
 #include "hip_common.h"
 #include "kernels.h"
+#include "tanh_f64.h"
 #include "kmajor_tile.h"
 
 #include <atomic>
@@ -311,7 +312,7 @@ void crt_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t N
         const double cp = h1 + h2;
         double v = (cp * mu_inv) * ldexp(1.0, -sh[e]);
         if (bias) v = v + bv[e];
-        if (TANH) v = tanh(v);
+        if (TANH) v = eshkol_tanh_f64(v);
         out[e] = v;
     }
     if (vec && (((uintptr_t)C & 15) == 0)) {

@@ -303,3 +303,32 @@ assert err <= float(os.environ["EXPECT_ERR"]), err
     r = run_child(body2, {"ESHKOL_MATMUL_ACCURACY": "exact", "EXPECT_ERR": "1e-14", "ESHKOL_GPU_THRESHOLD": "1",
                           "ESHKOL_GPU_VERBOSE": "1"})
     assert "native fp64 MFMA (budget met cheapest by native fp64)" in r.stderr
+
+
+def test_device_tanh_accuracy(gpu):
+    """The fused epilogues use the library's own fp64 tanh. Against a reference of twice
+    the precision (numpy longdouble) it must stay within 2 ulp everywhere: dense samples of
+    the whole range, tiny arguments (relative accuracy), the saturation edge, specials."""
+    import eshkol_amd as ea
+    from gpu_util import stream
+    lib = ea.load()
+    rng = np.random.default_rng(77)
+    x = np.concatenate([
+        rng.uniform(-20.0, 20.0, 400000), rng.uniform(-1.0, 1.0, 400000),
+        np.ldexp(rng.uniform(0.5, 1.0, 200000), rng.integers(-60, 6, 200000)) * rng.choice([-1.0, 1.0], 200000),
+        rng.uniform(18.5, 19.5, 1000), np.linspace(0.17, 0.18, 1001), np.linspace(0.34, 0.36, 1001),
+        [0.0, -0.0, 1e-300, -1e-300, 5e-324, 2.0 ** -28, 2.0 ** -27, 19.1, 19.2, 40.0, 710.0, -710.0, 1e308,
+         np.inf, -np.inf]])
+    dx, dy = ea.DeviceArray.from_host(x), ea.DeviceArray((x.size,))
+    assert lib.hip_elementwise_f64(dx.ptr, None, dy.ptr, x.size, 10, stream()) == 0
+    ea.synchronize()
+    got = dy.download()
+    want_ld = np.tanh(x.astype(np.longdouble))
+    want = want_ld.astype(np.float64)
+    err_ulp = np.abs((got.astype(np.longdouble) - want_ld) / np.spacing(np.maximum(np.abs(want), 5e-324)).astype(np.longdouble))
+    assert err_ulp.max() <= 2.0, (err_ulp.max(), x[np.argmax(err_ulp)])
+    assert np.array_equal(np.signbit(got), np.signbit(x))
+    out = ea.DeviceArray((1,))
+    assert lib.hip_elementwise_f64(ea.DeviceArray.from_host(np.array([np.nan])).ptr, None, out.ptr, 1, 10, stream()) == 0
+    ea.synchronize()
+    assert np.isnan(out.download()[0])
