@@ -110,7 +110,9 @@ template <int TM, int TN> struct TilesCfg {
 };
 
 /* next_tile(Tile&) -> bool hands out this workgroup's tiles in order;
- * epilogue(acc, tile) consumes a finished accumulator (LDS is free for it). */
+ * epilogue(acc, tile) consumes a finished accumulator (LDS buffer 1 is free for
+ * it, buffer 0 is not). A launch of single tiles needs one index table only:
+ * the second half of `table` is written when a next tile exists. */
 template <class Op, int TM, int TN, int PF, class Next, class Epi>
 __device__ __forceinline__ void run_tiles(int8_t* smem, const Source& cm, Next next_tile, Epi epilogue) {
     using C = Cfg<TM, TN>;
