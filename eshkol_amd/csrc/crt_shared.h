@@ -1,0 +1,77 @@
+/*
+ * Pieces the two CRT tiers (exact: ozaki_crt.hip, fast: ozaki_fast.hip) share:
+ * the byte form of a scaled operand element, the byte weights of a modulus, and
+ * the host-side hand-off of the row and column maxima's exponents.
+ */
+#ifndef ESHKOL_HIP_CRT_SHARED_H
+#define ESHKOL_HIP_CRT_SHARED_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+/* An integer s of magnitude below 2^53 as eight bytes: the low seven of its
+ * 64-bit two's complement, and 1 or 0 in the eighth for negative or not. Its
+ * value is sum_{i<7} b_i 256^i - b_7 256^7. */
+struct Scaled { uint32_t lo, hi; };
+
+/* x * 2^sh as such an integer, read straight off the bit pattern of x (sh is
+ * chosen by the callers so that the magnitude stays below 2^53).
+ * HALF_UP false: truncated towards zero (the exact tier, gpu_memory.mm:2560-2590);
+ * subnormal x are scaled like any other value.
+ * HALF_UP true: magnitude rounded half up, subnormal x count as zero (the fast
+ * tier's split, metal_softfloat.h:4148-4178). */
+template <bool HALF_UP>
+__device__ __forceinline__ Scaled scaled_integer(double x, int sh) {
+    const uint64_t bits = __double_as_longlong(x);
+    const int e = (int)((bits >> 52) & 0x7ff);
+    uint64_t mant = bits & 0xfffffffffffffull;
+    int e_eff = 1;
+    if (e != 0) { mant |= 1ull << 52; e_eff = e; }
+    else if (HALF_UP) mant = 0;
+    const int rs = 1075 - e_eff - sh;          /* value = mant * 2^-rs; rs <= 0 is excluded by the callers */
+    uint64_t t = mant;
+    if (HALF_UP) {
+        if (rs > 53) t = 0;
+        else if (rs > 0) t = (mant + (1ull << (rs - 1))) >> rs;
+    } else {
+        if (rs >= 64) t = 0;
+        else if (rs > 0) t = mant >> rs;
+    }
+    const uint64_t m = (uint64_t)((int64_t)bits >> 63);
+    const uint64_t v = (t ^ m) - m;
+    return { (uint32_t)v, (uint32_t)(v >> 32) & 0x01ffffffu };
+}
+
+/* Byte weights of a modulus p <= 256: 256^i mod p for the seven magnitude bytes
+ * and -(256^7) mod p for the sign byte, four to a word, so that two
+ * v_dot4_u32_u8 give x = sum b_i w_i < 2^19 congruent to the integer. */
+struct ByteWeights { uint32_t lo, hi; };
+constexpr ByteWeights byte_weights(int modulus) {
+    const uint32_t p = (uint32_t)modulus;
+    uint32_t c[8] = {}, pw = 1u % p;
+    for (int i = 0; i < 8; i++) { c[i] = pw; pw = pw * 256u % p; }
+    c[7] = (p - c[7]) % p;
+    return { c[0] | c[1] << 8 | c[2] << 16 | c[3] << 24, c[4] | c[5] << 8 | c[6] << 16 | c[7] << 24 };
+}
+
+/* ---- exponents of the maxima (implemented in ozaki_crt.hip) ---------------------- */
+
+/* What the host learns about one operand's row (or column) maxima. */
+struct CrtMaxima {
+    int nonfinite;              /* a NaN or an infinity among them */
+    int nonzero;                /* at least one maximum > 0 */
+    int e_min, e_max;           /* range of floor(log2 max) over the maxima > 0 */
+};
+constexpr int32_t CRT_FL_ZERO = INT32_MIN;      /* exponent entry of a maximum of zero */
+
+/* fl_a[i] = floor(log2 amax[i]) taken from the exponent field (CRT_FL_ZERO for a
+ * maximum of zero), likewise fl_b; waits for the device and fills out[0] (A) and
+ * out[1] (B). Exact unless a maximum lies within 2^-40 of a power of two AND the
+ * caller needs libm's floor(log2): the exact tier checks that itself. 0 on success. */
+int eshkol_crt_scan_exponents(const double* amax, uint64_t M, const double* bmax, uint64_t N,
+                              int32_t* fl_a, int32_t* fl_b, CrtMaxima out[2], hipStream_t st);
+
+/* In place: fl -> E - fl, and 0 where fl is CRT_FL_ZERO. */
+void eshkol_crt_shifts_from_exponents(int32_t* fl_a, uint64_t M, int32_t* fl_b, uint64_t N, int E, hipStream_t st);
+
+#endif

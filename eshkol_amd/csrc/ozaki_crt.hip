@@ -25,6 +25,7 @@
 #include "kernels.h"
 #include "tanh_f64.h"
 #include "kmajor_tile.h"
+#include "crt_shared.h"
 
 #include <atomic>
 #include <chrono>
@@ -44,45 +45,17 @@ namespace {
 constexpr int MAX_MODULI = 16;
 const int H_MODULI[MAX_MODULI] = { OZAKI_MODULI_16 };
 
-/* Byte weights of the moduli: 256^i mod p for the seven magnitude bytes, and
- * -(256^7) mod p for the sign byte (see scaled_integer). */
 struct ModuliTable { int p[MAX_MODULI]; uint32_t wlo[MAX_MODULI]; uint32_t whi[MAX_MODULI]; };
 constexpr ModuliTable make_table() {
     ModuliTable t{};
     const int m[MAX_MODULI] = { OZAKI_MODULI_16 };
     for (int l = 0; l < MAX_MODULI; l++) {
-        const uint32_t p = (uint32_t)m[l];
-        t.p[l] = m[l];
-        uint32_t c[8] = {}, pw = 1u % p;
-        for (int i = 0; i < 8; i++) { c[i] = pw; pw = pw * 256u % p; }
-        c[7] = (p - c[7]) % p;
-        t.wlo[l] = c[0] | c[1] << 8 | c[2] << 16 | c[3] << 24;
-        t.whi[l] = c[4] | c[5] << 8 | c[6] << 16 | c[7] << 24;
+        const ByteWeights w = byte_weights(m[l]);
+        t.p[l] = m[l]; t.wlo[l] = w.lo; t.whi[l] = w.hi;
     }
     return t;
 }
 constexpr ModuliTable TBL = make_table();
-
-/* trunc(x * 2^sh), an integer of magnitude below 2^53 by construction of sh, as
- * eight bytes: the low seven of its 64-bit two's complement, and 1 or 0 in the
- * eighth for negative or not. Its value is sum_{i<7} b_i 256^i - b_7 256^7. The
- * magnitude is read straight off the bit pattern: the right shift is the
- * truncation. */
-struct Scaled { uint32_t lo, hi; };
-__device__ __forceinline__ Scaled scaled_integer(double x, int sh) {
-    const uint64_t bits = __double_as_longlong(x);
-    const int e = (int)((bits >> 52) & 0x7ff);
-    uint64_t mant = bits & 0xfffffffffffffull;
-    int e_eff = 1;
-    if (e != 0) { mant |= 1ull << 52; e_eff = e; }
-    const int rs = 1075 - e_eff - sh;          /* value = mant * 2^-rs */
-    uint64_t t = mant;                         /* rs <= 0 is excluded by the host's range check */
-    if (rs >= 64) t = 0;
-    else if (rs > 0) t = mant >> rs;
-    const uint64_t m = (uint64_t)((int64_t)bits >> 63);
-    const uint64_t v = (t ^ m) - m;
-    return { (uint32_t)v, (uint32_t)(v >> 32) & 0x01ffffffu };
-}
 
 /* A word whose low byte is the int8 residue of s modulo p_L, the representative
  * in [-p/2, p/2). Five full-rate instructions: two byte dot products give
@@ -103,7 +76,7 @@ __device__ __forceinline__ uint32_t residue_byte(Scaled s) {
 /* Residues of two consecutive k of one row: one 16-bit store per plane. */
 template <int NMOD>
 __device__ __forceinline__ void split_pair(double x0, double x1, int sh, int8_t* out, uint64_t plane_stride) {
-    const Scaled s0 = scaled_integer(x0, sh), s1 = scaled_integer(x1, sh);
+    const Scaled s0 = scaled_integer<false>(x0, sh), s1 = scaled_integer<false>(x1, sh);
 #define ESHKOL_SPLIT_ONE(L)                                                           \
     if (L < NMOD)                                                                     \
         *(uint16_t*)(out + (uint64_t)L * plane_stride) =                              \
@@ -120,7 +93,7 @@ template <int NMOD>
 __device__ __forceinline__ void split_16(const double* x, int sh, int8_t* out, uint64_t plane_stride) {
     Scaled s[16];
 #pragma unroll
-    for (int e = 0; e < 16; e++) s[e] = scaled_integer(x[e], sh);
+    for (int e = 0; e < 16; e++) s[e] = scaled_integer<false>(x[e], sh);
 #define ESHKOL_SPLIT_ONE(L)                                                           \
     if (L < NMOD) {                                                                   \
         v4u_t w;                                                                      \
@@ -195,7 +168,7 @@ void crt_split_staged_kernel(const double* __restrict__ X, uint64_t rows, uint64
     }
     Scaled t[4];
 #pragma unroll
-    for (int e = 0; e < 4; e++) t[e] = scaled_integer(x[e], sh);
+    for (int e = 0; e < 4; e++) t[e] = scaled_integer<false>(x[e], sh);
 #define ESHKOL_SPLIT_ONE(L)                                                           \
     if (L < NMOD) {                                                                   \
         const uint32_t w01 = __builtin_amdgcn_perm(residue_byte<L>(t[1]), residue_byte<L>(t[0]), 0x0c0c0400u); \
@@ -342,7 +315,7 @@ void crt_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t N
  * candidates, takes the full host pass instead. */
 constexpr int SCAN_CAND = 64;
 constexpr int SCAN_THREADS = 1024;
-constexpr int32_t FL_ZERO = INT32_MIN;          /* marks a maximum of zero: shift 0 */
+constexpr int32_t FL_ZERO = CRT_FL_ZERO;        /* marks a maximum of zero: shift 0 */
 constexpr unsigned long long MANT_ONE = 1ull << 52, MANT_WINDOW = 1ull << 12;
 
 struct CrtScan {
@@ -579,6 +552,17 @@ int await_mailbox(uint32_t ticket, hipStream_t st) {
     return 0;
 }
 
+/* Runs the scan on the two vectors of maxima and waits for its summary. */
+const CrtScan* scan_maxima(const double* amax, uint64_t M, const double* bmax, uint64_t N,
+                           int32_t* fl_a, int32_t* fl_b, hipStream_t st) {
+    if (!ensure_mailbox()) return nullptr;
+    const uint32_t ticket = ++g_ticket ? g_ticket : ++g_ticket;            /* never 0: the mailbox starts zeroed */
+    hipLaunchKernelGGL(crt_scan_kernel, dim3(2), dim3(SCAN_THREADS), 0, st, amax, M, bmax, N, fl_a, fl_b,
+                       g_mailbox_dev, ticket);
+    if (!ESHKOL_HIP_OK(hipGetLastError()) || await_mailbox(ticket, st) != 0) return nullptr;
+    return g_mailbox;
+}
+
 /* device-resident constant tables for the contraction: identity pair lists and moduli */
 int32_t* g_tables = nullptr;   /* [0..16] pair_first, [17..32] pair index, [33..48] moduli */
 int ensure_tables(hipStream_t st) {
@@ -635,6 +619,21 @@ int crt_split_any(const double* X, uint64_t rows, uint64_t K, const int32_t* shi
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 }  // namespace
+
+int eshkol_crt_scan_exponents(const double* amax, uint64_t M, const double* bmax, uint64_t N,
+                              int32_t* fl_a, int32_t* fl_b, CrtMaxima out[2], hipStream_t st) {
+    const CrtScan* h = scan_maxima(amax, M, bmax, N, fl_a, fl_b, st);
+    if (!h) return -1;
+    for (int o = 0; o < 2; o++) {
+        out[o].nonfinite = h[o].nonfinite; out[o].nonzero = h[o].nonzero;
+        out[o].e_min = h[o].e_min; out[o].e_max = h[o].e_max;
+    }
+    return 0;
+}
+
+void eshkol_crt_shifts_from_exponents(int32_t* fl_a, uint64_t M, int32_t* fl_b, uint64_t N, int E, hipStream_t st) {
+    hipLaunchKernelGGL(crt_shift_kernel, dim3((unsigned)((M + N + 255) / 256)), dim3(256), 0, st, fl_a, M, fl_b, N, E);
+}
 
 extern "C" int hip_ozaki_crt_split_f64(const double* X, uint64_t rows, uint64_t K,
                                        const int32_t* shift, int num_moduli,
@@ -723,8 +722,7 @@ extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, dou
     int32_t* dnu = (int32_t*)eshkol_hip_workspace(WS_COLSHIFT, N * sizeof(int32_t));
     if (!amax || !bmax || !dmu || !dnu) return -1;
     char* host = (char*)pinned((M + N) * (sizeof(double) + sizeof(int32_t)));
-    if (!host || !ensure_mailbox()) return -1;
-    const CrtScan* h_scan = g_mailbox;
+    if (!host) return -1;
     double* h_amax = (double*)host;
     double* h_bmax = h_amax + M;
     int32_t* h_mu = (int32_t*)(h_bmax + N);
@@ -732,10 +730,8 @@ extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, dou
 
     if ((a_kmajor ? hip_colabsmax_f64(A, K, M, 0.0, amax, st) : hip_rowabsmax_f64(A, M, K, 0.0, amax, st)) != 0) return -1;
     if ((b_kmajor ? hip_colabsmax_f64(B, K, N, 0.0, bmax, st) : hip_rowabsmax_f64(B, N, K, 0.0, bmax, st)) != 0) return -1;
-    const uint32_t ticket = ++g_ticket ? g_ticket : ++g_ticket;            /* never 0: the mailbox starts zeroed */
-    hipLaunchKernelGGL(crt_scan_kernel, dim3(2), dim3(SCAN_THREADS), 0, st, amax, M, bmax, N, dmu, dnu,
-                       g_mailbox_dev, ticket);
-    if (!ESHKOL_HIP_OK(hipGetLastError()) || await_mailbox(ticket, st) != 0) return -1;
+    const CrtScan* h_scan = scan_maxima(amax, M, bmax, N, dmu, dnu, st);
+    if (!h_scan) return -1;
     if (h_scan[0].nonfinite || h_scan[1].nonfinite) return -1;          /* NaN/Inf input */
 
     /* frac bounds (gpu_memory.mm:403-417) and the range of floor(log2 max) per operand */

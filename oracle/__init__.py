@@ -227,3 +227,61 @@ def mlp_layer(X, W, b, num_moduli=16):
     rc = lib().oracle_mlp_layer_f64(_d(X), _d(W), bptr, _d(out), u64(batch), u64(in_f), u64(out_f),
                                     C.c_int(num_moduli))
     return out if rc == 0 else None
+
+
+class FastConstants(C.Structure):
+    _fields_ = [("num_moduli", C.c_int), ("cap", C.c_int), ("E", C.c_int), ("moduli", C.c_int * 16),
+                ("q", C.c_int * 16), ("log2P", C.c_double), ("P", C.c_double),
+                ("P_hi", C.c_float), ("P_lo", C.c_float)]
+
+
+def fast_constants(K, n_mod=11):
+    c = FastConstants()
+    L = lib()
+    L.oracle_ozaki_fast_constants.restype = C.c_int
+    rc = L.oracle_ozaki_fast_constants(u64(K), C.c_int(n_mod), C.byref(c))
+    return rc, c
+
+
+def ozaki_fast_stages(A, B, n_mod=11):
+    """Every stage of the reduced-precision CRT tier: exponents, residue planes, the
+    integers they are residues of, exact products, the reference's float-float C and
+    the exactly scaled integer product."""
+    A, B = _f64(A), _f64(B)
+    M, K = A.shape
+    N = B.shape[1]
+    L = lib()
+    rc, c = fast_constants(K, n_mod)
+    if rc != 0:
+        return None
+    n = c.num_moduli
+    ei, fj = np.empty(M, np.int32), np.empty(N, np.int32)
+    L.oracle_ozaki_fast_exponents(_d(A), _d(B), u64(M), u64(K), u64(N), ei.ctypes.data_as(i32p), fj.ctypes.data_as(i32p))
+    ap, bpl = np.empty((n, M, K), np.int8), np.empty((n, N, K), np.int8)
+    a_int, b_int = np.empty((M, K), np.int64), np.empty((N, K), np.int64)
+    i64p = C.POINTER(C.c_int64)
+    L.oracle_ozaki_fast_split_a(_d(A), u64(M), u64(K), ei.ctypes.data_as(i32p), C.byref(c), ap.ctypes.data_as(bp),
+                                a_int.ctypes.data_as(i64p))
+    L.oracle_ozaki_fast_split_b(_d(B), u64(K), u64(N), fj.ctypes.data_as(i32p), C.byref(c), bpl.ctypes.data_as(bp),
+                                b_int.ctypes.data_as(i64p))
+    G = np.empty((n, M, N), np.int32)
+    L.oracle_ozaki_fast_products(ap.ctypes.data_as(bp), bpl.ctypes.data_as(bp), u64(M), u64(K), u64(N), C.c_int(n),
+                                 G.ctypes.data_as(i32p))
+    out, exact = np.empty((M, N)), np.empty((M, N))
+    L.oracle_ozaki_fast_reconstruct(G.ctypes.data_as(i32p), u64(M), u64(N), C.byref(c), ei.ctypes.data_as(i32p),
+                                    fj.ctypes.data_as(i32p), _d(out))
+    L.oracle_ozaki_fast_exact_value(a_int.ctypes.data_as(i64p), b_int.ctypes.data_as(i64p), u64(M), u64(K), u64(N),
+                                    C.byref(c), ei.ctypes.data_as(i32p), fj.ctypes.data_as(i32p), _d(exact))
+    return dict(consts=c, num_moduli=n, E=c.E, moduli=list(c.moduli[:n]), q=list(c.q[:n]), ei=ei, fj=fj,
+                a_planes=ap, b_planes=bpl, a_int=a_int, b_int=b_int, G=G, C=out, C_exact=exact)
+
+
+def matmul_ozaki_fast(A, B, n_mod=11):
+    A, B = _f64(A), _f64(B)
+    M, K = A.shape
+    N = B.shape[1]
+    out = np.empty((M, N))
+    L = lib()
+    L.oracle_matmul_ozaki_fast_f64.restype = C.c_int
+    rc = L.oracle_matmul_ozaki_fast_f64(_d(A), _d(B), _d(out), u64(M), u64(K), u64(N), C.c_int(n_mod))
+    return rc, out

@@ -202,4 +202,33 @@ int oracle_mlp_layer_f64(const double* X, const double* W, const double* b, doub
 #ifdef __cplusplus
 }
 #endif
+/* ---- Ozaki-II reduced-precision ("fast") CRT tier (gpu_memory.mm:2802-3012,
+ *      metal_softfloat.h:4126-4246) ------------------------------------------ */
+typedef struct {
+    int num_moduli, cap, E;
+    int moduli[16];
+    int q[16];                  /* (P / p_l)^-1 mod p_l */
+    double log2P, P;
+    float P_hi, P_lo;           /* P as a float pair */
+} OracleFastConstants;
+
+int  oracle_ozaki_fast_cap(uint64_t K);
+int  oracle_ozaki_fast_moduli(int cap, int n_mod, int* out);
+int  oracle_ozaki_fast_constants(uint64_t K, int n_mod_req, OracleFastConstants* c);
+void oracle_ozaki_fast_exponents(const double* A, const double* B, uint64_t M, uint64_t K, uint64_t N,
+                                 int32_t* ei, int32_t* fj);
+/* planes [n][rows][K] int8; scaled (optional) [rows][K] int64: the integers the residues are taken of */
+void oracle_ozaki_fast_split_a(const double* A, uint64_t M, uint64_t K, const int32_t* ei,
+                               const OracleFastConstants* c, int8_t* planes, int64_t* scaled);
+void oracle_ozaki_fast_split_b(const double* B, uint64_t K, uint64_t N, const int32_t* fj,
+                               const OracleFastConstants* c, int8_t* planes, int64_t* scaled);
+void oracle_ozaki_fast_products(const int8_t* a_planes, const int8_t* b_planes, uint64_t M, uint64_t K, uint64_t N,
+                                int n, int32_t* G);
+void oracle_ozaki_fast_reconstruct(const int32_t* G, uint64_t M, uint64_t N, const OracleFastConstants* c,
+                                   const int32_t* ei, const int32_t* fj, double* C);
+void oracle_ozaki_fast_exact_value(const int64_t* a_scaled, const int64_t* b_scaled, uint64_t M, uint64_t K, uint64_t N,
+                                   const OracleFastConstants* c, const int32_t* ei, const int32_t* fj, double* C);
+int  oracle_matmul_ozaki_fast_f64(const double* A, const double* B, double* C,
+                                  uint64_t M, uint64_t K, uint64_t N, int n_mod);
+
 #endif
