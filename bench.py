@@ -170,6 +170,18 @@ def main():
             "vs_native": (flops / (w3 * 1e-3) / 1e9) / native_gflops}
         log("ozaki crt: %.3f ms/step %.1f GFLOP/s-eq" % (w3, flops / (w3 * 1e-3) / 1e9))
 
+        # the reduced-precision CRT tier on the same operands (11 moduli: the reference's ~1e-8 default)
+        os.dup2(devnull, 2)
+        try:
+            _, wf = timed(lambda: lib.hip_matmul_ozaki_fast_f64(dA.ptr, dB.ptr, dC.ptr, M, K, N, 11, st))
+        finally:
+            os.dup2(saved, 2)
+        tiers["ozaki_crt_fast_11_moduli"] = {
+            "ms": wf, "gflops_fp64_equiv": flops / (wf * 1e-3) / 1e9,
+            "vs_native": (flops / (wf * 1e-3) / 1e9) / native_gflops,
+            "note": "prime-power moduli <= 90 at K = 8192, E = 26 bits per operand, about 1e-8 normwise"}
+        log("ozaki crt fast (11 moduli): %.3f ms/step %.1f GFLOP/s-eq" % (wf, flops / (wf * 1e-3) / 1e9))
+
         if not args.no_stages:
             nmod = 16
             Mp, ldk = (M + 255) // 256 * 256, (K + 255) // 256 * 256

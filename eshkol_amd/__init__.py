@@ -45,6 +45,12 @@ class HipOzakiCrtStages(C.Structure):
                 ("num_moduli", i32), ("E", i32)]
 
 
+class HipOzakiFastStages(C.Structure):
+    _fields_ = [("a_planes", vp), ("b_planes", vp), ("w_planes", vp), ("shift_a", vp), ("shift_b", vp),
+                ("rows_a_padded", u64), ("rows_b_padded", u64), ("ldk", u64),
+                ("num_moduli", i32), ("E", i32), ("cap", i32), ("moduli", i32 * 16)]
+
+
 class HipOzakiInt8Stages(C.Structure):
     _fields_ = [("a_slices", vp), ("b_slices", vp), ("products", vp), ("rmax", vp), ("cmax", vp),
                 ("rows_a_padded", u64), ("rows_b_padded", u64), ("ldk", u64),
@@ -113,6 +119,9 @@ SIGNATURES = {
                                                 C.c_double, vp, vp, vp, C.c_int, vp, vp]),
     "hip_matmul_ozaki_crt_f64": (C.c_int, [vp, vp, vp, u64, u64, u64, C.c_int, C.c_int, vp, C.c_int, vp]),
     "hip_ozaki_crt_last_stages": (C.c_int, [C.POINTER(HipOzakiCrtStages)]),
+    "hip_matmul_ozaki_fast_f64": (C.c_int, [vp, vp, vp, u64, u64, u64, C.c_int, vp]),
+    "hip_matmul_ozaki_fast_f64_ex": (C.c_int, [vp, vp, vp, u64, u64, u64, C.c_int, C.c_int, C.c_int, vp]),
+    "hip_ozaki_fast_last_stages": (C.c_int, [C.POINTER(HipOzakiFastStages)]),
     "hip_ozaki_slice_f64": (C.c_int, [vp, u64, u64, vp, C.c_int, vp, u64, u64, vp]),
     "hip_ozaki_reconstruct_f64": (C.c_int, [vp, vp, vp, C.c_int, vp, vp, u64, u64, vp]),
     "hip_matmul_ozaki_int8_f64": (C.c_int, [vp, vp, vp, u64, u64, u64, C.c_int, vp]),

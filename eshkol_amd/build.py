@@ -27,6 +27,7 @@ SOURCES = [
     "ozaki_crt.hip",
     "ozaki_int8.hip",
     "elementwise.hip",
+    "ozaki_fast.hip",
     "peak_probe.hip",
 ]
 

@@ -85,6 +85,8 @@ batch_fn host_batch_matmul(void) {
 struct TierEnv {
     bool ozaki_int8 = false;     /* explicit INT8 slice override */
     bool ozaki_crt = false;      /* explicit CRT exact tier      */
+    bool ozaki_fast = false;     /* reduced-precision CRT tier, exact tier behind it */
+    int  fast_moduli = 11;       /* gpu_memory.mm:265 */
     int  T = 6;
     int  num_moduli = 16;
     bool adaptive = false;
@@ -103,6 +105,22 @@ void parse_env(void) {
     if (k && strcmp(k, "ozaki-crt") == 0) e.ozaki_crt = true;
     const char* sf = getenv("ESHKOL_SF64_KERNEL");               /* gpu_memory.mm:3030-3033 */
     if (sf && strcmp(sf, "ozaki") == 0) e.ozaki_crt = true;
+    /* gpu_memory.mm:1319-1343: ESHKOL_OZAKI_FAST (anything but "0") or the kernel name */
+    if (const char* f = getenv("ESHKOL_OZAKI_FAST")) { if (strcmp(f, "0") != 0) e.ozaki_fast = true; }
+    if ((sf && strcmp(sf, "ozaki-fast") == 0) || (k && strcmp(k, "ozaki-fast") == 0)) e.ozaki_fast = true;
+    if (const char* fm = getenv("ESHKOL_OZAKI_FAST_MODULI")) {
+        int v = atoi(fm);
+        if (v >= 2 && v <= 16) e.fast_moduli = v;
+        else {
+            fprintf(stderr, "[GPU] ESHKOL_OZAKI_FAST_MODULI=%d out of range [2,%d]; "
+                            "clamping to %d (default %d). Fewer moduli = faster/coarser.\n",
+                    v, 16, (v < 2 ? 2 : 16), e.fast_moduli);
+            e.fast_moduli = (v < 2) ? 2 : 16;
+        }
+    }
+    if (e.ozaki_fast)
+        fprintf(stderr, "[GPU] Ozaki-II FAST tier ENABLED: N=%d moduli (accuracy knob), "
+                        "int8 MFMA GEMMs + GPU split + fp64 CRT reconstruction\n", e.fast_moduli);
     if (const char* t = getenv("ESHKOL_OZAKI_CUDA_T")) {         /* gpu_memory_cuda.cpp:315-321 */
         int v = atoi(t);
         if (v >= 1 && v <= 8) e.T = v;
@@ -356,10 +374,29 @@ int hip_matmul_f64(EshkolGPUBuffer* A, EshkolGPUBuffer* B, EshkolGPUBuffer* C,
     const double work = 2.0 * (double)M * (double)K * (double)N;
 
     int tier = 0;          /* 0 native, 1 INT8 slices, 2 CRT */
+    /* The reduced-precision CRT tier comes first when it is switched on, and a miss
+     * falls through to the exact tier, never to a wrong result (gpu_memory.mm:3036-3052). */
+    if (env.ozaki_fast && M >= 512 && K >= 512 && N >= 512) {
+        auto t0 = std::chrono::steady_clock::now();
+        GPU_LOG("matmul %llux%llu @ %llux%llu -> Ozaki-II FAST (%d moduli)", (unsigned long long)M,
+                (unsigned long long)K, (unsigned long long)K, (unsigned long long)N, env.fast_moduli);
+        const int fr = hip_matmul_ozaki_fast_f64_ex(dA, dB, dC, M, K, N, ta, tb, env.fast_moduli, g_stream);
+        if (fr == 0 && ESHKOL_HIP_OK(hipStreamSynchronize(g_stream))) {
+            if (env.profile) {
+                double ns = std::chrono::duration<double, std::nano>(std::chrono::steady_clock::now() - t0).count();
+                fprintf(stderr, "[OZAKI_PROFILE] fast M=%llu K=%llu N=%llu moduli=%d ms=%.2f GFLOPS=%.1f\n",
+                        (unsigned long long)M, (unsigned long long)K, (unsigned long long)N, env.fast_moduli,
+                        ns / 1e6, work / ns);
+            }
+            mark_written(C);
+            return 0;
+        }
+        fprintf(stderr, "[GPU] Ozaki-II FAST dispatch returned %d; falling back to exact tier\n", fr);
+    }
     int ozT = env.T;
     double pred = 1.0;
     const char* why = "default";
-    if (env.ozaki_crt) {
+    if (env.ozaki_crt || env.ozaki_fast) {
         if (M >= 512 && K >= 512 && N >= 512) { tier = 2; why = "ESHKOL_HIP_F64_KERNEL/ESHKOL_SF64_KERNEL override"; }
     } else if (env.ozaki_int8) {
         if (M >= 1024 && N >= 1024 && K >= 1024) { tier = 1; why = "ESHKOL_CUDA_F64_KERNEL override"; }

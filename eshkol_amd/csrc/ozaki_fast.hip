@@ -1,0 +1,379 @@
+/*
+ * Ozaki-II reduced-precision ("fast") CRT tier: C = A*B from int8 matrix-core
+ * products modulo a handful of small prime powers, reconstructed by a
+ * fractional CRT. Follows ozaki_ii_fast_dispatch of the reference
+ * (lib/backend/gpu/gpu_memory.mm:2802-3012) and its kernels
+ * (lib/backend/gpu/metal_softfloat.h:4126-4246):
+ *
+ *   moduli   the n largest prime powers <= cap; cap is the reference's, the
+ *            largest p with K floor(p/2)^2 < 2^24 (there it keeps an f32 GEMM
+ *            exact; here it keeps the moduli, hence every integer of the tier,
+ *            the reference's)
+ *   E        floor((log2 P - log2 K - 2) / 2) in [1, 52]: a function of K and n only
+ *   e_i,f_j  exponents of the row / column maxima (frexp), so all scaling is by
+ *            powers of two and nothing in the pipeline needs libm
+ *   split    round-half-up(|x| 2^(E-e)) with x's sign, modulo p, in [-p/2, p/2]
+ *            with +p/2 for the even moduli's tie; int8 planes [row][k]
+ *   product  W_l = (A_l B_l^T) mod p_l               int8 MFMA, int32 accumulate
+ *   C        frac(sum_l ((W_l q_l) mod p_l) / p_l) centred, times P 2^(e_i+f_j-2E)
+ *
+ * The reference carries the last step in float pairs (Apple GPUs have no fp64);
+ * here it is plain fp64, which resolves 2^-52 of P instead of about 2^-45. The
+ * integers (residues, products modulo p) are the reference's bit for bit.
+ */
+#include "hip_common.h"
+#include "kernels.h"
+#include "kmajor_tile.h"
+#include "crt_shared.h"
+
+#include <cmath>
+#include <cstring>
+#include <vector>
+#include <algorithm>
+
+typedef double d2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t v4u_t __attribute__((ext_vector_type(4)));
+
+namespace {
+
+constexpr int FAST_MAX_MODULI = 16;             /* gpu_memory.mm:264 */
+
+/* What the split needs to know about the moduli; passed by value. */
+struct FastTable {
+    int n;
+    int p[FAST_MAX_MODULI];
+    uint32_t wlo[FAST_MAX_MODULI], whi[FAST_MAX_MODULI];
+    float pinv[FAST_MAX_MODULI];
+    uint32_t neg_half[FAST_MAX_MODULI];         /* the byte of -p/2 for even p, else 0x100 (never a byte) */
+};
+
+/* The int8 residue of s modulo p_l as a byte. Two byte dot products give x < 2^19
+ * congruent to s; one fma against 1.5 * 2^23 leaves the nearest integer to x/p in
+ * the low bits of a float; the low byte of x - (2^22 + q) p is the residue in
+ * [-p/2, p/2]. The even moduli are powers of two, their 1/p is exact, so their tie
+ * x = p/2 (mod p) comes out as +p/2 or -p/2 with the parity of q: -p/2 is folded
+ * to the +p/2 the reference stores (metal_softfloat.h:4174-4177). */
+__device__ __forceinline__ uint32_t fast_residue(Scaled s, const FastTable& t, int l) {
+    const uint32_t x = __builtin_amdgcn_udot4(s.lo, t.wlo[l], __builtin_amdgcn_udot4(s.hi, t.whi[l], 0u, false), false);
+    const float qm = fmaf((float)x, t.pinv[l], 12582912.0f);
+    uint32_t r = (uint32_t)(__mul24(__float_as_int(qm), -t.p[l]) + (int)x) & 0xffu;
+    if (r == t.neg_half[l]) r = (uint32_t)t.p[l] >> 1;
+    return r;
+}
+
+__device__ __forceinline__ uint32_t pack4(uint32_t r0, uint32_t r1, uint32_t r2, uint32_t r3) {
+    return r0 | r1 << 8 | r2 << 16 | r3 << 24;
+}
+
+/* Row-major X[rows][K], pitch a multiple of 16: a block takes 1024 k of one row,
+ * a thread four of them; the residues are collected in LDS and leave as 16-byte
+ * stores (the layout of the exact tier's split). */
+__global__ __launch_bounds__(256)
+void fast_split_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
+                       const int32_t* __restrict__ shift, FastTable tbl, int8_t* __restrict__ planes,
+                       uint64_t rows_padded, uint64_t ldk) {
+    __shared__ __align__(16) uint32_t stage[FAST_MAX_MODULI][256];
+    const uint32_t cpr = (uint32_t)((ldk + 1023) / 1024);
+    const uint64_t row = blockIdx.x / cpr;
+    const uint64_t kbase = (uint64_t)(blockIdx.x % cpr) * 1024;
+    const int tid = threadIdx.x;
+    const uint64_t k = kbase + 4 * (uint64_t)tid;
+    double x[4] = {0.0, 0.0, 0.0, 0.0};
+    int sh = 0;
+    if (row < rows && k < K) {
+        sh = shift[row];
+        const double* p = X + row * K + k;
+        if (k + 3 < K && (K & 1) == 0 && (((uintptr_t)X & 15) == 0)) {
+            const d2_t v0 = *(const d2_t*)p, v1 = *(const d2_t*)(p + 2);
+            x[0] = v0.x; x[1] = v0.y; x[2] = v1.x; x[3] = v1.y;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) if (k + e < K) x[e] = p[e];
+        }
+    }
+    Scaled s[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) s[e] = scaled_integer<true>(x[e], sh);
+#pragma unroll
+    for (int l = 0; l < FAST_MAX_MODULI; l++)
+        if (l < tbl.n)
+            stage[l][tid] = pack4(fast_residue(s[0], tbl, l), fast_residue(s[1], tbl, l),
+                                  fast_residue(s[2], tbl, l), fast_residue(s[3], tbl, l));
+    __syncthreads();
+    const uint64_t plane_stride = rows_padded * ldk;
+    for (int c = tid; c < tbl.n * 64; c += 256) {
+        const int plane = c >> 6, ch = c & 63;
+        const uint64_t kk = kbase + 16 * (uint64_t)ch;
+        if (kk < ldk)
+            *(v4u_t*)(planes + (uint64_t)plane * plane_stride + row * ldk + kk) = *(const v4u_t*)&stage[plane][4 * ch];
+    }
+}
+
+/* k-major X[K][rows] (B as the runtime stores it), same planes. */
+__global__ __launch_bounds__(256, 4)
+void fast_split_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
+                              const int32_t* __restrict__ shift, FastTable tbl, int8_t* __restrict__ planes,
+                              uint64_t rows_padded, uint64_t ldk) {
+    __shared__ __align__(16) double tile[kmaj::SMEM_DOUBLES];
+    const uint64_t plane_stride = rows_padded * ldk;
+    kmaj::for_each_16(X, rows, K, rows_padded, ldk, 0xffffffffu, tile,
+        [&](uint64_t row) { return (row < rows) ? shift[row] : 0; },
+        [&](uint64_t row, uint64_t k, const double* x, int sh) {
+            Scaled s[16];
+#pragma unroll
+            for (int e = 0; e < 16; e++) s[e] = scaled_integer<true>(x[e], sh);
+            int8_t* out = planes + row * ldk + k;
+#pragma unroll 1
+            for (int l = 0; l < tbl.n; l++) {
+                v4u_t w;
+#pragma unroll
+                for (int g = 0; g < 4; g++)
+                    w[g] = pack4(fast_residue(s[4 * g], tbl, l), fast_residue(s[4 * g + 1], tbl, l),
+                                 fast_residue(s[4 * g + 2], tbl, l), fast_residue(s[4 * g + 3], tbl, l));
+                *(v4u_t*)(out + (uint64_t)l * plane_stride) = w;
+            }
+        });
+}
+
+/* Fractional CRT (metal_softfloat.h:4183-4246) in fp64. lut[l][b] is
+ * ((b mod p_l) q_l mod p_l) / p_l for the int8 value b, correctly rounded; a
+ * block keeps the table in LDS. One thread: four consecutive columns of a row.
+ * S stays in [0, 1): every term is below 1, so one conditional subtraction is the
+ * reduction modulo 1 the reference performs with floor. */
+__global__ __launch_bounds__(256)
+void fast_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t N, int n,
+                             const double* __restrict__ lut, double P,
+                             const int32_t* __restrict__ sh_a, const int32_t* __restrict__ sh_b,
+                             double* __restrict__ C) {
+    __shared__ double s_lut[FAST_MAX_MODULI * 256];
+    for (int i = threadIdx.x; i < n * 256; i += 256) s_lut[i] = lut[i];
+    __syncthreads();
+    const uint32_t cpr = (uint32_t)(((N + 3) / 4 + 255) / 256);
+    const uint64_t row = blockIdx.x / cpr;
+    const uint64_t col = ((uint64_t)(blockIdx.x % cpr) * 256 + threadIdx.x) * 4;
+    if (col >= N) return;
+    const uint64_t tot = M * N, idx = row * N + col;
+    const int nvalid = (N - col < 4) ? (int)(N - col) : 4;
+    const bool vec = (nvalid == 4) && ((N & 3) == 0) && (((uintptr_t)W & 3) == 0);
+    double S[4] = {0.0, 0.0, 0.0, 0.0};
+    for (int l = 0; l < n; l++) {
+        const int8_t* w = W + (uint64_t)l * tot + idx;
+        uint32_t u = 0;
+        if (vec) u = *(const uint32_t*)w;
+        else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) if (e < nvalid) u |= (uint32_t)(uint8_t)w[e] << (8 * e);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            double s = S[e] + s_lut[l * 256 + ((u >> (8 * e)) & 0xffu)];
+            if (s >= 1.0) s -= 1.0;
+            S[e] = s;
+        }
+    }
+    const int sa = sh_a[row];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        if (e >= nvalid) break;
+        double f = S[e];
+        if (f >= 0.5) f -= 1.0;                                    /* centre to [-0.5, 0.5) */
+        C[idx + e] = ldexp(f * P, -(sa + sh_b[col + e]));
+    }
+}
+
+/* ---- host side -------------------------------------------------------------- */
+
+struct FastPlan {
+    int n = 0, cap = 0, E = 0;
+    int moduli[FAST_MAX_MODULI] = {}, q[FAST_MAX_MODULI] = {};
+    double log2P = 0.0, P = 0.0;
+    FastTable table = {};
+};
+
+/* gpu_memory.mm:2802-2814 */
+std::vector<int> build_moduli(int cap, int n_mod) {
+    std::vector<int> pp;
+    for (int p = 2; p <= cap; p++) {
+        bool pr = true;
+        for (int d = 2; d * d <= p; d++) if (p % d == 0) { pr = false; break; }
+        if (!pr) continue;
+        long v = p, best = p;
+        while (v * p <= cap) { v *= p; best = v; }
+        pp.push_back((int)best);
+    }
+    std::sort(pp.begin(), pp.end(), std::greater<int>());
+    if ((int)pp.size() > n_mod) pp.resize((size_t)n_mod);
+    return pp;
+}
+
+long mod_inverse(long a, long m) {
+    long t = 0, nt = 1, r = m, nr = ((a % m) + m) % m;
+    while (nr != 0) { const long qq = r / nr; long x = t - qq * nt; t = nt; nt = x; x = r - qq * nr; r = nr; nr = x; }
+    return (t % m + m) % m;
+}
+
+/* gpu_memory.mm:2831-2857; 0, or -4 where the reference gives up */
+int make_plan(uint64_t K, int n_mod, FastPlan* out) {
+    FastPlan f;
+    int cap = (int)floor(2.0 * sqrt(16777216.0 / (double)K));
+    if (cap > 255) cap = 255;
+    while (cap > 2 && (double)K * floor(cap / 2.0) * floor(cap / 2.0) >= 16777216.0) cap--;
+    if (cap < 2) {
+        fprintf(stderr, "[GPU] Ozaki-II FAST: K=%llu too large for the tier's moduli; falling back\n", (unsigned long long)K);
+        return -4;
+    }
+    if (n_mod > FAST_MAX_MODULI) n_mod = FAST_MAX_MODULI;
+    if (n_mod < 2) n_mod = 2;
+    const std::vector<int> mod = build_moduli(cap, n_mod);
+    if (mod.size() < 2) {
+        fprintf(stderr, "[GPU] Ozaki-II FAST: too few coprime moduli <= cap %d; falling back\n", cap);
+        return -4;
+    }
+    f.n = (int)mod.size(); f.cap = cap;
+    unsigned __int128 P = 1;
+    for (int p : mod) P *= (unsigned)p;
+    for (int l = 0; l < f.n; l++) {
+        const int p = mod[(size_t)l];
+        f.moduli[l] = p;
+        f.q[l] = (int)mod_inverse((long)((P / (unsigned)p) % (unsigned)p), p);
+        f.log2P += log2((double)p);
+        const ByteWeights w = byte_weights(p);
+        f.table.p[l] = p; f.table.wlo[l] = w.lo; f.table.whi[l] = w.hi;
+        f.table.pinv[l] = 1.0f / (float)p;
+        f.table.neg_half[l] = (p % 2 == 0) ? (uint32_t)(256 - p / 2) & 0xffu : 0x100u;
+    }
+    f.table.n = f.n;
+    int E = (int)floor((f.log2P - log2((double)K) - 2.0) / 2.0);
+    if (E > 52) E = 52;
+    if (E < 1) E = 1;
+    f.E = E;
+    f.P = (double)P;
+    *out = f;
+    return 0;
+}
+
+/* Device-resident tables of the current moduli: identity pair lists and the
+ * moduli for the contraction, the fraction table for the reconstruction. */
+int32_t* g_tables = nullptr;    /* [0..16] pair_first, [17..32] plane index, [33..48] moduli */
+double* g_lut = nullptr;        /* [16][256] */
+int g_tables_key[FAST_MAX_MODULI + 1] = {};
+
+int ensure_tables(const FastPlan& f, hipStream_t st) {
+    int key[FAST_MAX_MODULI + 1] = {};
+    key[0] = f.n;
+    for (int l = 0; l < f.n; l++) key[l + 1] = f.moduli[l];
+    if (g_tables && memcmp(key, g_tables_key, sizeof key) == 0) return 0;
+    if (!g_tables && !ESHKOL_HIP_OK(hipMalloc((void**)&g_tables, 49 * sizeof(int32_t)))) return -1;
+    if (!g_lut && !ESHKOL_HIP_OK(hipMalloc((void**)&g_lut, FAST_MAX_MODULI * 256 * sizeof(double)))) return -1;
+    int32_t h[49] = {};
+    for (int i = 0; i <= 16; i++) h[i] = i;
+    for (int i = 0; i < 16; i++) h[17 + i] = i;
+    for (int l = 0; l < f.n; l++) h[33 + l] = f.moduli[l];
+    std::vector<double> lut((size_t)FAST_MAX_MODULI * 256, 0.0);
+    for (int l = 0; l < f.n; l++) {
+        const int p = f.moduli[l];
+        for (int b = 0; b < 256; b++) {
+            const int w = (int)(int8_t)(uint8_t)b;
+            const int gg = ((w % p) + p) % p;
+            const int u = (gg * f.q[l]) % p;
+            lut[(size_t)l * 256 + (size_t)b] = (double)u / (double)p;
+        }
+    }
+    /* pageable sources: the copies are complete when the calls return */
+    if (!ESHKOL_HIP_OK(hipMemcpyAsync(g_tables, h, sizeof h, hipMemcpyHostToDevice, st)) ||
+        !ESHKOL_HIP_OK(hipMemcpyAsync(g_lut, lut.data(), lut.size() * sizeof(double), hipMemcpyHostToDevice, st)) ||
+        !ESHKOL_HIP_OK(hipStreamSynchronize(st))) return -1;
+    memcpy(g_tables_key, key, sizeof key);
+    return 0;
+}
+
+HipOzakiFastStages g_last = {};
+
+int split_any(const double* X, uint64_t rows, uint64_t K, const int32_t* shift, const FastTable& tbl,
+              int8_t* planes, uint64_t rows_padded, uint64_t ldk, bool kmajor, hipStream_t st) {
+    if (kmajor) {
+        if (kmaj::tile_count(rows_padded, ldk) > 0x7fffffffULL) return -1;
+        const dim3 grid((unsigned)kmaj::grid_blocks(rows_padded, ldk, eshkol_hip_num_cus()));
+        hipLaunchKernelGGL(fast_split_kmajor_kernel, grid, dim3(256), 0, st, X, rows, K, shift, tbl, planes,
+                           rows_padded, ldk);
+    } else {
+        const uint64_t nblk = ((ldk + 1023) / 1024) * rows_padded;
+        if (nblk > 0x7fffffffULL) return -1;
+        hipLaunchKernelGGL(fast_split_kernel, dim3((unsigned)nblk), dim3(256), 0, st, X, rows, K, shift, tbl, planes,
+                           rows_padded, ldk);
+    }
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
+}  // namespace
+
+extern "C" int hip_ozaki_fast_last_stages(HipOzakiFastStages* out) {
+    if (!out || !g_last.a_planes) return -1;
+    *out = g_last;
+    return 0;
+}
+
+extern "C" int hip_matmul_ozaki_fast_f64_ex(const double* A, const double* B, double* C,
+                                            uint64_t M, uint64_t K, uint64_t N,
+                                            int trans_a, int trans_b, int num_moduli, void* stream) {
+    if (!A || !B || !C || M == 0 || K == 0 || N == 0) return -1;
+    if (M > 0x7fffffffULL || N > 0x7fffffffULL) return -1;
+    if (K > 131071) return -4;          /* the contraction's int32 bound; the reference's f32 bound is 2^24 / (p/2)^2 */
+    FastPlan f;
+    const int prc = make_plan(K, num_moduli, &f);
+    if (prc != 0) return prc;
+    hipStream_t st = (hipStream_t)stream;
+    if (ensure_tables(f, st) != 0) return -1;
+    fprintf(stderr, "[GPU] Ozaki-II FAST: n_mod=%d E=%d cap=%d log2(P)=%.1f (int8 MFMA GEMMs)\n",
+            f.n, f.E, f.cap, f.log2P);                                  /* gpu_memory.mm:2859 */
+
+    const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ldk = round_up_sz(K, 256);
+    const bool a_kmajor = trans_a != 0, b_kmajor = trans_b == 0;
+    double* amax = (double*)eshkol_hip_workspace(WS_ROWSCALE, M * sizeof(double));
+    double* bmax = (double*)eshkol_hip_workspace(WS_COLSCALE, N * sizeof(double));
+    int32_t* sha = (int32_t*)eshkol_hip_workspace(WS_ROWSHIFT, M * sizeof(int32_t));
+    int32_t* shb = (int32_t*)eshkol_hip_workspace(WS_COLSHIFT, N * sizeof(int32_t));
+    int8_t* Ap = (int8_t*)eshkol_hip_workspace(WS_APLANES, (size_t)f.n * Mp * ldk);
+    int8_t* Bp = (int8_t*)eshkol_hip_workspace(WS_BPLANES, (size_t)f.n * Np * ldk);
+    int8_t* Wp = (int8_t*)eshkol_hip_workspace(WS_PRODUCTS, (size_t)f.n * M * N);
+    if (!amax || !bmax || !sha || !shb || !Ap || !Bp || !Wp) return -2;
+
+    if ((a_kmajor ? hip_colabsmax_f64(A, K, M, 0.0, amax, st) : hip_rowabsmax_f64(A, M, K, 0.0, amax, st)) != 0) return -1;
+    if ((b_kmajor ? hip_colabsmax_f64(B, K, N, 0.0, bmax, st) : hip_rowabsmax_f64(B, N, K, 0.0, bmax, st)) != 0) return -1;
+    /* frexp exponent e = floor(log2 max) + 1 (gpu_memory.mm:2886-2905); the split
+     * scales by 2^(E - e), so the per-row shift is (E - 1) - floor(log2 max) */
+    CrtMaxima mx[2];
+    if (eshkol_crt_scan_exponents(amax, M, bmax, N, sha, shb, mx, st) != 0) return -1;
+    if (mx[0].nonfinite || mx[1].nonfinite) return -1;                  /* NaN / Inf: not this tier's business */
+    eshkol_crt_shifts_from_exponents(sha, M, shb, N, f.E - 1, st);
+
+    if (split_any(A, M, K, sha, f.table, Ap, Mp, ldk, a_kmajor, st) != 0) return -1;
+    if (split_any(B, N, K, shb, f.table, Bp, Np, ldk, b_kmajor, st) != 0) return -1;
+
+    HipIgemmArgs ga;
+    memset(&ga, 0, sizeof ga);
+    ga.a_planes = Ap; ga.b_planes = Bp;
+    ga.a_plane_stride = Mp * ldk; ga.b_plane_stride = Np * ldk;
+    ga.ldk = (uint32_t)ldk; ga.M = (uint32_t)M; ga.N = (uint32_t)N; ga.n_out = (uint32_t)f.n;
+    ga.pair_first = g_tables; ga.pair_a = g_tables + 17; ga.pair_b = g_tables + 17;
+    ga.mode = 1; ga.max_pairs = 1; ga.modulus = g_tables + 33; ga.out_i8 = Wp;
+    if (hip_igemm_i8(&ga, st) != 0) return -1;
+
+    const uint64_t nblk = (((N + 3) / 4 + 255) / 256) * M;
+    if (nblk > 0x7fffffffULL) return -1;
+    hipLaunchKernelGGL(fast_reconstruct_kernel, dim3((unsigned)nblk), dim3(256), 0, st,
+                       Wp, M, N, f.n, g_lut, f.P, sha, shb, C);
+    if (!ESHKOL_HIP_OK(hipGetLastError())) return -3;
+
+    g_last.a_planes = Ap; g_last.b_planes = Bp; g_last.w_planes = Wp;
+    g_last.shift_a = sha; g_last.shift_b = shb;
+    g_last.rows_a_padded = Mp; g_last.rows_b_padded = Np; g_last.ldk = ldk;
+    g_last.num_moduli = f.n; g_last.E = f.E; g_last.cap = f.cap;
+    for (int l = 0; l < FAST_MAX_MODULI; l++) g_last.moduli[l] = (l < f.n) ? f.moduli[l] : 0;
+    return 0;
+}
+
+extern "C" int hip_matmul_ozaki_fast_f64(const double* A, const double* B, double* C,
+                                         uint64_t M, uint64_t K, uint64_t N, int num_moduli, void* stream) {
+    return hip_matmul_ozaki_fast_f64_ex(A, B, C, M, K, N, 0, 0, num_moduli, stream);
+}

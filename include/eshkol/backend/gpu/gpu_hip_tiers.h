@@ -167,6 +167,35 @@ typedef struct {
 } HipOzakiCrtStages;
 int hip_ozaki_crt_last_stages(HipOzakiCrtStages* out);
 
+/* ---- Ozaki-II reduced-precision ("fast") CRT tier -------------------------------
+ * ozaki_ii_fast_dispatch (lib/backend/gpu/gpu_memory.mm:2816-3012): the n largest
+ * prime powers below a K-dependent cap as moduli (gpu_memory.mm:2802-2842),
+ * power-of-two scaling by the frexp exponents of the row / column maxima,
+ * round-half-up integer split (metal_softfloat.h:4148-4178), exact modular
+ * products, fractional CRT (metal_softfloat.h:4183-4246; here in fp64 instead of
+ * float pairs). num_moduli is the accuracy knob, [2, 16], clamped; the
+ * reference's default is 11 (about 1e-8). Returns 0, -4 where the reference
+ * gives up (K too large for the moduli, fewer than two moduli under the cap),
+ * -1 on non-finite input or a device error, -2 when workspace cannot be had. */
+int hip_matmul_ozaki_fast_f64(const double* A, const double* B, double* C,
+                              uint64_t M, uint64_t K, uint64_t N, int num_moduli, void* stream);
+
+/* Device pointers to the stages of the last hip_matmul_ozaki_fast_f64 call (valid
+ * until the next tier call): residue planes [l][row padded to 256][ldk] of A and
+ * of B^T, product residues [l][M][N], the per-row and per-column shifts
+ * E - frexp exponent (0 for an all-zero row), and the moduli. */
+typedef struct {
+    const int8_t* a_planes;
+    const int8_t* b_planes;
+    const int8_t* w_planes;
+    const int32_t* shift_a;
+    const int32_t* shift_b;
+    uint64_t rows_a_padded, rows_b_padded, ldk;
+    int32_t num_moduli, E, cap;
+    int32_t moduli[16];
+} HipOzakiFastStages;
+int hip_ozaki_fast_last_stages(HipOzakiFastStages* out);
+
 /* ---- INT8 slice tier ----------------------------------------------------------
  * s base-128 slices of X[i,k] / scale[i] (gpu_cuda_kernels.cu:688-723):
  * planes[p][i][k], pitch ldk, rows_padded rows per plane, padding zero. With
@@ -228,6 +257,9 @@ int hip_convert_f64_to_16_kmajor(const double* in, uint16_t* out, uint64_t rows,
  * The Ozaki and reduced tiers turn both operands into planes [row][k]; an
  * operand stored k-major is read through LDS tiles, so neither form costs a
  * transposed copy. */
+int hip_matmul_ozaki_fast_f64_ex(const double* A, const double* B, double* C,
+                                 uint64_t M, uint64_t K, uint64_t N,
+                                 int trans_a, int trans_b, int num_moduli, void* stream);
 int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, double* C,
                                 uint64_t M, uint64_t K, uint64_t N,
                                 int trans_a, int trans_b, int num_moduli, int adaptive,

@@ -105,3 +105,34 @@ def run_reduced(A, B, dtype, round_output):
                                           dtype, 1 if round_output else 0, stream())
     assert rc == 0
     return ops.result()
+
+
+def run_fast(A, B, n_mod=11, want_stages=True, trans=None):
+    """The reduced-precision CRT tier on the device; trans = (trans_a, trans_b) hands the
+    operands over transposed (A as [K][M] / B as [N][K])."""
+    lib = ea.load()
+    ops = Operands(A, B)
+    if trans is None:
+        rc = lib.hip_matmul_ozaki_fast_f64(ops.dA.ptr, ops.dB.ptr, ops.dC.ptr, ops.M, ops.K, ops.N, n_mod, stream())
+    else:
+        ta, tb = trans
+        dA = ea.DeviceArray.from_host(np.ascontiguousarray(A.T)) if ta else ops.dA
+        dB = ea.DeviceArray.from_host(np.ascontiguousarray(B.T)) if tb else ops.dB
+        rc = lib.hip_matmul_ozaki_fast_f64_ex(dA.ptr, dB.ptr, ops.dC.ptr, ops.M, ops.K, ops.N, ta, tb, n_mod, stream())
+    if rc != 0:
+        return rc, None, None
+    Cg = ops.result()
+    if not want_stages:
+        return 0, Cg, None
+    sg = ea.HipOzakiFastStages()
+    assert lib.hip_ozaki_fast_last_stages(C.byref(sg)) == 0
+    n, M, K, N = sg.num_moduli, ops.M, ops.K, ops.N
+    ap = ea.download_raw(sg.a_planes, (n, sg.rows_a_padded, sg.ldk), np.int8)
+    bp = ea.download_raw(sg.b_planes, (n, sg.rows_b_padded, sg.ldk), np.int8)
+    st = dict(num_moduli=n, E=sg.E, cap=sg.cap, moduli=list(sg.moduli[:n]),
+              shift_a=ea.download_raw(sg.shift_a, (M,), np.int32), shift_b=ea.download_raw(sg.shift_b, (N,), np.int32),
+              a_planes=ap[:, :M, :K], b_planes=bp[:, :N, :K],
+              a_pad_clear=(not ap[:, M:, :].any()) and (not ap[:, :, K:].any()),
+              b_pad_clear=(not bp[:, N:, :].any()) and (not bp[:, :, K:].any()),
+              w_planes=ea.download_raw(sg.w_planes, (n, M, N), np.int8))
+    return 0, Cg, st

@@ -271,6 +271,38 @@ assert normwise(small, oracle.matmul_f64(A[:256, :256], B[:256, :256]), A[:256, 
     assert "out of range" in r.stderr                                          # loud clamp, still correct
 
 
+def test_tier_override_fast_crt(gpu):
+    """ESHKOL_OZAKI_FAST / ESHKOL_SF64_KERNEL=ozaki-fast (gpu_memory.mm:1319-1343): the reduced-precision
+    CRT tier first, the exact tier behind it when it declines; the moduli knob clamps loudly."""
+    body = r"""
+n = 512
+A = synth.normal(1, (n, n)); B = synth.normal(2, (n, n))
+got = ea.matmul_dispatch(A, B)
+n_mod = int(os.environ.get("EXPECT_MODULI", "11"))
+rc, want = oracle.matmul_ozaki_fast(A, B, n_mod)
+ref = A @ B
+# the oracle reconstructs in float pairs (2^-45 of P), the device in fp64: with 16 moduli P outgrows
+# the products and the float pairs lose more than the 11-modulus tier does
+assert rc == 0 and np.abs(got - want).max() <= (1e-9 if n_mod == 11 else 2e-8) * np.abs(ref).max()
+assert np.abs(got - ref).max() <= 5e-8 * np.abs(ref).max()
+bad = A.copy(); bad[3, 3] = np.inf                      # the fast tier declines, the exact tier declines, native answers
+out = ea.matmul_dispatch(bad, B)
+assert np.isinf(out[3]).any() or np.isnan(out[3]).any()
+"""
+    for env in ({"ESHKOL_OZAKI_FAST": "1"}, {"ESHKOL_SF64_KERNEL": "ozaki-fast"}, {"ESHKOL_HIP_F64_KERNEL": "ozaki-fast"}):
+        env = dict(env, ESHKOL_GPU_THRESHOLD="1", ESHKOL_GPU_VERBOSE="1", ESHKOL_OZAKI_PROFILE="1")
+        r = run_child(body, env)
+        assert "[GPU] Ozaki-II FAST tier ENABLED: N=11 moduli" in r.stderr
+        assert "[GPU] Ozaki-II FAST: n_mod=11 E=" in r.stderr and "[OZAKI_PROFILE] fast M=512" in r.stderr
+        assert "[GPU] Ozaki-II FAST dispatch returned -1; falling back to exact tier" in r.stderr
+    r = run_child(body, {"ESHKOL_OZAKI_FAST": "1", "ESHKOL_OZAKI_FAST_MODULI": "40", "EXPECT_MODULI": "16",
+                         "ESHKOL_GPU_THRESHOLD": "1"})
+    assert "ESHKOL_OZAKI_FAST_MODULI=40 out of range [2,16]; clamping to 16" in r.stderr
+    r = run_child("A = synth.normal(1, (512, 512)); ea.matmul_dispatch(A, A)",
+                  {"ESHKOL_OZAKI_FAST": "0", "ESHKOL_GPU_THRESHOLD": "1", "ESHKOL_GPU_VERBOSE": "1"})
+    assert "FAST" not in r.stderr and "native fp64 MFMA" in r.stderr           # "0" leaves it off
+
+
 def test_tier_override_int8_and_budget_selector(gpu):
     body = r"""
 n = 1024
