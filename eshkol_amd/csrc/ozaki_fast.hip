@@ -139,14 +139,20 @@ void fast_split_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint6
  * ((b mod p_l) q_l mod p_l) / p_l for the int8 value b, correctly rounded; a
  * block keeps the table in LDS. One thread: four consecutive columns of a row.
  * S stays in [0, 1): every term is below 1, so one conditional subtraction is the
- * reduction modulo 1 the reference performs with floor. */
+ * reduction modulo 1 the reference performs with floor.
+ * The number of planes is a template parameter so that a thread's loads of all
+ * planes are issued together (the kernel moves 8 + n bytes per element and has
+ * to keep HBM busy). */
+template <int NMOD>
 __global__ __launch_bounds__(256)
-void fast_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t N, int n,
+void fast_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t N,
                              const double* __restrict__ lut, double P,
                              const int32_t* __restrict__ sh_a, const int32_t* __restrict__ sh_b,
                              double* __restrict__ C) {
     __shared__ double s_lut[FAST_MAX_MODULI * 256];
-    for (int i = threadIdx.x; i < n * 256; i += 256) s_lut[i] = lut[i];
+    constexpr int n = NMOD;
+#pragma unroll
+    for (int i = 0; i < NMOD; i++) s_lut[i * 256 + threadIdx.x] = lut[i * 256 + threadIdx.x];
     __syncthreads();
     const uint32_t cpr = (uint32_t)(((N + 3) / 4 + 255) / 256);
     const uint64_t row = blockIdx.x / cpr;
@@ -155,29 +161,47 @@ void fast_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t 
     const uint64_t tot = M * N, idx = row * N + col;
     const int nvalid = (N - col < 4) ? (int)(N - col) : 4;
     const bool vec = (nvalid == 4) && ((N & 3) == 0) && (((uintptr_t)W & 3) == 0);
-    double S[4] = {0.0, 0.0, 0.0, 0.0};
-    for (int l = 0; l < n; l++) {
-        const int8_t* w = W + (uint64_t)l * tot + idx;
-        uint32_t u = 0;
-        if (vec) u = *(const uint32_t*)w;
-        else {
+    uint32_t u[NMOD];
+    if (vec) {
 #pragma unroll
-            for (int e = 0; e < 4; e++) if (e < nvalid) u |= (uint32_t)(uint8_t)w[e] << (8 * e);
+        for (int l = 0; l < NMOD; l++) u[l] = *(const uint32_t*)(W + (uint64_t)l * tot + idx);
+    } else {
+#pragma unroll
+        for (int l = 0; l < NMOD; l++) {
+            const int8_t* w = W + (uint64_t)l * tot + idx;
+            u[l] = 0;
+#pragma unroll
+            for (int e = 0; e < 4; e++) if (e < nvalid) u[l] |= (uint32_t)(uint8_t)w[e] << (8 * e);
         }
+    }
+    int sb[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int e = 0; e < 4; e++) if (e < nvalid) sb[e] = sh_b[col + e];
+    double S[4] = {0.0, 0.0, 0.0, 0.0};
+#pragma unroll
+    for (int l = 0; l < n; l++) {
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            double s = S[e] + s_lut[l * 256 + ((u >> (8 * e)) & 0xffu)];
+            double s = S[e] + s_lut[l * 256 + ((u[l] >> (8 * e)) & 0xffu)];
             if (s >= 1.0) s -= 1.0;
             S[e] = s;
         }
     }
     const int sa = sh_a[row];
+    double out[4];
 #pragma unroll
     for (int e = 0; e < 4; e++) {
-        if (e >= nvalid) break;
         double f = S[e];
         if (f >= 0.5) f -= 1.0;                                    /* centre to [-0.5, 0.5) */
-        C[idx + e] = ldexp(f * P, -(sa + sh_b[col + e]));
+        out[e] = ldexp(f * P, -(sa + sb[e]));
+    }
+    if (vec && (((uintptr_t)C & 15) == 0)) {
+        d2_t lo, hi;
+        lo.x = out[0]; lo.y = out[1]; hi.x = out[2]; hi.y = out[3];
+        ((d2_t*)(C + idx))[0] = lo; ((d2_t*)(C + idx))[1] = hi;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) if (e < nvalid) C[idx + e] = out[e];
     }
 }
 
@@ -361,8 +385,14 @@ extern "C" int hip_matmul_ozaki_fast_f64_ex(const double* A, const double* B, do
 
     const uint64_t nblk = (((N + 3) / 4 + 255) / 256) * M;
     if (nblk > 0x7fffffffULL) return -1;
-    hipLaunchKernelGGL(fast_reconstruct_kernel, dim3((unsigned)nblk), dim3(256), 0, st,
-                       Wp, M, N, f.n, g_lut, f.P, sha, shb, C);
+    switch (f.n) {
+#define CASE(n) case n: hipLaunchKernelGGL(fast_reconstruct_kernel<n>, dim3((unsigned)nblk), dim3(256), 0, st, \
+                                           Wp, M, N, g_lut, f.P, sha, shb, C); break;
+        CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8) CASE(9)
+        CASE(10) CASE(11) CASE(12) CASE(13) CASE(14) CASE(15) CASE(16)
+#undef CASE
+        default: return -1;
+    }
     if (!ESHKOL_HIP_OK(hipGetLastError())) return -3;
 
     g_last.a_planes = Ap; g_last.b_planes = Bp; g_last.w_planes = Wp;
