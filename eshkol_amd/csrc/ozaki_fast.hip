@@ -135,25 +135,26 @@ void fast_split_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint6
         });
 }
 
-/* Fractional CRT (metal_softfloat.h:4183-4246) in fp64. lut[l][b] is
- * ((b mod p_l) q_l mod p_l) / p_l for the int8 value b, correctly rounded; a
- * block keeps the table in LDS. One thread: four consecutive columns of a row.
- * S stays in [0, 1): every term is below 1, so one conditional subtraction is the
- * reduction modulo 1 the reference performs with floor.
- * The number of planes is a template parameter so that a thread's loads of all
- * planes are issued together (the kernel moves 8 + n bytes per element and has
- * to keep HBM busy). */
+/* Fractional CRT (metal_softfloat.h:4183-4246): frac(sum_l ((w_l q_l) mod p_l) / p_l),
+ * centred, times P 2^(e_i + f_j - 2E). The fractions are added in 64-bit fixed
+ * point, where "modulo 1" is the wrap of the integer and "centred" is reading it
+ * as signed: with d_l = floor(2^64 q_l / p_l), w_l d_l mod 2^64 is
+ * frac(w_l q_l / p_l) to within |w_l| 2^-64, so no modular reduction of w_l q_l is
+ * needed at all. d_l is held as four 16-bit limbs and each limb's sum over the
+ * moduli is one 24-bit multiply-add per residue into a 32-bit register
+ * (16 * 128 * 65535 < 2^27); the limbs are put together once per element. Total
+ * error below 2^-53 of P (the reference's float pairs resolve about 2^-45).
+ * One thread: four consecutive columns of a row. The number of planes is a
+ * template parameter so that a thread's loads of all planes are issued together
+ * (the kernel moves 8 + n bytes per element and has to keep HBM busy). */
+struct FracLimbs { int32_t d[FAST_MAX_MODULI][4]; };
+
 template <int NMOD>
 __global__ __launch_bounds__(256)
 void fast_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t N,
-                             const double* __restrict__ lut, double P,
+                             FracLimbs fl, double P_over_2_64,
                              const int32_t* __restrict__ sh_a, const int32_t* __restrict__ sh_b,
                              double* __restrict__ C) {
-    __shared__ double s_lut[FAST_MAX_MODULI * 256];
-    constexpr int n = NMOD;
-#pragma unroll
-    for (int i = 0; i < NMOD; i++) s_lut[i * 256 + threadIdx.x] = lut[i * 256 + threadIdx.x];
-    __syncthreads();
     const uint32_t cpr = (uint32_t)(((N + 3) / 4 + 255) / 256);
     const uint64_t row = blockIdx.x / cpr;
     const uint64_t col = ((uint64_t)(blockIdx.x % cpr) * 256 + threadIdx.x) * 4;
@@ -177,23 +178,29 @@ void fast_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t 
     int sb[4] = {0, 0, 0, 0};
 #pragma unroll
     for (int e = 0; e < 4; e++) if (e < nvalid) sb[e] = sh_b[col + e];
-    double S[4] = {0.0, 0.0, 0.0, 0.0};
+    int32_t acc[4][4];
 #pragma unroll
-    for (int l = 0; l < n; l++) {
+    for (int e = 0; e < 4; e++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[e][j] = 0;
+#pragma unroll
+    for (int l = 0; l < NMOD; l++) {
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            double s = S[e] + s_lut[l * 256 + ((u[l] >> (8 * e)) & 0xffu)];
-            if (s >= 1.0) s -= 1.0;
-            S[e] = s;
+            const int w = (int)(int8_t)(u[l] >> (8 * e));
+#pragma unroll
+            for (int j = 0; j < 4; j++) acc[e][j] += __mul24(w, fl.d[l][j]);
         }
     }
     const int sa = sh_a[row];
     double out[4];
 #pragma unroll
     for (int e = 0; e < 4; e++) {
-        double f = S[e];
-        if (f >= 0.5) f -= 1.0;                                    /* centre to [-0.5, 0.5) */
-        out[e] = ldexp(f * P, -(sa + sb[e]));
+        const int64_t S = (int64_t)acc[e][0] + ((int64_t)acc[e][1] << 16) + ((int64_t)acc[e][2] << 32) +
+                          (int64_t)((uint64_t)(int64_t)acc[e][3] << 48);
+        /* S / 2^64 is the centred fraction; (double)S in two halves */
+        const double f = fma((double)(int32_t)(S >> 32), 4294967296.0, (double)(uint32_t)S);
+        out[e] = ldexp(f * P_over_2_64, -(sa + sb[e]));
     }
     if (vec && (((uintptr_t)C & 15) == 0)) {
         d2_t lo, hi;
@@ -212,6 +219,7 @@ struct FastPlan {
     int moduli[FAST_MAX_MODULI] = {}, q[FAST_MAX_MODULI] = {};
     double log2P = 0.0, P = 0.0;
     FastTable table = {};
+    FracLimbs limbs = {};
 };
 
 /* gpu_memory.mm:2802-2814 */
@@ -265,6 +273,8 @@ int make_plan(uint64_t K, int n_mod, FastPlan* out) {
         f.table.p[l] = p; f.table.wlo[l] = w.lo; f.table.whi[l] = w.hi;
         f.table.pinv[l] = 1.0f / (float)p;
         f.table.neg_half[l] = (p % 2 == 0) ? (uint32_t)(256 - p / 2) & 0xffu : 0x100u;
+        const unsigned __int128 d = (((unsigned __int128)(unsigned)f.q[l]) << 64) / (unsigned)p;   /* < 2^64: q < p */
+        for (int j = 0; j < 4; j++) f.limbs.d[l][j] = (int32_t)((uint64_t)(d >> (16 * j)) & 0xffffu);
     }
     f.table.n = f.n;
     int E = (int)floor((f.log2P - log2((double)K) - 2.0) / 2.0);
@@ -277,9 +287,8 @@ int make_plan(uint64_t K, int n_mod, FastPlan* out) {
 }
 
 /* Device-resident tables of the current moduli: identity pair lists and the
- * moduli for the contraction, the fraction table for the reconstruction. */
+ * moduli for the contraction. */
 int32_t* g_tables = nullptr;    /* [0..16] pair_first, [17..32] plane index, [33..48] moduli */
-double* g_lut = nullptr;        /* [16][256] */
 int g_tables_key[FAST_MAX_MODULI + 1] = {};
 
 int ensure_tables(const FastPlan& f, hipStream_t st) {
@@ -288,24 +297,12 @@ int ensure_tables(const FastPlan& f, hipStream_t st) {
     for (int l = 0; l < f.n; l++) key[l + 1] = f.moduli[l];
     if (g_tables && memcmp(key, g_tables_key, sizeof key) == 0) return 0;
     if (!g_tables && !ESHKOL_HIP_OK(hipMalloc((void**)&g_tables, 49 * sizeof(int32_t)))) return -1;
-    if (!g_lut && !ESHKOL_HIP_OK(hipMalloc((void**)&g_lut, FAST_MAX_MODULI * 256 * sizeof(double)))) return -1;
     int32_t h[49] = {};
     for (int i = 0; i <= 16; i++) h[i] = i;
     for (int i = 0; i < 16; i++) h[17 + i] = i;
     for (int l = 0; l < f.n; l++) h[33 + l] = f.moduli[l];
-    std::vector<double> lut((size_t)FAST_MAX_MODULI * 256, 0.0);
-    for (int l = 0; l < f.n; l++) {
-        const int p = f.moduli[l];
-        for (int b = 0; b < 256; b++) {
-            const int w = (int)(int8_t)(uint8_t)b;
-            const int gg = ((w % p) + p) % p;
-            const int u = (gg * f.q[l]) % p;
-            lut[(size_t)l * 256 + (size_t)b] = (double)u / (double)p;
-        }
-    }
-    /* pageable sources: the copies are complete when the calls return */
+    /* pageable source: the copy is complete when the calls return */
     if (!ESHKOL_HIP_OK(hipMemcpyAsync(g_tables, h, sizeof h, hipMemcpyHostToDevice, st)) ||
-        !ESHKOL_HIP_OK(hipMemcpyAsync(g_lut, lut.data(), lut.size() * sizeof(double), hipMemcpyHostToDevice, st)) ||
         !ESHKOL_HIP_OK(hipStreamSynchronize(st))) return -1;
     memcpy(g_tables_key, key, sizeof key);
     return 0;
@@ -387,7 +384,7 @@ extern "C" int hip_matmul_ozaki_fast_f64_ex(const double* A, const double* B, do
     if (nblk > 0x7fffffffULL) return -1;
     switch (f.n) {
 #define CASE(n) case n: hipLaunchKernelGGL(fast_reconstruct_kernel<n>, dim3((unsigned)nblk), dim3(256), 0, st, \
-                                           Wp, M, N, g_lut, f.P, sha, shb, C); break;
+                                           Wp, M, N, f.limbs, ldexp(f.P, -64), sha, shb, C); break;
         CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8) CASE(9)
         CASE(10) CASE(11) CASE(12) CASE(13) CASE(14) CASE(15) CASE(16)
 #undef CASE
