@@ -21,6 +21,7 @@ LIB = os.path.join(LIBDIR, "libeshkol_gpu_hip.so")
 
 SOURCES = [
     "gpu_memory_hip.cpp",
+    "host_copy.cpp",
     "dgemm_f64.hip",
     "igemm_i8.hip",
     "hgemm_16.hip",

@@ -17,6 +17,7 @@
  * A tier that returns nonzero falls through to the native GEMM.
  */
 #include "hip_common.h"
+#include "host_copy.h"
 #include "kernels.h"
 #include "tiers.h"
 #include "eshkol/backend/gpu/gpu_memory.h"
@@ -51,6 +52,9 @@ std::mutex g_init_mutex;
 /* One stream, one workspace: GPU work from concurrent callers is serialised. */
 std::recursive_mutex g_gpu_mutex;
 hipStream_t g_stream = nullptr;
+/* second queue, for host copies that run beside the kernels of g_stream */
+hipStream_t g_copy_stream = nullptr;
+hipEvent_t g_ev_up = nullptr, g_ev_done[2] = {nullptr, nullptr};
 char g_arch[64] = "";
 
 constexpr uint32_t FLAG_WRAPPED_HOST = 1u << 0;   /* host memory is the caller's   */
@@ -93,6 +97,7 @@ struct TierEnv {
     bool profile = false;
     double budget = -1.0;        /* < 0: selector off */
     int  precision = 0;          /* ESHKOL_GPU_PRECISION: 0 exact, 1 high, 2 fast, 3 ml */
+    bool overlap = true;         /* ESHKOL_GPU_OVERLAP=0: no row panels in the host-memory dispatch */
 };
 TierEnv g_env;
 std::once_flag g_env_once;
@@ -136,6 +141,7 @@ void parse_env(void) {
     const char* ad = getenv("ESHKOL_OZAKI_ADAPTIVE");            /* gpu_memory.mm:2494 */
     e.adaptive = ad && strcmp(ad, "1") == 0;
     e.profile = getenv("ESHKOL_OZAKI_PROFILE") != nullptr;       /* gpu_memory.mm:2479 */
+    if (const char* o = getenv("ESHKOL_GPU_OVERLAP")) e.overlap = strcmp(o, "0") != 0;
     if (const char* a = getenv("ESHKOL_MATMUL_ACCURACY")) {      /* gpu_memory_cuda.cpp:527-539 */
         if (*a) {
             if (!strcmp(a, "fast")) e.budget = 1e-2;
@@ -309,8 +315,12 @@ int hip_wrap(void* host_ptr, size_t size_bytes, bool upload, bool copy_back, Esh
     void* d = staging_get(size_bytes);
     if (!d) return -1;
     if (upload) {
-        if (!ESHKOL_HIP_OK(hipMemcpyAsync(d, host_ptr, size_bytes, hipMemcpyHostToDevice, g_stream)) ||
-            !ESHKOL_HIP_OK(hipStreamSynchronize(g_stream))) { staging_put(d); return -1; }
+        /* returns once host_ptr has been read; the tail of the copy is ordered on g_stream */
+        if (eshkol_hip_upload(d, host_ptr, size_bytes, g_stream) != 0) {
+            (void)hipStreamSynchronize(g_stream);
+            staging_put(d);
+            return -1;
+        }
     }
     out->host_ptr = host_ptr;
     out->device_ptr = d;
@@ -326,13 +336,12 @@ int hip_sync(EshkolGPUBuffer* b, EshkolSyncDirection dir) {
     if (!ESHKOL_HIP_OK(hipStreamSynchronize(g_stream))) return -1;
     if ((b->flags & FLAG_WRAPPED_HOST) && b->backend_data && b->device_ptr) {
         if (dir == ESHKOL_SYNC_DEVICE_TO_HOST || dir == ESHKOL_SYNC_BIDIRECTIONAL) {
-            if (!ESHKOL_HIP_OK(hipMemcpy(b->backend_data, b->device_ptr, b->size_bytes,
-                                         hipMemcpyDeviceToHost))) return -1;
+            if (eshkol_hip_download(b->backend_data, b->device_ptr, b->size_bytes, g_stream) != 0) return -1;
             b->flags |= FLAG_HOST_CURRENT;
         }
         if (dir == ESHKOL_SYNC_HOST_TO_DEVICE) {
-            if (!ESHKOL_HIP_OK(hipMemcpy(b->device_ptr, b->backend_data, b->size_bytes,
-                                         hipMemcpyHostToDevice))) return -1;
+            if (eshkol_hip_upload(b->device_ptr, b->backend_data, b->size_bytes, g_stream) != 0 ||
+                !ESHKOL_HIP_OK(hipStreamSynchronize(g_stream))) return -1;
             b->flags |= FLAG_HOST_CURRENT;
         }
     }
@@ -345,7 +354,7 @@ void hip_free(EshkolGPUBuffer* b) {
         if (b->flags & FLAG_RESIDENT) return;
         if ((b->flags & FLAG_COPY_BACK) && !(b->flags & FLAG_HOST_CURRENT) &&
             b->backend_data && b->device_ptr)
-            hipMemcpy(b->backend_data, b->device_ptr, b->size_bytes, hipMemcpyDeviceToHost);
+            (void)eshkol_hip_download(b->backend_data, b->device_ptr, b->size_bytes, g_stream);
         if (b->device_ptr) staging_put(b->device_ptr);
         return;
     }
@@ -361,73 +370,84 @@ bool is_hip_buffer(const EshkolGPUBuffer* b) { return b && b->backend == ESHKOL_
 
 /* ---- matmul tiers -------------------------------------------------------- */
 
-/* C[MxN] = op(A)*op(B) on the tier the environment selects; ta/tb mark an
- * operand the caller holds transposed (A as [K][M], B as [N][K]). */
-int hip_matmul_f64(EshkolGPUBuffer* A, EshkolGPUBuffer* B, EshkolGPUBuffer* C,
-                   uint64_t M, uint64_t K, uint64_t N, int ta = 0, int tb = 0) {
-    const TierEnv& env = tier_env();
-    const double* dA = (const double*)A->device_ptr;
-    const double* dB = (const double*)B->device_ptr;
-    double* dC = (double*)C->device_ptr;
-    if (A->size_bytes < M * K * sizeof(double) || B->size_bytes < K * N * sizeof(double) ||
-        C->size_bytes < M * N * sizeof(double)) return -1;
-    const double work = 2.0 * (double)M * (double)K * (double)N;
-
+/* The tier the environment selects for a product of this shape. */
+struct TierChoice {
+    bool fast = false;     /* try the reduced-precision CRT tier first */
     int tier = 0;          /* 0 native, 1 INT8 slices, 2 CRT */
-    /* The reduced-precision CRT tier comes first when it is switched on, and a miss
-     * falls through to the exact tier, never to a wrong result (gpu_memory.mm:3036-3052). */
-    if (env.ozaki_fast && M >= 512 && K >= 512 && N >= 512) {
+    int T = 0;
+    double pred = 1.0;
+    const char* why = "default";
+};
+
+TierChoice choose_tier(uint64_t M, uint64_t K, uint64_t N) {
+    const TierEnv& env = tier_env();
+    TierChoice c;
+    c.T = env.T;
+    c.fast = env.ozaki_fast && M >= 512 && K >= 512 && N >= 512;
+    if (env.ozaki_crt || env.ozaki_fast) {
+        if (M >= 512 && K >= 512 && N >= 512) { c.tier = 2; c.why = "ESHKOL_HIP_F64_KERNEL/ESHKOL_SF64_KERNEL override"; }
+    } else if (env.ozaki_int8) {
+        if (M >= 1024 && N >= 1024 && K >= 1024) { c.tier = 1; c.why = "ESHKOL_CUDA_F64_KERNEL override"; }
+    } else if (env.budget >= 0.0) {
+        if (select_ozaki(M, K, N, env.budget, &c.T, &c.pred)) { c.tier = 1; c.why = "accuracy-budget selector"; }
+        else c.why = "budget met cheapest by native fp64";
+    }
+    return c;
+}
+
+/* C[MxN] = op(A)*op(B) on the chosen tier, with the ladder behind it: the
+ * reduced-precision CRT tier falls to the exact one, an Ozaki tier to native
+ * fp64, never to a wrong result (gpu_memory.mm:3036-3052). With wait the call
+ * returns after the device has finished (and feeds the cost model and the
+ * profile line); without, the work is queued on g_stream and device errors
+ * surface at the caller's synchronisation. */
+int run_tiers(const TierChoice& c, const double* dA, const double* dB, double* dC,
+              uint64_t M, uint64_t K, uint64_t N, int ta, int tb, bool wait) {
+    const TierEnv& env = tier_env();
+    const double work = 2.0 * (double)M * (double)K * (double)N;
+    auto finished = [&]() { return !wait || ESHKOL_HIP_OK(hipStreamSynchronize(g_stream)); };
+
+    if (c.fast) {
         auto t0 = std::chrono::steady_clock::now();
         GPU_LOG("matmul %llux%llu @ %llux%llu -> Ozaki-II FAST (%d moduli)", (unsigned long long)M,
                 (unsigned long long)K, (unsigned long long)K, (unsigned long long)N, env.fast_moduli);
         const int fr = hip_matmul_ozaki_fast_f64_ex(dA, dB, dC, M, K, N, ta, tb, env.fast_moduli, g_stream);
-        if (fr == 0 && ESHKOL_HIP_OK(hipStreamSynchronize(g_stream))) {
-            if (env.profile) {
+        if (fr == 0 && finished()) {
+            if (env.profile && wait) {
                 double ns = std::chrono::duration<double, std::nano>(std::chrono::steady_clock::now() - t0).count();
                 fprintf(stderr, "[OZAKI_PROFILE] fast M=%llu K=%llu N=%llu moduli=%d ms=%.2f GFLOPS=%.1f\n",
                         (unsigned long long)M, (unsigned long long)K, (unsigned long long)N, env.fast_moduli,
                         ns / 1e6, work / ns);
             }
-            mark_written(C);
             return 0;
         }
         fprintf(stderr, "[GPU] Ozaki-II FAST dispatch returned %d; falling back to exact tier\n", fr);
     }
-    int ozT = env.T;
-    double pred = 1.0;
-    const char* why = "default";
-    if (env.ozaki_crt || env.ozaki_fast) {
-        if (M >= 512 && K >= 512 && N >= 512) { tier = 2; why = "ESHKOL_HIP_F64_KERNEL/ESHKOL_SF64_KERNEL override"; }
-    } else if (env.ozaki_int8) {
-        if (M >= 1024 && N >= 1024 && K >= 1024) { tier = 1; why = "ESHKOL_CUDA_F64_KERNEL override"; }
-    } else if (env.budget >= 0.0) {
-        if (select_ozaki(M, K, N, env.budget, &ozT, &pred)) { tier = 1; why = "accuracy-budget selector"; }
-        else why = "budget met cheapest by native fp64";
-    }
 
-    if (tier != 0) {
+    if (c.tier != 0) {
         auto t0 = std::chrono::steady_clock::now();
         int rc;
-        if (tier == 2) {
+        if (c.tier == 2) {
             GPU_LOG("matmul %llux%llu @ %llux%llu -> Ozaki-II CRT exact (%s)",
                     (unsigned long long)M, (unsigned long long)K, (unsigned long long)K,
-                    (unsigned long long)N, why);
+                    (unsigned long long)N, c.why);
             rc = hip_matmul_ozaki_crt_f64_ex(dA, dB, dC, M, K, N, ta, tb, env.num_moduli,
                                              env.adaptive ? 1 : 0, nullptr, 0, g_stream);
         } else {
             GPU_LOG("matmul %llux%llu @ %llux%llu -> INT8-Ozaki T=%d (%s, ~%.2fx vs native)",
                     (unsigned long long)M, (unsigned long long)K, (unsigned long long)K,
-                    (unsigned long long)N, ozT, why, pred);
-            rc = hip_matmul_ozaki_int8_f64_ex(dA, dB, dC, M, K, N, ta, tb, ozT, g_stream);
+                    (unsigned long long)N, c.T, c.why, c.pred);
+            rc = hip_matmul_ozaki_int8_f64_ex(dA, dB, dC, M, K, N, ta, tb, c.T, g_stream);
         }
-        if (rc == 0 && ESHKOL_HIP_OK(hipStreamSynchronize(g_stream))) {
-            double ns = std::chrono::duration<double, std::nano>(std::chrono::steady_clock::now() - t0).count();
-            if (tier == 1) calibrate(ozT, work, ns);
-            if (env.profile)
-                fprintf(stderr, "[OZAKI_PROFILE] %s M=%llu K=%llu N=%llu ms=%.2f GFLOPS=%.1f\n",
-                        tier == 2 ? "exact" : "int8", (unsigned long long)M, (unsigned long long)K,
-                        (unsigned long long)N, ns / 1e6, work / ns);
-            mark_written(C);
+        if (rc == 0 && finished()) {
+            if (wait) {
+                double ns = std::chrono::duration<double, std::nano>(std::chrono::steady_clock::now() - t0).count();
+                if (c.tier == 1) calibrate(c.T, work, ns);
+                if (env.profile)
+                    fprintf(stderr, "[OZAKI_PROFILE] %s M=%llu K=%llu N=%llu ms=%.2f GFLOPS=%.1f\n",
+                            c.tier == 2 ? "exact" : "int8", (unsigned long long)M, (unsigned long long)K,
+                            (unsigned long long)N, ns / 1e6, work / ns);
+            }
             return 0;
         }
         GPU_LOG("matmul %llux%llu @ %llux%llu -> Ozaki tier fell back to native fp64",
@@ -435,16 +455,102 @@ int hip_matmul_f64(EshkolGPUBuffer* A, EshkolGPUBuffer* B, EshkolGPUBuffer* C,
     } else {
         GPU_LOG("matmul %llux%llu @ %llux%llu -> native fp64 MFMA (%s)",
                 (unsigned long long)M, (unsigned long long)K, (unsigned long long)K,
-                (unsigned long long)N, why);
+                (unsigned long long)N, c.why);
     }
 
     auto t0 = std::chrono::steady_clock::now();
     if (hip_dgemm_f64_ex(dA, dB, dC, M, K, N, ta, tb, g_stream) != 0) return -1;
-    if (!ESHKOL_HIP_OK(hipStreamSynchronize(g_stream))) return -1;
-    double ns = std::chrono::duration<double, std::nano>(std::chrono::steady_clock::now() - t0).count();
-    calibrate(0, work, ns);
-    mark_written(C);
+    if (!finished()) return -1;
+    if (wait) {
+        double ns = std::chrono::duration<double, std::nano>(std::chrono::steady_clock::now() - t0).count();
+        calibrate(0, work, ns);
+    }
     return 0;
+}
+
+/* ta/tb mark an operand the caller holds transposed (A as [K][M], B as [N][K]). */
+int hip_matmul_f64(EshkolGPUBuffer* A, EshkolGPUBuffer* B, EshkolGPUBuffer* C,
+                   uint64_t M, uint64_t K, uint64_t N, int ta = 0, int tb = 0) {
+    if (A->size_bytes < M * K * sizeof(double) || B->size_bytes < K * N * sizeof(double) ||
+        C->size_bytes < M * N * sizeof(double)) return -1;
+    const int rc = run_tiers(choose_tier(M, K, N), (const double*)A->device_ptr, (const double*)B->device_ptr,
+                             (double*)C->device_ptr, M, K, N, ta, tb, true);
+    if (rc == 0) mark_written(C);
+    return rc;
+}
+
+void release_copy_queue(void) {
+    if (g_ev_up) { hipEventDestroy(g_ev_up); g_ev_up = nullptr; }
+    for (hipEvent_t& e : g_ev_done) if (e) { hipEventDestroy(e); e = nullptr; }
+    if (g_copy_stream) { hipStreamDestroy(g_copy_stream); g_copy_stream = nullptr; }
+}
+
+/* C = A*B on host memory in row panels of A and C: while the device multiplies
+ * panel p, the host stages panel p+1 up and panel p-1 down on the copy queue,
+ * so that of the three transfers only B's is not hidden behind another or
+ * behind the products. Row panels leave every tier's result unchanged: the
+ * Ozaki tiers scale A by rows and B by columns, and a native tile does not
+ * depend on the other tiles of the launch (only the split of a last partial
+ * round may differ, which reorders a sum). The tier is chosen for the whole
+ * product. Returns false when the shape does not pay or anything failed; the
+ * caller then takes the one-piece path, which redoes the product. */
+constexpr size_t PANEL_MIN_BYTES = 128u << 20;      /* A and C together */
+
+bool panelled_matmul(const double* A, const double* B, double* C,
+                     uint64_t M, uint64_t K, uint64_t N, int reduced) {
+    const TierEnv& env = tier_env();
+    if (!g_copy_stream || !env.overlap || env.profile) return false;
+    const size_t a_bytes = M * K * sizeof(double), b_bytes = K * N * sizeof(double), c_bytes = M * N * sizeof(double);
+    if (a_bytes + c_bytes < PANEL_MIN_BYTES) return false;
+    const char *a0 = (const char*)A, *b0 = (const char*)B, *c0 = (const char*)C;
+    if ((c0 < a0 + a_bytes && a0 < c0 + c_bytes) || (c0 < b0 + b_bytes && b0 < c0 + c_bytes)) return false;
+    if (resident_find(A)) return false;
+    uint64_t rows = (((M + 7) / 8) + 127) & ~(uint64_t)127;
+    if (rows < 512) rows = 512;
+    const uint64_t panels = (M + rows - 1) / rows;
+    if (panels < 2) return false;
+
+    EshkolGPUBuffer bb{};
+    if (hip_wrap((void*)B, b_bytes, true, false, &bb) != 0) return false;
+    double* dA = (double*)staging_get(a_bytes);
+    double* dC = dA ? (double*)staging_get(c_bytes) : nullptr;
+    bool ok = dA && dC;
+    if (ok) {
+        GPU_LOG("matmul %llux%llu @ %llux%llu from host memory in %llu row panels of %llu",
+                (unsigned long long)M, (unsigned long long)K, (unsigned long long)K, (unsigned long long)N,
+                (unsigned long long)panels, (unsigned long long)rows);
+        const TierChoice choice = choose_tier(M, K, N);
+        const double* dB = (const double*)bb.device_ptr;
+        for (uint64_t p = 0; p < panels && ok; p++) {
+            const uint64_t r0 = p * rows, mp = (M - r0 < rows) ? M - r0 : rows;
+            ok = eshkol_hip_upload(dA + r0 * K, A + r0 * K, mp * K * sizeof(double), g_copy_stream) == 0 &&
+                 ESHKOL_HIP_OK(hipEventRecord(g_ev_up, g_copy_stream)) &&
+                 ESHKOL_HIP_OK(hipStreamWaitEvent(g_stream, g_ev_up, 0));
+            if (!ok) break;
+            const int rc = reduced
+                ? hip_matmul_reduced_f64(dA + r0 * K, dB, dC + r0 * N, mp, K, N, reduced, 1, g_stream)
+                : run_tiers(choice, dA + r0 * K, dB, dC + r0 * N, mp, K, N, 0, 0, false);
+            ok = rc == 0 && ESHKOL_HIP_OK(hipEventRecord(g_ev_done[p & 1], g_stream));
+            if (ok && p > 0) {
+                const uint64_t q0 = (p - 1) * rows;
+                ok = ESHKOL_HIP_OK(hipStreamWaitEvent(g_copy_stream, g_ev_done[(p - 1) & 1], 0)) &&
+                     eshkol_hip_download(C + q0 * N, dC + q0 * N, rows * N * sizeof(double), g_copy_stream) == 0;
+            }
+        }
+        if (ok) {
+            const uint64_t q0 = (panels - 1) * rows;
+            ok = ESHKOL_HIP_OK(hipStreamWaitEvent(g_copy_stream, g_ev_done[(panels - 1) & 1], 0)) &&
+                 eshkol_hip_download(C + q0 * N, dC + q0 * N, (M - q0) * N * sizeof(double), g_copy_stream) == 0;
+        }
+    }
+    /* both queues drained before the buffers go back, and device errors seen */
+    const bool drained = ESHKOL_HIP_OK(hipStreamSynchronize(g_copy_stream)) &&
+                         ESHKOL_HIP_OK(hipStreamSynchronize(g_stream));
+    if (dA) staging_put(dA);
+    if (dC) staging_put(dC);
+    hip_free(&bb);
+    if (!drained) (void)hipGetLastError();
+    return ok && drained;
 }
 
 }  // namespace
@@ -514,6 +620,14 @@ int eshkol_gpu_init(void) {
     }
     if (ok) ok = ESHKOL_HIP_OK(hipStreamCreate(&g_stream));
     if (ok) {
+        /* optional: without them the host-memory dispatch does not overlap copies and products */
+        bool extra = ESHKOL_HIP_OK(hipStreamCreate(&g_copy_stream)) &&
+                     ESHKOL_HIP_OK(hipEventCreateWithFlags(&g_ev_up, hipEventDisableTiming)) &&
+                     ESHKOL_HIP_OK(hipEventCreateWithFlags(&g_ev_done[0], hipEventDisableTiming)) &&
+                     ESHKOL_HIP_OK(hipEventCreateWithFlags(&g_ev_done[1], hipEventDisableTiming));
+        if (!extra) { (void)hipGetLastError(); release_copy_queue(); }
+    }
+    if (ok) {
         g_backend = ESHKOL_GPU_HIP;
         g_initialized.store(true, std::memory_order_release);
         GPU_LOG("initialized: AMD HIP (%s)", g_arch);
@@ -531,8 +645,11 @@ void eshkol_gpu_shutdown(void) {
     if (g_backend == ESHKOL_GPU_HIP) {
         if (g_stream) hipStreamSynchronize(g_stream);
         eshkol_hip_workspace_release();
+        eshkol_hip_copy_release();
         staging_release_all();
         resident_release_all();
+        if (g_copy_stream) hipStreamSynchronize(g_copy_stream);
+        release_copy_queue();
         if (g_stream) { hipStreamDestroy(g_stream); g_stream = nullptr; }
     }
     g_backend = ESHKOL_GPU_NONE;
@@ -725,7 +842,7 @@ int eshkol_gpu_resident_pin(const void* host_ptr, size_t size_bytes) {
     }
     void* d = r ? r->dev : nullptr;
     if (!d && !ESHKOL_HIP_OK(hipMalloc(&d, size_bytes))) return -1;
-    if (!ESHKOL_HIP_OK(hipMemcpyAsync(d, host_ptr, size_bytes, hipMemcpyHostToDevice, g_stream)) ||
+    if (eshkol_hip_upload(d, host_ptr, size_bytes, g_stream) != 0 ||
         !ESHKOL_HIP_OK(hipStreamSynchronize(g_stream))) {
         if (!r) hipFree(d);
         return -1;
@@ -739,7 +856,7 @@ int eshkol_gpu_resident_refresh(const void* host_ptr) {
     std::lock_guard<std::recursive_mutex> g(g_gpu_mutex);
     Resident* r = resident_find(host_ptr);
     if (!r) return -1;
-    if (!ESHKOL_HIP_OK(hipMemcpyAsync(r->dev, host_ptr, r->bytes, hipMemcpyHostToDevice, g_stream)) ||
+    if (eshkol_hip_upload(r->dev, host_ptr, r->bytes, g_stream) != 0 ||
         !ESHKOL_HIP_OK(hipStreamSynchronize(g_stream))) return -1;
     return 0;
 }
@@ -832,6 +949,7 @@ void eshkol_matmul_dispatch(const double* A, const double* B, double* C,
         if (!reduced && env.precision >= 2 && eshkol_gpu_should_use(num_elements)) reduced = 3;
         if (reduced || eshkol_gpu_should_use(num_elements)) {
             std::lock_guard<std::recursive_mutex> g(g_gpu_mutex);
+            if (panelled_matmul(A, B, C, M, K, N, reduced)) return;
             EshkolGPUBuffer ba{}, bb{}, bc{};
             const bool wa = hip_wrap((void*)A, M * K * sizeof(double), true, false, &ba) == 0;
             const bool wb = wa && hip_wrap((void*)B, K * N * sizeof(double), true, false, &bb) == 0;

@@ -80,6 +80,45 @@ def test_buffer_lifecycle(gpu):
     lib.eshkol_gpu_wait(None)
 
 
+@pytest.mark.parametrize("nbytes", [(1 << 20) - 8, (1 << 20) + 8, (16 << 20), (16 << 20) + 24,
+                                    5 * (16 << 20) + 4096 + 8, 9 * (16 << 20) - 8])
+def test_wrapped_host_memory_round_trip_through_the_staging_ring(gpu, nbytes):
+    """Uploads and downloads of caller-owned memory are staged through a ring of
+    pinned chunks by several threads; every byte has to arrive, whatever the
+    size is relative to a chunk, the ring, or a thread's share."""
+    lib = ea.load()
+    n = nbytes // 8
+    x = synth.normal(90 + (nbytes % 97), (n,))
+    y = np.full(n, np.nan)
+    bx, by = ea.EshkolGPUBuffer(), ea.EshkolGPUBuffer()
+    assert lib.eshkol_gpu_wrap_host(x.ctypes.data, x.nbytes, C.byref(bx)) == 0
+    assert lib.eshkol_gpu_wrap_host(y.ctypes.data, y.nbytes, C.byref(by)) == 0
+    assert lib.eshkol_gpu_elementwise_f64(C.byref(bx), None, C.byref(by), n, 4) == 0      # y = -x
+    assert lib.eshkol_gpu_sync(C.byref(by), ea.SYNC_DEVICE_TO_HOST) == 0
+    assert np.array_equal(y, -x)
+    # host -> device of changed contents, then the copy-back on free
+    y[:] = x * 2.0
+    assert lib.eshkol_gpu_sync(C.byref(by), ea.SYNC_HOST_TO_DEVICE) == 0
+    assert lib.eshkol_gpu_elementwise_f64(C.byref(by), None, C.byref(by), n, 4) == 0      # y = -y
+    lib.eshkol_gpu_free(C.byref(by))
+    assert np.array_equal(y, -2.0 * x)
+    lib.eshkol_gpu_free(C.byref(bx))
+
+
+def test_staged_copies_can_be_switched_off(gpu):
+    run_child("""
+assert lib.eshkol_gpu_init() == 1
+n = (40 << 20) // 8
+x = synth.normal(7, (n,)); y = np.zeros(n)
+bx, by = ea.EshkolGPUBuffer(), ea.EshkolGPUBuffer()
+assert lib.eshkol_gpu_wrap_host(x.ctypes.data, x.nbytes, C.byref(bx)) == 0
+assert lib.eshkol_gpu_wrap_host(y.ctypes.data, y.nbytes, C.byref(by)) == 0
+assert lib.eshkol_gpu_elementwise_f64(C.byref(bx), None, C.byref(by), n, 4) == 0
+lib.eshkol_gpu_free(C.byref(by)); lib.eshkol_gpu_free(C.byref(bx))
+assert np.array_equal(y, -x)
+""", {"ESHKOL_GPU_COPY_THREADS": "0"})
+
+
 def test_gpu_matmul_f64_on_device_buffers(gpu):
     lib = ea.load()
     M, K, N = 300, 200, 260
@@ -175,6 +214,48 @@ for i in range(4):
     r = run_child(body, {"ESHKOL_GPU_VERBOSE": "1"})
     assert "native fp64 MFMA" in r.stderr and "reduced tier" in r.stderr
     assert "batch matmul 4 x (96x160 @ 160x64) -> native fp64 MFMA, one strided launch" in r.stderr
+
+
+PANELLED = r"""
+assert lib.eshkol_gpu_init() == 1
+lib.eshkol_gpu_set_threshold(1)
+lib.hip_dgemm_set_tail_split(0)                  # a split last round reorders sums in the tiles it takes
+M, K, N = 4100, 2048, 2056                       # 7 panels of 640 rows, the last one of 260
+A = synth.normal(11, (M, K)); B = synth.normal(12, (K, N))
+got = ea.matmul_dispatch(A, B, DTYPE)
+dA, dB, dC = ea.DeviceArray.from_host(A), ea.DeviceArray.from_host(B), ea.DeviceArray((M, N))
+if DTYPE:
+    assert lib.hip_matmul_reduced_f64(dA.ptr, dB.ptr, dC.ptr, M, K, N, DTYPE, 1, None) == 0
+else:
+    assert lib.eshkol_gpu_matmul_f64(C.byref(dA.buf), C.byref(dB.buf), C.byref(dC.buf), M, K, N) == 0
+lib.eshkol_gpu_wait(None)
+whole = dC.download()
+assert np.array_equal(got, whole)
+# the same call again reuses the device copies' memory, and resident weights skip their upload
+assert lib.eshkol_gpu_resident_pin(B.ctypes.data, B.nbytes) == 0
+again = ea.matmul_dispatch(A, B, DTYPE)
+assert np.array_equal(again, got)
+lib.eshkol_gpu_resident_unpin(B.ctypes.data)
+"""
+
+
+@pytest.mark.parametrize("env,dtype,tier_line", [
+    ({}, 0, "native fp64 MFMA"),
+    ({"ESHKOL_HIP_F64_KERNEL": "ozaki-crt"}, 0, "Ozaki-II CRT exact"),
+    ({"ESHKOL_OZAKI_FAST": "1"}, 0, "Ozaki-II FAST"),
+    ({"ESHKOL_HIP_F64_KERNEL": "ozaki-int8"}, 0, "INT8-Ozaki T=6"),
+    ({}, 3, "row panels"),
+], ids=["native", "crt", "crt-fast", "int8-slices", "bf16"])
+def test_host_memory_dispatch_in_row_panels(gpu, env, dtype, tier_line):
+    """Large products on host memory go through the device in row panels of A
+    and C so that copies and products overlap; the result is the one-piece one."""
+    body = PANELLED.replace("DTYPE", str(dtype))
+    e = dict(env); e["ESHKOL_GPU_VERBOSE"] = "1"
+    r = run_child(body, e)
+    assert "in 7 row panels of 640" in r.stderr and tier_line in r.stderr
+    e["ESHKOL_GPU_OVERLAP"] = "0"
+    r = run_child(body, e)
+    assert "row panels" not in r.stderr and (dtype or tier_line in r.stderr)
 
 
 def test_batched_native_kernel(gpu):
