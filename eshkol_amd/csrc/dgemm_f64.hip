@@ -498,6 +498,32 @@ void dgemm_fixup_kernel(const double* __restrict__ partial, int tail, int pieces
 
 int g_tail_split = 1;
 
+/* Pieces per tile for a launch of `nwg` 128 x 128 tiles over `nkb` k-blocks that
+ * does not fill the device; 1 = leave it to the 64 x 64 kernel. Times in
+ * microseconds from two fits to measurements on this device (16 ... 144 tiles,
+ * K = 64 ... 16384):
+ *   whole: 4 + 0.86 per k-block, times the rounds four times as many small
+ *          tiles need;
+ *   cut:   10 + 0.04 per workgroup (two launches, the partial tiles' round
+ *          trip) + 2.2 per k-block of a piece, times 1.7 once some CUs hold two
+ *          workgroups.
+ * The fits are within 10 % of the measurements they came from; a cut has to
+ * win 5 % on them. */
+int small_launch_pieces(long long nwg, int nkb) {
+    const int cus = eshkol_hip_num_cus();
+    if (4 * nwg >= 3 * (long long)cus) return 1;
+    const double rounds = 4.0 * (double)nwg / cus;
+    const double whole = 4.0 + 0.86 * nkb * (rounds > 1.0 ? rounds : 1.0);
+    int best_p = 1;
+    double best = 0.95 * whole;
+    for (int p = 2; p <= 128 && nkb / p >= 4 && nwg * p <= 2 * cus; p++) {
+        const double crowd = (nwg * p <= cus) ? 1.0 : 1.7;
+        const double cost = 10.0 + 0.04 * (double)(nwg * p) + crowd * 2.2 * ((double)nkb / p);
+        if (cost < best) { best = cost; best_p = p; }
+    }
+    return best_p;
+}
+
 template <bool TA, bool TB, bool KTAIL>
 int launch_fast_k(const double* A, const double* B, double* C, int M, int N, int K, int batch, hipStream_t st) {
     constexpr int SMEM_BYTES = 2 * (Operand<128, TA, true, true>::TILE + Operand<128, !TB, true, true>::TILE)
@@ -549,6 +575,24 @@ int launch_fast_k(const double* A, const double* B, double* C, int M, int N, int
             return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
         }
     }
+    /* A launch of fewer tiles than CUs leaves CUs idle for its whole length: all
+     * its tiles are cut along k the same way (1024^3: 64 tiles, 59 -> 53 us;
+     * 512 x 2048 x 512: 16 tiles, 104 -> 33 us; 128 x 8192 x 128: 400 -> 47 us). */
+    const int small_p = (g_tail_split && batch == 1) ? small_launch_pieces(nwg, nkb) : 1;
+    if (small_p >= 2) {
+        const int kbpp = (nkb + small_p - 1) / small_p;
+        const int pieces = (nkb + kbpp - 1) / kbpp;
+        double* ws = pieces >= 2 ? (double*)eshkol_hip_workspace(WS_DGEMM_PARTIAL,
+                                         (size_t)nwg * pieces * 128 * 128 * sizeof(double)) : nullptr;
+        if (ws) {
+            sp.first_tile = 0; sp.tail = (int)nwg; sp.kb_per_piece = kbpp; sp.partial = ws;
+            hipLaunchKernelGGL(kern_split, dim3((unsigned)(nwg * pieces), 1), dim3(256), SMEM_BYTES, st,
+                               A, B, C, M, N, K, tiles_m, tiles_n, sp);
+            hipLaunchKernelGGL(dgemm_fixup_kernel, dim3((unsigned)nwg, 16), dim3(256), 0, st,
+                               ws, (int)nwg, pieces, 0, tiles_m, tiles_n, C, M, N);
+            return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+        }
+    }
     hipLaunchKernelGGL(kern, dim3((unsigned)nwg, (unsigned)batch), dim3(256), SMEM_BYTES, st,
                        A, B, C, M, N, K, tiles_m, tiles_n, sp);
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
@@ -591,7 +635,8 @@ int launch_shape(const double* A, const double* B, double* C, int m, int n, int 
      * at 8192^3; with both operands row-major the natural forms are faster. */
     constexpr bool ALK = TA || !TB;
     /* 16-byte operand chunks (even pitches, aligned bases) and at least one whole k-block */
-    if (g_fast_path && big_tiles >= 256 && vec && m >= 2 && n >= 2 && k >= BK)
+    const bool cut = g_tail_split && batch == 1 && small_launch_pieces(big_tiles, (k + BK - 1) / BK) >= 2;
+    if (g_fast_path && (big_tiles >= 192 || cut) && vec && m >= 2 && n >= 2 && k >= BK)
         return launch_fast<TA, TB>(A, B, C, m, n, k, batch, st);
     if (big_tiles >= 256) {
         return vec ? launch<128, 128, true, TA, TB, ALK, !TB>(A, B, C, m, n, k, batch, st)

@@ -299,10 +299,11 @@ int hip_probe_peak(int kind, int random_operands, double* rate, void* stream);
 void hip_dgemm_set_fast_path(int on);
 
 /* 1 (default): when the last round of 128 x 128 tiles of a large product would
- * leave more than half of the CUs idle, those tiles are cut along k, the pieces
- * multiplied side by side and added in a fixed order (deterministic, but the
- * summation order of those tiles differs from an unsplit launch); 0: every tile
- * is multiplied whole. */
+ * leave more than half of the CUs idle, or a product has too few tiles to fill
+ * the device at all, those tiles are cut along k, the pieces multiplied side by
+ * side and added in a fixed order (deterministic, but the summation order of
+ * those tiles differs from an unsplit launch); 0: every tile is multiplied
+ * whole. */
 void hip_dgemm_set_tail_split(int on);
 
 /* k-blocks kept in flight by the pipelined int8 kernel (1..3; 0 = simple kernel only). */

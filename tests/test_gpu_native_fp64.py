@@ -176,3 +176,37 @@ def test_k_split_last_round(gpu, M, K, N):
             assert normwise(cut, ref, A, B) <= TOL, (ta, tb)
         else:
             assert np.abs(cut - whole).max() <= 1e-11 * np.sqrt(K)
+
+
+@pytest.mark.parametrize("M,K,N", [(512, 2048, 512), (128, 8192, 128), (400, 1000, 400), (300, 1002, 1100),
+                                   (1536, 1024, 1536), (130, 4098, 258), (1152, 1152, 1152)])
+def test_k_split_of_a_launch_that_does_not_fill_the_device(gpu, M, K, N):
+    """Fewer 128 x 128 tiles than CUs: every tile is cut along k and the pieces are added in
+    a fixed order. Same bits on every run, within the tier's bound (against the whole launch
+    too), nothing stored outside C; for all three operand forms."""
+    import eshkol_amd as ea
+    from gpu_util import stream
+    lib = ea.load()
+    A, B = synth.normal(M + 5 * K, (M, K)), synth.normal(K + 5 * N, (K, N))
+    ref = oracle.matmul_f64(A, B)
+    forms = [(A, B, 0, 0), (A, np.ascontiguousarray(B.T), 0, 1), (np.ascontiguousarray(A.T), B, 1, 0)]
+    for X, Y, ta, tb in forms:
+        dX, dY = ea.DeviceArray.from_host(X), ea.DeviceArray.from_host(Y)
+        outs = []
+        try:
+            for split in (0, 1, 1):
+                lib.hip_dgemm_set_tail_split(split)
+                guard = np.full((M + 2, N), np.nan)
+                guard[0] = guard[-1] = 12345.0
+                dC = ea.DeviceArray.from_host(guard)
+                assert lib.hip_dgemm_f64_ex(dX.ptr, dY.ptr, dC.ptr + N * 8, M, K, N, ta, tb, stream()) == 0
+                ea.synchronize()
+                got = dC.download()
+                assert np.all(got[0] == 12345.0) and np.all(got[-1] == 12345.0)
+                outs.append(got[1:-1])
+        finally:
+            lib.hip_dgemm_set_tail_split(1)
+        whole, cut, again = outs
+        assert np.array_equal(cut, again), (ta, tb)
+        assert not np.array_equal(whole, cut), "the launch was expected to be cut along k"
+        assert normwise(cut, ref, A, B) <= 1e-14 and normwise(cut, whole, A, B) <= 1e-14
