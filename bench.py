@@ -304,14 +304,20 @@ def main():
     # ---- host-buffer entry: eshkol_matmul_dispatch on pageable host memory (PCIe inclusive) -----
     if "host" in want:
         Ch = np.empty((M, N))
-        t0 = time.perf_counter()
-        lib.eshkol_matmul_dispatch(A.ctypes.data, B.ctypes.data, Ch.ctypes.data, M, K, N, 0)
-        dt = time.perf_counter() - t0
+        calls = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            lib.eshkol_matmul_dispatch(A.ctypes.data, B.ctypes.data, Ch.ctypes.data, M, K, N, 0)
+            calls.append(time.perf_counter() - t0)
+        dt = min(calls[1:])
         tiers["host_buffers_eshkol_matmul_dispatch"] = {
-            "ms": dt * 1e3, "gflops": flops / dt / 1e9,
-            "note": "one call, operands and result in pageable host memory: two uploads, one download, "
-                    "device allocations included; never the headline value"}
-        log("eshkol_matmul_dispatch from host memory: %.1f ms %.1f GFLOP/s" % (dt * 1e3, flops / dt / 1e9))
+            "ms": dt * 1e3, "gflops": flops / dt / 1e9, "first_call_ms": calls[0] * 1e3,
+            "note": "operands and result in pageable host memory: two uploads, one download, copies staged "
+                    "through pinned chunks and overlapped with the product in row panels; the first call also "
+                    "allocates device buffers, the pinned ring and the copy threads and touches the result's "
+                    "pages; never the headline value"}
+        log("eshkol_matmul_dispatch from host memory: %.1f ms %.1f GFLOP/s (first call %.1f ms)"
+            % (dt * 1e3, flops / dt / 1e9, calls[0] * 1e3))
         del Ch
 
     # ---- CPU baseline on one host core ---------------------------------------------------------
