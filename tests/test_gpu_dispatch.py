@@ -258,6 +258,44 @@ def test_host_memory_dispatch_in_row_panels(gpu, env, dtype, tier_line):
     assert "row panels" not in r.stderr and (dtype or tier_line in r.stderr)
 
 
+def test_concurrent_callers_serialise_on_the_library(gpu):
+    """Calls from several host threads (the reference guards only initialisation,
+    gpu_memory_cuda.cpp:111, 844; this library serialises every call on one mutex):
+    large panelled products and small ones share the streams, the workspaces and
+    the staging ring, and give the bits of the same calls made one at a time."""
+    import threading
+    lib = ea.load()
+    assert lib.eshkol_gpu_init() == 1
+    old = lib.eshkol_gpu_get_threshold()
+    lib.eshkol_gpu_set_threshold(1)
+    shapes = [(4100, 2048, 2056), (300, 200, 260), (1024, 1024, 1024), (4096, 2048, 2048), (64, 4096, 96), (700, 50, 900)]
+    ops = [(synth.normal(20 + i, (m, k)), synth.normal(40 + i, (k, n))) for i, (m, k, n) in enumerate(shapes)]
+    want = [ea.matmul_dispatch(a, b) for a, b in ops]            # one at a time
+    got = [[None] * len(ops) for _ in range(2)]
+    errors = []
+
+    def worker(rep, i):
+        try:
+            got[rep][i] = ea.matmul_dispatch(*ops[i])
+        except Exception as e:                                     # pragma: no cover
+            errors.append(e)
+
+    try:
+        threads = [threading.Thread(target=worker, args=(rep, i)) for rep in range(2) for i in range(len(ops))]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+    finally:
+        lib.eshkol_gpu_set_threshold(old)
+    assert not errors
+    for rep in range(2):
+        for i, (a, b) in enumerate(ops):
+            assert np.array_equal(got[rep][i], want[i]), shapes[i]
+            if rep == 0 and a.shape[0] * a.shape[1] * b.shape[1] <= 2 ** 28:
+                assert normwise(want[i], oracle.matmul_f64(a, b), a, b) <= 1e-14
+
+
 def test_batched_native_kernel(gpu):
     """hip_dgemm_f64_batched against the oracle's batch loop: even and odd shapes
     (the odd ones leave matrices of the batch off 16-byte boundaries), integer
