@@ -552,15 +552,22 @@ int await_mailbox(uint32_t ticket, hipStream_t st) {
     return 0;
 }
 
-/* Runs the scan on the two vectors of maxima and waits for its summary. */
-const CrtScan* scan_maxima(const double* amax, uint64_t M, const double* bmax, uint64_t N,
-                           int32_t* fl_a, int32_t* fl_b, hipStream_t st) {
-    if (!ensure_mailbox()) return nullptr;
+/* Queues the scan of the two vectors of maxima; 0 on failure, else the ticket its
+ * summary will carry. */
+uint32_t scan_launch(const double* amax, uint64_t M, const double* bmax, uint64_t N,
+                     int32_t* fl_a, int32_t* fl_b, hipStream_t st) {
+    if (!ensure_mailbox()) return 0;
     const uint32_t ticket = ++g_ticket ? g_ticket : ++g_ticket;            /* never 0: the mailbox starts zeroed */
     hipLaunchKernelGGL(crt_scan_kernel, dim3(2), dim3(SCAN_THREADS), 0, st, amax, M, bmax, N, fl_a, fl_b,
                        g_mailbox_dev, ticket);
-    if (!ESHKOL_HIP_OK(hipGetLastError()) || await_mailbox(ticket, st) != 0) return nullptr;
-    return g_mailbox;
+    return ESHKOL_HIP_OK(hipGetLastError()) ? ticket : 0;
+}
+const CrtScan* scan_await(uint32_t ticket, hipStream_t st) {
+    return (ticket != 0 && await_mailbox(ticket, st) == 0) ? g_mailbox : nullptr;
+}
+const CrtScan* scan_maxima(const double* amax, uint64_t M, const double* bmax, uint64_t N,
+                           int32_t* fl_a, int32_t* fl_b, hipStream_t st) {
+    return scan_await(scan_launch(amax, M, bmax, N, fl_a, fl_b, st), st);
 }
 
 /* device-resident constant tables for the contraction: identity pair lists and moduli */
@@ -730,7 +737,72 @@ extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, dou
 
     if ((a_kmajor ? hip_colabsmax_f64(A, K, M, 0.0, amax, st) : hip_rowabsmax_f64(A, M, K, 0.0, amax, st)) != 0) return -1;
     if ((b_kmajor ? hip_colabsmax_f64(B, K, N, 0.0, bmax, st) : hip_rowabsmax_f64(B, N, K, 0.0, bmax, st)) != 0) return -1;
-    const CrtScan* h_scan = scan_maxima(amax, M, bmax, N, dmu, dnu, st);
+    const uint32_t ticket = scan_launch(amax, M, bmax, N, dmu, dnu, st);
+    if (!ticket) return -1;
+    const double log2K = log2((double)K);
+
+    /* Everything after the shifts, queued in one go. */
+    auto enqueue_products = [&](int n_mod, const HostCrt& crt, int E) -> int {
+        int8_t* Ap = (int8_t*)eshkol_hip_workspace(WS_APLANES, (size_t)n_mod * Mp * ldk);
+        int8_t* Bp = (int8_t*)eshkol_hip_workspace(WS_BPLANES, (size_t)n_mod * Np * ldk);
+        int8_t* Wp = (int8_t*)eshkol_hip_workspace(WS_PRODUCTS, (size_t)n_mod * M * N);
+        if (!Ap || !Bp || !Wp) return -1;
+        if (crt_split_any(A, M, K, dmu, n_mod, Ap, Mp, ldk, a_kmajor, st) != 0) return -1;
+        if (crt_split_any(B, N, K, dnu, n_mod, Bp, Np, ldk, b_kmajor, st) != 0) return -1;
+        HipIgemmArgs ga;
+        memset(&ga, 0, sizeof ga);
+        ga.a_planes = Ap; ga.b_planes = Bp;
+        ga.a_plane_stride = Mp * ldk; ga.b_plane_stride = Np * ldk;
+        ga.ldk = (uint32_t)ldk; ga.M = (uint32_t)M; ga.N = (uint32_t)N; ga.n_out = (uint32_t)n_mod;
+        ga.pair_first = g_tables; ga.pair_a = g_tables + 17; ga.pair_b = g_tables + 17;
+        ga.mode = 1; ga.max_pairs = 1; ga.modulus = g_tables + 33; ga.out_i8 = Wp;
+        if (hip_igemm_i8(&ga, st) != 0) return -1;
+        if (hip_ozaki_crt_reconstruct_f64(Wp, M, N, n_mod, crt.sl1, crt.sl2, crt.P1, crt.P2, crt.Pinv,
+                                          dmu, dnu, bias, act, C, st) != 0) return -1;
+        g_last.a_planes = Ap; g_last.b_planes = Bp; g_last.w_planes = Wp;
+        g_last.mu = dmu; g_last.nu = dnu;
+        g_last.rows_a_padded = Mp; g_last.rows_b_padded = Np; g_last.ldk = ldk;
+        g_last.num_moduli = n_mod; g_last.E = E;
+        return 0;
+    };
+    auto announce = [&](int n_mod, const HostCrt& crt) {
+        fprintf(stderr, "[GPU] Ozaki-II: N=%d%s, log2(P)=%.1f\n", n_mod,
+                adaptive ? " (adaptive)" : "", crt.log2P);       /* gpu_memory.mm:2503 */
+    };
+    auto in_range = [](int E, bool any, int e_min, int e_max) {
+        /* every shift E - floor(log2 max) must be an exponent ldexp can apply exactly */
+        return !any || (E - e_min <= 1023 && E - e_max >= -1022);
+    };
+
+    /* E = min(52, floor((log2 P - 1 - log2 K - frac_A - frac_B) / 2)) with both
+     * fractions below 1 (gpu_memory.mm:2510-2512): where even frac_A + frac_B = 2
+     * leaves 52 (16 moduli: every K this tier accepts), E does not depend on the
+     * operands, and the whole pipeline is queued behind the scan without waiting
+     * for it. Its summary is read afterwards; what it may still demand is a
+     * refusal (non-finite input, shifts out of range: C then holds no result) or
+     * the reference's own pass over the maxima, after which the products are
+     * queued a second time. */
+    const CrtScan* h_scan = nullptr;
+    bool announced = false;
+    if (!adaptive && !g_force_host_pass) {
+        const HostCrt& crt = crt_constants(num_moduli);
+        if (floor((crt.log2P - 3.0 - log2K) / 2.0) >= 52.0) {
+            const int E = 52;
+            hipLaunchKernelGGL(crt_shift_kernel, dim3((unsigned)((M + N + 255) / 256)), dim3(256), 0, st, dmu, M, dnu, N, E);
+            if (enqueue_products(num_moduli, crt, E) != 0) return -1;
+            announce(num_moduli, crt);
+            announced = true;
+            h_scan = scan_await(ticket, st);
+            if (!h_scan) return -1;
+            if (h_scan[0].nonfinite || h_scan[1].nonfinite) return -1;  /* NaN/Inf input */
+            if (!h_scan[0].extreme && !h_scan[1].extreme) {
+                for (int o = 0; o < 2; o++)
+                    if (!in_range(E, h_scan[o].nonzero != 0, h_scan[o].e_min, h_scan[o].e_max)) return -1;
+                return 0;
+            }
+        }
+    }
+    if (!h_scan) h_scan = scan_await(ticket, st);
     if (!h_scan) return -1;
     if (h_scan[0].nonfinite || h_scan[1].nonfinite) return -1;          /* NaN/Inf input */
 
@@ -776,7 +848,6 @@ extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, dou
         if (!ESHKOL_HIP_OK(hipMemcpyAsync(dnu, h_nu, N * sizeof(int32_t), hipMemcpyHostToDevice, st))) return -1;
     }
     const double frac_A = frac[0], frac_B = frac[1];
-    const double log2K = log2((double)K);
     if (adaptive) {                                   /* gpu_memory.mm:433-453 */
         std::call_once(g_cumul_once, [] {
             g_log2_cumul[0] = 0.0;
@@ -790,41 +861,14 @@ extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, dou
         num_moduli = chosen;
     }
     const HostCrt& crt = crt_constants(num_moduli);
-    fprintf(stderr, "[GPU] Ozaki-II: N=%d%s, log2(P)=%.1f\n", num_moduli,
-            adaptive ? " (adaptive)" : "", crt.log2P);       /* gpu_memory.mm:2503 */
-
     int E = (int)floor((crt.log2P - 1.0 - log2K - frac_A - frac_B) / 2.0);   /* gpu_memory.mm:2510-2512 */
     if (E > 52) E = 52;
     if (E < 0) E = 0;
-    /* every shift E - floor(log2 max) must be an exponent ldexp can apply exactly */
     for (int o = 0; o < 2; o++)
-        if (any[o] && (E - e_min[o] > 1023 || E - e_max[o] < -1022)) return -1;
+        if (!in_range(E, any[o], e_min[o], e_max[o])) return -1;
     hipLaunchKernelGGL(crt_shift_kernel, dim3((unsigned)((M + N + 255) / 256)), dim3(256), 0, st, dmu, M, dnu, N, E);
-
-    int8_t* Ap = (int8_t*)eshkol_hip_workspace(WS_APLANES, (size_t)num_moduli * Mp * ldk);
-    int8_t* Bp = (int8_t*)eshkol_hip_workspace(WS_BPLANES, (size_t)num_moduli * Np * ldk);
-    int8_t* Wp = (int8_t*)eshkol_hip_workspace(WS_PRODUCTS, (size_t)num_moduli * M * N);
-    if (!Ap || !Bp || !Wp) return -1;
-
-    if (crt_split_any(A, M, K, dmu, num_moduli, Ap, Mp, ldk, a_kmajor, st) != 0) return -1;
-    if (crt_split_any(B, N, K, dnu, num_moduli, Bp, Np, ldk, b_kmajor, st) != 0) return -1;
-
-    HipIgemmArgs ga;
-    memset(&ga, 0, sizeof ga);
-    ga.a_planes = Ap; ga.b_planes = Bp;
-    ga.a_plane_stride = Mp * ldk; ga.b_plane_stride = Np * ldk;
-    ga.ldk = (uint32_t)ldk; ga.M = (uint32_t)M; ga.N = (uint32_t)N; ga.n_out = (uint32_t)num_moduli;
-    ga.pair_first = g_tables; ga.pair_a = g_tables + 17; ga.pair_b = g_tables + 17;
-    ga.mode = 1; ga.max_pairs = 1; ga.modulus = g_tables + 33; ga.out_i8 = Wp;
-    if (hip_igemm_i8(&ga, st) != 0) return -1;
-
-    if (hip_ozaki_crt_reconstruct_f64(Wp, M, N, num_moduli, crt.sl1, crt.sl2, crt.P1, crt.P2, crt.Pinv,
-                                      dmu, dnu, bias, act, C, st) != 0) return -1;
-
-    g_last.a_planes = Ap; g_last.b_planes = Bp; g_last.w_planes = Wp;
-    g_last.mu = dmu; g_last.nu = dnu;
-    g_last.rows_a_padded = Mp; g_last.rows_b_padded = Np; g_last.ldk = ldk;
-    g_last.num_moduli = num_moduli; g_last.E = E;
+    if (enqueue_products(num_moduli, crt, E) != 0) return -1;
+    if (!announced) announce(num_moduli, crt);
     return 0;
 }
 
