@@ -151,7 +151,8 @@ int hip_ozaki_crt_reconstruct_f64(const int8_t* w_planes, uint64_t M, uint64_t N
 /* Whole tier: ozaki_ii_dispatch (gpu_memory.mm:2474-2665). num_moduli in
  * [2,16]; adaptive != 0 picks the count as ESHKOL_OZAKI_ADAPTIVE=1 does.
  * Returns -1 (caller falls back to the native tier) for K > 131071, non-finite
- * input, or scale factors outside the double range. */
+ * input, or scale factors outside the double range; the last two are found
+ * after the products have been queued, so C then holds no result. */
 int hip_matmul_ozaki_crt_f64(const double* A, const double* B, double* C,
                              uint64_t M, uint64_t K, uint64_t N,
                              int num_moduli, int adaptive,
