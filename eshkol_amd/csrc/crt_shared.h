@@ -64,12 +64,16 @@ struct CrtMaxima {
 };
 constexpr int32_t CRT_FL_ZERO = INT32_MIN;      /* exponent entry of a maximum of zero */
 
-/* fl_a[i] = floor(log2 amax[i]) taken from the exponent field (CRT_FL_ZERO for a
- * maximum of zero), likewise fl_b; waits for the device and fills out[0] (A) and
- * out[1] (B). Exact unless a maximum lies within 2^-40 of a power of two AND the
- * caller needs libm's floor(log2): the exact tier checks that itself. 0 on success. */
-int eshkol_crt_scan_exponents(const double* amax, uint64_t M, const double* bmax, uint64_t N,
-                              int32_t* fl_a, int32_t* fl_b, CrtMaxima out[2], hipStream_t st);
+/* Queues the scan: fl_a[i] = floor(log2 amax[i]) taken from the exponent field
+ * (CRT_FL_ZERO for a maximum of zero), likewise fl_b. Exact unless a maximum lies
+ * within 2^-40 of a power of two AND the caller needs libm's floor(log2): the
+ * exact tier checks that itself. Returns the ticket of the scan's summary, 0 on
+ * failure. The summary is written to host memory by the device: a caller queues
+ * what depends on fl_a / fl_b right away and asks for the summary afterwards. */
+uint32_t eshkol_crt_scan_launch(const double* amax, uint64_t M, const double* bmax, uint64_t N,
+                                int32_t* fl_a, int32_t* fl_b, hipStream_t st);
+/* Waits for that summary and fills out[0] (A) and out[1] (B). 0 on success. */
+int eshkol_crt_scan_result(uint32_t ticket, CrtMaxima out[2], hipStream_t st);
 
 /* In place: fl -> E - fl, and 0 where fl is CRT_FL_ZERO. */
 void eshkol_crt_shifts_from_exponents(int32_t* fl_a, uint64_t M, int32_t* fl_b, uint64_t N, int E, hipStream_t st);

@@ -627,9 +627,13 @@ int crt_split_any(const double* X, uint64_t rows, uint64_t K, const int32_t* shi
 }
 }  // namespace
 
-int eshkol_crt_scan_exponents(const double* amax, uint64_t M, const double* bmax, uint64_t N,
-                              int32_t* fl_a, int32_t* fl_b, CrtMaxima out[2], hipStream_t st) {
-    const CrtScan* h = scan_maxima(amax, M, bmax, N, fl_a, fl_b, st);
+uint32_t eshkol_crt_scan_launch(const double* amax, uint64_t M, const double* bmax, uint64_t N,
+                                int32_t* fl_a, int32_t* fl_b, hipStream_t st) {
+    return scan_launch(amax, M, bmax, N, fl_a, fl_b, st);
+}
+
+int eshkol_crt_scan_result(uint32_t ticket, CrtMaxima out[2], hipStream_t st) {
+    const CrtScan* h = scan_await(ticket, st);
     if (!h) return -1;
     for (int o = 0; o < 2; o++) {
         out[o].nonfinite = h[o].nonfinite; out[o].nonzero = h[o].nonzero;

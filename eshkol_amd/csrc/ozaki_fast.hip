@@ -363,9 +363,10 @@ extern "C" int hip_matmul_ozaki_fast_f64_ex(const double* A, const double* B, do
     if ((b_kmajor ? hip_colabsmax_f64(B, K, N, 0.0, bmax, st) : hip_rowabsmax_f64(B, N, K, 0.0, bmax, st)) != 0) return -1;
     /* frexp exponent e = floor(log2 max) + 1 (gpu_memory.mm:2886-2905); the split
      * scales by 2^(E - e), so the per-row shift is (E - 1) - floor(log2 max) */
-    CrtMaxima mx[2];
-    if (eshkol_crt_scan_exponents(amax, M, bmax, N, sha, shb, mx, st) != 0) return -1;
-    if (mx[0].nonfinite || mx[1].nonfinite) return -1;                  /* NaN / Inf: not this tier's business */
+    /* Nothing the host computes depends on the operands, so the whole pipeline is
+     * queued behind the scan and its summary (non-finite input?) is read at the end. */
+    const uint32_t ticket = eshkol_crt_scan_launch(amax, M, bmax, N, sha, shb, st);
+    if (!ticket) return -1;
     eshkol_crt_shifts_from_exponents(sha, M, shb, N, f.E - 1, st);
 
     if (split_any(A, M, K, sha, f.table, Ap, Mp, ldk, a_kmajor, st) != 0) return -1;
@@ -391,6 +392,9 @@ extern "C" int hip_matmul_ozaki_fast_f64_ex(const double* A, const double* B, do
         default: return -1;
     }
     if (!ESHKOL_HIP_OK(hipGetLastError())) return -3;
+    CrtMaxima mx[2];
+    if (eshkol_crt_scan_result(ticket, mx, st) != 0) return -1;
+    if (mx[0].nonfinite || mx[1].nonfinite) return -1;                  /* NaN / Inf: not this tier's business; C holds no result */
 
     g_last.a_planes = Ap; g_last.b_planes = Bp; g_last.w_planes = Wp;
     g_last.shift_a = sha; g_last.shift_b = shb;

@@ -177,7 +177,8 @@ int hip_ozaki_crt_last_stages(HipOzakiCrtStages* out);
  * float pairs). num_moduli is the accuracy knob, [2, 16], clamped; the
  * reference's default is 11 (about 1e-8). Returns 0, -4 where the reference
  * gives up (K too large for the moduli, fewer than two moduli under the cap),
- * -1 on non-finite input or a device error, -2 when workspace cannot be had. */
+ * -1 on non-finite input (found after the products were queued: C then holds
+ * no result) or a device error, -2 when workspace cannot be had. */
 int hip_matmul_ozaki_fast_f64(const double* A, const double* B, double* C,
                               uint64_t M, uint64_t K, uint64_t N, int num_moduli, void* stream);
 
