@@ -64,7 +64,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-stages", action="store_true")
     ap.add_argument("--only", default="", help="comma list of what to time besides native: crt,int8,reduced,mlp,backward,host")
-    ap.add_argument("--pmc-probe", default="", choices=["", "dgemm", "crt", "int8", "reduced"],
+    ap.add_argument("--pmc-probe", default="", choices=["", "dgemm", "crt", "fast", "int8", "reduced"],
                     help="run a calibration copy and three launches of one tier, for rocprofv3 --pmc")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -93,6 +93,7 @@ def main():
         dst.upload(synth.normal(12, (K, N)))
         calls = {"dgemm": lambda: lib.hip_dgemm_f64(src.ptr, dst.ptr, out.ptr, M, K, N, st),
                  "crt": lambda: lib.hip_matmul_ozaki_crt_f64(src.ptr, dst.ptr, out.ptr, M, K, N, 16, 0, None, 0, st),
+                 "fast": lambda: lib.hip_matmul_ozaki_fast_f64(src.ptr, dst.ptr, out.ptr, M, K, N, 11, st),
                  "int8": lambda: lib.hip_matmul_ozaki_int8_f64(src.ptr, dst.ptr, out.ptr, M, K, N, 6, st),
                  "reduced": lambda: lib.hip_matmul_reduced_f64(src.ptr, dst.ptr, out.ptr, M, K, N, 3, 0, st)}
         for _ in range(3):
