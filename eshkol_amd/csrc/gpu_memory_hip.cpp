@@ -98,6 +98,7 @@ struct TierEnv {
     double budget = -1.0;        /* < 0: selector off */
     int  precision = 0;          /* ESHKOL_GPU_PRECISION: 0 exact, 1 high, 2 fast, 3 ml */
     bool overlap = true;         /* ESHKOL_GPU_OVERLAP=0: no row panels in the host-memory dispatch */
+    bool crt_aligned = false;    /* ESHKOL_OZAKI_CRT_WEIGHTS=aligned: CRT weights split at a common bit */
 };
 TierEnv g_env;
 std::once_flag g_env_once;
@@ -142,6 +143,7 @@ void parse_env(void) {
     e.adaptive = ad && strcmp(ad, "1") == 0;
     e.profile = getenv("ESHKOL_OZAKI_PROFILE") != nullptr;       /* gpu_memory.mm:2479 */
     if (const char* o = getenv("ESHKOL_GPU_OVERLAP")) e.overlap = strcmp(o, "0") != 0;
+    if (const char* w = getenv("ESHKOL_OZAKI_CRT_WEIGHTS")) e.crt_aligned = strcmp(w, "aligned") == 0;
     if (const char* a = getenv("ESHKOL_MATMUL_ACCURACY")) {      /* gpu_memory_cuda.cpp:527-539 */
         if (*a) {
             if (!strcmp(a, "fast")) e.budget = 1e-2;
@@ -167,16 +169,28 @@ const TierEnv& tier_env(void) { std::call_once(g_env_once, parse_env); return g_
  * 8192^3 for the native kernel (0.059 ms, 15.2 ms). */
 const double OZAKI_TOL[9] = { 1.0, 1e-3, 1e-5, 1e-7, 1e-9, 1e-11, 1e-13, 1e-14, 1e-14 };
 struct GemmModel { double overhead_ns; double peak_gflops; };
-GemmModel g_model[9] = {
+constexpr int MODEL_CRT = 9;
+GemmModel g_model[10] = {
     /* native */ {  25000.0,  72000.0 },
     /* T1 */ { 160000.0, 505000.0 }, /* T2 */ { 225000.0, 325000.0 },
     /* T3 */ { 320000.0, 220000.0 }, /* T4 */ { 350000.0, 148000.0 },
     /* T5 */ { 245000.0, 107000.0 }, /* T6 */ { 345000.0,  81000.0 },
-    /* T7 */ { 350000.0,  63500.0 }, /* T8 */ { 315000.0,  51300.0 } };
+    /* T7 */ { 350000.0,  63500.0 }, /* T8 */ { 315000.0,  51300.0 },
+    /* Ozaki-II CRT exact, 16 moduli: 1.47 and 8.80 ms */ { 420000.0, 125000.0 } };
 const double OZAKI_SAFETY = 1.15;
 std::mutex g_model_mutex;
 
 double predict_ns(int idx, double work) { return g_model[idx].overhead_ns + work / g_model[idx].peak_gflops; }
+/* Reduced-precision CRT tier with n moduli: its times at 4096^3 and 8192^3 for
+ * n = 4 ... 16 (0.48 and 2.58 ms ... 1.39 and 8.87 ms) are linear in n on both
+ * coefficients; rate taken 5 % low like the others. */
+double predict_fast_ns(int n, double work) { return 135000.0 + 12000.0 * n + work * (0.42e-6 + 0.48e-6 * n); }
+/* Its guaranteed relative error with E bits kept per operand: measured normwise
+ * errors on well-conditioned operands are about 2^-E (1e-8 at E = 26); the
+ * guarantee is 32 times that, the margin the reference gives its slice tiers
+ * (gpu_memory_cuda.cpp:477-489). */
+double fast_tolerance(int E) { return ldexp(1.0, 5 - E); }
+
 void calibrate(int idx, double work, double measured_ns) {
     std::lock_guard<std::mutex> lk(g_model_mutex);
     double compute_ns = measured_ns - g_model[idx].overhead_ns;
@@ -184,17 +198,47 @@ void calibrate(int idx, double work, double measured_ns) {
     double achieved = work / compute_ns;
     if (achieved > g_model[idx].peak_gflops) g_model[idx].peak_gflops = achieved;
 }
-bool select_ozaki(uint64_t M, uint64_t K, uint64_t N, double budget, int* out_T, double* speedup) {
-    double work = 2.0 * (double)M * (double)K * (double)N;
-    double t_dg = predict_ns(0, work);
-    *out_T = 0; *speedup = 1.0;
-    if (K > 133000) return false;
-    int Treq = -1;
-    for (int T = 1; T <= 7; T++) if (OZAKI_TOL[T] <= budget) { Treq = T; break; }
-    if (Treq < 0) return false;
-    double t_oz = predict_ns(Treq, work);
-    if (t_oz * OZAKI_SAFETY < t_dg) { *out_T = Treq; *speedup = t_dg / t_oz; return true; }
-    return false;
+
+/* The routing decision of the accuracy budget (gpu_memory_cuda.cpp:546-566): the
+ * cheapest kernel that meets the budget, and native fp64 unless the winner is
+ * predicted 15 % faster. The reference's CUDA unit has the slice tier as its
+ * only alternative; here the two Ozaki-II tiers are candidates as well:
+ *   slices      smallest T with OZAKI_TOL[T] <= budget (none below 1e-14)
+ *   CRT fast    smallest moduli count whose E gives fast_tolerance(E) <= budget
+ *   CRT exact   every budget: its result is within 2 ulp of the exact product,
+ *               tighter than native fp64's own rounding over K terms
+ * Both CRT tiers need M, K, N >= 512 and K <= 131071, as their dispatch does. */
+struct Selection { int tier = 0; int T = 0; int fast_moduli = 0; double speedup = 1.0; };
+Selection select_tier(uint64_t M, uint64_t K, uint64_t N, double budget) {
+    const double work = 2.0 * (double)M * (double)K * (double)N;
+    const double t_native = predict_ns(0, work);
+    Selection best;
+    double t_best = t_native / OZAKI_SAFETY;
+    if (K <= 133000) {
+        for (int T = 1; T <= 7; T++) if (OZAKI_TOL[T] <= budget) {
+            const double t = predict_ns(T, work);
+            if (t < t_best) { t_best = t; best = Selection(); best.tier = 1; best.T = T; }
+            break;
+        }
+    }
+    if (M >= 512 && K >= 512 && N >= 512 && K <= 131071) {
+        for (int n = 2; n <= 16; n++) {
+            int32_t E = 0;
+            const int got = hip_ozaki_fast_plan(K, n, &E, nullptr, nullptr);
+            if (got < n) break;                       /* no more prime powers under the cap */
+            if (fast_tolerance(E) <= budget) {
+                const double t = predict_fast_ns(n, work);
+                if (t < t_best) { t_best = t; best = Selection(); best.tier = 3; best.fast_moduli = n; }
+                break;
+            }
+        }
+        /* the exact tier's guarantee and its cost model are those of sixteen moduli */
+        const TierEnv& env = tier_env();
+        const double t = predict_ns(MODEL_CRT, work);
+        if (env.num_moduli == 16 && !env.adaptive && t < t_best) { t_best = t; best = Selection(); best.tier = 2; }
+    }
+    if (best.tier != 0) best.speedup = t_native / t_best;
+    return best;
 }
 
 /* ---- buffers ------------------------------------------------------------- */
@@ -373,6 +417,8 @@ bool is_hip_buffer(const EshkolGPUBuffer* b) { return b && b->backend == ESHKOL_
 /* The tier the environment selects for a product of this shape. */
 struct TierChoice {
     bool fast = false;     /* try the reduced-precision CRT tier first */
+    int fast_moduli = 11;
+    bool crt_aligned = false;   /* CRT exact tier with its weights split at a common bit */
     int tier = 0;          /* 0 native, 1 INT8 slices, 2 CRT */
     int T = 0;
     double pred = 1.0;
@@ -383,13 +429,20 @@ TierChoice choose_tier(uint64_t M, uint64_t K, uint64_t N) {
     const TierEnv& env = tier_env();
     TierChoice c;
     c.T = env.T;
+    c.fast_moduli = env.fast_moduli;
+    c.crt_aligned = env.crt_aligned;
     c.fast = env.ozaki_fast && M >= 512 && K >= 512 && N >= 512;
     if (env.ozaki_crt || env.ozaki_fast) {
         if (M >= 512 && K >= 512 && N >= 512) { c.tier = 2; c.why = "ESHKOL_HIP_F64_KERNEL/ESHKOL_SF64_KERNEL override"; }
     } else if (env.ozaki_int8) {
         if (M >= 1024 && N >= 1024 && K >= 1024) { c.tier = 1; c.why = "ESHKOL_CUDA_F64_KERNEL override"; }
     } else if (env.budget >= 0.0) {
-        if (select_ozaki(M, K, N, env.budget, &c.T, &c.pred)) { c.tier = 1; c.why = "accuracy-budget selector"; }
+        const Selection sel = select_tier(M, K, N, env.budget);
+        c.pred = sel.speedup;
+        c.why = "accuracy-budget selector";
+        if (sel.tier == 1) { c.tier = 1; c.T = sel.T; }
+        else if (sel.tier == 2) { c.tier = 2; c.crt_aligned = true; }
+        else if (sel.tier == 3) { c.tier = 2; c.fast = true; c.fast_moduli = sel.fast_moduli; c.crt_aligned = true; }
         else c.why = "budget met cheapest by native fp64";
     }
     return c;
@@ -409,14 +462,14 @@ int run_tiers(const TierChoice& c, const double* dA, const double* dB, double* d
 
     if (c.fast) {
         auto t0 = std::chrono::steady_clock::now();
-        GPU_LOG("matmul %llux%llu @ %llux%llu -> Ozaki-II FAST (%d moduli)", (unsigned long long)M,
-                (unsigned long long)K, (unsigned long long)K, (unsigned long long)N, env.fast_moduli);
-        const int fr = hip_matmul_ozaki_fast_f64_ex(dA, dB, dC, M, K, N, ta, tb, env.fast_moduli, g_stream);
+        GPU_LOG("matmul %llux%llu @ %llux%llu -> Ozaki-II FAST (%d moduli; %s)", (unsigned long long)M,
+                (unsigned long long)K, (unsigned long long)K, (unsigned long long)N, c.fast_moduli, c.why);
+        const int fr = hip_matmul_ozaki_fast_f64_ex(dA, dB, dC, M, K, N, ta, tb, c.fast_moduli, g_stream);
         if (fr == 0 && finished()) {
             if (env.profile && wait) {
                 double ns = std::chrono::duration<double, std::nano>(std::chrono::steady_clock::now() - t0).count();
                 fprintf(stderr, "[OZAKI_PROFILE] fast M=%llu K=%llu N=%llu moduli=%d ms=%.2f GFLOPS=%.1f\n",
-                        (unsigned long long)M, (unsigned long long)K, (unsigned long long)N, env.fast_moduli,
+                        (unsigned long long)M, (unsigned long long)K, (unsigned long long)N, c.fast_moduli,
                         ns / 1e6, work / ns);
             }
             return 0;
@@ -428,11 +481,13 @@ int run_tiers(const TierChoice& c, const double* dA, const double* dB, double* d
         auto t0 = std::chrono::steady_clock::now();
         int rc;
         if (c.tier == 2) {
-            GPU_LOG("matmul %llux%llu @ %llux%llu -> Ozaki-II CRT exact (%s)",
+            GPU_LOG("matmul %llux%llu @ %llux%llu -> Ozaki-II CRT exact (%s)%s",
                     (unsigned long long)M, (unsigned long long)K, (unsigned long long)K,
-                    (unsigned long long)N, c.why);
+                    (unsigned long long)N, c.why, c.crt_aligned ? ", aligned weights" : "");
+            const int was = hip_ozaki_crt_set_aligned_weights(c.crt_aligned ? 1 : 0);
             rc = hip_matmul_ozaki_crt_f64_ex(dA, dB, dC, M, K, N, ta, tb, env.num_moduli,
                                              env.adaptive ? 1 : 0, nullptr, 0, g_stream);
+            hip_ozaki_crt_set_aligned_weights(was);
         } else {
             GPU_LOG("matmul %llux%llu @ %llux%llu -> INT8-Ozaki T=%d (%s, ~%.2fx vs native)",
                     (unsigned long long)M, (unsigned long long)K, (unsigned long long)K,
@@ -442,7 +497,7 @@ int run_tiers(const TierChoice& c, const double* dA, const double* dB, double* d
         if (rc == 0 && finished()) {
             if (wait) {
                 double ns = std::chrono::duration<double, std::nano>(std::chrono::steady_clock::now() - t0).count();
-                if (c.tier == 1) calibrate(c.T, work, ns);
+                calibrate(c.tier == 1 ? c.T : MODEL_CRT, work, ns);
                 if (env.profile)
                     fprintf(stderr, "[OZAKI_PROFILE] %s M=%llu K=%llu N=%llu ms=%.2f GFLOPS=%.1f\n",
                             c.tier == 2 ? "exact" : "int8", (unsigned long long)M, (unsigned long long)K,

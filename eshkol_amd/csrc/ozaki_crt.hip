@@ -457,8 +457,9 @@ void crt_shift_kernel(int32_t* __restrict__ fl_a, uint64_t M, int32_t* __restric
 /* ---- host bookkeeping ------------------------------------------------------ */
 
 struct HostCrt { double P1, P2, Pinv, log2P; double sl1[MAX_MODULI], sl2[MAX_MODULI]; int q[MAX_MODULI]; bool ready; };
-HostCrt g_crt[MAX_MODULI + 1];
+HostCrt g_crt[2][MAX_MODULI + 1];        /* [weights split as the reference does / at a common bit][moduli] */
 std::mutex g_crt_mutex;
+bool g_aligned_weights = false;
 
 int64_t ext_gcd(int64_t a, int64_t b, int64_t* x, int64_t* y) {
     if (a == 0) { *x = 0; *y = 1; return b; }
@@ -475,10 +476,19 @@ int mod_inverse(int64_t a, int64_t m) {
 }
 
 /* precompute_ozaki_constants, gpu_memory.mm:301-341. The volatile temporaries
- * keep the Dekker split free of fused contraction. */
-const HostCrt& crt_constants(int n) {
+ * keep the Dekker split free of fused contraction.
+ * The reference splits each weight s_l = (P / p_l) q_l relative to the weight's
+ * own exponent, so the lowest bits of the upper parts sl1 lie between 2^81 and
+ * 2^88 (sixteen moduli) and the sum of sl1_l w_l, up to 2^137, is not always
+ * representable: on N(0,1) operands about one element in 150 is off by a
+ * multiple of 2^81 in the scaled integer (2^-25 of a typical element; normwise
+ * 1e-11 ... 1e-10). That is the reference's result and the default here. With
+ * `aligned` every sl1 is a multiple of 2^e, e = bits(P) + 7 + ceil(log2 n) - 53,
+ * the partial sums are exact and the tier delivers what its scaling allows
+ * (normwise 1e-17); the kernels are the same, only these constants differ. */
+const HostCrt& crt_constants(int n, bool aligned) {
     std::lock_guard<std::mutex> lk(g_crt_mutex);
-    HostCrt& c = g_crt[n];
+    HostCrt& c = g_crt[aligned ? 1 : 0][n];
     if (c.ready) return c;
     __int128 P = 1;
     for (int l = 0; l < n; l++) P *= H_MODULI[l];
@@ -486,12 +496,22 @@ const HostCrt& crt_constants(int n) {
     c.P2 = (double)(P - (__int128)c.P1);
     c.Pinv = 1.0 / (double)P;
     c.log2P = log2((double)P);
+    int bits_P = 0;
+    for (__int128 t = P; t > 0; t >>= 1) bits_P++;
     for (int l = 0; l < n; l++) {
         const int p = H_MODULI[l];
         const __int128 Pp = P / p;
         c.q[l] = mod_inverse((int64_t)(Pp % p), p);
         const __int128 s = Pp * (__int128)c.q[l];
         const int bits_to_remove = 8 + (int)ceil(log2((double)n));
+        if (aligned) {
+            const int e = bits_P + (bits_to_remove - 1) - 53;
+            __int128 hi = s;
+            if (e > 0) hi = ((s + ((__int128)1 << (e - 1))) >> e) << e;
+            c.sl1[l] = (double)hi;
+            c.sl2[l] = (double)(s - hi);
+            continue;
+        }
         const double s_d = (double)s;
         const double factor = (double)(1LL << (bits_to_remove + 1)) + 1.0;
         volatile double t = factor * s_d;
@@ -502,6 +522,7 @@ const HostCrt& crt_constants(int n) {
     c.ready = true;
     return c;
 }
+const HostCrt& crt_constants(int n) { return crt_constants(n, g_aligned_weights); }
 
 double g_log2_cumul[MAX_MODULI + 1];
 std::once_flag g_cumul_once;
@@ -688,6 +709,12 @@ extern "C" int hip_ozaki_crt_reconstruct_f64(const int8_t* w_planes, uint64_t M,
 }
 
 extern "C" void hip_ozaki_crt_set_host_pass(int on) { g_force_host_pass = on != 0; }
+
+extern "C" int hip_ozaki_crt_set_aligned_weights(int on) {
+    const int was = g_aligned_weights ? 1 : 0;
+    g_aligned_weights = on != 0;
+    return was;
+}
 
 extern "C" int hip_ozaki_crt_last_stages(HipOzakiCrtStages* out) {
     if (!out || !g_last.a_planes) return -1;

@@ -245,20 +245,20 @@ long mod_inverse(long a, long m) {
 }
 
 /* gpu_memory.mm:2831-2857; 0, or -4 where the reference gives up */
-int make_plan(uint64_t K, int n_mod, FastPlan* out) {
+int make_plan(uint64_t K, int n_mod, FastPlan* out, bool quiet = false) {
     FastPlan f;
     int cap = (int)floor(2.0 * sqrt(16777216.0 / (double)K));
     if (cap > 255) cap = 255;
     while (cap > 2 && (double)K * floor(cap / 2.0) * floor(cap / 2.0) >= 16777216.0) cap--;
     if (cap < 2) {
-        fprintf(stderr, "[GPU] Ozaki-II FAST: K=%llu too large for the tier's moduli; falling back\n", (unsigned long long)K);
+        if (!quiet) fprintf(stderr, "[GPU] Ozaki-II FAST: K=%llu too large for the tier's moduli; falling back\n", (unsigned long long)K);
         return -4;
     }
     if (n_mod > FAST_MAX_MODULI) n_mod = FAST_MAX_MODULI;
     if (n_mod < 2) n_mod = 2;
     const std::vector<int> mod = build_moduli(cap, n_mod);
     if (mod.size() < 2) {
-        fprintf(stderr, "[GPU] Ozaki-II FAST: too few coprime moduli <= cap %d; falling back\n", cap);
+        if (!quiet) fprintf(stderr, "[GPU] Ozaki-II FAST: too few coprime moduli <= cap %d; falling back\n", cap);
         return -4;
     }
     f.n = (int)mod.size(); f.cap = cap;
@@ -327,6 +327,17 @@ int split_any(const double* X, uint64_t rows, uint64_t K, const int32_t* shift, 
 }
 
 }  // namespace
+
+extern "C" int hip_ozaki_fast_plan(uint64_t K, int num_moduli, int32_t* E, int32_t* cap, int32_t* moduli) {
+    if (K == 0 || K > 131071) return -4;
+    FastPlan f;
+    const int rc = make_plan(K, num_moduli, &f, true);
+    if (rc != 0) return rc;
+    if (E) *E = f.E;
+    if (cap) *cap = f.cap;
+    if (moduli) for (int l = 0; l < FAST_MAX_MODULI; l++) moduli[l] = (l < f.n) ? f.moduli[l] : 0;
+    return f.n;
+}
 
 extern "C" int hip_ozaki_fast_last_stages(HipOzakiFastStages* out) {
     if (!out || !g_last.a_planes) return -1;

@@ -158,6 +158,19 @@ int hip_matmul_ozaki_crt_f64(const double* A, const double* B, double* C,
                              int num_moduli, int adaptive,
                              const double* bias, int act, void* stream);
 
+/* How the CRT weights s_l = (P / p_l) q_l are split into the two doubles the
+ * accumulation uses. 0 (default): as the reference does (gpu_memory.mm:322-337),
+ * each relative to its own exponent; results equal the reference's bit for bit,
+ * including its defect: the upper parts then end at different bits, their
+ * weighted sum is not always representable, and on general operands about one
+ * element in 150 is wrong by 2^-25 of a typical element. 1: at one common bit
+ * position, which makes that sum exact (normwise error about 1e-17; same
+ * kernels, same residues and products). The environment variable
+ * ESHKOL_OZAKI_CRT_WEIGHTS=aligned selects 1 for the dispatcher's calls, and
+ * the accuracy-budget selector uses 1 when it picks this tier. Returns the
+ * previous setting. */
+int hip_ozaki_crt_set_aligned_weights(int on);
+
 /* Stage outputs of the last hip_matmul_ozaki_crt_f64 call, for parity checks:
  * device pointers into the library workspace (valid until the next call). */
 typedef struct {
@@ -197,6 +210,14 @@ typedef struct {
     int32_t moduli[16];
 } HipOzakiFastStages;
 int hip_ozaki_fast_last_stages(HipOzakiFastStages* out);
+
+/* What that tier would use for a contraction length K and a requested moduli
+ * count (gpu_memory.mm:2802-2857), without running anything: returns the number
+ * of moduli (it can be below the request when too few prime powers fit under
+ * the cap) or -4 where the tier gives up, and fills E (bits kept per operand),
+ * cap and moduli[16] where the pointers are not NULL. The accuracy-budget
+ * selector asks it for the smallest count whose E meets a budget. */
+int hip_ozaki_fast_plan(uint64_t K, int num_moduli, int32_t* E, int32_t* cap, int32_t* moduli);
 
 /* ---- INT8 slice tier ----------------------------------------------------------
  * s base-128 slices of X[i,k] / scale[i] (gpu_cuda_kernels.cu:688-723):

@@ -172,13 +172,16 @@ def matmul_ozaki_int8(A, B, T):
 
 # ---- CRT exact tier -----------------------------------------------------------
 
-def crt_constants(n):
+def crt_constants(n, aligned=False):
     c = CRTConstants()
-    lib().oracle_ozaki_crt_constants(C.c_int(n), C.byref(c))
+    if aligned:
+        lib().oracle_ozaki_crt_constants_aligned(C.c_int(n), C.byref(c))
+    else:
+        lib().oracle_ozaki_crt_constants(C.c_int(n), C.byref(c))
     return c
 
 
-def ozaki_crt_stages(A, B, num_moduli=16, adaptive=False):
+def ozaki_crt_stages(A, B, num_moduli=16, adaptive=False, aligned=False):
     """Every stage of the CRT tier: mu, nu, E, residue planes, products, C."""
     A, B = _f64(A), _f64(B)
     M, K = A.shape
@@ -187,7 +190,7 @@ def ozaki_crt_stages(A, B, num_moduli=16, adaptive=False):
     if adaptive:
         L.oracle_ozaki_adaptive_n.restype = C.c_int
         num_moduli = L.oracle_ozaki_adaptive_n(_d(A), _d(B), u64(M), u64(K), u64(N), C.c_int(num_moduli))
-    crt = crt_constants(num_moduli)
+    crt = crt_constants(num_moduli, aligned)
     n = crt.num_moduli
     mu = np.empty(M, dtype=np.int32)
     nu = np.empty(N, dtype=np.int32)
@@ -208,13 +211,18 @@ def ozaki_crt_stages(A, B, num_moduli=16, adaptive=False):
                 crt=crt, num_moduli=n)
 
 
-def matmul_ozaki_crt(A, B, num_moduli=16, adaptive=False):
+def matmul_ozaki_crt(A, B, num_moduli=16, adaptive=False, aligned=False):
     A, B = _f64(A), _f64(B)
     M, K = A.shape
     N = B.shape[1]
     out = np.empty((M, N))
-    rc = lib().oracle_matmul_ozaki_crt_f64(_d(A), _d(B), _d(out), u64(M), u64(K), u64(N),
+    L = lib()
+    L.oracle_ozaki_crt_use_aligned_weights(C.c_int(1 if aligned else 0))
+    try:
+        rc = L.oracle_matmul_ozaki_crt_f64(_d(A), _d(B), _d(out), u64(M), u64(K), u64(N),
                                            C.c_int(num_moduli), C.c_int(1 if adaptive else 0))
+    finally:
+        L.oracle_ozaki_crt_use_aligned_weights(C.c_int(0))
     return out if rc == 0 else None
 
 

@@ -145,6 +145,9 @@ typedef struct {
 /* precompute_ozaki_constants, gpu_memory.mm:301-341 (n clamped to [2,16] as
  * get_ozaki_crt does, 344-359). */
 void oracle_ozaki_crt_constants(int n, OracleCRTConstants* crt);
+/* the same constants with the weights split at one common bit position (not the reference's split) */
+void oracle_ozaki_crt_constants_aligned(int n, OracleCRTConstants* crt);
+void oracle_ozaki_crt_use_aligned_weights(int on);
 
 /* ozaki_compute_frac_bounds, gpu_memory.mm:376-420. */
 void oracle_ozaki_frac_bounds(const double* A, const double* B,

@@ -15,6 +15,12 @@
  * stated as fma(): that is what the reference's compiler (clang, contraction
  * on within a statement) emits on the machines the Metal path runs on.
  * Compile with -ffp-contract=off.
+ *
+ * One addition that is not the reference: oracle_ozaki_crt_constants_aligned
+ * gives the same constants with the CRT weights split at a common bit position
+ * (the split the library offers as an option, where the reference's own split
+ * makes the accumulation inexact). It is pinned by exact integer arithmetic in
+ * tests/test_oracle_ozaki.py, not by the reference.
  */
 #include "eshkol_oracle.h"
 #include <math.h>
@@ -45,8 +51,18 @@ static int mod_inverse(int64_t a, int64_t m) {
     return (int)((x % m + m) % m);
 }
 
-/* gpu_memory.mm:301-341, clamp of 344-353 */
-void oracle_ozaki_crt_constants(int n, OracleCRTConstants* crt) {
+/* gpu_memory.mm:301-341, clamp of 344-353. With aligned != 0 the weights
+ * s_l = (P / p_l) q_l are split at one common bit position instead (not in the
+ * reference): the reference takes the upper 40 bits of each weight by a
+ * Veltkamp split relative to that weight's own exponent, so the lowest bit of
+ * sl1 sits anywhere from 2^81 to 2^88 for sixteen moduli, and the sum of
+ * sl1_l w_l (up to 2^137) is then not always representable: on operands drawn
+ * from N(0,1) about one element in 150 comes back wrong by a multiple of 2^81 in
+ * the scaled integer, 2^-25 of a typical element. Aligned, every sl1 is a
+ * multiple of 2^e with e = bits(P) + 7 + ceil(log2 n) - 53, the partial sums
+ * are exact, and what is left are roundings of the low parts, about 2^-60 of
+ * a row's scale. */
+static void crt_constants(int n, int aligned, OracleCRTConstants* crt) {
     if (n < 2) n = 2;
     if (n > ORACLE_OZAKI_MAX_MODULI) n = ORACLE_OZAKI_MAX_MODULI;
     memset(crt, 0, sizeof *crt);
@@ -58,12 +74,22 @@ void oracle_ozaki_crt_constants(int n, OracleCRTConstants* crt) {
     crt->P2 = (double)(P - P1_int);
     crt->Pinv = 1.0 / (double)P;
     crt->log2P = log2((double)P);
+    int bits_P = 0;
+    for (__int128 t = P; t > 0; t >>= 1) bits_P++;
     for (int l = 0; l < n; l++) {
         int p = ORACLE_OZAKI_MODULI[l];
         __int128 Pp = P / p;
         crt->q[l] = mod_inverse((int64_t)(Pp % p), p);
         __int128 s = Pp * (__int128)crt->q[l];
         int bits_to_remove = 8 + (int)ceil(log2((double)n));
+        if (aligned) {
+            const int e = bits_P + (bits_to_remove - 1) - 53;
+            __int128 hi = s;
+            if (e > 0) hi = ((s + ((__int128)1 << (e - 1))) >> e) << e;
+            crt->sl1[l] = (double)hi;                 /* at most bits_P - e <= 53 significant bits: exact */
+            crt->sl2[l] = (double)(s - hi);
+            continue;
+        }
         double s_d = (double)s;
         double factor = (double)(1LL << (bits_to_remove + 1)) + 1.0;
         double t = factor * s_d;
@@ -73,6 +99,13 @@ void oracle_ozaki_crt_constants(int n, OracleCRTConstants* crt) {
         crt->sl2[l] = (double)(s - sl1_int);
     }
 }
+
+void oracle_ozaki_crt_constants(int n, OracleCRTConstants* crt) { crt_constants(n, 0, crt); }
+void oracle_ozaki_crt_constants_aligned(int n, OracleCRTConstants* crt) { crt_constants(n, 1, crt); }
+
+/* oracle_matmul_ozaki_crt_f64 and oracle_mlp_layer_f64 use the aligned weights while this is set */
+static int g_aligned_weights = 0;
+void oracle_ozaki_crt_use_aligned_weights(int on) { g_aligned_weights = on != 0; }
 
 static void row_col_max(const double* A, const double* B, uint64_t M, uint64_t K, uint64_t N,
                         double* rmax, double* cmax) {
@@ -248,7 +281,7 @@ int oracle_matmul_ozaki_crt_f64(const double* A, const double* B, double* C,
     if (num_moduli > ORACLE_OZAKI_MAX_MODULI) num_moduli = ORACLE_OZAKI_MAX_MODULI;
     if (adaptive) num_moduli = oracle_ozaki_adaptive_n(A, B, M, K, N, num_moduli);
     OracleCRTConstants crt;
-    oracle_ozaki_crt_constants(num_moduli, &crt);
+    crt_constants(num_moduli, g_aligned_weights, &crt);
     int* mu = (int*)malloc((size_t)M * sizeof(int));
     int* nu = (int*)malloc((size_t)N * sizeof(int));
     int8_t* ap = (int8_t*)malloc((size_t)num_moduli * M * K);

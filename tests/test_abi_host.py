@@ -196,3 +196,25 @@ def test_out_of_range_knobs_are_loud():
 def test_threshold_env_is_read_at_init():
     r = run_child('lib.eshkol_gpu_init(); print(lib.eshkol_gpu_get_threshold())', {"ESHKOL_GPU_THRESHOLD": "777"})
     assert r.returncode == 0 and r.stdout.strip().endswith("777")
+
+
+def test_fast_tier_plan_query_matches_the_oracle():
+    """hip_ozaki_fast_plan is host arithmetic only (cap, prime-power moduli, E): the
+    same numbers as the oracle's restatement of gpu_memory.mm:2802-2857 for every
+    moduli count, at contraction lengths on both sides of the cap's steps."""
+    import ctypes as C
+    import oracle
+    lib = ea.load()
+    for K in (1, 2, 64, 512, 1000, 1024, 4096, 8192, 20000, 65536, 131071):
+        for n in range(2, 17):
+            E, cap = C.c_int32(), C.c_int32()
+            mod = (C.c_int32 * 16)()
+            got = lib.hip_ozaki_fast_plan(K, n, C.byref(E), C.byref(cap), mod)
+            rc, c = oracle.fast_constants(K, n)
+            if rc != 0:
+                assert got == -4, (K, n)
+                continue
+            assert got == c.num_moduli and E.value == c.E and cap.value == c.cap, (K, n)
+            assert list(mod[:got]) == list(c.moduli[:got]) and not any(mod[got:])
+    assert lib.hip_ozaki_fast_plan(131072, 11, None, None, None) == -4
+    assert lib.hip_ozaki_fast_plan(0, 11, None, None, None) == -4

@@ -451,7 +451,31 @@ assert err <= float(os.environ["EXPECT_ERR"]), err
     r = run_child(body2, {"ESHKOL_MATMUL_ACCURACY": "fast", "EXPECT_ERR": "1e-3", "ESHKOL_GPU_THRESHOLD": "1",
                           "ESHKOL_GPU_VERBOSE": "1"})
     assert "INT8-Ozaki T=1 (accuracy-budget selector" in r.stderr
-    r = run_child(body2, {"ESHKOL_MATMUL_ACCURACY": "exact", "EXPECT_ERR": "1e-14", "ESHKOL_GPU_THRESHOLD": "1",
+    # a strict budget at this size is met cheapest by the Ozaki-II exact tier (2 ulp per element) ...
+    r = run_child(body2, {"ESHKOL_MATMUL_ACCURACY": "exact", "EXPECT_ERR": "1e-15", "ESHKOL_GPU_THRESHOLD": "1",
+                          "ESHKOL_GPU_VERBOSE": "1"})
+    assert "Ozaki-II CRT exact (accuracy-budget selector), aligned weights" in r.stderr
+    r = run_child(body2, {"ESHKOL_MATMUL_ACCURACY": "1e-13", "EXPECT_ERR": "1e-13", "ESHKOL_GPU_THRESHOLD": "1",
+                          "ESHKOL_GPU_VERBOSE": "1"})
+    assert "Ozaki-II CRT exact (accuracy-budget selector), aligned weights" in r.stderr
+    # the override by name keeps the reference's weights (and its error on such operands) unless told otherwise
+    r = run_child(body2, {"ESHKOL_HIP_F64_KERNEL": "ozaki-crt", "EXPECT_ERR": "1e-9", "ESHKOL_GPU_THRESHOLD": "1",
+                          "ESHKOL_GPU_VERBOSE": "1"})
+    assert "Ozaki-II CRT exact (" in r.stderr and "aligned weights" not in r.stderr
+    r = run_child(body2, {"ESHKOL_HIP_F64_KERNEL": "ozaki-crt", "ESHKOL_OZAKI_CRT_WEIGHTS": "aligned", "EXPECT_ERR": "1e-15",
+                          "ESHKOL_GPU_THRESHOLD": "1", "ESHKOL_GPU_VERBOSE": "1"})
+    assert "aligned weights" in r.stderr
+    # ... a middling one by the reduced-precision CRT tier with just enough moduli ...
+    r = run_child(body2, {"ESHKOL_MATMUL_ACCURACY": "1e-10", "EXPECT_ERR": "1e-10", "ESHKOL_GPU_THRESHOLD": "1",
+                          "ESHKOL_GPU_VERBOSE": "1"})
+    assert "Ozaki-II FAST (" in r.stderr and "accuracy-budget selector)" in r.stderr
+    # ... and with the exact tier cut down to fewer moduli (no longer exact) it is not a candidate
+    r = run_child(body2, {"ESHKOL_MATMUL_ACCURACY": "exact", "ESHKOL_OZAKI_NUM_MODULI": "12", "EXPECT_ERR": "1e-14",
+                          "ESHKOL_GPU_THRESHOLD": "1", "ESHKOL_GPU_VERBOSE": "1"})
+    assert "native fp64 MFMA (budget met cheapest by native fp64)" in r.stderr
+    # small products stay native whatever the budget
+    body3 = body2.replace("n = 4096", "n = 1024").replace("range(0, n, 587)", "range(0, n, 97)")
+    r = run_child(body3, {"ESHKOL_MATMUL_ACCURACY": "exact", "EXPECT_ERR": "1e-14", "ESHKOL_GPU_THRESHOLD": "1",
                           "ESHKOL_GPU_VERBOSE": "1"})
     assert "native fp64 MFMA (budget met cheapest by native fp64)" in r.stderr
 

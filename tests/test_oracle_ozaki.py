@@ -229,6 +229,65 @@ def test_crt_tier_meets_reference_gate_on_regimes():
                 assert abs(Cc[i, j] - ref[i, j]) / denom < 1e-9
 
 
+def _scaled_integer_products(A, B, mu, nu):
+    """The exact integers the tier multiplies: sum_k trunc(a 2^mu) trunc(b 2^nu)."""
+    import math
+    M, K = A.shape
+    N = B.shape[1]
+    ai = [[int(math.trunc(math.ldexp(float(A[i, k]), int(mu[i])))) for k in range(K)] for i in range(M)]
+    bi = [[int(math.trunc(math.ldexp(float(B[k, j]), int(nu[j])))) for k in range(K)] for j in range(N)]
+    return [[sum(x * y for x, y in zip(ai[i], bi[j])) for j in range(N)] for i in range(M)]
+
+
+def test_crt_weight_split_of_the_reference_loses_bits_and_the_aligned_one_does_not():
+    """The reference splits every CRT weight relative to the weight's own exponent
+    (gpu_memory.mm:322-337): the upper parts end at different bits, and their
+    weighted sum is not always representable. Pinned here as a fact of the reference
+    (the default mode reproduces it bit for bit), next to the split at a common bit
+    position, whose sum is exact."""
+    n = 16
+    P = 1
+    for m in MOD[:n]:
+        P *= m
+    ref_c, al_c = oracle.crt_constants(n), oracle.crt_constants(n, aligned=True)
+    lsb = lambda x: (int(x) & -int(x)).bit_length() - 1
+    ref_lsb = [lsb(ref_c.sl1[l]) for l in range(n)]
+    assert min(ref_lsb) == 81 and max(ref_lsb) == 88          # sum of 16 * 128 * 2^126 needs bits >= 2^84 only
+    e = P.bit_length() + 7 + 4 - 53
+    assert e == 84
+    for l, m in enumerate(MOD[:n]):
+        s = (P // m) * al_c.q[l]
+        assert al_c.q[l] == ref_c.q[l] and s % m == 1
+        assert int(al_c.sl1[l]) % (1 << e) == 0 and abs(s - int(al_c.sl1[l])) <= 1 << (e - 1)
+        assert abs(s - int(al_c.sl1[l]) - int(al_c.sl2[l])) <= 1 << (e - 1 - 52)
+    assert (al_c.P1, al_c.P2, al_c.Pinv) == (ref_c.P1, ref_c.P2, ref_c.Pinv)
+
+    A, B = synth.normal(1, (24, 256)), synth.normal(2, (256, 20))
+    so, sa = oracle.ozaki_crt_stages(A, B), oracle.ozaki_crt_stages(A, B, aligned=True)
+    assert np.array_equal(so["w_planes"], sa["w_planes"]) and np.array_equal(so["mu"], sa["mu"])
+    X = _scaled_integer_products(A, B, so["mu"], so["nu"])
+    bad_ref = 0
+    for i in range(A.shape[0]):
+        for j in range(B.shape[1]):
+            sh = int(so["mu"][i] + so["nu"][j])
+            exact = Fraction(X[i][j], 1 << sh)
+            err_ref = abs(Fraction(float(so["C"][i, j])) - exact) * (1 << sh)       # in units of the scaled integer
+            err_al = abs(Fraction(float(sa["C"][i, j])) - exact) * (1 << sh)
+            if err_ref > 2 ** 70:
+                bad_ref += 1
+                assert 2 ** 80 < err_ref < 2 ** 86                                  # a rounding at 2^134 ... 2^137
+            # aligned: roundings of the low parts (below 2^47) and of the result itself
+            assert err_al <= 2 ** 47 + abs(X[i][j]) // 2 ** 52, (i, j, float(err_al))
+    assert 1 <= bad_ref <= 24                                                        # about one element in 150
+    # whole-tier entry: the same numbers, and what they mean against the true product
+    ref = (A.astype(np.longdouble) @ B.astype(np.longdouble))
+    scale = np.linalg.norm(A) * np.linalg.norm(B)
+    Ca, Cr = oracle.matmul_ozaki_crt(A, B, aligned=True), oracle.matmul_ozaki_crt(A, B)
+    assert np.array_equal(Ca, sa["C"]) and np.array_equal(Cr, so["C"])
+    assert float(np.linalg.norm((Ca - ref).astype(np.float64))) / scale < 1e-16
+    assert float(np.linalg.norm((Cr - ref).astype(np.float64))) / scale > 1e-12
+
+
 def test_crt_small_exact_integer_products():
     # with 2-bit integers the true product is far below 2^53: it must come back exactly
     rng = np.random.default_rng(2)
