@@ -64,6 +64,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-stages", action="store_true")
     ap.add_argument("--only", default="", help="comma list of what to time besides native: crt,int8,reduced,mlp,backward,host")
+    ap.add_argument("--no-accuracy", action="store_true", help="skip the extended-precision check of sampled rows")
     ap.add_argument("--pmc-probe", default="", choices=["", "dgemm", "crt", "fast", "int8", "reduced"],
                     help="run a calibration copy and three launches of one tier, for rocprofv3 --pmc")
     args = ap.parse_args()
@@ -118,6 +119,23 @@ def main():
         wall_ms = (time.perf_counter() - t0) * 1e3
         return ev_ms / k, wall_ms / k
 
+    # Accuracy next to speed: the normwise error of the result's sampled rows against a product of the
+    # same rows in extended precision (numpy longdouble), ||C - C_ref||_F / (||A||_F ||B||_F).
+    acc_rows = [0, M // 3 + 1, (2 * M) // 3 + 2, M - 1]
+
+    def reference_rows(Ah, Bh):
+        if args.no_accuracy:
+            return None
+        Bl = Bh.astype(np.longdouble)
+        return (np.stack([Ah[r].astype(np.longdouble) @ Bl for r in acc_rows]),
+                float(np.linalg.norm(Ah[acc_rows]) * np.linalg.norm(Bh)))
+
+    def sampled_error(ref):
+        if ref is None:
+            return None
+        got = dC.download()[acc_rows]
+        return float(np.linalg.norm((got - ref[0]).astype(np.float64)) / ref[1])
+
     # ---- native fp64 tier: configuration 2 ------------------------------------
     log("generating N(0,1) operands %dx%d" % (n, n))
     A = synth.normal(11, (M, K))
@@ -126,6 +144,8 @@ def main():
     ev_ms, wall_ms = timed(lambda: lib.hip_dgemm_f64(dA.ptr, dB.ptr, dC.ptr, M, K, N, st))
     native_gflops = flops / (wall_ms * 1e-3) / 1e9
     achieved = flops / (ev_ms * 1e-3)
+    ref_normal = reference_rows(A, B)
+    native_error = sampled_error(ref_normal)
     log("native fp64: %.3f ms/step (events %.3f ms) %.1f GFLOP/s" % (wall_ms, ev_ms, native_gflops))
     # what the device itself sustains on a register-only MFMA loop / a large copy
     sustained = {}
@@ -143,7 +163,7 @@ def main():
                 "frac": achieved / PEAK["fp64_mfma"], "launch_ms": ev_ms,
                 "traffic": read_traffic("dgemm_8192_hbm_traffic.txt")}
     tiers = {"native_fp64": {"ms": wall_ms, "gflops": native_gflops, "frac_of_peak": achieved / PEAK["fp64_mfma"],
-                             "peak": "fp64 MFMA 78.6 TFLOP/s"}}
+                             "peak": "fp64 MFMA 78.6 TFLOP/s", "normwise_error_sampled_rows": native_error}}
 
     # non-square case of configuration 2 (tile edges)
     N2 = max(n // 8, 1)
@@ -166,9 +186,24 @@ def main():
             e3, w3 = timed(lambda: lib.hip_matmul_ozaki_crt_f64(dA.ptr, dB.ptr, dC.ptr, M, K, N, 16, 0, None, 0, st))
         finally:
             os.dup2(saved, 2)
+        ref_wide = reference_rows(Aw, Bw)
+        err_crt = sampled_error(ref_wide)
+        lib.hip_ozaki_crt_set_aligned_weights(1)
+        os.dup2(devnull, 2)
+        try:
+            lib.hip_matmul_ozaki_crt_f64(dA.ptr, dB.ptr, dC.ptr, M, K, N, 16, 0, None, 0, st)
+            hip.hipDeviceSynchronize()
+        finally:
+            os.dup2(saved, 2)
+            lib.hip_ozaki_crt_set_aligned_weights(0)
+        err_crt_aligned = sampled_error(ref_wide)
         tiers["ozaki_crt_exact_16_moduli"] = {
             "ms": w3, "gflops_fp64_equiv": flops / (w3 * 1e-3) / 1e9,
-            "vs_native": (flops / (w3 * 1e-3) / 1e9) / native_gflops}
+            "vs_native": (flops / (w3 * 1e-3) / 1e9) / native_gflops,
+            "normwise_error_sampled_rows": err_crt,
+            "normwise_error_with_aligned_weights": err_crt_aligned,
+            "note": "default weights reproduce the reference bit for bit, including its inexact accumulation; "
+                    "aligned weights (same kernels, same time) make it exact"}
         log("ozaki crt: %.3f ms/step %.1f GFLOP/s-eq" % (w3, flops / (w3 * 1e-3) / 1e9))
 
         # the reduced-precision CRT tier on the same operands (11 moduli: the reference's ~1e-8 default)
@@ -180,6 +215,7 @@ def main():
         tiers["ozaki_crt_fast_11_moduli"] = {
             "ms": wf, "gflops_fp64_equiv": flops / (wf * 1e-3) / 1e9,
             "vs_native": (flops / (wf * 1e-3) / 1e9) / native_gflops,
+            "normwise_error_sampled_rows": sampled_error(ref_wide),
             "note": "prime-power moduli <= 90 at K = 8192, E = 26 bits per operand, about 1e-8 normwise"}
         log("ozaki crt fast (11 moduli): %.3f ms/step %.1f GFLOP/s-eq" % (wf, flops / (wf * 1e-3) / 1e9))
 
@@ -225,7 +261,8 @@ def main():
                        k=max(3, steps // 2), w=2)
         tiers["ozaki_int8_slices_T6"] = {"ms": w4, "gflops_fp64_equiv": flops / (w4 * 1e-3) / 1e9,
                                          "vs_native": (flops / (w4 * 1e-3) / 1e9) / native_gflops,
-                                         "int8_TOPs": 28 * flops / (e4 * 1e-3) / 1e12}
+                                         "int8_TOPs": 28 * flops / (e4 * 1e-3) / 1e12,
+                                         "normwise_error_sampled_rows": sampled_error(ref_normal)}
         log("ozaki int8 T=6: %.3f ms/step %.1f GFLOP/s-eq" % (w4, flops / (w4 * 1e-3) / 1e9))
 
     # ---- reduced tier: configuration 4 ---------------------------------------------------
