@@ -245,7 +245,9 @@ lib.eshkol_gpu_resident_unpin(B.ctypes.data)
     ({"ESHKOL_OZAKI_FAST": "1"}, 0, "Ozaki-II FAST"),
     ({"ESHKOL_HIP_F64_KERNEL": "ozaki-int8"}, 0, "INT8-Ozaki T=6"),
     ({}, 3, "row panels"),
-], ids=["native", "crt", "crt-fast", "int8-slices", "bf16"])
+    ({}, 2, "row panels"),
+    ({"ESHKOL_MATMUL_ACCURACY": "1e-6"}, 0, "Ozaki-II FAST (9 moduli; accuracy-budget selector)"),
+], ids=["native", "crt", "crt-fast", "int8-slices", "bf16", "f16", "budget-1e-6"])
 def test_host_memory_dispatch_in_row_panels(gpu, env, dtype, tier_line):
     """Large products on host memory go through the device in row panels of A
     and C so that copies and products overlap; the result is the one-piece one."""
