@@ -112,3 +112,33 @@ def test_rejects_what_the_tier_cannot_represent(gpu):
     assert run_fast(An, B)[0] == -1
     Bi = B.copy(); Bi[1, 2] = np.inf
     assert run_fast(A, Bi)[0] == -1
+
+
+@pytest.mark.parametrize("n_mod", [3, 5, 8, 11, 14, 16])
+def test_error_stays_inside_the_tolerance_the_budget_selector_assumes(gpu, n_mod):
+    """The accuracy-budget selector credits this tier with a relative error of
+    2^(5 - E) for E bits kept per operand (32 times what well-conditioned operands
+    show). Checked here on N(0,1) operands, on operands of equal magnitude and
+    random sign (every rounding as large as it can be) and on rows of very
+    different scale (each row is scaled by its own maximum)."""
+    import ctypes as C
+    import eshkol_amd as ea
+    M, K, N = 256, 2048, 192
+    E = C.c_int32()
+    got_n = ea.load().hip_ozaki_fast_plan(K, n_mod, C.byref(E), None, None)
+    assert got_n == n_mod
+    tol = 2.0 ** (5 - E.value)
+    rng = np.random.default_rng(n_mod)
+    cases = [(synth.normal(3, (M, K)), synth.normal(4, (K, N))),
+             (np.where(rng.random((M, K)) < 0.5, -0.7, 0.7) * (1 + 1e-3 * rng.random((M, K))),
+              np.where(rng.random((K, N)) < 0.5, -1.3, 1.3) * (1 + 1e-3 * rng.random((K, N)))),
+             (synth.normal(5, (M, K)) * 2.0 ** rng.integers(-20, 20, (M, 1)),
+              synth.normal(6, (K, N)) * 2.0 ** rng.integers(-20, 20, (1, N)))]
+    for A, B in cases:
+        rc, Cg, _ = run_fast(A, B, n_mod, want_stages=False)
+        assert rc == 0
+        ref = A.astype(np.longdouble) @ B.astype(np.longdouble)
+        # row by row and column by column, so that small rows are not hidden behind large ones
+        err = np.abs((Cg - ref).astype(np.float64))
+        scale = np.linalg.norm(A, axis=1)[:, None] * np.linalg.norm(B, axis=0)[None, :]
+        assert (err / scale).max() <= tol, (n_mod, E.value, float((err / scale).max()), tol)
