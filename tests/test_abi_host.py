@@ -218,3 +218,17 @@ def test_fast_tier_plan_query_matches_the_oracle():
             assert list(mod[:got]) == list(c.moduli[:got]) and not any(mod[got:])
     assert lib.hip_ozaki_fast_plan(131072, 11, None, None, None) == -4
     assert lib.hip_ozaki_fast_plan(0, 11, None, None, None) == -4
+
+
+def test_bench_refuses_more_than_one_gpu_and_fails_loudly_without_a_device():
+    import subprocess, sys, os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode != 0 and "one GPU only" in (r.stdout + r.stderr)
+    import torch
+    if not torch.cuda.is_available():
+        r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--steps", "1", "--warmup", "0"],
+                           capture_output=True, text=True, timeout=300)
+        assert r.returncode != 0 and "no gfx950 device" in r.stderr     # no CPU path stands in for the GPU
+        assert not r.stdout.strip()                                     # and no result line is printed
