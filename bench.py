@@ -369,6 +369,40 @@ def main():
                     "pages; never the headline value"}
         log("eshkol_matmul_dispatch from host memory: %.1f ms %.1f GFLOP/s (first call %.1f ms)"
             % (dt * 1e3, flops / dt / 1e9, calls[0] * 1e3))
+        # what the boundary's copies are made of: plain hipMemcpy on the same pageable arrays, the
+        # same copies out of pinned memory, and the library's staged copies (wrap = upload, sync = download)
+        rates = {}
+        nbytes = A.nbytes
+        dtmp = ea.DeviceArray((M, K))
+
+        def gbps(fn, reps=3):
+            best = 1e9
+            for _ in range(reps):
+                t0 = time.perf_counter(); fn(); hip.hipDeviceSynchronize()
+                best = min(best, time.perf_counter() - t0)
+            return nbytes / best / 1e9
+
+        rates["hipMemcpy_pageable_to_device"] = gbps(lambda: hip.hipMemcpy(dtmp.ptr, A.ctypes.data, nbytes, ea.H2D))
+        rates["hipMemcpy_device_to_pageable"] = gbps(lambda: hip.hipMemcpy(Ch.ctypes.data, dtmp.ptr, nbytes, ea.D2H))
+        pinned = C.c_void_p()
+        hip.hipHostMalloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t, C.c_uint]
+        hip.hipHostFree.argtypes = [C.c_void_p]
+        if hip.hipHostMalloc(C.byref(pinned), nbytes, 0) == 0:
+            rates["hipMemcpy_pinned_to_device"] = gbps(lambda: hip.hipMemcpy(dtmp.ptr, pinned, nbytes, ea.H2D))
+            rates["hipMemcpy_device_to_pinned"] = gbps(lambda: hip.hipMemcpy(pinned, dtmp.ptr, nbytes, ea.D2H))
+            hip.hipHostFree(pinned)
+        dtmp.free()
+        wb = ea.EshkolGPUBuffer()
+
+        def staged_up():
+            assert lib.eshkol_gpu_wrap_host(Ch.ctypes.data, nbytes, C.byref(wb)) == 0
+            lib.eshkol_gpu_wait(None)
+        rates["library_wrap_pageable_to_device"] = gbps(staged_up, reps=1)
+        rates["library_sync_device_to_pageable"] = gbps(lambda: lib.eshkol_gpu_sync(C.byref(wb), ea.SYNC_DEVICE_TO_HOST))
+        wb.flags &= ~2                              # nothing to copy back on free
+        lib.eshkol_gpu_free(C.byref(wb))
+        tiers["host_copy_rates_GB_per_s_512MiB"] = rates
+        log("copy rates GB/s: " + json.dumps({k: round(v, 1) for k, v in rates.items()}))
         del Ch
 
     # ---- CPU baseline on one host core ---------------------------------------------------------
