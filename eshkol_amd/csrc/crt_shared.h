@@ -72,6 +72,13 @@ constexpr int32_t CRT_FL_ZERO = INT32_MIN;      /* exponent entry of a maximum o
  * what depends on fl_a / fl_b right away and asks for the summary afterwards. */
 uint32_t eshkol_crt_scan_launch(const double* amax, uint64_t M, const double* bmax, uint64_t N,
                                 int32_t* fl_a, int32_t* fl_b, hipStream_t st);
+/* The two CRT tiers print one marker line per call, as the reference does per
+ * dispatch (gpu_memory.mm:2503; its gates count those lines). A dispatcher that
+ * runs one product as several calls (row panels) lets the first call print and
+ * silences the rest with this switch. */
+void eshkol_crt_set_quiet(int quiet);
+int eshkol_crt_quiet(void);
+
 /* Waits for that summary and fills out[0] (A) and out[1] (B). 0 on success. */
 int eshkol_crt_scan_result(uint32_t ticket, CrtMaxima out[2], hipStream_t st);
 

@@ -18,6 +18,7 @@
  */
 #include "hip_common.h"
 #include "host_copy.h"
+#include "crt_shared.h"
 #include "kernels.h"
 #include "tiers.h"
 #include "eshkol/backend/gpu/gpu_memory.h"
@@ -582,6 +583,7 @@ bool panelled_matmul(const double* A, const double* B, double* C,
                  ESHKOL_HIP_OK(hipEventRecord(g_ev_up, g_copy_stream)) &&
                  ESHKOL_HIP_OK(hipStreamWaitEvent(g_stream, g_ev_up, 0));
             if (!ok) break;
+            if (p == 1) eshkol_crt_set_quiet(1);       /* one marker line per product, not per panel */
             const int rc = reduced
                 ? hip_matmul_reduced_f64(dA + r0 * K, dB, dC + r0 * N, mp, K, N, reduced, 1, g_stream)
                 : run_tiers(choice, dA + r0 * K, dB, dC + r0 * N, mp, K, N, 0, 0, false);
@@ -598,6 +600,7 @@ bool panelled_matmul(const double* A, const double* B, double* C,
                  eshkol_hip_download(C + q0 * N, dC + q0 * N, (M - q0) * N * sizeof(double), g_copy_stream) == 0;
         }
     }
+    eshkol_crt_set_quiet(0);
     /* both queues drained before the buffers go back, and device errors seen */
     const bool drained = ESHKOL_HIP_OK(hipStreamSynchronize(g_copy_stream)) &&
                          ESHKOL_HIP_OK(hipStreamSynchronize(g_stream));

@@ -648,6 +648,10 @@ int crt_split_any(const double* X, uint64_t rows, uint64_t K, const int32_t* shi
 }
 }  // namespace
 
+static int g_crt_quiet = 0;
+void eshkol_crt_set_quiet(int quiet) { g_crt_quiet = quiet; }
+int eshkol_crt_quiet(void) { return g_crt_quiet; }
+
 uint32_t eshkol_crt_scan_launch(const double* amax, uint64_t M, const double* bmax, uint64_t N,
                                 int32_t* fl_a, int32_t* fl_b, hipStream_t st) {
     return scan_launch(amax, M, bmax, N, fl_a, fl_b, st);
@@ -797,7 +801,7 @@ extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, dou
         return 0;
     };
     auto announce = [&](int n_mod, const HostCrt& crt) {
-        fprintf(stderr, "[GPU] Ozaki-II: N=%d%s, log2(P)=%.1f\n", n_mod,
+        if (!eshkol_crt_quiet()) fprintf(stderr, "[GPU] Ozaki-II: N=%d%s, log2(P)=%.1f\n", n_mod,
                 adaptive ? " (adaptive)" : "", crt.log2P);       /* gpu_memory.mm:2503 */
     };
     auto in_range = [](int E, bool any, int e_min, int e_max) {

@@ -356,7 +356,7 @@ extern "C" int hip_matmul_ozaki_fast_f64_ex(const double* A, const double* B, do
     if (prc != 0) return prc;
     hipStream_t st = (hipStream_t)stream;
     if (ensure_tables(f, st) != 0) return -1;
-    fprintf(stderr, "[GPU] Ozaki-II FAST: n_mod=%d E=%d cap=%d log2(P)=%.1f (int8 MFMA GEMMs)\n",
+    if (!eshkol_crt_quiet()) fprintf(stderr, "[GPU] Ozaki-II FAST: n_mod=%d E=%d cap=%d log2(P)=%.1f (int8 MFMA GEMMs)\n",
             f.n, f.E, f.cap, f.log2P);                                  /* gpu_memory.mm:2859 */
 
     const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ldk = round_up_sz(K, 256);

@@ -424,6 +424,56 @@ assert np.isinf(out[3]).any() or np.isnan(out[3]).any()
     assert "FAST" not in r.stderr and "native fp64 MFMA" in r.stderr           # "0" leaves it off
 
 
+GATE = r"""
+import re
+TOL = float(os.environ["GATE_TOL"])
+assert lib.eshkol_gpu_init() == 1
+fails = 0
+for regime in range(4):
+    for n in (512, 1024, 2048, 4096):
+        i = np.arange(n * n, dtype=np.float64)
+        A = [(i % 7) - 3, 1.0 + 0.5 * (i % 7), np.pi * (1.0 + (i % 11)), 2.0 ** ((i % 20) - 10) * (1.0 + 0.1 * (i % 3))][regime].reshape(n, n)
+        B = [(i % 5) - 2, 0.5 + 0.25 * (i % 5), np.e * ((i % 9) - 4.0), 2.0 ** ((i % 18) - 9) * (1.0 + 0.1 * (i % 4))][regime].reshape(n, n)
+        Cd = ea.matmul_dispatch(A, B)
+        worst = 0.0
+        for pr in range(5):
+            for pc in range(5):
+                ii, jj = (pr * (n - 1)) // 4, (pc * (n - 1)) // 4
+                ref = 0.0
+                for a, b in zip(A[ii].tolist(), B[:, jj].tolist()):          # the probe's own k-ascending f64 sum
+                    ref += a * b
+                denom = abs(ref) if abs(ref) > 1e-9 else 1.0
+                worst = max(worst, abs(Cd[ii, jj] - ref) / denom)
+        print("REGIME=%d N=%d MAXREL=%g VERDICT=%s" % (regime, n, worst, "PASS" if worst < TOL else "FAIL"))
+        fails += worst >= TOL
+print("SUMMARY total_fail=%d" % fails)
+assert fails == 0
+"""
+
+
+@pytest.mark.parametrize("kernel,tol", [("ozaki", "1e-9"), ("ozaki-fast", "1e-7")], ids=["exact", "fast"])
+def test_reference_gates_for_the_ozaki_tiers_through_the_dispatcher(gpu, kernel, tol):
+    """tests/gpu/ozaki_correctness_test.esk + ozaki_correctness_gate.sh:79-136 and
+    tests/gpu/ozaki_fast_test.esk + ozaki_fast_gate.sh: four fill regimes at
+    N = 512 ... 4096, a 5 x 5 grid of probes against a plain f64 sum, the gates'
+    own tolerance and denominator; and what the gates read off stderr: one
+    dispatch marker per product and no other Ozaki-II line for the exact tier
+    (sixteen products, also at 4096 where the dispatcher works in row panels), the
+    FAST marker and no fall-back for the reduced-precision tier."""
+    r = run_child(GATE, {"ESHKOL_SF64_KERNEL": kernel, "ESHKOL_GPU_THRESHOLD": "1", "ESHKOL_GPU_VERBOSE": "1",
+                         "GATE_TOL": tol})
+    assert "SUMMARY total_fail=0" in r.stdout and "VERDICT=FAIL" not in r.stdout
+    lines = r.stderr.splitlines()
+    import re
+    if kernel == "ozaki":
+        pat = re.compile(r"^\[GPU\] Ozaki-II: N=[0-9]+( \(adaptive\))?, log2\(P\)=")
+        assert sum(1 for l in lines if pat.match(l)) == 16
+        assert not [l for l in lines if l.startswith("[GPU] Ozaki-II:") and not pat.match(l)]      # the gate's poison guard
+    else:
+        assert sum(1 for l in lines if l.startswith("[GPU] Ozaki-II FAST: n_mod=11")) == 16
+        assert "falling back to exact tier" not in r.stderr
+
+
 def test_tier_override_int8_and_budget_selector(gpu):
     body = r"""
 n = 1024
