@@ -162,6 +162,45 @@ def test_elementwise_family_and_transpose(gpu):
     assert lib.eshkol_gpu_softmax_f64(C.byref(da.buf), C.byref(do.buf), 10, 500) == -1
 
 
+def test_known_answers_of_the_reference_elementwise_and_transpose_tests(gpu):
+    """tests/gpu/elementwise_correctness_test.esk and transpose_correctness_test.esk,
+    through eshkol_gpu_elementwise_f64 / eshkol_gpu_transpose_f64."""
+    lib = ea.load()
+
+    def ew(op, a, b=None):
+        a = np.ascontiguousarray(a, dtype=np.float64)
+        da, do = ea.DeviceArray.from_host(a), ea.DeviceArray(a.shape)
+        db = ea.DeviceArray.from_host(np.ascontiguousarray(b, dtype=np.float64)) if b is not None else None
+        assert lib.eshkol_gpu_elementwise_f64(C.byref(da.buf), C.byref(db.buf) if db else None, C.byref(do.buf),
+                                              a.size, op) == 0
+        return do.download()
+
+    def tr(a):
+        a = np.ascontiguousarray(a, dtype=np.float64)
+        da, dt = ea.DeviceArray.from_host(a), ea.DeviceArray(a.shape[::-1])
+        assert lib.eshkol_gpu_transpose_f64(C.byref(da.buf), C.byref(dt.buf), a.shape[0], a.shape[1]) == 0
+        return dt.download()
+
+    A, B = np.array([[1., 2.], [3., 4.]]), np.array([[5., 6.], [7., 8.]])
+    assert np.array_equal(ew(0, A, B), [[6, 8], [10, 12]])
+    assert np.array_equal(ew(1, A, B), [[-4, -4], [-4, -4]])
+    assert np.array_equal(ew(2, A, B), [[5, 12], [21, 32]])
+    assert abs(ew(3, A, B)[0, 0] - 0.2) < 1e-10
+    Cm, D = np.arange(1., 10.).reshape(3, 3), np.arange(9., 0., -1.).reshape(3, 3)
+    cd = ew(0, Cm, D)
+    assert np.all(cd == 10.0)
+    assert np.array_equal(ew(2, cd, Cm), 10.0 * Cm)                       # chained
+    assert np.array_equal(ew(0, A, B), ew(0, B, A))                      # commutative
+    AB = np.array([[6., 8.], [10., 12.]])
+    assert np.array_equal(ew(0, ew(0, A, B), AB), ew(0, A, ew(0, B, AB)))   # associative on these values
+    A23 = np.array([[1., 2., 3.], [4., 5., 6.]])
+    assert np.array_equal(tr(A23), [[1, 4], [2, 5], [3, 6]]) and np.array_equal(tr(tr(A23)), A23)
+    assert np.array_equal(tr(A), [[1, 3], [2, 4]])
+    M2 = np.arange(5000.).reshape(50, 100)
+    M2T = tr(M2)
+    assert (M2T[0, 0], M2T[1, 0], M2T[0, 1]) == (0.0, 1.0, 100.0) and abs(M2T.sum() - M2.sum()) < 1e-6
+
+
 def test_dispatch_threshold_and_fallback_ladder(gpu):
     body = r"""
 A = synth.normal(1, (200, 150)); B = synth.normal(2, (150, 300))
