@@ -201,6 +201,51 @@ def test_known_answers_of_the_reference_elementwise_and_transpose_tests(gpu):
     assert (M2T[0, 0], M2T[1, 0], M2T[0, 1]) == (0.0, 1.0, 100.0) and abs(M2T.sum() - M2.sum()) < 1e-6
 
 
+def test_differential_gate_workload_gpu_against_the_compiled_reference_cpu(gpu):
+    """tests/gpu/gpu_correctness_gate.esk:22-76 with gpu_correctness_gate.sh:55,364-390:
+    the gate's sin/cos workload through the GPU entry points and through the CPU
+    matmul of the reference itself (compiled in place by the oracle's recipe), its
+    RESULT values compared at the gate's relative tolerance 1e-4 (they agree to
+    1e-13 and better)."""
+    if not os.path.exists(oracle.REF_PATH):
+        pytest.skip("the compiled reference is not in this tree")
+    lib = ea.load()
+    n = k = 512
+    i = np.arange(n * k, dtype=np.float64)
+    A = (1.0001 + np.sin(i * 0.001)).reshape(n, k)
+    B = (1.0002 + np.cos(i * 0.0013)).reshape(k, n)
+    old = lib.eshkol_gpu_get_threshold()
+    lib.eshkol_gpu_set_threshold(1)
+    try:
+        Cg = ea.matmul_dispatch(A, B)
+    finally:
+        lib.eshkol_gpu_set_threshold(old)
+    ref = C.CDLL(oracle.REF_PATH)
+    dp = C.POINTER(C.c_double)
+    ref.eshkol_matmul_f64.argtypes = [dp, dp, dp, C.c_uint64, C.c_uint64, C.c_uint64]
+    Cc = np.empty((n, n))
+    ref.eshkol_matmul_f64(A.ctypes.data_as(dp), B.ctypes.data_as(dp), Cc.ctypes.data_as(dp), n, k, n)
+    da, db, do = ea.DeviceArray.from_host(A.ravel()), ea.DeviceArray.from_host(B.ravel()), ea.DeviceArray((n * k,))
+    assert lib.eshkol_gpu_elementwise_f64(C.byref(da.buf), C.byref(db.buf), C.byref(do.buf), n * k, 0) == 0
+    add = do.download()
+    assert lib.eshkol_gpu_elementwise_f64(C.byref(da.buf), C.byref(db.buf), C.byref(do.buf), n * k, 2) == 0
+    mul = do.download()
+    dc, dt, dtt = ea.DeviceArray.from_host(Cg), ea.DeviceArray((n, n)), ea.DeviceArray((n, n))
+    assert lib.eshkol_gpu_transpose_f64(C.byref(dc.buf), C.byref(dt.buf), n, n) == 0
+    assert lib.eshkol_gpu_transpose_f64(C.byref(dt.buf), C.byref(dtt.buf), n, n) == 0
+    Ctt = dtt.download()
+    gpu_results = {"matmul-checksum": Cg.sum(), "matmul-c00": Cg[0, 0], "matmul-cmid": Cg[256, 256],
+                   "matmul-clast": Cg[511, 511], "add-checksum": add.sum(), "mul-checksum": mul.sum(),
+                   "transpose-roundtrip-c00": Ctt[0, 0], "transpose-roundtrip-clast": Ctt[511, 511]}
+    cpu_results = {"matmul-checksum": Cc.sum(), "matmul-c00": Cc[0, 0], "matmul-cmid": Cc[256, 256],
+                   "matmul-clast": Cc[511, 511], "add-checksum": (A + B).sum(), "mul-checksum": (A * B).sum(),
+                   "transpose-roundtrip-c00": Cc[0, 0], "transpose-roundtrip-clast": Cc[511, 511]}
+    for name, g in gpu_results.items():
+        c = cpu_results[name]
+        assert abs(g - c) / max(abs(c), 1e-300) <= 1e-4, name          # the gate's bar
+        assert abs(g - c) / abs(c) <= 1e-13, name                      # what the two actually differ by
+
+
 def test_dispatch_threshold_and_fallback_ladder(gpu):
     body = r"""
 A = synth.normal(1, (200, 150)); B = synth.normal(2, (150, 300))
