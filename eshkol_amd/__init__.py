@@ -123,6 +123,8 @@ SIGNATURES = {
     "hip_matmul_ozaki_fast_f64_ex": (C.c_int, [vp, vp, vp, u64, u64, u64, C.c_int, C.c_int, C.c_int, vp]),
     "hip_ozaki_fast_last_stages": (C.c_int, [C.POINTER(HipOzakiFastStages)]),
     "hip_ozaki_crt_set_aligned_weights": (C.c_int, [C.c_int]),
+    "hip_select_tier_for_budget": (C.c_int, [u64, u64, u64, C.c_double, C.POINTER(C.c_int32), C.POINTER(C.c_int32),
+                                             C.POINTER(C.c_double)]),
     "hip_ozaki_fast_plan": (C.c_int, [u64, C.c_int, C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
     "hip_ozaki_slice_f64": (C.c_int, [vp, u64, u64, vp, C.c_int, vp, u64, u64, vp]),
     "hip_ozaki_reconstruct_f64": (C.c_int, [vp, vp, vp, C.c_int, vp, vp, u64, u64, vp]),

@@ -867,6 +867,20 @@ int hip_matmul_backward_f64(const double* grad_out, const double* A, const doubl
     return 0;
 }
 
+/* The accuracy-budget decision for a shape, without running anything (host
+ * arithmetic only): tier 0 native fp64, 1 INT8 slices with *T, 2 Ozaki-II exact
+ * with aligned weights, 3 Ozaki-II reduced precision with *fast_moduli moduli;
+ * *speedup is the predicted ratio to native. budget <= 0 means the strictest. */
+int hip_select_tier_for_budget(uint64_t M, uint64_t K, uint64_t N, double budget,
+                               int32_t* T, int32_t* fast_moduli, double* speedup) {
+    if (!(budget > 0.0)) budget = 1e-15;
+    const Selection sel = select_tier(M, K, N, budget);
+    if (T) *T = sel.T;
+    if (fast_moduli) *fast_moduli = sel.fast_moduli;
+    if (speedup) *speedup = sel.speedup;
+    return sel.tier;
+}
+
 /* reference gpu_memory_cuda.cpp:1055-1083: single-precision operands. */
 int eshkol_gpu_matmul_f32(EshkolGPUBuffer* A, EshkolGPUBuffer* B, EshkolGPUBuffer* C,
                           uint64_t M, uint64_t K, uint64_t N) {

@@ -211,6 +211,15 @@ typedef struct {
 } HipOzakiFastStages;
 int hip_ozaki_fast_last_stages(HipOzakiFastStages* out);
 
+/* What ESHKOL_MATMUL_ACCURACY=<budget> would choose for a product of this shape
+ * (the selector of gpu_memory_cuda.cpp:546-566 with the two Ozaki-II tiers as
+ * further candidates), without running anything; host arithmetic only. Returns
+ * 0 native fp64, 1 INT8 slices (*T), 2 Ozaki-II exact tier with aligned
+ * weights, 3 Ozaki-II reduced-precision tier (*fast_moduli); *speedup is the
+ * cost model's predicted ratio to native. Pointers may be NULL. */
+int hip_select_tier_for_budget(uint64_t M, uint64_t K, uint64_t N, double budget,
+                               int32_t* T, int32_t* fast_moduli, double* speedup);
+
 /* What that tier would use for a contraction length K and a requested moduli
  * count (gpu_memory.mm:2802-2857), without running anything: returns the number
  * of moduli (it can be below the request when too few prime powers fit under

@@ -232,3 +232,37 @@ def test_bench_refuses_more_than_one_gpu_and_fails_loudly_without_a_device():
                            capture_output=True, text=True, timeout=300)
         assert r.returncode != 0 and "no gfx950 device" in r.stderr     # no CPU path stands in for the GPU
         assert not r.stdout.strip()                                     # and no result line is printed
+
+
+def test_accuracy_budget_selector_decisions():
+    """The selector is host arithmetic over a cost model seeded with measured times:
+    what it picks per budget at the headline size, that small products stay native,
+    that a tighter budget never gets a cheaper kernel, and that the slice tier's T
+    follows the reference's tolerance table (gpu_memory_cuda.cpp:477-489)."""
+    import ctypes as C
+    lib = ea.load()
+
+    def pick(M, K, N, budget):
+        T, n, sp = C.c_int32(), C.c_int32(), C.c_double()
+        tier = lib.hip_select_tier_for_budget(M, K, N, budget, C.byref(T), C.byref(n), C.byref(sp))
+        return tier, T.value, n.value, sp.value
+
+    n = 8192
+    assert pick(n, n, n, 1e-2)[:2] == (1, 1) and pick(n, n, n, 1e-5)[:2] == (1, 2) and pick(n, n, n, 1e-7)[:2] == (1, 3)
+    assert pick(n, n, n, 1e-9)[:2] == (1, 4)
+    for budget in (1e-10, 1e-11, 1e-13, 1e-14, 1e-15, 0.0):
+        tier, _, _, sp = pick(n, n, n, budget)
+        assert tier == 2 and 1.5 < sp < 2.0, budget                # the exact tier, where the reference has DGEMM only
+    last = 1e9
+    for budget in (1e-2, 1e-3, 1e-5, 1e-7, 1e-9, 1e-11, 1e-13, 1e-15):
+        sp = pick(n, n, n, budget)[3]
+        assert sp <= last * 1.0001, budget                          # tighter budgets are never predicted cheaper
+        last = sp
+    for budget in (1e-2, 1e-9, 1e-15):
+        assert pick(256, 256, 256, budget)[0] == 0 and pick(1024, 1024, 1024, budget)[0] == 0
+    assert pick(4096, 4096, 4096, 1e-15)[0] == 2 and pick(4096, 4096, 4096, 1e-2)[:2] == (1, 1)
+    for budget, lo, hi in ((1e-8, 11, 13), (1e-9, 12, 14), (1e-11, 14, 16)):
+        tier, _, moduli, sp = pick(4096, 4096, 4096, budget)       # shorter K, larger moduli: the reduced-precision
+        assert tier == 3 and lo <= moduli <= hi and sp > 1.3       # CRT tier with just enough of them
+    assert pick(4096, 200000, 4096, 1e-15)[0] == 0                  # beyond the int32-exact contraction length
+    assert pick(8192, 8192, 300, 1e-15)[0] in (0, 1)                # the CRT tiers need 512 in every dimension
