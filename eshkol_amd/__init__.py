@@ -131,6 +131,8 @@ SIGNATURES = {
     "hip_matmul_ozaki_int8_f64": (C.c_int, [vp, vp, vp, u64, u64, u64, C.c_int, vp]),
     "hip_ozaki_int8_last_stages": (C.c_int, [C.POINTER(HipOzakiInt8Stages)]),
     "hip_matmul_reduced_f64": (C.c_int, [vp, vp, vp, u64, u64, u64, C.c_int, C.c_int, vp]),
+    "hip_matmul_reduced_f64_noalloc": (C.c_int, [vp, vp, vp, u64, u64, u64, C.c_int, C.c_int, vp]),
+    "hip_matmul_reduced_f64_noalloc_limit": (C.c_size_t, []),
     "hip_matmul_ozaki_crt_f64_ex": (C.c_int, [vp, vp, vp, u64, u64, u64, C.c_int, C.c_int, C.c_int, C.c_int,
                                               vp, C.c_int, vp]),
     "hip_matmul_ozaki_int8_f64_ex": (C.c_int, [vp, vp, vp, u64, u64, u64, C.c_int, C.c_int, C.c_int, vp]),

@@ -685,6 +685,9 @@ int eshkol_gpu_init(void) {
                      ESHKOL_HIP_OK(hipEventCreateWithFlags(&g_ev_done[1], hipEventDisableTiming));
         if (!extra) { (void)hipGetLastError(); release_copy_queue(); }
     }
+    if (ok && eshkol_hip_noalloc_setup() != 0)
+        fprintf(stderr, "[GPU] the static scratch of hip_matmul_reduced_f64_noalloc is unavailable; "
+                        "that entry point will fail\n");
     if (ok) {
         g_backend = ESHKOL_GPU_HIP;
         g_initialized.store(true, std::memory_order_release);

@@ -23,6 +23,7 @@
 #include "kmajor_tile.h"
 
 #include <cstring>
+#include <mutex>
 
 typedef int v4i_t __attribute__((ext_vector_type(4)));
 typedef float v4f_t __attribute__((ext_vector_type(4)));
@@ -472,6 +473,20 @@ extern "C" int hip_hgemm_16(const uint16_t* A, const uint16_t* Bt, uint64_t M, u
     return hgemm_any(A, Bt, M, K, N, ld, is_bf16, 0, C, (hipStream_t)stream);
 }
 
+namespace {
+/* Narrow both operands into the 16-bit copies A16 [Mp][ld] and B16 [Np][ld] the
+ * caller provides (every element of both, padding included, is written), then
+ * multiply. One stored k-major (B as given, A when the caller holds A^T) is
+ * narrowed through LDS tiles, so no transposed fp64 copy is made. */
+int reduced_pipeline(const double* A, const double* B, double* C, uint64_t M, uint64_t K, uint64_t N,
+                     int trans_a, int trans_b, int is_bf16, int round_output,
+                     uint16_t* A16, uint16_t* B16, uint64_t Mp, uint64_t Np, uint64_t ld, hipStream_t st) {
+    if (convert_any(A, A16, M, K, Mp, ld, is_bf16, trans_a != 0, st) != 0) return -1;
+    if (convert_any(B, B16, N, K, Np, ld, is_bf16, trans_b == 0, st) != 0) return -1;
+    return hgemm_any(A16, B16, M, K, N, ld, is_bf16, round_output ? 2 : 1, C, st);
+}
+}  // namespace
+
 extern "C" int hip_matmul_reduced_f64_ex(const double* A, const double* B, double* C,
                                          uint64_t M, uint64_t K, uint64_t N,
                                          int trans_a, int trans_b,
@@ -480,17 +495,65 @@ extern "C" int hip_matmul_reduced_f64_ex(const double* A, const double* B, doubl
     if (dtype != 2 && dtype != 3) return -1;
     if (M > 0x7fffffffULL || K > 0x3fffffffULL || N > 0x7fffffffULL) return -1;
     hipStream_t st = (hipStream_t)stream;
-    const int is_bf16 = (dtype == 3);
     const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ld = round_up_sz(K, 128);
-    /* 16-bit copies [row][k] of both operands; one stored k-major (B as given, A
-     * when the caller holds A^T) is narrowed through LDS tiles, so no transposed
-     * fp64 copy is made. */
     uint16_t* A16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_A, Mp * ld * 2);
     uint16_t* B16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_B, Np * ld * 2);
     if (!A16 || !B16) return -1;
-    if (convert_any(A, A16, M, K, Mp, ld, is_bf16, trans_a != 0, st) != 0) return -1;
-    if (convert_any(B, B16, N, K, Np, ld, is_bf16, trans_b == 0, st) != 0) return -1;
-    return hgemm_any(A16, B16, M, K, N, ld, is_bf16, round_output ? 2 : 1, C, st);
+    return reduced_pipeline(A, B, C, M, K, N, trans_a, trans_b, dtype == 3, round_output, A16, B16, Mp, Np, ld, st);
+}
+
+/* ---- the reduced tier without any allocation ------------------------------------
+ * The 16-bit operand copies live in a device array that is part of the code
+ * object, so the call reaches neither hipMalloc nor the grow-only workspace.
+ * Host code never uses the array's name as an address: each device holds its
+ * own copy, whose address hipGetSymbolAddress returns once per device. */
+namespace {
+constexpr size_t NOALLOC_SCRATCH_BYTES = 32u << 20;
+constexpr int NOALLOC_MAX_DEVICES = 16;
+__device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+unsigned char* g_scratch_ptr[NOALLOC_MAX_DEVICES] = {};
+std::mutex g_scratch_mutex;
+
+/* The current device's copy of the array, or NULL. */
+unsigned char* noalloc_scratch(void) {
+    int dev = -1;
+    if (!ESHKOL_HIP_OK(hipGetDevice(&dev)) || dev < 0 || dev >= NOALLOC_MAX_DEVICES) return nullptr;
+    std::lock_guard<std::mutex> lk(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        if (!ESHKOL_HIP_OK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch))) || !ptr) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = (unsigned char*)ptr;
+    }
+    return g_scratch_ptr[dev];
+}
+}  // namespace
+
+int eshkol_hip_noalloc_setup(void) { return noalloc_scratch() ? 0 : -1; }
+
+extern "C" size_t hip_matmul_reduced_f64_noalloc_limit(void) { return NOALLOC_SCRATCH_BYTES; }
+
+extern "C" int hip_matmul_reduced_f64_noalloc(const double* A, const double* B, double* C,
+                                              uint64_t M, uint64_t K, uint64_t N,
+                                              int dtype, int round_output, void* stream) {
+    if (!A || !B || !C || M == 0 || K == 0 || N == 0) return -1;
+    if (dtype != 2 && dtype != 3) return -1;
+    if (M > 0x7fffffffULL || K > 0x3fffffffULL || N > 0x7fffffffULL) return -1;
+    const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ld = round_up_sz(K, 128);
+    const uint64_t a_bytes = Mp * ld * 2, b_bytes = Np * ld * 2;          /* multiples of 256 */
+    if (a_bytes + b_bytes > NOALLOC_SCRATCH_BYTES) {
+        fprintf(stderr, "[GPU] hip_matmul_reduced_f64_noalloc: %llux%llux%llu needs %llu bytes of 16-bit "
+                        "operand copies, the static scratch holds %llu; use hip_matmul_reduced_f64\n",
+                (unsigned long long)M, (unsigned long long)K, (unsigned long long)N,
+                (unsigned long long)(a_bytes + b_bytes), (unsigned long long)NOALLOC_SCRATCH_BYTES);
+        return -3;
+    }
+    unsigned char* base = noalloc_scratch();
+    if (!base) return -1;
+    return reduced_pipeline(A, B, C, M, K, N, 0, 0, dtype == 3, round_output,
+                            (uint16_t*)base, (uint16_t*)(base + a_bytes), Mp, Np, ld, (hipStream_t)stream);
 }
 
 extern "C" int hip_matmul_reduced_f64(const double* A, const double* B, double* C,

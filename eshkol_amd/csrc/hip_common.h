@@ -42,6 +42,10 @@ enum {
 void* eshkol_hip_workspace(int slot, size_t bytes);
 void  eshkol_hip_workspace_release(void);
 
+/* Looks up, once per device, the current device's address of the static scratch
+ * array behind hip_matmul_reduced_f64_noalloc (hgemm_16.hip). 0 on success. */
+int eshkol_hip_noalloc_setup(void);
+
 /* compute units of the current device (256 if the query fails) */
 static inline int eshkol_hip_num_cus(void) {
     static int cached = 0;

@@ -269,6 +269,22 @@ int hip_matmul_reduced_f64(const double* A, const double* B, double* C,
                            uint64_t M, uint64_t K, uint64_t N,
                            int dtype, int round_output, void* stream);
 
+/* The same product as hip_matmul_reduced_f64, for callers that cannot allocate
+ * device memory: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc. It has no counterpart in the reference. The 16-bit
+ * operand copies live in a device array that is part of the library's code
+ * object (hip_matmul_reduced_f64_noalloc_limit() bytes per GPU, held until the
+ * process ends) instead of the grow-only workspace, and the call reaches no
+ * hipMalloc, hipFree or allocating library routine. Returns -3 with a message
+ * on stderr when 2 * (roundup(M,256) + roundup(N,256)) * roundup(K,128) bytes
+ * exceed that limit, otherwise what hip_matmul_reduced_f64 returns, and the
+ * same bits in C. Every call on a GPU shares that GPU's array: calls that
+ * overlap on one GPU (two streams, two threads) race. */
+int hip_matmul_reduced_f64_noalloc(const double* A, const double* B, double* C,
+                                   uint64_t M, uint64_t K, uint64_t N,
+                                   int dtype, int round_output, void* stream);
+size_t hip_matmul_reduced_f64_noalloc_limit(void);
+
 /* 16-bit operands already in device memory (A [M][K], Bt [N][K], pitch ld
  * elements, multiple of 64, rows padded to multiples of 256 with zeros), fp32
  * result C[M][N]: the contraction alone (BASELINE configuration 4). */
