@@ -687,15 +687,18 @@ extern "C" void hip_dgemm_set_tail_split(int on) { g_tail_split = on ? 1 : 0; }
 extern "C" int hip_dgemm_f64_ex(const double* A, const double* B, double* C,
                                 uint64_t M, uint64_t K, uint64_t N,
                                 int trans_a, int trans_b, void* stream) {
+    EshkolHipCall bracket(stream);
     return dgemm_any(A, B, C, M, K, N, trans_a, trans_b, 1, stream);
 }
 
 extern "C" int hip_dgemm_f64(const double* A, const double* B, double* C,
                              uint64_t M, uint64_t K, uint64_t N, void* stream) {
+    EshkolHipCall bracket(stream);
     return dgemm_any(A, B, C, M, K, N, 0, 0, 1, stream);
 }
 
 extern "C" int hip_dgemm_f64_batched(const double* A, const double* B, double* C,
                                      uint64_t batch, uint64_t M, uint64_t K, uint64_t N, void* stream) {
+    EshkolHipCall bracket(stream);
     return dgemm_any(A, B, C, M, K, N, 0, 0, batch, stream);
 }

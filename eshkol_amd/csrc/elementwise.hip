@@ -222,6 +222,7 @@ extern "C" int hip_rowabsmax_f64(const double* A, uint64_t M, uint64_t K, double
 
 extern "C" int hip_colabsmax_f64(const double* X, uint64_t K, uint64_t R, double zero_value,
                                  double* cmax, void* stream) {
+    EshkolHipCall bracket(stream);
     if (!X || !cmax || K == 0 || R == 0) return -1;
     const uint64_t gx = (R + 63) / 64;
     if (gx > 0x7fffffffULL) return -1;

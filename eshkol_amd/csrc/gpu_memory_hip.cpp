@@ -147,16 +147,27 @@ void parse_env(void) {
     if (const char* w = getenv("ESHKOL_OZAKI_CRT_WEIGHTS")) e.crt_aligned = strcmp(w, "aligned") == 0;
     if (const char* a = getenv("ESHKOL_MATMUL_ACCURACY")) {      /* gpu_memory_cuda.cpp:527-539 */
         if (*a) {
+            /* "exact", "full" and anything unparseable are the reference's strictest
+             * request, which it always answers with DGEMM (gpu_memory_cuda.cpp:
+             * 546-566, "never silently degrades"): budget 0 admits native fp64 only. */
             if (!strcmp(a, "fast")) e.budget = 1e-2;
-            else if (!strcmp(a, "exact") || !strcmp(a, "full")) e.budget = 1e-15;
-            else { e.budget = atof(a); if (!(e.budget > 0.0)) e.budget = 1e-15; }
+            else if (!strcmp(a, "exact") || !strcmp(a, "full")) e.budget = 0.0;
+            else { e.budget = atof(a); if (!(e.budget > 0.0)) e.budget = 0.0; }
         }
     }
-    if (const char* p = getenv("ESHKOL_GPU_PRECISION")) {        /* gpu_memory.mm:1346-1351 */
+    if (const char* p = getenv("ESHKOL_GPU_PRECISION")) {        /* gpu_memory.mm:174, 1346-1351 */
         if (!strcmp(p, "high")) e.precision = 1;
         else if (!strcmp(p, "fast")) e.precision = 2;
         else if (!strcmp(p, "ml")) e.precision = 3;
     }
+    /* The reference's "fast" tier multiplies in f32 (about 6e-8) and its "ml" tier
+     * in fp24 (about 1e-5). Neither format has a matrix-core path of its own here;
+     * the accuracy-budget selector reaches the same error levels on the int8
+     * matrix cores, faster than an f32 kernel would: the settings act as budgets
+     * of 1e-7 and 1e-5 unless ESHKOL_MATMUL_ACCURACY asks for something else.
+     * They never select a 16-bit product: that is the tensor dtype's business. */
+    if (e.budget < 0.0 && e.precision == 2) e.budget = 1e-7;
+    if (e.budget < 0.0 && e.precision == 3) e.budget = 1e-5;
     g_env = e;
 }
 const TierEnv& tier_env(void) { std::call_once(g_env_once, parse_env); return g_env; }
@@ -206,9 +217,19 @@ void calibrate(int idx, double work, double measured_ns) {
  * only alternative; here the two Ozaki-II tiers are candidates as well:
  *   slices      smallest T with OZAKI_TOL[T] <= budget (none below 1e-14)
  *   CRT fast    smallest moduli count whose E gives fast_tolerance(E) <= budget
- *   CRT exact   every budget: its result is within 2 ulp of the exact product,
- *               tighter than native fp64's own rounding over K terms
+ *   CRT exact   budgets >= CRT_EXACT_TOL (1e-15, normwise): every element of A
+ *               is truncated at 2^-52 of its row's largest magnitude and every
+ *               element of B at 2^-52 of its column's, the rest is exact, so
+ *               |C - AB|_ij <= K 2^-51 rmax_i cmax_j, hence at most K 2^-51 in
+ *               the norm the budget is stated in (||C - AB||_F / (||A||_F ||B||_F))
+ *               and about 1e-17 measured on random operands. It is a normwise
+ *               guarantee relative to the row and column maxima, not a
+ *               componentwise one: an entry far below its row's maximum loses
+ *               its low bits, where native fp64 would keep them. Budgets below
+ *               1e-15, and the names exact / full, therefore stay on native
+ *               fp64, as in the reference.
  * Both CRT tiers need M, K, N >= 512 and K <= 131071, as their dispatch does. */
+constexpr double CRT_EXACT_TOL = 1e-15;
 struct Selection { int tier = 0; int T = 0; int fast_moduli = 0; double speedup = 1.0; };
 Selection select_tier(uint64_t M, uint64_t K, uint64_t N, double budget) {
     const double work = 2.0 * (double)M * (double)K * (double)N;
@@ -236,7 +257,9 @@ Selection select_tier(uint64_t M, uint64_t K, uint64_t N, double budget) {
         /* the exact tier's guarantee and its cost model are those of sixteen moduli */
         const TierEnv& env = tier_env();
         const double t = predict_ns(MODEL_CRT, work);
-        if (env.num_moduli == 16 && !env.adaptive && t < t_best) { t_best = t; best = Selection(); best.tier = 2; }
+        if (env.num_moduli == 16 && !env.adaptive && budget >= CRT_EXACT_TOL && t < t_best) {
+            t_best = t; best = Selection(); best.tier = 2;
+        }
     }
     if (best.tier != 0) best.speedup = t_native / t_best;
     return best;
@@ -544,11 +567,11 @@ void release_copy_queue(void) {
 /* C = A*B on host memory in row panels of A and C: while the device multiplies
  * panel p, the host stages panel p+1 up and panel p-1 down on the copy queue,
  * so that of the three transfers only B's is not hidden behind another or
- * behind the products. Row panels leave every tier's result unchanged: the
- * Ozaki tiers scale A by rows and B by columns, and a native tile does not
- * depend on the other tiles of the launch (only the split of a last partial
- * round may differ, which reorders a sum). The tier is chosen for the whole
- * product. Returns false when the shape does not pay or anything failed; the
+ * behind the products. Row panels leave a tier's result unchanged: the Ozaki
+ * tiers scale A by rows and B by columns, and a native tile does not depend on
+ * the other tiles of the launch (only the split of a last partial round may
+ * differ, which reorders a sum); the one exception is refused below. The tier
+ * is chosen for the whole product. Returns false when the shape does not pay or anything failed; the
  * caller then takes the one-piece path, which redoes the product. */
 constexpr size_t PANEL_MIN_BYTES = 128u << 20;      /* A and C together */
 
@@ -561,6 +584,13 @@ bool panelled_matmul(const double* A, const double* B, double* C,
     const char *a0 = (const char*)A, *b0 = (const char*)B, *c0 = (const char*)C;
     if ((c0 < a0 + a_bytes && a0 < c0 + c_bytes) || (c0 < b0 + b_bytes && b0 < c0 + c_bytes)) return false;
     if (resident_find(A)) return false;
+    /* Row panels leave a tier's result unchanged only while nothing in it depends
+     * on all rows of A at once. The exact CRT tier's exponent E (and, in adaptive
+     * mode, its moduli count) comes from the largest fractional part of log2 over
+     * all row maxima unless sixteen moduli make it 52 whatever the data
+     * (gpu_memory.mm:2510-2512): with fewer moduli or the adaptive count the
+     * product is made in one piece. */
+    if (!reduced && (env.num_moduli != 16 || env.adaptive) && choose_tier(M, K, N).tier == 2) return false;
     uint64_t rows = (((M + 7) / 8) + 127) & ~(uint64_t)127;
     if (rows < 512) rows = 512;
     const uint64_t panels = (M + rows - 1) / rows;
@@ -623,11 +653,38 @@ int eshkol_hip_verbose(void) {
 
 hipStream_t eshkol_hip_stream(void) { return g_stream; }
 
+namespace {
+int g_call_depth = 0;                    /* guarded by g_gpu_mutex */
+hipEvent_t g_ev_last_call = nullptr;     /* end of the previous bracketed call's work */
+hipStream_t g_last_call_stream = nullptr;
+bool g_last_call_recorded = false;
+}
+
+void eshkol_hip_enter(hipStream_t stream) {
+    g_gpu_mutex.lock();
+    if (++g_call_depth != 1) return;
+    if (g_last_call_recorded && g_last_call_stream != stream)
+        (void)hipStreamWaitEvent(stream, g_ev_last_call, 0);
+}
+
+void eshkol_hip_leave(hipStream_t stream) {
+    if (--g_call_depth == 0) {
+        if (!g_ev_last_call && !ESHKOL_HIP_OK(hipEventCreateWithFlags(&g_ev_last_call, hipEventDisableTiming))) {
+            (void)hipGetLastError();
+            g_ev_last_call = nullptr;
+        }
+        g_last_call_recorded = g_ev_last_call && ESHKOL_HIP_OK(hipEventRecord(g_ev_last_call, stream));
+        g_last_call_stream = stream;
+    }
+    g_gpu_mutex.unlock();
+}
+
 void* eshkol_hip_workspace(int slot, size_t bytes) {
     if (slot < 0 || slot >= WS_COUNT) return nullptr;
     Slot& s = g_ws[slot];
     if (s.bytes >= bytes && s.ptr) return s.ptr;
-    if (s.ptr) { hipStreamSynchronize(g_stream); hipFree(s.ptr); s.ptr = nullptr; s.bytes = 0; }
+    /* a slot may still be in use by kernels a caller queued on a stream of its own */
+    if (s.ptr) { (void)hipDeviceSynchronize(); hipFree(s.ptr); s.ptr = nullptr; s.bytes = 0; }
     size_t want = round_up_sz(bytes ? bytes : 256, 256);
     if (!ESHKOL_HIP_OK(hipMalloc(&s.ptr, want))) { s.ptr = nullptr; return nullptr; }
     s.bytes = want;
@@ -712,6 +769,8 @@ void eshkol_gpu_shutdown(void) {
         if (g_copy_stream) hipStreamSynchronize(g_copy_stream);
         release_copy_queue();
         if (g_stream) { hipStreamDestroy(g_stream); g_stream = nullptr; }
+        if (g_ev_last_call) { hipEventDestroy(g_ev_last_call); g_ev_last_call = nullptr; }
+        g_last_call_recorded = false; g_last_call_stream = nullptr;
     }
     g_backend = ESHKOL_GPU_NONE;
     g_initialized.store(false, std::memory_order_release);
@@ -856,6 +915,7 @@ int hip_matmul_backward_f64(const double* grad_out, const double* A, const doubl
                             uint64_t M, uint64_t K, uint64_t N,
                             int tier, int T, void* stream) {
     if (!grad_out || !A || !B || (!grad_A && !grad_B)) return -1;
+    EshkolHipCall bracket(stream);
     auto one = [&](const double* X, const double* Y, double* Z, uint64_t m, uint64_t k, uint64_t n,
                    int ta, int tb) -> int {
         switch (tier) {
@@ -873,10 +933,11 @@ int hip_matmul_backward_f64(const double* grad_out, const double* A, const doubl
 /* The accuracy-budget decision for a shape, without running anything (host
  * arithmetic only): tier 0 native fp64, 1 INT8 slices with *T, 2 Ozaki-II exact
  * with aligned weights, 3 Ozaki-II reduced precision with *fast_moduli moduli;
- * *speedup is the predicted ratio to native. budget <= 0 means the strictest. */
+ * *speedup is the predicted ratio to native. budget <= 0 is the strictest request
+ * (the names exact / full): native fp64 only. */
 int hip_select_tier_for_budget(uint64_t M, uint64_t K, uint64_t N, double budget,
                                int32_t* T, int32_t* fast_moduli, double* speedup) {
-    if (!(budget > 0.0)) budget = 1e-15;
+    if (!(budget > 0.0)) budget = 0.0;
     const Selection sel = select_tier(M, K, N, budget);
     if (T) *T = sel.T;
     if (fast_moduli) *fast_moduli = sel.fast_moduli;
@@ -1017,11 +1078,8 @@ void eshkol_matmul_dispatch(const double* A, const double* B, double* C,
     if (g_backend == ESHKOL_GPU_NONE) eshkol_gpu_init();
 
     if (g_backend == ESHKOL_GPU_HIP && A && B && C && M && K && N) {
-        const TierEnv& env = tier_env();
         /* dtype 2/3 bypass the element threshold (gpu_memory_cuda.cpp:1125). */
-        int reduced = (dtype == 2) ? 2 : (dtype == 3) ? 3 : 0;
-        /* ESHKOL_GPU_PRECISION fast/ml ask for the reduced tier on f64 tensors. */
-        if (!reduced && env.precision >= 2 && eshkol_gpu_should_use(num_elements)) reduced = 3;
+        const int reduced = (dtype == 2) ? 2 : (dtype == 3) ? 3 : 0;
         if (reduced || eshkol_gpu_should_use(num_elements)) {
             std::lock_guard<std::recursive_mutex> g(g_gpu_mutex);
             if (panelled_matmul(A, B, C, M, K, N, reduced)) return;

@@ -470,6 +470,7 @@ extern "C" int hip_convert_f64_to_16_kmajor(const double* in, uint16_t* out, uin
 
 extern "C" int hip_hgemm_16(const uint16_t* A, const uint16_t* Bt, uint64_t M, uint64_t K, uint64_t N,
                             uint64_t ld, int is_bf16, float* C, void* stream) {
+    EshkolHipCall bracket(stream);
     return hgemm_any(A, Bt, M, K, N, ld, is_bf16, 0, C, (hipStream_t)stream);
 }
 
@@ -491,6 +492,7 @@ extern "C" int hip_matmul_reduced_f64_ex(const double* A, const double* B, doubl
                                          uint64_t M, uint64_t K, uint64_t N,
                                          int trans_a, int trans_b,
                                          int dtype, int round_output, void* stream) {
+    EshkolHipCall bracket(stream);
     if (!A || !B || !C || M == 0 || K == 0 || N == 0) return -1;
     if (dtype != 2 && dtype != 3) return -1;
     if (M > 0x7fffffffULL || K > 0x3fffffffULL || N > 0x7fffffffULL) return -1;

@@ -42,6 +42,22 @@ enum {
 void* eshkol_hip_workspace(int slot, size_t bytes);
 void  eshkol_hip_workspace_release(void);
 
+/* Brackets a public tier entry point (hip_matmul_*, hip_dgemm_*, hip_igemm_i8,
+ * hip_colabsmax_f64): takes the library's recursive mutex, the one the eshkol_*
+ * entry points hold, and orders `stream` behind the stream the previous bracketed
+ * call queued its work on. The tiers share the grow-only workspace, the scan
+ * mailbox and per-process tables; with the bracket, callers on several threads
+ * or streams are serialised on the host and their kernels on the device. */
+void eshkol_hip_enter(hipStream_t stream);
+void eshkol_hip_leave(hipStream_t stream);
+struct EshkolHipCall {
+    hipStream_t st;
+    explicit EshkolHipCall(void* stream) : st((hipStream_t)stream) { eshkol_hip_enter(st); }
+    ~EshkolHipCall() { eshkol_hip_leave(st); }
+    EshkolHipCall(const EshkolHipCall&) = delete;
+    EshkolHipCall& operator=(const EshkolHipCall&) = delete;
+};
+
 /* Looks up, once per device, the current device's address of the static scratch
  * array behind hip_matmul_reduced_f64_noalloc (hgemm_16.hip). 0 on success. */
 int eshkol_hip_noalloc_setup(void);

@@ -417,6 +417,7 @@ extern "C" void hip_igemm_set_prefetch(int pf) { if (pf >= 0 && pf <= 3) g_prefe
 extern "C" void hip_igemm_set_persistent(int on) { g_persistent = on ? 1 : 0; }
 
 extern "C" int hip_igemm_i8(const HipIgemmArgs* args, void* stream) {
+    EshkolHipCall bracket(stream);
     if (!args || !args->a_planes || !args->b_planes || !args->pair_first || !args->pair_a || !args->pair_b)
         return -1;
     const HipIgemmArgs& a = *args;

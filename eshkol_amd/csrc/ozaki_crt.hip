@@ -731,6 +731,7 @@ extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, dou
                                            int trans_a, int trans_b,
                                            int num_moduli, int adaptive,
                                            const double* bias, int act, void* stream) {
+    EshkolHipCall bracket(stream);
     if (!A || !B || !C || M == 0 || K == 0 || N == 0) return -1;
     if (M > 0x7fffffffULL || N > 0x7fffffffULL) return -1;
     /* int32 accumulation of |a*b| <= 128*128 is exact while K*16384 < 2^31 */

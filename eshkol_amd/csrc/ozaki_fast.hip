@@ -348,6 +348,7 @@ extern "C" int hip_ozaki_fast_last_stages(HipOzakiFastStages* out) {
 extern "C" int hip_matmul_ozaki_fast_f64_ex(const double* A, const double* B, double* C,
                                             uint64_t M, uint64_t K, uint64_t N,
                                             int trans_a, int trans_b, int num_moduli, void* stream) {
+    EshkolHipCall bracket(stream);
     if (!A || !B || !C || M == 0 || K == 0 || N == 0) return -1;
     if (M > 0x7fffffffULL || N > 0x7fffffffULL) return -1;
     if (K > 131071) return -4;          /* the contraction's int32 bound; the reference's f32 bound is 2^24 / (p/2)^2 */

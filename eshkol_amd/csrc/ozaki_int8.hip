@@ -226,6 +226,7 @@ extern "C" int hip_ozaki_int8_last_stages(HipOzakiInt8Stages* out) {
 extern "C" int hip_matmul_ozaki_int8_f64_ex(const double* A, const double* B, double* C,
                                             uint64_t M, uint64_t K, uint64_t N,
                                             int trans_a, int trans_b, int T, void* stream) {
+    EshkolHipCall bracket(stream);
     if (!A || !B || !C || M == 0 || K == 0 || N == 0) return -1;
     if (M > 0x7fffffffULL || K > 0x7fffffffULL || N > 0x7fffffffULL) return -1;
     if (T < 1 || T > 8) return -1;

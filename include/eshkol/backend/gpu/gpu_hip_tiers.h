@@ -14,9 +14,21 @@
  * Conventions: plain C, device pointers, sizes as uint64_t in (M, K, N) order,
  * `stream` is a hipStream_t passed as void* (NULL = the null stream). Return 0
  * on success, -1 on a bad argument, an unsupported shape or a launch failure.
- * Launchers do not synchronise. Tier pipelines (hip_matmul_*) may synchronise
- * internally and use the library's cached device workspace, so calls into them
- * must not overlap; eshkol_gpu_init() must have succeeded first.
+ * Launchers do not synchronise. eshkol_gpu_init() must have succeeded first.
+ *
+ * Threads and streams. The tier pipelines (hip_matmul_*), hip_dgemm_f64*,
+ * hip_igemm_i8, hip_hgemm_16 and hip_colabsmax_f64 share the library's cached
+ * device workspace and per-process tables. Each of them takes the library's
+ * one recursive mutex (the same the eshkol_* entry points hold) for the length
+ * of the call and, when its stream differs from the stream of the previous such
+ * call, makes its stream wait for that call's work: they may be called from any
+ * thread, on any stream, beside eshkol_* calls, and are serialised on the host
+ * and on the device. The stage launchers (split, slice, convert, reconstruct,
+ * rowabsmax, transpose, elementwise, bias) touch only the memory they are
+ * given and take no lock. The hip_*_set_* switches are process-wide tuning
+ * hooks read by later calls: set them before other threads are inside the
+ * library, not beside them. hip_matmul_reduced_f64_noalloc takes no lock and
+ * orders nothing (see there).
  */
 #ifndef ESHKOL_GPU_HIP_TIERS_H
 #define ESHKOL_GPU_HIP_TIERS_H

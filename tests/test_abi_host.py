@@ -250,9 +250,14 @@ def test_accuracy_budget_selector_decisions():
     n = 8192
     assert pick(n, n, n, 1e-2)[:2] == (1, 1) and pick(n, n, n, 1e-5)[:2] == (1, 2) and pick(n, n, n, 1e-7)[:2] == (1, 3)
     assert pick(n, n, n, 1e-9)[:2] == (1, 4)
-    for budget in (1e-10, 1e-11, 1e-13, 1e-14, 1e-15, 0.0):
+    for budget in (1e-10, 1e-11, 1e-13, 1e-14, 1e-15):
         tier, _, _, sp = pick(n, n, n, budget)
-        assert tier == 2 and 1.5 < sp < 2.0, budget                # the exact tier, where the reference has DGEMM only
+        assert tier == 2 and 1.5 < sp < 2.5, budget                # the exact tier, where the reference has DGEMM only
+    # below the exact tier's stated normwise tolerance, and for the names exact / full (budget 0),
+    # native fp64 only: the reference never degrades its strictest request (gpu_memory_cuda.cpp:546-566)
+    for budget in (9e-16, 1e-16, 0.0, -1.0):
+        assert pick(n, n, n, budget)[0] == 0, budget
+        assert pick(4096, 4096, 4096, budget)[0] == 0, budget
     last = 1e9
     for budget in (1e-2, 1e-3, 1e-5, 1e-7, 1e-9, 1e-11, 1e-13, 1e-15):
         sp = pick(n, n, n, budget)[3]

@@ -587,8 +587,13 @@ assert err <= float(os.environ["EXPECT_ERR"]), err
     r = run_child(body2, {"ESHKOL_MATMUL_ACCURACY": "fast", "EXPECT_ERR": "1e-3", "ESHKOL_GPU_THRESHOLD": "1",
                           "ESHKOL_GPU_VERBOSE": "1"})
     assert "INT8-Ozaki T=1 (accuracy-budget selector" in r.stderr
-    # a strict budget at this size is met cheapest by the Ozaki-II exact tier (2 ulp per element) ...
-    r = run_child(body2, {"ESHKOL_MATMUL_ACCURACY": "exact", "EXPECT_ERR": "1e-15", "ESHKOL_GPU_THRESHOLD": "1",
+    # the names exact / full are the reference's strictest request: native fp64, never an Ozaki tier ...
+    for name in ("exact", "full"):
+        r = run_child(body2, {"ESHKOL_MATMUL_ACCURACY": name, "EXPECT_ERR": "1e-15", "ESHKOL_GPU_THRESHOLD": "1",
+                              "ESHKOL_GPU_VERBOSE": "1"})
+        assert "native fp64 MFMA (budget met cheapest by native fp64)" in r.stderr and "Ozaki" not in r.stderr
+    # ... a numeric budget down to 1e-15 (normwise) at this size is met cheapest by the Ozaki-II exact tier ...
+    r = run_child(body2, {"ESHKOL_MATMUL_ACCURACY": "1e-15", "EXPECT_ERR": "1e-15", "ESHKOL_GPU_THRESHOLD": "1",
                           "ESHKOL_GPU_VERBOSE": "1"})
     assert "Ozaki-II CRT exact (accuracy-budget selector), aligned weights" in r.stderr
     r = run_child(body2, {"ESHKOL_MATMUL_ACCURACY": "1e-13", "EXPECT_ERR": "1e-13", "ESHKOL_GPU_THRESHOLD": "1",
@@ -606,14 +611,65 @@ assert err <= float(os.environ["EXPECT_ERR"]), err
                           "ESHKOL_GPU_VERBOSE": "1"})
     assert "Ozaki-II FAST (" in r.stderr and "accuracy-budget selector)" in r.stderr
     # ... and with the exact tier cut down to fewer moduli (no longer exact) it is not a candidate
-    r = run_child(body2, {"ESHKOL_MATMUL_ACCURACY": "exact", "ESHKOL_OZAKI_NUM_MODULI": "12", "EXPECT_ERR": "1e-14",
+    r = run_child(body2, {"ESHKOL_MATMUL_ACCURACY": "1e-15", "ESHKOL_OZAKI_NUM_MODULI": "12", "EXPECT_ERR": "1e-14",
                           "ESHKOL_GPU_THRESHOLD": "1", "ESHKOL_GPU_VERBOSE": "1"})
     assert "native fp64 MFMA (budget met cheapest by native fp64)" in r.stderr
     # small products stay native whatever the budget
     body3 = body2.replace("n = 4096", "n = 1024").replace("range(0, n, 587)", "range(0, n, 97)")
-    r = run_child(body3, {"ESHKOL_MATMUL_ACCURACY": "exact", "EXPECT_ERR": "1e-14", "ESHKOL_GPU_THRESHOLD": "1",
+    r = run_child(body3, {"ESHKOL_MATMUL_ACCURACY": "1e-15", "EXPECT_ERR": "1e-14", "ESHKOL_GPU_THRESHOLD": "1",
                           "ESHKOL_GPU_VERBOSE": "1"})
     assert "native fp64 MFMA (budget met cheapest by native fp64)" in r.stderr
+
+
+def test_precision_settings_keep_the_error_level_of_the_reference_tiers(gpu):
+    """ESHKOL_GPU_PRECISION=fast is the reference's f32 tier (about 6e-8) and =ml its fp24
+    tier (about 1e-5), gpu_memory.mm:174, 1346-1351. Here they are accuracy budgets of 1e-7
+    and 1e-5 on f64 tensors: the error stays at that level (never the 4e-3 of a 16-bit
+    product), and an explicit ESHKOL_MATMUL_ACCURACY wins."""
+    body = r"""
+n = 4096
+A = synth.normal(1, (n, n)); B = synth.normal(2, (n, n))
+got = ea.matmul_dispatch(A, B)
+rows = list(range(0, n, 587))
+ref = A[rows].astype(np.longdouble) @ B.astype(np.longdouble)
+err = normwise(got[rows], ref, A[rows], B)
+print("ERR %.3e" % err)
+assert err <= float(os.environ["EXPECT_ERR"]), err
+"""
+    common = {"ESHKOL_GPU_THRESHOLD": "1", "ESHKOL_GPU_VERBOSE": "1"}
+    r = run_child(body, dict(common, ESHKOL_GPU_PRECISION="fast", EXPECT_ERR="1e-7"))
+    assert "accuracy-budget selector" in r.stderr and "reduced tier" not in r.stderr
+    r = run_child(body, dict(common, ESHKOL_GPU_PRECISION="ml", EXPECT_ERR="1e-5"))
+    assert "accuracy-budget selector" in r.stderr and "reduced tier" not in r.stderr
+    r = run_child(body, dict(common, ESHKOL_GPU_PRECISION="high", EXPECT_ERR="1e-15"))
+    assert "native fp64 MFMA (default)" in r.stderr
+    r = run_child(body, dict(common, ESHKOL_GPU_PRECISION="ml", ESHKOL_MATMUL_ACCURACY="1e-13", EXPECT_ERR="1e-13"))
+    assert "Ozaki-II CRT exact (accuracy-budget selector)" in r.stderr
+    # small products: native fp64 whatever the setting
+    small = body.replace("n = 4096", "n = 600").replace("range(0, n, 587)", "range(0, n, 97)")
+    r = run_child(small, dict(common, ESHKOL_GPU_PRECISION="fast", EXPECT_ERR="1e-15"))
+    assert "native fp64 MFMA" in r.stderr
+
+
+def test_cut_down_exact_tier_is_not_multiplied_in_row_panels(gpu):
+    """With fewer than sixteen moduli (or the adaptive count) the exact tier's exponent E
+    depends on all rows of A together, so the host-memory dispatcher must not cut A into row
+    panels: the result has to be the one-piece result, which is the oracle's bit for bit."""
+    body = r"""
+M, K, N = 8192 + 512, 1536, 512                          # A and C together above the panel threshold
+A = synth.wide_range(5, (M, K), -6, 6); B = synth.wide_range(6, (K, N), -6, 6)
+got = ea.matmul_dispatch(A, B)
+rows = [0, 1, 777, 4095, 4096, 8191, 8192, M - 1]
+want = oracle.matmul_ozaki_crt(A, B, num_moduli=12)
+assert np.array_equal(got, want), int((got != want).sum())
+"""
+    r = run_child(body, {"ESHKOL_HIP_F64_KERNEL": "ozaki-crt", "ESHKOL_OZAKI_NUM_MODULI": "12",
+                         "ESHKOL_GPU_THRESHOLD": "1", "ESHKOL_GPU_VERBOSE": "1"})
+    assert "row panels" not in r.stderr and "Ozaki-II CRT exact" in r.stderr
+    # sixteen moduli: E is 52 whatever the data, panels are used and the bits are still the oracle's
+    body16 = body.replace("num_moduli=12", "num_moduli=16")
+    r = run_child(body16, {"ESHKOL_HIP_F64_KERNEL": "ozaki-crt", "ESHKOL_GPU_THRESHOLD": "1", "ESHKOL_GPU_VERBOSE": "1"})
+    assert "row panels" in r.stderr
 
 
 def test_device_tanh_accuracy(gpu):

@@ -325,3 +325,42 @@ def test_mlp_layer():
     Y = oracle.mlp_layer(X, W, b)
     expect = np.tanh(oracle.matmul_ozaki_crt(X, W) + b[None, :])
     assert np.abs(Y - expect).max() <= 4 * np.finfo(np.float64).eps
+
+
+def test_crt_exact_tier_guarantee_is_normwise_not_componentwise():
+    """What the accuracy-budget selector may promise for the exact tier. Every element of A
+    is truncated at 2^-52 of its row's largest magnitude, every element of B at 2^-52 of its
+    column's, and the rest is exact: |C - AB|_ij <= K 2^-51 rmax_i cmax_j (plus the final
+    rounding), which bounds the error in the norm the budget is stated in but not per
+    element. Rows whose entries span 2^60 show it: the product of the small entries of row 0
+    with the small entries of a column is lost entirely, where native fp64 keeps it."""
+    K = 512
+    A = synth.uniform(91, (4, K), 0.5, 1.0)
+    B = synth.uniform(92, (K, 3), 0.5, 1.0)
+    A[0, 1:] *= 2.0 ** -60                      # row 0: one entry of size 1, the rest 2^-60 of it
+    B[1:, 0] *= 2.0 ** -60                      # column 0 likewise
+    A[0, 0] = 0.0                               # ... and the two large entries never meet
+    A[0, 5] = 0.75
+    B[0, 0] = 0.625
+    exact = [[sum(Fraction(float(A[i, k])) * Fraction(float(B[k, j])) for k in range(K)) for j in range(3)]
+             for i in range(4)]
+    rmax, cmax = np.abs(A).max(axis=1), np.abs(B).max(axis=0)
+    for aligned in (True, False):
+        C = oracle.matmul_ozaki_crt(A, B, aligned=aligned)
+        for i in range(4):
+            for j in range(3):
+                err = abs(Fraction(float(C[i, j])) - exact[i][j])
+                bound = Fraction(K) * Fraction(1, 2 ** 51) * Fraction(float(rmax[i])) * Fraction(float(cmax[j]))
+                if aligned:
+                    assert err <= bound + abs(exact[i][j]) * Fraction(1, 2 ** 52), (i, j, float(err), float(bound))
+    Ca = oracle.matmul_ozaki_crt(A, B, aligned=True)
+    # C[0,0] is a sum of products of order 2^-60: all of them are below the truncation, which
+    # cuts at 2^-52 of the row's maximum 0.75 (and of the column's 0.625)
+    assert exact[0][0] > 0 and float(exact[0][0]) < 2.0 ** -55
+    assert abs(Fraction(float(Ca[0, 0])) - exact[0][0]) > exact[0][0] / 4          # componentwise: lost
+    native = float(np.dot(A[0], B[:, 0]))
+    assert abs(Fraction(native) - exact[0][0]) <= exact[0][0] * Fraction(K, 2 ** 52)   # native fp64 keeps it
+    # ... while in the norm of the budget the tier is far inside 1e-15
+    num = sum((Fraction(float(Ca[i, j])) - exact[i][j]) ** 2 for i in range(4) for j in range(3))
+    den = sum(Fraction(float(x)) ** 2 for x in A.ravel()) * sum(Fraction(float(x)) ** 2 for x in B.ravel())
+    assert float(num) ** 0.5 / float(den) ** 0.5 < 1e-15
