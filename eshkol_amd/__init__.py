@@ -36,25 +36,27 @@ class HipIgemmArgs(C.Structure):
     _fields_ = [("a_planes", vp), ("b_planes", vp), ("a_plane_stride", u64), ("b_plane_stride", u64),
                 ("ldk", u32), ("M", u32), ("N", u32), ("n_out", u32),
                 ("pair_first", vp), ("pair_a", vp), ("pair_b", vp),
-                ("mode", i32), ("max_pairs", i32), ("modulus", vp), ("out_i32", vp), ("out_i8", vp)]
+                ("mode", i32), ("max_pairs", i32), ("modulus", vp), ("out_i32", vp), ("out_i8", vp),
+                ("layout", i32)]
 
 
 class HipOzakiCrtStages(C.Structure):
     _fields_ = [("a_planes", vp), ("b_planes", vp), ("w_planes", vp), ("mu", vp), ("nu", vp),
                 ("rows_a_padded", u64), ("rows_b_padded", u64), ("ldk", u64),
-                ("num_moduli", i32), ("E", i32)]
+                ("num_moduli", i32), ("E", i32), ("layout", i32)]
 
 
 class HipOzakiFastStages(C.Structure):
     _fields_ = [("a_planes", vp), ("b_planes", vp), ("w_planes", vp), ("shift_a", vp), ("shift_b", vp),
                 ("rows_a_padded", u64), ("rows_b_padded", u64), ("ldk", u64),
-                ("num_moduli", i32), ("E", i32), ("cap", i32), ("moduli", i32 * 16)]
+                ("num_moduli", i32), ("E", i32), ("cap", i32), ("moduli", i32 * 16),
+                ("layout", i32)]
 
 
 class HipOzakiInt8Stages(C.Structure):
     _fields_ = [("a_slices", vp), ("b_slices", vp), ("products", vp), ("rmax", vp), ("cmax", vp),
                 ("rows_a_padded", u64), ("rows_b_padded", u64), ("ldk", u64),
-                ("s", i32), ("nbuf", i32)]
+                ("s", i32), ("nbuf", i32), ("layout", i32)]
 
 
 BUF = C.POINTER(EshkolGPUBuffer)
@@ -142,6 +144,10 @@ SIGNATURES = {
     "hip_convert_f64_to_16": (C.c_int, [vp, vp, u64, u64, u64, u64, C.c_int, vp]),
     "hip_probe_peak": (C.c_int, [C.c_int, C.c_int, dp, vp]),
     "hip_igemm_set_persistent": (None, [C.c_int]),
+    "hip_igemm_set_direct": (None, [C.c_int]),
+    "hip_igemm_plane_layout": (C.c_int, [u64, u64, C.c_int]),
+    "hip_ozaki_crt_split_planes_f64": (C.c_int, [vp, u64, u64, vp, C.c_int, vp, u64, u64, C.c_int, C.c_int, vp]),
+    "hip_ozaki_slice_planes_f64": (C.c_int, [vp, u64, u64, vp, C.c_int, vp, u64, u64, C.c_int, C.c_int, vp]),
     "hip_dgemm_set_tail_split": (None, [C.c_int]),
     "hip_ozaki_crt_set_host_pass": (None, [C.c_int]),
     "hip_igemm_set_prefetch": (None, [C.c_int]),
@@ -257,6 +263,19 @@ def download_raw(ptr, shape, dtype):
     if rc != 0:
         raise RuntimeError("hipMemcpy D2H failed: %d" % rc)
     return out
+
+
+def deinterleave(planes, layout):
+    """Operand planes [n][rows][ldk] as the library stores them -> plain [n][rows][ldk].
+    layout 1 (HipIgemmArgs.layout): rows in blocks of 32, inside a block the 16-byte
+    k-chunks slow and the row fast."""
+    if not layout:
+        return planes
+    n, rows, ldk = planes.shape
+    item = planes.dtype.itemsize
+    per = 16 // item                                  # elements per 16-byte chunk
+    y = planes.reshape(n, rows // 32, ldk // per, 32, per).transpose(0, 1, 3, 2, 4)
+    return np.ascontiguousarray(y).reshape(n, rows, ldk)
 
 
 def synchronize():

@@ -32,6 +32,7 @@
 #include "hip_common.h"
 #include "kernels.h"
 #include "gemm_pipe.h"
+#include "gemm_pipe2.h"
 
 typedef int v4i_t __attribute__((ext_vector_type(4)));
 typedef int v16i_t __attribute__((ext_vector_type(16)));
@@ -248,6 +249,135 @@ void igemm_i8_persistent_kernel(HipIgemmArgs g, int tiles_m, int tiles_n, int ch
     pipe::run_tiles<I8Op, TM, TN, PF>(smem_i8, cm, next_tile, epi);
 }
 
+/* ---- interleaved planes: operands never pass through registers on their way
+ * to LDS (gemm_pipe2.h) ---------------------------------------------------------
+ * Four waves stacked along M, each with a 64 x 256 accumulator: acc[t][u] is
+ * the transposed 32 x 32 tile of rows m0 + 64 wave + 32 t + lane%32 and columns
+ * n0 + 32 u + 8 v + 4 (lane/32) + 0..3 in registers 4v .. 4v+3. The epilogue
+ * is private to a wave (no workgroup barrier): residues are packed four to a
+ * word, parked in the wave's own 32 x 128-byte LDS stage and leave as 16-byte
+ * stores, eight lanes to a 128-byte row segment. */
+__device__ __forceinline__ void epilogue_direct(const HipIgemmArgs& g, int o, int m0, int n0,
+                                                v16i_t (&acc)[pipe2::TM][pipe2::TN], int8_t* stage) {
+    constexpr int TM = pipe2::TM, TN = pipe2::TN;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int li = lane & 31, lh = lane >> 5;
+
+    if (g.mode == 0) {
+        int32_t* out = g.out_i32 + (size_t)o * g.M * g.N;
+        const bool vec_ok = (g.N % 4 == 0);
+#pragma unroll
+        for (int t = 0; t < TM; t++) {
+            const int row = m0 + wave * 64 + t * 32 + li;
+#pragma unroll
+            for (int u = 0; u < TN; u++) {
+                asm volatile("" : "+a"(acc[t][u]));      /* keep the tile in the accumulator file until here */
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const int col = n0 + u * 32 + 8 * v + 4 * lh;
+                    if (row < (int)g.M) {
+                        int32_t* p = out + (size_t)row * g.N + col;
+                        if (vec_ok && col + 3 < (int)g.N) {
+                            v4i_t w = {acc[t][u][4 * v], acc[t][u][4 * v + 1],
+                                       acc[t][u][4 * v + 2], acc[t][u][4 * v + 3]};
+                            *(v4i_t*)p = w;
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; e++)
+                                if (col + e < (int)g.N) p[e] = acc[t][u][4 * v + e];
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+        return;
+    }
+
+    /* mode 1: the exact reduction modulo p of epilogue() above */
+    const int p = pipe2::scalar_load(g.modulus + o);
+    const int c20 = (1 << 20) % p;
+    const float pinv = 1.0f / (float)p;
+    constexpr int EP = pipe2::EPI_PITCH;
+    int8_t* out = g.out_i8 + (size_t)o * g.M * g.N;
+    const bool vec_ok = (g.N % 16 == 0) && (((uintptr_t)out & 15) == 0);
+#pragma unroll
+    for (int t = 0; t < TM; t++) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {                     /* columns 128 h .. 128 h + 127 of the tile */
+#pragma unroll
+            for (int uu = 0; uu < 4; uu++) {
+                const int u = 4 * h + uu;
+                asm volatile("" : "+a"(acc[t][u]));
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    int r[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int s = acc[t][u][4 * v + e];
+                        const int x = __mul24(s >> 20, c20) + (s & 0xfffff);
+                        const float qm = fmaf((float)x, pinv, 12582912.0f);
+                        r[e] = __mul24(__float_as_int(qm), -p) + x;
+                    }
+                    const uint32_t lo2 = __builtin_amdgcn_perm((uint32_t)r[1], (uint32_t)r[0], 0x0c0c0400u);
+                    const uint32_t hi2 = __builtin_amdgcn_perm((uint32_t)r[3], (uint32_t)r[2], 0x04000c0cu);
+                    *(uint32_t*)(stage + li * EP + uu * 32 + 8 * v + 4 * lh) = lo2 | hi2;
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            /* the wave's LDS accesses complete in order: its reads see its writes */
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int c = lane + 64 * i;
+                const int lrow = c >> 3, ch = c & 7;
+                const int row = m0 + wave * 64 + t * 32 + lrow, col = n0 + 128 * h + 16 * ch;
+                const v4i_t val = *(const v4i_t*)(stage + lrow * EP + ch * 16);
+                if (row < (int)g.M && col < (int)g.N) {
+                    int8_t* dst = out + (size_t)row * g.N + col;
+                    if (vec_ok && col + 15 < (int)g.N) {
+                        *(v4i_t*)dst = val;
+                    } else {
+                        const int8_t* src = stage + lrow * EP + ch * 16;
+                        for (int e = 0; e < 16 && col + e < (int)g.N; e++) dst[e] = src[e];
+                    }
+                }
+            }
+        }
+    }
+}
+
+/* One workgroup per CU walks the tile ids blockIdx.x, blockIdx.x + gridDim.x, ...
+ * as the persistent kernel above does. */
+__global__ __launch_bounds__(256, 1)
+void igemm_i8_direct_kernel(HipIgemmArgs g, int tiles_m, int tiles_n, int chunk, int n_ids) {
+    extern __shared__ __align__(16) int8_t smem_i8[];
+    pipe::Source cm;
+    cm.a_planes = g.a_planes; cm.b_planes = g.b_planes;
+    cm.a_plane_stride = g.a_plane_stride; cm.b_plane_stride = g.b_plane_stride;
+    cm.ld = (int)g.ldk;
+
+    int next_id = (int)blockIdx.x;
+    auto next_tile = [&](pipe::Tile& t) -> bool {
+        while (next_id < n_ids) {
+            int o, tm, tn;
+            const bool real = map_workgroup(next_id, tiles_m, tiles_n, (int)g.n_out, chunk, &o, &tm, &tn);
+            next_id += (int)gridDim.x;
+            if (!real) continue;
+            const int pair_lo = pipe2::scalar_load(g.pair_first + o);
+            t.m0 = tm * pipe2::BM; t.n0 = tn * pipe2::BN; t.tag = o;
+            t.a_idx = g.pair_a + pair_lo; t.b_idx = g.pair_b + pair_lo;
+            t.npairs = pipe2::scalar_load(g.pair_first + o + 1) - pair_lo;
+            if (t.npairs > 0) return true;
+        }
+        return false;
+    };
+    auto epi = [&](v16i_t (&acc)[pipe2::TM][pipe2::TN], const pipe::Tile& t, int8_t* stage) {
+        epilogue_direct(g, t.tag, t.m0, t.n0, acc, stage);
+    };
+    pipe2::run_tiles<I8Op>(smem_i8, cm, next_tile, epi);
+}
+
 /* ---- simple kernel --------------------------------------------------------- */
 
 constexpr int SBK = 64;
@@ -341,6 +471,7 @@ void igemm_i8_simple_kernel(HipIgemmArgs g, int tiles_m, int tiles_n, int chunk)
     epilogue<TM, TN>(g, o, m0, n0, acc, smem_i8);
 }
 
+int g_direct = 1;       /* big launches take interleaved planes and the direct-to-LDS kernel */
 int g_prefetch = 2;     /* blocks in flight in the pipelined kernel */
 int g_persistent = 1;   /* pipelined kernel as one workgroup per CU walking a tile list */
 
@@ -400,6 +531,31 @@ int launch_persistent(const HipIgemmArgs& a, hipStream_t st) {
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 
+int launch_direct(const HipIgemmArgs& a, hipStream_t st) {
+    constexpr int SMEM = pipe2::SMEM_BYTES;
+    static bool attr_set = false;
+    static int num_cus = 0;
+    auto kern = igemm_i8_direct_kernel;
+    if (!attr_set) {
+        if (!ESHKOL_HIP_OK(hipFuncSetAttribute((const void*)kern,
+                hipFuncAttributeMaxDynamicSharedMemorySize, SMEM))) return -1;
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (!ESHKOL_HIP_OK(hipGetDevice(&dev)) || !ESHKOL_HIP_OK(hipGetDeviceProperties(&prop, dev))) return -1;
+        num_cus = prop.multiProcessorCount;
+        attr_set = true;
+    }
+    const int tiles_m = (int)((a.M + pipe2::BM - 1) / pipe2::BM), tiles_n = (int)((a.N + pipe2::BN - 1) / pipe2::BN);
+    const int chunk = (tiles_m * tiles_n + 7) / 8;
+    const long long n_ids = 8LL * chunk * a.n_out;
+    if (n_ids > 0x7fffffffLL || n_ids <= 0) return -1;
+    long long grid = (num_cus / 8) * 8;             /* one workgroup per CU, a multiple of the XCD count */
+    if (grid < 8) grid = 8;
+    if (grid > n_ids) grid = n_ids;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), SMEM, st, a, tiles_m, tiles_n, chunk, (int)n_ids);
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
 int launch_simple(const HipIgemmArgs& a, hipStream_t st) {
     constexpr int BM = 128, BN = 128;
     constexpr int MAIN = 2 * (BM + BN) * SPITCH, EPI = BM * (BN + 16);
@@ -416,6 +572,18 @@ extern "C" void hip_igemm_set_prefetch(int pf) { if (pf >= 0 && pf <= 3) g_prefe
  * walking a list of tiles, 0 as one workgroup per tile. Same results. */
 extern "C" void hip_igemm_set_persistent(int on) { g_persistent = on ? 1 : 0; }
 
+/* Tuning hook: 0 keeps every launch on row-major planes and the register-staged
+ * kernels. Same results. */
+extern "C" void hip_igemm_set_direct(int on) { g_direct = on ? 1 : 0; }
+
+/* The plane layout the tiers should produce for a contraction of n_out output
+ * planes of M x N: 1 (interleaved, for the direct-to-LDS kernel) when the launch
+ * has enough 256 x 256 tiles to be worth a workgroup per CU, else 0. */
+extern "C" int hip_igemm_plane_layout(uint64_t M, uint64_t N, int n_out) {
+    const uint64_t big = ((M + 255) / 256) * ((N + 255) / 256) * (uint64_t)(n_out > 0 ? n_out : 0);
+    return (g_direct && big >= 128) ? 1 : 0;
+}
+
 extern "C" int hip_igemm_i8(const HipIgemmArgs* args, void* stream) {
     EshkolHipCall bracket(stream);
     if (!args || !args->a_planes || !args->b_planes || !args->pair_first || !args->pair_a || !args->pair_b)
@@ -429,6 +597,14 @@ extern "C" int hip_igemm_i8(const HipIgemmArgs* args, void* stream) {
     else if (a.mode == 1) { if (!a.out_i8 || !a.modulus) return -1; }
     else return -1;
     hipStream_t st = (hipStream_t)stream;
+    if (a.layout == 1) {
+        /* interleaved planes: whole groups of four 128-byte k-blocks per product,
+         * every output plane with 1..64 products, row counts padded to 256 */
+        if (a.ldk % 512 != 0 || a.max_pairs < 1) return -1;
+        if ((a.a_plane_stride % (32ull * a.ldk)) || (a.b_plane_stride % (32ull * a.ldk))) return -1;
+        return launch_direct(a, st);
+    }
+    if (a.layout != 0) return -1;
     /* Operand planes are padded to multiples of 256 rows, so either tiling reads
      * in bounds. The pipelined kernel needs whole groups of prefetched blocks
      * per product and at most 64 products per output plane. */

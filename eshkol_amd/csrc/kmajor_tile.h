@@ -17,6 +17,15 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+/* Byte offset of element (row, k) inside one int8 / 16-bit operand plane with a
+ * row pitch of ld bytes (k counted in bytes). layout 0: [rows][ld]. layout 1,
+ * "interleaved": rows in blocks of 32, inside a block the 16-byte k-chunks slow
+ * and the row fast, so that the 32-row x 32-byte operand fragment of a 32x32
+ * matrix-core instruction is 1 KiB of contiguous memory (gemm_pipe2.h). */
+__device__ __forceinline__ uint64_t eshkol_plane_offset(int layout, uint64_t row, uint64_t k, uint64_t ld) {
+    return layout ? (row >> 5) * (32 * ld) + (k >> 4) * 512 + (row & 31) * 16 + (k & 15) : row * ld + k;
+}
+
 namespace kmaj {
 
 typedef double d2_t __attribute__((ext_vector_type(2)));

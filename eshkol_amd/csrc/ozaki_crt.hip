@@ -192,26 +192,83 @@ void crt_split_staged_kernel(const double* __restrict__ X, uint64_t rows, uint64
     }
 }
 
+/* Row-major X[rows][K], interleaved planes (rows_padded and ldk multiples of 32).
+ * A block takes 32 rows x 32 k, a thread four consecutive k of one row (eight
+ * lanes read 256 contiguous bytes of a row). What the block produces is, per
+ * plane, one operand fragment: 1 KiB of contiguous memory, written by one wave
+ * as 16-byte stores. */
+template <int NMOD>
+__global__ __launch_bounds__(256)
+void crt_split_il_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
+                         const int32_t* __restrict__ shift, int8_t* __restrict__ planes,
+                         uint64_t rows_padded, uint64_t ldk) {
+    __shared__ __align__(16) uint32_t stage[NMOD][256];
+    const uint32_t kt = (uint32_t)(ldk / 32);
+    const uint64_t rb = blockIdx.x / kt, kb = blockIdx.x % kt;
+    const int tid = threadIdx.x;
+    const uint64_t row = rb * 32 + (uint64_t)(tid >> 3), k = kb * 32 + 4 * (uint64_t)(tid & 7);
+    double x[4] = {0.0, 0.0, 0.0, 0.0};
+    int sh = 0;
+    if (row < rows && k < K) {
+        sh = shift[row];
+        const double* p = X + row * K + k;
+        if (k + 3 < K && (K & 1) == 0 && (((uintptr_t)X & 15) == 0)) {
+            const d2_t v0 = *(const d2_t*)p, v1 = *(const d2_t*)(p + 2);
+            x[0] = v0.x; x[1] = v0.y; x[2] = v1.x; x[3] = v1.y;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) if (k + e < K) x[e] = p[e];
+        }
+    }
+    Scaled t[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) t[e] = scaled_integer<false>(x[e], sh);
+#define ESHKOL_SPLIT_ONE(L)                                                           \
+    if (L < NMOD) {                                                                   \
+        const uint32_t w01 = __builtin_amdgcn_perm(residue_byte<L>(t[1]), residue_byte<L>(t[0]), 0x0c0c0400u); \
+        const uint32_t w23 = __builtin_amdgcn_perm(residue_byte<L>(t[3]), residue_byte<L>(t[2]), 0x0c0c0400u); \
+        stage[L][tid] = __builtin_amdgcn_perm(w23, w01, 0x05040100u);                 \
+    }
+    ESHKOL_SPLIT_ONE(0)  ESHKOL_SPLIT_ONE(1)  ESHKOL_SPLIT_ONE(2)  ESHKOL_SPLIT_ONE(3)
+    ESHKOL_SPLIT_ONE(4)  ESHKOL_SPLIT_ONE(5)  ESHKOL_SPLIT_ONE(6)  ESHKOL_SPLIT_ONE(7)
+    ESHKOL_SPLIT_ONE(8)  ESHKOL_SPLIT_ONE(9)  ESHKOL_SPLIT_ONE(10) ESHKOL_SPLIT_ONE(11)
+    ESHKOL_SPLIT_ONE(12) ESHKOL_SPLIT_ONE(13) ESHKOL_SPLIT_ONE(14) ESHKOL_SPLIT_ONE(15)
+#undef ESHKOL_SPLIT_ONE
+    __syncthreads();
+    /* stage[plane][8 r + j] holds k 4j .. 4j+3 of row r; fragment order is
+     * [k-chunk c][row r][16 bytes]: chunk c of row r is words 8 r + 4 c .. + 3 */
+    const uint64_t plane_stride = rows_padded * ldk;
+    int8_t* frag = planes + rb * (32 * ldk) + kb * 1024;
+#pragma unroll
+    for (int j = 0; j < NMOD * 64 / 256 + (NMOD * 64 % 256 != 0); j++) {
+        const int c = tid + 256 * j;
+        const int plane = c >> 6, q = c & 63;
+        if (plane < NMOD)
+            *(v4u_t*)(frag + (uint64_t)plane * plane_stride + 16 * q) =
+                *(const v4u_t*)&stage[plane][8 * (q & 31) + 4 * (q >> 5)];
+    }
+}
+
 /* k-major X[K][rows] (B as the runtime stores it), same output. */
 template <int NMOD>
 __global__ __launch_bounds__(256, 4)
 void crt_split_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
                              const int32_t* __restrict__ shift, int8_t* __restrict__ planes,
-                             uint64_t rows_padded, uint64_t ldk, uint32_t group) {
+                             uint64_t rows_padded, uint64_t ldk, uint32_t group, int layout) {
     __shared__ __align__(16) double tile[kmaj::SMEM_DOUBLES];
     const uint64_t plane_stride = rows_padded * ldk;
     if ((ldk & 15) == 0 && (((uintptr_t)planes & 15) == 0)) {
         kmaj::for_each_16(X, rows, K, rows_padded, ldk, group, tile,
             [&](uint64_t row) { return (row < rows) ? shift[row] : 0; },
             [&](uint64_t row, uint64_t k, const double* x, int sh) {
-                split_16<NMOD>(x, sh, planes + row * ldk + k, plane_stride);
+                split_16<NMOD>(x, sh, planes + eshkol_plane_offset(layout, row, k, ldk), plane_stride);
             });
         return;
     }
     kmaj::for_each_pair(X, rows, K, rows_padded, ldk, group, tile,
         [&](uint64_t row) { return (row < rows) ? shift[row] : 0; },
         [&](uint64_t row, uint64_t k, double x0, double x1, int sh) {
-            split_pair<NMOD>(x0, x1, sh, planes + row * ldk + k, plane_stride);
+            split_pair<NMOD>(x0, x1, sh, planes + eshkol_plane_offset(layout, row, k, ldk), plane_stride);
         });
 }
 
@@ -609,11 +666,17 @@ bool g_force_host_pass = false;
 
 template <int NMOD>
 void launch_split(const double* X, uint64_t rows, uint64_t K, const int32_t* shift, int8_t* planes,
-                  uint64_t rows_padded, uint64_t ldk, bool kmajor, hipStream_t st) {
+                  uint64_t rows_padded, uint64_t ldk, bool kmajor, int layout, hipStream_t st) {
     if (kmajor) {
         dim3 grid((unsigned)kmaj::grid_blocks(rows_padded, ldk, eshkol_hip_num_cus()));
         hipLaunchKernelGGL(crt_split_kmajor_kernel<NMOD>, grid, dim3(256), 0, st, X, rows, K, shift, planes,
-                           rows_padded, ldk, 0xffffffffu);
+                           rows_padded, ldk, 0xffffffffu, layout);
+        return;
+    }
+    if (layout == 1) {
+        dim3 grid((unsigned)((rows_padded / 32) * (ldk / 32)));
+        hipLaunchKernelGGL(crt_split_il_kernel<NMOD>, grid, dim3(256), 0, st, X, rows, K, shift, planes,
+                           rows_padded, ldk);
         return;
     }
     if (ldk % 16 == 0 && ((uintptr_t)planes & 15) == 0) {
@@ -631,15 +694,17 @@ void launch_split(const double* X, uint64_t rows, uint64_t K, const int32_t* shi
 
 namespace {
 int crt_split_any(const double* X, uint64_t rows, uint64_t K, const int32_t* shift, int num_moduli,
-                  int8_t* planes, uint64_t rows_padded, uint64_t ldk, bool kmajor, void* stream) {
+                  int8_t* planes, uint64_t rows_padded, uint64_t ldk, bool kmajor, int layout, void* stream) {
     if (!X || !shift || !planes || rows == 0 || K == 0) return -1;
     if (num_moduli < 2 || num_moduli > MAX_MODULI) return -1;
     if (rows_padded < rows || ldk < K || (ldk & 1)) return -1;
+    if (layout != 0 && layout != 1) return -1;
+    if (layout == 1 && ((rows_padded & 31) || (ldk & 31) || ((uintptr_t)planes & 15))) return -1;
     if (((ldk / 2 + 255) / 256) * rows_padded > 0x7fffffffULL) return -1;
     if (kmaj::tile_count(rows_padded, ldk) > 0x7fffffffULL) return -1;
     hipStream_t st = (hipStream_t)stream;
     switch (num_moduli) {
-#define CASE(n) case n: launch_split<n>(X, rows, K, shift, planes, rows_padded, ldk, kmajor, st); break;
+#define CASE(n) case n: launch_split<n>(X, rows, K, shift, planes, rows_padded, ldk, kmajor, layout, st); break;
         CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8) CASE(9)
         CASE(10) CASE(11) CASE(12) CASE(13) CASE(14) CASE(15) CASE(16)
 #undef CASE
@@ -674,13 +739,20 @@ void eshkol_crt_shifts_from_exponents(int32_t* fl_a, uint64_t M, int32_t* fl_b, 
 extern "C" int hip_ozaki_crt_split_f64(const double* X, uint64_t rows, uint64_t K,
                                        const int32_t* shift, int num_moduli,
                                        int8_t* planes, uint64_t rows_padded, uint64_t ldk, void* stream) {
-    return crt_split_any(X, rows, K, shift, num_moduli, planes, rows_padded, ldk, false, stream);
+    return crt_split_any(X, rows, K, shift, num_moduli, planes, rows_padded, ldk, false, 0, stream);
 }
 
 extern "C" int hip_ozaki_crt_split_kmajor_f64(const double* X, uint64_t rows, uint64_t K,
                                               const int32_t* shift, int num_moduli,
                                               int8_t* planes, uint64_t rows_padded, uint64_t ldk, void* stream) {
-    return crt_split_any(X, rows, K, shift, num_moduli, planes, rows_padded, ldk, true, stream);
+    return crt_split_any(X, rows, K, shift, num_moduli, planes, rows_padded, ldk, true, 0, stream);
+}
+
+extern "C" int hip_ozaki_crt_split_planes_f64(const double* X, uint64_t rows, uint64_t K,
+                                              const int32_t* shift, int num_moduli,
+                                              int8_t* planes, uint64_t rows_padded, uint64_t ldk,
+                                              int kmajor, int layout, void* stream) {
+    return crt_split_any(X, rows, K, shift, num_moduli, planes, rows_padded, ldk, kmajor != 0, layout, stream);
 }
 
 extern "C" int hip_ozaki_crt_reconstruct_f64(const int8_t* w_planes, uint64_t M, uint64_t N, int num_moduli,
@@ -753,7 +825,10 @@ extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, dou
     hipStream_t st = (hipStream_t)stream;
     if (ensure_tables(st) != 0) return -1;
 
-    const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ldk = round_up_sz(K, 256);
+    /* planes interleaved (and the k pitch padded to whole groups of four 128-byte
+     * blocks) when the contraction will take the kernel that wants them so */
+    const int layout = hip_igemm_plane_layout(M, N, num_moduli);
+    const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ldk = round_up_sz(K, layout ? 512 : 256);
     /* Both operands come out as planes [row][k]. An operand stored with k
      * contiguous (A as given, B when the caller holds B^T) is read row by row;
      * one stored k-major (B as given, A when the caller holds A^T) is read
@@ -783,8 +858,8 @@ extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, dou
         int8_t* Bp = (int8_t*)eshkol_hip_workspace(WS_BPLANES, (size_t)n_mod * Np * ldk);
         int8_t* Wp = (int8_t*)eshkol_hip_workspace(WS_PRODUCTS, (size_t)n_mod * M * N);
         if (!Ap || !Bp || !Wp) return -1;
-        if (crt_split_any(A, M, K, dmu, n_mod, Ap, Mp, ldk, a_kmajor, st) != 0) return -1;
-        if (crt_split_any(B, N, K, dnu, n_mod, Bp, Np, ldk, b_kmajor, st) != 0) return -1;
+        if (crt_split_any(A, M, K, dmu, n_mod, Ap, Mp, ldk, a_kmajor, layout, st) != 0) return -1;
+        if (crt_split_any(B, N, K, dnu, n_mod, Bp, Np, ldk, b_kmajor, layout, st) != 0) return -1;
         HipIgemmArgs ga;
         memset(&ga, 0, sizeof ga);
         ga.a_planes = Ap; ga.b_planes = Bp;
@@ -792,13 +867,14 @@ extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, dou
         ga.ldk = (uint32_t)ldk; ga.M = (uint32_t)M; ga.N = (uint32_t)N; ga.n_out = (uint32_t)n_mod;
         ga.pair_first = g_tables; ga.pair_a = g_tables + 17; ga.pair_b = g_tables + 17;
         ga.mode = 1; ga.max_pairs = 1; ga.modulus = g_tables + 33; ga.out_i8 = Wp;
+        ga.layout = layout;
         if (hip_igemm_i8(&ga, st) != 0) return -1;
         if (hip_ozaki_crt_reconstruct_f64(Wp, M, N, n_mod, crt.sl1, crt.sl2, crt.P1, crt.P2, crt.Pinv,
                                           dmu, dnu, bias, act, C, st) != 0) return -1;
         g_last.a_planes = Ap; g_last.b_planes = Bp; g_last.w_planes = Wp;
         g_last.mu = dmu; g_last.nu = dnu;
         g_last.rows_a_padded = Mp; g_last.rows_b_padded = Np; g_last.ldk = ldk;
-        g_last.num_moduli = n_mod; g_last.E = E;
+        g_last.num_moduli = n_mod; g_last.E = E; g_last.layout = layout;
         return 0;
     };
     auto announce = [&](int n_mod, const HostCrt& crt) {

@@ -109,11 +109,55 @@ void fast_split_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
     }
 }
 
+/* Row-major X[rows][K], interleaved planes (rows_padded and ldk multiples of 32):
+ * a block takes 32 rows x 32 k, a thread four consecutive k of one row, and each
+ * plane's share of the block is one operand fragment, 1 KiB of contiguous memory
+ * (the layout of the exact tier's interleaved split). */
+__global__ __launch_bounds__(256)
+void fast_split_il_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
+                          const int32_t* __restrict__ shift, FastTable tbl, int8_t* __restrict__ planes,
+                          uint64_t rows_padded, uint64_t ldk) {
+    __shared__ __align__(16) uint32_t stage[FAST_MAX_MODULI][256];
+    const uint32_t kt = (uint32_t)(ldk / 32);
+    const uint64_t rb = blockIdx.x / kt, kb = blockIdx.x % kt;
+    const int tid = threadIdx.x;
+    const uint64_t row = rb * 32 + (uint64_t)(tid >> 3), k = kb * 32 + 4 * (uint64_t)(tid & 7);
+    double x[4] = {0.0, 0.0, 0.0, 0.0};
+    int sh = 0;
+    if (row < rows && k < K) {
+        sh = shift[row];
+        const double* p = X + row * K + k;
+        if (k + 3 < K && (K & 1) == 0 && (((uintptr_t)X & 15) == 0)) {
+            const d2_t v0 = *(const d2_t*)p, v1 = *(const d2_t*)(p + 2);
+            x[0] = v0.x; x[1] = v0.y; x[2] = v1.x; x[3] = v1.y;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) if (k + e < K) x[e] = p[e];
+        }
+    }
+    Scaled s[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) s[e] = scaled_integer<true>(x[e], sh);
+#pragma unroll
+    for (int l = 0; l < FAST_MAX_MODULI; l++)
+        if (l < tbl.n)
+            stage[l][tid] = pack4(fast_residue(s[0], tbl, l), fast_residue(s[1], tbl, l),
+                                  fast_residue(s[2], tbl, l), fast_residue(s[3], tbl, l));
+    __syncthreads();
+    const uint64_t plane_stride = rows_padded * ldk;
+    int8_t* frag = planes + rb * (32 * ldk) + kb * 1024;
+    for (int c = tid; c < tbl.n * 64; c += 256) {
+        const int plane = c >> 6, q = c & 63;
+        *(v4u_t*)(frag + (uint64_t)plane * plane_stride + 16 * q) =
+            *(const v4u_t*)&stage[plane][8 * (q & 31) + 4 * (q >> 5)];
+    }
+}
+
 /* k-major X[K][rows] (B as the runtime stores it), same planes. */
 __global__ __launch_bounds__(256, 4)
 void fast_split_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
                               const int32_t* __restrict__ shift, FastTable tbl, int8_t* __restrict__ planes,
-                              uint64_t rows_padded, uint64_t ldk) {
+                              uint64_t rows_padded, uint64_t ldk, int layout) {
     __shared__ __align__(16) double tile[kmaj::SMEM_DOUBLES];
     const uint64_t plane_stride = rows_padded * ldk;
     kmaj::for_each_16(X, rows, K, rows_padded, ldk, 0xffffffffu, tile,
@@ -122,7 +166,7 @@ void fast_split_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint6
             Scaled s[16];
 #pragma unroll
             for (int e = 0; e < 16; e++) s[e] = scaled_integer<true>(x[e], sh);
-            int8_t* out = planes + row * ldk + k;
+            int8_t* out = planes + eshkol_plane_offset(layout, row, k, ldk);
 #pragma unroll 1
             for (int l = 0; l < tbl.n; l++) {
                 v4u_t w;
@@ -311,11 +355,16 @@ int ensure_tables(const FastPlan& f, hipStream_t st) {
 HipOzakiFastStages g_last = {};
 
 int split_any(const double* X, uint64_t rows, uint64_t K, const int32_t* shift, const FastTable& tbl,
-              int8_t* planes, uint64_t rows_padded, uint64_t ldk, bool kmajor, hipStream_t st) {
+              int8_t* planes, uint64_t rows_padded, uint64_t ldk, bool kmajor, int layout, hipStream_t st) {
     if (kmajor) {
         if (kmaj::tile_count(rows_padded, ldk) > 0x7fffffffULL) return -1;
         const dim3 grid((unsigned)kmaj::grid_blocks(rows_padded, ldk, eshkol_hip_num_cus()));
         hipLaunchKernelGGL(fast_split_kmajor_kernel, grid, dim3(256), 0, st, X, rows, K, shift, tbl, planes,
+                           rows_padded, ldk, layout);
+    } else if (layout == 1) {
+        const uint64_t nblk = (rows_padded / 32) * (ldk / 32);
+        if (nblk > 0x7fffffffULL) return -1;
+        hipLaunchKernelGGL(fast_split_il_kernel, dim3((unsigned)nblk), dim3(256), 0, st, X, rows, K, shift, tbl, planes,
                            rows_padded, ldk);
     } else {
         const uint64_t nblk = ((ldk + 1023) / 1024) * rows_padded;
@@ -360,7 +409,8 @@ extern "C" int hip_matmul_ozaki_fast_f64_ex(const double* A, const double* B, do
     if (!eshkol_crt_quiet()) fprintf(stderr, "[GPU] Ozaki-II FAST: n_mod=%d E=%d cap=%d log2(P)=%.1f (int8 MFMA GEMMs)\n",
             f.n, f.E, f.cap, f.log2P);                                  /* gpu_memory.mm:2859 */
 
-    const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ldk = round_up_sz(K, 256);
+    const int layout = hip_igemm_plane_layout(M, N, f.n);
+    const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ldk = round_up_sz(K, layout ? 512 : 256);
     const bool a_kmajor = trans_a != 0, b_kmajor = trans_b == 0;
     double* amax = (double*)eshkol_hip_workspace(WS_ROWSCALE, M * sizeof(double));
     double* bmax = (double*)eshkol_hip_workspace(WS_COLSCALE, N * sizeof(double));
@@ -381,8 +431,8 @@ extern "C" int hip_matmul_ozaki_fast_f64_ex(const double* A, const double* B, do
     if (!ticket) return -1;
     eshkol_crt_shifts_from_exponents(sha, M, shb, N, f.E - 1, st);
 
-    if (split_any(A, M, K, sha, f.table, Ap, Mp, ldk, a_kmajor, st) != 0) return -1;
-    if (split_any(B, N, K, shb, f.table, Bp, Np, ldk, b_kmajor, st) != 0) return -1;
+    if (split_any(A, M, K, sha, f.table, Ap, Mp, ldk, a_kmajor, layout, st) != 0) return -1;
+    if (split_any(B, N, K, shb, f.table, Bp, Np, ldk, b_kmajor, layout, st) != 0) return -1;
 
     HipIgemmArgs ga;
     memset(&ga, 0, sizeof ga);
@@ -391,6 +441,7 @@ extern "C" int hip_matmul_ozaki_fast_f64_ex(const double* A, const double* B, do
     ga.ldk = (uint32_t)ldk; ga.M = (uint32_t)M; ga.N = (uint32_t)N; ga.n_out = (uint32_t)f.n;
     ga.pair_first = g_tables; ga.pair_a = g_tables + 17; ga.pair_b = g_tables + 17;
     ga.mode = 1; ga.max_pairs = 1; ga.modulus = g_tables + 33; ga.out_i8 = Wp;
+    ga.layout = layout;
     if (hip_igemm_i8(&ga, st) != 0) return -1;
 
     const uint64_t nblk = (((N + 3) / 4 + 255) / 256) * M;
@@ -411,7 +462,7 @@ extern "C" int hip_matmul_ozaki_fast_f64_ex(const double* A, const double* B, do
     g_last.a_planes = Ap; g_last.b_planes = Bp; g_last.w_planes = Wp;
     g_last.shift_a = sha; g_last.shift_b = shb;
     g_last.rows_a_padded = Mp; g_last.rows_b_padded = Np; g_last.ldk = ldk;
-    g_last.num_moduli = f.n; g_last.E = f.E; g_last.cap = f.cap;
+    g_last.num_moduli = f.n; g_last.E = f.E; g_last.cap = f.cap; g_last.layout = layout;
     for (int l = 0; l < FAST_MAX_MODULI; l++) g_last.moduli[l] = (l < f.n) ? f.moduli[l] : 0;
     return 0;
 }

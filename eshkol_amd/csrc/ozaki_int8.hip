@@ -86,20 +86,47 @@ void slice_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
     slice_group<G>(x, sc, s, planes + row * ldk + k, rows_padded * ldk);
 }
 
+/* Row-major X[rows][K], interleaved planes (rows_padded and ldk multiples of 32).
+ * A block takes 32 rows x 32 k, a thread four consecutive k of one row: the four
+ * lanes of a 16-byte chunk and eight consecutive rows make a 128-byte segment,
+ * so a wave's 4-byte stores fill two whole lines per plane. */
+__global__ __launch_bounds__(256)
+void slice_il_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
+                     const double* __restrict__ scale, int s, int8_t* __restrict__ planes,
+                     uint64_t rows_padded, uint64_t ldk) {
+    const uint32_t kt = (uint32_t)(ldk / 32);
+    const uint64_t rb = blockIdx.x / kt, kb = blockIdx.x % kt;
+    const int tid = threadIdx.x;
+    const uint64_t row = rb * 32 + (uint64_t)(tid >> 3), k = kb * 32 + 4 * (uint64_t)(tid & 7);
+    double x[4] = {0.0, 0.0, 0.0, 0.0}, sc = 1.0;
+    if (row < rows) {
+        sc = scale[row];
+        const double* p = X + row * K + k;
+        if (k + 4 <= K && (K & 1) == 0 && (((uintptr_t)X & 15) == 0)) {
+            const d2_t v0 = *(const d2_t*)p, v1 = *(const d2_t*)(p + 2);
+            x[0] = v0.x; x[1] = v0.y; x[2] = v1.x; x[3] = v1.y;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) if (k + e < K) x[e] = p[e];
+        }
+    }
+    slice_group<4>(x, sc, s, planes + eshkol_plane_offset(1, row, k, ldk), rows_padded * ldk);
+}
+
 /* k-major X[K][rows] (B as the runtime stores it), same output: the job of the
  * reference's B kernel (gpu_cuda_kernels.cu:706-723), which scatters transposed
  * bytes; here the transposition happens in LDS and the stores stay contiguous. */
 __global__ __launch_bounds__(256, 4)
 void slice_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
                          const double* __restrict__ scale, int s, int8_t* __restrict__ planes,
-                         uint64_t rows_padded, uint64_t ldk) {
+                         uint64_t rows_padded, uint64_t ldk, int layout) {
     __shared__ __align__(16) double tile[kmaj::SMEM_DOUBLES];
     const uint64_t plane_stride = rows_padded * ldk;
     if ((ldk & 15) == 0 && (((uintptr_t)planes & 15) == 0)) {
         kmaj::for_each_16(X, rows, K, rows_padded, ldk, 0xffffffffu, tile,
             [&](uint64_t row) { return (row < rows) ? scale[row] : 1.0; },
             [&](uint64_t row, uint64_t k, const double* x, double sc) {
-                slice_group<16>(x, sc, s, planes + row * ldk + k, plane_stride);
+                slice_group<16>(x, sc, s, planes + eshkol_plane_offset(layout, row, k, ldk), plane_stride);
             });
         return;
     }
@@ -107,7 +134,7 @@ void slice_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K
         [&](uint64_t row) { return (row < rows) ? scale[row] : 1.0; },
         [&](uint64_t row, uint64_t k, double x0, double x1, double sc) {
             const double x[2] = {x0, x1};
-            slice_group<2>(x, sc, s, planes + row * ldk + k, plane_stride);
+            slice_group<2>(x, sc, s, planes + eshkol_plane_offset(layout, row, k, ldk), plane_stride);
         });
 }
 
@@ -172,14 +199,20 @@ constexpr int MAX_BUF = 128, MAX_PAIRS = 128;
 
 namespace {
 int slice_any(const double* X, uint64_t rows, uint64_t K, const double* scale, int s,
-              int8_t* planes, uint64_t rows_padded, uint64_t ldk, bool kmajor, void* stream) {
+              int8_t* planes, uint64_t rows_padded, uint64_t ldk, bool kmajor, int layout, void* stream) {
     if (!X || !scale || !planes || rows == 0 || K == 0 || s < 1 || s > 16) return -1;
     if (rows_padded < rows || ldk < K || (ldk & 1)) return -1;
+    if (layout != 0 && layout != 1) return -1;
+    if (layout == 1 && ((rows_padded & 31) || (ldk & 31) || ((uintptr_t)planes & 15))) return -1;
     const int g = (ldk % 4 == 0 && ((uintptr_t)planes & 3) == 0) ? 4 : 2;
-    const uint64_t nblk = kmajor ? kmaj::grid_blocks(rows_padded, ldk, eshkol_hip_num_cus()) : ((ldk / g + 255) / 256) * rows_padded;
+    const uint64_t nblk = kmajor ? kmaj::grid_blocks(rows_padded, ldk, eshkol_hip_num_cus())
+                        : layout ? (rows_padded / 32) * (ldk / 32) : ((ldk / g + 255) / 256) * rows_padded;
     if (nblk > 0x7fffffffULL || (kmajor && kmaj::tile_count(rows_padded, ldk) > 0x7fffffffULL)) return -1;
     if (kmajor)
         hipLaunchKernelGGL(slice_kmajor_kernel, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
+                           X, rows, K, scale, s, planes, rows_padded, ldk, layout);
+    else if (layout == 1)
+        hipLaunchKernelGGL(slice_il_kernel, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
                            X, rows, K, scale, s, planes, rows_padded, ldk);
     else if (g == 4)
         hipLaunchKernelGGL(slice_kernel<4>, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
@@ -193,12 +226,18 @@ int slice_any(const double* X, uint64_t rows, uint64_t K, const double* scale, i
 
 extern "C" int hip_ozaki_slice_f64(const double* X, uint64_t rows, uint64_t K, const double* scale, int s,
                                    int8_t* planes, uint64_t rows_padded, uint64_t ldk, void* stream) {
-    return slice_any(X, rows, K, scale, s, planes, rows_padded, ldk, false, stream);
+    return slice_any(X, rows, K, scale, s, planes, rows_padded, ldk, false, 0, stream);
 }
 
 extern "C" int hip_ozaki_slice_kmajor_f64(const double* X, uint64_t rows, uint64_t K, const double* scale, int s,
                                           int8_t* planes, uint64_t rows_padded, uint64_t ldk, void* stream) {
-    return slice_any(X, rows, K, scale, s, planes, rows_padded, ldk, true, stream);
+    return slice_any(X, rows, K, scale, s, planes, rows_padded, ldk, true, 0, stream);
+}
+
+extern "C" int hip_ozaki_slice_planes_f64(const double* X, uint64_t rows, uint64_t K, const double* scale, int s,
+                                          int8_t* planes, uint64_t rows_padded, uint64_t ldk,
+                                          int kmajor, int layout, void* stream) {
+    return slice_any(X, rows, K, scale, s, planes, rows_padded, ldk, kmajor != 0, layout, stream);
 }
 
 extern "C" int hip_ozaki_reconstruct_f64(double* C, const int32_t* Gall, const double* d_weights, int nbuf,
@@ -268,8 +307,10 @@ extern "C" int hip_matmul_ozaki_int8_f64_ex(const double* A, const double* B, do
     }
     plan->first[nbuf] = npairs;
 
-    const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ldk = round_up_sz(K, 256);
-    /* Both operands come out as slice planes [row][k]. One stored with k
+    const int layout = hip_igemm_plane_layout(M, N, nbuf);
+    const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ldk = round_up_sz(K, layout ? 512 : 256);
+    /* Both operands come out as slice planes [row][k] (interleaved when the
+     * contraction takes the kernel that wants them so). One stored with k
      * contiguous is read row by row, one stored k-major (B as given, A when the
      * caller holds A^T) through LDS tiles: no transposed fp64 copy either way. */
     const bool a_kmajor = trans_a != 0, b_kmajor = trans_b == 0;
@@ -288,8 +329,8 @@ extern "C" int hip_matmul_ozaki_int8_f64_ex(const double* A, const double* B, do
      * the maxima and reported as failure so the caller uses the native GEMM. */
     if (!ESHKOL_HIP_OK(hipMemcpyAsync(h_max, rmax, M * sizeof(double), hipMemcpyDeviceToHost, st))) return -1;
     if (!ESHKOL_HIP_OK(hipMemcpyAsync(h_max + M, cmax, N * sizeof(double), hipMemcpyDeviceToHost, st))) return -1;
-    if (slice_any(A, M, K, rmax, s, As, Mp, ldk, a_kmajor, st) != 0) return -1;
-    if (slice_any(B, N, K, cmax, s, Bs, Np, ldk, b_kmajor, st) != 0) return -1;
+    if (slice_any(A, M, K, rmax, s, As, Mp, ldk, a_kmajor, layout, st) != 0) return -1;
+    if (slice_any(B, N, K, cmax, s, Bs, Np, ldk, b_kmajor, layout, st) != 0) return -1;
 
     HipIgemmArgs ga;
     memset(&ga, 0, sizeof ga);
@@ -297,7 +338,7 @@ extern "C" int hip_matmul_ozaki_int8_f64_ex(const double* A, const double* B, do
     ga.a_plane_stride = Mp * ldk; ga.b_plane_stride = Np * ldk;
     ga.ldk = (uint32_t)ldk; ga.M = (uint32_t)M; ga.N = (uint32_t)N; ga.n_out = (uint32_t)nbuf;
     ga.pair_first = dplan->first; ga.pair_a = dplan->pa; ga.pair_b = dplan->pb;
-    ga.mode = 0; ga.max_pairs = s; ga.out_i32 = G;
+    ga.mode = 0; ga.max_pairs = s; ga.out_i32 = G; ga.layout = layout;
     if (hip_igemm_i8(&ga, st) != 0) return -1;
     if (hip_ozaki_reconstruct_f64(C, G, dplan->w, nbuf, rmax, cmax, M, N, st) != 0) return -1;
 
@@ -307,7 +348,7 @@ extern "C" int hip_matmul_ozaki_int8_f64_ex(const double* A, const double* B, do
     g_last.a_slices = As; g_last.b_slices = Bs; g_last.products = G;
     g_last.rmax = rmax; g_last.cmax = cmax;
     g_last.rows_a_padded = Mp; g_last.rows_b_padded = Np; g_last.ldk = ldk;
-    g_last.s = s; g_last.nbuf = nbuf;
+    g_last.s = s; g_last.nbuf = nbuf; g_last.layout = layout;
     return 0;
 }
 

@@ -131,8 +131,22 @@ typedef struct {
     const int32_t* modulus;
     int32_t* out_i32;
     int8_t*  out_i8;
+    /* 0: planes are [rows][ldk]. 1: interleaved, the layout the tiers use for
+     * products that fill the device: rows in blocks of 32, inside a block the
+     * 16-byte k-chunks slow and the row fast,
+     *   offset(row, k) = (row/32) * 32*ldk + (k/16) * 512 + (row%32) * 16 + k%16,
+     * so the 32-row x 32-byte operand fragment of one matrix-core instruction is
+     * 1 KiB of contiguous memory. Needs ldk % 512 == 0 and max_pairs >= 1 (every
+     * output plane at least one product). */
+    int32_t layout;
 } HipIgemmArgs;
 int hip_igemm_i8(const HipIgemmArgs* args, void* stream);
+
+/* The layout (HipIgemmArgs.layout) the tiers give their operand planes for a
+ * contraction of n_out output planes of M x N: 1 when the launch has at least
+ * 128 tiles of 256 x 256 and so takes the direct-to-LDS kernel, else 0. With 1
+ * the k pitch is padded to a multiple of 512. */
+int hip_igemm_plane_layout(uint64_t M, uint64_t N, int n_out);
 
 /* ---- Ozaki-II CRT exact tier ------------------------------------------------
  * Residue planes of trunc(X[i,k] * 2^shift[i]) modulo the first num_moduli
@@ -149,6 +163,14 @@ int hip_ozaki_crt_split_f64(const double* X, uint64_t rows, uint64_t K,
 int hip_ozaki_crt_split_kmajor_f64(const double* X, uint64_t rows, uint64_t K,
                                    const int32_t* shift, int num_moduli,
                                    int8_t* planes, uint64_t rows_padded, uint64_t ldk, void* stream);
+
+/* Either of the two with the plane layout as an argument (HipIgemmArgs.layout;
+ * layout 1 needs rows_padded and ldk to be multiples of 32 and planes 16-byte
+ * aligned). */
+int hip_ozaki_crt_split_planes_f64(const double* X, uint64_t rows, uint64_t K,
+                                   const int32_t* shift, int num_moduli,
+                                   int8_t* planes, uint64_t rows_padded, uint64_t ldk,
+                                   int kmajor, int layout, void* stream);
 
 /* CRT accumulation, reconstruction and inverse scaling (gpu_memory.mm:2626-2655)
  * from the int8 residue products w_planes[l][M][N]; optional fused dense-layer
@@ -190,6 +212,7 @@ typedef struct {
     const int32_t* mu; const int32_t* nu;
     uint64_t rows_a_padded, rows_b_padded, ldk;
     int32_t num_moduli, E;
+    int32_t layout;             /* of a_planes and b_planes: HipIgemmArgs.layout */
 } HipOzakiCrtStages;
 int hip_ozaki_crt_last_stages(HipOzakiCrtStages* out);
 
@@ -220,6 +243,7 @@ typedef struct {
     uint64_t rows_a_padded, rows_b_padded, ldk;
     int32_t num_moduli, E, cap;
     int32_t moduli[16];
+    int32_t layout;             /* of a_planes and b_planes: HipIgemmArgs.layout */
 } HipOzakiFastStages;
 int hip_ozaki_fast_last_stages(HipOzakiFastStages* out);
 
@@ -253,6 +277,11 @@ int hip_ozaki_slice_f64(const double* X, uint64_t rows, uint64_t K, const double
 int hip_ozaki_slice_kmajor_f64(const double* X, uint64_t rows, uint64_t K, const double* scale, int s,
                                int8_t* planes, uint64_t rows_padded, uint64_t ldk, void* stream);
 
+/* Either of the two with the plane layout as an argument (HipIgemmArgs.layout). */
+int hip_ozaki_slice_planes_f64(const double* X, uint64_t rows, uint64_t K, const double* scale, int s,
+                               int8_t* planes, uint64_t rows_padded, uint64_t ldk,
+                               int kmajor, int layout, void* stream);
+
 /* cuda_ozaki_reconstruct_f64 (gpu_cuda_kernels.cu:728-741, 779-798), weights
  * already in device memory. */
 int hip_ozaki_reconstruct_f64(double* C, const int32_t* Gall, const double* d_weights, int nbuf,
@@ -268,6 +297,7 @@ typedef struct {
     const double* rmax; const double* cmax;
     uint64_t rows_a_padded, rows_b_padded, ldk;
     int32_t s, nbuf;
+    int32_t layout;             /* of a_slices and b_slices: HipIgemmArgs.layout */
 } HipOzakiInt8Stages;
 int hip_ozaki_int8_last_stages(HipOzakiInt8Stages* out);
 
@@ -368,6 +398,12 @@ void hip_dgemm_set_tail_split(int on);
 
 /* k-blocks kept in flight by the pipelined int8 kernel (1..3; 0 = simple kernel only). */
 void hip_igemm_set_prefetch(int pf);
+
+/* 1 (default): contractions with at least 128 tiles take interleaved operand
+ * planes and the kernel that loads them straight into LDS and MFMA registers;
+ * 0: row-major planes and the register-staged kernels everywhere. Same results;
+ * the switch exists to compare them. */
+void hip_igemm_set_direct(int on);
 
 /* 1 (default): the pipelined int8 kernel runs as one workgroup per CU walking a
  * list of tiles, its operand stream continuous across tile boundaries; 0: one

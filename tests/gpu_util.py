@@ -67,8 +67,8 @@ def run_crt(A, B, num_moduli=16, adaptive=False, bias=None, act=0, want_stages=T
     sg = ea.HipOzakiCrtStages()
     assert lib.hip_ozaki_crt_last_stages(C.byref(sg)) == 0
     n, M, K, N = sg.num_moduli, ops.M, ops.K, ops.N
-    ap = ea.download_raw(sg.a_planes, (n, sg.rows_a_padded, sg.ldk), np.int8)
-    bp = ea.download_raw(sg.b_planes, (n, sg.rows_b_padded, sg.ldk), np.int8)
+    ap = ea.deinterleave(ea.download_raw(sg.a_planes, (n, sg.rows_a_padded, sg.ldk), np.int8), sg.layout)
+    bp = ea.deinterleave(ea.download_raw(sg.b_planes, (n, sg.rows_b_padded, sg.ldk), np.int8), sg.layout)
     st = dict(num_moduli=n, E=sg.E,
               mu=ea.download_raw(sg.mu, (M,), np.int32), nu=ea.download_raw(sg.nu, (N,), np.int32),
               a_planes=ap[:, :M, :K], b_planes=bp[:, :N, :K],
@@ -90,8 +90,8 @@ def run_int8(A, B, T, want_stages=True):
     sg = ea.HipOzakiInt8Stages()
     assert lib.hip_ozaki_int8_last_stages(C.byref(sg)) == 0
     s, M, K, N = sg.s, ops.M, ops.K, ops.N
-    As = ea.download_raw(sg.a_slices, (s, sg.rows_a_padded, sg.ldk), np.int8)
-    Bs = ea.download_raw(sg.b_slices, (s, sg.rows_b_padded, sg.ldk), np.int8)
+    As = ea.deinterleave(ea.download_raw(sg.a_slices, (s, sg.rows_a_padded, sg.ldk), np.int8), sg.layout)
+    Bs = ea.deinterleave(ea.download_raw(sg.b_slices, (s, sg.rows_b_padded, sg.ldk), np.int8), sg.layout)
     st = dict(s=s, nbuf=sg.nbuf, a_slices=As[:, :M, :K], b_slices=Bs[:, :N, :K],
               pad_clear=not (As[:, M:, :].any() or As[:, :, K:].any() or Bs[:, N:, :].any() or Bs[:, :, K:].any()),
               products=ea.download_raw(sg.products, (sg.nbuf, M, N), np.int32),
@@ -127,8 +127,8 @@ def run_fast(A, B, n_mod=11, want_stages=True, trans=None):
     sg = ea.HipOzakiFastStages()
     assert lib.hip_ozaki_fast_last_stages(C.byref(sg)) == 0
     n, M, K, N = sg.num_moduli, ops.M, ops.K, ops.N
-    ap = ea.download_raw(sg.a_planes, (n, sg.rows_a_padded, sg.ldk), np.int8)
-    bp = ea.download_raw(sg.b_planes, (n, sg.rows_b_padded, sg.ldk), np.int8)
+    ap = ea.deinterleave(ea.download_raw(sg.a_planes, (n, sg.rows_a_padded, sg.ldk), np.int8), sg.layout)
+    bp = ea.deinterleave(ea.download_raw(sg.b_planes, (n, sg.rows_b_padded, sg.ldk), np.int8), sg.layout)
     st = dict(num_moduli=n, E=sg.E, cap=sg.cap, moduli=list(sg.moduli[:n]),
               shift_a=ea.download_raw(sg.shift_a, (M,), np.int32), shift_b=ea.download_raw(sg.shift_b, (N,), np.int32),
               a_planes=ap[:, :M, :K], b_planes=bp[:, :N, :K],

@@ -14,7 +14,8 @@ from gpu_util import stream
 pytestmark = pytest.mark.gpu
 
 MODULI = [256, 255, 253, 251, 247, 241, 239, 233, 229, 227, 223, 217, 211, 199, 197, 193]
-KERNELS = {"simple": (0, 0), "pipelined": (2, 0), "persistent": (2, 1), "pipelined-1": (1, 0), "persistent-1": (1, 1)}
+KERNELS = {"simple": (0, 0), "pipelined": (2, 0), "persistent": (2, 1), "pipelined-1": (1, 0), "persistent-1": (1, 1),
+           "direct": (2, 1)}           # interleaved planes, operands loaded straight into LDS / MFMA registers
 
 
 def pad(n, m):
@@ -28,10 +29,23 @@ def planes(rng, n_planes, rows, K, lo=-128, hi=128):
     return out
 
 
+def interleave(x):
+    """[n][rows][ldk] -> the interleaved layout: rows in blocks of 32, inside a block the
+    16-byte k-chunks slow and the row fast; ldk padded to a multiple of 512 first."""
+    n, rows, ldk = x.shape
+    if ldk % 512:
+        x = np.concatenate([x, np.zeros((n, rows, pad(ldk, 512) - ldk), np.int8)], axis=2)
+        ldk = x.shape[2]
+    y = x.reshape(n, rows // 32, 32, ldk // 16, 16).transpose(0, 1, 3, 2, 4)
+    return np.ascontiguousarray(y).reshape(n, rows, ldk)
+
+
 def run(a, b, M, N, plan, mode, kernel):
     """plan: list of lists of (a_plane, b_plane) per output plane."""
     lib = ea.load()
     pf, pers = KERNELS[kernel]
+    if kernel == "direct":
+        a, b = interleave(a), interleave(b)
     first = np.cumsum([0] + [len(p) for p in plan]).astype(np.int32)
     pa = np.array([t[0] for p in plan for t in p], np.int32)
     pb = np.array([t[1] for p in plan for t in p], np.int32)
@@ -46,6 +60,7 @@ def run(a, b, M, N, plan, mode, kernel):
     g.ldk, g.M, g.N, g.n_out = a.shape[2], M, N, n_out
     g.pair_first, g.pair_a, g.pair_b = dF.ptr, dPa.ptr, dPb.ptr
     g.mode, g.max_pairs, g.modulus = mode, max(len(p) for p in plan), dMod.ptr
+    g.layout = 1 if kernel == "direct" else 0
     if mode == 1:
         g.out_i8 = out.ptr
     else:

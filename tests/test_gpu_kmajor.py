@@ -153,3 +153,42 @@ def test_narrowing(gpu, K, R, is_bf16):
     a = pa.download()
     assert np.array_equal(a, pb.download())
     assert not a[R:, :].any() and not a[:, K:].any()
+
+
+@pytest.mark.parametrize("K,R", [(1, 1), (7, 5), (129, 33), (300, 70), (1000, 513), (1024, 1024), (2049, 511)])
+@pytest.mark.parametrize("nmod", [2, 16])
+def test_interleaved_crt_planes_hold_the_same_residues(gpu, K, R, nmod):
+    """Interleaved planes (rows in blocks of 32, 16-byte k-chunks slow, rows fast) from both
+    operand orders, put back in order, are the row-major planes byte for byte, padding included."""
+    lib = ea.load()
+    X = synth.wide_range(K + 11 * R, (K, R), -8, 8)
+    shift = (20 - np.floor(np.log2(np.maximum(np.abs(X).max(axis=0), 1e-300)))).astype(np.int32)
+    Rp, ldk = pad(R, 256), pad(K, 512)
+    dX, dXt, dsh = dev(X), dev(X.T), dev(shift, np.int32)
+    ref = ea.DeviceArray.from_host(np.full((nmod, Rp, ldk), 78, np.int8))
+    assert lib.hip_ozaki_crt_split_f64(dXt.ptr, R, K, dsh.ptr, nmod, ref.ptr, Rp, ldk, stream()) == 0
+    for kmajor, src in ((1, dX), (0, dXt)):
+        out = ea.DeviceArray.from_host(np.full((nmod, Rp, ldk), 77, np.int8))
+        assert lib.hip_ozaki_crt_split_planes_f64(src.ptr, R, K, dsh.ptr, nmod, out.ptr, Rp, ldk, kmajor, 1, stream()) == 0
+        ea.synchronize()
+        assert np.array_equal(ea.deinterleave(out.download(), 1), ref.download()), kmajor
+    odd = ea.DeviceArray((nmod, Rp + 1, ldk), np.int8)
+    assert lib.hip_ozaki_crt_split_planes_f64(dXt.ptr, R, K, dsh.ptr, nmod, odd.ptr, Rp + 1, ldk, 0, 1, stream()) == -1
+
+
+@pytest.mark.parametrize("K,R", [(1, 1), (7, 5), (129, 33), (300, 70), (1000, 513), (1024, 1024), (2049, 511)])
+def test_interleaved_slice_planes_hold_the_same_slices(gpu, K, R):
+    lib = ea.load()
+    s = 7
+    X = synth.normal(K + 13 * R, (K, R))
+    scale = np.abs(X).max(axis=0)
+    scale[scale == 0.0] = 1.0
+    Rp, ldk = pad(R, 256), pad(K, 512)
+    dX, dXt, dsc = dev(X), dev(X.T), dev(scale)
+    ref = ea.DeviceArray.from_host(np.full((s, Rp, ldk), 78, np.int8))
+    assert lib.hip_ozaki_slice_f64(dXt.ptr, R, K, dsc.ptr, s, ref.ptr, Rp, ldk, stream()) == 0
+    for kmajor, src in ((1, dX), (0, dXt)):
+        out = ea.DeviceArray.from_host(np.full((s, Rp, ldk), 77, np.int8))
+        assert lib.hip_ozaki_slice_planes_f64(src.ptr, R, K, dsc.ptr, s, out.ptr, Rp, ldk, kmajor, 1, stream()) == 0
+        ea.synchronize()
+        assert np.array_equal(ea.deinterleave(out.download(), 1), ref.download()), kmajor
