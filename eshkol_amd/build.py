@@ -51,6 +51,32 @@ COMMON = [
 ]
 
 
+# Kernels whose main loop issues its loads from inline assembly (gemm_pipe2.h): a
+# register the compiler spills while such a load is still in flight would be saved
+# before its data has arrived. They must therefore compile without any vector
+# spill; the compiler's resource remarks are checked after every build.
+NO_SPILL = {"igemm_i8.hip": ["igemm_i8_direct_kernel"]}
+
+
+def _check_no_spill(src, remarks):
+    wanted = NO_SPILL.get(src, [])
+    current, seen = None, set()
+    for line in remarks.splitlines():
+        if "Function Name:" in line:
+            name = line.split("Function Name:")[1].split()[0]
+            current = next((w for w in wanted if w in name), None)
+            if current:
+                seen.add(current)
+        elif current and ("ScratchSize" in line or "VGPRs Spill" in line):
+            value = int(line.split(":")[-1].split("[")[0].strip())
+            if value != 0:
+                raise RuntimeError("%s: kernel %s spills vector registers (%s); its asynchronous loads "
+                                   "do not survive that" % (src, current, line.strip()))
+    missing = [w for w in wanted if w not in seen]
+    if missing:
+        raise RuntimeError("%s: no resource remarks for %s; cannot prove it is free of spills" % (src, missing))
+
+
 def _newer(target, deps):
     if not os.path.exists(target):
         return False
@@ -67,9 +93,17 @@ def _compile(src, force):
     if not force and _newer(obj, [path] + headers):
         return obj
     cmd = [HIPCC] + COMMON + EXTRA.get(src, []) + ["-x", "hip", "-c", path, "-o", obj]
+    if src in NO_SPILL:
+        cmd.insert(1, "-Rpass-analysis=kernel-resource-usage")
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s\n%s" % (src, res.stdout, res.stderr))
+    if src in NO_SPILL:
+        try:
+            _check_no_spill(src, res.stderr)
+        except RuntimeError:
+            os.remove(obj)
+            raise
     return obj
 
 

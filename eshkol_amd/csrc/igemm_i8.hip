@@ -249,6 +249,22 @@ void igemm_i8_persistent_kernel(HipIgemmArgs g, int tiles_m, int tiles_n, int ch
     pipe::run_tiles<I8Op, TM, TN, PF>(smem_i8, cm, next_tile, epi);
 }
 
+/* Per modulus p <= 256, for the direct kernel's residue epilogue: the smallest
+ * multiple of p that is >= 2^31, and the byte weights 256^i mod p (i = 0..3)
+ * packed into a word. Tables instead of divisions per tile: the kernel has no
+ * vector registers to spare for them. */
+struct ModulusTables { uint32_t start[257]; uint32_t wbytes[257]; };
+constexpr ModulusTables make_modulus_tables() {
+    ModulusTables t{};
+    for (uint32_t p = 1; p <= 256; p++) {
+        t.start[p] = (uint32_t)(((0x80000000ull + p - 1) / p) * p);
+        const uint32_t w0 = 1u % p, w1 = 256u % p, w2 = w1 * w1 % p, w3 = w2 * w1 % p;
+        t.wbytes[p] = w0 | w1 << 8 | w2 << 16 | w3 << 24;
+    }
+    return t;
+}
+__device__ const ModulusTables MOD_TABLES = make_modulus_tables();
+
 /* ---- interleaved planes: operands never pass through registers on their way
  * to LDS (gemm_pipe2.h) ---------------------------------------------------------
  * Four waves stacked along M, each with a 64 x 256 accumulator: acc[t][u] is
@@ -295,9 +311,14 @@ __device__ __forceinline__ void epilogue_direct(const HipIgemmArgs& g, int o, in
         return;
     }
 
-    /* mode 1: the exact reduction modulo p of epilogue() above */
+    /* mode 1. Adding the smallest multiple of p that is not below 2^31 makes the
+     * sum (|sum| < 2^31 for every K the tiers accept) a non-negative 32-bit word
+     * of the same residue class. One byte dot product with 256^i mod p gives
+     * x < 2^18 congruent to it; the nearest-multiple step of epilogue() above then
+     * leaves the residue in the low byte: five instructions per element. */
     const int p = pipe2::scalar_load(g.modulus + o);
-    const int c20 = (1 << 20) % p;
+    const uint32_t wbytes = (uint32_t)pipe2::scalar_load((const int32_t*)&MOD_TABLES.wbytes[p & 0x1ff]);
+    const uint32_t lift = (uint32_t)pipe2::scalar_load((const int32_t*)&MOD_TABLES.start[p & 0x1ff]);
     const float pinv = 1.0f / (float)p;
     constexpr int EP = pipe2::EPI_PITCH;
     int8_t* out = g.out_i8 + (size_t)o * g.M * g.N;
@@ -315,8 +336,7 @@ __device__ __forceinline__ void epilogue_direct(const HipIgemmArgs& g, int o, in
                     int r[4];
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        const int s = acc[t][u][4 * v + e];
-                        const int x = __mul24(s >> 20, c20) + (s & 0xfffff);
+                        const int x = (int)__builtin_amdgcn_udot4((uint32_t)acc[t][u][4 * v + e] + lift, wbytes, 0u, false);
                         const float qm = fmaf((float)x, pinv, 12582912.0f);
                         r[e] = __mul24(__float_as_int(qm), -p) + x;
                     }
