@@ -100,9 +100,11 @@ struct Source {
 struct Tile {
     int m0, n0;                 /* first row of the A planes / of the B planes */
     int tag;                    /* caller's: output plane */
-    const int32_t* a_idx;       /* plane indices of the tile's products (device memory), or NULL for plane 0 */
+    const int32_t* a_idx;       /* plane indices of the tile's products (device memory), or NULL: */
     const int32_t* b_idx;
     int npairs;                 /* >= 1 */
+    int a_plane0 = 0;           /* the one plane a list-less tile multiplies (run_tiles of gemm_pipe2.h only) */
+    int b_plane0 = 0;
 };
 
 template <int TM, int TN> struct TilesCfg {

@@ -159,12 +159,13 @@ __device__ __forceinline__ void run_tiles(int8_t* smem, const Source& cm, Next n
     const int8_t* c_b = wave_rows_b(cur);
     const int32_t* c_ai = cur.a_idx;
     const int32_t* c_bi = cur.b_idx;
+    int c_pa = cur.a_plane0, c_pb = cur.b_plane0;
     int c_t = 0, c_j = 0, c_np = cur.npairs;
     bool c_in_next = false;                     /* the cursor has crossed into nxt */
     v4i_t rs_a, rs_b;
     auto point_at_product = [&]() {
-        const int ia = c_ai ? scalar_load(c_ai + c_t) : 0;
-        const int ib = c_bi ? scalar_load(c_bi + c_t) : 0;
+        const int ia = c_ai ? scalar_load(c_ai + c_t) : c_pa;
+        const int ib = c_bi ? scalar_load(c_bi + c_t) : c_pb;
         rs_a = rsrc_words(c_a + (size_t)ia * cm.a_plane_stride);
         rs_b = rsrc_words(c_b + (size_t)ib * cm.b_plane_stride);
     };
@@ -181,6 +182,7 @@ __device__ __forceinline__ void run_tiles(int8_t* smem, const Source& cm, Next n
             c_in_next = true;
             c_a = wave_rows_a(nxt); c_b = wave_rows_b(nxt);
             c_ai = nxt.a_idx; c_bi = nxt.b_idx; c_np = nxt.npairs;
+            c_pa = nxt.a_plane0; c_pb = nxt.b_plane0;
             c_t = 0; c_j = 0; c_soff = 0;
             point_at_product();
         }

@@ -1137,11 +1137,14 @@ void eshkol_batch_matmul_dispatch(const double* a, const double* b, double* c,
         if (wa && wb && wc) {
             int rc = 0;
             if (reduced) {
-                for (int64_t i = 0; i < batch && rc == 0; i++)
-                    rc = hip_matmul_reduced_f64((const double*)ba.device_ptr + (size_t)i * M * K,
-                                                (const double*)bb.device_ptr + (size_t)i * K * N,
-                                                (double*)bc.device_ptr + (size_t)i * M * N,
-                                                (uint64_t)M, (uint64_t)K, (uint64_t)N, dtype, 1, g_stream);
+                /* all products in one strided launch, as the reference's
+                 * cublasGemmStridedBatchedEx does (gpu_memory_cuda.cpp:763-771) */
+                GPU_LOG("batch matmul %lld x (%lldx%lld @ %lldx%lld) -> reduced tier (%s in, fp32 accumulate), one strided launch",
+                        (long long)batch, (long long)M, (long long)K, (long long)K, (long long)N,
+                        dtype == 2 ? "f16" : "bf16");
+                rc = hip_matmul_reduced_f64_batched((const double*)ba.device_ptr, (const double*)bb.device_ptr,
+                                                    (double*)bc.device_ptr, (uint64_t)batch,
+                                                    (uint64_t)M, (uint64_t)K, (uint64_t)N, dtype, 1, g_stream);
             } else {
                 GPU_LOG("batch matmul %lld x (%lldx%lld @ %lldx%lld) -> native fp64 MFMA, one strided launch",
                         (long long)batch, (long long)M, (long long)K, (long long)K, (long long)N);

@@ -20,6 +20,7 @@
 #include "hip_common.h"
 #include "kernels.h"
 #include "gemm_pipe.h"
+#include "gemm_pipe2.h"
 #include "kmajor_tile.h"
 
 #include <cstring>
@@ -69,11 +70,16 @@ __device__ __forceinline__ uint32_t narrow_pair(double x0, double x1) {
     return (uint32_t)h0 | ((uint32_t)h1 << 16);
 }
 
+/* Every narrowing kernel converts `gridDim.y` matrices stored back to back
+ * (X + b * rows * K -> out + b * rows_padded * ld). */
+
 /* Row-major X[rows][K]. One thread: two consecutive k of one row. */
 template <bool BF16>
 __global__ __launch_bounds__(256)
 void convert_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
                     uint16_t* __restrict__ out, uint64_t rows_padded, uint64_t ld) {
+    X += (uint64_t)blockIdx.y * rows * K;
+    out += (uint64_t)blockIdx.y * rows_padded * ld;
     const uint32_t cpr = (uint32_t)((ld / 2 + 255) / 256);
     const uint64_t row = blockIdx.x / cpr;
     const uint64_t k = ((uint64_t)(blockIdx.x % cpr) * 256 + threadIdx.x) * 2;
@@ -91,12 +97,60 @@ void convert_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
     *(uint32_t*)(out + row * ld + k) = narrow_pair<BF16>(x0, x1);
 }
 
+/* Row-major X[rows][K] into the interleaved layout (rows_padded a multiple of 32,
+ * ld of 64 elements). A block takes 32 rows x 64 k: eight lanes read 512
+ * contiguous bytes of a row, a lane narrows eight k into one 16-byte chunk, and
+ * the chunks of eight consecutive rows are 128 contiguous output bytes. */
+template <bool BF16>
+__global__ __launch_bounds__(256)
+void convert_il_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
+                       uint16_t* __restrict__ out, uint64_t rows_padded, uint64_t ld) {
+    X += (uint64_t)blockIdx.y * rows * K;
+    out += (uint64_t)blockIdx.y * rows_padded * ld;
+    const uint32_t kt = (uint32_t)(ld / 64);
+    const uint64_t rb = blockIdx.x / kt, kb = blockIdx.x % kt;
+    const int tid = threadIdx.x;
+    const uint64_t row = rb * 32 + (uint64_t)(tid >> 3), k = kb * 64 + 8 * (uint64_t)(tid & 7);
+    double x[8] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0};
+    if (row < rows && k < K) {
+        const double* p = X + row * K + k;
+        if (k + 8 <= K && (K & 1) == 0 && (((uintptr_t)X & 15) == 0)) {
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) { const d2_t v = *(const d2_t*)(p + e); x[e] = v.x; x[e + 1] = v.y; }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) if (k + e < K) x[e] = p[e];
+        }
+    }
+    v4i_t w;
+#pragma unroll
+    for (int e = 0; e < 4; e++) w[e] = (int)narrow_pair<BF16>(x[2 * e], x[2 * e + 1]);
+    *(v4i_t*)((int8_t*)out + eshkol_plane_offset(1, row, 2 * k, 2 * ld)) = w;
+}
+
 /* k-major X[K][rows] (B as the runtime stores it), same output. */
 template <bool BF16>
 __global__ __launch_bounds__(256, 4)
 void convert_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
-                           uint16_t* __restrict__ out, uint64_t rows_padded, uint64_t ld) {
+                           uint16_t* __restrict__ out, uint64_t rows_padded, uint64_t ld, int layout) {
     __shared__ __align__(16) double tile[kmaj::SMEM_DOUBLES];
+    X += (uint64_t)blockIdx.y * rows * K;
+    out += (uint64_t)blockIdx.y * rows_padded * ld;
+    if (layout == 1) {
+        /* sixteen k per thread: two 16-byte chunks of one row */
+        kmaj::for_each_16(X, rows, K, rows_padded, ld, 0xffffffffu, tile,
+            [](uint64_t) { return 0; },
+            [&](uint64_t row, uint64_t k, const double* x, int) {
+#pragma unroll
+                for (int c = 0; c < 2; c++) {
+                    v4i_t w;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) w[e] = (int)narrow_pair<BF16>(x[8 * c + 2 * e], x[8 * c + 2 * e + 1]);
+                    *(v4i_t*)((int8_t*)out + eshkol_plane_offset(1, row, 2 * k + 16 * c, 2 * ld)) = w;
+                }
+            });
+        return;
+    }
     kmaj::for_each_pair(X, rows, K, rows_padded, ld, 0xffffffffu, tile,
         [](uint64_t) { return 0; },
         [&](uint64_t row, uint64_t k, double x0, double x1, int) {
@@ -120,9 +174,13 @@ template <bool BF16, int TM, int TN>
 __global__ __launch_bounds__(256)
 void hgemm_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ Bt,
                   int M, int N, int ld_bytes, int out_mode, void* __restrict__ Cout,
-                  int tiles_m, int tiles_n) {
+                  int tiles_m, int tiles_n, uint64_t a_stride, uint64_t b_stride) {
     using C = Cfg<TM, TN>;
     extern __shared__ __align__(16) int8_t smem_h[];
+    /* blockIdx.y: one of the products stored back to back (strides in bytes) */
+    A = (const uint16_t*)((const int8_t*)A + (uint64_t)blockIdx.y * a_stride);
+    Bt = (const uint16_t*)((const int8_t*)Bt + (uint64_t)blockIdx.y * b_stride);
+    Cout = (int8_t*)Cout + (uint64_t)blockIdx.y * (uint64_t)M * (uint64_t)N * (out_mode == 0 ? 4u : 8u);
     int8_t* As = smem_h;
     int8_t* Bs = smem_h + 2 * C::A_TILE;
 
@@ -374,6 +432,120 @@ void hgemm_pipe_kernel(const uint16_t* __restrict__ A, const uint16_t* __restric
     pipe::run_tiles<H16Op<BF16>, 4, 4, PF>(smem_h, cm, next_tile, epi);
 }
 
+/* ---- interleaved operands, loaded straight into LDS and MFMA registers
+ * (gemm_pipe2.h): four waves stacked along M, wave tile 64 x 256. acc[t][u] is
+ * the transposed 32 x 32 tile of rows m0 + 64 wave + 32 t + lane%32, columns
+ * n0 + 32 u + 8 v + 4 (lane/32) + 0..3 in registers 4v .. 4v+3. A batch of
+ * products is one launch: a tile's batch index is its operand plane. */
+template <bool BF16>
+__device__ __forceinline__ void store_tile_direct(v16f_t (&acc)[pipe2::TM][pipe2::TN], int m0, int n0, int M, int N,
+                                                  int out_mode, void* Cout) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int li = lane & 31, lh = lane >> 5;
+#pragma unroll
+    for (int t = 0; t < pipe2::TM; t++) {
+        const int row = m0 + wave * 64 + t * 32 + li;
+#pragma unroll
+        for (int u = 0; u < pipe2::TN; u++) {
+            asm volatile("" : "+a"(acc[t][u]));          /* keep the tile in the accumulator file until here */
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int col = n0 + u * 32 + 8 * v + 4 * lh;
+                float f[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    float x = acc[t][u][4 * v + e];
+                    if (out_mode == 2) x = round16<BF16>(x);
+                    f[e] = x;
+                }
+                if (row < M) {
+                    if (out_mode == 0) {
+                        float* p = (float*)Cout + (size_t)row * N + col;
+                        if ((N & 3) == 0 && col + 3 < N) *(v4f_t*)p = (v4f_t){f[0], f[1], f[2], f[3]};
+                        else for (int e = 0; e < 4; e++) if (col + e < N) p[e] = f[e];
+                    } else {
+                        double* p = (double*)Cout + (size_t)row * N + col;
+                        if ((N & 1) == 0 && col + 3 < N) {
+                            *(d2_t*)p = (d2_t){(double)f[0], (double)f[1]};
+                            *(d2_t*)(p + 2) = (d2_t){(double)f[2], (double)f[3]};
+                        } else {
+                            for (int e = 0; e < 4; e++) if (col + e < N) p[e] = (double)f[e];
+                        }
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
+}
+
+template <bool BF16>
+__global__ __launch_bounds__(256, 1)
+void hgemm_direct_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ Bt,
+                         int M, int N, int ld_bytes, int out_mode, void* __restrict__ Cout,
+                         int tiles_m, int tiles_n, int n_ids, uint64_t a_stride, uint64_t b_stride, int batch) {
+    extern __shared__ __align__(16) int8_t smem_h[];
+    pipe::Source cm;
+    cm.a_planes = (const int8_t*)A; cm.b_planes = (const int8_t*)Bt;
+    cm.a_plane_stride = a_stride; cm.b_plane_stride = b_stride;
+    cm.ld = ld_bytes;
+
+    const int per_matrix = tiles_m * tiles_n;
+    const int per_xcd = n_ids >> 3;                  /* XCD x owns tile numbers [x * per_xcd, (x + 1) * per_xcd) */
+    int next_id = (int)blockIdx.x;
+    auto next_tile = [&](pipe::Tile& t) -> bool {
+        while (next_id < n_ids) {
+            const int id = next_id;
+            next_id += (int)gridDim.x;
+            const int L = (id & 7) * per_xcd + (id >> 3);
+            const int b = L / per_matrix, in_matrix = L - b * per_matrix;
+            if (b >= batch) continue;                /* padding ids of the last XCD */
+            const int GM = 8;
+            const int width = GM * tiles_n;
+            const int group = in_matrix / width;
+            const int first_m = group * GM;
+            const int gsize = (tiles_m - first_m < GM) ? tiles_m - first_m : GM;
+            const int in_group = in_matrix - group * width;
+            t.m0 = (first_m + in_group % gsize) * 256;
+            t.n0 = (in_group / gsize) * 256;
+            t.tag = b; t.a_idx = nullptr; t.b_idx = nullptr; t.npairs = 1;
+            t.a_plane0 = b; t.b_plane0 = b;
+            return true;
+        }
+        return false;
+    };
+    const uint64_t c_bytes = (uint64_t)M * (uint64_t)N * (out_mode == 0 ? 4u : 8u);
+    auto epi = [&](v16f_t (&acc)[pipe2::TM][pipe2::TN], const pipe::Tile& t, int8_t*) {
+        store_tile_direct<BF16>(acc, t.m0, t.n0, M, N, out_mode, (int8_t*)Cout + (uint64_t)t.tag * c_bytes);
+    };
+    pipe2::run_tiles<H16Op<BF16>>(smem_h, cm, next_tile, epi);
+}
+
+template <bool BF16>
+int launch_direct(const uint16_t* A, const uint16_t* Bt, int M, int N, int ld_bytes, int out_mode, void* C,
+                  int batch, uint64_t a_stride, uint64_t b_stride, hipStream_t st) {
+    constexpr int SMEM = pipe2::SMEM_BYTES;
+    static bool attr_set = false;
+    static int num_cus = 0;
+    auto kern = hgemm_direct_kernel<BF16>;
+    if (!attr_set) {
+        if (!ESHKOL_HIP_OK(hipFuncSetAttribute((const void*)kern,
+                hipFuncAttributeMaxDynamicSharedMemorySize, SMEM))) return -1;
+        num_cus = eshkol_hip_num_cus();
+        attr_set = true;
+    }
+    const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
+    const long long total = (long long)tiles_m * tiles_n * batch;
+    if (total > 0x7ffffff0LL) return -1;
+    const int n_ids = (int)((total + 7) / 8 * 8);            /* padded so every XCD owns the same count */
+    int grid = (num_cus / 8) * 8;
+    if (grid < 8) grid = 8;
+    if (grid > n_ids) grid = n_ids;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), SMEM, st,
+                       A, Bt, M, N, ld_bytes, out_mode, C, tiles_m, tiles_n, n_ids, a_stride, b_stride, batch);
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
 template <bool BF16>
 int launch_pipe(const uint16_t* A, const uint16_t* Bt, int M, int N, int ld_bytes, int out_mode, void* C,
                 hipStream_t st) {
@@ -402,7 +574,7 @@ int launch_pipe(const uint16_t* A, const uint16_t* Bt, int M, int N, int ld_byte
 
 template <bool BF16, int TM, int TN>
 int launch(const uint16_t* A, const uint16_t* Bt, int M, int N, int ld_bytes, int out_mode, void* C,
-           hipStream_t st) {
+           int batch, uint64_t a_stride, uint64_t b_stride, hipStream_t st) {
     using Cf = Cfg<TM, TN>;
     static bool attr_set = false;
     auto kern = hgemm_kernel<BF16, TM, TN>;
@@ -414,94 +586,175 @@ int launch(const uint16_t* A, const uint16_t* Bt, int M, int N, int ld_bytes, in
     const int tiles_m = (M + Cf::BM - 1) / Cf::BM, tiles_n = (N + Cf::BN - 1) / Cf::BN;
     const long long nwg = (long long)tiles_m * tiles_n;
     if (nwg > 0x7fffffffLL) return -1;
-    hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(256), Cf::SMEM_BYTES, st,
-                       A, Bt, M, N, ld_bytes, out_mode, C, tiles_m, tiles_n);
+    /* the batch rides on the grid's y axis, at most 65535 products per launch */
+    const uint64_t c_bytes = (uint64_t)M * (uint64_t)N * (out_mode == 0 ? 4u : 8u);
+    for (int b0 = 0; b0 < batch; b0 += 65535) {
+        const int nb = (batch - b0 < 65535) ? batch - b0 : 65535;
+        hipLaunchKernelGGL(kern, dim3((unsigned)nwg, (unsigned)nb), dim3(256), Cf::SMEM_BYTES, st,
+                           (const uint16_t*)((const int8_t*)A + (uint64_t)b0 * a_stride),
+                           (const uint16_t*)((const int8_t*)Bt + (uint64_t)b0 * b_stride),
+                           M, N, ld_bytes, out_mode, (void*)((int8_t*)C + (uint64_t)b0 * c_bytes),
+                           tiles_m, tiles_n, a_stride, b_stride);
+    }
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 
-int hgemm_any(const uint16_t* A, const uint16_t* Bt, uint64_t M, uint64_t K, uint64_t N, uint64_t ld,
-              int is_bf16, int out_mode, void* C, hipStream_t st) {
-    if (!A || !Bt || !C || M == 0 || K == 0 || N == 0) return -1;
-    if (M > 0x7fffffffULL || N > 0x7fffffffULL || ld < K || ld % 64 != 0 || ld * 2 > 0x7fffffffULL) return -1;
+/* batch products stored back to back: A [batch][rows_a][ld], Bt [batch][rows_b][ld]
+ * (rows_a, rows_b the padded row counts), C [batch][M][N]. */
+int hgemm_any(const uint16_t* A, const uint16_t* Bt, uint64_t batch, uint64_t M, uint64_t K, uint64_t N,
+              uint64_t rows_a, uint64_t rows_b, uint64_t ld,
+              int is_bf16, int layout, int out_mode, void* C, hipStream_t st) {
+    if (!A || !Bt || !C || M == 0 || K == 0 || N == 0 || batch == 0) return -1;
+    if (M > 0x7fffffffULL || N > 0x7fffffffULL || batch > 0x7fffffffULL) return -1;
+    if (ld < K || ld % 64 != 0 || ld * 2 > 0x7fffffffULL) return -1;
+    if (rows_a < M || rows_b < N || rows_a % 256 != 0 || rows_b % 256 != 0) return -1;
     if (((uintptr_t)A & 15) || ((uintptr_t)Bt & 15)) return -1;
-    const int m = (int)M, n = (int)N, ldb = (int)(ld * 2);
+    const int m = (int)M, n = (int)N, ldb = (int)(ld * 2), nb = (int)batch;
+    const uint64_t a_stride = rows_a * ld * 2, b_stride = rows_b * ld * 2;
+    if (layout == 1) {
+        /* interleaved operands: whole groups of four 128-byte k-blocks */
+        if (ldb % 512 != 0) return -1;
+        return is_bf16 ? launch_direct<true>(A, Bt, m, n, ldb, out_mode, C, nb, a_stride, b_stride, st)
+                       : launch_direct<false>(A, Bt, m, n, ldb, out_mode, C, nb, a_stride, b_stride, st);
+    }
+    if (layout != 0) return -1;
     const long long big = (long long)((M + 255) / 256) * ((N + 255) / 256);
     /* the pipelined kernel wants whole pairs of 128-byte k-blocks and more than two per tile */
-    if (big >= 128 && ldb % 256 == 0 && ldb >= 512)
+    if (batch == 1 && big >= 128 && ldb % 256 == 0 && ldb >= 512)
         return is_bf16 ? launch_pipe<true>(A, Bt, m, n, ldb, out_mode, C, st)
                        : launch_pipe<false>(A, Bt, m, n, ldb, out_mode, C, st);
-    if (big >= 256)
-        return is_bf16 ? launch<true, 4, 4>(A, Bt, m, n, ldb, out_mode, C, st)
-                       : launch<false, 4, 4>(A, Bt, m, n, ldb, out_mode, C, st);
-    return is_bf16 ? launch<true, 2, 2>(A, Bt, m, n, ldb, out_mode, C, st)
-                   : launch<false, 2, 2>(A, Bt, m, n, ldb, out_mode, C, st);
+    if (big * (long long)batch >= 256 && M >= 192 && N >= 192)
+        return is_bf16 ? launch<true, 4, 4>(A, Bt, m, n, ldb, out_mode, C, nb, a_stride, b_stride, st)
+                       : launch<false, 4, 4>(A, Bt, m, n, ldb, out_mode, C, nb, a_stride, b_stride, st);
+    return is_bf16 ? launch<true, 2, 2>(A, Bt, m, n, ldb, out_mode, C, nb, a_stride, b_stride, st)
+                   : launch<false, 2, 2>(A, Bt, m, n, ldb, out_mode, C, nb, a_stride, b_stride, st);
 }
 
 }  // namespace
 
 namespace {
-int convert_any(const double* in, uint16_t* out, uint64_t rows, uint64_t cols,
-                uint64_t rows_padded, uint64_t ld, int is_bf16, bool kmajor, void* stream) {
-    if (!in || !out || rows == 0 || cols == 0 || rows_padded < rows || ld < cols || (ld & 1)) return -1;
-    const uint64_t nblk = kmajor ? kmaj::grid_blocks(rows_padded, ld, eshkol_hip_num_cus()) : ((ld / 2 + 255) / 256) * rows_padded;
+int g_direct16 = 1;
+
+int convert_any(const double* in, uint16_t* out, uint64_t batch, uint64_t rows, uint64_t cols,
+                uint64_t rows_padded, uint64_t ld, int is_bf16, bool kmajor, int layout, void* stream) {
+    if (!in || !out || rows == 0 || cols == 0 || batch == 0 || rows_padded < rows || ld < cols || (ld & 1)) return -1;
+    if (layout != 0 && layout != 1) return -1;
+    if (layout == 1 && ((rows_padded & 31) || (ld & 63) || ((uintptr_t)out & 15))) return -1;
+    const uint64_t nblk = kmajor ? kmaj::grid_blocks(rows_padded, ld, eshkol_hip_num_cus())
+                        : layout ? (rows_padded / 32) * (ld / 64) : ((ld / 2 + 255) / 256) * rows_padded;
     if (nblk > 0x7fffffffULL || (kmajor && kmaj::tile_count(rows_padded, ld) > 0x7fffffffULL)) return -1;
     hipStream_t st = (hipStream_t)stream;
-    const dim3 grid((unsigned)nblk), block(256);
-    if (kmajor) {
-        if (is_bf16) hipLaunchKernelGGL(convert_kmajor_kernel<true>, grid, block, 0, st, in, rows, cols, out, rows_padded, ld);
-        else         hipLaunchKernelGGL(convert_kmajor_kernel<false>, grid, block, 0, st, in, rows, cols, out, rows_padded, ld);
-    } else {
-        if (is_bf16) hipLaunchKernelGGL(convert_kernel<true>, grid, block, 0, st, in, rows, cols, out, rows_padded, ld);
-        else         hipLaunchKernelGGL(convert_kernel<false>, grid, block, 0, st, in, rows, cols, out, rows_padded, ld);
+    for (uint64_t b0 = 0; b0 < batch; b0 += 65535) {
+        const uint64_t nb = (batch - b0 < 65535) ? batch - b0 : 65535;
+        const double* x = in + b0 * rows * cols;
+        uint16_t* o = out + b0 * rows_padded * ld;
+        const dim3 grid((unsigned)nblk, (unsigned)nb), block(256);
+        if (kmajor) {
+            if (is_bf16) hipLaunchKernelGGL(convert_kmajor_kernel<true>, grid, block, 0, st, x, rows, cols, o, rows_padded, ld, layout);
+            else         hipLaunchKernelGGL(convert_kmajor_kernel<false>, grid, block, 0, st, x, rows, cols, o, rows_padded, ld, layout);
+        } else if (layout == 1) {
+            if (is_bf16) hipLaunchKernelGGL(convert_il_kernel<true>, grid, block, 0, st, x, rows, cols, o, rows_padded, ld);
+            else         hipLaunchKernelGGL(convert_il_kernel<false>, grid, block, 0, st, x, rows, cols, o, rows_padded, ld);
+        } else {
+            if (is_bf16) hipLaunchKernelGGL(convert_kernel<true>, grid, block, 0, st, x, rows, cols, o, rows_padded, ld);
+            else         hipLaunchKernelGGL(convert_kernel<false>, grid, block, 0, st, x, rows, cols, o, rows_padded, ld);
+        }
     }
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
+
+/* Padded operand shape and plane layout of the reduced tier for a batch of
+ * M x K x N products: interleaved 16-bit operands (and a k pitch of whole
+ * 512-byte groups) when the launch has enough 256 x 256 tiles for the
+ * direct-to-LDS kernel and the matrices are not much smaller than a tile. */
+struct ReducedShape { uint64_t Mp, Np, ld; int layout; };
+ReducedShape reduced_shape(uint64_t batch, uint64_t M, uint64_t K, uint64_t N) {
+    ReducedShape r;
+    r.Mp = round_up_sz(M, 256); r.Np = round_up_sz(N, 256);
+    r.layout = hip_hgemm_plane_layout(M, N, batch);
+    r.ld = round_up_sz(K, r.layout ? 256 : 128);
+    return r;
+}
+
+/* Narrow both operands into the 16-bit copies A16 [batch][Mp][ld] and B16
+ * [batch][Np][ld] the caller provides (every element of both, padding included,
+ * is written), then multiply. One stored k-major (B as given, A when the caller
+ * holds A^T) is narrowed through LDS tiles, so no transposed fp64 copy is made. */
+int reduced_pipeline(const double* A, const double* B, double* C, uint64_t batch, uint64_t M, uint64_t K, uint64_t N,
+                     int trans_a, int trans_b, int is_bf16, int round_output,
+                     uint16_t* A16, uint16_t* B16, const ReducedShape& sh, hipStream_t st) {
+    if (convert_any(A, A16, batch, M, K, sh.Mp, sh.ld, is_bf16, trans_a != 0, sh.layout, st) != 0) return -1;
+    if (convert_any(B, B16, batch, N, K, sh.Np, sh.ld, is_bf16, trans_b == 0, sh.layout, st) != 0) return -1;
+    return hgemm_any(A16, B16, batch, M, K, N, sh.Mp, sh.Np, sh.ld, is_bf16, sh.layout, round_output ? 2 : 1, C, st);
+}
 }  // namespace
+
+/* Tuning hook: 0 keeps the 16-bit tier on row-major operands and the
+ * register-staged kernels. Same results. */
+extern "C" void hip_hgemm_set_direct(int on) { g_direct16 = on ? 1 : 0; }
+
+extern "C" int hip_hgemm_plane_layout(uint64_t M, uint64_t N, uint64_t batch) {
+    const uint64_t tiles = ((M + 255) / 256) * ((N + 255) / 256) * batch;
+    return (g_direct16 && tiles >= 128 && M >= 192 && N >= 192) ? 1 : 0;
+}
 
 extern "C" int hip_convert_f64_to_16(const double* in, uint16_t* out, uint64_t rows, uint64_t cols,
                                      uint64_t rows_padded, uint64_t ld, int is_bf16, void* stream) {
-    return convert_any(in, out, rows, cols, rows_padded, ld, is_bf16, false, stream);
+    return convert_any(in, out, 1, rows, cols, rows_padded, ld, is_bf16, false, 0, stream);
 }
 
 extern "C" int hip_convert_f64_to_16_kmajor(const double* in, uint16_t* out, uint64_t rows, uint64_t cols,
                                             uint64_t rows_padded, uint64_t ld, int is_bf16, void* stream) {
-    return convert_any(in, out, rows, cols, rows_padded, ld, is_bf16, true, stream);
+    return convert_any(in, out, 1, rows, cols, rows_padded, ld, is_bf16, true, 0, stream);
+}
+
+extern "C" int hip_convert_f64_to_16_planes(const double* in, uint16_t* out, uint64_t batch, uint64_t rows, uint64_t cols,
+                                            uint64_t rows_padded, uint64_t ld, int is_bf16,
+                                            int kmajor, int layout, void* stream) {
+    return convert_any(in, out, batch, rows, cols, rows_padded, ld, is_bf16, kmajor != 0, layout, stream);
 }
 
 extern "C" int hip_hgemm_16(const uint16_t* A, const uint16_t* Bt, uint64_t M, uint64_t K, uint64_t N,
                             uint64_t ld, int is_bf16, float* C, void* stream) {
     EshkolHipCall bracket(stream);
-    return hgemm_any(A, Bt, M, K, N, ld, is_bf16, 0, C, (hipStream_t)stream);
+    return hgemm_any(A, Bt, 1, M, K, N, round_up_sz(M, 256), round_up_sz(N, 256), ld, is_bf16, 0, 0, C, (hipStream_t)stream);
 }
 
-namespace {
-/* Narrow both operands into the 16-bit copies A16 [Mp][ld] and B16 [Np][ld] the
- * caller provides (every element of both, padding included, is written), then
- * multiply. One stored k-major (B as given, A when the caller holds A^T) is
- * narrowed through LDS tiles, so no transposed fp64 copy is made. */
-int reduced_pipeline(const double* A, const double* B, double* C, uint64_t M, uint64_t K, uint64_t N,
-                     int trans_a, int trans_b, int is_bf16, int round_output,
-                     uint16_t* A16, uint16_t* B16, uint64_t Mp, uint64_t Np, uint64_t ld, hipStream_t st) {
-    if (convert_any(A, A16, M, K, Mp, ld, is_bf16, trans_a != 0, st) != 0) return -1;
-    if (convert_any(B, B16, N, K, Np, ld, is_bf16, trans_b == 0, st) != 0) return -1;
-    return hgemm_any(A16, B16, M, K, N, ld, is_bf16, round_output ? 2 : 1, C, st);
+extern "C" int hip_hgemm_16_batched(const uint16_t* A, const uint16_t* Bt, uint64_t batch,
+                                    uint64_t M, uint64_t K, uint64_t N,
+                                    uint64_t rows_a_padded, uint64_t rows_b_padded, uint64_t ld,
+                                    int is_bf16, int layout, float* C, void* stream) {
+    EshkolHipCall bracket(stream);
+    return hgemm_any(A, Bt, batch, M, K, N, rows_a_padded, rows_b_padded, ld, is_bf16, layout, 0, C, (hipStream_t)stream);
 }
-}  // namespace
+
+extern "C" int hip_matmul_reduced_f64_batched_ex(const double* A, const double* B, double* C,
+                                                 uint64_t batch, uint64_t M, uint64_t K, uint64_t N,
+                                                 int trans_a, int trans_b,
+                                                 int dtype, int round_output, void* stream) {
+    EshkolHipCall bracket(stream);
+    if (!A || !B || !C || M == 0 || K == 0 || N == 0 || batch == 0) return -1;
+    if (dtype != 2 && dtype != 3) return -1;
+    if (M > 0x7fffffffULL || K > 0x3fffffffULL || N > 0x7fffffffULL || batch > 0x7fffffffULL) return -1;
+    hipStream_t st = (hipStream_t)stream;
+    const ReducedShape sh = reduced_shape(batch, M, K, N);
+    uint16_t* A16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_A, batch * sh.Mp * sh.ld * 2);
+    uint16_t* B16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_B, batch * sh.Np * sh.ld * 2);
+    if (!A16 || !B16) return -1;
+    return reduced_pipeline(A, B, C, batch, M, K, N, trans_a, trans_b, dtype == 3, round_output, A16, B16, sh, st);
+}
+
+extern "C" int hip_matmul_reduced_f64_batched(const double* A, const double* B, double* C,
+                                              uint64_t batch, uint64_t M, uint64_t K, uint64_t N,
+                                              int dtype, int round_output, void* stream) {
+    return hip_matmul_reduced_f64_batched_ex(A, B, C, batch, M, K, N, 0, 0, dtype, round_output, stream);
+}
 
 extern "C" int hip_matmul_reduced_f64_ex(const double* A, const double* B, double* C,
                                          uint64_t M, uint64_t K, uint64_t N,
                                          int trans_a, int trans_b,
                                          int dtype, int round_output, void* stream) {
-    EshkolHipCall bracket(stream);
-    if (!A || !B || !C || M == 0 || K == 0 || N == 0) return -1;
-    if (dtype != 2 && dtype != 3) return -1;
-    if (M > 0x7fffffffULL || K > 0x3fffffffULL || N > 0x7fffffffULL) return -1;
-    hipStream_t st = (hipStream_t)stream;
-    const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ld = round_up_sz(K, 128);
-    uint16_t* A16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_A, Mp * ld * 2);
-    uint16_t* B16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_B, Np * ld * 2);
-    if (!A16 || !B16) return -1;
-    return reduced_pipeline(A, B, C, M, K, N, trans_a, trans_b, dtype == 3, round_output, A16, B16, Mp, Np, ld, st);
+    return hip_matmul_reduced_f64_batched_ex(A, B, C, 1, M, K, N, trans_a, trans_b, dtype, round_output, stream);
 }
 
 /* ---- the reduced tier without any allocation ------------------------------------
@@ -543,8 +796,8 @@ extern "C" int hip_matmul_reduced_f64_noalloc(const double* A, const double* B, 
     if (!A || !B || !C || M == 0 || K == 0 || N == 0) return -1;
     if (dtype != 2 && dtype != 3) return -1;
     if (M > 0x7fffffffULL || K > 0x3fffffffULL || N > 0x7fffffffULL) return -1;
-    const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ld = round_up_sz(K, 128);
-    const uint64_t a_bytes = Mp * ld * 2, b_bytes = Np * ld * 2;          /* multiples of 256 */
+    const ReducedShape sh = reduced_shape(1, M, K, N);
+    const uint64_t a_bytes = sh.Mp * sh.ld * 2, b_bytes = sh.Np * sh.ld * 2;          /* multiples of 256 */
     if (a_bytes + b_bytes > NOALLOC_SCRATCH_BYTES) {
         fprintf(stderr, "[GPU] hip_matmul_reduced_f64_noalloc: %llux%llux%llu needs %llu bytes of 16-bit "
                         "operand copies, the static scratch holds %llu; use hip_matmul_reduced_f64\n",
@@ -554,8 +807,8 @@ extern "C" int hip_matmul_reduced_f64_noalloc(const double* A, const double* B, 
     }
     unsigned char* base = noalloc_scratch();
     if (!base) return -1;
-    return reduced_pipeline(A, B, C, M, K, N, 0, 0, dtype == 3, round_output,
-                            (uint16_t*)base, (uint16_t*)(base + a_bytes), Mp, Np, ld, (hipStream_t)stream);
+    return reduced_pipeline(A, B, C, 1, M, K, N, 0, 0, dtype == 3, round_output,
+                            (uint16_t*)base, (uint16_t*)(base + a_bytes), sh, (hipStream_t)stream);
 }
 
 extern "C" int hip_matmul_reduced_f64(const double* A, const double* B, double* C,

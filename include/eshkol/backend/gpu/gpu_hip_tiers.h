@@ -311,6 +311,14 @@ int hip_matmul_reduced_f64(const double* A, const double* B, double* C,
                            uint64_t M, uint64_t K, uint64_t N,
                            int dtype, int round_output, void* stream);
 
+/* batch products stored back to back (A [batch][M][K], B [batch][K][N],
+ * C [batch][M][N]) in one launch each of the two narrowing kernels and of the
+ * contraction: the strided-batched call of the reference's 16-bit tier
+ * (cuda_batch_matmul_f16_from_f64, gpu_memory_cuda.cpp:736-784). */
+int hip_matmul_reduced_f64_batched(const double* A, const double* B, double* C,
+                                   uint64_t batch, uint64_t M, uint64_t K, uint64_t N,
+                                   int dtype, int round_output, void* stream);
+
 /* The same product as hip_matmul_reduced_f64, for callers that cannot allocate
  * device memory: code under HIP graph capture, tight serving loops, harnesses
  * that forbid hipMalloc. It has no counterpart in the reference. The 16-bit
@@ -318,7 +326,7 @@ int hip_matmul_reduced_f64(const double* A, const double* B, double* C,
  * object (hip_matmul_reduced_f64_noalloc_limit() bytes per GPU, held until the
  * process ends) instead of the grow-only workspace, and the call reaches no
  * hipMalloc, hipFree or allocating library routine. Returns -3 with a message
- * on stderr when 2 * (roundup(M,256) + roundup(N,256)) * roundup(K,128) bytes
+ * on stderr when 2 * (roundup(M,256) + roundup(N,256)) * roundup(K,256) bytes
  * exceed that limit, otherwise what hip_matmul_reduced_f64 returns, and the
  * same bits in C. Every call on a GPU shares that GPU's array: calls that
  * overlap on one GPU (two streams, two threads) race. */
@@ -333,6 +341,19 @@ size_t hip_matmul_reduced_f64_noalloc_limit(void);
 int hip_hgemm_16(const uint16_t* A, const uint16_t* Bt, uint64_t M, uint64_t K, uint64_t N,
                  uint64_t ld, int is_bf16, float* C, void* stream);
 
+/* The contraction for a batch of products whose 16-bit operands are stored back
+ * to back (A [batch][rows_a_padded][ld], Bt [batch][rows_b_padded][ld], both row
+ * counts multiples of 256), result C [batch][M][N] fp32, one launch. layout 0:
+ * operands [row][ld]. layout 1: interleaved (HipIgemmArgs.layout with k counted
+ * in bytes; needs ld to be a multiple of 256 elements), the layout
+ * hip_hgemm_plane_layout() says the tier uses when the launch has at least 128
+ * tiles of 256 x 256 and M, N >= 192. */
+int hip_hgemm_16_batched(const uint16_t* A, const uint16_t* Bt, uint64_t batch,
+                         uint64_t M, uint64_t K, uint64_t N,
+                         uint64_t rows_a_padded, uint64_t rows_b_padded, uint64_t ld,
+                         int is_bf16, int layout, float* C, void* stream);
+int hip_hgemm_plane_layout(uint64_t M, uint64_t N, uint64_t batch);
+
 /* RNE narrowing of f64 storage to f16/bf16 (runtime_tensor_dtype.cpp:37-109),
  * out[i][k] with pitch ld and rows_padded rows, padding zero. */
 int hip_convert_f64_to_16(const double* in, uint16_t* out, uint64_t rows, uint64_t cols,
@@ -341,6 +362,13 @@ int hip_convert_f64_to_16(const double* in, uint16_t* out, uint64_t rows, uint64
 /* The same narrowing from a k-major operand in[cols][rows]: out[i][k] = in[k][i]. */
 int hip_convert_f64_to_16_kmajor(const double* in, uint16_t* out, uint64_t rows, uint64_t cols,
                                  uint64_t rows_padded, uint64_t ld, int is_bf16, void* stream);
+
+/* Both narrowing kernels with batch and plane layout as arguments: `batch`
+ * matrices stored back to back, kmajor != 0 for in[cols][rows], layout as in
+ * hip_hgemm_16_batched (layout 1 needs rows_padded % 32 == 0, ld % 64 == 0). */
+int hip_convert_f64_to_16_planes(const double* in, uint16_t* out, uint64_t batch, uint64_t rows, uint64_t cols,
+                                 uint64_t rows_padded, uint64_t ld, int is_bf16,
+                                 int kmajor, int layout, void* stream);
 
 /* ---- operands held transposed, and the backward pass ---------------------------
  * The tier pipelines with the trans_a / trans_b meaning of hip_dgemm_f64_ex.
@@ -404,6 +432,9 @@ void hip_igemm_set_prefetch(int pf);
  * 0: row-major planes and the register-staged kernels everywhere. Same results;
  * the switch exists to compare them. */
 void hip_igemm_set_direct(int on);
+
+/* The same switch for the 16-bit tier. */
+void hip_hgemm_set_direct(int on);
 
 /* 1 (default): the pipelined int8 kernel runs as one workgroup per CU walking a
  * list of tiles, its operand stream continuous across tile boundaries; 0: one

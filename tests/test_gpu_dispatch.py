@@ -408,6 +408,26 @@ def test_batched_native_kernel(gpu):
     assert lib.hip_dgemm_f64_batched(da.ptr, db.ptr, dc.ptr, 0, M, K, N, st) == -1
 
 
+def test_batched_dispatch_of_16_bit_tensors_is_one_launch(gpu):
+    """eshkol_batch_matmul_dispatch with dtype 2 / 3 (gpu_memory_cuda.cpp:736-784: one strided
+    launch for all experts): many small experts from host memory, against the reference's reduced
+    statement per matrix, with the dispatcher's own log line as evidence of the single launch."""
+    body = r"""
+batch, M, K, N = 64, 128, 256, 128
+a = synth.normal(1, (batch, M, K), 1.0 / np.sqrt(K)); b = synth.normal(2, (batch, K, N), 1.0 / np.sqrt(K))
+for dtype in (2, 3):
+    ar, br = oracle.reduce_precision(a, dtype), oracle.reduce_precision(b, dtype)
+    c = np.full((batch, M, N), np.nan)
+    lib.eshkol_batch_matmul_dispatch(ar.ctypes.data, br.ctypes.data, c.ctypes.data, batch, M, K, N, dtype)
+    for i in range(batch):
+        assert normwise(c[i], oracle.matmul_f64(ar[i], br[i]), ar[i], br[i]) <= 1e-2, (dtype, i)
+assert rt.oracle_hostrt_batch_calls() == 0
+"""
+    r = run_child(body, {"ESHKOL_GPU_VERBOSE": "1"})
+    assert r.stderr.count("reduced tier (f16 in, fp32 accumulate), one strided launch") == 1
+    assert r.stderr.count("reduced tier (bf16 in, fp32 accumulate), one strided launch") == 1
+
+
 def test_resident_tensors_skip_the_upload(gpu):
     body = r"""
 lib.eshkol_gpu_set_threshold(1)

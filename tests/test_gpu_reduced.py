@@ -94,3 +94,96 @@ def test_full_size_config4_sampled(gpu):
     Ci = run_reduced(Ai, Bi, 3, round_output=False)
     assert np.array_equal(Ci.sum(axis=1), Ai @ Bi.sum(axis=1))
     assert np.array_equal(Ci[rows][:, cols], Ai[rows] @ Bi[:, cols])
+
+
+def _interleaved16(x):
+    """uint16 [rows][ld] -> the interleaved plane: rows in blocks of 32, 16-byte chunks slow, rows fast."""
+    rows, ld = x.shape
+    y = x.reshape(rows // 32, 32, ld // 8, 8).transpose(0, 2, 1, 3)
+    return np.ascontiguousarray(y).reshape(rows, ld)
+
+
+@pytest.mark.parametrize("is_bf16", [0, 1])
+@pytest.mark.parametrize("rows,cols", [(1, 1), (37, 150), (300, 70), (513, 1000), (1024, 1024)])
+def test_interleaved_narrowing_holds_the_same_values(gpu, rows, cols, is_bf16):
+    """The interleaved 16-bit planes, from either operand order and for a batch, are the
+    row-major planes element for element, padding included."""
+    lib = ea.load()
+    batch = 3
+    x = synth.normal(rows + 3 * cols, (batch, rows, cols)) * 3.0
+    rp, ld = -(-rows // 256) * 256, -(-cols // 256) * 256
+    d_in = ea.DeviceArray.from_host(x)
+    d_in_t = ea.DeviceArray.from_host(np.ascontiguousarray(x.transpose(0, 2, 1)))
+    ref = ea.DeviceArray.from_host(np.full((batch, rp, ld), 0x7878, np.uint16))
+    assert lib.hip_convert_f64_to_16_planes(d_in.ptr, ref.ptr, batch, rows, cols, rp, ld, is_bf16, 0, 0, stream()) == 0
+    ea.synchronize()
+    want = ref.download()
+    assert not want[:, rows:].any() and not want[:, :, cols:].any()
+    one = ea.DeviceArray.from_host(np.full((rp, ld), 0x7777, np.uint16))
+    assert lib.hip_convert_f64_to_16(ea.DeviceArray.from_host(x[1]).ptr, one.ptr, rows, cols, rp, ld, is_bf16, stream()) == 0
+    ea.synchronize()
+    assert np.array_equal(one.download(), want[1])
+    for kmajor, src in ((0, d_in), (1, d_in_t)):
+        for layout in (0, 1):
+            out = ea.DeviceArray.from_host(np.full((batch, rp, ld), 0x7777, np.uint16))
+            assert lib.hip_convert_f64_to_16_planes(src.ptr, out.ptr, batch, rows, cols, rp, ld, is_bf16,
+                                                    kmajor, layout, stream()) == 0
+            ea.synchronize()
+            got = out.download()
+            for b in range(batch):
+                expect = _interleaved16(want[b]) if layout else want[b]
+                assert np.array_equal(got[b], expect), (kmajor, layout, b)
+
+
+@pytest.mark.parametrize("dtype", [2, 3])
+@pytest.mark.parametrize("batch,M,K,N", [(64, 128, 256, 128), (5, 33, 70, 65), (3, 300, 129, 257), (8, 1024, 512, 1024),
+                                         (2, 2048, 300, 2304)])
+def test_batched_reduced_tier_in_one_launch(gpu, batch, M, K, N, dtype):
+    """hip_matmul_reduced_f64_batched: many small experts (the simple kernel, batch on the grid)
+    and batches that fill the device (interleaved operands, batch as the operand plane) give,
+    matrix for matrix, the bits of the single-product entry point, and meet the tier's bound
+    against the reference statement."""
+    print("batched reduced", batch, M, K, N, dtype, flush=True)
+    lib = ea.load()
+    a = synth.normal(batch + M, (batch, M, K), 1.0 / np.sqrt(K))
+    b = synth.normal(batch + N, (batch, K, N), 1.0 / np.sqrt(K))
+    da, db, dc = ea.DeviceArray.from_host(a), ea.DeviceArray.from_host(b), ea.DeviceArray((batch, M, N))
+    assert lib.hip_matmul_reduced_f64_batched(da.ptr, db.ptr, dc.ptr, batch, M, K, N, dtype, 1, stream()) == 0
+    ea.synchronize()
+    got = dc.download()
+    for i in sorted({0, 1, batch // 2, batch - 1}):
+        single = run_reduced(a[i], b[i], dtype, round_output=True)
+        ar, br = oracle.reduce_precision(a[i], dtype), oracle.reduce_precision(b[i], dtype)
+        assert normwise(got[i], oracle.matmul_f64(ar, br), ar, br) <= TOL, i
+        # fp32 sums of the same operands in a possibly different order, then rounded to 16 bits:
+        # equal up to one unit of that rounding, and exactly equal when both took the same kernel
+        assert normwise(got[i], single, ar, br) <= 1e-4, i
+    assert lib.hip_matmul_reduced_f64_batched(da.ptr, db.ptr, dc.ptr, 0, M, K, N, dtype, 1, stream()) == -1
+
+
+def test_interleaved_contraction_config4_reduced_size(gpu):
+    """bf16 operands resident in the interleaved layout, fp32 out, through hip_hgemm_16_batched:
+    the direct-to-LDS kernel against the row-major one on the same operands. Integer operands make
+    every fp32 sum exact, so the two must agree bit for bit there."""
+    lib = ea.load()
+    n = 2048
+    i = np.arange(n * n, dtype=np.int64).reshape(n, n)
+    cases = [(((i * 7 + i // n) % 7 - 3).astype(np.float64), ((i * 5 + i // n) % 5 - 2).astype(np.float64), True),
+             (synth.normal(4, (n, n), 1.0 / np.sqrt(n)), synth.normal(5, (n, n), 1.0 / np.sqrt(n)), False)]
+    for A, B, exact in cases:
+        dA, dB = ea.DeviceArray.from_host(A), ea.DeviceArray.from_host(B)
+        outs = []
+        for layout in (0, 1):
+            a16, b16 = ea.DeviceArray((n, n), np.uint16), ea.DeviceArray((n, n), np.uint16)
+            assert lib.hip_convert_f64_to_16_planes(dA.ptr, a16.ptr, 1, n, n, n, n, 1, 0, layout, stream()) == 0
+            assert lib.hip_convert_f64_to_16_planes(dB.ptr, b16.ptr, 1, n, n, n, n, 1, 1, layout, stream()) == 0
+            dC = ea.DeviceArray((n, n), np.float32)
+            assert lib.hip_hgemm_16_batched(a16.ptr, b16.ptr, 1, n, n, n, n, n, n, 1, layout, dC.ptr, stream()) == 0
+            ea.synchronize()
+            outs.append(dC.download().astype(np.float64))
+        Ar, Br = oracle.reduce_precision(A, 3), oracle.reduce_precision(B, 3)
+        ref = oracle.matmul_f64(Ar[:64], Br)
+        for o in outs:
+            assert normwise(o[:64], ref, Ar[:64], Br) <= 1e-6
+        if exact:
+            assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0][:64], ref)
