@@ -352,7 +352,16 @@ void staging_release_all(void) {
     g_staging.clear();
 }
 
-struct Resident { const void* host; size_t bytes; void* dev; };
+/* A resident tensor used as the second operand of the exact CRT tier also keeps
+ * what that tier derives from it alone (column maxima, residue planes), made on
+ * first use and dropped when the tensor is refreshed or unpinned. */
+struct Resident {
+    const void* host; size_t bytes; void* dev;
+    void* prepared = nullptr;           /* hip_ozaki_crt_prepare_operand_b handle */
+    uint64_t prep_K = 0, prep_N = 0;
+    int prep_moduli = 0;
+    bool prep_refused = false;          /* the tier would not prepare this operand: do not ask again */
+};
 std::vector<Resident> g_resident;
 
 Resident* resident_find(const void* host) {
@@ -360,9 +369,38 @@ Resident* resident_find(const void* host) {
     return nullptr;
 }
 
+Resident* resident_find_device(const void* dev) {
+    for (Resident& r : g_resident) if (r.dev == dev) return &r;
+    return nullptr;
+}
+
+void resident_drop_prepared(Resident& r) {
+    if (r.prepared) hip_ozaki_crt_release_prepared(r.prepared);
+    r.prepared = nullptr; r.prep_K = r.prep_N = 0; r.prep_moduli = 0; r.prep_refused = false;
+}
+
 void resident_release_all(void) {
-    for (Resident& r : g_resident) hipFree(r.dev);
+    for (Resident& r : g_resident) { resident_drop_prepared(r); hipFree(r.dev); }
     g_resident.clear();
+}
+
+/* The prepared form of the resident tensor at device address dB as the K x N second
+ * operand of the exact tier, made on first use; NULL if dB is not resident or the
+ * tier declines (then the call prepares nothing and splits B as always). */
+void* resident_prepared_b(const double* dB, uint64_t M, uint64_t K, uint64_t N, int moduli) {
+    Resident* r = resident_find_device(dB);
+    if (!r || r->bytes != K * N * sizeof(double)) return nullptr;
+    if (r->prepared && (r->prep_K != K || r->prep_N != N || r->prep_moduli != moduli)) resident_drop_prepared(*r);
+    if (!r->prepared && !r->prep_refused) {
+        if (hip_ozaki_crt_prepare_operand_b(dB, K, N, 0, moduli, M, &r->prepared, g_stream) == 0) {
+            r->prep_K = K; r->prep_N = N; r->prep_moduli = moduli;
+            GPU_LOG("resident operand %p: residue planes of the exact tier prepared (%llux%llu, %d moduli)",
+                    r->host, (unsigned long long)K, (unsigned long long)N, moduli);
+        } else {
+            r->prepared = nullptr; r->prep_refused = true;
+        }
+    }
+    return r->prepared;
 }
 
 int hip_wrap(void* host_ptr, size_t size_bytes, bool upload, bool copy_back, EshkolGPUBuffer* out) {
@@ -509,8 +547,13 @@ int run_tiers(const TierChoice& c, const double* dA, const double* dB, double* d
                     (unsigned long long)M, (unsigned long long)K, (unsigned long long)K,
                     (unsigned long long)N, c.why, c.crt_aligned ? ", aligned weights" : "");
             const int was = hip_ozaki_crt_set_aligned_weights(c.crt_aligned ? 1 : 0);
-            rc = hip_matmul_ozaki_crt_f64_ex(dA, dB, dC, M, K, N, ta, tb, env.num_moduli,
-                                             env.adaptive ? 1 : 0, nullptr, 0, g_stream);
+            void* prepared = (tb == 0 && !env.adaptive) ? resident_prepared_b(dB, M, K, N, env.num_moduli) : nullptr;
+            if (prepared)
+                rc = hip_matmul_ozaki_crt_prepared_f64(dA, prepared, dC, M, K, N, ta, env.num_moduli, 0,
+                                                       nullptr, 0, g_stream);
+            else
+                rc = hip_matmul_ozaki_crt_f64_ex(dA, dB, dC, M, K, N, ta, tb, env.num_moduli,
+                                                 env.adaptive ? 1 : 0, nullptr, 0, g_stream);
             hip_ozaki_crt_set_aligned_weights(was);
         } else {
             GPU_LOG("matmul %llux%llu @ %llux%llu -> INT8-Ozaki T=%d (%s, ~%.2fx vs native)",
@@ -970,6 +1013,7 @@ int eshkol_gpu_resident_pin(const void* host_ptr, size_t size_bytes) {
     if (!host_ptr || size_bytes == 0 || g_backend != ESHKOL_GPU_HIP) return -1;
     std::lock_guard<std::recursive_mutex> g(g_gpu_mutex);
     Resident* r = resident_find(host_ptr);
+    if (r) resident_drop_prepared(*r);              /* the contents are about to be uploaded again */
     if (r && r->bytes != size_bytes) {
         hipStreamSynchronize(g_stream);
         hipFree(r->dev);
@@ -983,7 +1027,7 @@ int eshkol_gpu_resident_pin(const void* host_ptr, size_t size_bytes) {
         if (!r) hipFree(d);
         return -1;
     }
-    if (!r) g_resident.push_back({host_ptr, size_bytes, d});
+    if (!r) { Resident nr; nr.host = host_ptr; nr.bytes = size_bytes; nr.dev = d; g_resident.push_back(nr); }
     return 0;
 }
 
@@ -992,6 +1036,7 @@ int eshkol_gpu_resident_refresh(const void* host_ptr) {
     std::lock_guard<std::recursive_mutex> g(g_gpu_mutex);
     Resident* r = resident_find(host_ptr);
     if (!r) return -1;
+    resident_drop_prepared(*r);
     if (eshkol_hip_upload(r->dev, host_ptr, r->bytes, g_stream) != 0 ||
         !ESHKOL_HIP_OK(hipStreamSynchronize(g_stream))) return -1;
     return 0;
@@ -1003,6 +1048,7 @@ void eshkol_gpu_resident_unpin(const void* host_ptr) {
     Resident* r = resident_find(host_ptr);
     if (!r) return;
     hipStreamSynchronize(g_stream);
+    resident_drop_prepared(*r);
     hipFree(r->dev);
     g_resident.erase(g_resident.begin() + (r - g_resident.data()));
 }

@@ -798,11 +798,30 @@ extern "C" int hip_ozaki_crt_last_stages(HipOzakiCrtStages* out) {
     return 0;
 }
 
-extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, double* C,
-                                           uint64_t M, uint64_t K, uint64_t N,
-                                           int trans_a, int trans_b,
-                                           int num_moduli, int adaptive,
-                                           const double* bias, int act, void* stream) {
+/* ---- a second operand prepared once (constant weights) ----------------------------
+ * What the tier derives from B alone: its column maxima and its residue planes.
+ * With sixteen moduli the exponent E is 52 whatever the operands are, so the
+ * planes of a B that does not change do not change either, and a layer that
+ * multiplies fresh activations by the same weights need only split the
+ * activations. The planes are the bytes the tier would compute itself, so the
+ * result is the same bit for bit. */
+namespace {
+struct CrtPreparedB {
+    uint32_t magic;
+    const double* src;          /* the operand the planes were made from */
+    uint64_t K, N, rows_padded, ldk;
+    int trans_b, n_mod, layout;
+    double* bmax;               /* [N] column maxima, device */
+    int8_t* planes;             /* [n_mod][rows_padded][ldk], device */
+};
+constexpr uint32_t PREPARED_MAGIC = 0x43525442u;
+}  // namespace
+
+static int crt_matmul_impl(const double* A, const double* B, double* C,
+                           uint64_t M, uint64_t K, uint64_t N,
+                           int trans_a, int trans_b,
+                           int num_moduli, int adaptive,
+                           const double* bias, int act, void* stream, const CrtPreparedB* prepared) {
     EshkolHipCall bracket(stream);
     if (!A || !B || !C || M == 0 || K == 0 || N == 0) return -1;
     if (M > 0x7fffffffULL || N > 0x7fffffffULL) return -1;
@@ -834,8 +853,14 @@ extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, dou
      * one stored k-major (B as given, A when the caller holds A^T) is read
      * through LDS tiles: no transposed fp64 copy is made either way. */
     const bool a_kmajor = trans_a != 0, b_kmajor = trans_b == 0;
+    /* prepared planes apply when they are what this call would compute: same
+     * operand shape, moduli, layout and pitch, and E fixed at 52 (checked below) */
+    const bool use_prepared = prepared && !adaptive && !g_force_host_pass && prepared->n_mod == num_moduli &&
+                              prepared->K == K && prepared->N == N && prepared->trans_b == trans_b &&
+                              prepared->layout == layout && prepared->ldk == ldk && prepared->rows_padded == Np &&
+                              floor((crt_constants(num_moduli).log2P - 3.0 - log2((double)K)) / 2.0) >= 52.0;
     double* amax = (double*)eshkol_hip_workspace(WS_ROWSCALE, M * sizeof(double));
-    double* bmax = (double*)eshkol_hip_workspace(WS_COLSCALE, N * sizeof(double));
+    double* bmax = use_prepared ? prepared->bmax : (double*)eshkol_hip_workspace(WS_COLSCALE, N * sizeof(double));
     int32_t* dmu = (int32_t*)eshkol_hip_workspace(WS_ROWSHIFT, M * sizeof(int32_t));
     int32_t* dnu = (int32_t*)eshkol_hip_workspace(WS_COLSHIFT, N * sizeof(int32_t));
     if (!amax || !bmax || !dmu || !dnu) return -1;
@@ -847,19 +872,20 @@ extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, dou
     int32_t* h_nu = h_mu + M;
 
     if ((a_kmajor ? hip_colabsmax_f64(A, K, M, 0.0, amax, st) : hip_rowabsmax_f64(A, M, K, 0.0, amax, st)) != 0) return -1;
-    if ((b_kmajor ? hip_colabsmax_f64(B, K, N, 0.0, bmax, st) : hip_rowabsmax_f64(B, N, K, 0.0, bmax, st)) != 0) return -1;
+    if (!use_prepared &&
+        (b_kmajor ? hip_colabsmax_f64(B, K, N, 0.0, bmax, st) : hip_rowabsmax_f64(B, N, K, 0.0, bmax, st)) != 0) return -1;
     const uint32_t ticket = scan_launch(amax, M, bmax, N, dmu, dnu, st);
     if (!ticket) return -1;
     const double log2K = log2((double)K);
 
     /* Everything after the shifts, queued in one go. */
-    auto enqueue_products = [&](int n_mod, const HostCrt& crt, int E) -> int {
+    auto enqueue_products = [&](int n_mod, const HostCrt& crt, int E, bool b_ready) -> int {
         int8_t* Ap = (int8_t*)eshkol_hip_workspace(WS_APLANES, (size_t)n_mod * Mp * ldk);
-        int8_t* Bp = (int8_t*)eshkol_hip_workspace(WS_BPLANES, (size_t)n_mod * Np * ldk);
+        int8_t* Bp = b_ready ? prepared->planes : (int8_t*)eshkol_hip_workspace(WS_BPLANES, (size_t)n_mod * Np * ldk);
         int8_t* Wp = (int8_t*)eshkol_hip_workspace(WS_PRODUCTS, (size_t)n_mod * M * N);
         if (!Ap || !Bp || !Wp) return -1;
         if (crt_split_any(A, M, K, dmu, n_mod, Ap, Mp, ldk, a_kmajor, layout, st) != 0) return -1;
-        if (crt_split_any(B, N, K, dnu, n_mod, Bp, Np, ldk, b_kmajor, layout, st) != 0) return -1;
+        if (!b_ready && crt_split_any(B, N, K, dnu, n_mod, Bp, Np, ldk, b_kmajor, layout, st) != 0) return -1;
         HipIgemmArgs ga;
         memset(&ga, 0, sizeof ga);
         ga.a_planes = Ap; ga.b_planes = Bp;
@@ -901,7 +927,7 @@ extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, dou
         if (floor((crt.log2P - 3.0 - log2K) / 2.0) >= 52.0) {
             const int E = 52;
             hipLaunchKernelGGL(crt_shift_kernel, dim3((unsigned)((M + N + 255) / 256)), dim3(256), 0, st, dmu, M, dnu, N, E);
-            if (enqueue_products(num_moduli, crt, E) != 0) return -1;
+            if (enqueue_products(num_moduli, crt, E, use_prepared) != 0) return -1;
             announce(num_moduli, crt);
             announced = true;
             h_scan = scan_await(ticket, st);
@@ -979,9 +1005,80 @@ extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, dou
     for (int o = 0; o < 2; o++)
         if (!in_range(E, any[o], e_min[o], e_max[o])) return -1;
     hipLaunchKernelGGL(crt_shift_kernel, dim3((unsigned)((M + N + 255) / 256)), dim3(256), 0, st, dmu, M, dnu, N, E);
-    if (enqueue_products(num_moduli, crt, E) != 0) return -1;
+    /* this path recomputes the shifts (libm on every maximum, or another E): the
+     * planes are split again from B itself, prepared or not */
+    if (enqueue_products(num_moduli, crt, E, false) != 0) return -1;
     if (!announced) announce(num_moduli, crt);
     return 0;
+}
+
+extern "C" int hip_matmul_ozaki_crt_f64_ex(const double* A, const double* B, double* C,
+                                           uint64_t M, uint64_t K, uint64_t N,
+                                           int trans_a, int trans_b,
+                                           int num_moduli, int adaptive,
+                                           const double* bias, int act, void* stream) {
+    return crt_matmul_impl(A, B, C, M, K, N, trans_a, trans_b, num_moduli, adaptive, bias, act, stream, nullptr);
+}
+
+extern "C" int hip_ozaki_crt_prepare_operand_b(const double* B, uint64_t K, uint64_t N, int trans_b,
+                                               int num_moduli, uint64_t M_expected, void** handle, void* stream) {
+    if (!B || !handle || K == 0 || N == 0 || K > 131071 || N > 0x7fffffffULL) return -1;
+    *handle = nullptr;
+    if (num_moduli < 2 || num_moduli > MAX_MODULI) return -1;
+    EshkolHipCall bracket(stream);
+    hipStream_t st = (hipStream_t)stream;
+    const HostCrt& crt = crt_constants(num_moduli);
+    /* only where E does not depend on the operands (gpu_memory.mm:2510-2512) */
+    if (!(floor((crt.log2P - 3.0 - log2((double)K)) / 2.0) >= 52.0)) return -1;
+    const int layout = hip_igemm_plane_layout(M_expected ? M_expected : 1, N, num_moduli);
+    const uint64_t Np = round_up_sz(N, 256), ldk = round_up_sz(K, layout ? 512 : 256);
+    const bool b_kmajor = trans_b == 0;
+    CrtPreparedB* pb = new CrtPreparedB();
+    pb->magic = PREPARED_MAGIC; pb->src = B; pb->K = K; pb->N = N; pb->rows_padded = Np; pb->ldk = ldk;
+    pb->trans_b = trans_b; pb->n_mod = num_moduli; pb->layout = layout; pb->bmax = nullptr; pb->planes = nullptr;
+    int32_t* fl = nullptr;
+    auto fail = [&]() {
+        if (pb->bmax) hipFree(pb->bmax);
+        if (pb->planes) hipFree(pb->planes);
+        if (fl) hipFree(fl);
+        delete pb;
+        return -1;
+    };
+    if (!ESHKOL_HIP_OK(hipMalloc((void**)&pb->bmax, N * sizeof(double))) ||
+        !ESHKOL_HIP_OK(hipMalloc((void**)&pb->planes, (size_t)num_moduli * Np * ldk)) ||
+        !ESHKOL_HIP_OK(hipMalloc((void**)&fl, 2 * N * sizeof(int32_t)))) { (void)hipGetLastError(); return fail(); }
+    if ((b_kmajor ? hip_colabsmax_f64(B, K, N, 0.0, pb->bmax, st) : hip_rowabsmax_f64(B, N, K, 0.0, pb->bmax, st)) != 0)
+        return fail();
+    /* the scan takes two vectors of maxima: B's stand in for both */
+    const CrtScan* h = scan_maxima(pb->bmax, N, pb->bmax, N, fl, fl + N, st);
+    if (!h || h[1].nonfinite || h[1].extreme) return fail();     /* such a B takes the full pass on every call */
+    if (h[1].nonzero && !(52 - h[1].e_min <= 1023 && 52 - h[1].e_max >= -1022)) return fail();
+    hipLaunchKernelGGL(crt_shift_kernel, dim3((unsigned)((2 * N + 255) / 256)), dim3(256), 0, st, fl, N, fl + N, N, 52);
+    if (crt_split_any(B, N, K, fl + N, num_moduli, pb->planes, Np, ldk, b_kmajor, layout, st) != 0) return fail();
+    if (!ESHKOL_HIP_OK(hipStreamSynchronize(st))) return fail();
+    hipFree(fl);
+    *handle = pb;
+    return 0;
+}
+
+extern "C" void hip_ozaki_crt_release_prepared(void* handle) {
+    CrtPreparedB* pb = (CrtPreparedB*)handle;
+    if (!pb || pb->magic != PREPARED_MAGIC) return;
+    EshkolHipCall bracket(nullptr);
+    (void)hipDeviceSynchronize();
+    hipFree(pb->bmax);
+    hipFree(pb->planes);
+    pb->magic = 0;
+    delete pb;
+}
+
+extern "C" int hip_matmul_ozaki_crt_prepared_f64(const double* A, const void* prepared_b, double* C,
+                                                 uint64_t M, uint64_t K, uint64_t N, int trans_a,
+                                                 int num_moduli, int adaptive,
+                                                 const double* bias, int act, void* stream) {
+    const CrtPreparedB* pb = (const CrtPreparedB*)prepared_b;
+    if (!pb || pb->magic != PREPARED_MAGIC || pb->K != K || pb->N != N) return -1;
+    return crt_matmul_impl(A, pb->src, C, M, K, N, trans_a, pb->trans_b, num_moduli, adaptive, bias, act, stream, pb);
 }
 
 extern "C" int hip_matmul_ozaki_crt_f64(const double* A, const double* B, double* C,

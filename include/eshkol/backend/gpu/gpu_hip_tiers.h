@@ -192,6 +192,30 @@ int hip_matmul_ozaki_crt_f64(const double* A, const double* B, double* C,
                              int num_moduli, int adaptive,
                              const double* bias, int act, void* stream);
 
+/* A second operand that does not change between calls (a layer's weights),
+ * prepared once: the tier keeps what it derives from B alone (column maxima,
+ * residue planes: num_moduli * roundup(N,256) * roundup(K,512) bytes of device
+ * memory) in *handle, and hip_matmul_ozaki_crt_prepared_f64 then splits only A.
+ * No counterpart in the reference, which re-wraps and re-splits every operand
+ * on every call (gpu_memory_cuda.cpp:1136-1145, gpu_memory.mm:2538-2583). The
+ * result is the one hip_matmul_ozaki_crt_f64_ex gives on the same operands, bit
+ * for bit: the planes are the same bytes. Prepared only where the exponent E
+ * does not depend on the operands (sixteen moduli at every K the tier accepts;
+ * -1 otherwise, and for a B with non-finite entries or a column maximum within
+ * 2^-40 of a power of two). M_expected is the row count of the products to
+ * come: it selects the plane layout (hip_igemm_plane_layout); a call whose
+ * shape wants the other layout, or adaptive != 0, simply splits B again. B
+ * must stay valid and unchanged while the handle lives; eshkol_gpu_resident_pin
+ * tensors get this treatment by themselves when the dispatcher routes a product
+ * to this tier. */
+int hip_ozaki_crt_prepare_operand_b(const double* B, uint64_t K, uint64_t N, int trans_b,
+                                    int num_moduli, uint64_t M_expected, void** handle, void* stream);
+int hip_matmul_ozaki_crt_prepared_f64(const double* A, const void* prepared_b, double* C,
+                                      uint64_t M, uint64_t K, uint64_t N, int trans_a,
+                                      int num_moduli, int adaptive,
+                                      const double* bias, int act, void* stream);
+void hip_ozaki_crt_release_prepared(void* handle);
+
 /* How the CRT weights s_l = (P / p_l) q_l are split into the two doubles the
  * accumulation uses. 0 (default): as the reference does (gpu_memory.mm:322-337),
  * each relative to its own exponent; results equal the reference's bit for bit,

@@ -466,6 +466,33 @@ lib.eshkol_gpu_shutdown()
     run_child(body)
 
 
+def test_resident_weights_keep_their_residue_planes(gpu):
+    """A pinned weight matrix used as the second operand of the exact tier is split once:
+    later products (fresh activations) reuse its planes and give the bits of the unpinned
+    path; eshkol_gpu_resident_refresh drops them, so changed weights are split again."""
+    body = r"""
+M, K, N = 1024, 1024, 1536
+W = synth.xavier_uniform(5, K, N)
+want = {}
+for seed in (1, 2):
+    X = synth.normal(seed, (M, K))
+    want[seed] = ea.matmul_dispatch(X, W)                       # nothing pinned: W is split on every call
+    assert np.array_equal(want[seed], oracle.matmul_ozaki_crt(X, W))
+assert lib.eshkol_gpu_resident_pin(W.ctypes.data, W.nbytes) == 0
+for rep in range(2):
+    for seed in (1, 2):
+        assert np.array_equal(ea.matmul_dispatch(synth.normal(seed, (M, K)), W), want[seed])
+W[17, :] *= 3.0                                                 # the host tensor changes ...
+assert lib.eshkol_gpu_resident_refresh(W.ctypes.data) == 0      # ... and the runtime says so
+X = synth.normal(1, (M, K))
+assert np.array_equal(ea.matmul_dispatch(X, W), oracle.matmul_ozaki_crt(X, W))
+lib.eshkol_gpu_resident_unpin(W.ctypes.data)
+assert np.array_equal(ea.matmul_dispatch(X, W), oracle.matmul_ozaki_crt(X, W))
+"""
+    r = run_child(body, {"ESHKOL_HIP_F64_KERNEL": "ozaki-crt", "ESHKOL_GPU_THRESHOLD": "1", "ESHKOL_GPU_VERBOSE": "1"})
+    assert r.stderr.count("residue planes of the exact tier prepared") == 2      # once after pin, once after refresh
+
+
 def test_threshold_env_forces_gpu(gpu):
     body = r"""
 A = synth.normal(1, (8, 8)); B = np.eye(8)

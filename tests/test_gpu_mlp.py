@@ -52,3 +52,57 @@ def test_mlp_config5_full_size_sampled(gpu):
         assert np.abs(got[rows][:, cols] - want).max() <= ATOL
         assert np.all(np.abs(got) <= 1.0)
         h = got
+
+
+@pytest.mark.parametrize("batch,dims", [(128, [512, 640, 512]), (2048, [1024, 2048, 1024])])
+def test_prepared_weights_give_the_same_bits(gpu, batch, dims):
+    """Weights prepared once (hip_ozaki_crt_prepare_operand_b: their column maxima and residue
+    planes kept between calls) against the ordinary entry point that splits them on every call:
+    the planes are the same bytes, so every activation must be identical, for fresh inputs too;
+    a call whose shape the prepared form does not fit (other layout) still gives the same result."""
+    import ctypes as C
+    lib = ea.load()
+    st = lib.eshkol_hip_get_stream()
+    layers = [(synth.xavier_uniform(30 + i, dims[i], dims[i + 1]), synth.uniform(40 + i, (dims[i + 1],), -0.05, 0.05))
+              for i in range(len(dims) - 1)]
+    dW = [ea.DeviceArray.from_host(W) for W, _ in layers]
+    dB = [ea.DeviceArray.from_host(b) for _, b in layers]
+    handles = []
+    for i, (W, _) in enumerate(layers):
+        h = C.c_void_p()
+        assert lib.hip_ozaki_crt_prepare_operand_b(dW[i].ptr, W.shape[0], W.shape[1], 0, 16, batch, C.byref(h), st) == 0
+        handles.append(h)
+
+    def run(X, prepared, rows):
+        src = ea.DeviceArray.from_host(X)
+        outs = []
+        for i, (W, _) in enumerate(layers):
+            out = ea.DeviceArray((rows, W.shape[1]))
+            if prepared:
+                rc = lib.hip_matmul_ozaki_crt_prepared_f64(src.ptr, handles[i], out.ptr, rows, W.shape[0], W.shape[1],
+                                                           0, 16, 0, dB[i].ptr, 1, st)
+            else:
+                rc = lib.hip_matmul_ozaki_crt_f64(src.ptr, dW[i].ptr, out.ptr, rows, W.shape[0], W.shape[1],
+                                                  16, 0, dB[i].ptr, 1, st)
+            assert rc == 0
+            ea.synchronize()
+            outs.append(out.download())
+            src = out
+        return outs
+
+    for seed in (1, 2):
+        X = synth.normal(seed, (batch, dims[0]))
+        for got, want in zip(run(X, True, batch), run(X, False, batch)):
+            assert np.array_equal(got, want)
+    # 40 rows: too few tiles for the layout the planes were prepared in at the larger size
+    X = synth.normal(3, (40, dims[0]))
+    for got, want in zip(run(X, True, 40), run(X, False, 40)):
+        assert np.array_equal(got, want)
+    for h in handles:
+        lib.hip_ozaki_crt_release_prepared(h)
+    # what cannot be prepared is refused, not approximated: fewer moduli make E depend on the data
+    h = C.c_void_p()
+    assert lib.hip_ozaki_crt_prepare_operand_b(dW[0].ptr, dims[0], dims[1], 0, 12, batch, C.byref(h), st) == -1
+    bad = layers[0][0].copy(); bad[3, 4] = np.inf
+    assert lib.hip_ozaki_crt_prepare_operand_b(ea.DeviceArray.from_host(bad).ptr, dims[0], dims[1], 0, 16, batch,
+                                               C.byref(h), st) == -1
