@@ -63,7 +63,7 @@ def main():
     ap.add_argument("--size", type=int, default=8192)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-stages", action="store_true")
-    ap.add_argument("--only", default="", help="comma list of what to time besides native: crt,int8,reduced,mlp,backward,host")
+    ap.add_argument("--only", default="", help="comma list of what to time besides native: crt,int8,reduced,mlp,backward,host,sizes,c1")
     ap.add_argument("--no-accuracy", action="store_true", help="skip the extended-precision check of sampled rows")
     ap.add_argument("--pmc-probe", default="", choices=["", "dgemm", "crt", "fast", "int8", "reduced"],
                     help="run a calibration copy and three launches of one tier, for rocprofv3 --pmc")
@@ -82,7 +82,7 @@ def main():
     flops = 2.0 * M * N * K
     steps, warm = args.steps, args.warmup
     timer = ea.Timer()
-    want = set(args.only.split(",")) if args.only else {"crt", "int8", "reduced", "mlp", "backward", "host"}
+    want = set(args.only.split(",")) if args.only else {"crt", "int8", "reduced", "mlp", "backward", "host", "sizes", "c1"}
 
     if args.pmc_probe:
         # Short program for `rocprofv3 --pmc ...` runs: a 512 MiB device copy of known size
@@ -147,6 +147,18 @@ def main():
             return None
         got = dC.download()[acc_rows]
         return float(np.linalg.norm((got - ref[0]).astype(np.float64)) / ref[1])
+
+    def hbm_stage(ms, nbytes):
+        return {"ms": ms, "GBps": nbytes / (ms * 1e-3) / 1e9, "frac_of_hbm": nbytes / (ms * 1e-3) / PEAK["hbm"],
+                "algorithmic_bytes": nbytes}
+
+    class Quiet:
+        """The CRT tiers print one marker line per call on stderr, as the reference does."""
+        def __enter__(self):
+            self.null, self.saved = os.open(os.devnull, os.O_WRONLY), os.dup(2)
+            os.dup2(self.null, 2)
+        def __exit__(self, *a):
+            os.dup2(self.saved, 2); os.close(self.null); os.close(self.saved)
 
     # ---- native fp64 tier: configuration 2 ------------------------------------
     log("generating N(0,1) operands %dx%d" % (n, n))
@@ -233,11 +245,22 @@ def main():
 
         if not args.no_stages:
             nmod = 16
-            Mp, ldk = (M + 255) // 256 * 256, (K + 255) // 256 * 256
+            # the exact tier's stages on their own, on the buffers of its last call
+            with Quiet():
+                assert lib.hip_matmul_ozaki_crt_f64(dA.ptr, dB.ptr, dC.ptr, M, K, N, 16, 0, None, 0, st) == 0
+            hip.hipDeviceSynchronize()
             sg = ea.HipOzakiCrtStages()
             assert lib.hip_ozaki_crt_last_stages(C.byref(sg)) == 0
-            # split: 8*M*K read + nmod*M*K written
-            e, _ = timed(lambda: lib.hip_ozaki_crt_split_f64(dA.ptr, M, K, sg.mu, nmod, sg.a_planes, Mp, ldk, st), settle_ms=40.0)
+            Mp, Np, ldk, lay = sg.rows_a_padded, sg.rows_b_padded, sg.ldk, sg.layout
+            scratch = ea.DeviceArray((max(M, N),))
+            # maxima: 8*M*K read each (a second read of the operands: overhead, not algorithmic work of the tier)
+            ema, _ = timed(lambda: lib.hip_rowabsmax_f64(dA.ptr, M, K, 0.0, scratch.ptr, st), settle_ms=40.0)
+            emb, _ = timed(lambda: lib.hip_colabsmax_f64(dB.ptr, K, N, 0.0, scratch.ptr, st), settle_ms=40.0)
+            # split: 8*M*K read + nmod*M*K written; A row by row, B k-major through LDS tiles
+            ea_, _ = timed(lambda: lib.hip_ozaki_crt_split_planes_f64(dA.ptr, M, K, sg.mu, nmod, sg.a_planes, Mp, ldk, 0, lay, st),
+                           settle_ms=40.0)
+            eb_, _ = timed(lambda: lib.hip_ozaki_crt_split_planes_f64(dB.ptr, N, K, sg.nu, nmod, sg.b_planes, Np, ldk, 1, lay, st),
+                           settle_ms=40.0)
             split_bytes = 8.0 * M * K + nmod * M * K
             # contraction: nmod int8 GEMMs
             ga = ea.HipIgemmArgs()
@@ -245,11 +268,11 @@ def main():
                                      229, 227, 223, 217, 211, 199, 197, 193])]).astype(np.int32)
             dT = ea.DeviceArray.from_host(tables)
             ga.a_planes, ga.b_planes = sg.a_planes, sg.b_planes
-            ga.a_plane_stride, ga.b_plane_stride = Mp * ldk, sg.rows_b_padded * ldk
+            ga.a_plane_stride, ga.b_plane_stride = Mp * ldk, Np * ldk
             ga.ldk, ga.M, ga.N, ga.n_out = ldk, M, N, nmod
             ga.pair_first, ga.pair_a, ga.pair_b = dT.ptr, dT.ptr + 17 * 4, dT.ptr + 17 * 4
             ga.mode, ga.modulus, ga.out_i8 = 1, dT.ptr + 33 * 4, sg.w_planes
-            ga.max_pairs = 1
+            ga.max_pairs, ga.layout = 1, lay
             eg, _ = timed(lambda: lib.hip_igemm_i8(C.byref(ga), st), settle_ms=40.0)
             # reconstruct: nmod*M*N read + 8*M*N written
             ones = (C.c_double * 16)(*([1.0] * 16))
@@ -258,13 +281,46 @@ def main():
                           settle_ms=40.0)
             rec_bytes = float(nmod) * M * N + 8.0 * M * N
             tiers["ozaki_crt_exact_16_moduli"]["stages"] = {
-                "split_A": {"ms": e, "GBps": split_bytes / (e * 1e-3) / 1e9, "frac_of_hbm": split_bytes / (e * 1e-3) / PEAK["hbm"],
-                            "algorithmic_bytes": split_bytes},
+                "plane_layout": "interleaved" if lay else "row-major",
+                "rowmax_A": hbm_stage(ema, 8.0 * M * K), "colmax_B": hbm_stage(emb, 8.0 * K * N),
+                "split_A": hbm_stage(ea_, split_bytes), "split_B_kmajor": hbm_stage(eb_, split_bytes),
                 "int8_contraction": {"ms": eg, "TOPs": nmod * flops / (eg * 1e-3) / 1e12,
                                      "frac_of_int8_peak": nmod * flops / (eg * 1e-3) / PEAK["int8_mfma"]},
-                "reconstruct": {"ms": er, "GBps": rec_bytes / (er * 1e-3) / 1e9, "frac_of_hbm": rec_bytes / (er * 1e-3) / PEAK["hbm"],
-                                "algorithmic_bytes": rec_bytes}}
-            dT.free()
+                "reconstruct": hbm_stage(er, rec_bytes)}
+            # the same contraction on row-major planes with the register-staged kernel, for comparison
+            ga.layout = 0
+            eg0, _ = timed(lambda: lib.hip_igemm_i8(C.byref(ga), st), settle_ms=40.0)
+            tiers["ozaki_crt_exact_16_moduli"]["stages"]["int8_contraction_register_staged_kernel"] = {
+                "ms": eg0, "TOPs": nmod * flops / (eg0 * 1e-3) / 1e12,
+                "note": "same launch through the kernel that stages both operands through registers (planes read as row-major: "
+                        "timing only)"}
+
+            # the reduced-precision CRT tier's streaming stages (11 moduli)
+            with Quiet():
+                assert lib.hip_matmul_ozaki_fast_f64(dA.ptr, dB.ptr, dC.ptr, M, K, N, 11, st) == 0
+            hip.hipDeviceSynchronize()
+            fg = ea.HipOzakiFastStages()
+            assert lib.hip_ozaki_fast_last_stages(C.byref(fg)) == 0
+            nf = fg.num_moduli
+            efa, _ = timed(lambda: lib.hip_ozaki_fast_split_planes_f64(dA.ptr, M, K, fg.shift_a, nf, fg.a_planes, fg.rows_a_padded,
+                                                                      fg.ldk, 0, fg.layout, st), settle_ms=40.0)
+            efb, _ = timed(lambda: lib.hip_ozaki_fast_split_planes_f64(dB.ptr, N, K, fg.shift_b, nf, fg.b_planes, fg.rows_b_padded,
+                                                                      fg.ldk, 1, fg.layout, st), settle_ms=40.0)
+            efr, _ = timed(lambda: lib.hip_ozaki_fast_reconstruct_f64(fg.w_planes, M, N, K, nf, fg.shift_a, fg.shift_b, dC.ptr, st),
+                           settle_ms=40.0)
+            ga.n_out, ga.layout, ga.a_planes, ga.b_planes, ga.out_i8 = nf, fg.layout, fg.a_planes, fg.b_planes, fg.w_planes
+            ga.a_plane_stride, ga.b_plane_stride, ga.ldk = fg.rows_a_padded * fg.ldk, fg.rows_b_padded * fg.ldk, fg.ldk
+            tables[33:33 + 16] = list(fg.moduli)
+            tables[33:33 + 16][tables[33:33 + 16] == 0] = 1
+            dT.upload(tables)
+            efg, _ = timed(lambda: lib.hip_igemm_i8(C.byref(ga), st), settle_ms=40.0)
+            fb = 8.0 * M * K + nf * M * K
+            tiers["ozaki_crt_fast_11_moduli"]["stages"] = {
+                "split_A": hbm_stage(efa, fb), "split_B_kmajor": hbm_stage(efb, fb),
+                "int8_contraction": {"ms": efg, "TOPs": nf * flops / (efg * 1e-3) / 1e12,
+                                     "frac_of_int8_peak": nf * flops / (efg * 1e-3) / PEAK["int8_mfma"]},
+                "reconstruct": hbm_stage(efr, float(nf) * M * N + 8.0 * M * N)}
+            dT.free(); scratch.free()
         del Aw, Bw
 
     # ---- INT8 slice tier, T = 6 -----------------------------------------------------
@@ -277,6 +333,23 @@ def main():
                                          "int8_TOPs": 28 * flops / (e4 * 1e-3) / 1e12,
                                          "normwise_error_sampled_rows": sampled_error(ref_normal)}
         log("ozaki int8 T=6: %.3f ms/step %.1f GFLOP/s-eq" % (w4, flops / (w4 * 1e-3) / 1e9))
+        if not args.no_stages:
+            ig = ea.HipOzakiInt8Stages()
+            assert lib.hip_ozaki_int8_last_stages(C.byref(ig)) == 0
+            s7 = ig.s
+            esa, _ = timed(lambda: lib.hip_ozaki_slice_planes_f64(dA.ptr, M, K, ig.rmax, s7, ig.a_slices, ig.rows_a_padded, ig.ldk,
+                                                                 0, ig.layout, st), settle_ms=40.0)
+            esb, _ = timed(lambda: lib.hip_ozaki_slice_planes_f64(dB.ptr, N, K, ig.cmax, s7, ig.b_slices, ig.rows_b_padded, ig.ldk,
+                                                                 1, ig.layout, st), settle_ms=40.0)
+            wts = ea.DeviceArray.from_host(np.array([2.0 ** (-7 * (d + 2)) for d in range(ig.nbuf)]))
+            esr, _ = timed(lambda: lib.hip_ozaki_reconstruct_f64(dC.ptr, ig.products, wts.ptr, ig.nbuf, ig.rmax, ig.cmax, M, N, st),
+                           settle_ms=40.0)
+            sb = 8.0 * M * K + s7 * M * K
+            tiers["ozaki_int8_slices_T6"]["stages"] = {
+                "slice_A": hbm_stage(esa, sb), "slice_B_kmajor": hbm_stage(esb, sb),
+                "reconstruct": hbm_stage(esr, 4.0 * ig.nbuf * M * N + 8.0 * M * N),
+                "int8_contraction_ms_by_difference": e4 - esa - esb - esr}
+            wts.free()
 
     # ---- reduced tier: configuration 4 ---------------------------------------------------
     if "reduced" in want:
@@ -295,12 +368,43 @@ def main():
         assert lib.hip_convert_f64_to_16(dBt.ptr, b16.ptr, N, K, Np, ld, 1, st) == 0
         dC32 = ea.DeviceArray((M, N), np.float32)
         e6, w6 = timed(lambda: lib.hip_hgemm_16(a16.ptr, b16.ptr, M, K, N, ld, 1, dC32.ptr, st), settle_ms=40.0)
+        # the same with the bf16 operands resident in the interleaved layout the tier itself uses
+        lay16 = lib.hip_hgemm_plane_layout(M, N, 1)
+        ld2 = (K + 255) // 256 * 256
+        a16i, b16i = ea.DeviceArray((Mp, ld2), np.uint16), ea.DeviceArray((Np, ld2), np.uint16)
+        eca, _ = timed(lambda: lib.hip_convert_f64_to_16_planes(dA.ptr, a16i.ptr, 1, M, K, Mp, ld2, 1, 0, lay16, st), settle_ms=40.0)
+        ecb, _ = timed(lambda: lib.hip_convert_f64_to_16_planes(dB.ptr, b16i.ptr, 1, N, K, Np, ld2, 1, 1, lay16, st), settle_ms=40.0)
+        e6i, w6i = timed(lambda: lib.hip_hgemm_16_batched(a16i.ptr, b16i.ptr, 1, M, K, N, Mp, Np, ld2, 1, lay16, dC32.ptr, st),
+                         settle_ms=40.0)
         tiers["reduced_bf16_fp32acc"] = {
-            "f64_storage_in_out": {"ms": w5, "gflops": flops / (w5 * 1e-3) / 1e9},
-            "bf16_in_fp32_out": {"ms": w6, "gflops": flops / (w6 * 1e-3) / 1e9,
-                                 "frac_of_bf16_peak": flops / (e6 * 1e-3) / PEAK["bf16_mfma"]}}
-        log("reduced bf16: %.3f ms (f64 storage), %.3f ms (bf16 operands)" % (w5, w6))
-        for d in (a16, b16, dBt, dC32):
+            "f64_storage_in_out": {"ms": w5, "gflops": flops / (w5 * 1e-3) / 1e9,
+                                   "stages": {"narrow_A": hbm_stage(eca, 10.0 * M * K), "narrow_B_kmajor": hbm_stage(ecb, 10.0 * K * N)}},
+            "bf16_in_fp32_out": {"ms": w6i, "gflops": flops / (w6i * 1e-3) / 1e9,
+                                 "frac_of_bf16_peak": flops / (e6i * 1e-3) / PEAK["bf16_mfma"],
+                                 "operand_layout": "interleaved" if lay16 else "row-major"},
+            "bf16_in_fp32_out_row_major_operands": {"ms": w6, "gflops": flops / (w6 * 1e-3) / 1e9,
+                                                    "frac_of_bf16_peak": flops / (e6 * 1e-3) / PEAK["bf16_mfma"]}}
+        log("reduced bf16: %.3f ms (f64 storage), %.3f ms (bf16 operands interleaved), %.3f ms (row-major)" % (w5, w6i, w6))
+        for d in (a16, b16, a16i, b16i, dBt, dC32):
+            d.free()
+        # many small experts (the reference's strided-batched case): one launch per stage against a loop of calls
+        nb, em, ek, en = 64, 128, 256, 128
+        xa = ea.DeviceArray.from_host(synth.normal(63, (nb, em, ek), 1.0 / np.sqrt(ek)))
+        xb = ea.DeviceArray.from_host(synth.normal(64, (nb, ek, en), 1.0 / np.sqrt(ek)))
+        xc = ea.DeviceArray((nb, em, en))
+
+        def expert_loop():
+            for i in range(nb):
+                lib.hip_matmul_reduced_f64(xa.ptr + i * em * ek * 8, xb.ptr + i * ek * en * 8, xc.ptr + i * em * en * 8,
+                                           em, ek, en, 3, 1, st)
+            return 0
+        _, wl = timed(expert_loop, settle_ms=20.0)
+        _, wo = timed(lambda: lib.hip_matmul_reduced_f64_batched(xa.ptr, xb.ptr, xc.ptr, nb, em, ek, en, 3, 1, st), settle_ms=20.0)
+        tiers["reduced_bf16_batch_of_64_experts_128x256x128"] = {
+            "one_launch_per_stage_ms": wo, "loop_of_64_calls_ms": wl, "speedup": wl / wo,
+            "gflops": 2.0 * nb * em * ek * en / (wo * 1e-3) / 1e9}
+        log("batched reduced tier, 64 experts: %.3f ms in one launch per stage, %.3f ms as a loop" % (wo, wl))
+        for d in (xa, xb, xc):
             d.free()
         del Ar, Br
 
@@ -330,11 +434,110 @@ def main():
         finally:
             os.dup2(saved, 2)
         mlp_flops = 2.0 * batch * sum(dims[i] * dims[i + 1] for i in range(3))
+        # the same pass with the weights prepared once (their column maxima and residue planes kept)
+        handles = []
+        for i in range(3):
+            h = C.c_void_p()
+            assert lib.hip_ozaki_crt_prepare_operand_b(Ws[i].ptr, dims[i], dims[i + 1], 0, 16, batch, C.byref(h), st) == 0
+            handles.append(h)
+
+        def mlp_forward_prepared():
+            src = X
+            for i in range(3):
+                rc = lib.hip_matmul_ozaki_crt_prepared_f64(src.ptr, handles[i], acts[i].ptr, batch, dims[i], dims[i + 1],
+                                                           0, 16, 0, bs[i].ptr, 1, st)
+                if rc != 0:
+                    return rc
+                src = acts[i]
+            return 0
+        os.dup2(devnull, 2)
+        try:
+            mlp_forward(); hip.hipDeviceSynchronize()
+            plain = acts[2].download()
+            e7p, w7p = timed(mlp_forward_prepared, settle_ms=40.0)
+        finally:
+            os.dup2(saved, 2)
+        same = bool(np.array_equal(plain, acts[2].download()))
+        for h in handles:
+            lib.hip_ozaki_crt_release_prepared(h)
         tiers["mlp_forward_exact_tier_batch4096_1024_4096_4096_1024"] = {
             "ms": w7, "gflops_fp64_equiv": mlp_flops / (w7 * 1e-3) / 1e9,
-            "note": "three GEMMs, bias add + tanh fused in the reconstruct epilogue"}
-        log("mlp forward (exact tier): %.3f ms %.1f GFLOP/s-eq" % (w7, mlp_flops / (w7 * 1e-3) / 1e9))
+            "with_prepared_weights_ms": w7p, "with_prepared_weights_gflops_fp64_equiv": mlp_flops / (w7p * 1e-3) / 1e9,
+            "prepared_output_bit_identical": same,
+            "note": "three GEMMs, bias add + tanh fused in the reconstruct epilogue; prepared = the weights' column "
+                    "maxima and residue planes computed once instead of on every forward pass"}
+        log("mlp forward (exact tier): %.3f ms %.1f GFLOP/s-eq; with prepared weights %.3f ms (same bits: %s)"
+            % (w7, mlp_flops / (w7 * 1e-3) / 1e9, w7p, same))
         for d in [X] + Ws + bs + acts:
+            d.free()
+
+    # ---- smaller cubes: where each tier starts to pay (the crossover the reference documents at
+    #      gpu_memory_cuda.cpp:454-461), N(0,1) operands resident in HBM -------------------------------
+    if "sizes" in want:
+        sweep = {}
+        for m in (1024, 2048, 4096):
+            if m >= n:
+                continue
+            sa, sb_, sc = ea.DeviceArray((m, m)), ea.DeviceArray((m, m)), ea.DeviceArray((m, m))
+            sa.upload(np.ascontiguousarray(A[:m, :m])); sb_.upload(np.ascontiguousarray(B[:m, :m]))
+            f = 2.0 * m ** 3
+            en_, _ = timed(lambda: lib.hip_dgemm_f64(sa.ptr, sb_.ptr, sc.ptr, m, m, m, st), k=20, settle_ms=40.0)
+            with Quiet():
+                ec_, _ = timed(lambda: lib.hip_matmul_ozaki_crt_f64(sa.ptr, sb_.ptr, sc.ptr, m, m, m, 16, 0, None, 0, st),
+                               k=20, settle_ms=40.0)
+            sweep["%d^3" % m] = {"native_fp64_ms": en_, "native_fp64_gflops": f / (en_ * 1e-3) / 1e9,
+                                 "native_frac_of_peak": f / (en_ * 1e-3) / PEAK["fp64_mfma"],
+                                 "ozaki_crt_exact_ms": ec_, "ozaki_crt_exact_gflops_fp64_equiv": f / (ec_ * 1e-3) / 1e9,
+                                 "exact_vs_native": en_ / ec_}
+            for d in (sa, sb_, sc):
+                d.free()
+        tiers["size_sweep_device_resident"] = sweep
+        log("size sweep: " + json.dumps({k: (round(v["native_fp64_gflops"]), round(v["ozaki_crt_exact_gflops_fp64_equiv"]))
+                                         for k, v in sweep.items()}))
+
+    # ---- configuration 1: 256^3, uniform[-1,1] (below the dispatcher's default element threshold, so the
+    #      runtime multiplies it on the reference's CPU path): the GPU kernel on resident operands, the
+    #      dispatcher forced onto the GPU from host memory, and the reference's CPU matmul ---------------
+    if "c1" in want:
+        m = 256
+        A1, B1 = synth.uniform(1, (m, m)), synth.uniform(2, (m, m))
+        d1a, d1b, d1c = ea.DeviceArray.from_host(A1), ea.DeviceArray.from_host(B1), ea.DeviceArray((m, m))
+        ev, _ = timed(lambda: lib.hip_dgemm_f64(d1a.ptr, d1b.ptr, d1c.ptr, m, m, m, st), k=200, w=20)
+        f1 = 2.0 * m ** 3
+        c1 = {"gpu_resident_operands": {"us": ev * 1e3, "gflops": f1 / (ev * 1e-3) / 1e9,
+                                        "frac_of_peak": f1 / (ev * 1e-3) / PEAK["fp64_mfma"]}}
+        C1 = np.empty((m, m))
+        old_thr = lib.eshkol_gpu_get_threshold()
+        lib.eshkol_gpu_set_threshold(1)
+        ts = []
+        for _ in range(30):
+            t0 = time.perf_counter()
+            lib.eshkol_matmul_dispatch(A1.ctypes.data, B1.ctypes.data, C1.ctypes.data, m, m, m, 0)
+            ts.append(time.perf_counter() - t0)
+        lib.eshkol_gpu_set_threshold(old_thr)
+        med = sorted(ts[5:])[len(ts[5:]) // 2]
+        c1["gpu_through_eshkol_matmul_dispatch_host_memory"] = {"us": med * 1e6, "gflops": f1 / med / 1e9,
+                                                                "note": "threshold lowered to send it to the GPU; with the "
+                                                                        "default threshold the runtime keeps 256^2 outputs on the CPU"}
+        if not args.no_cpu:
+            import oracle
+            dp = C.POINTER(C.c_double)
+            if os.path.exists(oracle.REF_PATH):
+                refl = C.CDLL(oracle.REF_PATH)
+                fn, kind = refl.eshkol_matmul_f64, "reference"
+            else:
+                fn, kind = oracle.lib().oracle_matmul_f64, "port"
+            fn.argtypes = [dp, dp, dp, C.c_uint64, C.c_uint64, C.c_uint64]
+            ts = []
+            for _ in range(40):
+                t0 = time.perf_counter()
+                fn(A1.ctypes.data_as(dp), B1.ctypes.data_as(dp), C1.ctypes.data_as(dp), m, m, m)
+                ts.append(time.perf_counter() - t0)
+            med = sorted(ts[5:])[len(ts[5:]) // 2]
+            c1["cpu_reference_path_one_core"] = {"us": med * 1e6, "gflops": f1 / med / 1e9, "kind": kind}
+        tiers["config1_256^3_uniform"] = c1
+        log("configuration 1 (256^3): " + json.dumps({k: round(v["us"], 1) for k, v in c1.items()}) + " us")
+        for d in (d1a, d1b, d1c):
             d.free()
 
     # ---- matmul backward (both gradients, native tier) ------------------------------------------

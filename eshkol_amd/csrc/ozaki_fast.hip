@@ -388,6 +388,38 @@ extern "C" int hip_ozaki_fast_plan(uint64_t K, int num_moduli, int32_t* E, int32
     return f.n;
 }
 
+/* The tier's two streaming stages on their own (moduli and E from the plan for K). */
+extern "C" int hip_ozaki_fast_split_planes_f64(const double* X, uint64_t rows, uint64_t K, const int32_t* shift,
+                                               int num_moduli, int8_t* planes, uint64_t rows_padded, uint64_t ldk,
+                                               int kmajor, int layout, void* stream) {
+    if (!X || !shift || !planes || rows == 0 || K == 0 || K > 131071) return -1;
+    if (rows_padded < rows || ldk < K || (ldk & 15) || ((uintptr_t)planes & 15)) return -1;
+    if (layout != 0 && layout != 1) return -1;
+    if (layout == 1 && ((rows_padded & 31) || (ldk & 31))) return -1;
+    FastPlan f;
+    if (make_plan(K, num_moduli, &f, true) != 0) return -1;
+    return split_any(X, rows, K, shift, f.table, planes, rows_padded, ldk, kmajor != 0, layout, (hipStream_t)stream);
+}
+
+extern "C" int hip_ozaki_fast_reconstruct_f64(const int8_t* w_planes, uint64_t M, uint64_t N, uint64_t K, int num_moduli,
+                                              const int32_t* shift_a, const int32_t* shift_b, double* C, void* stream) {
+    if (!w_planes || !shift_a || !shift_b || !C || M == 0 || N == 0 || K == 0 || K > 131071) return -1;
+    FastPlan f;
+    if (make_plan(K, num_moduli, &f, true) != 0) return -1;
+    const uint64_t nblk = (((N + 3) / 4 + 255) / 256) * M;
+    if (nblk > 0x7fffffffULL) return -1;
+    hipStream_t st = (hipStream_t)stream;
+    switch (f.n) {
+#define CASE(n) case n: hipLaunchKernelGGL(fast_reconstruct_kernel<n>, dim3((unsigned)nblk), dim3(256), 0, st, \
+                                           w_planes, M, N, f.limbs, ldexp(f.P, -64), shift_a, shift_b, C); break;
+        CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8) CASE(9)
+        CASE(10) CASE(11) CASE(12) CASE(13) CASE(14) CASE(15) CASE(16)
+#undef CASE
+        default: return -1;
+    }
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
 extern "C" int hip_ozaki_fast_last_stages(HipOzakiFastStages* out) {
     if (!out || !g_last.a_planes) return -1;
     *out = g_last;

@@ -271,6 +271,17 @@ typedef struct {
 } HipOzakiFastStages;
 int hip_ozaki_fast_last_stages(HipOzakiFastStages* out);
 
+/* The tier's two streaming stages on their own, with the moduli hip_ozaki_fast_plan
+ * gives for (K, num_moduli): the split of one operand into residue planes
+ * (shift[i] = E - 1 - floor(log2 max_i), 0 for an all-zero row; ldk a multiple
+ * of 16; layout as HipIgemmArgs.layout) and the fractional CRT of the product
+ * residues w_planes[l][M][N] back to fp64. */
+int hip_ozaki_fast_split_planes_f64(const double* X, uint64_t rows, uint64_t K, const int32_t* shift,
+                                    int num_moduli, int8_t* planes, uint64_t rows_padded, uint64_t ldk,
+                                    int kmajor, int layout, void* stream);
+int hip_ozaki_fast_reconstruct_f64(const int8_t* w_planes, uint64_t M, uint64_t N, uint64_t K, int num_moduli,
+                                   const int32_t* shift_a, const int32_t* shift_b, double* C, void* stream);
+
 /* What ESHKOL_MATMUL_ACCURACY=<budget> would choose for a product of this shape
  * (the selector of gpu_memory_cuda.cpp:546-566 with the two Ozaki-II tiers as
  * further candidates), without running anything; host arithmetic only. Returns
