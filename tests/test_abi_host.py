@@ -271,3 +271,26 @@ def test_accuracy_budget_selector_decisions():
         assert tier == 3 and lo <= moduli <= hi and sp > 1.3       # CRT tier with just enough of them
     assert pick(4096, 200000, 4096, 1e-15)[0] == 0                  # beyond the int32-exact contraction length
     assert pick(8192, 8192, 300, 1e-15)[0] in (0, 1)                # the CRT tiers need 512 in every dimension
+
+
+def test_plane_layout_decisions_are_host_arithmetic():
+    """Which operand layout the tiers produce for a contraction (interleaved planes for the
+    kernel that loads them straight into LDS, row-major otherwise) depends on the tile count
+    only; no device is involved in the answer."""
+    lib = ea.load()
+    assert lib.hip_igemm_plane_layout(8192, 8192, 16) == 1
+    assert lib.hip_igemm_plane_layout(1024, 1024, 16) == 1          # 4 x 4 tiles x 16 planes
+    assert lib.hip_igemm_plane_layout(1024, 1024, 7) == 0           # 112 tiles: too few
+    assert lib.hip_igemm_plane_layout(512, 512, 16) == 0
+    assert lib.hip_igemm_plane_layout(40, 4096, 16) == 1            # 16 tile columns x 16 planes
+    assert lib.hip_hgemm_plane_layout(8192, 8192, 1) == 1
+    assert lib.hip_hgemm_plane_layout(1024, 1024, 1) == 0
+    assert lib.hip_hgemm_plane_layout(1024, 1024, 8) == 1           # a batch fills the device
+    assert lib.hip_hgemm_plane_layout(128, 128, 64) == 0            # small experts: 128 x 128 tiles, batch on the grid
+    lib.hip_igemm_set_direct(0)
+    lib.hip_hgemm_set_direct(0)
+    try:
+        assert lib.hip_igemm_plane_layout(8192, 8192, 16) == 0 and lib.hip_hgemm_plane_layout(8192, 8192, 1) == 0
+    finally:
+        lib.hip_igemm_set_direct(1)
+        lib.hip_hgemm_set_direct(1)
