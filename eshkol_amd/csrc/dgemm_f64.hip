@@ -275,12 +275,17 @@ __device__ __forceinline__ void lds_only_barrier() {
  * tile in `partial` (dgemm_fixup_kernel adds the pieces up in order). */
 struct SplitArgs { int first_tile, tail, kb_per_piece; double* partial; };
 
-template <bool TA, bool TB, bool KTAIL, bool SPLIT>
-__global__ __launch_bounds__(256, 2)
+template <bool TA, bool TB, bool KTAIL, bool SPLIT, int TS = 128>
+__global__ __launch_bounds__(256, TS == 128 ? 2 : 4)
 void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ B,
                        double* __restrict__ C, int M, int N, int K,
                        int tiles_m, int tiles_n, SplitArgs sp) {
-    constexpr int BM = 128, BN = 128;
+    /* TS: edge of the block tile. 128 (wave tile 64 x 64) is the kernel of large
+     * launches; 64 (wave tile 32 x 32, four workgroups to a CU) serves launches
+     * that would leave CUs idle or half a round empty with the large tile. */
+    static_assert(TS == 128 || (TS == 64 && !SPLIT), "cut tiles are 128 x 128");
+    constexpr int BM = TS, BN = TS;
+    constexpr int TT = TS / 32;                  /* 16 x 16 MFMA tiles per wave and dimension */
     using OpA = Operand<BM, TA, true, true>;
     using OpB = Operand<BN, !TB, true, true>;
     constexpr int LDA = OpA::LD_S, LDB = OpB::LD_S;
@@ -360,30 +365,30 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
         }
     };
 
-    d4_t acc[4][4];
+    d4_t acc[TT][TT];
 #pragma unroll
-    for (int t = 0; t < 4; t++)
+    for (int t = 0; t < TT; t++)
 #pragma unroll
-        for (int u = 0; u < 4; u++) acc[t][u] = (d4_t){0.0, 0.0, 0.0, 0.0};
+        for (int u = 0; u < TT; u++) acc[t][u] = (d4_t){0.0, 0.0, 0.0, 0.0};
 
-    double af[2][4], bf[2][4];
-    const int a_off = (4 * lg) * LDA + wm * 64 + li;
-    const int b_off = (4 * lg) * LDB + wn * 64 + li;
+    double af[2][TT], bf[2][TT];
+    const int a_off = (4 * lg) * LDA + wm * (BM / 2) + li;
+    const int b_off = (4 * lg) * LDB + wn * (BN / 2) + li;
     auto ldfrag = [&](int buf, int st, auto which) {
         constexpr int W = decltype(which)::value;
         const double* ab = As + buf * OpA::TILE + a_off + st * LDA;
         const double* bb = Bs + buf * OpB::TILE + b_off + st * LDB;
 #pragma unroll
-        for (int t = 0; t < 4; t++) af[W][t] = ab[t * 16];
+        for (int t = 0; t < TT; t++) af[W][t] = ab[t * 16];
 #pragma unroll
-        for (int u = 0; u < 4; u++) bf[W][u] = bb[u * 16];
+        for (int u = 0; u < TT; u++) bf[W][u] = bb[u * 16];
     };
     auto mfma_step = [&](auto which) {
         constexpr int W = decltype(which)::value;
 #pragma unroll
-        for (int t = 0; t < 4; t++)
+        for (int t = 0; t < TT; t++)
 #pragma unroll
-            for (int u = 0; u < 4; u++)
+            for (int u = 0; u < TT; u++)
                 acc[t][u] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[W][t], bf[W][u], acc[t][u], 0, 0, 0);
     };
 
@@ -404,21 +409,27 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
         /* the block after next, clamped: requests past the end are never consumed */
         const int kb2 = (kb + 2 < kb_hi) ? kb + 2 : kb_hi - 1;
 
+        /* per step: NM MFMAs, TT fragment reads (pairs), and in step 2 the LDS writes of
+         * the next block (3 per chunk pair), in step 3 its successor's global loads */
+        constexpr int NM = TT * TT;
+        constexpr int WR_PER = 2;                  /* 64 x 64: six LDS writes behind three of the four MFMAs */
+        constexpr int GL = OpA::CHUNKS + OpB::CHUNKS;
+
         ldfrag(cur, 1, I1{});
         mfma_step(I0{});
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
+        for (int i = 0; i < NM; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (i < 4) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (i < TT) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
 
         ldfrag(cur, 2, I0{});
         mfma_step(I1{});
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
+        for (int i = 0; i < NM; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (i < 4) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (i < TT) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
 
@@ -427,10 +438,11 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
         b.sstore(Bs + (cur ^ 1) * OpB::TILE, tid);
         mfma_step(I0{});
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
+        for (int i = 0; i < NM; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (i < 4) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            if (i >= 2 && i < 14) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            if (i < TT) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (TS == 128) { if (i >= 2 && i < 14) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); }
+            else if (i >= 1) __builtin_amdgcn_sched_group_barrier(0x200, WR_PER, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
         lds_only_barrier();
@@ -439,33 +451,33 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
         gload(kb2);
         mfma_step(I1{});
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
+        for (int i = 0; i < NM; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (i < 4) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            if (i < 8) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            if (i < TT) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (i < GL) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
     }
 
-    if (SPLIT) {
+    if constexpr (SPLIT) {
         double* out = sp.partial + (size_t)blockIdx.x * (BM * BN);
 #pragma unroll
-        for (int t = 0; t < 4; t++)
+        for (int t = 0; t < TT; t++)
 #pragma unroll
-            for (int u = 0; u < 4; u++)
+            for (int u = 0; u < TT; u++)
 #pragma unroll
                 for (int r = 0; r < 4; r++)
                     out[(wm * 64 + t * 16 + 4 * r + lg) * BN + wn * 64 + u * 16 + li] = acc[t][u][r];
         return;
     }
 #pragma unroll
-    for (int t = 0; t < 4; t++)
+    for (int t = 0; t < TT; t++)
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            const int col = n0 + wn * 64 + u * 16 + li;
+        for (int u = 0; u < TT; u++) {
+            const int col = n0 + wn * (BN / 2) + u * 16 + li;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                const int row = m0 + wm * 64 + t * 16 + 4 * r + lg;
+                const int row = m0 + wm * (BM / 2) + t * 16 + 4 * r + lg;
                 if (row < M && col < N) C[(size_t)row * N + col] = acc[t][u][r];
             }
         }
@@ -604,6 +616,29 @@ int launch_fast(const double* A, const double* B, double* C, int M, int N, int K
                          : launch_fast_k<TA, TB, true>(A, B, C, M, N, K, batch, st);
 }
 
+/* The straight-line kernel with 64 x 64 tiles, every tile whole: four workgroups
+ * to a CU, four times as many tiles to spread over the device. */
+template <bool TA, bool TB, bool KTAIL>
+int launch_fast64_k(const double* A, const double* B, double* C, int M, int N, int K, int batch, hipStream_t st) {
+    constexpr int SMEM_BYTES = 2 * (Operand<64, TA, true, true>::TILE + Operand<64, !TB, true, true>::TILE)
+                               * (int)sizeof(double);
+    auto kern = dgemm_fast_kernel<TA, TB, KTAIL, false, 64>;
+    const int tiles_m = (M + 63) / 64, tiles_n = (N + 63) / 64;
+    const long long nwg = (long long)tiles_m * tiles_n;
+    if (nwg > 0x7fffffffLL || batch < 1 || batch > 65535) return -1;
+    const SplitArgs sp = {0, 1, 0, nullptr};
+    hipLaunchKernelGGL(kern, dim3((unsigned)nwg, (unsigned)batch), dim3(256), SMEM_BYTES, st,
+                       A, B, C, M, N, K, tiles_m, tiles_n, sp);
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+template <bool TA, bool TB>
+int launch_fast64(const double* A, const double* B, double* C, int M, int N, int K, int batch, hipStream_t st) {
+    return (K % BK == 0) ? launch_fast64_k<TA, TB, false>(A, B, C, M, N, K, batch, st)
+                         : launch_fast64_k<TA, TB, true>(A, B, C, M, N, K, batch, st);
+}
+
+int g_small_tile = 1;       /* 0 never, 1 where it measures faster, 2 wherever it is legal */
+
 int g_fast_path = 1;
 
 template <int BM, int BN, bool VEC, bool TA, bool TB, bool ALK, bool BLK>
@@ -636,6 +671,12 @@ int launch_shape(const double* A, const double* B, double* C, int m, int n, int 
     constexpr bool ALK = TA || !TB;
     /* 16-byte operand chunks (even pitches, aligned bases) and at least one whole k-block */
     const bool cut = g_tail_split && batch == 1 && small_launch_pieces(big_tiles, (k + BK - 1) / BK) >= 2;
+    const bool straight = g_fast_path && vec && m >= 2 && n >= 2 && k >= BK;
+    /* 64 x 64 tiles win where the large tile has to be cut along k to occupy a quarter to a
+     * third of the device (1024^3: 50 against 57 us; 1000 x 700 x 1300: 61 against 66); with fewer
+     * large tiles the cut pieces win, with more the large tile does (measured 256^3 ... 8192^3) */
+    if (straight && (g_small_tile == 2 || (g_small_tile == 1 && batch == 1 && big_tiles >= 56 && big_tiles <= 96 && k >= 512)))
+        return launch_fast64<TA, TB>(A, B, C, m, n, k, batch, st);
     if (g_fast_path && (big_tiles >= 192 || cut) && vec && m >= 2 && n >= 2 && k >= BK)
         return launch_fast<TA, TB>(A, B, C, m, n, k, batch, st);
     if (big_tiles >= 256) {
@@ -683,6 +724,9 @@ int dgemm_any(const double* A, const double* B, double* C, uint64_t M, uint64_t 
 extern "C" void hip_dgemm_set_fast_path(int on) { g_fast_path = on ? 1 : 0; }
 /* 0 keeps every tile whole (results then equal the bounds-checked kernel's bit for bit). */
 extern "C" void hip_dgemm_set_tail_split(int on) { g_tail_split = on ? 1 : 0; }
+/* 0: the straight-line kernel uses 128 x 128 tiles only; 1 (default): 64 x 64 tiles where
+ * they measure faster; 2: 64 x 64 tiles wherever the straight-line kernel applies. */
+extern "C" void hip_dgemm_set_small_tile(int mode) { if (mode >= 0 && mode <= 2) g_small_tile = mode; }
 
 extern "C" int hip_dgemm_f64_ex(const double* A, const double* B, double* C,
                                 uint64_t M, uint64_t K, uint64_t N,

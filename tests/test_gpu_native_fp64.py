@@ -194,6 +194,7 @@ def test_k_split_of_a_launch_that_does_not_fill_the_device(gpu, M, K, N):
         dX, dY = ea.DeviceArray.from_host(X), ea.DeviceArray.from_host(Y)
         outs = []
         try:
+            lib.hip_dgemm_set_small_tile(0)     # this test is about the large tiles cut along k
             for split in (0, 1, 1):
                 lib.hip_dgemm_set_tail_split(split)
                 guard = np.full((M + 2, N), np.nan)
@@ -206,7 +207,42 @@ def test_k_split_of_a_launch_that_does_not_fill_the_device(gpu, M, K, N):
                 outs.append(got[1:-1])
         finally:
             lib.hip_dgemm_set_tail_split(1)
+            lib.hip_dgemm_set_small_tile(1)
         whole, cut, again = outs
         assert np.array_equal(cut, again), (ta, tb)
         assert not np.array_equal(whole, cut), "the launch was expected to be cut along k"
         assert normwise(cut, ref, A, B) <= 1e-14 and normwise(cut, whole, A, B) <= 1e-14
+
+
+@pytest.mark.parametrize("M,K,N", [(1024, 1024, 1024), (1000, 700, 1300), (130, 4098, 258), (64, 16, 64), (2, 16, 2),
+                                   (900, 1001 * 2, 1100), (2048, 512, 2048)])
+def test_small_tile_kernel_gives_the_bits_of_the_large_one(gpu, M, K, N):
+    """The straight-line kernel with 64 x 64 tiles (launches that would otherwise be cut along k)
+    sums every output element in the same order as the 128 x 128 one: with whole tiles the two
+    must agree bit for bit, for all three operand forms, edge tiles and k-tails included, and
+    store nothing outside C."""
+    import eshkol_amd as ea
+    from gpu_util import stream
+    lib = ea.load()
+    A, B = synth.normal(M + 11 * K, (M, K)), synth.normal(K + 11 * N, (K, N))
+    forms = [(A, B, 0, 0), (A, np.ascontiguousarray(B.T), 0, 1), (np.ascontiguousarray(A.T), B, 1, 0)]
+    try:
+        lib.hip_dgemm_set_tail_split(0)
+        for X, Y, ta, tb in forms:
+            dX, dY = ea.DeviceArray.from_host(X), ea.DeviceArray.from_host(Y)
+            outs = []
+            for mode in (0, 2):
+                lib.hip_dgemm_set_small_tile(mode)
+                guard = np.full((M + 2, N), np.nan)
+                guard[0] = guard[-1] = 12345.0
+                dC = ea.DeviceArray.from_host(guard)
+                assert lib.hip_dgemm_f64_ex(dX.ptr, dY.ptr, dC.ptr + N * 8, M, K, N, ta, tb, stream()) == 0
+                ea.synchronize()
+                got = dC.download()
+                assert np.all(got[0] == 12345.0) and np.all(got[-1] == 12345.0)
+                outs.append(got[1:-1])
+            assert np.array_equal(outs[0], outs[1]), (ta, tb)
+            assert normwise(outs[1], oracle.matmul_f64(A, B), A, B) <= TOL
+    finally:
+        lib.hip_dgemm_set_tail_split(1)
+        lib.hip_dgemm_set_small_tile(1)
