@@ -158,6 +158,28 @@ void convert_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint64_t
         });
 }
 
+/* k-major X[K][rows], interleaved planes: no LDS (kmajor_tile.h); sixteen k of one
+ * row are two 16-byte chunks. */
+template <bool BF16>
+__global__ __launch_bounds__(256, 4)
+void convert_kmajor_il_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
+                              uint16_t* __restrict__ out, uint64_t rows_padded, uint64_t ld) {
+    X += (uint64_t)blockIdx.y * rows * K;
+    out += (uint64_t)blockIdx.y * rows_padded * ld;
+    uint64_t row, k;
+    kmaj::il_thread(rows_padded, &row, &k);
+    if (row >= rows_padded || k >= ld) return;
+    double x[16];
+    kmaj::load_k16(X, rows, K, row, k, x);
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+        v4i_t w;
+#pragma unroll
+        for (int e = 0; e < 4; e++) w[e] = (int)narrow_pair<BF16>(x[8 * c + 2 * e], x[8 * c + 2 * e + 1]);
+        *(v4i_t*)((int8_t*)out + eshkol_plane_offset(1, row, 2 * k + 16 * c, 2 * ld)) = w;
+    }
+}
+
 template <int TM, int TN> struct Cfg {
     static constexpr int NT = 256;
     static constexpr int BM = 2 * TM * 32;
@@ -640,7 +662,8 @@ int convert_any(const double* in, uint16_t* out, uint64_t batch, uint64_t rows, 
     if (!in || !out || rows == 0 || cols == 0 || batch == 0 || rows_padded < rows || ld < cols || (ld & 1)) return -1;
     if (layout != 0 && layout != 1) return -1;
     if (layout == 1 && ((rows_padded & 31) || (ld & 63) || ((uintptr_t)out & 15))) return -1;
-    const uint64_t nblk = kmajor ? kmaj::grid_blocks(rows_padded, ld, eshkol_hip_num_cus())
+    const uint64_t nblk = kmajor ? (layout ? kmaj::il_blocks(rows_padded, ld)
+                                           : kmaj::grid_blocks(rows_padded, ld, eshkol_hip_num_cus()))
                         : layout ? (rows_padded / 32) * (ld / 64) : ((ld / 2 + 255) / 256) * rows_padded;
     if (nblk > 0x7fffffffULL || (kmajor && kmaj::tile_count(rows_padded, ld) > 0x7fffffffULL)) return -1;
     hipStream_t st = (hipStream_t)stream;
@@ -649,7 +672,10 @@ int convert_any(const double* in, uint16_t* out, uint64_t batch, uint64_t rows, 
         const double* x = in + b0 * rows * cols;
         uint16_t* o = out + b0 * rows_padded * ld;
         const dim3 grid((unsigned)nblk, (unsigned)nb), block(256);
-        if (kmajor) {
+        if (kmajor && layout == 1) {
+            if (is_bf16) hipLaunchKernelGGL(convert_kmajor_il_kernel<true>, grid, block, 0, st, x, rows, cols, o, rows_padded, ld);
+            else         hipLaunchKernelGGL(convert_kmajor_il_kernel<false>, grid, block, 0, st, x, rows, cols, o, rows_padded, ld);
+        } else if (kmajor) {
             if (is_bf16) hipLaunchKernelGGL(convert_kmajor_kernel<true>, grid, block, 0, st, x, rows, cols, o, rows_padded, ld, layout);
             else         hipLaunchKernelGGL(convert_kmajor_kernel<false>, grid, block, 0, st, x, rows, cols, o, rows_padded, ld, layout);
         } else if (layout == 1) {

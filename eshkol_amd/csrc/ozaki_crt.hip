@@ -272,6 +272,21 @@ void crt_split_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint64
         });
 }
 
+/* k-major X[K][rows], interleaved planes: no LDS (kmajor_tile.h). */
+template <int NMOD>
+__global__ __launch_bounds__(256, 4)
+void crt_split_kmajor_il_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
+                                const int32_t* __restrict__ shift, int8_t* __restrict__ planes,
+                                uint64_t rows_padded, uint64_t ldk) {
+    uint64_t row, k;
+    kmaj::il_thread(rows_padded, &row, &k);
+    if (row >= rows_padded || k >= ldk) return;
+    double x[16];
+    kmaj::load_k16(X, rows, K, row, k, x);
+    const int sh = (row < rows) ? shift[row] : 0;
+    split_16<NMOD>(x, sh, planes + eshkol_plane_offset(1, row, k, ldk), rows_padded * ldk);
+}
+
 struct CrtConsts {
     double sl1[MAX_MODULI], sl2[MAX_MODULI];
     double P1, P2, Pinv;
@@ -667,6 +682,12 @@ bool g_force_host_pass = false;
 template <int NMOD>
 void launch_split(const double* X, uint64_t rows, uint64_t K, const int32_t* shift, int8_t* planes,
                   uint64_t rows_padded, uint64_t ldk, bool kmajor, int layout, hipStream_t st) {
+    if (kmajor && layout == 1) {
+        dim3 grid((unsigned)kmaj::il_blocks(rows_padded, ldk));
+        hipLaunchKernelGGL(crt_split_kmajor_il_kernel<NMOD>, grid, dim3(256), 0, st, X, rows, K, shift, planes,
+                           rows_padded, ldk);
+        return;
+    }
     if (kmajor) {
         dim3 grid((unsigned)kmaj::grid_blocks(rows_padded, ldk, eshkol_hip_num_cus()));
         hipLaunchKernelGGL(crt_split_kmajor_kernel<NMOD>, grid, dim3(256), 0, st, X, rows, K, shift, planes,

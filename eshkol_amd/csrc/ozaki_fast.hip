@@ -179,6 +179,33 @@ void fast_split_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint6
         });
 }
 
+/* k-major X[K][rows], interleaved planes: no LDS (kmajor_tile.h). */
+__global__ __launch_bounds__(256, 4)
+void fast_split_kmajor_il_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
+                                 const int32_t* __restrict__ shift, FastTable tbl, int8_t* __restrict__ planes,
+                                 uint64_t rows_padded, uint64_t ldk) {
+    uint64_t row, k;
+    kmaj::il_thread(rows_padded, &row, &k);
+    if (row >= rows_padded || k >= ldk) return;
+    double x[16];
+    kmaj::load_k16(X, rows, K, row, k, x);
+    const int sh = (row < rows) ? shift[row] : 0;
+    Scaled s[16];
+#pragma unroll
+    for (int e = 0; e < 16; e++) s[e] = scaled_integer<true>(x[e], sh);
+    int8_t* out = planes + eshkol_plane_offset(1, row, k, ldk);
+    const uint64_t plane_stride = rows_padded * ldk;
+#pragma unroll 1
+    for (int l = 0; l < tbl.n; l++) {
+        v4u_t w;
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+            w[g] = pack4(fast_residue(s[4 * g], tbl, l), fast_residue(s[4 * g + 1], tbl, l),
+                         fast_residue(s[4 * g + 2], tbl, l), fast_residue(s[4 * g + 3], tbl, l));
+        *(v4u_t*)(out + (uint64_t)l * plane_stride) = w;
+    }
+}
+
 /* Fractional CRT (metal_softfloat.h:4183-4246): frac(sum_l ((w_l q_l) mod p_l) / p_l),
  * centred, times P 2^(e_i + f_j - 2E). The fractions are added in 64-bit fixed
  * point, where "modulo 1" is the wrap of the integer and "centred" is reading it
@@ -356,7 +383,12 @@ HipOzakiFastStages g_last = {};
 
 int split_any(const double* X, uint64_t rows, uint64_t K, const int32_t* shift, const FastTable& tbl,
               int8_t* planes, uint64_t rows_padded, uint64_t ldk, bool kmajor, int layout, hipStream_t st) {
-    if (kmajor) {
+    if (kmajor && layout == 1) {
+        const uint64_t nblk = kmaj::il_blocks(rows_padded, ldk);
+        if (nblk > 0x7fffffffULL) return -1;
+        hipLaunchKernelGGL(fast_split_kmajor_il_kernel, dim3((unsigned)nblk), dim3(256), 0, st, X, rows, K, shift, tbl,
+                           planes, rows_padded, ldk);
+    } else if (kmajor) {
         if (kmaj::tile_count(rows_padded, ldk) > 0x7fffffffULL) return -1;
         const dim3 grid((unsigned)kmaj::grid_blocks(rows_padded, ldk, eshkol_hip_num_cus()));
         hipLaunchKernelGGL(fast_split_kmajor_kernel, grid, dim3(256), 0, st, X, rows, K, shift, tbl, planes,

@@ -138,6 +138,20 @@ void slice_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K
         });
 }
 
+/* k-major X[K][rows], interleaved planes: no LDS (kmajor_tile.h). */
+__global__ __launch_bounds__(256, 4)
+void slice_kmajor_il_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
+                            const double* __restrict__ scale, int s, int8_t* __restrict__ planes,
+                            uint64_t rows_padded, uint64_t ldk) {
+    uint64_t row, k;
+    kmaj::il_thread(rows_padded, &row, &k);
+    if (row >= rows_padded || k >= ldk) return;
+    double x[16];
+    kmaj::load_k16(X, rows, K, row, k, x);
+    const double sc = (row < rows) ? scale[row] : 1.0;
+    slice_group<16>(x, sc, s, planes + eshkol_plane_offset(1, row, k, ldk), rows_padded * ldk);
+}
+
 /* gpu_cuda_kernels.cu:728-741, COLS (2 or 4) consecutive columns per thread; the
  * wider form needs N to be a multiple of 4. The buffers of one element are read
  * four at a time so that a wave keeps several kilobytes of loads in flight. */
@@ -205,10 +219,14 @@ int slice_any(const double* X, uint64_t rows, uint64_t K, const double* scale, i
     if (layout != 0 && layout != 1) return -1;
     if (layout == 1 && ((rows_padded & 31) || (ldk & 31) || ((uintptr_t)planes & 15))) return -1;
     const int g = (ldk % 4 == 0 && ((uintptr_t)planes & 3) == 0) ? 4 : 2;
-    const uint64_t nblk = kmajor ? kmaj::grid_blocks(rows_padded, ldk, eshkol_hip_num_cus())
+    const uint64_t nblk = kmajor ? (layout ? kmaj::il_blocks(rows_padded, ldk)
+                                           : kmaj::grid_blocks(rows_padded, ldk, eshkol_hip_num_cus()))
                         : layout ? (rows_padded / 32) * (ldk / 32) : ((ldk / g + 255) / 256) * rows_padded;
     if (nblk > 0x7fffffffULL || (kmajor && kmaj::tile_count(rows_padded, ldk) > 0x7fffffffULL)) return -1;
-    if (kmajor)
+    if (kmajor && layout == 1)
+        hipLaunchKernelGGL(slice_kmajor_il_kernel, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
+                           X, rows, K, scale, s, planes, rows_padded, ldk);
+    else if (kmajor)
         hipLaunchKernelGGL(slice_kmajor_kernel, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
                            X, rows, K, scale, s, planes, rows_padded, ldk, layout);
     else if (layout == 1)

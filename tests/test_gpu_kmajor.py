@@ -192,3 +192,57 @@ def test_interleaved_slice_planes_hold_the_same_slices(gpu, K, R):
         assert lib.hip_ozaki_slice_planes_f64(src.ptr, R, K, dsc.ptr, s, out.ptr, Rp, ldk, kmajor, 1, stream()) == 0
         ea.synchronize()
         assert np.array_equal(ea.deinterleave(out.download(), 1), ref.download()), kmajor
+
+
+@pytest.mark.parametrize("K,R", [(40, 33), (97, 96), (129, 160), (500, 289)])
+def test_interleaved_planes_with_the_least_padding_the_layout_allows(gpu, K, R):
+    """Rows padded to 32 and the k pitch to 32 bytes only (64 elements for 16-bit planes): the
+    k-major kernels, whose blocks are larger than that, must stay inside the planes (sentinel
+    bytes behind the last one) and still fill the padding with zeros."""
+    lib = ea.load()
+    nmod, s = 5, 3
+    X = synth.normal(K + 17 * R, (K, R))
+    shift = (20 - np.floor(np.log2(np.abs(X).max(axis=0)))).astype(np.int32)
+    scale = np.abs(X).max(axis=0)
+    Rp, ldk = pad(R, 32), pad(K, 32)
+    dX, dXt, dsh, dsc = dev(X), dev(X.T), dev(shift, np.int32), dev(scale)
+
+    def run(planes, call_ref, call):
+        ref = ea.DeviceArray.from_host(np.full((planes, Rp, ldk), 78, np.int8))
+        assert call_ref(ref.ptr) == 0
+        for kmajor, src in ((1, dX), (0, dXt)):
+            out = ea.DeviceArray.from_host(np.full((planes + 1, Rp, ldk), 77, np.int8))
+            assert call(src.ptr, out.ptr, kmajor) == 0
+            ea.synchronize()
+            got = out.download()
+            assert np.all(got[planes] == 77), kmajor
+            assert np.array_equal(ea.deinterleave(got[:planes], 1), ref.download()), kmajor
+
+    run(nmod, lambda r: lib.hip_ozaki_crt_split_f64(dXt.ptr, R, K, dsh.ptr, nmod, r, Rp, ldk, stream()),
+        lambda x, o, km: lib.hip_ozaki_crt_split_planes_f64(x, R, K, dsh.ptr, nmod, o, Rp, ldk, km, 1, stream()))
+    run(s, lambda r: lib.hip_ozaki_slice_f64(dXt.ptr, R, K, dsc.ptr, s, r, Rp, ldk, stream()),
+        lambda x, o, km: lib.hip_ozaki_slice_planes_f64(x, R, K, dsc.ptr, s, o, Rp, ldk, km, 1, stream()))
+    ld = pad(K, 64)
+    for is_bf16 in (0, 1):
+        ref = ea.DeviceArray.from_host(np.full((Rp, ld), 7, np.uint16))
+        assert lib.hip_convert_f64_to_16(dXt.ptr, ref.ptr, R, K, Rp, ld, is_bf16, stream()) == 0
+        for kmajor, src in ((1, dX), (0, dXt)):
+            out = ea.DeviceArray.from_host(np.full((2, Rp, ld), 9, np.uint16))
+            assert lib.hip_convert_f64_to_16_planes(src.ptr, out.ptr, 1, R, K, Rp, ld, is_bf16, kmajor, 1, stream()) == 0
+            ea.synchronize()
+            got = out.download()
+            assert np.all(got[1] == 9), kmajor
+            assert np.array_equal(ea.deinterleave(got[:1], 1)[0], ref.download()), kmajor
+    # the reduced-precision CRT tier has no entry for plain row-major planes: all four forms must agree
+    nf = 8
+    got = {}
+    for kmajor, src in ((1, dX), (0, dXt)):
+        for layout in (0, 1):
+            out = ea.DeviceArray.from_host(np.full((nf + 1, Rp, ldk), 77, np.int8))
+            assert lib.hip_ozaki_fast_split_planes_f64(src.ptr, R, K, dsh.ptr, nf, out.ptr, Rp, ldk, kmajor, layout, stream()) == 0
+            ea.synchronize()
+            g = out.download()
+            assert np.all(g[nf] == 77), (kmajor, layout)
+            got[kmajor, layout] = ea.deinterleave(g[:nf], layout)
+    assert all(np.array_equal(got[0, 0], g) for g in got.values())
+    assert got[0, 0].any() and not got[0, 0][:, R:].any() and not got[0, 0][:, :, K:].any()
