@@ -1167,8 +1167,9 @@ void eshkol_batch_matmul_dispatch(const double* a, const double* b, double* c,
                                   int64_t batch, int64_t M, int64_t K, int64_t N, int32_t dtype) {
     if (g_backend == ESHKOL_GPU_NONE) eshkol_gpu_init();
     /* 16-bit tensors always take the GPU (as the reference's CUDA unit does);
-     * f64 batches take the native fp64 kernel, strided over the batch in one
-     * launch, once the whole output reaches the element threshold. */
+     * f64 batches go to the GPU once the whole output reaches the element
+     * threshold: the native fp64 kernel strided over the batch in one launch,
+     * unless the tier selection sends products of this shape elsewhere. */
     const bool reduced = (dtype == 2 || dtype == 3);
     const bool valid = a && b && c && batch > 0 && M > 0 && K > 0 && N > 0;
     if (valid && g_backend == ESHKOL_GPU_HIP &&
@@ -1191,6 +1192,23 @@ void eshkol_batch_matmul_dispatch(const double* a, const double* b, double* c,
                 rc = hip_matmul_reduced_f64_batched((const double*)ba.device_ptr, (const double*)bb.device_ptr,
                                                     (double*)bc.device_ptr, (uint64_t)batch,
                                                     (uint64_t)M, (uint64_t)K, (uint64_t)N, dtype, 1, g_stream);
+            } else if (const TierChoice choice = choose_tier((uint64_t)M, (uint64_t)K, (uint64_t)N);
+                       choice.tier != 0 || choice.fast) {
+                /* The reference's batch entry has no tier logic (gpu_memory_cuda.cpp:1165-1175).
+                 * Here a batch of products that the selector or an override sends to an
+                 * Ozaki tier takes that tier matrix by matrix (such products are large:
+                 * each fills the device by itself), queued back to back on one stream. */
+                GPU_LOG("batch matmul %lld x (%lldx%lld @ %lldx%lld) -> tier chosen per product, %lld launches of it",
+                        (long long)batch, (long long)M, (long long)K, (long long)K, (long long)N, (long long)batch);
+                const int was_quiet = eshkol_crt_quiet();
+                for (int64_t i = 0; i < batch && rc == 0; i++) {
+                    rc = run_tiers(choice, (const double*)ba.device_ptr + (size_t)i * M * K,
+                                   (const double*)bb.device_ptr + (size_t)i * K * N,
+                                   (double*)bc.device_ptr + (size_t)i * M * N,
+                                   (uint64_t)M, (uint64_t)K, (uint64_t)N, 0, 0, false);
+                    eshkol_crt_set_quiet(1);            /* one marker line per batch */
+                }
+                eshkol_crt_set_quiet(was_quiet);
             } else {
                 GPU_LOG("batch matmul %lld x (%lldx%lld @ %lldx%lld) -> native fp64 MFMA, one strided launch",
                         (long long)batch, (long long)M, (long long)K, (long long)K, (long long)N);

@@ -428,6 +428,33 @@ assert rt.oracle_hostrt_batch_calls() == 0
     assert r.stderr.count("reduced tier (bf16 in, fp32 accumulate), one strided launch") == 1
 
 
+def test_batched_f64_products_follow_the_tier_selection(gpu):
+    """A batch of f64 products that an override (or the accuracy budget) sends to an Ozaki tier
+    takes that tier matrix by matrix: the same bits as dispatching each product on its own.
+    Products too small for the tier stay on the one strided native launch."""
+    body = r"""
+lib.eshkol_gpu_set_threshold(1)
+batch, n = 3, 512
+a = synth.wide_range(1, (batch, n, n)); b = synth.wide_range(2, (batch, n, n))
+c = np.full((batch, n, n), np.nan)
+lib.eshkol_batch_matmul_dispatch(a.ctypes.data, b.ctypes.data, c.ctypes.data, batch, n, n, n, 0)
+for i in range(batch):
+    assert np.array_equal(c[i], ea.matmul_dispatch(a[i], b[i])), i
+    assert ulp_distance(c[i], oracle.matmul_ozaki_crt(a[i], b[i])).max() <= 2
+m = 96
+cs = np.full((batch, m, m), np.nan)
+sa, sb = np.ascontiguousarray(a[:, :m, :m]), np.ascontiguousarray(b[:, :m, :m])
+lib.eshkol_batch_matmul_dispatch(sa.ctypes.data, sb.ctypes.data, cs.ctypes.data, batch, m, m, m, 0)
+for i in range(batch):
+    assert normwise(cs[i], oracle.matmul_f64(sa[i], sb[i]), sa[i], sb[i]) <= 1e-14
+assert rt.oracle_hostrt_batch_calls() == 0
+"""
+    r = run_child(body, {"ESHKOL_HIP_F64_KERNEL": "ozaki-crt", "ESHKOL_GPU_VERBOSE": "1"})
+    assert r.stderr.count("tier chosen per product, 3 launches of it") == 1
+    assert r.stderr.count("native fp64 MFMA, one strided launch") == 1
+    assert r.stderr.count("[GPU] Ozaki-II: N=16") == 1 + 3          # one marker for the batch, one per single dispatch
+
+
 def test_resident_tensors_skip_the_upload(gpu):
     body = r"""
 lib.eshkol_gpu_set_threshold(1)
