@@ -58,6 +58,8 @@
 
 namespace pipe2 {
 
+typedef int v2i_t __attribute__((ext_vector_type(2)));
+
 using pipe::v4i_t;
 using pipe::IC;
 using pipe::static_for;
@@ -74,6 +76,30 @@ constexpr int RING = DEPTH * STAGE;
 constexpr int EPI_PITCH = 128 + 16;
 constexpr int EPI_WAVE_BYTES = 32 * EPI_PITCH;        /* per wave: 32 rows x 128 output bytes */
 constexpr int SMEM_BYTES = RING + 4 * EPI_WAVE_BYTES;
+
+/* A 32 x 32 block of 4-byte words on its way out of a wave. The 32x32 MFMAs
+ * leave it transposed: lane l holds row l % 32, and its registers 4v .. 4v+3 the
+ * columns 8v + 4 (l / 32) + 0..3, so a store straight from the registers would
+ * put 16 bytes into each of 64 places. park_block() writes the block into the
+ * wave's LDS stage as rows of 128 bytes (pitch EPI_PITCH: the 16-byte accesses of
+ * eight lanes, in either direction, fall into distinct banks); afterwards eight
+ * lanes read a row and a store instruction writes whole 128-byte lines. The
+ * wave's LDS accesses complete in order: its reads see its writes, and the next
+ * block's writes come after this block's reads. */
+__device__ __forceinline__ void park_block(int8_t* stage, int v, v4i_t words) {
+    const int lane = threadIdx.x & 63;
+    *(v4i_t*)(stage + (lane & 31) * EPI_PITCH + 32 * v + 16 * (lane >> 5)) = words;
+}
+/* i = 0..3: the 16 bytes of row lane/8 + 8 i, words 4 (lane % 8) .. + 3 */
+__device__ __forceinline__ v4i_t parked_row16(const int8_t* stage, int i) {
+    const int lane = threadIdx.x & 63;
+    return *(const v4i_t*)(stage + ((lane >> 3) + 8 * i) * EPI_PITCH + 16 * (lane & 7));
+}
+/* i = 0..7: the 8 bytes of row lane/16 + 4 i, words 2 (lane % 16), + 1 */
+__device__ __forceinline__ v2i_t parked_row8(const int8_t* stage, int i) {
+    const int lane = threadIdx.x & 63;
+    return *(const v2i_t*)(stage + ((lane >> 4) + 4 * i) * EPI_PITCH + 8 * (lane & 15));
+}
 constexpr int WAIT_STEADY = 36;                       /* see the issue order above */
 constexpr int WAIT_START = 3 * 16 + 8 + 6 - 16;       /* after the prologue: all but block 0's loads may be pending */
 

@@ -461,18 +461,20 @@ void hgemm_pipe_kernel(const uint16_t* __restrict__ A, const uint16_t* __restric
  * products is one launch: a tile's batch index is its operand plane. */
 template <bool BF16>
 __device__ __forceinline__ void store_tile_direct(v16f_t (&acc)[pipe2::TM][pipe2::TN], int m0, int n0, int M, int N,
-                                                  int out_mode, void* Cout) {
+                                                  int out_mode, void* Cout, int8_t* stage) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int li = lane & 31, lh = lane >> 5;
+    const bool vec_f32 = (N & 3) == 0, vec_f64 = (N & 1) == 0;
 #pragma unroll
     for (int t = 0; t < pipe2::TM; t++) {
-        const int row = m0 + wave * 64 + t * 32 + li;
+        const int row0 = m0 + wave * 64 + t * 32;
 #pragma unroll
         for (int u = 0; u < pipe2::TN; u++) {
             asm volatile("" : "+a"(acc[t][u]));          /* keep the tile in the accumulator file until here */
+            /* the block goes through the wave's LDS stage so that a store instruction
+             * writes whole lines: eight lanes a 128-byte row segment of fp32, sixteen
+             * lanes 256 bytes of fp64 */
 #pragma unroll
             for (int v = 0; v < 4; v++) {
-                const int col = n0 + u * 32 + 8 * v + 4 * lh;
                 float f[4];
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
@@ -480,23 +482,35 @@ __device__ __forceinline__ void store_tile_direct(v16f_t (&acc)[pipe2::TM][pipe2
                     if (out_mode == 2) x = round16<BF16>(x);
                     f[e] = x;
                 }
-                if (row < M) {
-                    if (out_mode == 0) {
-                        float* p = (float*)Cout + (size_t)row * N + col;
-                        if ((N & 3) == 0 && col + 3 < N) *(v4f_t*)p = (v4f_t){f[0], f[1], f[2], f[3]};
-                        else for (int e = 0; e < 4; e++) if (col + e < N) p[e] = f[e];
-                    } else {
-                        double* p = (double*)Cout + (size_t)row * N + col;
-                        if ((N & 1) == 0 && col + 3 < N) {
-                            *(d2_t*)p = (d2_t){(double)f[0], (double)f[1]};
-                            *(d2_t*)(p + 2) = (d2_t){(double)f[2], (double)f[3]};
-                        } else {
-                            for (int e = 0; e < 4; e++) if (col + e < N) p[e] = (double)f[e];
-                        }
-                    }
-                }
+                pipe2::park_block(stage, v, (v4i_t){__float_as_int(f[0]), __float_as_int(f[1]),
+                                                    __float_as_int(f[2]), __float_as_int(f[3])});
                 __builtin_amdgcn_sched_barrier(0);
             }
+            const int cb = n0 + u * 32;
+            if (out_mode == 0) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const v4i_t w = pipe2::parked_row16(stage, i);
+                    const int row = row0 + (lane >> 3) + 8 * i, col = cb + 4 * (lane & 7);
+                    if (row < M && col < N) {
+                        float* p = (float*)Cout + (size_t)row * N + col;
+                        if (vec_f32 && col + 3 < N) *(v4i_t*)p = w;
+                        else for (int e = 0; e < 4; e++) if (col + e < N) p[e] = __int_as_float(w[e]);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const pipe2::v2i_t w = pipe2::parked_row8(stage, i);
+                    const int row = row0 + (lane >> 4) + 4 * i, col = cb + 2 * (lane & 15);
+                    if (row < M && col < N) {
+                        double* p = (double*)Cout + (size_t)row * N + col;
+                        if (vec_f64 && col + 1 < N) *(d2_t*)p = (d2_t){(double)__int_as_float(w[0]), (double)__int_as_float(w[1])};
+                        else for (int e = 0; e < 2; e++) if (col + e < N) p[e] = (double)__int_as_float(w[e]);
+                    }
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
     }
 }
@@ -537,8 +551,8 @@ void hgemm_direct_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
         return false;
     };
     const uint64_t c_bytes = (uint64_t)M * (uint64_t)N * (out_mode == 0 ? 4u : 8u);
-    auto epi = [&](v16f_t (&acc)[pipe2::TM][pipe2::TN], const pipe::Tile& t, int8_t*) {
-        store_tile_direct<BF16>(acc, t.m0, t.n0, M, N, out_mode, (int8_t*)Cout + (uint64_t)t.tag * c_bytes);
+    auto epi = [&](v16f_t (&acc)[pipe2::TM][pipe2::TN], const pipe::Tile& t, int8_t* stage) {
+        store_tile_direct<BF16>(acc, t.m0, t.n0, M, N, out_mode, (int8_t*)Cout + (uint64_t)t.tag * c_bytes, stage);
     };
     pipe2::run_tiles<H16Op<BF16>>(smem_h, cm, next_tile, epi);
 }

@@ -289,23 +289,24 @@ __device__ __forceinline__ void epilogue_direct(const HipIgemmArgs& g, int o, in
 #pragma unroll
             for (int u = 0; u < TN; u++) {
                 asm volatile("" : "+a"(acc[t][u]));      /* keep the tile in the accumulator file until here */
+                /* through the wave's LDS stage, so that eight lanes write a 128-byte row segment */
 #pragma unroll
                 for (int v = 0; v < 4; v++) {
-                    const int col = n0 + u * 32 + 8 * v + 4 * lh;
-                    if (row < (int)g.M) {
-                        int32_t* p = out + (size_t)row * g.N + col;
-                        if (vec_ok && col + 3 < (int)g.N) {
-                            v4i_t w = {acc[t][u][4 * v], acc[t][u][4 * v + 1],
-                                       acc[t][u][4 * v + 2], acc[t][u][4 * v + 3]};
-                            *(v4i_t*)p = w;
-                        } else {
-#pragma unroll
-                            for (int e = 0; e < 4; e++)
-                                if (col + e < (int)g.N) p[e] = acc[t][u][4 * v + e];
-                        }
-                    }
+                    pipe2::park_block(stage, v, (v4i_t){acc[t][u][4 * v], acc[t][u][4 * v + 1],
+                                                        acc[t][u][4 * v + 2], acc[t][u][4 * v + 3]});
                     __builtin_amdgcn_sched_barrier(0);
                 }
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const v4i_t w = pipe2::parked_row16(stage, i);
+                    const int orow = row - li + (lane >> 3) + 8 * i, col = n0 + u * 32 + 4 * (lane & 7);
+                    if (orow < (int)g.M && col < (int)g.N) {
+                        int32_t* p = out + (size_t)orow * g.N + col;
+                        if (vec_ok && col + 3 < (int)g.N) *(v4i_t*)p = w;
+                        else for (int e = 0; e < 4; e++) if (col + e < (int)g.N) p[e] = w[e];
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
         return;
