@@ -673,9 +673,13 @@ int launch_shape(const double* A, const double* B, double* C, int m, int n, int 
     const bool cut = g_tail_split && batch == 1 && small_launch_pieces(big_tiles, (k + BK - 1) / BK) >= 2;
     const bool straight = g_fast_path && vec && m >= 2 && n >= 2 && k >= BK;
     /* 64 x 64 tiles win where the large tile has to be cut along k to occupy a quarter to a
-     * third of the device (1024^3: 50 against 57 us; 1000 x 700 x 1300: 61 against 66); with fewer
-     * large tiles the cut pieces win, with more the large tile does (measured 256^3 ... 8192^3) */
-    if (straight && (g_small_tile == 2 || (g_small_tile == 1 && batch == 1 && big_tiles >= 56 && big_tiles <= 96 && k >= 512)))
+     * third of the device (1024^3: 50 against 57 us; 1000 x 700 x 1300: 61 against 66), as long
+     * as k is short: one small-tile workgroup per CU sustains two thirds of the peak, the cut
+     * large tiles nine tenths but with a second launch to add them up (1024 x 1024 outputs:
+     * equal near k = 3000; 1152 x 1280: near k = 1024). With fewer large tiles the cut pieces
+     * win, with more the large tile does (measured 256^3 ... 8192^3). */
+    if (straight && (g_small_tile == 2 || (g_small_tile == 1 && batch == 1 && big_tiles >= 56 && big_tiles <= 96 &&
+                                           k >= 64 && (uint64_t)k * (uint64_t)big_tiles <= 2048u * 64u)))
         return launch_fast64<TA, TB>(A, B, C, m, n, k, batch, st);
     if (g_fast_path && (big_tiles >= 192 || cut) && vec && m >= 2 && n >= 2 && k >= BK)
         return launch_fast<TA, TB>(A, B, C, m, n, k, batch, st);

@@ -461,8 +461,8 @@ void hip_dgemm_set_tail_split(int on);
 
 /* Tile size of the straight-line fp64 kernel. 0: 128 x 128 only; 1 (default):
  * 64 x 64 tiles for the launches that measure faster with them (56 to 96 large
- * tiles, e.g. 1024^3, which would otherwise be cut along k); 2: 64 x 64 wherever
- * that kernel applies. The summation order inside a tile is the same, so all three
+ * tiles and k * tiles <= 131072, e.g. 1024^3, which would otherwise be cut along
+ * k); 2: 64 x 64 wherever that kernel applies. The summation order inside a tile is the same, so all three
  * give the same bits as long as no tile is cut along k. */
 void hip_dgemm_set_small_tile(int mode);
 
