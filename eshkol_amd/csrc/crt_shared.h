@@ -54,6 +54,15 @@ constexpr ByteWeights byte_weights(int modulus) {
     return { c[0] | c[1] << 8 | c[2] << 16 | c[3] << 24, c[4] | c[5] << 8 | c[6] << 16 | c[7] << 24 };
 }
 
+/* ---- maxima with the shifts beside them (implemented in elementwise.hip) ------------
+ * hip_rowabsmax_f64 / hip_colabsmax_f64 that also write, when shift is not null,
+ * shift[i] = E - floor(log2 max_i) (0 for a maximum of zero): what the split of a
+ * CRT tier needs when its exponent E is known before the operands are looked at. */
+int eshkol_rowabsmax_shift_f64(const double* A, uint64_t M, uint64_t K, double zero_value,
+                               double* rmax, int32_t* shift, int E, hipStream_t stream);
+int eshkol_colabsmax_shift_f64(const double* X, uint64_t K, uint64_t R, double zero_value,
+                               double* cmax, int32_t* shift, int E, hipStream_t stream);
+
 /* ---- exponents of the maxima (implemented in ozaki_crt.hip) ---------------------- */
 
 /* What the host learns about one operand's row (or column) maxima. */
@@ -64,14 +73,13 @@ struct CrtMaxima {
 };
 constexpr int32_t CRT_FL_ZERO = INT32_MIN;      /* exponent entry of a maximum of zero */
 
-/* Queues the scan: fl_a[i] = floor(log2 amax[i]) taken from the exponent field
- * (CRT_FL_ZERO for a maximum of zero), likewise fl_b. Exact unless a maximum lies
- * within 2^-40 of a power of two AND the caller needs libm's floor(log2): the
- * exact tier checks that itself. Returns the ticket of the scan's summary, 0 on
- * failure. The summary is written to host memory by the device: a caller queues
- * what depends on fl_a / fl_b right away and asks for the summary afterwards. */
-uint32_t eshkol_crt_scan_launch(const double* amax, uint64_t M, const double* bmax, uint64_t N,
-                                int32_t* fl_a, int32_t* fl_b, hipStream_t st);
+/* Queues the scan of the two vectors of maxima for its summary (a NaN or an
+ * infinity among them? the range of their exponents), on a stream of the
+ * library's own behind everything queued on st so far: what follows on st does
+ * not wait for it. The summary is written to host memory by the device; ask for
+ * it after queueing the rest of the pipeline. Returns the summary's ticket, 0 on
+ * failure. For callers whose shifts came with the maxima (above). */
+uint32_t eshkol_crt_scan_launch_aside(const double* amax, uint64_t M, const double* bmax, uint64_t N, hipStream_t st);
 /* The two CRT tiers print one marker line per call, as the reference does per
  * dispatch (gpu_memory.mm:2503; its gates count those lines). A dispatcher that
  * runs one product as several calls (row panels) lets the first call print and
@@ -81,8 +89,5 @@ int eshkol_crt_quiet(void);
 
 /* Waits for that summary and fills out[0] (A) and out[1] (B). 0 on success. */
 int eshkol_crt_scan_result(uint32_t ticket, CrtMaxima out[2], hipStream_t st);
-
-/* In place: fl -> E - fl, and 0 where fl is CRT_FL_ZERO. */
-void eshkol_crt_shifts_from_exponents(int32_t* fl_a, uint64_t M, int32_t* fl_b, uint64_t N, int E, hipStream_t st);
 
 #endif

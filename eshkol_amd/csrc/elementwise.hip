@@ -5,6 +5,7 @@
  */
 #include "hip_common.h"
 #include "kernels.h"
+#include "crt_shared.h"
 #include "tanh_f64.h"
 
 namespace {
@@ -39,9 +40,20 @@ __device__ __forceinline__ void absmax_step(double v, double* m) {
     else if (a > *m) *m = a;
 }
 
+/* E - floor(log2 m) for a maximum m > 0 (exponent field; subnormals by their
+ * leading bit), 0 for m = 0: the per-row shift of the CRT tiers when E does not
+ * depend on the operands (gpu_memory.mm:2524-2532). */
+__device__ __forceinline__ int32_t shift_of_maximum(double m, int E) {
+    if (!(m > 0.0)) return 0;
+    const unsigned long long bits = (unsigned long long)__double_as_longlong(m);
+    const int ef = (int)(bits >> 52);
+    const int e = ef ? ef - 1023 : (63 - __clzll((long long)(bits & 0xfffffffffffffull))) - 1074;
+    return E - e;
+}
+
 __global__ __launch_bounds__(256)
 void rowabsmax_f64_kernel(const double* __restrict__ A, uint64_t M, uint64_t K,
-                          double zero_value, double* __restrict__ rmax) {
+                          double zero_value, double* __restrict__ rmax, int32_t* __restrict__ shift, int E) {
     const int lane = threadIdx.x & 63;
     const uint64_t row = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= M) return;
@@ -65,7 +77,10 @@ void rowabsmax_f64_kernel(const double* __restrict__ A, uint64_t M, uint64_t K,
         double o = __shfl_xor(m, off, 64);
         if (o > m) m = o;
     }
-    if (lane == 0) rmax[row] = (m > 0.0) ? m : zero_value;
+    if (lane == 0) {
+        rmax[row] = (m > 0.0) ? m : zero_value;
+        if (shift) shift[row] = shift_of_maximum(m, E);
+    }
 }
 
 /* Column maxima of a row-major X[K][R] in two steps: a block takes 64 columns
@@ -94,7 +109,7 @@ void colabsmax_partial_kernel(const double* __restrict__ X, uint64_t K, uint64_t
 
 __global__ __launch_bounds__(256)
 void colabsmax_fold_kernel(const double* __restrict__ partial, uint64_t R, int slices,
-                           double zero_value, double* __restrict__ out) {
+                           double zero_value, double* __restrict__ out, int32_t* __restrict__ shift, int E) {
     const uint64_t col = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     if (col >= R) return;
     double m = 0.0;
@@ -108,6 +123,7 @@ void colabsmax_fold_kernel(const double* __restrict__ partial, uint64_t R, int s
     }
     for (; s < slices; s++) { const double o = partial[(uint64_t)s * R + col]; if (o > m) m = o; }
     out[col] = (m > 0.0) ? m : zero_value;
+    if (shift) shift[col] = shift_of_maximum(m, E);
 }
 
 __device__ __forceinline__ double apply_op(int op, double a, double b, bool has_b) {
@@ -210,18 +226,28 @@ extern "C" int hip_transpose_f64(const double* in, double* out, uint64_t rows, u
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 
-extern "C" int hip_rowabsmax_f64(const double* A, uint64_t M, uint64_t K, double zero_value,
-                                 double* rmax, void* stream) {
+int eshkol_rowabsmax_shift_f64(const double* A, uint64_t M, uint64_t K, double zero_value,
+                               double* rmax, int32_t* shift, int E, hipStream_t stream) {
     if (!A || !rmax || M == 0 || K == 0) return -1;
     const uint64_t g = (M + 3) / 4;
     if (g > 0x7fffffffULL) return -1;
-    hipLaunchKernelGGL(rowabsmax_f64_kernel, dim3((unsigned)g), dim3(256), 0, (hipStream_t)stream,
-                       A, M, K, zero_value, rmax);
+    hipLaunchKernelGGL(rowabsmax_f64_kernel, dim3((unsigned)g), dim3(256), 0, stream,
+                       A, M, K, zero_value, rmax, shift, E);
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
+extern "C" int hip_rowabsmax_f64(const double* A, uint64_t M, uint64_t K, double zero_value,
+                                 double* rmax, void* stream) {
+    return eshkol_rowabsmax_shift_f64(A, M, K, zero_value, rmax, nullptr, 0, (hipStream_t)stream);
 }
 
 extern "C" int hip_colabsmax_f64(const double* X, uint64_t K, uint64_t R, double zero_value,
                                  double* cmax, void* stream) {
+    return eshkol_colabsmax_shift_f64(X, K, R, zero_value, cmax, nullptr, 0, (hipStream_t)stream);
+}
+
+int eshkol_colabsmax_shift_f64(const double* X, uint64_t K, uint64_t R, double zero_value,
+                               double* cmax, int32_t* shift, int E, hipStream_t stream) {
     EshkolHipCall bracket(stream);
     if (!X || !cmax || K == 0 || R == 0) return -1;
     const uint64_t gx = (R + 63) / 64;
@@ -235,7 +261,7 @@ extern "C" int hip_colabsmax_f64(const double* X, uint64_t K, uint64_t R, double
     hipLaunchKernelGGL(colabsmax_partial_kernel, dim3((unsigned)gx, (unsigned)slices), dim3(256), 0,
                        (hipStream_t)stream, X, K, R, rows_per_slice, partial);
     hipLaunchKernelGGL(colabsmax_fold_kernel, dim3((unsigned)((R + 255) / 256)), dim3(256), 0,
-                       (hipStream_t)stream, partial, R, slices, zero_value, cmax);
+                       (hipStream_t)stream, partial, R, slices, zero_value, cmax, shift, E);
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 

@@ -449,7 +449,7 @@ void crt_scan_kernel(const double* __restrict__ amax, uint64_t M, const double* 
                 if (e > my_emax) my_emax = e;
                 if ((n != MANT_ONE && n < MANT_ONE + MANT_WINDOW) || n >= 2 * MANT_ONE - MANT_WINDOW) my_extreme = 1;
             }
-            fl[i] = f;
+            if (fl) fl[i] = f;
         }
     }
     /* fold within the wave first: a thousand atomics on one LDS word would take
@@ -618,10 +618,14 @@ void* pinned(size_t bytes) {
 CrtScan* g_mailbox = nullptr;         /* host address; [2] */
 CrtScan* g_mailbox_dev = nullptr;     /* the same memory as the device sees it */
 uint32_t g_ticket = 0;
+hipStream_t g_scan_stream = nullptr;  /* where a scan that nothing on the device waits for runs */
+hipEvent_t g_scan_event = nullptr;
 bool ensure_mailbox() {
     if (g_mailbox) return true;
     void* h = nullptr;
     void* d = nullptr;
+    if (!g_scan_stream && !ESHKOL_HIP_OK(hipStreamCreateWithFlags(&g_scan_stream, hipStreamNonBlocking))) return false;
+    if (!g_scan_event && !ESHKOL_HIP_OK(hipEventCreateWithFlags(&g_scan_event, hipEventDisableTiming))) return false;
     if (!ESHKOL_HIP_OK(hipHostMalloc(&h, 2 * sizeof(CrtScan), hipHostMallocMapped))) return false;
     if (!ESHKOL_HIP_OK(hipHostGetDevicePointer(&d, h, 0))) { (void)hipHostFree(h); return false; }
     memset(h, 0, 2 * sizeof(CrtScan));
@@ -647,20 +651,26 @@ int await_mailbox(uint32_t ticket, hipStream_t st) {
 
 /* Queues the scan of the two vectors of maxima; 0 on failure, else the ticket its
  * summary will carry. */
+hipStream_t g_scan_ran_on = nullptr;  /* the stream the last scan was queued on: what a wait drains if the ticket does not show */
 uint32_t scan_launch(const double* amax, uint64_t M, const double* bmax, uint64_t N,
                      int32_t* fl_a, int32_t* fl_b, hipStream_t st) {
     if (!ensure_mailbox()) return 0;
+    g_scan_ran_on = st;
     const uint32_t ticket = ++g_ticket ? g_ticket : ++g_ticket;            /* never 0: the mailbox starts zeroed */
     hipLaunchKernelGGL(crt_scan_kernel, dim3(2), dim3(SCAN_THREADS), 0, st, amax, M, bmax, N, fl_a, fl_b,
                        g_mailbox_dev, ticket);
     return ESHKOL_HIP_OK(hipGetLastError()) ? ticket : 0;
 }
-const CrtScan* scan_await(uint32_t ticket, hipStream_t st) {
-    return (ticket != 0 && await_mailbox(ticket, st) == 0) ? g_mailbox : nullptr;
+/* The same scan for its summary alone, on the library's side stream behind what
+ * st holds so far. */
+uint32_t scan_launch_aside(const double* amax, uint64_t M, const double* bmax, uint64_t N, hipStream_t st) {
+    if (!ensure_mailbox()) return 0;
+    if (!ESHKOL_HIP_OK(hipEventRecord(g_scan_event, st)) ||
+        !ESHKOL_HIP_OK(hipStreamWaitEvent(g_scan_stream, g_scan_event, 0))) return 0;
+    return scan_launch(amax, M, bmax, N, nullptr, nullptr, g_scan_stream);
 }
-const CrtScan* scan_maxima(const double* amax, uint64_t M, const double* bmax, uint64_t N,
-                           int32_t* fl_a, int32_t* fl_b, hipStream_t st) {
-    return scan_await(scan_launch(amax, M, bmax, N, fl_a, fl_b, st), st);
+const CrtScan* scan_await(uint32_t ticket) {
+    return (ticket != 0 && await_mailbox(ticket, g_scan_ran_on) == 0) ? g_mailbox : nullptr;
 }
 
 /* device-resident constant tables for the contraction: identity pair lists and moduli */
@@ -738,23 +748,19 @@ static int g_crt_quiet = 0;
 void eshkol_crt_set_quiet(int quiet) { g_crt_quiet = quiet; }
 int eshkol_crt_quiet(void) { return g_crt_quiet; }
 
-uint32_t eshkol_crt_scan_launch(const double* amax, uint64_t M, const double* bmax, uint64_t N,
-                                int32_t* fl_a, int32_t* fl_b, hipStream_t st) {
-    return scan_launch(amax, M, bmax, N, fl_a, fl_b, st);
+uint32_t eshkol_crt_scan_launch_aside(const double* amax, uint64_t M, const double* bmax, uint64_t N, hipStream_t st) {
+    return scan_launch_aside(amax, M, bmax, N, st);
 }
 
 int eshkol_crt_scan_result(uint32_t ticket, CrtMaxima out[2], hipStream_t st) {
-    const CrtScan* h = scan_await(ticket, st);
+    (void)st;
+    const CrtScan* h = scan_await(ticket);
     if (!h) return -1;
     for (int o = 0; o < 2; o++) {
         out[o].nonfinite = h[o].nonfinite; out[o].nonzero = h[o].nonzero;
         out[o].e_min = h[o].e_min; out[o].e_max = h[o].e_max;
     }
     return 0;
-}
-
-void eshkol_crt_shifts_from_exponents(int32_t* fl_a, uint64_t M, int32_t* fl_b, uint64_t N, int E, hipStream_t st) {
-    hipLaunchKernelGGL(crt_shift_kernel, dim3((unsigned)((M + N + 255) / 256)), dim3(256), 0, st, fl_a, M, fl_b, N, E);
 }
 
 extern "C" int hip_ozaki_crt_split_f64(const double* X, uint64_t rows, uint64_t K,
@@ -833,6 +839,7 @@ struct CrtPreparedB {
     uint64_t K, N, rows_padded, ldk;
     int trans_b, n_mod, layout;
     double* bmax;               /* [N] column maxima, device */
+    int32_t* nu;                /* [N] shifts 52 - floor(log2 max), device */
     int8_t* planes;             /* [n_mod][rows_padded][ldk], device */
 };
 constexpr uint32_t PREPARED_MAGIC = 0x43525442u;
@@ -892,15 +899,29 @@ static int crt_matmul_impl(const double* A, const double* B, double* C,
     int32_t* h_mu = (int32_t*)(h_bmax + N);
     int32_t* h_nu = h_mu + M;
 
-    if ((a_kmajor ? hip_colabsmax_f64(A, K, M, 0.0, amax, st) : hip_rowabsmax_f64(A, M, K, 0.0, amax, st)) != 0) return -1;
-    if (!use_prepared &&
-        (b_kmajor ? hip_colabsmax_f64(B, K, N, 0.0, bmax, st) : hip_rowabsmax_f64(B, N, K, 0.0, bmax, st)) != 0) return -1;
-    const uint32_t ticket = scan_launch(amax, M, bmax, N, dmu, dnu, st);
-    if (!ticket) return -1;
+    /* E = min(52, floor((log2 P - 1 - log2 K - frac_A - frac_B) / 2)) with both
+     * fractions below 1 (gpu_memory.mm:2510-2512): where even frac_A + frac_B = 2
+     * leaves 52 (16 moduli: every K this tier accepts), E does not depend on the
+     * operands. Then the kernels that find the maxima write the shifts as well, the
+     * scan of the maxima (non-finite input? shifts in range? a maximum so close to a
+     * power of two that libm's log2 may round across it?) runs beside the pipeline
+     * on a stream of its own, and nothing on the device waits for it. */
     const double log2K = log2((double)K);
+    const bool fixed_E = !adaptive && !g_force_host_pass &&
+                         floor((crt_constants(num_moduli).log2P - 3.0 - log2K) / 2.0) >= 52.0;
+    int32_t* const mu_out = fixed_E ? dmu : nullptr;
+    int32_t* const nu_out = fixed_E ? dnu : nullptr;
+    if ((a_kmajor ? eshkol_colabsmax_shift_f64(A, K, M, 0.0, amax, mu_out, 52, st)
+                  : eshkol_rowabsmax_shift_f64(A, M, K, 0.0, amax, mu_out, 52, st)) != 0) return -1;
+    if (!use_prepared &&
+        (b_kmajor ? eshkol_colabsmax_shift_f64(B, K, N, 0.0, bmax, nu_out, 52, st)
+                  : eshkol_rowabsmax_shift_f64(B, N, K, 0.0, bmax, nu_out, 52, st)) != 0) return -1;
+    const uint32_t ticket = fixed_E ? scan_launch_aside(amax, M, bmax, N, st) : scan_launch(amax, M, bmax, N, dmu, dnu, st);
+    if (!ticket) return -1;
 
     /* Everything after the shifts, queued in one go. */
     auto enqueue_products = [&](int n_mod, const HostCrt& crt, int E, bool b_ready) -> int {
+        const int32_t* nu = b_ready ? prepared->nu : dnu;
         int8_t* Ap = (int8_t*)eshkol_hip_workspace(WS_APLANES, (size_t)n_mod * Mp * ldk);
         int8_t* Bp = b_ready ? prepared->planes : (int8_t*)eshkol_hip_workspace(WS_BPLANES, (size_t)n_mod * Np * ldk);
         int8_t* Wp = (int8_t*)eshkol_hip_workspace(WS_PRODUCTS, (size_t)n_mod * M * N);
@@ -917,9 +938,9 @@ static int crt_matmul_impl(const double* A, const double* B, double* C,
         ga.layout = layout;
         if (hip_igemm_i8(&ga, st) != 0) return -1;
         if (hip_ozaki_crt_reconstruct_f64(Wp, M, N, n_mod, crt.sl1, crt.sl2, crt.P1, crt.P2, crt.Pinv,
-                                          dmu, dnu, bias, act, C, st) != 0) return -1;
+                                          dmu, nu, bias, act, C, st) != 0) return -1;
         g_last.a_planes = Ap; g_last.b_planes = Bp; g_last.w_planes = Wp;
-        g_last.mu = dmu; g_last.nu = dnu;
+        g_last.mu = dmu; g_last.nu = (int32_t*)nu;
         g_last.rows_a_padded = Mp; g_last.rows_b_padded = Np; g_last.ldk = ldk;
         g_last.num_moduli = n_mod; g_last.E = E; g_last.layout = layout;
         return 0;
@@ -933,35 +954,28 @@ static int crt_matmul_impl(const double* A, const double* B, double* C,
         return !any || (E - e_min <= 1023 && E - e_max >= -1022);
     };
 
-    /* E = min(52, floor((log2 P - 1 - log2 K - frac_A - frac_B) / 2)) with both
-     * fractions below 1 (gpu_memory.mm:2510-2512): where even frac_A + frac_B = 2
-     * leaves 52 (16 moduli: every K this tier accepts), E does not depend on the
-     * operands, and the whole pipeline is queued behind the scan without waiting
-     * for it. Its summary is read afterwards; what it may still demand is a
-     * refusal (non-finite input, shifts out of range: C then holds no result) or
-     * the reference's own pass over the maxima, after which the products are
-     * queued a second time. */
+    /* With E fixed the whole pipeline is queued at once. The scan's summary is read
+     * afterwards; what it may still demand is a refusal (non-finite input, shifts
+     * out of range: C then holds no result) or the reference's own pass over the
+     * maxima, after which the products are queued a second time. */
     const CrtScan* h_scan = nullptr;
     bool announced = false;
-    if (!adaptive && !g_force_host_pass) {
+    if (fixed_E) {
         const HostCrt& crt = crt_constants(num_moduli);
-        if (floor((crt.log2P - 3.0 - log2K) / 2.0) >= 52.0) {
-            const int E = 52;
-            hipLaunchKernelGGL(crt_shift_kernel, dim3((unsigned)((M + N + 255) / 256)), dim3(256), 0, st, dmu, M, dnu, N, E);
-            if (enqueue_products(num_moduli, crt, E, use_prepared) != 0) return -1;
-            announce(num_moduli, crt);
-            announced = true;
-            h_scan = scan_await(ticket, st);
-            if (!h_scan) return -1;
-            if (h_scan[0].nonfinite || h_scan[1].nonfinite) return -1;  /* NaN/Inf input */
-            if (!h_scan[0].extreme && !h_scan[1].extreme) {
-                for (int o = 0; o < 2; o++)
-                    if (!in_range(E, h_scan[o].nonzero != 0, h_scan[o].e_min, h_scan[o].e_max)) return -1;
-                return 0;
-            }
+        const int E = 52;
+        if (enqueue_products(num_moduli, crt, E, use_prepared) != 0) return -1;
+        announce(num_moduli, crt);
+        announced = true;
+        h_scan = scan_await(ticket);
+        if (!h_scan) return -1;
+        if (h_scan[0].nonfinite || h_scan[1].nonfinite) return -1;  /* NaN/Inf input */
+        if (!h_scan[0].extreme && !h_scan[1].extreme) {
+            for (int o = 0; o < 2; o++)
+                if (!in_range(E, h_scan[o].nonzero != 0, h_scan[o].e_min, h_scan[o].e_max)) return -1;
+            return 0;
         }
     }
-    if (!h_scan) h_scan = scan_await(ticket, st);
+    if (!h_scan) h_scan = scan_await(ticket);
     if (!h_scan) return -1;
     if (h_scan[0].nonfinite || h_scan[1].nonfinite) return -1;          /* NaN/Inf input */
 
@@ -1056,28 +1070,27 @@ extern "C" int hip_ozaki_crt_prepare_operand_b(const double* B, uint64_t K, uint
     const bool b_kmajor = trans_b == 0;
     CrtPreparedB* pb = new CrtPreparedB();
     pb->magic = PREPARED_MAGIC; pb->src = B; pb->K = K; pb->N = N; pb->rows_padded = Np; pb->ldk = ldk;
-    pb->trans_b = trans_b; pb->n_mod = num_moduli; pb->layout = layout; pb->bmax = nullptr; pb->planes = nullptr;
-    int32_t* fl = nullptr;
+    pb->trans_b = trans_b; pb->n_mod = num_moduli; pb->layout = layout;
+    pb->bmax = nullptr; pb->nu = nullptr; pb->planes = nullptr;
     auto fail = [&]() {
         if (pb->bmax) hipFree(pb->bmax);
+        if (pb->nu) hipFree(pb->nu);
         if (pb->planes) hipFree(pb->planes);
-        if (fl) hipFree(fl);
         delete pb;
         return -1;
     };
     if (!ESHKOL_HIP_OK(hipMalloc((void**)&pb->bmax, N * sizeof(double))) ||
-        !ESHKOL_HIP_OK(hipMalloc((void**)&pb->planes, (size_t)num_moduli * Np * ldk)) ||
-        !ESHKOL_HIP_OK(hipMalloc((void**)&fl, 2 * N * sizeof(int32_t)))) { (void)hipGetLastError(); return fail(); }
-    if ((b_kmajor ? hip_colabsmax_f64(B, K, N, 0.0, pb->bmax, st) : hip_rowabsmax_f64(B, N, K, 0.0, pb->bmax, st)) != 0)
+        !ESHKOL_HIP_OK(hipMalloc((void**)&pb->nu, N * sizeof(int32_t))) ||
+        !ESHKOL_HIP_OK(hipMalloc((void**)&pb->planes, (size_t)num_moduli * Np * ldk))) { (void)hipGetLastError(); return fail(); }
+    if ((b_kmajor ? eshkol_colabsmax_shift_f64(B, K, N, 0.0, pb->bmax, pb->nu, 52, st)
+                  : eshkol_rowabsmax_shift_f64(B, N, K, 0.0, pb->bmax, pb->nu, 52, st)) != 0)
         return fail();
     /* the scan takes two vectors of maxima: B's stand in for both */
-    const CrtScan* h = scan_maxima(pb->bmax, N, pb->bmax, N, fl, fl + N, st);
+    const CrtScan* h = scan_await(scan_launch(pb->bmax, N, pb->bmax, N, nullptr, nullptr, st));
     if (!h || h[1].nonfinite || h[1].extreme) return fail();     /* such a B takes the full pass on every call */
     if (h[1].nonzero && !(52 - h[1].e_min <= 1023 && 52 - h[1].e_max >= -1022)) return fail();
-    hipLaunchKernelGGL(crt_shift_kernel, dim3((unsigned)((2 * N + 255) / 256)), dim3(256), 0, st, fl, N, fl + N, N, 52);
-    if (crt_split_any(B, N, K, fl + N, num_moduli, pb->planes, Np, ldk, b_kmajor, layout, st) != 0) return fail();
+    if (crt_split_any(B, N, K, pb->nu, num_moduli, pb->planes, Np, ldk, b_kmajor, layout, st) != 0) return fail();
     if (!ESHKOL_HIP_OK(hipStreamSynchronize(st))) return fail();
-    hipFree(fl);
     *handle = pb;
     return 0;
 }
@@ -1088,6 +1101,7 @@ extern "C" void hip_ozaki_crt_release_prepared(void* handle) {
     EshkolHipCall bracket(nullptr);
     (void)hipDeviceSynchronize();
     hipFree(pb->bmax);
+    hipFree(pb->nu);
     hipFree(pb->planes);
     pb->magic = 0;
     delete pb;

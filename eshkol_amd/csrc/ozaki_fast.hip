@@ -485,15 +485,17 @@ extern "C" int hip_matmul_ozaki_fast_f64_ex(const double* A, const double* B, do
     int8_t* Wp = (int8_t*)eshkol_hip_workspace(WS_PRODUCTS, (size_t)f.n * M * N);
     if (!amax || !bmax || !sha || !shb || !Ap || !Bp || !Wp) return -2;
 
-    if ((a_kmajor ? hip_colabsmax_f64(A, K, M, 0.0, amax, st) : hip_rowabsmax_f64(A, M, K, 0.0, amax, st)) != 0) return -1;
-    if ((b_kmajor ? hip_colabsmax_f64(B, K, N, 0.0, bmax, st) : hip_rowabsmax_f64(B, N, K, 0.0, bmax, st)) != 0) return -1;
     /* frexp exponent e = floor(log2 max) + 1 (gpu_memory.mm:2886-2905); the split
-     * scales by 2^(E - e), so the per-row shift is (E - 1) - floor(log2 max) */
-    /* Nothing the host computes depends on the operands, so the whole pipeline is
-     * queued behind the scan and its summary (non-finite input?) is read at the end. */
-    const uint32_t ticket = eshkol_crt_scan_launch(amax, M, bmax, N, sha, shb, st);
+     * scales by 2^(E - e), so the per-row shift is (E - 1) - floor(log2 max): the
+     * kernels that find the maxima write it beside them. Nothing the host computes
+     * depends on the operands, so the whole pipeline is queued at once; the scan of
+     * the maxima (non-finite input?) runs beside it and is read at the end. */
+    if ((a_kmajor ? eshkol_colabsmax_shift_f64(A, K, M, 0.0, amax, sha, f.E - 1, st)
+                  : eshkol_rowabsmax_shift_f64(A, M, K, 0.0, amax, sha, f.E - 1, st)) != 0) return -1;
+    if ((b_kmajor ? eshkol_colabsmax_shift_f64(B, K, N, 0.0, bmax, shb, f.E - 1, st)
+                  : eshkol_rowabsmax_shift_f64(B, N, K, 0.0, bmax, shb, f.E - 1, st)) != 0) return -1;
+    const uint32_t ticket = eshkol_crt_scan_launch_aside(amax, M, bmax, N, st);
     if (!ticket) return -1;
-    eshkol_crt_shifts_from_exponents(sha, M, shb, N, f.E - 1, st);
 
     if (split_any(A, M, K, sha, f.table, Ap, Mp, ldk, a_kmajor, layout, st) != 0) return -1;
     if (split_any(B, N, K, shb, f.table, Bp, Np, ldk, b_kmajor, layout, st) != 0) return -1;
