@@ -160,6 +160,7 @@ SIGNATURES = {
     "hip_ozaki_slice_planes_f64": (C.c_int, [vp, u64, u64, vp, C.c_int, vp, u64, u64, C.c_int, C.c_int, vp]),
     "hip_dgemm_set_tail_split": (None, [C.c_int]),
     "hip_dgemm_set_small_tile": (None, [C.c_int]),
+    "hip_dgemm_set_prefetch_depth": (None, [C.c_int]),
     "hip_ozaki_crt_set_host_pass": (None, [C.c_int]),
     "hip_igemm_set_prefetch": (None, [C.c_int]),
 }

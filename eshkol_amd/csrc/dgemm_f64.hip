@@ -44,7 +44,7 @@ constexpr int BK = 16;
  * KMAJ = true:  the matrix is stored k by k with the row index contiguous (B
  *   as given, A when the caller holds its transpose); LDS tile [BK][R+4], a
  *   lane reads one 8-byte value per MFMA step.
- * The pads make every LDS read of a wave hit distinct banks. Both forms hand
+ * The pads make every LDS access of a wave hit distinct banks. Both forms hand
  * the MFMA the value at (row li + 16 t, k = 4 lg + s), so they are
  * interchangeable on either side of the instruction. */
 template <int R, bool KMAJ, bool VEC, bool LK = KMAJ> struct Operand {
@@ -52,7 +52,13 @@ template <int R, bool KMAJ, bool VEC, bool LK = KMAJ> struct Operand {
      * row-major one it means the pair a thread loaded is written as two 8-byte
      * values one LDS row apart (a transpose on the way in). */
     static_assert(LK || !KMAJ, "a k-major matrix keeps its form in LDS");
-    static constexpr int LD_S = LK ? R + 4 : BK + 2;
+    /* k-major tile of a k-major matrix: a thread writes 16 bytes of one LDS row,
+     * pitch R + 4. k-major tile of a row-major matrix: the eight lanes that loaded
+     * 128 contiguous bytes of a matrix row write sixteen LDS rows, two apart per
+     * lane: an odd pitch puts those rows 4 banks apart, so that sixteen lanes'
+     * 8-byte writes cover all 32 banks (with R + 4 they fell on two bank pairs,
+     * four deep, and the writes held up the fragment reads behind them). */
+    static constexpr int LD_S = LK ? (KMAJ ? R + 4 : R + 1) : BK + 2;
     static constexpr int TILE = LK ? BK * LD_S : R * LD_S;
     static constexpr int CHUNKS = R * BK / 2 / 256;   /* 16-byte chunks per thread */
     static constexpr int T = R / 32;                  /* 16-row tiles per wave */
@@ -275,7 +281,7 @@ __device__ __forceinline__ void lds_only_barrier() {
  * tile in `partial` (dgemm_fixup_kernel adds the pieces up in order). */
 struct SplitArgs { int first_tile, tail, kb_per_piece; double* partial; };
 
-template <bool TA, bool TB, bool KTAIL, bool SPLIT, int TS = 128>
+template <bool TA, bool TB, bool KTAIL, bool SPLIT, int TS = 128, int PF = 1>
 __global__ __launch_bounds__(256, TS == 128 ? 2 : 4)
 void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ B,
                        double* __restrict__ C, int M, int N, int K,
@@ -283,7 +289,14 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
     /* TS: edge of the block tile. 128 (wave tile 64 x 64) is the kernel of large
      * launches; 64 (wave tile 32 x 32, four workgroups to a CU) serves launches
      * that would leave CUs idle or half a round empty with the large tile. */
+    /* PF: how many k-blocks ahead of the LDS writes the global loads run. With 1 a
+     * load has three steps of MFMAs to land (one staging set, refilled as soon as
+     * the LDS writes have emptied it): enough when other workgroups share the CU
+     * or a step is 1024 cycles long. With 2 (two staging sets, block j in set
+     * j % 2) it has a whole k-block more: for the small tile, whose step is 256
+     * cycles, when a CU holds one workgroup. */
     static_assert(TS == 128 || (TS == 64 && !SPLIT), "cut tiles are 128 x 128");
+    static_assert(PF == 1 || PF == 2, "one or two staging sets");
     constexpr int BM = TS, BN = TS;
     constexpr int TT = TS / 32;                  /* 16 x 16 MFMA tiles per wave and dimension */
     using OpA = Operand<BM, TA, true, true>;
@@ -346,22 +359,23 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
     const size_t a_step = TA ? (size_t)BK * M : (size_t)BK;     /* doubles per k-block */
     const size_t b_step = TB ? (size_t)BK : (size_t)BK * N;
 
-    OpA a;
-    OpB b;
+    OpA a[PF];
+    OpB b[PF];
     /* KTAIL: K is not a multiple of 16. A chunk whose k lies beyond K reads the
      * same chunk of k-block 0 instead (valid memory, K >= 16) and is zeroed. */
-    auto gload = [&](int kb) {
+    auto gload = [&](int kb, auto set) {
+        constexpr int S = decltype(set)::value;
 #pragma unroll
         for (int r = 0; r < OpA::CHUNKS; r++) {
             const bool ok = !KTAIL || (kb * BK + ka[r] < K);
             const d2_t v = *(const d2_t*)(pa[r] + (size_t)(ok ? kb : 0) * a_step);
-            a.reg[r] = ok ? v : (d2_t){0.0, 0.0};
+            a[S].reg[r] = ok ? v : (d2_t){0.0, 0.0};
         }
 #pragma unroll
         for (int r = 0; r < OpB::CHUNKS; r++) {
             const bool ok = !KTAIL || (kb * BK + kbo[r] < K);
             const d2_t v = *(const d2_t*)(pb[r] + (size_t)(ok ? kb : 0) * b_step);
-            b.reg[r] = ok ? v : (d2_t){0.0, 0.0};
+            b[S].reg[r] = ok ? v : (d2_t){0.0, 0.0};
         }
     };
 
@@ -397,17 +411,25 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
     const int piece = SPLIT ? (int)(blockIdx.x / (unsigned)sp.tail) : 0;
     const int kb_lo = SPLIT ? piece * sp.kb_per_piece : 0;
     const int kb_hi = SPLIT ? ((kb_lo + sp.kb_per_piece < nkb_all) ? kb_lo + sp.kb_per_piece : nkb_all) : nkb_all;
-    gload(kb_lo);
-    a.sstore(As, tid);
-    b.sstore(Bs, tid);
-    gload(kb_hi - kb_lo > 1 ? kb_lo + 1 : kb_lo);
+    auto clamped = [&](int kb) { return kb < kb_hi ? kb : kb_hi - 1; };   /* requests past the end are never consumed */
+    gload(kb_lo, I0{});
+    a[0].sstore(As, tid);
+    b[0].sstore(Bs, tid);
+    if constexpr (PF == 2) {
+        gload(clamped(kb_lo + 1), I1{});
+        gload(clamped(kb_lo + 2), I0{});
+    } else {
+        gload(clamped(kb_lo + 1), I0{});
+    }
     __syncthreads();
     ldfrag(0, 0, I0{});
 
-    for (int kb = kb_lo; kb < kb_hi; kb++) {
-        const int cur = (kb - kb_lo) & 1;
-        /* the block after next, clamped: requests past the end are never consumed */
-        const int kb2 = (kb + 2 < kb_hi) ? kb + 2 : kb_hi - 1;
+    /* one k-block; `parity` = (kb - kb_lo) % 2 is its LDS buffer and, with two
+     * staging sets, the set the block after it is not in */
+    auto block = [&](int kb, auto parity) {
+        constexpr int cur = decltype(parity)::value;
+        using NextSet = std::integral_constant<int, PF == 2 ? (cur ^ 1) : 0>;    /* holds block kb + 1 */
+        const int kb2 = clamped(kb + 1 + PF);
 
         /* per step: NM MFMAs, TT fragment reads (pairs), and in step 2 the LDS writes of
          * the next block (3 per chunk pair), in step 3 its successor's global loads */
@@ -415,12 +437,23 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
         constexpr int WR_PER = 2;                  /* 64 x 64: six LDS writes behind three of the four MFMAs */
         constexpr int GL = OpA::CHUNKS + OpB::CHUNKS;
 
+        /* With two staging sets block kb + 1 has been in registers for a whole k-block:
+         * its LDS writes go here, into the buffer every wave left behind at the last
+         * barrier, and are long finished when this block's barrier asks for them. */
         ldfrag(cur, 1, I1{});
+        if constexpr (PF == 2) {
+            a[NextSet::value].sstore(As + (cur ^ 1) * OpA::TILE, tid);
+            b[NextSet::value].sstore(Bs + (cur ^ 1) * OpB::TILE, tid);
+        }
         mfma_step(I0{});
 #pragma unroll
         for (int i = 0; i < NM; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             if (i < TT) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (PF == 2) {
+                if (TS == 128) { if (i >= 2 && i < 14) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); }
+                else if (i >= 1) __builtin_amdgcn_sched_group_barrier(0x200, WR_PER, 0);
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
 
@@ -434,21 +467,25 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
         __builtin_amdgcn_sched_barrier(0);
 
         ldfrag(cur, 3, I1{});
-        a.sstore(As + (cur ^ 1) * OpA::TILE, tid);
-        b.sstore(Bs + (cur ^ 1) * OpB::TILE, tid);
+        if constexpr (PF == 1) {
+            a[NextSet::value].sstore(As + (cur ^ 1) * OpA::TILE, tid);
+            b[NextSet::value].sstore(Bs + (cur ^ 1) * OpB::TILE, tid);
+        }
         mfma_step(I0{});
 #pragma unroll
         for (int i = 0; i < NM; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             if (i < TT) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            if (TS == 128) { if (i >= 2 && i < 14) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); }
-            else if (i >= 1) __builtin_amdgcn_sched_group_barrier(0x200, WR_PER, 0);
+            if (PF == 1) {
+                if (TS == 128) { if (i >= 2 && i < 14) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0); }
+                else if (i >= 1) __builtin_amdgcn_sched_group_barrier(0x200, WR_PER, 0);
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
         lds_only_barrier();
 
         ldfrag(cur ^ 1, 0, I0{});
-        gload(kb2);
+        gload(kb2, NextSet{});
         mfma_step(I1{});
 #pragma unroll
         for (int i = 0; i < NM; i++) {
@@ -457,7 +494,13 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
             if (i < GL) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
+    };
+    int kb = kb_lo;
+    for (; kb + 1 < kb_hi; kb += 2) {
+        block(kb, I0{});
+        block(kb + 1, I1{});
     }
+    if (kb < kb_hi) block(kb, I0{});
 
     if constexpr (SPLIT) {
         double* out = sp.partial + (size_t)blockIdx.x * (BM * BN);
@@ -510,46 +553,102 @@ void dgemm_fixup_kernel(const double* __restrict__ partial, int tail, int pieces
 
 int g_tail_split = 1;
 
-/* Pieces per tile for a launch of `nwg` 128 x 128 tiles over `nkb` k-blocks that
- * does not fill the device; 1 = leave it to the 64 x 64 kernel. Times in
- * microseconds from two fits to measurements on this device (16 ... 144 tiles,
- * K = 64 ... 16384):
- *   whole: 4 + 0.86 per k-block, times the rounds four times as many small
- *          tiles need;
- *   cut:   10 + 0.04 per workgroup (two launches, the partial tiles' round
- *          trip) + 2.2 per k-block of a piece, times 1.7 once some CUs hold two
- *          workgroups.
- * The fits are within 10 % of the measurements they came from; a cut has to
- * win 5 % on them. */
-int small_launch_pieces(long long nwg, int nkb) {
+/* What a launch of the straight-line kernels is expected to take, in microseconds,
+ * from fits to measurements on this device (16 ... 6400 tiles, K = 256 ... 8192; the
+ * fits are within a few per cent of the measurements they came from). A CU works
+ * through the tiles it is given at a fixed rate per k-block whether they share the
+ * CU or follow one another, so a launch takes as long as its fullest CU:
+ *   128 x 128 tiles: 10 + 1.82 per k-block and tile of the fullest CU;
+ *   64 x 64 tiles:   10 + 0.46 per k-block and tile of the fullest CU (0.483 where
+ *                    no CU holds more than one): four small tiles cost 2 % more
+ *                    than a large one, and fill the device four times finer;
+ *   large tiles cut along k into p pieces (launches that do not fill the device):
+ *                    10 + 0.04 per workgroup (two launches, the partial tiles' round
+ *                    trip) + 2.2 per k-block of a piece, times 1.7 once some CUs
+ *                    hold two workgroups;
+ *   a last round of large tiles cut along k: the full rounds, plus that round's
+ *                    share ceil(p tail / slots) / p + 0.006 p, plus 15 for the two
+ *                    extra launches. */
+constexpr double US_KB_128 = 1.82, US_KB_64 = 0.46, US_KB_64_ALONE = 0.483, US_LAUNCH = 10.0;
+
+/* pieces per tile for a launch of `nwg` large tiles that does not fill the device (1 = whole) and its time */
+int small_launch_pieces(long long nwg, int nkb, double* us = nullptr) {
     const int cus = eshkol_hip_num_cus();
-    if (4 * nwg >= 3 * (long long)cus) return 1;
-    const double rounds = 4.0 * (double)nwg / cus;
-    const double whole = 4.0 + 0.86 * nkb * (rounds > 1.0 ? rounds : 1.0);
     int best_p = 1;
-    double best = 0.95 * whole;
-    for (int p = 2; p <= 128 && nkb / p >= 4 && nwg * p <= 2 * cus; p++) {
-        const double crowd = (nwg * p <= cus) ? 1.0 : 1.7;
-        const double cost = 10.0 + 0.04 * (double)(nwg * p) + crowd * 2.2 * ((double)nkb / p);
-        if (cost < best) { best = cost; best_p = p; }
+    double best = US_LAUNCH + US_KB_128 * nkb * (double)((nwg + cus - 1) / cus);
+    if (4 * nwg < 3 * (long long)cus) {
+        for (int p = 2; p <= 128 && nkb / p >= 4 && nwg * p <= 2 * cus; p++) {
+            const double crowd = (nwg * p <= cus) ? 1.0 : 1.7;
+            const double cost = 10.0 + 0.04 * (double)(nwg * p) + crowd * 2.2 * ((double)nkb / p);
+            if (cost < 0.95 * best) { best = cost; best_p = p; }
+        }
     }
+    if (us) *us = best;
     return best_p;
 }
+
+/* pieces per tile of the last, partial round of a launch of more than `slots` large tiles (1 = whole) and the launch's time */
+int tail_round_pieces(long long nwg, int nkb, double* share = nullptr) {
+    const int slots = 2 * eshkol_hip_num_cus();
+    const int tail = (int)(nwg % slots);
+    int best_p = 1;
+    double best = 1.0;
+    if (nwg > slots && tail > 0) {
+        for (int p = 2; p <= 32 && nkb / p >= 4; p++) {
+            const long long rounds = ((long long)p * tail + slots - 1) / slots;
+            const double cost = (double)rounds / p + 0.006 * p;
+            if (cost < best - 1e-9) { best = cost; best_p = p; }
+        }
+        if (!(best < 0.9)) { best = 1.0; best_p = 1; }
+    }
+    if (share) *share = best;
+    return best_p;
+}
+
+/* time of the large-tile path as launch_fast_k would run it */
+double large_tile_us(long long nwg, int nkb, bool may_cut) {
+    const int cus = eshkol_hip_num_cus(), slots = 2 * cus;
+    if (may_cut && nwg > slots && nwg % slots != 0) {
+        double share;
+        if (tail_round_pieces(nwg, nkb, &share) >= 2)
+            return US_LAUNCH + 15.0 + 2.0 * US_KB_128 * nkb * ((double)(nwg / slots) + share);
+    }
+    if (may_cut && 4 * nwg < 3 * (long long)cus) {
+        double us;
+        small_launch_pieces(nwg, nkb, &us);
+        return us;
+    }
+    return US_LAUNCH + US_KB_128 * nkb * (double)((nwg + cus - 1) / cus);
+}
+
+double small_tile_us(long long nwg64, int nkb) {
+    const int cus = eshkol_hip_num_cus();
+    const long long per_cu = (nwg64 + cus - 1) / cus;
+    return US_LAUNCH + (per_cu <= 1 ? US_KB_64_ALONE : US_KB_64) * nkb * (double)per_cu;
+}
+
+/* 0 (default) and 2: global loads two k-blocks ahead of their LDS writes wherever that
+ * variant holds its registers (all but the 128-tile kernel with a k-tail); 1: one ahead. */
+int g_prefetch_depth = 0;
 
 template <bool TA, bool TB, bool KTAIL>
 int launch_fast_k(const double* A, const double* B, double* C, int M, int N, int K, int batch, hipStream_t st) {
     constexpr int SMEM_BYTES = 2 * (Operand<128, TA, true, true>::TILE + Operand<128, !TB, true, true>::TILE)
                                * (int)sizeof(double);
     static bool attr_set = false;
-    auto kern = dgemm_fast_kernel<TA, TB, KTAIL, false>;
-    auto kern_split = dgemm_fast_kernel<TA, TB, KTAIL, true>;
+    /* with a k-tail the two-set variant of this tile size runs out of registers */
+    constexpr int DEEP = KTAIL ? 1 : 2;
+    auto kern1 = dgemm_fast_kernel<TA, TB, KTAIL, false, 128, 1>;
+    auto kern2 = dgemm_fast_kernel<TA, TB, KTAIL, false, 128, DEEP>;
+    auto kern_split1 = dgemm_fast_kernel<TA, TB, KTAIL, true, 128, 1>;
+    auto kern_split2 = dgemm_fast_kernel<TA, TB, KTAIL, true, 128, DEEP>;
     if (!attr_set) {
-        if (!ESHKOL_HIP_OK(hipFuncSetAttribute((const void*)kern,
-                hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES))) return -1;
-        if (!ESHKOL_HIP_OK(hipFuncSetAttribute((const void*)kern_split,
-                hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES))) return -1;
+        for (const void* f : {(const void*)kern1, (const void*)kern2, (const void*)kern_split1, (const void*)kern_split2})
+            if (!ESHKOL_HIP_OK(hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES))) return -1;
         attr_set = true;
     }
+    auto kern = g_prefetch_depth == 1 ? kern1 : kern2;
+    auto kern_split = g_prefetch_depth == 1 ? kern_split1 : kern_split2;
     const int tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
     const long long nwg = (long long)tiles_m * tiles_n;
     if (nwg > 0x7fffffffLL || batch < 1 || batch > 65535) return -1;
@@ -564,17 +663,11 @@ int launch_fast_k(const double* A, const double* B, double* C, int M, int N, int
      * the pieces go through a workspace and are added in a fixed order. */
     const int slots = 2 * eshkol_hip_num_cus();
     const int tail = (int)(nwg % slots), nkb = (K + BK - 1) / BK;
-    if (g_tail_split && batch == 1 && nwg > slots && tail > 0) {
-        int best_p = 1;
-        double best = 1.0;
-        for (int p = 2; p <= 32 && nkb / p >= 4; p++) {
-            const long long rounds = ((long long)p * tail + slots - 1) / slots;
-            const double cost = (double)rounds / p + 0.006 * p;
-            if (cost < best - 1e-9) { best = cost; best_p = p; }
-        }
+    const int best_p = (g_tail_split && batch == 1) ? tail_round_pieces(nwg, nkb) : 1;
+    if (best_p >= 2) {
         const int kbpp = (nkb + best_p - 1) / best_p;
         const int pieces = (nkb + kbpp - 1) / kbpp;
-        double* ws = (best < 0.9 && pieces >= 2) ? (double*)eshkol_hip_workspace(WS_DGEMM_PARTIAL,
+        double* ws = (pieces >= 2) ? (double*)eshkol_hip_workspace(WS_DGEMM_PARTIAL,
                                          (size_t)tail * pieces * 128 * 128 * sizeof(double)) : nullptr;
         if (ws) {
             sp.first_tile = (int)(nwg - tail); sp.tail = tail; sp.kb_per_piece = kbpp; sp.partial = ws;
@@ -622,7 +715,7 @@ template <bool TA, bool TB, bool KTAIL>
 int launch_fast64_k(const double* A, const double* B, double* C, int M, int N, int K, int batch, hipStream_t st) {
     constexpr int SMEM_BYTES = 2 * (Operand<64, TA, true, true>::TILE + Operand<64, !TB, true, true>::TILE)
                                * (int)sizeof(double);
-    auto kern = dgemm_fast_kernel<TA, TB, KTAIL, false, 64>;
+    auto kern = g_prefetch_depth == 1 ? dgemm_fast_kernel<TA, TB, KTAIL, false, 64, 1> : dgemm_fast_kernel<TA, TB, KTAIL, false, 64, 2>;
     const int tiles_m = (M + 63) / 64, tiles_n = (N + 63) / 64;
     const long long nwg = (long long)tiles_m * tiles_n;
     if (nwg > 0x7fffffffLL || batch < 1 || batch > 65535) return -1;
@@ -670,16 +763,19 @@ int launch_shape(const double* A, const double* B, double* C, int m, int n, int 
      * at 8192^3; with both operands row-major the natural forms are faster. */
     constexpr bool ALK = TA || !TB;
     /* 16-byte operand chunks (even pitches, aligned bases) and at least one whole k-block */
-    const bool cut = g_tail_split && batch == 1 && small_launch_pieces(big_tiles, (k + BK - 1) / BK) >= 2;
+    const int nkb = (k + BK - 1) / BK;
+    const bool may_cut = g_tail_split && batch == 1;
+    const bool cut = may_cut && small_launch_pieces(big_tiles, nkb) >= 2;
     const bool straight = g_fast_path && vec && m >= 2 && n >= 2 && k >= BK;
-    /* 64 x 64 tiles win where the large tile has to be cut along k to occupy a quarter to a
-     * third of the device (1024^3: 50 against 57 us; 1000 x 700 x 1300: 61 against 66), as long
-     * as k is short: one small-tile workgroup per CU sustains two thirds of the peak, the cut
-     * large tiles nine tenths but with a second launch to add them up (1024 x 1024 outputs:
-     * equal near k = 3000; 1152 x 1280: near k = 1024). With fewer large tiles the cut pieces
-     * win, with more the large tile does (measured 256^3 ... 8192^3). */
-    if (straight && (g_small_tile == 2 || (g_small_tile == 1 && batch == 1 && big_tiles >= 56 && big_tiles <= 96 &&
-                                           k >= 64 && (uint64_t)k * (uint64_t)big_tiles <= 2048u * 64u)))
+    /* Tile size of the straight-line kernel: whichever the fits above expect to finish
+     * first. Small tiles win where large ones would leave CUs idle or a round half
+     * empty and k is too short for cutting them to pay (1024^3: 41 us against 55 for
+     * the cut large tiles and 58 for whole ones; 2304 x 2304 x 2048: 360 against 463;
+     * 3072^3: 1075 against 1078 cut and 1385 whole); large tiles win full rounds by
+     * 2 % and, cut along k, launches of a few tiles with a long k. */
+    const long long small_tiles = (long long)((m + 63) / 64) * (long long)((n + 63) / 64) * batch;
+    if (straight && (g_small_tile == 2 ||
+                     (g_small_tile == 1 && small_tile_us(small_tiles, nkb) < large_tile_us(big_tiles, nkb, may_cut))))
         return launch_fast64<TA, TB>(A, B, C, m, n, k, batch, st);
     if (g_fast_path && (big_tiles >= 192 || cut) && vec && m >= 2 && n >= 2 && k >= BK)
         return launch_fast<TA, TB>(A, B, C, m, n, k, batch, st);
@@ -730,6 +826,7 @@ extern "C" void hip_dgemm_set_fast_path(int on) { g_fast_path = on ? 1 : 0; }
 extern "C" void hip_dgemm_set_tail_split(int on) { g_tail_split = on ? 1 : 0; }
 /* 0: the straight-line kernel uses 128 x 128 tiles only; 1 (default): 64 x 64 tiles where
  * they measure faster; 2: 64 x 64 tiles wherever the straight-line kernel applies. */
+extern "C" void hip_dgemm_set_prefetch_depth(int depth) { g_prefetch_depth = (depth == 1 || depth == 2) ? depth : 0; }
 extern "C" void hip_dgemm_set_small_tile(int mode) { if (mode >= 0 && mode <= 2) g_small_tile = mode; }
 
 extern "C" int hip_dgemm_f64_ex(const double* A, const double* B, double* C,

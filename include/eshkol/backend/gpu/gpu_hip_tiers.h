@@ -460,11 +460,18 @@ void hip_dgemm_set_fast_path(int on);
 void hip_dgemm_set_tail_split(int on);
 
 /* Tile size of the straight-line fp64 kernel. 0: 128 x 128 only; 1 (default):
- * 64 x 64 tiles for the launches that measure faster with them (56 to 96 large
- * tiles and k * tiles <= 131072, e.g. 1024^3, which would otherwise be cut along
- * k); 2: 64 x 64 wherever that kernel applies. The summation order inside a tile is the same, so all three
- * give the same bits as long as no tile is cut along k. */
+ * 64 x 64 tiles for the launches expected to finish sooner with them (large
+ * tiles would leave CUs idle or a round of tiles half empty, and k is too short
+ * for cutting them along k to pay: 1024^3, 2304 x 2304 x 2048, 3072^3 ...);
+ * 2: 64 x 64 wherever that kernel applies. The summation order inside a tile
+ * is the same, so all three give the same bits as long as no tile is cut
+ * along k. */
 void hip_dgemm_set_small_tile(int mode);
+
+/* How many k-blocks the straight-line fp64 kernels' global loads run ahead of
+ * their LDS writes. 0 (default) and 2: two, wherever that variant holds its
+ * registers; 1: one. Same bits; the switch exists to compare them. */
+void hip_dgemm_set_prefetch_depth(int depth);
 
 /* k-blocks kept in flight by the pipelined int8 kernel (1..3; 0 = simple kernel only). */
 void hip_igemm_set_prefetch(int pf);

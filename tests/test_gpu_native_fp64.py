@@ -154,6 +154,7 @@ def test_k_split_last_round(gpu, M, K, N):
         dX, dY = ea.DeviceArray.from_host(X), ea.DeviceArray.from_host(Y)
         outs = []
         try:
+            lib.hip_dgemm_set_small_tile(0)     # this test is about the large tiles of a cut last round
             for split in (0, 1, 1):
                 lib.hip_dgemm_set_tail_split(split)
                 guard = np.full((M + 2, N), np.nan)
@@ -166,6 +167,7 @@ def test_k_split_last_round(gpu, M, K, N):
                 outs.append(got[1:-1])
         finally:
             lib.hip_dgemm_set_tail_split(1)
+            lib.hip_dgemm_set_small_tile(1)
         whole, cut, again = outs
         assert np.array_equal(cut, again), (ta, tb)
         same = (whole == cut)
@@ -246,3 +248,36 @@ def test_small_tile_kernel_gives_the_bits_of_the_large_one(gpu, M, K, N):
     finally:
         lib.hip_dgemm_set_tail_split(1)
         lib.hip_dgemm_set_small_tile(1)
+
+
+@pytest.mark.parametrize("M,K,N", [(1024, 1024, 1024), (2304, 512, 2304), (3072, 640, 3072), (520, 4096, 500), (2048, 2048, 2048),
+                                   (4096, 256, 4100), (300, 1002, 1100)])
+def test_the_tile_size_chosen_by_itself_changes_no_bits_of_whole_tiles(gpu, M, K, N):
+    """The library picks the tile size of the straight-line kernel from the launch's shape.
+    With every tile whole (no cuts along k) all choices sum in the same order: the default
+    must give the bits of both forced sizes, and with cuts allowed stay within the tier's bound."""
+    import eshkol_amd as ea
+    from gpu_util import stream
+    lib = ea.load()
+    A, B = synth.normal(M + 13 * K, (M, K)), synth.normal(K + 13 * N, (K, N))
+    dA, dB, dC = ea.DeviceArray.from_host(A), ea.DeviceArray.from_host(B), ea.DeviceArray((M, N))
+    outs = {}
+    try:
+        for split, mode in ((0, 0), (0, 1), (0, 2), (1, 1)):
+            lib.hip_dgemm_set_tail_split(split); lib.hip_dgemm_set_small_tile(mode)
+            assert lib.hip_dgemm_f64(dA.ptr, dB.ptr, dC.ptr, M, K, N, stream()) == 0
+            ea.synchronize()
+            outs[split, mode] = dC.download()
+    finally:
+        lib.hip_dgemm_set_tail_split(1); lib.hip_dgemm_set_small_tile(1)
+    assert np.array_equal(outs[0, 0], outs[0, 1]) and np.array_equal(outs[0, 0], outs[0, 2])
+    assert normwise(outs[1, 1], oracle.matmul_f64(A, B), A, B) <= TOL
+    for depth in (1, 2):                      # both prefetch depths of the kernels: same bits
+        lib.hip_dgemm_set_prefetch_depth(depth)
+        try:
+            lib.hip_dgemm_set_tail_split(0)
+            assert lib.hip_dgemm_f64(dA.ptr, dB.ptr, dC.ptr, M, K, N, stream()) == 0
+            ea.synchronize()
+            assert np.array_equal(dC.download(), outs[0, 0]), depth
+        finally:
+            lib.hip_dgemm_set_prefetch_depth(0); lib.hip_dgemm_set_tail_split(1)
