@@ -176,27 +176,27 @@ const TierEnv& tier_env(void) { std::call_once(g_env_once, parse_env); return g_
  * Same shape as the reference's (gpu_memory_cuda.cpp:485-566): per kernel
  * t_ns = overhead + work/peak, peak self-calibrates upward from measured calls.
  * Seeds are MI355X measurements of this library: the line through the times
- * at 4096^3 and 8192^3 for the slice tiers (T1 0.42 and 2.23 ms ... T8 2.86
- * and 20.7 ms, rates taken 5 % low: devices differ by that much), 1024^3 and
- * 8192^3 for the native kernel (0.059 ms, 15.2 ms). */
+ * at 4096^3 and 8192^3 for the slice tiers (T1 0.43 and 2.08 ms ... T8 2.73
+ * and 20.3 ms, rates taken 5 % low: devices differ by that much), 1024^3 and
+ * 8192^3 for the native kernel (0.041 ms, 14.6 ms). */
 const double OZAKI_TOL[9] = { 1.0, 1e-3, 1e-5, 1e-7, 1e-9, 1e-11, 1e-13, 1e-14, 1e-14 };
 struct GemmModel { double overhead_ns; double peak_gflops; };
 constexpr int MODEL_CRT = 9;
 GemmModel g_model[10] = {
-    /* native */ {  25000.0,  72000.0 },
-    /* T1 */ { 160000.0, 505000.0 }, /* T2 */ { 225000.0, 325000.0 },
-    /* T3 */ { 320000.0, 220000.0 }, /* T4 */ { 350000.0, 148000.0 },
-    /* T5 */ { 245000.0, 107000.0 }, /* T6 */ { 345000.0,  81000.0 },
-    /* T7 */ { 350000.0,  63500.0 }, /* T8 */ { 315000.0,  51300.0 },
-    /* Ozaki-II CRT exact, 16 moduli: 1.47 and 8.80 ms */ { 420000.0, 125000.0 } };
+    /* native */ {  13000.0,  75000.0 },
+    /* T1 */ { 195000.0, 554000.0 }, /* T2 */ { 220000.0, 332000.0 },
+    /* T3 */ { 245000.0, 215000.0 }, /* T4 */ { 375000.0, 152000.0 },
+    /* T5 */ { 290000.0, 110500.0 }, /* T6 */ { 375000.0,  83500.0 },
+    /* T7 */ { 235000.0,  64300.0 }, /* T8 */ { 220000.0,  52000.0 },
+    /* Ozaki-II CRT exact, 16 moduli: 1.36 and 7.90 ms */ { 425000.0, 140000.0 } };
 const double OZAKI_SAFETY = 1.15;
 std::mutex g_model_mutex;
 
 double predict_ns(int idx, double work) { return g_model[idx].overhead_ns + work / g_model[idx].peak_gflops; }
 /* Reduced-precision CRT tier with n moduli: its times at 4096^3 and 8192^3 for
- * n = 4 ... 16 (0.48 and 2.58 ms ... 1.39 and 8.87 ms) are linear in n on both
+ * n = 4 ... 16 (0.46 and 2.35 ms ... 1.27 and 7.91 ms) are linear in n on both
  * coefficients; rate taken 5 % low like the others. */
-double predict_fast_ns(int n, double work) { return 135000.0 + 12000.0 * n + work * (0.42e-6 + 0.48e-6 * n); }
+double predict_fast_ns(int n, double work) { return 140000.0 + 11200.0 * n + work * (0.342e-6 + 0.433e-6 * n); }
 /* Its guaranteed relative error with E bits kept per operand: measured normwise
  * errors on well-conditioned operands are about 2^-E (1e-8 at E = 26); the
  * guarantee is 32 times that, the margin the reference gives its slice tiers
