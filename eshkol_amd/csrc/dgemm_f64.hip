@@ -325,20 +325,21 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
      * rows: they load valid memory and feed outputs that are never stored. */
     const double* pa[OpA::CHUNKS];
     const double* pb[OpB::CHUNKS];
-    int ka[OpA::CHUNKS], kbo[OpB::CHUNKS];       /* first k of the chunk inside a k-block */
+    /* first k of chunk r inside a k-block (recomputed where the k-tail needs it: the few
+     * registers it would take to keep them are the ones this kernel does not have) */
+    auto ka_of = [&](int r) { const int c = tid + 256 * r; return TA ? c / (BM / 2) : 2 * (c & 7); };
+    auto kbo_of = [&](int r) { const int c = tid + 256 * r; return TB ? 2 * (c & 7) : c / (BN / 2); };
 #pragma unroll
     for (int r = 0; r < OpA::CHUNKS; r++) {
         const int c = tid + 256 * r;
         if (TA) {
             int m = m0 + 2 * (c % (BM / 2));
             m = (m < M - 2) ? m : M - 2;
-            ka[r] = c / (BM / 2);
-            pa[r] = A + (size_t)ka[r] * M + m;
+            pa[r] = A + (size_t)ka_of(r) * M + m;
         } else {
             int m = m0 + (c >> 3);
             m = (m < M - 1) ? m : M - 1;
-            ka[r] = 2 * (c & 7);
-            pa[r] = A + (size_t)m * K + ka[r];
+            pa[r] = A + (size_t)m * K + ka_of(r);
         }
     }
 #pragma unroll
@@ -347,13 +348,11 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
         if (TB) {
             int n = n0 + (c >> 3);
             n = (n < N - 1) ? n : N - 1;
-            kbo[r] = 2 * (c & 7);
-            pb[r] = B + (size_t)n * K + kbo[r];
+            pb[r] = B + (size_t)n * K + kbo_of(r);
         } else {
             int n = n0 + 2 * (c % (BN / 2));
             n = (n < N - 2) ? n : N - 2;
-            kbo[r] = c / (BN / 2);
-            pb[r] = B + (size_t)kbo[r] * N + n;
+            pb[r] = B + (size_t)kbo_of(r) * N + n;
         }
     }
     const size_t a_step = TA ? (size_t)BK * M : (size_t)BK;     /* doubles per k-block */
@@ -363,17 +362,21 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
     OpB b[PF];
     /* KTAIL: K is not a multiple of 16. A chunk whose k lies beyond K reads the
      * same chunk of k-block 0 instead (valid memory, K >= 16) and is zeroed. */
-    auto gload = [&](int kb, auto set) {
+    /* `masked` (a compile-time flag): the block may be the one that holds the k-tail.
+     * Only the last requests of a workgroup pay for the selects; all others are plain
+     * loads, as in the variant without a tail. */
+    auto gload = [&](int kb, auto set, auto masked) {
         constexpr int S = decltype(set)::value;
+        constexpr bool MASK = KTAIL && decltype(masked)::value;
 #pragma unroll
         for (int r = 0; r < OpA::CHUNKS; r++) {
-            const bool ok = !KTAIL || (kb * BK + ka[r] < K);
+            const bool ok = !MASK || (kb * BK + ka_of(r) < K);
             const d2_t v = *(const d2_t*)(pa[r] + (size_t)(ok ? kb : 0) * a_step);
             a[S].reg[r] = ok ? v : (d2_t){0.0, 0.0};
         }
 #pragma unroll
         for (int r = 0; r < OpB::CHUNKS; r++) {
-            const bool ok = !KTAIL || (kb * BK + kbo[r] < K);
+            const bool ok = !MASK || (kb * BK + kbo_of(r) < K);
             const d2_t v = *(const d2_t*)(pb[r] + (size_t)(ok ? kb : 0) * b_step);
             b[S].reg[r] = ok ? v : (d2_t){0.0, 0.0};
         }
@@ -412,21 +415,21 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
     const int kb_lo = SPLIT ? piece * sp.kb_per_piece : 0;
     const int kb_hi = SPLIT ? ((kb_lo + sp.kb_per_piece < nkb_all) ? kb_lo + sp.kb_per_piece : nkb_all) : nkb_all;
     auto clamped = [&](int kb) { return kb < kb_hi ? kb : kb_hi - 1; };   /* requests past the end are never consumed */
-    gload(kb_lo, I0{});
+    gload(kb_lo, I0{}, I1{});
     a[0].sstore(As, tid);
     b[0].sstore(Bs, tid);
     if constexpr (PF == 2) {
-        gload(clamped(kb_lo + 1), I1{});
-        gload(clamped(kb_lo + 2), I0{});
+        gload(clamped(kb_lo + 1), I1{}, I1{});
+        gload(clamped(kb_lo + 2), I0{}, I1{});
     } else {
-        gload(clamped(kb_lo + 1), I0{});
+        gload(clamped(kb_lo + 1), I0{}, I1{});
     }
     __syncthreads();
     ldfrag(0, 0, I0{});
 
     /* one k-block; `parity` = (kb - kb_lo) % 2 is its LDS buffer and, with two
      * staging sets, the set the block after it is not in */
-    auto block = [&](int kb, auto parity) {
+    auto block = [&](int kb, auto parity, auto masked) {
         constexpr int cur = decltype(parity)::value;
         using NextSet = std::integral_constant<int, PF == 2 ? (cur ^ 1) : 0>;    /* holds block kb + 1 */
         const int kb2 = clamped(kb + 1 + PF);
@@ -485,7 +488,7 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
         lds_only_barrier();
 
         ldfrag(cur ^ 1, 0, I0{});
-        gload(kb2, NextSet{});
+        gload(kb2, NextSet{}, masked);
         mfma_step(I1{});
 #pragma unroll
         for (int i = 0; i < NM; i++) {
@@ -495,12 +498,26 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
         }
         __builtin_amdgcn_sched_barrier(0);
     };
+    /* the blocks whose request (1 + PF blocks ahead) cannot reach the last block of k
+     * run without the tail's selects; the few that follow run with them */
     int kb = kb_lo;
-    for (; kb + 1 < kb_hi; kb += 2) {
-        block(kb, I0{});
-        block(kb + 1, I1{});
+    if constexpr (KTAIL) {
+        for (; kb + 1 + (1 + PF) < kb_hi - 1; kb += 2) {     /* block kb + 1 requests block kb + 2 + PF: not the last */
+            block(kb, I0{}, I0{});
+            block(kb + 1, I1{}, I0{});
+        }
+        for (; kb + 1 < kb_hi; kb += 2) {          /* kb - kb_lo is even here: the parities stay compile-time */
+            block(kb, I0{}, I1{});
+            block(kb + 1, I1{}, I1{});
+        }
+        if (kb < kb_hi) block(kb, I0{}, I1{});
+    } else {
+        for (; kb + 1 < kb_hi; kb += 2) {
+            block(kb, I0{}, I0{});
+            block(kb + 1, I1{}, I0{});
+        }
+        if (kb < kb_hi) block(kb, I0{}, I0{});
     }
-    if (kb < kb_hi) block(kb, I0{});
 
     if constexpr (SPLIT) {
         double* out = sp.partial + (size_t)blockIdx.x * (BM * BN);
@@ -774,8 +791,12 @@ int launch_shape(const double* A, const double* B, double* C, int m, int n, int 
      * 3072^3: 1075 against 1078 cut and 1385 whole); large tiles win full rounds by
      * 2 % and, cut along k, launches of a few tiles with a long k. */
     const long long small_tiles = (long long)((m + 63) / 64) * (long long)((n + 63) / 64) * batch;
+    /* (the small tile's rate holds up to about two rounds of large tiles; beyond, its
+     * four-fold operand traffic tells: 5120^3 3.86 ms against 3.63 for large tiles with
+     * a cut last round, where the fits call it even) */
     if (straight && (g_small_tile == 2 ||
-                     (g_small_tile == 1 && small_tile_us(small_tiles, nkb) < large_tile_us(big_tiles, nkb, may_cut))))
+                     (g_small_tile == 1 && big_tiles < 4LL * eshkol_hip_num_cus() &&
+                      small_tile_us(small_tiles, nkb) < large_tile_us(big_tiles, nkb, may_cut))))
         return launch_fast64<TA, TB>(A, B, C, m, n, k, batch, st);
     if (g_fast_path && (big_tiles >= 192 || cut) && vec && m >= 2 && n >= 2 && k >= BK)
         return launch_fast<TA, TB>(A, B, C, m, n, k, batch, st);
