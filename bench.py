@@ -69,8 +69,8 @@ def main():
                     help="run a calibration copy and three launches of one tier, for rocprofv3 --pmc")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        sys.exit("bench.py: this build measures one GPU only (the path shards by rows of A with no "
-                 "exchange; see DESIGN.md). Run with --gpus 1.")
+        sys.exit("bench.py: this build measures one GPU only (the path would shard by rows of A, one "
+                 "broadcast of B and no further exchange). Run with --gpus 1.")
 
     import eshkol_amd as ea
     from eshkol_amd import synth
