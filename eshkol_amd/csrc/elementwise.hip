@@ -97,8 +97,17 @@ void colabsmax_partial_kernel(const double* __restrict__ X, uint64_t K, uint64_t
     const uint64_t k0 = (uint64_t)blockIdx.y * rows_per_slice;
     const uint64_t k1 = (k0 + rows_per_slice < K) ? k0 + rows_per_slice : K;
     double m = 0.0;
-    if (col < R)
-        for (uint64_t k = k0 + part; k < k1; k += 4) absmax_step(X[k * R + col], &m);
+    if (col < R) {
+        uint64_t k = k0 + part;
+        for (; k + 28 < k1; k += 32) {          /* eight loads in flight per thread, not one */
+            double v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) v[u] = X[(k + 4 * u) * R + col];
+#pragma unroll
+            for (int u = 0; u < 8; u++) absmax_step(v[u], &m);
+        }
+        for (; k < k1; k += 4) absmax_step(X[k * R + col], &m);
+    }
     red[part][c] = m;
     __syncthreads();
     if (part == 0 && col < R) {
