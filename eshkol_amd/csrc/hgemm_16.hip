@@ -125,7 +125,7 @@ void convert_il_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
     v4i_t w;
 #pragma unroll
     for (int e = 0; e < 4; e++) w[e] = (int)narrow_pair<BF16>(x[2 * e], x[2 * e + 1]);
-    *(v4i_t*)((int8_t*)out + eshkol_plane_offset(1, row, 2 * k, 2 * ld)) = w;
+    eshkol_store_streaming((v4i_t*)((int8_t*)out + eshkol_plane_offset(1, row, 2 * k, 2 * ld)), w);
 }
 
 /* k-major X[K][rows] (B as the runtime stores it), same output. */
@@ -146,7 +146,7 @@ void convert_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint64_t
                     v4i_t w;
 #pragma unroll
                     for (int e = 0; e < 4; e++) w[e] = (int)narrow_pair<BF16>(x[8 * c + 2 * e], x[8 * c + 2 * e + 1]);
-                    *(v4i_t*)((int8_t*)out + eshkol_plane_offset(1, row, 2 * k + 16 * c, 2 * ld)) = w;
+                    eshkol_store_streaming((v4i_t*)((int8_t*)out + eshkol_plane_offset(1, row, 2 * k + 16 * c, 2 * ld)), w);
                 }
             });
         return;
@@ -176,7 +176,7 @@ void convert_kmajor_il_kernel(const double* __restrict__ X, uint64_t rows, uint6
         v4i_t w;
 #pragma unroll
         for (int e = 0; e < 4; e++) w[e] = (int)narrow_pair<BF16>(x[8 * c + 2 * e], x[8 * c + 2 * e + 1]);
-        *(v4i_t*)((int8_t*)out + eshkol_plane_offset(1, row, 2 * k + 16 * c, 2 * ld)) = w;
+        eshkol_store_streaming((v4i_t*)((int8_t*)out + eshkol_plane_offset(1, row, 2 * k + 16 * c, 2 * ld)), w);
     }
 }
 

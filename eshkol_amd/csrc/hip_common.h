@@ -76,4 +76,17 @@ static inline int eshkol_hip_num_cus(void) {
 
 static inline size_t round_up_sz(size_t v, size_t m) { return (v + m - 1) / m * m; }
 
+/* A store whose line nothing on the device reads again soon (operand planes on
+ * their way to HBM: gigabytes written once, read by a later kernel): the
+ * non-temporal form keeps such lines from displacing what the caches hold and
+ * measured 5-7 % on the kernels that mix reads and writes about evenly
+ * (slices of 8192^2: 0.203 -> 0.190 ms). Only for stores that fill whole lines by
+ * themselves or with their neighbours in the wave: 8-byte pieces of a line sent
+ * this way are not merged on the way out (the slice tier's reconstruction ran
+ * twice as long with them). */
+#ifdef __HIPCC__
+template <class T>
+__device__ __forceinline__ void eshkol_store_streaming(T* p, T v) { __builtin_nontemporal_store(v, p); }
+#endif
+
 #endif

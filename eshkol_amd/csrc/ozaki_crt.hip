@@ -103,7 +103,7 @@ __device__ __forceinline__ void split_16(const double* x, int sh, int8_t* out, u
             const uint32_t w23 = __builtin_amdgcn_perm(residue_byte<L>(s[4 * g + 3]), residue_byte<L>(s[4 * g + 2]), 0x0c0c0400u); \
             w[g] = __builtin_amdgcn_perm(w23, w01, 0x05040100u);                      \
         }                                                                             \
-        *(v4u_t*)(out + (uint64_t)L * plane_stride) = w;                              \
+        eshkol_store_streaming((v4u_t*)(out + (uint64_t)L * plane_stride), w);        \
     }
     ESHKOL_SPLIT_ONE(0)  ESHKOL_SPLIT_ONE(1)  ESHKOL_SPLIT_ONE(2)  ESHKOL_SPLIT_ONE(3)
     ESHKOL_SPLIT_ONE(4)  ESHKOL_SPLIT_ONE(5)  ESHKOL_SPLIT_ONE(6)  ESHKOL_SPLIT_ONE(7)
@@ -244,8 +244,8 @@ void crt_split_il_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K
         const int c = tid + 256 * j;
         const int plane = c >> 6, q = c & 63;
         if (plane < NMOD)
-            *(v4u_t*)(frag + (uint64_t)plane * plane_stride + 16 * q) =
-                *(const v4u_t*)&stage[plane][8 * (q & 31) + 4 * (q >> 5)];
+            eshkol_store_streaming((v4u_t*)(frag + (uint64_t)plane * plane_stride + 16 * q),
+                                   *(const v4u_t*)&stage[plane][8 * (q & 31) + 4 * (q >> 5)]);
     }
 }
 

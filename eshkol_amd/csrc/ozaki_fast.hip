@@ -148,8 +148,8 @@ void fast_split_il_kernel(const double* __restrict__ X, uint64_t rows, uint64_t 
     int8_t* frag = planes + rb * (32 * ldk) + kb * 1024;
     for (int c = tid; c < tbl.n * 64; c += 256) {
         const int plane = c >> 6, q = c & 63;
-        *(v4u_t*)(frag + (uint64_t)plane * plane_stride + 16 * q) =
-            *(const v4u_t*)&stage[plane][8 * (q & 31) + 4 * (q >> 5)];
+        eshkol_store_streaming((v4u_t*)(frag + (uint64_t)plane * plane_stride + 16 * q),
+                               *(const v4u_t*)&stage[plane][8 * (q & 31) + 4 * (q >> 5)]);
     }
 }
 
@@ -174,7 +174,7 @@ void fast_split_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint6
                 for (int g = 0; g < 4; g++)
                     w[g] = pack4(fast_residue(s[4 * g], tbl, l), fast_residue(s[4 * g + 1], tbl, l),
                                  fast_residue(s[4 * g + 2], tbl, l), fast_residue(s[4 * g + 3], tbl, l));
-                *(v4u_t*)(out + (uint64_t)l * plane_stride) = w;
+                eshkol_store_streaming((v4u_t*)(out + (uint64_t)l * plane_stride), w);
             }
         });
 }
@@ -202,7 +202,7 @@ void fast_split_kmajor_il_kernel(const double* __restrict__ X, uint64_t rows, ui
         for (int g = 0; g < 4; g++)
             w[g] = pack4(fast_residue(s[4 * g], tbl, l), fast_residue(s[4 * g + 1], tbl, l),
                          fast_residue(s[4 * g + 2], tbl, l), fast_residue(s[4 * g + 3], tbl, l));
-        *(v4u_t*)(out + (uint64_t)l * plane_stride) = w;
+        eshkol_store_streaming((v4u_t*)(out + (uint64_t)l * plane_stride), w);
     }
 }
 

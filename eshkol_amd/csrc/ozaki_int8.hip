@@ -48,12 +48,12 @@ __device__ __forceinline__ void slice_group(const double* x, double sc, int s, i
         }
         int8_t* o = out + (uint64_t)p * plane_stride;
         if (G == 2) *(uint16_t*)o = (uint16_t)w[0];
-        else if (G == 4) *(uint32_t*)o = w[0];
+        else if (G == 4) eshkol_store_streaming((uint32_t*)o, w[0]);
         else {
             v4u_t v;
 #pragma unroll
             for (int e = 0; e < 4; e++) v[e] = w[e % ((G + 3) / 4)];
-            *(v4u_t*)o = v;
+            eshkol_store_streaming((v4u_t*)o, v);
         }
     }
 }
@@ -189,6 +189,17 @@ void reconstruct_kernel(double* __restrict__ C, const int32_t* __restrict__ Gall
         for (int e = 0; e < COLS; e++) acc[e] = acc[e] + w * (double)gv[e];
     }
     const double r = rmax[row];
+    if (vec && (((uintptr_t)C & 15) == 0)) {
+        /* the reference's operations in its order; the results leave two to a store */
+#pragma unroll
+        for (int e = 0; e < COLS; e += 2) {
+            d2_t v;
+            v.x = (acc[e] * r) * cmax[col + e];
+            v.y = (acc[e + 1] * r) * cmax[col + e + 1];
+            *(d2_t*)(C + idx + e) = v;
+        }
+        return;
+    }
 #pragma unroll
     for (int e = 0; e < COLS; e++)
         if (e < nvalid) C[idx + e] = (acc[e] * r) * cmax[col + e];
