@@ -459,7 +459,9 @@ void hgemm_pipe_kernel(const uint16_t* __restrict__ A, const uint16_t* __restric
  * the transposed 32 x 32 tile of rows m0 + 64 wave + 32 t + lane%32, columns
  * n0 + 32 u + 8 v + 4 (lane/32) + 0..3 in registers 4v .. 4v+3. A batch of
  * products is one launch: a tile's batch index is its operand plane. */
-template <bool BF16>
+/* INTERIOR: the tile lies inside the matrix and its rows can move as 16-byte pieces: the
+ * stores then carry no bounds and no branches, and one address serves a block. */
+template <bool BF16, bool INTERIOR>
 __device__ __forceinline__ void store_tile_direct(v16f_t (&acc)[pipe2::TM][pipe2::TN], int m0, int n0, int M, int N,
                                                   int out_mode, void* Cout, int8_t* stage) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -487,7 +489,24 @@ __device__ __forceinline__ void store_tile_direct(v16f_t (&acc)[pipe2::TM][pipe2
                 __builtin_amdgcn_sched_barrier(0);
             }
             const int cb = n0 + u * 32;
-            if (out_mode == 0) {
+            if constexpr (INTERIOR) {
+                if (out_mode == 0) {
+                    v4i_t w[4];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) w[i] = pipe2::parked_row16(stage, i);
+                    float* p = (float*)Cout + (size_t)(row0 + (lane >> 3)) * N + cb + 4 * (lane & 7);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) *(v4i_t*)(p + (size_t)(8 * i) * N) = w[i];
+                } else {
+                    pipe2::v2i_t w[8];
+#pragma unroll
+                    for (int i = 0; i < 8; i++) w[i] = pipe2::parked_row8(stage, i);
+                    double* p = (double*)Cout + (size_t)(row0 + (lane >> 4)) * N + cb + 2 * (lane & 15);
+#pragma unroll
+                    for (int i = 0; i < 8; i++)
+                        *(d2_t*)(p + (size_t)(4 * i) * N) = (d2_t){(double)__int_as_float(w[i][0]), (double)__int_as_float(w[i][1])};
+                }
+            } else if (out_mode == 0) {
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const v4i_t w = pipe2::parked_row16(stage, i);
@@ -552,7 +571,10 @@ void hgemm_direct_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
     };
     const uint64_t c_bytes = (uint64_t)M * (uint64_t)N * (out_mode == 0 ? 4u : 8u);
     auto epi = [&](v16f_t (&acc)[pipe2::TM][pipe2::TN], const pipe::Tile& t, int8_t* stage) {
-        store_tile_direct<BF16>(acc, t.m0, t.n0, M, N, out_mode, (int8_t*)Cout + (uint64_t)t.tag * c_bytes, stage);
+        void* Ct = (int8_t*)Cout + (uint64_t)t.tag * c_bytes;
+        const bool interior = t.m0 + pipe2::BM <= M && t.n0 + pipe2::BN <= N && (N & 3) == 0 && (((uintptr_t)Ct & 15) == 0);
+        if (interior) store_tile_direct<BF16, true>(acc, t.m0, t.n0, M, N, out_mode, Ct, stage);
+        else store_tile_direct<BF16, false>(acc, t.m0, t.n0, M, N, out_mode, Ct, stage);
     };
     pipe2::run_tiles<H16Op<BF16>>(smem_h, cm, next_tile, epi);
 }
