@@ -283,6 +283,9 @@ __device__ __forceinline__ void epilogue_direct(const HipIgemmArgs& g, int o, in
     if (g.mode == 0) {
         int32_t* out = g.out_i32 + (size_t)o * g.M * g.N;
         const bool vec_ok = (g.N % 4 == 0);
+        /* a tile inside the matrix: no bounds, no branches, one address per block (the same for every lane) */
+        const bool interior0 = vec_ok && (((uintptr_t)out & 15) == 0) &&
+                               m0 + pipe2::BM <= (int)g.M && n0 + pipe2::BN <= (int)g.N;
 #pragma unroll
         for (int t = 0; t < TM; t++) {
             const int row = m0 + wave * 64 + t * 32 + li;
@@ -296,14 +299,23 @@ __device__ __forceinline__ void epilogue_direct(const HipIgemmArgs& g, int o, in
                                                         acc[t][u][4 * v + 2], acc[t][u][4 * v + 3]});
                     __builtin_amdgcn_sched_barrier(0);
                 }
+                if (interior0) {
+                    v4i_t w[4];
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const v4i_t w = pipe2::parked_row16(stage, i);
-                    const int orow = row - li + (lane >> 3) + 8 * i, col = n0 + u * 32 + 4 * (lane & 7);
-                    if (orow < (int)g.M && col < (int)g.N) {
-                        int32_t* p = out + (size_t)orow * g.N + col;
-                        if (vec_ok && col + 3 < (int)g.N) *(v4i_t*)p = w;
-                        else for (int e = 0; e < 4; e++) if (col + e < (int)g.N) p[e] = w[e];
+                    for (int i = 0; i < 4; i++) w[i] = pipe2::parked_row16(stage, i);
+                    int32_t* p = out + (size_t)(row - li + (lane >> 3)) * g.N + (n0 + u * 32 + 4 * (lane & 7));
+#pragma unroll
+                    for (int i = 0; i < 4; i++) *(v4i_t*)(p + (size_t)(8 * i) * g.N) = w[i];
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const v4i_t w = pipe2::parked_row16(stage, i);
+                        const int orow = row - li + (lane >> 3) + 8 * i, col = n0 + u * 32 + 4 * (lane & 7);
+                        if (orow < (int)g.M && col < (int)g.N) {
+                            int32_t* p = out + (size_t)orow * g.N + col;
+                            if (vec_ok && col + 3 < (int)g.N) *(v4i_t*)p = w;
+                            else for (int e = 0; e < 4; e++) if (col + e < (int)g.N) p[e] = w[e];
+                        }
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
