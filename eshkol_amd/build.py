@@ -8,6 +8,7 @@ one shared library whose exported symbols are the C ABI declared in
 include/eshkol/backend/gpu/gpu_memory.h and gpu_hip_tiers.h.
 """
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -77,6 +78,55 @@ def _check_no_spill(src, remarks):
         raise RuntimeError("%s: no resource remarks for %s; cannot prove it is free of spills" % (src, missing))
 
 
+def sgpr_to_vmem_hazards(asm):
+    """Places in gfx9 assembly text where a memory instruction reads a scalar
+    register fewer than five wait states after a vector instruction wrote it
+    (v_readlane of a spilled scalar, v_readfirstlane, a compare). The compiler
+    keeps that distance between its own instructions; it does not look inside an
+    asm statement, so a memory instruction issued from one can land right behind
+    the reload of its address. Returns a list of (line number, text, wait states)."""
+    def sregs(tok):
+        m = re.fullmatch(r"s(\d+)", tok)
+        if m:
+            return {int(m.group(1))}
+        m = re.fullmatch(r"s\[(\d+):(\d+)\]", tok)
+        if m:
+            return set(range(int(m.group(1)), int(m.group(2)) + 1))
+        return set()
+    pending, found = [], []
+    for no, raw in enumerate(asm.split("\n"), 1):
+        line = raw.split(";")[0].strip()
+        if not line or line.endswith(":") or line.startswith("."):
+            continue
+        parts = line.replace(",", " ").split()
+        op, ops = parts[0], parts[1:]
+        if op.startswith(("buffer_", "global_", "flat_", "scratch_")):
+            used = set()
+            for t in ops:
+                used |= sregs(t)
+            for regs, ws, _ in pending:
+                if regs & used and ws < 5:
+                    found.append((no, line, ws))
+        step = int(ops[0]) + 1 if op == "s_nop" and ops else 1
+        pending = [(r, ws + step, l) for (r, ws, l) in pending if ws + step < 5]
+        if op.startswith("v_") and ops and sregs(ops[0]):
+            pending.append((sregs(ops[0]), 0, no))
+    return found
+
+
+def _check_hazards(src):
+    """Compiles src to assembly with the flags of the build and scans it."""
+    path = os.path.join(CSRC, src)
+    cmd = [HIPCC] + COMMON + EXTRA.get(src, []) + ["-x", "hip", "-S", "--cuda-device-only", path, "-o", "-"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc -S failed for %s:\n%s" % (src, res.stderr))
+    found = sgpr_to_vmem_hazards(res.stdout)
+    if found:
+        raise RuntimeError("%s: memory instructions read scalar registers too soon after a vector instruction "
+                           "wrote them:\n%s" % (src, "\n".join("  line %d: %s (%d wait states)" % f for f in found[:10])))
+
+
 def _newer(target, deps):
     if not os.path.exists(target):
         return False
@@ -109,8 +159,12 @@ def _compile(src, force):
 
 def build(force=False, verbose=False):
     os.makedirs(OBJDIR, exist_ok=True)
+    stale = [s for s in NO_SPILL if force or not _newer(LIB, [os.path.join(CSRC, f) for f in os.listdir(CSRC)])]
     with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
+        checks = [pool.submit(_check_hazards, s) for s in stale]      # the kernels that issue loads from asm
         objs = list(pool.map(lambda s: _compile(s, force), SOURCES))
+        for c in checks:
+            c.result()
     if force or not _newer(LIB, objs):
         cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs + ["-ldl", "-lpthread"]
         res = subprocess.run(cmd, capture_output=True, text=True)
