@@ -301,7 +301,12 @@ struct CrtConsts {
  * use: the kernel moves 24 bytes per element and has to keep HBM busy. So is
  * the tanh epilogue: its code would otherwise cost every launch three quarters
  * of its occupancy in registers. */
-template <int NMOD, bool TANH>
+/* VEC: N is a multiple of four and W and C are aligned for 4- and 16-byte
+ * accesses (the launcher checks): every thread then has four whole elements, and
+ * the kernel carries none of the byte-wise path, whose address arithmetic the
+ * compiler would otherwise place in front of both paths (a third of the
+ * kernel's vector instructions: it is bound by them, not by HBM). */
+template <int NMOD, bool TANH, bool VEC>
 __global__ __launch_bounds__(256)
 void crt_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t N, CrtConsts cc,
                             const int32_t* __restrict__ mu, const int32_t* __restrict__ nu,
@@ -311,12 +316,13 @@ void crt_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t N
     const uint64_t col = ((uint64_t)(blockIdx.x % cpr) * 256 + threadIdx.x) * 4;
     if (col >= N) return;
     const uint64_t tot = M * N, idx = row * N + col;
-    const int nvalid = (N - col < 4) ? (int)(N - col) : 4;
-    const bool vec = (nvalid == 4) && ((N & 3) == 0) && (((uintptr_t)W & 3) == 0);
+    const int nvalid = VEC ? 4 : ((N - col < 4) ? (int)(N - col) : 4);
+    const bool vec = VEC || ((nvalid == 4) && ((N & 3) == 0) && (((uintptr_t)W & 3) == 0));
     uint32_t u[NMOD];
     if (vec) {
+        const int8_t* p = W + idx;                 /* one address, then a step per plane */
 #pragma unroll
-        for (int l = 0; l < NMOD; l++) u[l] = *(const uint32_t*)(W + (uint64_t)l * tot + idx);
+        for (int l = 0; l < NMOD; l++) { u[l] = *(const uint32_t*)p; p += tot; }
     } else {
 #pragma unroll
         for (int l = 0; l < NMOD; l++) {
@@ -360,7 +366,7 @@ void crt_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t N
         if (TANH) v = eshkol_tanh_f64(v);
         out[e] = v;
     }
-    if (vec && (((uintptr_t)C & 15) == 0)) {
+    if (VEC || (vec && (((uintptr_t)C & 15) == 0))) {
         d2_t* o = (d2_t*)(C + idx);
         d2_t lo, hi;
         lo.x = out[0]; lo.y = out[1]; hi.x = out[2]; hi.y = out[3];
@@ -796,16 +802,18 @@ extern "C" int hip_ozaki_crt_reconstruct_f64(const int8_t* w_planes, uint64_t M,
     for (int l = 0; l < num_moduli; l++) { cc.sl1[l] = sl1[l]; cc.sl2[l] = sl2[l]; }
     cc.P1 = P1; cc.P2 = P2; cc.Pinv = Pinv; cc.n = num_moduli;
     dim3 grid((unsigned)((((N + 3) / 4 + 255) / 256) * M));
+    const bool vec = (N % 4 == 0) && (((uintptr_t)w_planes & 3) == 0) && (((uintptr_t)C & 15) == 0);
     switch (num_moduli) {
+#define LAUNCH(n, tanh, v) hipLaunchKernelGGL((crt_reconstruct_kernel<n, tanh, v>), grid, dim3(256), 0,    \
+                                              (hipStream_t)stream, w_planes, M, N, cc, mu, nu, bias, C)
 #define CASE(n) case n:                                                                                   \
-        if (act == 1) hipLaunchKernelGGL((crt_reconstruct_kernel<n, true>), grid, dim3(256), 0, (hipStream_t)stream,  \
-                                         w_planes, M, N, cc, mu, nu, bias, C);                            \
-        else hipLaunchKernelGGL((crt_reconstruct_kernel<n, false>), grid, dim3(256), 0, (hipStream_t)stream,           \
-                                w_planes, M, N, cc, mu, nu, bias, C);                                     \
+        if (act == 1) { if (vec) LAUNCH(n, true, true); else LAUNCH(n, true, false); }                     \
+        else { if (vec) LAUNCH(n, false, true); else LAUNCH(n, false, false); }                            \
         break;
         CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8) CASE(9)
         CASE(10) CASE(11) CASE(12) CASE(13) CASE(14) CASE(15) CASE(16)
 #undef CASE
+#undef LAUNCH
         default: return -1;
     }
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;

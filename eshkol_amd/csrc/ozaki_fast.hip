@@ -220,7 +220,10 @@ void fast_split_kmajor_il_kernel(const double* __restrict__ X, uint64_t rows, ui
  * (the kernel moves 8 + n bytes per element and has to keep HBM busy). */
 struct FracLimbs { int32_t d[FAST_MAX_MODULI][4]; };
 
-template <int NMOD>
+/* VEC: N is a multiple of four and W and C are aligned for 4- and 16-byte
+ * accesses (the launcher checks): the kernel then carries none of the byte-wise
+ * path, whose address arithmetic would otherwise sit in front of both paths. */
+template <int NMOD, bool VEC>
 __global__ __launch_bounds__(256)
 void fast_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t N,
                              FracLimbs fl, double P_over_2_64,
@@ -231,12 +234,13 @@ void fast_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t 
     const uint64_t col = ((uint64_t)(blockIdx.x % cpr) * 256 + threadIdx.x) * 4;
     if (col >= N) return;
     const uint64_t tot = M * N, idx = row * N + col;
-    const int nvalid = (N - col < 4) ? (int)(N - col) : 4;
-    const bool vec = (nvalid == 4) && ((N & 3) == 0) && (((uintptr_t)W & 3) == 0);
+    const int nvalid = VEC ? 4 : ((N - col < 4) ? (int)(N - col) : 4);
+    const bool vec = VEC || ((nvalid == 4) && ((N & 3) == 0) && (((uintptr_t)W & 3) == 0));
     uint32_t u[NMOD];
     if (vec) {
+        const int8_t* p = W + idx;                 /* one address, then a step per plane */
 #pragma unroll
-        for (int l = 0; l < NMOD; l++) u[l] = *(const uint32_t*)(W + (uint64_t)l * tot + idx);
+        for (int l = 0; l < NMOD; l++) { u[l] = *(const uint32_t*)p; p += tot; }
     } else {
 #pragma unroll
         for (int l = 0; l < NMOD; l++) {
@@ -273,7 +277,7 @@ void fast_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t 
         const double f = fma((double)(int32_t)(S >> 32), 4294967296.0, (double)(uint32_t)S);
         out[e] = ldexp(f * P_over_2_64, -(sa + sb[e]));
     }
-    if (vec && (((uintptr_t)C & 15) == 0)) {
+    if (VEC || (vec && (((uintptr_t)C & 15) == 0))) {
         d2_t lo, hi;
         lo.x = out[0]; lo.y = out[1]; hi.x = out[2]; hi.y = out[3];
         ((d2_t*)(C + idx))[0] = lo; ((d2_t*)(C + idx))[1] = hi;
@@ -441,9 +445,14 @@ extern "C" int hip_ozaki_fast_reconstruct_f64(const int8_t* w_planes, uint64_t M
     const uint64_t nblk = (((N + 3) / 4 + 255) / 256) * M;
     if (nblk > 0x7fffffffULL) return -1;
     hipStream_t st = (hipStream_t)stream;
+    const bool vec = (N % 4 == 0) && (((uintptr_t)w_planes & 3) == 0) && (((uintptr_t)C & 15) == 0);
     switch (f.n) {
-#define CASE(n) case n: hipLaunchKernelGGL(fast_reconstruct_kernel<n>, dim3((unsigned)nblk), dim3(256), 0, st, \
-                                           w_planes, M, N, f.limbs, ldexp(f.P, -64), shift_a, shift_b, C); break;
+#define CASE(n) case n:                                                                                          \
+        if (vec) hipLaunchKernelGGL((fast_reconstruct_kernel<n, true>), dim3((unsigned)nblk), dim3(256), 0, st,   \
+                                    w_planes, M, N, f.limbs, ldexp(f.P, -64), shift_a, shift_b, C);               \
+        else hipLaunchKernelGGL((fast_reconstruct_kernel<n, false>), dim3((unsigned)nblk), dim3(256), 0, st,      \
+                                w_planes, M, N, f.limbs, ldexp(f.P, -64), shift_a, shift_b, C);                   \
+        break;
         CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8) CASE(9)
         CASE(10) CASE(11) CASE(12) CASE(13) CASE(14) CASE(15) CASE(16)
 #undef CASE
@@ -512,9 +521,14 @@ extern "C" int hip_matmul_ozaki_fast_f64_ex(const double* A, const double* B, do
 
     const uint64_t nblk = (((N + 3) / 4 + 255) / 256) * M;
     if (nblk > 0x7fffffffULL) return -1;
+    const bool vec = (N % 4 == 0) && (((uintptr_t)Wp & 3) == 0) && (((uintptr_t)C & 15) == 0);
     switch (f.n) {
-#define CASE(n) case n: hipLaunchKernelGGL(fast_reconstruct_kernel<n>, dim3((unsigned)nblk), dim3(256), 0, st, \
-                                           Wp, M, N, f.limbs, ldexp(f.P, -64), sha, shb, C); break;
+#define CASE(n) case n:                                                                                          \
+        if (vec) hipLaunchKernelGGL((fast_reconstruct_kernel<n, true>), dim3((unsigned)nblk), dim3(256), 0, st,   \
+                                    Wp, M, N, f.limbs, ldexp(f.P, -64), sha, shb, C);                             \
+        else hipLaunchKernelGGL((fast_reconstruct_kernel<n, false>), dim3((unsigned)nblk), dim3(256), 0, st,      \
+                                Wp, M, N, f.limbs, ldexp(f.P, -64), sha, shb, C);                                 \
+        break;
         CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8) CASE(9)
         CASE(10) CASE(11) CASE(12) CASE(13) CASE(14) CASE(15) CASE(16)
 #undef CASE
