@@ -47,22 +47,33 @@ struct FastTable {
     uint32_t neg_half[FAST_MAX_MODULI];         /* the byte of -p/2 for even p, else 0x100 (never a byte) */
 };
 
-/* The int8 residue of s modulo p_l as a byte. Two byte dot products give x < 2^19
- * congruent to s; one fma against 1.5 * 2^23 leaves the nearest integer to x/p in
- * the low bits of a float; the low byte of x - (2^22 + q) p is the residue in
- * [-p/2, p/2]. The even moduli are powers of two, their 1/p is exact, so their tie
- * x = p/2 (mod p) comes out as +p/2 or -p/2 with the parity of q: -p/2 is folded
- * to the +p/2 the reference stores (metal_softfloat.h:4174-4177). */
-__device__ __forceinline__ uint32_t fast_residue(Scaled s, const FastTable& t, int l) {
+/* The int8 residues of four integers modulo p_l, packed into a word. Two byte
+ * dot products give x < 2^19 congruent to s; one fma against 1.5 * 2^23 leaves the
+ * nearest integer to x/p in the low bits of a float; the low byte of
+ * x - (2^22 + q) p is the residue in [-p/2, p/2]: five instructions, and the four
+ * low bytes are gathered by two byte permutes and an or. The even moduli are
+ * powers of two, their 1/p is exact, so their tie x = p/2 (mod p) comes out as
+ * +p/2 or -p/2 with the parity of q: -p/2 is folded to the +p/2 the reference
+ * stores (metal_softfloat.h:4174-4177). Only an even modulus pays for that test
+ * (the branch is the same for every lane): there is at most one among the
+ * moduli, and the split is bound by its vector instructions. */
+__device__ __forceinline__ uint32_t fast_residue_raw(Scaled s, const FastTable& t, int l) {
     const uint32_t x = __builtin_amdgcn_udot4(s.lo, t.wlo[l], __builtin_amdgcn_udot4(s.hi, t.whi[l], 0u, false), false);
     const float qm = fmaf((float)x, t.pinv[l], 12582912.0f);
-    uint32_t r = (uint32_t)(__mul24(__float_as_int(qm), -t.p[l]) + (int)x) & 0xffu;
-    if (r == t.neg_half[l]) r = (uint32_t)t.p[l] >> 1;
-    return r;
+    return (uint32_t)(__mul24(__float_as_int(qm), -t.p[l]) + (int)x);         /* the residue is the low byte */
 }
 
-__device__ __forceinline__ uint32_t pack4(uint32_t r0, uint32_t r1, uint32_t r2, uint32_t r3) {
-    return r0 | r1 << 8 | r2 << 16 | r3 << 24;
+__device__ __forceinline__ uint32_t fast_residues4(Scaled s0, Scaled s1, Scaled s2, Scaled s3, const FastTable& t, int l) {
+    uint32_t r0 = fast_residue_raw(s0, t, l), r1 = fast_residue_raw(s1, t, l);
+    uint32_t r2 = fast_residue_raw(s2, t, l), r3 = fast_residue_raw(s3, t, l);
+    if (t.neg_half[l] != 0x100u) {
+        const uint32_t nh = t.neg_half[l], half = (uint32_t)t.p[l] >> 1;
+        r0 = ((r0 & 0xffu) == nh) ? half : r0;
+        r1 = ((r1 & 0xffu) == nh) ? half : r1;
+        r2 = ((r2 & 0xffu) == nh) ? half : r2;
+        r3 = ((r3 & 0xffu) == nh) ? half : r3;
+    }
+    return __builtin_amdgcn_perm(r1, r0, 0x0c0c0400u) | __builtin_amdgcn_perm(r3, r2, 0x04000c0cu);
 }
 
 /* Row-major X[rows][K], pitch a multiple of 16: a block takes 1024 k of one row,
@@ -97,8 +108,7 @@ void fast_split_kernel(const double* __restrict__ X, uint64_t rows, uint64_t K,
 #pragma unroll
     for (int l = 0; l < FAST_MAX_MODULI; l++)
         if (l < tbl.n)
-            stage[l][tid] = pack4(fast_residue(s[0], tbl, l), fast_residue(s[1], tbl, l),
-                                  fast_residue(s[2], tbl, l), fast_residue(s[3], tbl, l));
+            stage[l][tid] = fast_residues4(s[0], s[1], s[2], s[3], tbl, l);
     __syncthreads();
     const uint64_t plane_stride = rows_padded * ldk;
     for (int c = tid; c < tbl.n * 64; c += 256) {
@@ -141,8 +151,7 @@ void fast_split_il_kernel(const double* __restrict__ X, uint64_t rows, uint64_t 
 #pragma unroll
     for (int l = 0; l < FAST_MAX_MODULI; l++)
         if (l < tbl.n)
-            stage[l][tid] = pack4(fast_residue(s[0], tbl, l), fast_residue(s[1], tbl, l),
-                                  fast_residue(s[2], tbl, l), fast_residue(s[3], tbl, l));
+            stage[l][tid] = fast_residues4(s[0], s[1], s[2], s[3], tbl, l);
     __syncthreads();
     const uint64_t plane_stride = rows_padded * ldk;
     int8_t* frag = planes + rb * (32 * ldk) + kb * 1024;
@@ -172,8 +181,7 @@ void fast_split_kmajor_kernel(const double* __restrict__ X, uint64_t rows, uint6
                 v4u_t w;
 #pragma unroll
                 for (int g = 0; g < 4; g++)
-                    w[g] = pack4(fast_residue(s[4 * g], tbl, l), fast_residue(s[4 * g + 1], tbl, l),
-                                 fast_residue(s[4 * g + 2], tbl, l), fast_residue(s[4 * g + 3], tbl, l));
+                    w[g] = fast_residues4(s[4 * g], s[4 * g + 1], s[4 * g + 2], s[4 * g + 3], tbl, l);
                 eshkol_store_streaming((v4u_t*)(out + (uint64_t)l * plane_stride), w);
             }
         });
@@ -200,8 +208,7 @@ void fast_split_kmajor_il_kernel(const double* __restrict__ X, uint64_t rows, ui
         v4u_t w;
 #pragma unroll
         for (int g = 0; g < 4; g++)
-            w[g] = pack4(fast_residue(s[4 * g], tbl, l), fast_residue(s[4 * g + 1], tbl, l),
-                         fast_residue(s[4 * g + 2], tbl, l), fast_residue(s[4 * g + 3], tbl, l));
+            w[g] = fast_residues4(s[4 * g], s[4 * g + 1], s[4 * g + 2], s[4 * g + 3], tbl, l);
         eshkol_store_streaming((v4u_t*)(out + (uint64_t)l * plane_stride), w);
     }
 }
