@@ -38,6 +38,32 @@ def test_reduced_matches_reference_statement(gpu, M, K, N, dtype):
         assert normwise(wide, oracle.matmul_reduced_f32acc(A, B, dtype, False), Ar, Br) <= 1e-6
 
 
+@pytest.mark.parametrize("dtype", [2, 3])
+@pytest.mark.parametrize("M,K,N", [(3072, 256, 3072), (3000, 200, 2900)])
+def test_rounded_output_of_the_kernel_for_large_products(gpu, M, K, N, dtype):
+    """From 128 tiles of 256 x 256 on, the tier's contraction is the kernel that loads its
+    operands straight into LDS and MFMA registers, with an epilogue of its own for every
+    output form. Its rounded f64 output must be its unrounded one rounded to the 16-bit type,
+    value for value: whole tiles (3072^2) and ragged edges, with infinities, an infinity minus
+    infinity and a sum beyond the 16-bit type's range among the results."""
+    print("reduced, large, rounded", M, K, N, dtype, flush=True)
+    A = oracle.reduce_precision(synth.normal(900 + M, (M, K), 1.0 / np.sqrt(K)), dtype)
+    B = oracle.reduce_precision(synth.normal(950 + N, (K, N), 1.0 / np.sqrt(K)), dtype)
+    A[0, 0] = np.inf; B[0, 0] = 1.0                   # row 0: infinities
+    A[1, 0] = np.inf; A[1, 1] = -np.inf; B[0, 1] = 1.0; B[1, 1] = 1.0     # inf - inf: NaN
+    A[2, :] = (65504.0 if dtype == 2 else 1.0e38) / K; B[:, 2] = 2.0      # finite in fp32, beyond f16 once rounded
+    A, B = oracle.reduce_precision(A, dtype), oracle.reduce_precision(B, dtype)
+    wide = run_reduced(A, B, dtype, round_output=False)
+    narrow = run_reduced(A, B, dtype, round_output=True)
+    assert np.isinf(wide[0, 0]) and np.isnan(wide[1, 1]) and np.isfinite(wide[2, 2])
+    if dtype == 2:
+        assert np.isinf(narrow[2, 2])
+    ref = oracle.matmul_f64(A[3:67], B[:, 3:])
+    assert normwise(wide[3:67, 3:], ref, A[3:67], B[:, 3:]) <= 1e-6
+    ok = (np.abs(wide) >= 2.0 ** -14) | (wide == 0) | np.isnan(wide)    # outside the reference's f16 subnormal quirk
+    assert np.array_equal(narrow[ok], oracle.reduce_precision(wide, dtype)[ok], equal_nan=True)
+
+
 @pytest.mark.parametrize("is_bf16", [0, 1])
 def test_device_narrowing_is_round_to_nearest_even(gpu, is_bf16):
     lib = ea.load()
