@@ -78,8 +78,11 @@ constexpr int32_t CRT_FL_ZERO = INT32_MIN;      /* exponent entry of a maximum o
  * library's own behind everything queued on st so far: what follows on st does
  * not wait for it. The summary is written to host memory by the device; ask for
  * it after queueing the rest of the pipeline. Returns the summary's ticket, 0 on
- * failure. For callers whose shifts came with the maxima (above). */
-uint32_t eshkol_crt_scan_launch_aside(const double* amax, uint64_t M, const double* bmax, uint64_t N, hipStream_t st);
+ * failure. For callers whose shifts came with the maxima (above). For a small
+ * product (operand_elems = M K + K N) the scan is queued on st itself: there the
+ * device waits for the host, and three calls cost more than ten microseconds in line. */
+uint32_t eshkol_crt_scan_launch_aside(const double* amax, uint64_t M, const double* bmax, uint64_t N, hipStream_t st,
+                                      uint64_t operand_elems);
 /* The two CRT tiers print one marker line per call, as the reference does per
  * dispatch (gpu_memory.mm:2503; its gates count those lines). A dispatcher that
  * runs one product as several calls (row panels) lets the first call print and

@@ -668,9 +668,15 @@ uint32_t scan_launch(const double* amax, uint64_t M, const double* bmax, uint64_
     return ESHKOL_HIP_OK(hipGetLastError()) ? ticket : 0;
 }
 /* The same scan for its summary alone, on the library's side stream behind what
- * st holds so far. */
-uint32_t scan_launch_aside(const double* amax, uint64_t M, const double* bmax, uint64_t N, hipStream_t st) {
+ * st holds so far. operand_elems = M K + K N of the product: below ASIDE_FROM the
+ * pipeline's kernels last a few microseconds each and the device waits for the
+ * host to queue them, so the event, the wait and the launch on a second stream
+ * cost more (three calls) than the scan's ten microseconds in line do. */
+constexpr uint64_t ASIDE_FROM = 6u << 20;
+uint32_t scan_launch_aside(const double* amax, uint64_t M, const double* bmax, uint64_t N, hipStream_t st,
+                           uint64_t operand_elems) {
     if (!ensure_mailbox()) return 0;
+    if (operand_elems < ASIDE_FROM) return scan_launch(amax, M, bmax, N, nullptr, nullptr, st);
     if (!ESHKOL_HIP_OK(hipEventRecord(g_scan_event, st)) ||
         !ESHKOL_HIP_OK(hipStreamWaitEvent(g_scan_stream, g_scan_event, 0))) return 0;
     return scan_launch(amax, M, bmax, N, nullptr, nullptr, g_scan_stream);
@@ -754,8 +760,9 @@ static int g_crt_quiet = 0;
 void eshkol_crt_set_quiet(int quiet) { g_crt_quiet = quiet; }
 int eshkol_crt_quiet(void) { return g_crt_quiet; }
 
-uint32_t eshkol_crt_scan_launch_aside(const double* amax, uint64_t M, const double* bmax, uint64_t N, hipStream_t st) {
-    return scan_launch_aside(amax, M, bmax, N, st);
+uint32_t eshkol_crt_scan_launch_aside(const double* amax, uint64_t M, const double* bmax, uint64_t N, hipStream_t st,
+                                      uint64_t operand_elems) {
+    return scan_launch_aside(amax, M, bmax, N, st, operand_elems);
 }
 
 int eshkol_crt_scan_result(uint32_t ticket, CrtMaxima out[2], hipStream_t st) {
@@ -924,7 +931,8 @@ static int crt_matmul_impl(const double* A, const double* B, double* C,
     if (!use_prepared &&
         (b_kmajor ? eshkol_colabsmax_shift_f64(B, K, N, 0.0, bmax, nu_out, 52, st)
                   : eshkol_rowabsmax_shift_f64(B, N, K, 0.0, bmax, nu_out, 52, st)) != 0) return -1;
-    const uint32_t ticket = fixed_E ? scan_launch_aside(amax, M, bmax, N, st) : scan_launch(amax, M, bmax, N, dmu, dnu, st);
+    const uint32_t ticket = fixed_E ? scan_launch_aside(amax, M, bmax, N, st, M * K + K * N)
+                                    : scan_launch(amax, M, bmax, N, dmu, dnu, st);
     if (!ticket) return -1;
 
     /* Everything after the shifts, queued in one go. */
