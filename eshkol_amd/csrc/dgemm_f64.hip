@@ -148,8 +148,8 @@ __device__ __forceinline__ void tile_of_index(int L, int tiles_m, int tiles_n, i
 
 /* Workgroup -> position in the tile order: XCD x (workgroups x, x+8, ...) takes
  * the x-th eighth of the launch's positions, so neighbours in the order share an L2. */
-__device__ __forceinline__ void tile_of_workgroup(int tiles_m, int tiles_n, int* tm, int* tn) {
-    const int nwg = gridDim.x, wg = blockIdx.x;
+__device__ __forceinline__ void tile_of_workgroup(int nwg, int tiles_m, int tiles_n, int* tm, int* tn) {
+    const int wg = blockIdx.x;
     const int q = nwg >> 3, r = nwg & 7;
     const int xcd = wg & 7, seq = wg >> 3;
     const int L = xcd * q + (xcd < r ? xcd : r) + seq;
@@ -176,7 +176,7 @@ void dgemm_mfma_kernel(const double* __restrict__ A, const double* __restrict__ 
     C += (size_t)blockIdx.y * M * N;
 
     int tm, tn;
-    tile_of_workgroup(tiles_m, tiles_n, &tm, &tn);
+    tile_of_workgroup((int)gridDim.x, tiles_m, tiles_n, &tm, &tn);
     const int m0 = tm * BM, n0 = tn * BN;
 
     const int tid = threadIdx.x;
@@ -276,10 +276,13 @@ __device__ __forceinline__ void lds_only_barrier() {
 }
 
 /* SPLIT: the launch covers the last `tail` tiles of the tile order, each cut
- * along k into pieces of kb_per_piece k-blocks; workgroup piece * tail + i
- * multiplies piece `piece` of tail tile i and leaves the whole 128 x 128 partial
- * tile in `partial` (dgemm_fixup_kernel adds the pieces up in order). */
-struct SplitArgs { int first_tile, tail, kb_per_piece; double* partial; };
+ * along k into pieces of kb_per_piece k-blocks; workgroup whole + piece * tail + i
+ * multiplies piece `piece` of tail tile i and leaves the whole partial tile in
+ * `partial` (dgemm_fixup_kernel adds the pieces up in order). The first `whole`
+ * workgroups of such a launch compute the tiles at positions 0 .. whole - 1 of
+ * the tile order whole, as an unsplit launch of `whole` workgroups would (small
+ * tiles only; 0 for large ones). */
+struct SplitArgs { int first_tile, tail, kb_per_piece; double* partial; int whole; };
 
 template <bool TA, bool TB, bool KTAIL, bool SPLIT, int TS = 128, int PF = 1>
 __global__ __launch_bounds__(256, TS == 128 ? 2 : 4)
@@ -295,7 +298,7 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
      * or a step is 1024 cycles long. With 2 (two staging sets, block j in set
      * j % 2) it has a whole k-block more: for the small tile, whose step is 256
      * cycles, when a CU holds one workgroup. */
-    static_assert(TS == 128 || (TS == 64 && !SPLIT), "cut tiles are 128 x 128");
+    static_assert(TS == 128 || TS == 64, "tile edges");
     static_assert(PF == 1 || PF == 2, "one or two staging sets");
     constexpr int BM = TS, BN = TS;
     constexpr int TT = TS / 32;                  /* 16 x 16 MFMA tiles per wave and dimension */
@@ -311,8 +314,13 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
     C += (size_t)blockIdx.y * M * N;
 
     int tm, tn;
-    if (SPLIT) tile_of_index(sp.first_tile + (int)(blockIdx.x % (unsigned)sp.tail), tiles_m, tiles_n, &tm, &tn);
-    else tile_of_workgroup(tiles_m, tiles_n, &tm, &tn);
+    /* in a cut launch: this workgroup multiplies a piece (else one of the leading whole
+     * tiles, which only launches of small tiles have: the large tile's cut variants
+     * have no register to spare for the distinction) */
+    const bool is_piece = SPLIT && (TS == 128 || (int)blockIdx.x >= sp.whole);
+    const int piece_wg = !SPLIT ? 0 : (TS == 128) ? (int)blockIdx.x : (int)blockIdx.x - sp.whole;
+    if (is_piece) tile_of_index(sp.first_tile + (int)((unsigned)piece_wg % (unsigned)sp.tail), tiles_m, tiles_n, &tm, &tn);
+    else tile_of_workgroup(SPLIT ? sp.whole : (int)gridDim.x, tiles_m, tiles_n, &tm, &tn);
     const int m0 = tm * BM, n0 = tn * BN;
 
     const int tid = threadIdx.x;
@@ -411,9 +419,9 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
 
     /* this workgroup's k-blocks [kb_lo, kb_hi): all of them unless the tile is split */
     const int nkb_all = (K + BK - 1) / BK;
-    const int piece = SPLIT ? (int)(blockIdx.x / (unsigned)sp.tail) : 0;
-    const int kb_lo = SPLIT ? piece * sp.kb_per_piece : 0;
-    const int kb_hi = SPLIT ? ((kb_lo + sp.kb_per_piece < nkb_all) ? kb_lo + sp.kb_per_piece : nkb_all) : nkb_all;
+    const int piece = is_piece ? (int)((unsigned)piece_wg / (unsigned)sp.tail) : 0;
+    const int kb_lo = is_piece ? piece * sp.kb_per_piece : 0;
+    const int kb_hi = is_piece ? ((kb_lo + sp.kb_per_piece < nkb_all) ? kb_lo + sp.kb_per_piece : nkb_all) : nkb_all;
     auto clamped = [&](int kb) { return kb < kb_hi ? kb : kb_hi - 1; };   /* requests past the end are never consumed */
     gload(kb_lo, I0{}, I1{});
     a[0].sstore(As, tid);
@@ -519,15 +527,15 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
         if (kb < kb_hi) block(kb, I0{}, I0{});
     }
 
-    if constexpr (SPLIT) {
-        double* out = sp.partial + (size_t)blockIdx.x * (BM * BN);
+    if (is_piece) {
+        double* out = sp.partial + (size_t)piece_wg * (BM * BN);
 #pragma unroll
         for (int t = 0; t < TT; t++)
 #pragma unroll
             for (int u = 0; u < TT; u++)
 #pragma unroll
                 for (int r = 0; r < 4; r++)
-                    out[(wm * 64 + t * 16 + 4 * r + lg) * BN + wn * 64 + u * 16 + li] = acc[t][u][r];
+                    out[(wm * (BM / 2) + t * 16 + 4 * r + lg) * BN + wn * (BN / 2) + u * 16 + li] = acc[t][u][r];
         return;
     }
 #pragma unroll
@@ -544,22 +552,25 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
 }
 
 /* Adds up the partial tiles of dgemm_fast_kernel<..., SPLIT>: piece 0 first, so the
- * result does not depend on which workgroup finished when. grid (tail, 16): a
- * workgroup sums eight rows of one tile, a thread four consecutive columns. */
+ * result does not depend on which workgroup finished when. TS: the tile's edge.
+ * grid (tail, TS / (1024 / TS)): a thread sums four consecutive columns of a row,
+ * TS / 4 threads a row, a workgroup 1024 / TS rows of one tile. */
+template <int TS>
 __global__ __launch_bounds__(256)
 void dgemm_fixup_kernel(const double* __restrict__ partial, int tail, int pieces, int first_tile,
                         int tiles_m, int tiles_n, double* __restrict__ C, int M, int N) {
+    constexpr int PER_ROW = TS / 4, ROWS = 256 / PER_ROW;
     int tm, tn;
     tile_of_index(first_tile + (int)blockIdx.x, tiles_m, tiles_n, &tm, &tn);
-    const int lrow = (int)blockIdx.y * 8 + (threadIdx.x >> 5), lcol = 4 * (threadIdx.x & 31);
-    const double* p = partial + (size_t)blockIdx.x * (128 * 128) + lrow * 128 + lcol;
+    const int lrow = (int)blockIdx.y * ROWS + (int)(threadIdx.x / PER_ROW), lcol = 4 * (int)(threadIdx.x % PER_ROW);
+    const double* p = partial + (size_t)blockIdx.x * (TS * TS) + lrow * TS + lcol;
     d2_t s0 = *(const d2_t*)p, s1 = *(const d2_t*)(p + 2);
     for (int q = 1; q < pieces; q++) {
-        const double* pq = p + (size_t)q * tail * (128 * 128);
+        const double* pq = p + (size_t)q * tail * (TS * TS);
         const d2_t v0 = *(const d2_t*)pq, v1 = *(const d2_t*)(pq + 2);
         s0.x += v0.x; s0.y += v0.y; s1.x += v1.x; s1.y += v1.y;
     }
-    const int row = tm * 128 + lrow, col = tn * 128 + lcol;
+    const int row = tm * TS + lrow, col = tn * TS + lcol;
     if (row >= M) return;
     double* c = C + (size_t)row * N + col;
     if (col < N) c[0] = s0.x;
@@ -638,10 +649,34 @@ double large_tile_us(long long nwg, int nkb, bool may_cut) {
     return US_LAUNCH + US_KB_128 * nkb * (double)((nwg + cus - 1) / cus);
 }
 
-double small_tile_us(long long nwg64, int nkb) {
+/* Small tiles beyond the last multiple of the CU count make some CUs work a whole
+ * tile longer than the others (1536^3: 576 tiles on 256 CUs, three on some, two on
+ * most). Those leftover tiles are cut along k into p pieces each, in the same
+ * launch behind the whole tiles, so that every CU gets a piece or so of them:
+ * pieces per leftover tile (1 = whole) and the launch's expected time, which is
+ * the fullest CU's whole tiles and pieces plus 8 us for the launch that adds the
+ * pieces up and the partial tiles' round trip. */
+int small_tile_tail_pieces(long long nwg64, int nkb, bool may_cut, double* us = nullptr) {
     const int cus = eshkol_hip_num_cus();
+    const long long full = nwg64 / cus, rem = nwg64 % cus;
     const long long per_cu = (nwg64 + cus - 1) / cus;
-    return US_LAUNCH + (per_cu <= 1 ? US_KB_64_ALONE : US_KB_64) * nkb * (double)per_cu;
+    double best = US_LAUNCH + (per_cu <= 1 ? US_KB_64_ALONE : US_KB_64) * nkb * (double)per_cu;
+    int best_p = 1;
+    if (may_cut && full >= 1 && rem > 0) {
+        for (int p = 2; p <= 16 && nkb / p >= 4; p++) {
+            const long long rounds = (p * rem + cus - 1) / cus;
+            const double cost = US_LAUNCH + 8.0 + US_KB_64 * nkb * ((double)full + (double)rounds / p) + 0.5 * (double)rounds;
+            if (cost < 0.95 * best && (best_p == 1 || cost < best)) { best = cost; best_p = p; }
+        }
+    }
+    if (us) *us = best;
+    return best_p;
+}
+
+double small_tile_us(long long nwg64, int nkb, bool may_cut) {
+    double us;
+    small_tile_tail_pieces(nwg64, nkb, may_cut, &us);
+    return us;
 }
 
 /* 0 (default) and 2: global loads two k-blocks ahead of their LDS writes wherever that
@@ -669,7 +704,7 @@ int launch_fast_k(const double* A, const double* B, double* C, int M, int N, int
     const int tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
     const long long nwg = (long long)tiles_m * tiles_n;
     if (nwg > 0x7fffffffLL || batch < 1 || batch > 65535) return -1;
-    SplitArgs sp = {0, 1, 0, nullptr};
+    SplitArgs sp = {0, 1, 0, nullptr, 0};
 
     /* Two workgroups fit on a CU, so a launch runs in rounds of `slots` tiles, and
      * a last round of a few tiles takes as long as a full one. Its tiles are
@@ -692,7 +727,7 @@ int launch_fast_k(const double* A, const double* B, double* C, int M, int N, int
                                A, B, C, M, N, K, tiles_m, tiles_n, sp);
             hipLaunchKernelGGL(kern_split, dim3((unsigned)(tail * pieces), 1), dim3(256), SMEM_BYTES, st,
                                A, B, C, M, N, K, tiles_m, tiles_n, sp);
-            hipLaunchKernelGGL(dgemm_fixup_kernel, dim3((unsigned)tail, 16), dim3(256), 0, st,
+            hipLaunchKernelGGL(dgemm_fixup_kernel<128>, dim3((unsigned)tail, 16), dim3(256), 0, st,
                                ws, tail, pieces, sp.first_tile, tiles_m, tiles_n, C, M, N);
             return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
         }
@@ -710,7 +745,7 @@ int launch_fast_k(const double* A, const double* B, double* C, int M, int N, int
             sp.first_tile = 0; sp.tail = (int)nwg; sp.kb_per_piece = kbpp; sp.partial = ws;
             hipLaunchKernelGGL(kern_split, dim3((unsigned)(nwg * pieces), 1), dim3(256), SMEM_BYTES, st,
                                A, B, C, M, N, K, tiles_m, tiles_n, sp);
-            hipLaunchKernelGGL(dgemm_fixup_kernel, dim3((unsigned)nwg, 16), dim3(256), 0, st,
+            hipLaunchKernelGGL(dgemm_fixup_kernel<128>, dim3((unsigned)nwg, 16), dim3(256), 0, st,
                                ws, (int)nwg, pieces, 0, tiles_m, tiles_n, C, M, N);
             return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
         }
@@ -736,7 +771,28 @@ int launch_fast64_k(const double* A, const double* B, double* C, int M, int N, i
     const int tiles_m = (M + 63) / 64, tiles_n = (N + 63) / 64;
     const long long nwg = (long long)tiles_m * tiles_n;
     if (nwg > 0x7fffffffLL || batch < 1 || batch > 65535) return -1;
-    const SplitArgs sp = {0, 1, 0, nullptr};
+    SplitArgs sp = {0, 1, 0, nullptr, 0};
+    /* leftover tiles cut along k, in one launch with the whole ones (small_tile_tail_pieces) */
+    const int nkb = (K + BK - 1) / BK;
+    const int p = small_tile_tail_pieces(nwg, nkb, g_tail_split && batch == 1);
+    if (p >= 2) {
+        const int cus = eshkol_hip_num_cus();
+        const int tail = (int)(nwg % cus), whole = (int)(nwg - tail);
+        const int kbpp = (nkb + p - 1) / p;
+        const int pieces = (nkb + kbpp - 1) / kbpp;
+        double* ws = pieces >= 2 ? (double*)eshkol_hip_workspace(WS_DGEMM_PARTIAL,
+                                         (size_t)tail * pieces * 64 * 64 * sizeof(double)) : nullptr;
+        if (ws) {
+            auto kern_cut = g_prefetch_depth == 1 ? dgemm_fast_kernel<TA, TB, KTAIL, true, 64, 1>
+                                                  : dgemm_fast_kernel<TA, TB, KTAIL, true, 64, 2>;
+            sp.first_tile = whole; sp.tail = tail; sp.kb_per_piece = kbpp; sp.partial = ws; sp.whole = whole;
+            hipLaunchKernelGGL(kern_cut, dim3((unsigned)(whole + tail * pieces), 1), dim3(256), SMEM_BYTES, st,
+                               A, B, C, M, N, K, tiles_m, tiles_n, sp);
+            hipLaunchKernelGGL(dgemm_fixup_kernel<64>, dim3((unsigned)tail, 4), dim3(256), 0, st,
+                               ws, tail, pieces, whole, tiles_m, tiles_n, C, M, N);
+            return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+        }
+    }
     hipLaunchKernelGGL(kern, dim3((unsigned)nwg, (unsigned)batch), dim3(256), SMEM_BYTES, st,
                        A, B, C, M, N, K, tiles_m, tiles_n, sp);
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
@@ -796,7 +852,7 @@ int launch_shape(const double* A, const double* B, double* C, int m, int n, int 
      * a cut last round, where the fits call it even) */
     if (straight && (g_small_tile == 2 ||
                      (g_small_tile == 1 && big_tiles < 4LL * eshkol_hip_num_cus() &&
-                      small_tile_us(small_tiles, nkb) < large_tile_us(big_tiles, nkb, may_cut))))
+                      small_tile_us(small_tiles, nkb, may_cut) < large_tile_us(big_tiles, nkb, may_cut))))
         return launch_fast64<TA, TB>(A, B, C, m, n, k, batch, st);
     if (g_fast_path && (big_tiles >= 192 || cut) && vec && m >= 2 && n >= 2 && k >= BK)
         return launch_fast<TA, TB>(A, B, C, m, n, k, batch, st);

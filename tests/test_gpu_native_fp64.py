@@ -250,6 +250,47 @@ def test_small_tile_kernel_gives_the_bits_of_the_large_one(gpu, M, K, N):
         lib.hip_dgemm_set_small_tile(1)
 
 
+@pytest.mark.parametrize("M,K,N", [(1536, 1024, 1536), (1280, 1288, 1280), (1300, 2000, 1250), (1792, 1024, 1800)])
+def test_k_split_of_the_small_tiles_left_over(gpu, M, K, N):
+    """64 x 64 tiles beyond the last multiple of the CU count are cut along k, in the same
+    launch behind the whole ones, and their pieces added in a fixed order. Same result on
+    every run, the whole tiles bit-identical to an uncut launch, everything within the
+    tier's bound, nothing stored outside C; for all three operand forms, with edge tiles
+    and k-tails."""
+    import eshkol_amd as ea
+    from gpu_util import stream
+    lib = ea.load()
+    A, B = synth.normal(M + 17 * K, (M, K)), synth.normal(K + 17 * N, (K, N))
+    ref = oracle.matmul_f64(A, B)
+    forms = [(A, B, 0, 0), (A, np.ascontiguousarray(B.T), 0, 1), (np.ascontiguousarray(A.T), B, 1, 0)]
+    for X, Y, ta, tb in forms:
+        dX, dY = ea.DeviceArray.from_host(X), ea.DeviceArray.from_host(Y)
+        outs = []
+        try:
+            lib.hip_dgemm_set_small_tile(2)
+            for split in (0, 1, 1):
+                lib.hip_dgemm_set_tail_split(split)
+                guard = np.full((M + 2, N), np.nan)
+                guard[0] = guard[-1] = 12345.0
+                dC = ea.DeviceArray.from_host(guard)
+                assert lib.hip_dgemm_f64_ex(dX.ptr, dY.ptr, dC.ptr + N * 8, M, K, N, ta, tb, stream()) == 0
+                ea.synchronize()
+                got = dC.download()
+                assert np.all(got[0] == 12345.0) and np.all(got[-1] == 12345.0)
+                outs.append(got[1:-1])
+        finally:
+            lib.hip_dgemm_set_tail_split(1)
+            lib.hip_dgemm_set_small_tile(1)
+        whole, cut, again = outs
+        assert np.array_equal(cut, again), (ta, tb)
+        same = (whole == cut)
+        assert not same.all(), "the launch was expected to cut its leftover tiles"
+        assert same.mean() > 0.5                      # the whole tiles are untouched
+        assert np.isfinite(cut).all()
+        assert normwise(cut, ref, A, B) <= TOL, (ta, tb)
+        assert normwise(cut, whole, A, B) <= 1e-14
+
+
 @pytest.mark.parametrize("M,K,N", [(1024, 1024, 1024), (2304, 512, 2304), (3072, 640, 3072), (520, 4096, 500), (2048, 2048, 2048),
                                    (4096, 256, 4100), (300, 1002, 1100)])
 def test_the_tile_size_chosen_by_itself_changes_no_bits_of_whole_tiles(gpu, M, K, N):
