@@ -475,7 +475,7 @@ def main():
     #      gpu_memory_cuda.cpp:454-461), N(0,1) operands resident in HBM -------------------------------
     if "sizes" in want:
         sweep = {}
-        for m in (1024, 2048, 4096):
+        for m in (1024, 1536, 2048, 3072, 4096):
             if m >= n:
                 continue
             sa, sb_, sc = ea.DeviceArray((m, m)), ea.DeviceArray((m, m)), ea.DeviceArray((m, m))
