@@ -666,7 +666,8 @@ int small_tile_tail_pieces(long long nwg64, int nkb, bool may_cut, double* us = 
         for (int p = 2; p <= 16 && nkb / p >= 4; p++) {
             const long long rounds = (p * rem + cus - 1) / cus;
             const double cost = US_LAUNCH + 8.0 + US_KB_64 * nkb * ((double)full + (double)rounds / p) + 0.5 * (double)rounds;
-            if (cost < 0.95 * best && (best_p == 1 || cost < best)) { best = cost; best_p = p; }
+            /* cutting must beat the whole launch by 5 per cent; among cuts the cheapest wins */
+            if (best_p == 1 ? cost < 0.95 * best : cost < best) { best = cost; best_p = p; }
         }
     }
     if (us) *us = best;
