@@ -199,6 +199,8 @@ def hip_runtime():
     h.hipMemset.argtypes = [vp, C.c_int, C.c_size_t]
     h.hipDeviceSynchronize.restype = C.c_int
     h.hipStreamSynchronize.argtypes = [vp]
+    h.hipStreamCreate.argtypes = [C.POINTER(vp)]
+    h.hipStreamDestroy.argtypes = [vp]
     h.hipEventCreate.argtypes = [C.POINTER(vp)]
     h.hipEventRecord.argtypes = [vp, vp]
     h.hipEventSynchronize.argtypes = [vp]

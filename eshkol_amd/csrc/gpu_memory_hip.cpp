@@ -294,10 +294,10 @@ int hip_alloc(size_t size_bytes, EshkolMemoryType mem_type, EshkolGPUBuffer* out
     return 0;
 }
 
-/* Staged wrap: device copy of caller-owned host memory. Registration of
- * existing host memory is not available on the target machines, so this is the
- * reference's fallback branch (gpu_memory_cuda.cpp:811-820). */
 /* ---- device copies of host tensors -------------------------------------------
+ * A wrapped host buffer is a device copy of caller-owned memory: registration of
+ * existing host memory is not available on the target machines, so this is the
+ * reference's fallback branch (gpu_memory_cuda.cpp:811-820).
  * Staging pool: the device side of a wrapped host buffer comes from a small
  * cache of earlier allocations, so a matmul on host memory does not pay
  * hipMalloc/hipFree (each a device-wide synchronisation) per operand per call.
@@ -698,26 +698,30 @@ hipStream_t eshkol_hip_stream(void) { return g_stream; }
 
 namespace {
 int g_call_depth = 0;                    /* guarded by g_gpu_mutex */
-hipEvent_t g_ev_last_call = nullptr;     /* end of the previous bracketed call's work */
 hipStream_t g_last_call_stream = nullptr;
-bool g_last_call_recorded = false;
+bool g_last_call_pending = false;        /* a bracketed call has queued work on g_last_call_stream */
 }
 
+/* Calls share the workspaces, so the work of one must be over before the next
+ * touches them. On one stream the stream's own order sees to that and nothing
+ * is queued for it: an event recorded behind every call put a marker between
+ * any two kernels of consecutive calls, and the device spends 5-7 us on each.
+ * A call that arrives on another stream than the one before it waits on the
+ * host until the device has drained (the earlier stream may be gone by then,
+ * so the wait names no stream). */
 void eshkol_hip_enter(hipStream_t stream) {
     g_gpu_mutex.lock();
     if (++g_call_depth != 1) return;
-    if (g_last_call_recorded && g_last_call_stream != stream)
-        (void)hipStreamWaitEvent(stream, g_ev_last_call, 0);
+    if (g_last_call_pending && g_last_call_stream != stream) {
+        if (!ESHKOL_HIP_OK(hipDeviceSynchronize())) (void)hipGetLastError();
+        g_last_call_pending = false;
+    }
 }
 
 void eshkol_hip_leave(hipStream_t stream) {
     if (--g_call_depth == 0) {
-        if (!g_ev_last_call && !ESHKOL_HIP_OK(hipEventCreateWithFlags(&g_ev_last_call, hipEventDisableTiming))) {
-            (void)hipGetLastError();
-            g_ev_last_call = nullptr;
-        }
-        g_last_call_recorded = g_ev_last_call && ESHKOL_HIP_OK(hipEventRecord(g_ev_last_call, stream));
         g_last_call_stream = stream;
+        g_last_call_pending = true;
     }
     g_gpu_mutex.unlock();
 }
@@ -812,8 +816,7 @@ void eshkol_gpu_shutdown(void) {
         if (g_copy_stream) hipStreamSynchronize(g_copy_stream);
         release_copy_queue();
         if (g_stream) { hipStreamDestroy(g_stream); g_stream = nullptr; }
-        if (g_ev_last_call) { hipEventDestroy(g_ev_last_call); g_ev_last_call = nullptr; }
-        g_last_call_recorded = false; g_last_call_stream = nullptr;
+        g_last_call_pending = false; g_last_call_stream = nullptr;
     }
     g_backend = ESHKOL_GPU_NONE;
     g_initialized.store(false, std::memory_order_release);

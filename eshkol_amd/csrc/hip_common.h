@@ -44,8 +44,8 @@ void  eshkol_hip_workspace_release(void);
 
 /* Brackets a public tier entry point (hip_matmul_*, hip_dgemm_*, hip_igemm_i8,
  * hip_colabsmax_f64): takes the library's recursive mutex, the one the eshkol_*
- * entry points hold, and orders `stream` behind the stream the previous bracketed
- * call queued its work on. The tiers share the grow-only workspace, the scan
+ * entry points hold, and, if the previous bracketed call queued its work on
+ * another stream, waits until the device is idle. The tiers share the grow-only workspace, the scan
  * mailbox and per-process tables; with the bracket, callers on several threads
  * or streams are serialised on the host and their kernels on the device. */
 void eshkol_hip_enter(hipStream_t stream);

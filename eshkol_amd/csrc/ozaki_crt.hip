@@ -631,7 +631,7 @@ bool ensure_mailbox() {
     void* h = nullptr;
     void* d = nullptr;
     if (!g_scan_stream && !ESHKOL_HIP_OK(hipStreamCreateWithFlags(&g_scan_stream, hipStreamNonBlocking))) return false;
-    if (!g_scan_event && !ESHKOL_HIP_OK(hipEventCreateWithFlags(&g_scan_event, hipEventDisableTiming))) return false;
+    if (!g_scan_event && !ESHKOL_HIP_OK(hipEventCreateWithFlags(&g_scan_event, hipEventDisableTiming | hipEventReleaseToDevice))) return false;
     if (!ESHKOL_HIP_OK(hipHostMalloc(&h, 2 * sizeof(CrtScan), hipHostMallocMapped))) return false;
     if (!ESHKOL_HIP_OK(hipHostGetDevicePointer(&d, h, 0))) { (void)hipHostFree(h); return false; }
     memset(h, 0, 2 * sizeof(CrtScan));

@@ -21,9 +21,10 @@
  * device workspace and per-process tables. Each of them takes the library's
  * one recursive mutex (the same the eshkol_* entry points hold) for the length
  * of the call and, when its stream differs from the stream of the previous such
- * call, makes its stream wait for that call's work: they may be called from any
- * thread, on any stream, beside eshkol_* calls, and are serialised on the host
- * and on the device. The stage launchers (split, slice, convert, reconstruct,
+ * call, first waits on the host until the device is idle (consecutive calls on
+ * one stream, the usual case, are ordered by the stream and pay nothing): they
+ * may be called from any thread, on any stream, beside eshkol_* calls, and are
+ * serialised on the host and on the device. The stage launchers (split, slice, convert, reconstruct,
  * rowabsmax, transpose, elementwise, bias) touch only the memory they are
  * given and take no lock. The hip_*_set_* switches are process-wide tuning
  * hooks read by later calls: set them before other threads are inside the

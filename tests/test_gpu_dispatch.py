@@ -382,6 +382,60 @@ def test_concurrent_callers_serialise_on_the_library(gpu):
                 assert normwise(want[i], oracle.matmul_f64(a, b), a, b) <= 1e-14
 
 
+def test_calls_that_change_streams_wait_for_the_call_before(gpu):
+    """The tier pipelines share one workspace (planes, partial sums), so a call on
+    another stream than the call before it must not start before that call's work
+    is over. Products queued alternately on two streams of the caller and on the
+    library's, with no synchronisation of the caller's between them, give the bits
+    of the same products made one at a time, and so does a call made after a
+    stream it followed has been destroyed."""
+    lib = ea.init(); hip = ea.hip_runtime()
+    streams = [C.c_void_p(), C.c_void_p()]
+    for s in streams:
+        assert hip.hipStreamCreate(C.byref(s)) == 0
+    own = C.c_void_p(lib.eshkol_hip_get_stream())
+    shapes = [(1024, 1024, 1024), (768, 512, 640), (1536, 1024, 1280), (512, 2048, 512)]
+    ops = [(ea.DeviceArray.from_host(synth.normal(60 + i, (m, k))), ea.DeviceArray.from_host(synth.normal(70 + i, (k, n))))
+           for i, (m, k, n) in enumerate(shapes)]
+
+    def product(kind, i, stream, out):
+        m, k, n = shapes[i]
+        a, b = ops[i]
+        if kind == 0:
+            return lib.hip_dgemm_f64(a.ptr, b.ptr, out.ptr, m, k, n, stream)
+        if kind == 1:
+            return lib.hip_matmul_ozaki_crt_f64(a.ptr, b.ptr, out.ptr, m, k, n, 16, 0, None, 0, stream)
+        return lib.hip_matmul_ozaki_int8_f64(a.ptr, b.ptr, out.ptr, m, k, n, 4, stream)
+
+    plan = [(kind, i) for kind in (1, 0, 2) for i in range(len(shapes))]
+    want = []
+    for kind, i in plan:                                   # one at a time on the library's stream
+        out = ea.DeviceArray((shapes[i][0], shapes[i][2]))
+        assert product(kind, i, own, out) == 0
+        assert hip.hipDeviceSynchronize() == 0
+        want.append(out.download()); out.free()
+    outs = [ea.DeviceArray((shapes[i][0], shapes[i][2])) for _, i in plan]
+    order = [streams[0], streams[1], own]
+    for j, (kind, i) in enumerate(plan):                   # back to back, the stream changing every call
+        assert product(kind, i, order[j % 3], outs[j]) == 0
+    assert hip.hipDeviceSynchronize() == 0
+    for j, (kind, i) in enumerate(plan):
+        assert np.array_equal(outs[j].download(), want[j]), (kind, shapes[i])
+    # a stream that is gone by the time the next call arrives
+    assert product(1, 0, streams[1], outs[0]) == 0
+    assert hip.hipStreamSynchronize(streams[1]) == 0 and hip.hipStreamDestroy(streams[1]) == 0
+    assert product(1, 1, streams[0], outs[1]) == 0
+    assert hip.hipStreamSynchronize(streams[0]) == 0
+    assert np.array_equal(outs[0].download(), want[0]) and np.array_equal(outs[1].download(), want[1])
+    assert hip.hipStreamDestroy(streams[0]) == 0
+    assert product(0, 2, own, outs[6]) == 0 and hip.hipDeviceSynchronize() == 0
+    assert np.array_equal(outs[6].download(), want[6])
+    for o in outs:
+        o.free()
+    for a, b in ops:
+        a.free(); b.free()
+
+
 def test_batched_native_kernel(gpu):
     """hip_dgemm_f64_batched against the oracle's batch loop: even and odd shapes
     (the odd ones leave matrices of the batch off 16-byte boundaries), integer
