@@ -18,6 +18,7 @@
 #include "hip_common.h"
 #include "kernels.h"
 #include "kmajor_tile.h"
+#include "crt_shared.h"
 
 #include <cmath>
 #include <cstring>
@@ -205,20 +206,29 @@ void reconstruct_kernel(double* __restrict__ C, const int32_t* __restrict__ Gall
         if (e < nvalid) C[idx + e] = (acc[e] * r) * cmax[col + e];
 }
 
-void* g_pinned = nullptr;
-size_t g_pinned_bytes = 0;
-void* pinned(size_t bytes) {
-    if (g_pinned_bytes >= bytes) return g_pinned;
-    if (g_pinned) hipHostFree(g_pinned);
-    g_pinned = nullptr; g_pinned_bytes = 0;
-    if (!ESHKOL_HIP_OK(hipHostMalloc(&g_pinned, bytes, hipHostMallocDefault))) return nullptr;
-    g_pinned_bytes = bytes;
-    return g_pinned;
-}
-
 HipOzakiInt8Stages g_last = {};
 
 constexpr int MAX_BUF = 128, MAX_PAIRS = 128;
+
+/* The buffer plan of a call (gpu_memory_cuda.cpp:367-389): weight and pair list
+ * of every int32 product buffer. It depends on T and K alone, so the device
+ * keeps the last one and a call uploads it only when it differs (guarded by the
+ * library mutex every entry point holds). */
+struct Plan { double w[MAX_BUF]; int32_t first[MAX_BUF + 1]; int32_t pa[MAX_PAIRS]; int32_t pb[MAX_PAIRS]; };
+Plan g_plan_host;             /* what g_plan_dev holds */
+Plan* g_plan_dev = nullptr;
+bool g_plan_valid = false;
+const Plan* plan_on_device(const Plan& plan, hipStream_t st) {
+    if (!g_plan_dev && !ESHKOL_HIP_OK(hipMalloc((void**)&g_plan_dev, sizeof(Plan)))) { g_plan_dev = nullptr; return nullptr; }
+    if (g_plan_valid && memcmp(&g_plan_host, &plan, sizeof(Plan)) == 0) return g_plan_dev;
+    /* kernels of an earlier call may still read the old plan */
+    g_plan_valid = false;
+    if (!ESHKOL_HIP_OK(hipStreamSynchronize(st)) ||
+        !ESHKOL_HIP_OK(hipMemcpy(g_plan_dev, &plan, sizeof(Plan), hipMemcpyHostToDevice))) return nullptr;
+    g_plan_host = plan;
+    g_plan_valid = true;
+    return g_plan_dev;
+}
 
 }  // namespace
 
@@ -314,10 +324,9 @@ extern "C" int hip_matmul_ozaki_int8_f64_ex(const double* A, const double* B, do
     /* buffer plan, gpu_memory_cuda.cpp:367-389 */
     long long cap = (long long)(2147483647.0 / ((double)K * 16129.0));
     if (cap < 1) return -1;
-    struct Plan { double w[MAX_BUF]; int32_t first[MAX_BUF + 1]; int32_t pa[MAX_PAIRS]; int32_t pb[MAX_PAIRS]; };
-    Plan* plan = (Plan*)pinned(sizeof(Plan) + (M + N) * sizeof(double));
-    if (!plan) return -1;
-    double* h_max = (double*)(plan + 1);
+    Plan plan_host;
+    memset(&plan_host, 0, sizeof plan_host);
+    Plan* const plan = &plan_host;
     int nbuf = 0, npairs = 0;
     for (int d = 0; d <= T; d++) {
         int pp[16], pq[16], n = 0;
@@ -345,19 +354,20 @@ extern "C" int hip_matmul_ozaki_int8_f64_ex(const double* A, const double* B, do
     const bool a_kmajor = trans_a != 0, b_kmajor = trans_b == 0;
     double* rmax = (double*)eshkol_hip_workspace(WS_ROWSCALE, M * sizeof(double));
     double* cmax = (double*)eshkol_hip_workspace(WS_COLSCALE, N * sizeof(double));
-    Plan* dplan  = (Plan*)eshkol_hip_workspace(WS_MISC, sizeof(Plan));
+    const Plan* dplan = plan_on_device(plan_host, st);
     int8_t* As   = (int8_t*)eshkol_hip_workspace(WS_APLANES, (size_t)s * Mp * ldk);
     int8_t* Bs   = (int8_t*)eshkol_hip_workspace(WS_BPLANES, (size_t)s * Np * ldk);
     int32_t* G   = (int32_t*)eshkol_hip_workspace(WS_PRODUCTS, (size_t)nbuf * M * N * sizeof(int32_t));
     if (!rmax || !cmax || !dplan || !As || !Bs || !G) return -1;
 
-    if (!ESHKOL_HIP_OK(hipMemcpyAsync(dplan, plan, sizeof(Plan), hipMemcpyHostToDevice, st))) return -1;
     if ((a_kmajor ? hip_colabsmax_f64(A, K, M, 1.0, rmax, st) : hip_rowabsmax_f64(A, M, K, 1.0, rmax, st)) != 0) return -1;
     if ((b_kmajor ? hip_colabsmax_f64(B, K, N, 1.0, cmax, st) : hip_rowabsmax_f64(B, N, K, 1.0, cmax, st)) != 0) return -1;
     /* NaN/Inf input is unspecified in the reference; here it is detected through
-     * the maxima and reported as failure so the caller uses the native GEMM. */
-    if (!ESHKOL_HIP_OK(hipMemcpyAsync(h_max, rmax, M * sizeof(double), hipMemcpyDeviceToHost, st))) return -1;
-    if (!ESHKOL_HIP_OK(hipMemcpyAsync(h_max + M, cmax, N * sizeof(double), hipMemcpyDeviceToHost, st))) return -1;
+     * the maxima and reported as failure so the caller uses the native GEMM. The
+     * scan of the maxima runs beside the pipeline and writes its summary to host
+     * memory itself: no copy command, and the call returns with its work queued. */
+    const uint32_t ticket = eshkol_crt_scan_launch_aside(rmax, M, cmax, N, st, M * K + K * N);
+    if (!ticket) return -1;
     if (slice_any(A, M, K, rmax, s, As, Mp, ldk, a_kmajor, layout, st) != 0) return -1;
     if (slice_any(B, N, K, cmax, s, Bs, Np, ldk, b_kmajor, layout, st) != 0) return -1;
 
@@ -371,8 +381,9 @@ extern "C" int hip_matmul_ozaki_int8_f64_ex(const double* A, const double* B, do
     if (hip_igemm_i8(&ga, st) != 0) return -1;
     if (hip_ozaki_reconstruct_f64(C, G, dplan->w, nbuf, rmax, cmax, M, N, st) != 0) return -1;
 
-    if (!ESHKOL_HIP_OK(hipStreamSynchronize(st))) return -1;
-    for (uint64_t i = 0; i < M + N; i++) if (!std::isfinite(h_max[i])) return -1;
+    CrtMaxima mx[2];
+    if (eshkol_crt_scan_result(ticket, mx, st) != 0) return -1;
+    if (mx[0].nonfinite || mx[1].nonfinite) return -1;
 
     g_last.a_slices = As; g_last.b_slices = Bs; g_last.products = G;
     g_last.rmax = rmax; g_last.cmax = cmax;
