@@ -16,7 +16,8 @@ TOL = 1e-14
 
 SHAPES = [(1, 1, 1), (2, 2, 2), (1, 100, 1), (3, 5, 4), (5, 7, 3), (16, 16, 16), (64, 64, 64),
           (65, 67, 66), (37, 130, 9), (128, 128, 128), (129, 257, 131), (256, 256, 256),
-          (300, 17, 500), (512, 1000, 64), (1000, 33, 1000), (1024, 1024, 1024)]
+          (300, 17, 500), (512, 1000, 64), (1000, 33, 1000), (1024, 1024, 1024),
+          (1, 100003, 1), (70001, 3, 5), (5, 3, 70001), (2, 2, 65537), (65537, 2, 2), (9, 70000, 131)]
 
 
 @pytest.mark.parametrize("M,K,N", SHAPES)

@@ -44,7 +44,8 @@ def check_all_stages(A, B, n_mod=11, trans=None):
     return Cg, so
 
 
-SHAPES = [(1, 1, 1), (5, 3, 4), (64, 128, 64), (100, 200, 90), (257, 129, 255), (33, 2049, 65), (512, 640, 384)]
+SHAPES = [(1, 1, 1), (5, 3, 4), (64, 128, 64), (100, 200, 90), (257, 129, 255), (33, 2049, 65), (512, 640, 384),
+          (3, 131071, 2), (3001, 2, 2), (2, 2, 3001), (1, 1031, 513)]
 
 
 @pytest.mark.parametrize("M,K,N", SHAPES)

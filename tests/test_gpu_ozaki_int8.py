@@ -28,7 +28,8 @@ def check_all_stages(A, B, T):
 
 @pytest.mark.parametrize("M,K,N,T", [(1, 1, 1, 6), (5, 3, 4, 6), (64, 128, 64, 6), (100, 200, 90, 4),
                                      (257, 129, 255, 6), (300, 260, 280, 7), (512, 512, 512, 6),
-                                     (33, 2049, 65, 2), (640, 1024, 384, 8), (96, 96, 96, 1)])
+                                     (33, 2049, 65, 2), (640, 1024, 384, 8), (96, 96, 96, 1),
+                                     (3, 133000, 2, 6), (3001, 2, 2, 6), (2, 2, 3001, 4), (1, 1031, 513, 6)])
 def test_all_stages(gpu, M, K, N, T):
     print("int8", M, K, N, T, flush=True)
     A, B = synth.normal(500 + M, (M, K)), synth.normal(600 + N, (K, N))

@@ -17,7 +17,8 @@ TOL = 1e-2
 
 @pytest.mark.parametrize("dtype", [2, 3])
 @pytest.mark.parametrize("M,K,N", [(1, 1, 1), (5, 3, 4), (64, 128, 64), (100, 200, 90), (257, 129, 255),
-                                   (512, 512, 512), (33, 2049, 65), (1024, 768, 640)])
+                                   (512, 512, 512), (33, 2049, 65), (1024, 768, 640),
+                                   (1, 20001, 1), (9001, 3, 5), (5, 3, 9001), (2, 2, 65537)])
 def test_reduced_matches_reference_statement(gpu, M, K, N, dtype):
     print("reduced", M, K, N, dtype, flush=True)
     A = synth.normal(700 + M, (M, K), 1.0 / np.sqrt(K))      # configuration 4's input law
