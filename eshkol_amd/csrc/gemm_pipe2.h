@@ -241,12 +241,14 @@ __device__ __forceinline__ void run_tiles(int8_t* smem, const Source& cm, Next n
      * k-step (LDS stage nstage, k-step nks) is read into fb[W ^ 1]; after MFMA
      * 8 ... 15 comes mem(i - 8). The order is pinned: nothing crosses a
      * sched_barrier(0). */
-    auto kstep = [&](auto which, auto slot, auto kstep_c, int nstage, int nks, auto mem) {
+    auto kstep = [&](auto which, auto slot, auto kstep_c, int nstage, int nks, auto mem, auto fresh) {
         constexpr int W = decltype(which)::value, S = decltype(slot)::value, KS = decltype(kstep_c)::value;
+        constexpr bool FRESH = decltype(fresh)::value != 0;
         const int8_t* nb = smem + nstage * STAGE + nks * FRAG + lane * 16;
         static_for<TM * TN>([&](auto idx) {
             constexpr int I = decltype(idx)::value, T = I / TN, U = I % TN;
-            Op::mfma(fb[W][U], ra[S][T][KS], acc[T][U]);
+            if constexpr (FRESH) Op::mfma_first(fb[W][U], ra[S][T][KS], acc[T][U]);
+            else Op::mfma(fb[W][U], ra[S][T][KS], acc[T][U]);
             if constexpr (I < TN) fb[W ^ 1][I] = *(const v4i_t*)(nb + I * 4 * FRAG);
             else mem(IC<I - TN>{});
             __builtin_amdgcn_sched_barrier(0);
@@ -265,11 +267,43 @@ __device__ __forceinline__ void run_tiles(int8_t* smem, const Source& cm, Next n
     wait_loads<WAIT_START>(ra[0]);
     bool first_tile = true;
 
+    /* DEPTH k-blocks. In a tile's first group the sixteen sums start with their
+     * first product (the instruction adds it to the constant 0): no accumulator
+     * is cleared, which would be 256 instructions per tile with the matrix pipe idle. */
+    auto group = [&](auto first_of_tile) {
+        constexpr int FIRST = decltype(first_of_tile)::value;
+        static_for<DEPTH>([&](auto s) {
+            constexpr int S = decltype(s)::value;
+            constexpr int SP = (S + DEPTH - 1) % DEPTH, SN = (S + 1) % DEPTH;
+
+            kstep(I0{}, IC<S>{}, IC<0>{}, S, 1, [&](auto m) {
+                constexpr int Mi = decltype(m)::value;
+                if constexpr (Mi == 0) load_hidden<3 * FRAG>(ra[SP][0][3], rs_a, voff[0], c_soff);
+                if constexpr (Mi == 1) load_hidden<3 * FRAG>(ra[SP][1][3], rs_a, voff[1], c_soff);
+                if constexpr (Mi == 2) advance();
+            }, IC<(FIRST && S == 0) ? 1 : 0>{});
+            kstep(I1{}, IC<S>{}, IC<1>{}, S, 2, [&](auto m) {
+                constexpr int Mi = decltype(m)::value;
+                if constexpr (Mi == 0) load_hidden<0>(ra[S][0][0], rs_a, voff[0], c_soff);
+                if constexpr (Mi == 1) load_hidden<0>(ra[S][1][0], rs_a, voff[1], c_soff);
+            }, I0{});
+            kstep(I0{}, IC<S>{}, IC<2>{}, S, 3, [&](auto m) {
+                constexpr int Mi = decltype(m)::value;
+                if constexpr (Mi == 0) load_hidden<FRAG>(ra[S][0][1], rs_a, voff[0], c_soff);
+                if constexpr (Mi == 1) load_hidden<FRAG>(ra[S][1][1], rs_a, voff[1], c_soff);
+            }, I0{});
+            wait_loads<WAIT_STEADY>(ra[SN]);
+            pipe::lds_barrier();
+            kstep(I1{}, IC<S>{}, IC<3>{}, SN, 0, [&](auto m) {
+                constexpr int Mi = decltype(m)::value;
+                if constexpr (Mi == 0) load_hidden<2 * FRAG>(ra[S][0][2], rs_a, voff[0], c_soff);
+                if constexpr (Mi == 1) load_hidden<2 * FRAG>(ra[S][1][2], rs_a, voff[1], c_soff);
+                issue_b_one(IC<S>{}, m);
+            }, I0{});
+        });
+    };
+
     for (;;) {
-#pragma unroll
-        for (int t = 0; t < TM; t++)
-#pragma unroll
-            for (int u = 0; u < TN; u++) Op::zero(acc[t][u]);
         if (first_tile) {
             first_tile = false;
             pipe::lds_barrier();                   /* block 0 is in its stage, whichever wave requested it */
@@ -277,38 +311,9 @@ __device__ __forceinline__ void run_tiles(int8_t* smem, const Source& cm, Next n
             for (int u = 0; u < TN; u++) fb[0][u] = *(const v4i_t*)(smem + lane * 16 + u * 4 * FRAG);
         }
 
-        const int nkb = cur.npairs * nkb_per;      /* a multiple of DEPTH */
-        for (int g0 = 0; g0 < nkb; g0 += DEPTH) {
-            static_for<DEPTH>([&](auto s) {
-                constexpr int S = decltype(s)::value;
-                constexpr int SP = (S + DEPTH - 1) % DEPTH, SN = (S + 1) % DEPTH;
-
-                kstep(I0{}, IC<S>{}, IC<0>{}, S, 1, [&](auto m) {
-                    constexpr int Mi = decltype(m)::value;
-                    if constexpr (Mi == 0) load_hidden<3 * FRAG>(ra[SP][0][3], rs_a, voff[0], c_soff);
-                    if constexpr (Mi == 1) load_hidden<3 * FRAG>(ra[SP][1][3], rs_a, voff[1], c_soff);
-                    if constexpr (Mi == 2) advance();
-                });
-                kstep(I1{}, IC<S>{}, IC<1>{}, S, 2, [&](auto m) {
-                    constexpr int Mi = decltype(m)::value;
-                    if constexpr (Mi == 0) load_hidden<0>(ra[S][0][0], rs_a, voff[0], c_soff);
-                    if constexpr (Mi == 1) load_hidden<0>(ra[S][1][0], rs_a, voff[1], c_soff);
-                });
-                kstep(I0{}, IC<S>{}, IC<2>{}, S, 3, [&](auto m) {
-                    constexpr int Mi = decltype(m)::value;
-                    if constexpr (Mi == 0) load_hidden<FRAG>(ra[S][0][1], rs_a, voff[0], c_soff);
-                    if constexpr (Mi == 1) load_hidden<FRAG>(ra[S][1][1], rs_a, voff[1], c_soff);
-                });
-                wait_loads<WAIT_STEADY>(ra[SN]);
-                pipe::lds_barrier();
-                kstep(I1{}, IC<S>{}, IC<3>{}, SN, 0, [&](auto m) {
-                    constexpr int Mi = decltype(m)::value;
-                    if constexpr (Mi == 0) load_hidden<2 * FRAG>(ra[S][0][2], rs_a, voff[0], c_soff);
-                    if constexpr (Mi == 1) load_hidden<2 * FRAG>(ra[S][1][2], rs_a, voff[1], c_soff);
-                    issue_b_one(IC<S>{}, m);
-                });
-            });
-        }
+        const int nkb = cur.npairs * nkb_per;      /* a multiple of DEPTH, at least DEPTH */
+        group(I1{});
+        for (int g0 = DEPTH; g0 < nkb; g0 += DEPTH) group(I0{});
         epilogue(acc, cur, epi_stage);
         if (!nx_has) break;
         cur = nxt;

@@ -353,6 +353,16 @@ template <bool BF16> struct H16Op {
             acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h_t, first),
                                                          __builtin_bit_cast(v8h_t, second), acc, 0, 0, 0);
     }
+    /* the first product of a sum: the instruction takes the constant 0 as its addend */
+    static __device__ __forceinline__ void mfma_first(const v4i_t& first, const v4i_t& second, v16f_t& acc) {
+        const v16f_t none = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        if (BF16)
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8b_t, first),
+                                                          __builtin_bit_cast(v8b_t, second), none, 0, 0, 0);
+        else
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h_t, first),
+                                                         __builtin_bit_cast(v8h_t, second), none, 0, 0, 0);
+    }
     static __device__ __forceinline__ void zero(v16f_t& acc) {
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[r] = 0.0f;

@@ -44,6 +44,11 @@ struct I8Op {
     static __device__ __forceinline__ void mfma(const v4i_t& first, const v4i_t& second, v16i_t& acc) {
         acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(first, second, acc, 0, 0, 0);
     }
+    /* the first product of a sum: the instruction takes the constant 0 as its addend */
+    static __device__ __forceinline__ void mfma_first(const v4i_t& first, const v4i_t& second, v16i_t& acc) {
+        const v16i_t none = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(first, second, none, 0, 0, 0);
+    }
     static __device__ __forceinline__ void zero(v16i_t& acc) {
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[r] = 0;
