@@ -59,9 +59,12 @@ constexpr ByteWeights byte_weights(int modulus) {
  * shift[i] = E - floor(log2 max_i) (0 for a maximum of zero): what the split of a
  * CRT tier needs when its exponent E is known before the operands are looked at. */
 int eshkol_rowabsmax_shift_f64(const double* A, uint64_t M, uint64_t K, double zero_value,
-                               double* rmax, int32_t* shift, int E, hipStream_t stream);
+                               double* rmax, int32_t* shift, int E, hipStream_t stream, hipEvent_t done = nullptr);
 int eshkol_colabsmax_shift_f64(const double* X, uint64_t K, uint64_t R, double zero_value,
-                               double* cmax, int32_t* shift, int E, hipStream_t stream);
+                               double* cmax, int32_t* shift, int E, hipStream_t stream, hipEvent_t done = nullptr);
+/* done, when given, becomes the completion event of the launch's last kernel
+ * (the kernel's own completion signal: no marker is queued behind it, which
+ * would hold the next kernel of the stream back by 6-7 us). */
 
 /* ---- exponents of the maxima (implemented in ozaki_crt.hip) ---------------------- */
 
@@ -82,7 +85,12 @@ constexpr int32_t CRT_FL_ZERO = INT32_MIN;      /* exponent entry of a maximum o
  * product (operand_elems = M K + K N) the scan is queued on st itself: there the
  * device waits for the host, and three calls cost more than ten microseconds in line. */
 uint32_t eshkol_crt_scan_launch_aside(const double* amax, uint64_t M, const double* bmax, uint64_t N, hipStream_t st,
-                                      uint64_t operand_elems);
+                                      uint64_t operand_elems, bool event_attached = false);
+/* The event the side stream waits for before that scan, or null when a product of
+ * this size has its scan queued in line. A caller that hands it to the launcher
+ * of the last maxima kernel (`done` above) passes event_attached = true and
+ * spares the stream a marker; otherwise the event is recorded behind st. */
+hipEvent_t eshkol_crt_scan_event(uint64_t operand_elems);
 /* The two CRT tiers print one marker line per call, as the reference does per
  * dispatch (gpu_memory.mm:2503; its gates count those lines). A dispatcher that
  * runs one product as several calls (row panels) lets the first call print and

@@ -4,6 +4,7 @@
  * single-precision GEMM of eshkol_gpu_matmul_f32.
  */
 #include "hip_common.h"
+#include <hip/hip_ext.h>
 #include "kernels.h"
 #include "crt_shared.h"
 #include "tanh_f64.h"
@@ -236,12 +237,12 @@ extern "C" int hip_transpose_f64(const double* in, double* out, uint64_t rows, u
 }
 
 int eshkol_rowabsmax_shift_f64(const double* A, uint64_t M, uint64_t K, double zero_value,
-                               double* rmax, int32_t* shift, int E, hipStream_t stream) {
+                               double* rmax, int32_t* shift, int E, hipStream_t stream, hipEvent_t done) {
     if (!A || !rmax || M == 0 || K == 0) return -1;
     const uint64_t g = (M + 3) / 4;
     if (g > 0x7fffffffULL) return -1;
-    hipLaunchKernelGGL(rowabsmax_f64_kernel, dim3((unsigned)g), dim3(256), 0, stream,
-                       A, M, K, zero_value, rmax, shift, E);
+    hipExtLaunchKernelGGL(rowabsmax_f64_kernel, dim3((unsigned)g), dim3(256), 0, stream, nullptr, done, 0,
+                          A, M, K, zero_value, rmax, shift, E);
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 
@@ -256,7 +257,7 @@ extern "C" int hip_colabsmax_f64(const double* X, uint64_t K, uint64_t R, double
 }
 
 int eshkol_colabsmax_shift_f64(const double* X, uint64_t K, uint64_t R, double zero_value,
-                               double* cmax, int32_t* shift, int E, hipStream_t stream) {
+                               double* cmax, int32_t* shift, int E, hipStream_t stream, hipEvent_t done) {
     EshkolHipCall bracket(stream);
     if (!X || !cmax || K == 0 || R == 0) return -1;
     const uint64_t gx = (R + 63) / 64;
@@ -269,8 +270,8 @@ int eshkol_colabsmax_shift_f64(const double* X, uint64_t K, uint64_t R, double z
     if (!partial) return -1;
     hipLaunchKernelGGL(colabsmax_partial_kernel, dim3((unsigned)gx, (unsigned)slices), dim3(256), 0,
                        (hipStream_t)stream, X, K, R, rows_per_slice, partial);
-    hipLaunchKernelGGL(colabsmax_fold_kernel, dim3((unsigned)((R + 255) / 256)), dim3(256), 0,
-                       (hipStream_t)stream, partial, R, slices, zero_value, cmax, shift, E);
+    hipExtLaunchKernelGGL(colabsmax_fold_kernel, dim3((unsigned)((R + 255) / 256)), dim3(256), 0,
+                          (hipStream_t)stream, nullptr, done, 0, partial, R, slices, zero_value, cmax, shift, E);
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 

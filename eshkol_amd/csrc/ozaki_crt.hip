@@ -673,11 +673,16 @@ uint32_t scan_launch(const double* amax, uint64_t M, const double* bmax, uint64_
  * host to queue them, so the event, the wait and the launch on a second stream
  * cost more (three calls) than the scan's ten microseconds in line do. */
 constexpr uint64_t ASIDE_FROM = 6u << 20;
+hipEvent_t scan_event(uint64_t operand_elems) {
+    return (operand_elems >= ASIDE_FROM && ensure_mailbox()) ? g_scan_event : nullptr;
+}
+/* event_attached: the caller made scan_event() the completion event of the last
+ * kernel the scan depends on, so no marker needs to be queued behind st. */
 uint32_t scan_launch_aside(const double* amax, uint64_t M, const double* bmax, uint64_t N, hipStream_t st,
-                           uint64_t operand_elems) {
+                           uint64_t operand_elems, bool event_attached) {
     if (!ensure_mailbox()) return 0;
     if (operand_elems < ASIDE_FROM) return scan_launch(amax, M, bmax, N, nullptr, nullptr, st);
-    if (!ESHKOL_HIP_OK(hipEventRecord(g_scan_event, st)) ||
+    if ((!event_attached && !ESHKOL_HIP_OK(hipEventRecord(g_scan_event, st))) ||
         !ESHKOL_HIP_OK(hipStreamWaitEvent(g_scan_stream, g_scan_event, 0))) return 0;
     return scan_launch(amax, M, bmax, N, nullptr, nullptr, g_scan_stream);
 }
@@ -761,9 +766,10 @@ void eshkol_crt_set_quiet(int quiet) { g_crt_quiet = quiet; }
 int eshkol_crt_quiet(void) { return g_crt_quiet; }
 
 uint32_t eshkol_crt_scan_launch_aside(const double* amax, uint64_t M, const double* bmax, uint64_t N, hipStream_t st,
-                                      uint64_t operand_elems) {
-    return scan_launch_aside(amax, M, bmax, N, st, operand_elems);
+                                      uint64_t operand_elems, bool event_attached) {
+    return scan_launch_aside(amax, M, bmax, N, st, operand_elems, event_attached);
 }
+hipEvent_t eshkol_crt_scan_event(uint64_t operand_elems) { return scan_event(operand_elems); }
 
 int eshkol_crt_scan_result(uint32_t ticket, CrtMaxima out[2], hipStream_t st) {
     (void)st;
@@ -926,12 +932,15 @@ static int crt_matmul_impl(const double* A, const double* B, double* C,
                          floor((crt_constants(num_moduli).log2P - 3.0 - log2K) / 2.0) >= 52.0;
     int32_t* const mu_out = fixed_E ? dmu : nullptr;
     int32_t* const nu_out = fixed_E ? dnu : nullptr;
-    if ((a_kmajor ? eshkol_colabsmax_shift_f64(A, K, M, 0.0, amax, mu_out, 52, st)
-                  : eshkol_rowabsmax_shift_f64(A, M, K, 0.0, amax, mu_out, 52, st)) != 0) return -1;
+    /* the last kernel that writes maxima carries the event the scan's stream waits for */
+    const hipEvent_t fork = fixed_E ? scan_event(M * K + K * N) : nullptr;
+    const hipEvent_t fork_a = use_prepared ? fork : nullptr, fork_b = use_prepared ? nullptr : fork;
+    if ((a_kmajor ? eshkol_colabsmax_shift_f64(A, K, M, 0.0, amax, mu_out, 52, st, fork_a)
+                  : eshkol_rowabsmax_shift_f64(A, M, K, 0.0, amax, mu_out, 52, st, fork_a)) != 0) return -1;
     if (!use_prepared &&
-        (b_kmajor ? eshkol_colabsmax_shift_f64(B, K, N, 0.0, bmax, nu_out, 52, st)
-                  : eshkol_rowabsmax_shift_f64(B, N, K, 0.0, bmax, nu_out, 52, st)) != 0) return -1;
-    const uint32_t ticket = fixed_E ? scan_launch_aside(amax, M, bmax, N, st, M * K + K * N)
+        (b_kmajor ? eshkol_colabsmax_shift_f64(B, K, N, 0.0, bmax, nu_out, 52, st, fork_b)
+                  : eshkol_rowabsmax_shift_f64(B, N, K, 0.0, bmax, nu_out, 52, st, fork_b)) != 0) return -1;
+    const uint32_t ticket = fixed_E ? scan_launch_aside(amax, M, bmax, N, st, M * K + K * N, fork != nullptr)
                                     : scan_launch(amax, M, bmax, N, dmu, dnu, st);
     if (!ticket) return -1;
 

@@ -508,9 +508,11 @@ extern "C" int hip_matmul_ozaki_fast_f64_ex(const double* A, const double* B, do
      * the maxima (non-finite input?) runs beside it and is read at the end. */
     if ((a_kmajor ? eshkol_colabsmax_shift_f64(A, K, M, 0.0, amax, sha, f.E - 1, st)
                   : eshkol_rowabsmax_shift_f64(A, M, K, 0.0, amax, sha, f.E - 1, st)) != 0) return -1;
-    if ((b_kmajor ? eshkol_colabsmax_shift_f64(B, K, N, 0.0, bmax, shb, f.E - 1, st)
-                  : eshkol_rowabsmax_shift_f64(B, N, K, 0.0, bmax, shb, f.E - 1, st)) != 0) return -1;
-    const uint32_t ticket = eshkol_crt_scan_launch_aside(amax, M, bmax, N, st, M * K + K * N);
+    /* the last kernel that writes maxima carries the event the scan's stream waits for */
+    const hipEvent_t fork = eshkol_crt_scan_event(M * K + K * N);
+    if ((b_kmajor ? eshkol_colabsmax_shift_f64(B, K, N, 0.0, bmax, shb, f.E - 1, st, fork)
+                  : eshkol_rowabsmax_shift_f64(B, N, K, 0.0, bmax, shb, f.E - 1, st, fork)) != 0) return -1;
+    const uint32_t ticket = eshkol_crt_scan_launch_aside(amax, M, bmax, N, st, M * K + K * N, fork != nullptr);
     if (!ticket) return -1;
 
     if (split_any(A, M, K, sha, f.table, Ap, Mp, ldk, a_kmajor, layout, st) != 0) return -1;

@@ -361,12 +361,14 @@ extern "C" int hip_matmul_ozaki_int8_f64_ex(const double* A, const double* B, do
     if (!rmax || !cmax || !dplan || !As || !Bs || !G) return -1;
 
     if ((a_kmajor ? hip_colabsmax_f64(A, K, M, 1.0, rmax, st) : hip_rowabsmax_f64(A, M, K, 1.0, rmax, st)) != 0) return -1;
-    if ((b_kmajor ? hip_colabsmax_f64(B, K, N, 1.0, cmax, st) : hip_rowabsmax_f64(B, N, K, 1.0, cmax, st)) != 0) return -1;
+    const hipEvent_t fork = eshkol_crt_scan_event(M * K + K * N);     /* carried by the last maxima kernel */
+    if ((b_kmajor ? eshkol_colabsmax_shift_f64(B, K, N, 1.0, cmax, nullptr, 0, st, fork)
+                  : eshkol_rowabsmax_shift_f64(B, N, K, 1.0, cmax, nullptr, 0, st, fork)) != 0) return -1;
     /* NaN/Inf input is unspecified in the reference; here it is detected through
      * the maxima and reported as failure so the caller uses the native GEMM. The
      * scan of the maxima runs beside the pipeline and writes its summary to host
      * memory itself: no copy command, and the call returns with its work queued. */
-    const uint32_t ticket = eshkol_crt_scan_launch_aside(rmax, M, cmax, N, st, M * K + K * N);
+    const uint32_t ticket = eshkol_crt_scan_launch_aside(rmax, M, cmax, N, st, M * K + K * N, fork != nullptr);
     if (!ticket) return -1;
     if (slice_any(A, M, K, rmax, s, As, Mp, ldk, a_kmajor, layout, st) != 0) return -1;
     if (slice_any(B, N, K, cmax, s, Bs, Np, ldk, b_kmajor, layout, st) != 0) return -1;
