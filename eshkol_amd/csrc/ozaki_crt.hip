@@ -610,7 +610,7 @@ void* g_pinned = nullptr;
 size_t g_pinned_bytes = 0;
 void* pinned(size_t bytes) {
     if (g_pinned_bytes >= bytes) return g_pinned;
-    if (g_pinned) hipHostFree(g_pinned);
+    if (g_pinned) (void)hipHostFree(g_pinned);
     g_pinned = nullptr; g_pinned_bytes = 0;
     if (!ESHKOL_HIP_OK(hipHostMalloc(&g_pinned, bytes, hipHostMallocDefault))) return nullptr;
     g_pinned_bytes = bytes;
@@ -699,7 +699,7 @@ int ensure_tables(hipStream_t st) {
     for (int i = 0; i < 16; i++) { h[17 + i] = i; h[33 + i] = H_MODULI[i]; }
     if (!ESHKOL_HIP_OK(hipMalloc((void**)&g_tables, sizeof h))) { g_tables = nullptr; return -1; }
     if (!ESHKOL_HIP_OK(hipMemcpyAsync(g_tables, h, sizeof h, hipMemcpyHostToDevice, st)) ||
-        !ESHKOL_HIP_OK(hipStreamSynchronize(st))) { hipFree(g_tables); g_tables = nullptr; return -1; }
+        !ESHKOL_HIP_OK(hipStreamSynchronize(st))) { (void)hipFree(g_tables); g_tables = nullptr; return -1; }
     return 0;
 }
 
@@ -1098,9 +1098,9 @@ extern "C" int hip_ozaki_crt_prepare_operand_b(const double* B, uint64_t K, uint
     pb->trans_b = trans_b; pb->n_mod = num_moduli; pb->layout = layout;
     pb->bmax = nullptr; pb->nu = nullptr; pb->planes = nullptr;
     auto fail = [&]() {
-        if (pb->bmax) hipFree(pb->bmax);
-        if (pb->nu) hipFree(pb->nu);
-        if (pb->planes) hipFree(pb->planes);
+        if (pb->bmax) (void)hipFree(pb->bmax);
+        if (pb->nu) (void)hipFree(pb->nu);
+        if (pb->planes) (void)hipFree(pb->planes);
         delete pb;
         return -1;
     };
@@ -1125,9 +1125,9 @@ extern "C" void hip_ozaki_crt_release_prepared(void* handle) {
     if (!pb || pb->magic != PREPARED_MAGIC) return;
     EshkolHipCall bracket(nullptr);
     (void)hipDeviceSynchronize();
-    hipFree(pb->bmax);
-    hipFree(pb->nu);
-    hipFree(pb->planes);
+    (void)hipFree(pb->bmax);
+    (void)hipFree(pb->nu);
+    (void)hipFree(pb->planes);
     pb->magic = 0;
     delete pb;
 }
