@@ -1123,7 +1123,7 @@ extern "C" int hip_ozaki_crt_prepare_operand_b(const double* B, uint64_t K, uint
 extern "C" void hip_ozaki_crt_release_prepared(void* handle) {
     CrtPreparedB* pb = (CrtPreparedB*)handle;
     if (!pb || pb->magic != PREPARED_MAGIC) return;
-    EshkolHipCall bracket(nullptr);
+    EshkolHipCall bracket(eshkol_hip_stream());     /* queues nothing: no caller's stream to order against */
     (void)hipDeviceSynchronize();
     (void)hipFree(pb->bmax);
     (void)hipFree(pb->nu);
