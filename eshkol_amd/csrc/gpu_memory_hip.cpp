@@ -176,27 +176,30 @@ const TierEnv& tier_env(void) { std::call_once(g_env_once, parse_env); return g_
  * Same shape as the reference's (gpu_memory_cuda.cpp:485-566): per kernel
  * t_ns = overhead + work/peak, peak self-calibrates upward from measured calls.
  * Seeds are MI355X measurements of this library: the line through the times
- * at 4096^3 and 8192^3 for the slice tiers (T1 0.43 and 2.08 ms ... T8 2.73
- * and 20.3 ms, rates taken 5 % low: devices differ by that much), 1024^3 and
- * 8192^3 for the native kernel (0.041 ms, 14.6 ms). */
+ * at 4096^3 and 8192^3 for the slice tiers (T1 0.36 and 1.89 ms ... T8 2.63
+ * and 21.1 ms) and the exact tier (1.17 and 7.73 ms), rates taken 5 % low
+ * (devices differ by that much); 1024^3 and 8192^3 for the native kernel
+ * (0.041 ms, 14.5 ms). Such a line overstates the tiers below 4096^3 (the exact
+ * tier at 2048^3: 0.35 ms predicted, 0.22 measured, level with native), which
+ * errs towards native fp64 where the two are close. */
 const double OZAKI_TOL[9] = { 1.0, 1e-3, 1e-5, 1e-7, 1e-9, 1e-11, 1e-13, 1e-14, 1e-14 };
 struct GemmModel { double overhead_ns; double peak_gflops; };
 constexpr int MODEL_CRT = 9;
 GemmModel g_model[10] = {
     /* native */ {  13000.0,  75000.0 },
-    /* T1 */ { 195000.0, 554000.0 }, /* T2 */ { 220000.0, 332000.0 },
-    /* T3 */ { 245000.0, 215000.0 }, /* T4 */ { 375000.0, 152000.0 },
-    /* T5 */ { 290000.0, 110500.0 }, /* T6 */ { 375000.0,  83500.0 },
-    /* T7 */ { 235000.0,  64300.0 }, /* T8 */ { 220000.0,  52000.0 },
-    /* Ozaki-II CRT exact, 16 moduli: 1.36 and 7.90 ms */ { 425000.0, 140000.0 } };
+    /* T1 */ { 145000.0, 602000.0 }, /* T2 */ { 153000.0, 346000.0 },
+    /* T3 */ { 162000.0, 222000.0 }, /* T4 */ { 188000.0, 155000.0 },
+    /* T5 */ { 188000.0, 111800.0 }, /* T6 */ { 151000.0,  82000.0 },
+    /* T7 */ {  65000.0,  62200.0 }, /* T8 */ {  60000.0,  49500.0 },
+    /* Ozaki-II CRT exact, 16 moduli */ { 233000.0, 139000.0 } };
 const double OZAKI_SAFETY = 1.15;
 std::mutex g_model_mutex;
 
 double predict_ns(int idx, double work) { return g_model[idx].overhead_ns + work / g_model[idx].peak_gflops; }
 /* Reduced-precision CRT tier with n moduli: its times at 4096^3 and 8192^3 for
- * n = 4 ... 16 (0.46 and 2.35 ms ... 1.27 and 7.91 ms) are linear in n on both
+ * n = 4 ... 16 (0.41 and 2.28 ms ... 1.16 and 7.63 ms) are linear in n on both
  * coefficients; rate taken 5 % low like the others. */
-double predict_fast_ns(int n, double work) { return 140000.0 + 11200.0 * n + work * (0.342e-6 + 0.433e-6 * n); }
+double predict_fast_ns(int n, double work) { return 125000.0 + 7000.0 * n + work * (0.360e-6 + 0.4195e-6 * n); }
 /* Its guaranteed relative error with E bits kept per operand: measured normwise
  * errors on well-conditioned operands are about 2^-E (1e-8 at E = 26); the
  * guarantee is 32 times that, the margin the reference gives its slice tiers
@@ -254,10 +257,11 @@ Selection select_tier(uint64_t M, uint64_t K, uint64_t N, double budget) {
                 break;
             }
         }
-        /* the exact tier's guarantee and its cost model are those of sixteen moduli */
+        /* the exact tier's guarantee and its cost model are those of sixteen moduli;
+         * within 5 % of a cheaper kernel it is preferred: it gives more for the same */
         const TierEnv& env = tier_env();
         const double t = predict_ns(MODEL_CRT, work);
-        if (env.num_moduli == 16 && !env.adaptive && budget >= CRT_EXACT_TOL && t < t_best) {
+        if (env.num_moduli == 16 && !env.adaptive && budget >= CRT_EXACT_TOL && 0.95 * t < t_best) {
             t_best = t; best = Selection(); best.tier = 2;
         }
     }

@@ -330,7 +330,9 @@ lib.eshkol_gpu_resident_unpin(B.ctypes.data)
     ({"ESHKOL_HIP_F64_KERNEL": "ozaki-int8"}, 0, "INT8-Ozaki T=6"),
     ({}, 3, "row panels"),
     ({}, 2, "row panels"),
-    ({"ESHKOL_MATMUL_ACCURACY": "1e-6"}, 0, "Ozaki-II FAST (9 moduli; accuracy-budget selector)"),
+    # two kernels meet this budget at nearly the same predicted cost: either is a right answer
+    ({"ESHKOL_MATMUL_ACCURACY": "1e-6"}, 0, ("Ozaki-II FAST (9 moduli; accuracy-budget selector)",
+                                             "INT8-Ozaki T=3 (accuracy-budget selector")),
 ], ids=["native", "crt", "crt-fast", "int8-slices", "bf16", "f16", "budget-1e-6"])
 def test_host_memory_dispatch_in_row_panels(gpu, env, dtype, tier_line):
     """Large products on host memory go through the device in row panels of A
@@ -338,10 +340,11 @@ def test_host_memory_dispatch_in_row_panels(gpu, env, dtype, tier_line):
     body = PANELLED.replace("DTYPE", str(dtype))
     e = dict(env); e["ESHKOL_GPU_VERBOSE"] = "1"
     r = run_child(body, e)
-    assert "in 7 row panels of 640" in r.stderr and tier_line in r.stderr
+    lines = tier_line if isinstance(tier_line, tuple) else (tier_line,)
+    assert "in 7 row panels of 640" in r.stderr and any(l in r.stderr for l in lines)
     e["ESHKOL_GPU_OVERLAP"] = "0"
     r = run_child(body, e)
-    assert "row panels" not in r.stderr and (dtype or tier_line in r.stderr)
+    assert "row panels" not in r.stderr and (dtype or any(l in r.stderr for l in lines))
 
 
 def test_concurrent_callers_serialise_on_the_library(gpu):
