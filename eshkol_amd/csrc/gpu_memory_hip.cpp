@@ -11,8 +11,10 @@
  *         -> INT8 slice tier with T = ESHKOL_OZAKI_CUDA_T, if M,N,K >= 1024
  *      ESHKOL_HIP_F64_KERNEL = ozaki-crt, or ESHKOL_SF64_KERNEL = ozaki
  *         -> Ozaki-II CRT exact tier, if M,K,N >= 512
- *   2. ESHKOL_MATMUL_ACCURACY set -> cheapest of {native, INT8 slices at the
- *      smallest T whose guaranteed error meets the budget} by the cost model
+ *   2. ESHKOL_MATMUL_ACCURACY set -> cheapest, by the cost model, of {native,
+ *      INT8 slices at the smallest T whose guaranteed error meets the budget,
+ *      the reduced-precision CRT tier at the smallest moduli count that does,
+ *      the CRT exact tier where its normwise bound does}
  *   3. native fp64 MFMA GEMM
  * A tier that returns nonzero falls through to the native GEMM.
  */
@@ -220,19 +222,22 @@ void calibrate(int idx, double work, double measured_ns) {
  * only alternative; here the two Ozaki-II tiers are candidates as well:
  *   slices      smallest T with OZAKI_TOL[T] <= budget (none below 1e-14)
  *   CRT fast    smallest moduli count whose E gives fast_tolerance(E) <= budget
- *   CRT exact   budgets >= CRT_EXACT_TOL (1e-15, normwise): every element of A
- *               is truncated at 2^-52 of its row's largest magnitude and every
- *               element of B at 2^-52 of its column's, the rest is exact, so
- *               |C - AB|_ij <= K 2^-51 rmax_i cmax_j, hence at most K 2^-51 in
- *               the norm the budget is stated in (||C - AB||_F / (||A||_F ||B||_F))
- *               and about 1e-17 measured on random operands. It is a normwise
- *               guarantee relative to the row and column maxima, not a
+ *   CRT exact   budgets >= crt_exact_tolerance(K) = sqrt(K) 2^-51 + 2^-53, which is a
+ *               bound, not a measurement: the tier multiplies A' = trunc(A 2^mu) 2^-mu
+ *               and B' likewise without further error (aligned weights) and rounds
+ *               once. |A - A'|_ik < 2^-52 rmax_i and rmax_i <= ||A_i||_2, so
+ *               ||A - A'||_F <= sqrt(K) 2^-52 ||A||_F, the same for B, ||A'||_F <=
+ *               ||A||_F, hence ||C - AB||_F <= (2 sqrt(K) 2^-52 + 2^-53) ||A||_F ||B||_F
+ *               in the norm the budget is stated in: 4.0e-14 at K = 8192, 1.0e-14
+ *               at K = 512 (about 1e-17 measured on random operands). It is a
+ *               normwise guarantee relative to the row and column maxima, not a
  *               componentwise one: an entry far below its row's maximum loses
- *               its low bits, where native fp64 would keep them. Budgets below
- *               1e-15, and the names exact / full, therefore stay on native
- *               fp64, as in the reference.
+ *               its low bits, where native fp64 would keep them. Tighter budgets,
+ *               and the names exact / full, therefore stay on native fp64 (or
+ *               the slice tier's T = 7 where that is cheaper), as the reference
+ *               answers them with DGEMM (gpu_memory_cuda.cpp:536-538, 554-556).
  * Both CRT tiers need M, K, N >= 512 and K <= 131071, as their dispatch does. */
-constexpr double CRT_EXACT_TOL = 1e-15;
+double crt_exact_tolerance(uint64_t K) { return sqrt((double)K) * ldexp(1.0, -51) + ldexp(1.0, -53); }
 struct Selection { int tier = 0; int T = 0; int fast_moduli = 0; double speedup = 1.0; };
 Selection select_tier(uint64_t M, uint64_t K, uint64_t N, double budget) {
     const double work = 2.0 * (double)M * (double)K * (double)N;
@@ -261,7 +266,7 @@ Selection select_tier(uint64_t M, uint64_t K, uint64_t N, double budget) {
          * within 5 % of a cheaper kernel it is preferred: it gives more for the same */
         const TierEnv& env = tier_env();
         const double t = predict_ns(MODEL_CRT, work);
-        if (env.num_moduli == 16 && !env.adaptive && budget >= CRT_EXACT_TOL && 0.95 * t < t_best) {
+        if (env.num_moduli == 16 && !env.adaptive && budget >= crt_exact_tolerance(K) && 0.95 * t < t_best) {
             t_best = t; best = Selection(); best.tier = 2;
         }
     }

@@ -250,22 +250,27 @@ def test_accuracy_budget_selector_decisions():
     n = 8192
     assert pick(n, n, n, 1e-2)[:2] == (1, 1) and pick(n, n, n, 1e-5)[:2] == (1, 2) and pick(n, n, n, 1e-7)[:2] == (1, 3)
     assert pick(n, n, n, 1e-9)[:2] == (1, 4)
-    for budget in (1e-10, 1e-11, 1e-13, 1e-14, 1e-15):
+    for budget in (1e-10, 1e-11, 1e-13, 4.1e-14):
         tier, _, _, sp = pick(n, n, n, budget)
-        assert tier == 2 and 1.5 < sp < 2.5, budget                # the exact tier, where the reference has DGEMM only
-    # below the exact tier's stated normwise tolerance, and for the names exact / full (budget 0),
-    # native fp64 only: the reference never degrades its strictest request (gpu_memory_cuda.cpp:546-566)
-    for budget in (9e-16, 1e-16, 0.0, -1.0):
+        assert tier == 2 and 1.5 < sp < 2.5, budget                # the exact tier, where the reference has T = 5 ... 7
+    # The exact tier is a candidate only where its normwise BOUND sqrt(K) 2^-51 + 2^-53 meets the
+    # budget (4.03e-14 at K = 8192, 2.85e-14 at K = 4096), not where its measured 1e-17 would.
+    # Tighter budgets, and the names exact / full (budget 0), get native fp64: the reference never
+    # degrades its strictest requests (gpu_memory_cuda.cpp:536-538, 546-566)
+    for budget in (4.0e-14, 1e-14, 1e-15, 9e-16, 1e-16, 0.0, -1.0):
         assert pick(n, n, n, budget)[0] == 0, budget
+    for budget in (2.8e-14, 1e-14, 1e-15, 1e-16, 0.0, -1.0):
         assert pick(4096, 4096, 4096, budget)[0] == 0, budget
+    assert pick(4096, 4096, 4096, 2.9e-14)[0] == 2
+    assert pick(4096, 512, 4096, 1.1e-14)[0] in (0, 2) and pick(4096, 512, 4096, 1.0e-14)[0] == 0
     last = 1e9
-    for budget in (1e-2, 1e-3, 1e-5, 1e-7, 1e-9, 1e-11, 1e-13, 1e-15):
+    for budget in (1e-2, 1e-3, 1e-5, 1e-7, 1e-9, 1e-11, 1e-13, 1e-14, 1e-15):
         sp = pick(n, n, n, budget)[3]
         assert sp <= last * 1.0001, budget                          # tighter budgets are never predicted cheaper
         last = sp
     for budget in (1e-2, 1e-9, 1e-15):
         assert pick(256, 256, 256, budget)[0] == 0 and pick(1024, 1024, 1024, budget)[0] == 0
-    assert pick(4096, 4096, 4096, 1e-15)[0] == 2 and pick(4096, 4096, 4096, 1e-2)[:2] == (1, 1)
+    assert pick(4096, 4096, 4096, 1e-13)[0] == 2 and pick(4096, 4096, 4096, 1e-2)[:2] == (1, 1)
     # the exact tier pays from about 3072^3 on (measured 0.56 ms against 0.81 native); at 2048^3 the two are level
     assert pick(3072, 3072, 3072, 1e-13)[0] == 2 and pick(2048, 2048, 2048, 1e-13)[0] == 0
     for budget, lo, hi in ((1e-8, 11, 13), (1e-9, 12, 14), (1e-11, 14, 16)):

@@ -723,13 +723,28 @@ assert err <= float(os.environ["EXPECT_ERR"]), err
         r = run_child(body2, {"ESHKOL_MATMUL_ACCURACY": name, "EXPECT_ERR": "1e-15", "ESHKOL_GPU_THRESHOLD": "1",
                               "ESHKOL_GPU_VERBOSE": "1"})
         assert "native fp64 MFMA (budget met cheapest by native fp64)" in r.stderr and "Ozaki" not in r.stderr
-    # ... a numeric budget down to 1e-15 (normwise) at this size is met cheapest by the Ozaki-II exact tier ...
-    r = run_child(body2, {"ESHKOL_MATMUL_ACCURACY": "1e-15", "EXPECT_ERR": "1e-15", "ESHKOL_GPU_THRESHOLD": "1",
-                          "ESHKOL_GPU_VERBOSE": "1"})
-    assert "Ozaki-II CRT exact (accuracy-budget selector), aligned weights" in r.stderr
-    r = run_child(body2, {"ESHKOL_MATMUL_ACCURACY": "1e-13", "EXPECT_ERR": "1e-13", "ESHKOL_GPU_THRESHOLD": "1",
-                          "ESHKOL_GPU_VERBOSE": "1"})
-    assert "Ozaki-II CRT exact (accuracy-budget selector), aligned weights" in r.stderr
+    # ... a numeric budget the exact tier's normwise bound meets (sqrt(K) 2^-51 = 2.85e-14 at K = 4096) is met
+    # cheapest by that tier ...
+    for budget in ("1e-13", "3e-14"):
+        r = run_child(body2, {"ESHKOL_MATMUL_ACCURACY": budget, "EXPECT_ERR": budget, "ESHKOL_GPU_THRESHOLD": "1",
+                              "ESHKOL_GPU_VERBOSE": "1"})
+        assert "Ozaki-II CRT exact (accuracy-budget selector), aligned weights" in r.stderr
+    # ... and a tighter one stays native like the names do, although the tier measures 1e-17 on such operands:
+    # an entry far below its row's largest keeps its low bits there. Row 0 of A carries one entry of 2^60
+    # that meets a zero row of B, so the row's result is made of the small entries alone; the exact tier
+    # would cut them at 2^8.
+    wide = r"""
+n = 4096
+A = synth.normal(1, (n, n)); B = synth.normal(2, (n, n))
+A[0, 0] = 2.0 ** 60; B[0, :] = 0.0
+got = ea.matmul_dispatch(A, B)
+ref = A[:1].astype(np.longdouble) @ B.astype(np.longdouble)
+rel = float(np.max(np.abs(got[0] - ref[0]) / (np.abs(A[0, 1:]) @ np.abs(B[1:]))))
+print("ROW0 %.3e" % rel)
+assert rel <= 1e-14, rel
+"""
+    r = run_child(wide, {"ESHKOL_MATMUL_ACCURACY": "1e-15", "ESHKOL_GPU_THRESHOLD": "1", "ESHKOL_GPU_VERBOSE": "1"})
+    assert "native fp64 MFMA (budget met cheapest by native fp64)" in r.stderr and "Ozaki" not in r.stderr
     # the override by name keeps the reference's weights (and its error on such operands) unless told otherwise
     r = run_child(body2, {"ESHKOL_HIP_F64_KERNEL": "ozaki-crt", "EXPECT_ERR": "1e-9", "ESHKOL_GPU_THRESHOLD": "1",
                           "ESHKOL_GPU_VERBOSE": "1"})
