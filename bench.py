@@ -37,22 +37,28 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def read_traffic(name):
-    """HBM bytes per launch from the committed rocprofv3 --pmc summary, if any."""
+def read_traffic(name, kernel):
+    """HBM bytes per launch from the committed rocprofv3 --pmc summary, and the file it came
+    from: (bytes, source). The figure is a record of an earlier run of the same command, not
+    something this run measures, so it is only passed on when the summary names the kernel
+    this run's roofline is about (its KERNEL line); otherwise (None, None)."""
     path = os.path.join(ROOT, "profiles", name)
     if not os.path.exists(path):
-        return None
-    vals = {}
+        return None, None
+    vals, measured_kernel = {}, ""
     for line in open(path):
         if "=" in line and not line.lstrip().startswith("#"):
             k, v = line.split("=", 1)
+            if k.strip() == "KERNEL":
+                measured_kernel = v.strip()
+                continue
             try:
                 vals[k.strip()] = float(v.split()[0])
             except ValueError:
                 pass
-    if "HBM_BYTES_PER_LAUNCH" in vals:
-        return vals["HBM_BYTES_PER_LAUNCH"]
-    return None
+    if "HBM_BYTES_PER_LAUNCH" in vals and measured_kernel and measured_kernel == kernel.split("<")[0]:
+        return vals["HBM_BYTES_PER_LAUNCH"], "profiles/" + name
+    return None, None
 
 
 def main():
@@ -173,19 +179,23 @@ def main():
     log("native fp64: %.3f ms/step (events %.3f ms) %.1f GFLOP/s" % (wall_ms, ev_ms, native_gflops))
     # what the device itself sustains on a register-only MFMA loop / a large copy
     sustained = {}
+    probe = ea.load_probe()
     for name, kind, rnd in (("fp64_mfma_constant_operands", 0, 0), ("fp64_mfma_random_operands", 0, 1),
                             ("int8_mfma_constant_operands", 1, 0), ("int8_mfma_random_operands", 1, 1),
                             ("bf16_mfma_constant_operands", 2, 0), ("bf16_mfma_random_operands", 2, 1),
                             ("hbm_copy_read_plus_write", 3, 0)):
         rate = C.c_double()
-        if lib.hip_probe_peak(kind, rnd, C.byref(rate), st) == 0:
+        if probe.hip_probe_peak(kind, rnd, C.byref(rate), st) == 0:
             sustained[name] = rate.value / 1e12
     log("device sustains (T/s):", json.dumps(sustained))
     fast = (M % 128 == 0 and N % 128 == 0 and K % 16 == 0)
-    roofline = {"bound": "mfma", "kernel": "dgemm_fast_kernel<NN>" if fast else "dgemm_mfma_kernel<128,128>",
+    kernel = "dgemm_fast_kernel<NN>" if fast else "dgemm_mfma_kernel<128,128>"
+    traffic, traffic_source = read_traffic("dgemm_8192_hbm_traffic.txt", kernel)
+    roofline = {"bound": "mfma", "kernel": kernel,
                 "achieved": achieved / 1e12, "peak": PEAK["fp64_mfma"] / 1e12, "unit": "TFLOP/s",
                 "frac": achieved / PEAK["fp64_mfma"], "launch_ms": ev_ms,
-                "traffic": read_traffic("dgemm_8192_hbm_traffic.txt")}
+                "traffic": traffic if (M, K, N) == (8192, 8192, 8192) else None,
+                "traffic_source": traffic_source if (M, K, N) == (8192, 8192, 8192) else None}
     tiers = {"native_fp64": {"ms": wall_ms, "gflops": native_gflops, "frac_of_peak": achieved / PEAK["fp64_mfma"],
                              "peak": "fp64 MFMA 78.6 TFLOP/s", "normwise_error_sampled_rows": native_error}}
 

@@ -61,7 +61,7 @@ class HipOzakiInt8Stages(C.Structure):
 
 BUF = C.POINTER(EshkolGPUBuffer)
 
-# name -> (restype, argtypes); every symbol the two public headers declare
+# name -> (restype, argtypes); every symbol the two public headers and the testing header declare
 SIGNATURES = {
     # gpu_memory.h
     "eshkol_gpu_init": (C.c_int, []),
@@ -142,7 +142,6 @@ SIGNATURES = {
     "hip_matmul_backward_f64": (C.c_int, [vp, vp, vp, vp, vp, u64, u64, u64, C.c_int, C.c_int, vp]),
     "hip_hgemm_16": (C.c_int, [vp, vp, u64, u64, u64, u64, C.c_int, vp, vp]),
     "hip_convert_f64_to_16": (C.c_int, [vp, vp, u64, u64, u64, u64, C.c_int, vp]),
-    "hip_probe_peak": (C.c_int, [C.c_int, C.c_int, dp, vp]),
     "hip_igemm_set_persistent": (None, [C.c_int]),
     "hip_ozaki_crt_prepare_operand_b": (C.c_int, [vp, u64, u64, C.c_int, C.c_int, u64, C.POINTER(vp), vp]),
     "hip_matmul_ozaki_crt_prepared_f64": (C.c_int, [vp, vp, vp, u64, u64, u64, C.c_int, C.c_int, C.c_int, vp, C.c_int, vp]),
@@ -186,6 +185,18 @@ def load():
         fn.argtypes = args
     _lib = lib
     return lib
+
+
+def load_probe():
+    """The device probe of the benchmark (libeshkol_gpu_probe.so: register-only MFMA
+    loops and a large copy). Not part of the product library."""
+    path = os.path.join(PKG, "lib", "libeshkol_gpu_probe.so")
+    if not os.path.exists(path):
+        raise RuntimeError("libeshkol_gpu_probe.so is not built (%s); run `python -m eshkol_amd.build`" % path)
+    probe = C.CDLL(path)
+    probe.hip_probe_peak.restype = C.c_int
+    probe.hip_probe_peak.argtypes = [C.c_int, C.c_int, dp, vp]
+    return probe
 
 
 def hip_runtime():

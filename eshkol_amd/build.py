@@ -30,8 +30,11 @@ SOURCES = [
     "ozaki_int8.hip",
     "elementwise.hip",
     "ozaki_fast.hip",
-    "peak_probe.hip",
 ]
+# A device probe for the benchmark (register-only MFMA loops, a large copy): a
+# library of its own, so that the product library carries no measurement code.
+PROBE_LIB = os.path.join(LIBDIR, "libeshkol_gpu_probe.so")
+PROBE_SOURCES = ["peak_probe.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
@@ -114,6 +117,97 @@ def sgpr_to_vmem_hazards(asm):
     return found
 
 
+def hidden_load_violations(asm, kernels, limit=400000):
+    """Places in gfx9 assembly text where an instruction of one of the named kernels touches
+    a vector register that a vector memory load may still be writing. The kernels of
+    gemm_pipe2.h issue their loads from asm statements and wait for them with hand-counted
+    `s_waitcnt vmcnt(N)`, so the compiler neither knows that a ring register's value arrives
+    late nor checks the counts: a copy of such a register that the compiler places before the
+    wait (v_mov, v_accvgpr_write, a spill), or a count that is too large, would use stale data
+    with no error. The model is the hardware's: loads return in issue order, so after
+    vmcnt(N) every load but the N youngest has landed (stores share the counter but only make
+    a wait stricter); loads into LDS hold a place in that order and write no register. Every
+    path of the control-flow graph is followed, a state being the ordered destinations of the
+    loads in flight. Returns a list of (kernel, line number, text, registers). What this does
+    not see is whether a load INTO LDS has landed before the barrier that publishes it: that
+    rests on the counts and on the bit-exact tests."""
+    def vregs(tok):
+        m = re.fullmatch(r"v(\d+)", tok)
+        if m:
+            return frozenset({int(m.group(1))})
+        m = re.fullmatch(r"v\[(\d+):(\d+)\]", tok)
+        if m:
+            return frozenset(range(int(m.group(1)), int(m.group(2)) + 1))
+        return frozenset()
+
+    bodies, cur = {}, None
+    for no, raw in enumerate(asm.split("\n"), 1):
+        text = raw.split(";")[0].strip()
+        if text.endswith(":") and not text.startswith(".") and not raw.startswith(("\t", " ")):
+            cur = text[:-1] if any(k in text for k in kernels) else None
+            if cur:
+                bodies[cur] = []
+        elif cur is not None:
+            if text.startswith((".end_amdhsa_kernel", ".Lfunc_end")):
+                cur = None
+            elif text:
+                bodies[cur].append((no, text))
+
+    found = []
+    for kernel, body in bodies.items():
+        blocks, label_at, block = [], {}, []
+        for no, text in body:
+            if text.endswith(":"):
+                if block:
+                    blocks.append(block)
+                    block = []
+                label_at[text[:-1]] = len(blocks)
+            elif not text.startswith("."):
+                block.append((no, text))
+                op = text.split()[0]
+                if op in ("s_branch", "s_endpgm") or op.startswith("s_cbranch"):
+                    blocks.append(block)
+                    block = []
+        if block:
+            blocks.append(block)
+        seen, work, bad = set(), [(0, ())], {}
+        while work:
+            bi, state = work.pop()
+            if (bi, state) in seen or bi >= len(blocks):
+                continue
+            seen.add((bi, state))
+            if len(seen) > limit:
+                raise RuntimeError("%s: too many pipeline states to follow" % kernel)
+            fifo, succ = list(state), None
+            for no, text in blocks[bi]:
+                parts = text.replace(",", " ").split()
+                op, ops = parts[0], parts[1:]
+                if op == "s_waitcnt":
+                    m = re.search(r"vmcnt\((\d+)\)", text)
+                    if m and len(fifo) > int(m.group(1)):
+                        fifo = fifo[len(fifo) - int(m.group(1)):]
+                    continue
+                used = frozenset().union(*[vregs(t) for t in ops]) if ops else frozenset()
+                if used:
+                    for regs in fifo:
+                        if regs & used:
+                            bad.setdefault(no, (text, sorted(regs & used)))
+                            break
+                if op.startswith(("buffer_load", "global_load", "flat_load", "scratch_load")):
+                    fifo.append(frozenset() if "lds" in ops else vregs(ops[0]))
+                    fifo = fifo[-63:]                     # the counter saturates there; older loads have landed
+                if op == "s_endpgm":
+                    succ = []
+                elif op == "s_branch":
+                    succ = [label_at[ops[0]]]
+                elif op.startswith("s_cbranch"):
+                    succ = [label_at[ops[0]], bi + 1]
+            for t in ([bi + 1] if succ is None else succ):
+                work.append((t, tuple(fifo)))
+        found += [(kernel, no) + v for no, v in sorted(bad.items())]
+    return found
+
+
 def _check_hazards(src):
     """Compiles src to assembly with the flags of the build and scans it."""
     path = os.path.join(CSRC, src)
@@ -125,6 +219,10 @@ def _check_hazards(src):
     if found:
         raise RuntimeError("%s: memory instructions read scalar registers too soon after a vector instruction "
                            "wrote them:\n%s" % (src, "\n".join("  line %d: %s (%d wait states)" % f for f in found[:10])))
+    late = hidden_load_violations(res.stdout, NO_SPILL[src])
+    if late:
+        raise RuntimeError("%s: registers are used while a load issued from an asm statement may still be writing "
+                           "them:\n%s" % (src, "\n".join("  %s line %d: %s %s" % f for f in late[:10])))
 
 
 def _newer(target, deps):
@@ -139,7 +237,7 @@ def _compile(src, force):
     obj = os.path.join(OBJDIR, os.path.splitext(src)[0] + ".o")
     headers = [os.path.join(CSRC, h) for h in os.listdir(CSRC) if h.endswith(".h")]
     headers += [os.path.join(ROOT, "include", "eshkol", "backend", "gpu", h)
-                for h in ("gpu_memory.h", "gpu_hip_tiers.h")]
+                for h in ("gpu_memory.h", "gpu_hip_tiers.h", "gpu_hip_testing.h")]
     if not force and _newer(obj, [path] + headers):
         return obj
     cmd = [HIPCC] + COMMON + EXTRA.get(src, []) + ["-x", "hip", "-c", path, "-o", obj]
@@ -160,16 +258,17 @@ def _compile(src, force):
 def build(force=False, verbose=False):
     os.makedirs(OBJDIR, exist_ok=True)
     stale = [s for s in NO_SPILL if force or not _newer(LIB, [os.path.join(CSRC, f) for f in os.listdir(CSRC)])]
-    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
+    with ThreadPoolExecutor(max_workers=8) as pool:
         checks = [pool.submit(_check_hazards, s) for s in stale]      # the kernels that issue loads from asm
-        objs = list(pool.map(lambda s: _compile(s, force), SOURCES))
+        objs = list(pool.map(lambda s: _compile(s, force), SOURCES + PROBE_SOURCES))
         for c in checks:
             c.result()
-    if force or not _newer(LIB, objs):
-        cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs + ["-ldl", "-lpthread"]
-        res = subprocess.run(cmd, capture_output=True, text=True)
-        if res.returncode != 0:
-            raise RuntimeError("link failed:\n%s\n%s" % (res.stdout, res.stderr))
+    for lib, members in ((LIB, objs[:len(SOURCES)]), (PROBE_LIB, objs[len(SOURCES):])):
+        if force or not _newer(lib, members):
+            cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + members + ["-ldl", "-lpthread"]
+            res = subprocess.run(cmd, capture_output=True, text=True)
+            if res.returncode != 0:
+                raise RuntimeError("link failed:\n%s\n%s" % (res.stdout, res.stderr))
     if verbose:
         print("built", LIB)
     return LIB

@@ -899,13 +899,13 @@ int dgemm_any(const double* A, const double* B, double* C, uint64_t M, uint64_t 
 }  // namespace
 
 /* 0 routes every shape through the bounds-checked kernel (for comparisons). */
-extern "C" void hip_dgemm_set_fast_path(int on) { g_fast_path = on ? 1 : 0; }
+extern "C" void hip_dgemm_set_fast_path(int on) { EshkolHipLock lk; g_fast_path = on ? 1 : 0; }
 /* 0 keeps every tile whole (results then equal the bounds-checked kernel's bit for bit). */
-extern "C" void hip_dgemm_set_tail_split(int on) { g_tail_split = on ? 1 : 0; }
+extern "C" void hip_dgemm_set_tail_split(int on) { EshkolHipLock lk; g_tail_split = on ? 1 : 0; }
 /* 0: the straight-line kernel uses 128 x 128 tiles only; 1 (default): 64 x 64 tiles where
  * they measure faster; 2: 64 x 64 tiles wherever the straight-line kernel applies. */
-extern "C" void hip_dgemm_set_prefetch_depth(int depth) { g_prefetch_depth = (depth == 1 || depth == 2) ? depth : 0; }
-extern "C" void hip_dgemm_set_small_tile(int mode) { if (mode >= 0 && mode <= 2) g_small_tile = mode; }
+extern "C" void hip_dgemm_set_prefetch_depth(int depth) { EshkolHipLock lk; g_prefetch_depth = (depth == 1 || depth == 2) ? depth : 0; }
+extern "C" void hip_dgemm_set_small_tile(int mode) { EshkolHipLock lk; if (mode >= 0 && mode <= 2) g_small_tile = mode; }
 
 extern "C" int hip_dgemm_f64_ex(const double* A, const double* B, double* C,
                                 uint64_t M, uint64_t K, uint64_t N,

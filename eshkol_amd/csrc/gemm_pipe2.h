@@ -126,7 +126,7 @@ __device__ __forceinline__ void load_hidden(v4i_t& dst, const v4i_t& rs, uint32_
 template <int IMM>
 __device__ __forceinline__ void load_to_lds(uint32_t lds, const v4i_t& rs, uint32_t voff, uint32_t soff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen offset:%4 lds"
-                 :: "s"(lds), "v"(voff), "s"(rs), "s"(soff), "n"(IMM) : "memory");
+                 :: "s"(lds), "v"(voff), "s"(rs), "s"(soff), "n"(IMM) : "memory", "m0");
 }
 
 /* at most N loads still pending; the eight registers are the A fragments of the

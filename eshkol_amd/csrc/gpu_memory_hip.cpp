@@ -735,6 +735,9 @@ void eshkol_hip_leave(hipStream_t stream) {
     g_gpu_mutex.unlock();
 }
 
+void eshkol_hip_lock(void) { g_gpu_mutex.lock(); }
+void eshkol_hip_unlock(void) { g_gpu_mutex.unlock(); }
+
 void* eshkol_hip_workspace(int slot, size_t bytes) {
     if (slot < 0 || slot >= WS_COUNT) return nullptr;
     Slot& s = g_ws[slot];

@@ -780,7 +780,7 @@ int reduced_pipeline(const double* A, const double* B, double* C, uint64_t batch
 
 /* Tuning hook: 0 keeps the 16-bit tier on row-major operands and the
  * register-staged kernels. Same results. */
-extern "C" void hip_hgemm_set_direct(int on) { g_direct16 = on ? 1 : 0; }
+extern "C" void hip_hgemm_set_direct(int on) { EshkolHipLock lk; g_direct16 = on ? 1 : 0; }
 
 extern "C" int hip_hgemm_plane_layout(uint64_t M, uint64_t N, uint64_t batch) {
     const uint64_t tiles = ((M + 255) / 256) * ((N + 255) / 256) * batch;

@@ -58,6 +58,18 @@ struct EshkolHipCall {
     EshkolHipCall& operator=(const EshkolHipCall&) = delete;
 };
 
+/* The same mutex without the stream bookkeeping: for the process-wide switches
+ * and read-outs of gpu_hip_testing.h, so that none changes under a call that
+ * is inside the library. */
+void eshkol_hip_lock(void);
+void eshkol_hip_unlock(void);
+struct EshkolHipLock {
+    EshkolHipLock() { eshkol_hip_lock(); }
+    ~EshkolHipLock() { eshkol_hip_unlock(); }
+    EshkolHipLock(const EshkolHipLock&) = delete;
+    EshkolHipLock& operator=(const EshkolHipLock&) = delete;
+};
+
 /* Looks up, once per device, the current device's address of the static scratch
  * array behind hip_matmul_reduced_f64_noalloc (hgemm_16.hip). 0 on success. */
 int eshkol_hip_noalloc_setup(void);

@@ -631,14 +631,14 @@ int launch_simple(const HipIgemmArgs& a, hipStream_t st) {
 }  // namespace
 
 /* Tuning hook: k-blocks in flight in the pipelined kernel (1..3), 0 = simple kernel only. */
-extern "C" void hip_igemm_set_prefetch(int pf) { if (pf >= 0 && pf <= 3) g_prefetch = pf; }
+extern "C" void hip_igemm_set_prefetch(int pf) { EshkolHipLock lk; if (pf >= 0 && pf <= 3) g_prefetch = pf; }
 /* Tuning hook: 1 (default) runs the pipelined kernel as one workgroup per CU
  * walking a list of tiles, 0 as one workgroup per tile. Same results. */
-extern "C" void hip_igemm_set_persistent(int on) { g_persistent = on ? 1 : 0; }
+extern "C" void hip_igemm_set_persistent(int on) { EshkolHipLock lk; g_persistent = on ? 1 : 0; }
 
 /* Tuning hook: 0 keeps every launch on row-major planes and the register-staged
  * kernels. Same results. */
-extern "C" void hip_igemm_set_direct(int on) { g_direct = on ? 1 : 0; }
+extern "C" void hip_igemm_set_direct(int on) { EshkolHipLock lk; g_direct = on ? 1 : 0; }
 
 /* The plane layout the tiers should produce for a contraction of n_out output
  * planes of M x N: 1 (interleaved, for the direct-to-LDS kernel) when the launch

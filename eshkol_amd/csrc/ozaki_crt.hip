@@ -832,15 +832,17 @@ extern "C" int hip_ozaki_crt_reconstruct_f64(const int8_t* w_planes, uint64_t M,
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 
-extern "C" void hip_ozaki_crt_set_host_pass(int on) { g_force_host_pass = on != 0; }
+extern "C" void hip_ozaki_crt_set_host_pass(int on) { EshkolHipLock lk; g_force_host_pass = on != 0; }
 
 extern "C" int hip_ozaki_crt_set_aligned_weights(int on) {
+    EshkolHipLock lk;
     const int was = g_aligned_weights ? 1 : 0;
     g_aligned_weights = on != 0;
     return was;
 }
 
 extern "C" int hip_ozaki_crt_last_stages(HipOzakiCrtStages* out) {
+    EshkolHipLock lk;
     if (!out || !g_last.a_planes) return -1;
     *out = g_last;
     return 0;

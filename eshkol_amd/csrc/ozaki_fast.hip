@@ -469,6 +469,7 @@ extern "C" int hip_ozaki_fast_reconstruct_f64(const int8_t* w_planes, uint64_t M
 }
 
 extern "C" int hip_ozaki_fast_last_stages(HipOzakiFastStages* out) {
+    EshkolHipLock lk;
     if (!out || !g_last.a_planes) return -1;
     *out = g_last;
     return 0;

@@ -296,6 +296,7 @@ extern "C" int hip_ozaki_reconstruct_f64(double* C, const int32_t* Gall, const d
 }
 
 extern "C" int hip_ozaki_int8_last_stages(HipOzakiInt8Stages* out) {
+    EshkolHipLock lk;
     if (!out || !g_last.a_slices) return -1;
     *out = g_last;
     return 0;

@@ -13,9 +13,15 @@
  *
  * The memory probe is a plain 16-byte-per-lane copy of a buffer much larger
  * than the caches: the read+write rate HBM sustains.
+ *
+ * Built into libeshkol_gpu_probe.so, which only the benchmark loads: it is not
+ * part of libeshkol_gpu_hip.so and shares nothing with it.
  */
-#include "hip_common.h"
-#include "kernels.h"
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include "eshkol/backend/gpu/gpu_hip_testing.h"
+
+#define ESHKOL_HIP_OK(call) ((call) == hipSuccess)
 
 typedef int v4i_t __attribute__((ext_vector_type(4)));
 typedef int v16i_t __attribute__((ext_vector_type(16)));
@@ -124,8 +130,8 @@ extern "C" int hip_probe_peak(int kind, int random_operands, double* rate, void*
     float ms = 0.0f;
     if (kind == 3) {
         const size_t bytes = (size_t)1 << 30;
-        char* buf = (char*)eshkol_hip_workspace(WS_MISC, 2 * bytes);
-        if (buf) {
+        char* buf = nullptr;
+        if (ESHKOL_HIP_OK(hipMalloc((void**)&buf, 2 * bytes))) {
             for (int rep = 0; rep < 2; rep++) {
                 if (rep == 1) (void)hipEventRecord(e0, st);
                 hipLaunchKernelGGL(probe_copy, dim3(256 * 16), dim3(256), 0, st,
@@ -136,9 +142,11 @@ extern "C" int hip_probe_peak(int kind, int random_operands, double* rate, void*
                 *rate = 2.0 * (double)bytes / (ms * 1e-3);
                 rc = 0;
             }
+            (void)hipFree(buf);
         }
     } else {
-        int* sink = (int*)eshkol_hip_workspace(WS_MISC, 256);
+        int* sink = nullptr;
+        if (!ESHKOL_HIP_OK(hipMalloc((void**)&sink, 256))) sink = nullptr;
         const int wgs = 1024;
         const int iters = (kind == 0) ? 20000 : 40000;
         const double per_mfma = (kind == 0) ? 2048.0 : (kind == 1) ? 65536.0 : 32768.0;
@@ -154,6 +162,7 @@ extern "C" int hip_probe_peak(int kind, int random_operands, double* rate, void*
                 *rate = (double)wgs * 4.0 * iters * 8.0 * per_mfma / (ms * 1e-3);
                 rc = 0;
             }
+            (void)hipFree(sink);
         }
     }
     (void)hipEventDestroy(e0);

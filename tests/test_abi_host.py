@@ -29,10 +29,17 @@ def declared_functions(header):
 def test_library_exports_every_declared_symbol():
     lib = ea.load()
     declared = declared_functions("gpu_memory.h") + declared_functions("gpu_hip_tiers.h")
-    assert len(declared) >= 45
-    for name in declared:
+    hooks = declared_functions("gpu_hip_testing.h")
+    assert len(declared) >= 45 and len(hooks) >= 12
+    for name in declared + [h for h in hooks if not h.startswith("hip_probe_")]:
         assert hasattr(lib, name), name
         assert name in ea.SIGNATURES, "binding table is missing %s" % name
+    # the product headers declare no switch, read-out or probe, and the product library carries no probe:
+    # that one lives in a library of its own, which only the benchmark loads
+    assert not [n for n in declared if "_last_stages" in n or n.startswith("hip_probe_")]
+    assert [n for n in declared if "_set_" in n] == ["eshkol_gpu_set_threshold", "hip_ozaki_crt_set_aligned_weights"]
+    assert not hasattr(lib, "hip_probe_peak")
+    assert hasattr(ea.load_probe(), "hip_probe_peak")
     assert C.c_size_t.in_dll(lib, "g_gpu_threshold").value in (100000, int(os.environ.get("ESHKOL_GPU_THRESHOLD", 100000)))
 
 

@@ -1,5 +1,6 @@
-"""The build's scan for scalar-register hazards around memory instructions issued from asm statements."""
-from eshkol_amd.build import sgpr_to_vmem_hazards
+"""The build's scans of the kernels that issue memory instructions from asm statements: scalar-register
+hazards in front of them, and registers used while such a load may still be writing them."""
+from eshkol_amd.build import hidden_load_violations, sgpr_to_vmem_hazards
 
 RELOAD_THEN_ATOMIC = """
 	v_readlane_b32 s10, v233, 9
@@ -45,3 +46,47 @@ def test_other_scalar_registers_and_scalar_writers_do_not_count():
 """
     found = sgpr_to_vmem_hazards(asm)
     assert [(f[0], f[2]) for f in found] == [(8, 4)]
+
+
+RING = """
+ring_kernel:
+	buffer_load_dwordx4 v[0:3], v20, s[8:11], s20 offen
+	buffer_load_dwordx4 v[4:7], v20, s[8:11], s20 offen offset:1024
+	buffer_load_dwordx4 v20, s[12:15], s20 offen lds
+.LBB0_1:
+	s_waitcnt vmcnt(%d)
+	v_mfma_i32_32x32x32_i8 a[0:15], v[8:11], v[0:3], a[0:15]
+	buffer_load_dwordx4 v[0:3], v20, s[8:11], s20 offen
+	s_waitcnt vmcnt(2)
+	%s
+	v_mfma_i32_32x32x32_i8 a[0:15], v[8:11], v[4:7], a[0:15]
+	buffer_load_dwordx4 v[4:7], v20, s[8:11], s20 offen offset:1024
+	buffer_load_dwordx4 v20, s[12:15], s20 offen lds
+	s_cbranch_scc1 .LBB0_1
+	s_waitcnt vmcnt(0)
+	s_endpgm
+	.end_amdhsa_kernel
+other_kernel:
+	global_load_dword v1, v2, s[0:1]
+	v_add_u32 v1, v1, v1
+	s_endpgm
+"""
+
+
+def test_a_ring_register_read_after_a_sufficient_wait_is_fine_on_every_path():
+    # vmcnt(2): the first load has landed, at the loop's entry and on its back edge alike
+    assert hidden_load_violations(RING % (2, "s_nop 0"), ["ring_kernel"]) == []
+
+
+def test_a_wait_count_one_too_large_is_found():
+    found = hidden_load_violations(RING % (3, "s_nop 0"), ["ring_kernel"])
+    # the MFMA reads the register in flight, and the next load into it would overtake nothing but is flagged too
+    assert [(f[0], f[1], f[3]) for f in found] == [("ring_kernel", 8, [0, 1, 2, 3]), ("ring_kernel", 9, [0, 1, 2, 3])]
+
+
+def test_a_copy_of_a_ring_register_before_its_wait_is_found():
+    # what a compiler that does not know about the hidden load might insert: a move out of a register in flight
+    found = hidden_load_violations(RING % (2, "v_accvgpr_write_b32 a20, v0"), ["ring_kernel"])
+    assert [(f[1], f[3]) for f in found] == [(11, [0])]
+    # only the named kernels are scanned (other_kernel relies on the compiler's own waits)
+    assert hidden_load_violations(RING % (2, "s_nop 0"), ["other_kernel"]) != []
