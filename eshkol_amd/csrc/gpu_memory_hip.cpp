@@ -102,6 +102,9 @@ struct TierEnv {
     int  precision = 0;          /* ESHKOL_GPU_PRECISION: 0 exact, 1 high, 2 fast, 3 ml */
     bool overlap = true;         /* ESHKOL_GPU_OVERLAP=0: no row panels in the host-memory dispatch */
     bool crt_aligned = false;    /* ESHKOL_OZAKI_CRT_WEIGHTS=aligned: CRT weights split at a common bit */
+    /* ESHKOL_GPU_PREPARED_BYTES: device memory the residue planes kept for pinned tensors may
+     * take in all (16 bytes per element of each tensor, twice its own size); 0 keeps none */
+    size_t prepared_cap = (size_t)32 << 30;
 };
 TierEnv g_env;
 std::once_flag g_env_once;
@@ -147,6 +150,11 @@ void parse_env(void) {
     e.profile = getenv("ESHKOL_OZAKI_PROFILE") != nullptr;       /* gpu_memory.mm:2479 */
     if (const char* o = getenv("ESHKOL_GPU_OVERLAP")) e.overlap = strcmp(o, "0") != 0;
     if (const char* w = getenv("ESHKOL_OZAKI_CRT_WEIGHTS")) e.crt_aligned = strcmp(w, "aligned") == 0;
+    if (const char* pc = getenv("ESHKOL_GPU_PREPARED_BYTES")) {
+        char* end = nullptr;
+        const unsigned long long v = strtoull(pc, &end, 10);
+        if (end != pc) e.prepared_cap = (size_t)v;
+    }
     if (const char* a = getenv("ESHKOL_MATMUL_ACCURACY")) {      /* gpu_memory_cuda.cpp:527-539 */
         if (*a) {
             /* "exact", "full" and anything unparseable are the reference's strictest
@@ -368,9 +376,11 @@ struct Resident {
     const void* host; size_t bytes; void* dev;
     void* prepared = nullptr;           /* hip_ozaki_crt_prepare_operand_b handle */
     uint64_t prep_K = 0, prep_N = 0;
-    int prep_moduli = 0;
-    bool prep_refused = false;          /* the tier would not prepare this operand: do not ask again */
+    int prep_moduli = 0, prep_layout = 0;
+    size_t prep_bytes = 0;
+    bool prep_refused = false;          /* the tier would not prepare these contents: do not ask again until they change */
 };
+size_t g_prepared_bytes = 0;            /* planes held for all resident tensors together */
 std::vector<Resident> g_resident;
 
 Resident* resident_find(const void* host) {
@@ -384,8 +394,9 @@ Resident* resident_find_device(const void* dev) {
 }
 
 void resident_drop_prepared(Resident& r) {
-    if (r.prepared) hip_ozaki_crt_release_prepared(r.prepared);
-    r.prepared = nullptr; r.prep_K = r.prep_N = 0; r.prep_moduli = 0; r.prep_refused = false;
+    if (r.prepared) { hip_ozaki_crt_release_prepared(r.prepared); g_prepared_bytes -= r.prep_bytes; }
+    r.prepared = nullptr; r.prep_K = r.prep_N = 0; r.prep_moduli = 0; r.prep_layout = 0; r.prep_bytes = 0;
+    r.prep_refused = false;
 }
 
 void resident_release_all(void) {
@@ -394,19 +405,44 @@ void resident_release_all(void) {
 }
 
 /* The prepared form of the resident tensor at device address dB as the K x N second
- * operand of the exact tier, made on first use; NULL if dB is not resident or the
- * tier declines (then the call prepares nothing and splits B as always). */
+ * operand of the exact tier, made on first use; NULL if dB is not resident, the
+ * tier declines or the byte cap is reached (then the call prepares nothing and
+ * splits B as always, which a verbose run says once per tensor). Planes made for
+ * the other plane layout (a product whose row count puts it on the other side of
+ * hip_igemm_plane_layout) are made again for this one: keeping them would mean
+ * splitting B on every such call while they sit in device memory unused. A
+ * failed allocation is not remembered; a refusal that depends on the contents
+ * is, until pin or refresh bring new contents. */
 void* resident_prepared_b(const double* dB, uint64_t M, uint64_t K, uint64_t N, int moduli) {
     Resident* r = resident_find_device(dB);
     if (!r || r->bytes != K * N * sizeof(double)) return nullptr;
-    if (r->prepared && (r->prep_K != K || r->prep_N != N || r->prep_moduli != moduli)) resident_drop_prepared(*r);
+    const int layout = hip_igemm_plane_layout(M, N, moduli);
+    if (r->prepared && (r->prep_K != K || r->prep_N != N || r->prep_moduli != moduli || r->prep_layout != layout)) {
+        if (r->prep_K == K && r->prep_N == N && r->prep_moduli == moduli)
+            GPU_LOG("resident operand %p: residue planes are in the %s layout, this product wants the other: "
+                    "preparing them again", r->host, r->prep_layout ? "interleaved" : "row-major");
+        resident_drop_prepared(*r);
+    }
     if (!r->prepared && !r->prep_refused) {
-        if (hip_ozaki_crt_prepare_operand_b(dB, K, N, 0, moduli, M, &r->prepared, g_stream) == 0) {
-            r->prep_K = K; r->prep_N = N; r->prep_moduli = moduli;
-            GPU_LOG("resident operand %p: residue planes of the exact tier prepared (%llux%llu, %d moduli)",
-                    r->host, (unsigned long long)K, (unsigned long long)N, moduli);
+        const size_t want = (size_t)moduli * round_up_sz(N, 256) * round_up_sz(K, layout ? 512 : 256);
+        const size_t cap = tier_env().prepared_cap;
+        if (g_prepared_bytes + want > cap) {
+            GPU_LOG("resident operand %p: %zu bytes of residue planes would exceed ESHKOL_GPU_PREPARED_BYTES=%zu "
+                    "(%zu in use); this operand is split on every call", r->host, want, cap, g_prepared_bytes);
+            r->prep_refused = true;
+            return nullptr;
+        }
+        const int rc = hip_ozaki_crt_prepare_operand_b(dB, K, N, 0, moduli, M, &r->prepared, g_stream);
+        if (rc == 0) {
+            r->prep_K = K; r->prep_N = N; r->prep_moduli = moduli; r->prep_layout = layout; r->prep_bytes = want;
+            g_prepared_bytes += want;
+            GPU_LOG("resident operand %p: residue planes of the exact tier prepared (%llux%llu, %d moduli, %zu bytes)",
+                    r->host, (unsigned long long)K, (unsigned long long)N, moduli, want);
         } else {
-            r->prepared = nullptr; r->prep_refused = true;
+            r->prepared = nullptr;
+            r->prep_refused = (rc != -2);           /* -2: no memory right now, ask again next time */
+            GPU_LOG("resident operand %p: the exact tier %s; it is split on every call", r->host,
+                    rc == -2 ? "has no memory for residue planes right now" : "does not prepare these contents");
         }
     }
     return r->prepared;
@@ -821,7 +857,11 @@ void eshkol_gpu_shutdown(void) {
     std::lock_guard<std::recursive_mutex> g(g_gpu_mutex);
     if (g_backend == ESHKOL_GPU_HIP) {
         if (g_stream) hipStreamSynchronize(g_stream);
+        (void)hipDeviceSynchronize();               /* the scan's stream and callers' own streams included */
         eshkol_hip_workspace_release();
+        eshkol_hip_crt_release();
+        eshkol_hip_fast_release();
+        eshkol_hip_int8_release();
         eshkol_hip_copy_release();
         staging_release_all();
         resident_release_all();

@@ -606,19 +606,29 @@ void hgemm_direct_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
     pipe2::run_tiles<H16Op<BF16>>(smem_h, cm, next_tile, epi);
 }
 
+/* The dynamic-LDS attribute of a kernel, set once per kernel and process: a list
+ * under a mutex instead of a static flag per launcher, so that the first calls
+ * of two threads do not race and so that hip_matmul_reduced_f64_noalloc's
+ * set-up can run every launcher's part ahead of its first call. */
+bool kernel_ready(const void* kern, int smem) {
+    static std::mutex m;
+    static const void* done[16];
+    static int n_done = 0;
+    std::lock_guard<std::mutex> lk(m);
+    for (int i = 0; i < n_done; i++) if (done[i] == kern) return true;
+    if (!ESHKOL_HIP_OK(hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem))) return false;
+    if (n_done < 16) done[n_done++] = kern;
+    return true;
+}
+
 template <bool BF16>
 int launch_direct(const uint16_t* A, const uint16_t* Bt, int M, int N, int ld_bytes, int out_mode, void* C,
                   int batch, uint64_t a_stride, uint64_t b_stride, hipStream_t st) {
     constexpr int SMEM = pipe2::SMEM_BYTES;
-    static bool attr_set = false;
-    static int num_cus = 0;
     auto kern = hgemm_direct_kernel<BF16>;
-    if (!attr_set) {
-        if (!ESHKOL_HIP_OK(hipFuncSetAttribute((const void*)kern,
-                hipFuncAttributeMaxDynamicSharedMemorySize, SMEM))) return -1;
-        num_cus = eshkol_hip_num_cus();
-        attr_set = true;
-    }
+    if (!kernel_ready((const void*)kern, SMEM)) return -1;
+    const int num_cus = eshkol_hip_num_cus();
+    if (!A) return 0;                                        /* set-up only */
     const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
     const long long total = (long long)tiles_m * tiles_n * batch;
     if (total > 0x7ffffff0LL) return -1;
@@ -635,18 +645,10 @@ template <bool BF16>
 int launch_pipe(const uint16_t* A, const uint16_t* Bt, int M, int N, int ld_bytes, int out_mode, void* C,
                 hipStream_t st) {
     constexpr int SMEM = pipe::TilesCfg<4, 4>::SMEM_MAIN;
-    static bool attr_set = false;
-    static int num_cus = 0;
     auto kern = hgemm_pipe_kernel<BF16, 2>;
-    if (!attr_set) {
-        if (!ESHKOL_HIP_OK(hipFuncSetAttribute((const void*)kern,
-                hipFuncAttributeMaxDynamicSharedMemorySize, SMEM))) return -1;
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (!ESHKOL_HIP_OK(hipGetDevice(&dev)) || !ESHKOL_HIP_OK(hipGetDeviceProperties(&prop, dev))) return -1;
-        num_cus = prop.multiProcessorCount;
-        attr_set = true;
-    }
+    if (!kernel_ready((const void*)kern, SMEM)) return -1;
+    const int num_cus = eshkol_hip_num_cus();
+    if (!A) return 0;                                        /* set-up only */
     const int tiles_m = (M + 255) / 256, tiles_n = (N + 255) / 256;
     const int n_ids = (tiles_m * tiles_n + 7) / 8 * 8;      /* padded so every XCD owns the same count */
     int grid = (num_cus / 8) * 8;
@@ -661,13 +663,9 @@ template <bool BF16, int TM, int TN>
 int launch(const uint16_t* A, const uint16_t* Bt, int M, int N, int ld_bytes, int out_mode, void* C,
            int batch, uint64_t a_stride, uint64_t b_stride, hipStream_t st) {
     using Cf = Cfg<TM, TN>;
-    static bool attr_set = false;
     auto kern = hgemm_kernel<BF16, TM, TN>;
-    if (!attr_set) {
-        if (!ESHKOL_HIP_OK(hipFuncSetAttribute((const void*)kern,
-                hipFuncAttributeMaxDynamicSharedMemorySize, Cf::SMEM_BYTES))) return -1;
-        attr_set = true;
-    }
+    if (!kernel_ready((const void*)kern, Cf::SMEM_BYTES)) return -1;
+    if (!A) return 0;                                        /* set-up only */
     const int tiles_m = (M + Cf::BM - 1) / Cf::BM, tiles_n = (N + Cf::BN - 1) / Cf::BN;
     const long long nwg = (long long)tiles_m * tiles_n;
     if (nwg > 0x7fffffffLL) return -1;
@@ -875,7 +873,23 @@ unsigned char* noalloc_scratch(void) {
 }
 }  // namespace
 
-int eshkol_hip_noalloc_setup(void) { return noalloc_scratch() ? 0 : -1; }
+/* Everything hip_matmul_reduced_f64_noalloc would otherwise do on its first
+ * call with some shape: the scratch address, every contraction kernel's LDS
+ * attribute, the CU count. After it the entry point only launches kernels. */
+int eshkol_hip_noalloc_setup(void) {
+    if (!noalloc_scratch()) return -1;
+    (void)eshkol_hip_num_cus();
+    int rc = 0;
+    rc |= launch_direct<true>(nullptr, nullptr, 0, 0, 0, 0, nullptr, 0, 0, 0, nullptr);
+    rc |= launch_direct<false>(nullptr, nullptr, 0, 0, 0, 0, nullptr, 0, 0, 0, nullptr);
+    rc |= launch_pipe<true>(nullptr, nullptr, 0, 0, 0, 0, nullptr, nullptr);
+    rc |= launch_pipe<false>(nullptr, nullptr, 0, 0, 0, 0, nullptr, nullptr);
+    rc |= launch<true, 4, 4>(nullptr, nullptr, 0, 0, 0, 0, nullptr, 0, 0, 0, nullptr);
+    rc |= launch<false, 4, 4>(nullptr, nullptr, 0, 0, 0, 0, nullptr, 0, 0, 0, nullptr);
+    rc |= launch<true, 2, 2>(nullptr, nullptr, 0, 0, 0, 0, nullptr, 0, 0, 0, nullptr);
+    rc |= launch<false, 2, 2>(nullptr, nullptr, 0, 0, 0, 0, nullptr, 0, 0, 0, nullptr);
+    return rc == 0 ? 0 : -1;
+}
 
 extern "C" size_t hip_matmul_reduced_f64_noalloc_limit(void) { return NOALLOC_SCRATCH_BYTES; }
 

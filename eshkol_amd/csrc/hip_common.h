@@ -42,6 +42,14 @@ enum {
 void* eshkol_hip_workspace(int slot, size_t bytes);
 void  eshkol_hip_workspace_release(void);
 
+/* What each tier keeps for the life of the process besides the workspace (small
+ * device tables, the scan's pinned mailbox, stream and event): released by
+ * eshkol_gpu_shutdown(), with the library mutex held and the device idle; the
+ * next call after a new eshkol_gpu_init() makes them again. */
+void eshkol_hip_crt_release(void);
+void eshkol_hip_fast_release(void);
+void eshkol_hip_int8_release(void);
+
 /* Brackets a public tier entry point (hip_matmul_*, hip_dgemm_*, hip_igemm_i8,
  * hip_colabsmax_f64): takes the library's recursive mutex, the one the eshkol_*
  * entry points hold, and, if the previous bracketed call queued its work on

@@ -832,6 +832,17 @@ extern "C" int hip_ozaki_crt_reconstruct_f64(const int8_t* w_planes, uint64_t M,
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 
+void eshkol_hip_crt_release(void) {
+    if (g_tables) { (void)hipFree(g_tables); g_tables = nullptr; }
+    if (g_mailbox) { (void)hipHostFree(g_mailbox); g_mailbox = nullptr; g_mailbox_dev = nullptr; }
+    if (g_pinned) { (void)hipHostFree(g_pinned); g_pinned = nullptr; g_pinned_bytes = 0; }
+    if (g_scan_event) { (void)hipEventDestroy(g_scan_event); g_scan_event = nullptr; }
+    if (g_scan_stream) { (void)hipStreamDestroy(g_scan_stream); g_scan_stream = nullptr; }
+    g_scan_ran_on = nullptr;
+    g_ticket = 0;
+    g_last = HipOzakiCrtStages{};
+}
+
 extern "C" void hip_ozaki_crt_set_host_pass(int on) { EshkolHipLock lk; g_force_host_pass = on != 0; }
 
 extern "C" int hip_ozaki_crt_set_aligned_weights(int on) {
@@ -1108,7 +1119,7 @@ extern "C" int hip_ozaki_crt_prepare_operand_b(const double* B, uint64_t K, uint
     };
     if (!ESHKOL_HIP_OK(hipMalloc((void**)&pb->bmax, N * sizeof(double))) ||
         !ESHKOL_HIP_OK(hipMalloc((void**)&pb->nu, N * sizeof(int32_t))) ||
-        !ESHKOL_HIP_OK(hipMalloc((void**)&pb->planes, (size_t)num_moduli * Np * ldk))) { (void)hipGetLastError(); return fail(); }
+        !ESHKOL_HIP_OK(hipMalloc((void**)&pb->planes, (size_t)num_moduli * Np * ldk))) { (void)hipGetLastError(); fail(); return -2; }
     if ((b_kmajor ? eshkol_colabsmax_shift_f64(B, K, N, 0.0, pb->bmax, pb->nu, 52, st)
                   : eshkol_rowabsmax_shift_f64(B, N, K, 0.0, pb->bmax, pb->nu, 52, st)) != 0)
         return fail();

@@ -468,6 +468,12 @@ extern "C" int hip_ozaki_fast_reconstruct_f64(const int8_t* w_planes, uint64_t M
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 
+void eshkol_hip_fast_release(void) {
+    if (g_tables) { (void)hipFree(g_tables); g_tables = nullptr; }
+    memset(g_tables_key, 0, sizeof g_tables_key);
+    g_last = HipOzakiFastStages{};
+}
+
 extern "C" int hip_ozaki_fast_last_stages(HipOzakiFastStages* out) {
     EshkolHipLock lk;
     if (!out || !g_last.a_planes) return -1;

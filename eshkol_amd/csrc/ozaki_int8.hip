@@ -295,6 +295,12 @@ extern "C" int hip_ozaki_reconstruct_f64(double* C, const int32_t* Gall, const d
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 
+void eshkol_hip_int8_release(void) {
+    if (g_plan_dev) { (void)hipFree(g_plan_dev); g_plan_dev = nullptr; }
+    g_plan_valid = false;
+    g_last = HipOzakiInt8Stages{};
+}
+
 extern "C" int hip_ozaki_int8_last_stages(HipOzakiInt8Stages* out) {
     EshkolHipLock lk;
     if (!out || !g_last.a_slices) return -1;

@@ -577,6 +577,75 @@ assert np.array_equal(ea.matmul_dispatch(X, W), oracle.matmul_ozaki_crt(X, W))
     assert r.stderr.count("residue planes of the exact tier prepared") == 2      # once after pin, once after refresh
 
 
+def test_resident_planes_follow_the_plane_layout_and_the_byte_cap(gpu):
+    """Planes prepared for one plane layout are made again when a product wants the other
+    (512 rows: 64 tiles, row-major planes; 1024 rows: 128 tiles, interleaved), with a line in
+    the verbose log, instead of staying in memory unused while B is split on every call; and
+    ESHKOL_GPU_PREPARED_BYTES bounds what they may take (0: none). Results are the unpinned
+    path's either way."""
+    body = r"""
+K, N = 1024, 512
+W = synth.xavier_uniform(5, K, N)
+assert lib.eshkol_gpu_resident_pin(W.ctypes.data, W.nbytes) == 0
+for M in (512, 1024, 1024, 512):
+    X = synth.normal(M, (M, K))
+    assert np.array_equal(ea.matmul_dispatch(X, W), oracle.matmul_ozaki_crt(X, W)), M
+lib.eshkol_gpu_resident_unpin(W.ctypes.data)
+"""
+    env = {"ESHKOL_HIP_F64_KERNEL": "ozaki-crt", "ESHKOL_GPU_THRESHOLD": "1", "ESHKOL_GPU_VERBOSE": "1"}
+    r = run_child(body, env)
+    assert r.stderr.count("residue planes of the exact tier prepared") == 3
+    assert r.stderr.count("this product wants the other: preparing them again") == 2
+    r = run_child(body, dict(env, ESHKOL_GPU_PREPARED_BYTES="0"))
+    assert "residue planes of the exact tier prepared" not in r.stderr
+    assert r.stderr.count("would exceed ESHKOL_GPU_PREPARED_BYTES=0") == 1       # said once, then remembered
+
+
+def test_shutdown_releases_what_the_tiers_keep_and_a_new_init_starts_over(gpu):
+    """eshkol_gpu_shutdown() frees the tiers' own tables, the scan's mailbox, stream and event
+    besides workspace, staging and resident memory; after eshkol_gpu_init() every tier works
+    again and gives the same bits."""
+    body = r"""
+n = 1024
+A = synth.wide_range(1, (n, n), -6, 6); B = synth.wide_range(2, (n, n), -6, 6)
+def all_tiers():
+    st = lib.eshkol_hip_get_stream()
+    dA, dB, dC = ea.DeviceArray.from_host(A), ea.DeviceArray.from_host(B), ea.DeviceArray((n, n))
+    out = []
+    for call in (lambda: lib.hip_matmul_ozaki_crt_f64(dA.ptr, dB.ptr, dC.ptr, n, n, n, 16, 0, None, 0, st),
+                 lambda: lib.hip_matmul_ozaki_fast_f64(dA.ptr, dB.ptr, dC.ptr, n, n, n, 11, st),
+                 lambda: lib.hip_matmul_ozaki_int8_f64(dA.ptr, dB.ptr, dC.ptr, n, n, n, 4, st),
+                 lambda: lib.hip_matmul_reduced_f64(dA.ptr, dB.ptr, dC.ptr, n, n, n, 3, 0, st)):
+        assert call() == 0
+        ea.synchronize()
+        out.append(dC.download())
+    for d in (dA, dB, dC):
+        d.free()
+    return out
+assert lib.eshkol_gpu_init() == 1
+hip = ea.hip_runtime()
+def free_bytes():
+    f, t = C.c_size_t(), C.c_size_t()
+    assert hip.hipMemGetInfo(C.byref(f), C.byref(t)) == 0
+    return f.value
+base = free_bytes()
+first = all_tiers()
+assert np.array_equal(first[0], oracle.matmul_ozaki_crt(A, B))
+held = base - free_bytes()
+lib.eshkol_gpu_shutdown()
+assert lib.eshkol_gpu_get_backend() == ea.GPU_NONE
+released = held - (base - free_bytes())
+print("HELD %d RELEASED %d" % (held, released))
+assert held > (16 << 20) and released >= held - (4 << 20)        # workspace and tables are gone
+assert lib.eshkol_gpu_init() == 1
+again = all_tiers()
+for a, b in zip(first, again):
+    assert np.array_equal(a, b)
+lib.eshkol_gpu_shutdown()
+"""
+    run_child(body)
+
+
 def test_threshold_env_forces_gpu(gpu):
     body = r"""
 A = synth.normal(1, (8, 8)); B = np.eye(8)

@@ -36,6 +36,42 @@ def test_noalloc_equals_workspace_entry_point_twice_in_a_row():
     assert np.abs(got2 - ref).max() <= 2e-2 * np.abs(ref).max() + 0.2
 
 
+def test_noalloc_takes_no_device_memory_on_first_use_of_a_shape():
+    """Shapes this process has not multiplied before, one per contraction kernel the entry point
+    can reach (the direct kernel on interleaved operands, the small-tile kernel): the device's
+    free memory is the same before and after, i.e. neither the call nor anything it sets up on
+    first use (kernel attributes, the CU count) allocates. Results against the workspace entry
+    point afterwards, which may allocate."""
+    import ctypes as C
+    lib = ea.init()
+    hip = ea.hip_runtime()
+    hip.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+
+    def free_bytes():
+        free, total = C.c_size_t(), C.c_size_t()
+        assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+        return free.value
+
+    cases = [((4096, 384, 4096), 3, 0), ((310, 205, 99), 2, 1)]
+    held = []
+    for (M, K, N), dtype, rnd in cases:
+        print("case: noalloc first use %dx%dx%d dtype %d" % (M, K, N, dtype), flush=True)
+        held.append((Operands(synth.normal(21, (M, K), 1.0), synth.normal(22, (K, N), 1.0)), dtype, rnd))
+    ea.synchronize()
+    before = free_bytes()
+    got = []
+    for ops, dtype, rnd in held:
+        assert lib.hip_matmul_reduced_f64_noalloc(ops.dA.ptr, ops.dB.ptr, ops.dC.ptr, ops.M, ops.K, ops.N,
+                                                  dtype, rnd, stream()) == 0
+        ea.synchronize()
+        assert free_bytes() == before
+        got.append(ops.result())
+    for (ops, dtype, rnd), g in zip(held, got):
+        assert lib.hip_matmul_reduced_f64(ops.dA.ptr, ops.dB.ptr, ops.dC.ptr, ops.M, ops.K, ops.N,
+                                          dtype, rnd, stream()) == 0
+        assert np.array_equal(g, ops.result())
+
+
 def test_noalloc_rejects_sizes_beyond_its_scratch():
     lib = ea.init()
     limit = lib.hip_matmul_reduced_f64_noalloc_limit()
