@@ -14,6 +14,8 @@ LIB_PATH = os.path.join(HERE, "liboracle.so")
 HOSTRT_PATH = os.path.join(HERE, "liboracle_hostrt.so")
 REF_PATH = os.path.join(HERE, "_ref", "libeshkol_ref.so")
 REF_SSE2_PATH = os.path.join(HERE, "_ref", "libeshkol_ref_sse2.so")
+# the same reference sources built with -DESHKOL_GPU_ENABLED: the caller side of the GPU boundary
+REF_GPU_PATH = os.path.join(HERE, "_ref", "libeshkol_ref_gpu.so")
 
 u64, i64 = C.c_uint64, C.c_int64
 dp = C.POINTER(C.c_double)

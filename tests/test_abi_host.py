@@ -308,3 +308,21 @@ def test_plane_layout_decisions_are_host_arithmetic():
     finally:
         lib.hip_igemm_set_direct(1)
         lib.hip_hgemm_set_direct(1)
+
+
+def test_reference_caller_links_against_the_library():
+    """oracle/_ref/libeshkol_ref_gpu.so (the reference's matmul sources built with
+    -DESHKOL_GPU_ENABLED) resolves every eshkol_gpu_* symbol it calls from libeshkol_gpu_hip.so,
+    and without a reason to use the GPU it multiplies on its own CPU path."""
+    if not os.path.exists(oracle.REF_GPU_PATH):
+        pytest.skip("oracle/_ref/libeshkol_ref_gpu.so not built (no reference tree)")
+    from test_gpu_reference_caller import run_child
+    body = r"""
+n = 96
+A, B = synth.normal(6, (n, n)), synth.normal(7, (n, n))
+assert np.array_equal(fwd(caller, A, B), fwd(cpu, A, B))
+gA, gB = bwd(caller, A, A, B); wA, wB = bwd(cpu, A, A, B)
+assert np.array_equal(gA, wA) and np.array_equal(gB, wB)
+"""
+    r = run_child(body, {"ESHKOL_GPU_VERBOSE": "1"})
+    assert "[GPU] matmul" not in r.stderr

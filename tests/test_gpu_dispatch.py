@@ -634,14 +634,18 @@ assert np.array_equal(first[0], oracle.matmul_ozaki_crt(A, B))
 held = base - free_bytes()
 lib.eshkol_gpu_shutdown()
 assert lib.eshkol_gpu_get_backend() == ea.GPU_NONE
-released = held - (base - free_bytes())
+after_first = free_bytes()
+released = held - (base - after_first)
 print("HELD %d RELEASED %d" % (held, released))
-assert held > (16 << 20) and released >= held - (4 << 20)        # workspace and tables are gone
+# the workspace (64 MiB of planes and products at this size) and the tiers' tables are gone; what the HIP
+# runtime itself took on the first launches stays with it
+assert held > (48 << 20) and released >= held - (16 << 20)
 assert lib.eshkol_gpu_init() == 1
 again = all_tiers()
 for a, b in zip(first, again):
     assert np.array_equal(a, b)
 lib.eshkol_gpu_shutdown()
+assert after_first - free_bytes() <= (2 << 20)                   # a second cycle leaves nothing behind
 """
     run_child(body)
 
