@@ -228,6 +228,26 @@ def matmul_ozaki_crt(A, B, num_moduli=16, adaptive=False, aligned=False):
     return out if rc == 0 else None
 
 
+def matmul_ozaki_crt_refrep(A, B, mode, num_moduli=16, aligned=False):
+    """The exact tier with the reference's own choice of representative at the half-way
+    class of the modulus 256 (mode 1: its residue formula on the exact sum; mode 2: the
+    Metal kernel's partial reductions). Returns (C, n_half, n_plus)."""
+    A, B = _f64(A), _f64(B)
+    M, K = A.shape
+    N = B.shape[1]
+    out = np.empty((M, N))
+    half, plus = u64(0), u64(0)
+    L = lib()
+    L.oracle_ozaki_crt_use_aligned_weights(C.c_int(1 if aligned else 0))
+    try:
+        rc = L.oracle_matmul_ozaki_crt_refrep_f64(_d(A), _d(B), _d(out), u64(M), u64(K), u64(N),
+                                                  C.c_int(num_moduli), C.c_int(mode), C.byref(half), C.byref(plus))
+    finally:
+        L.oracle_ozaki_crt_use_aligned_weights(C.c_int(0))
+    assert rc == 0
+    return out, half.value, plus.value
+
+
 def mlp_layer(X, W, b, num_moduli=16):
     X, W = _f64(X), _f64(W)
     batch, in_f = X.shape

@@ -193,6 +193,21 @@ int oracle_matmul_ozaki_crt_f64(const double* A, const double* B, double* C,
                                 uint64_t M, uint64_t K, uint64_t N,
                                 int num_moduli, int adaptive);
 
+/* The same tier with the representatives the reference's floating-point residue
+ * formulas give (mode 1: gpu_memory.mm:2573-2583 applied to the exact sum; mode 2:
+ * the Metal kernel's partial reductions every 1008 k, metal_softfloat.h:3907-4100):
+ * the half-way class of the modulus 256 comes out as +128 or -128 there, always
+ * -128 above. n_half / n_plus count the elements in that class / those returned
+ * as +128. Test infrastructure for quantifying what the choice changes. */
+void oracle_ozaki_crt_products_refrep(const double* A, const double* B,
+                                      uint64_t M, uint64_t K, uint64_t N,
+                                      const int* mu, const int* nu, int num_moduli, int mode,
+                                      int16_t* w16);
+int oracle_matmul_ozaki_crt_refrep_f64(const double* A, const double* B, double* C,
+                                       uint64_t M, uint64_t K, uint64_t N,
+                                       int num_moduli, int mode,
+                                       uint64_t* n_half, uint64_t* n_plus);
+
 /* ---- MLP layer (BASELINE config 5) --------------------------------------- */
 
 /* y = tanh(x*W + b): matmul via the exact tier, then the broadcast add

@@ -305,6 +305,119 @@ int oracle_matmul_ozaki_crt_f64(const double* A, const double* B, double* C,
     return rc;
 }
 
+/* ---- the reference's own representatives ------------------------------------------
+ * The functions above take every residue by integer arithmetic in [-p/2, p/2), so
+ * the class 128 of the modulus 256 is always -128. The reference computes its
+ * residues in floating point, where the half-way case of the one even modulus
+ * comes out as +128 or -128 by the parity of the rounded quotient:
+ *   inputs  (gpu_memory.mm:2573-2583)       a_l = (float)(A' - p rint(A' (1/p))), in double
+ *   products (metal_softfloat.h:3907-4100)  float sums of 63 k-blocks of 16 (1008 k),
+ *            each reduced as v - p rint(v (1/p)) in float and added up, the total
+ *            reduced the same way once more.
+ * Modulo p nothing changes, so the exact product is the same; but the
+ * reference's weighted sum S1 is not exact (its weights end at different bits),
+ * and +128 instead of -128 moves that sum by 256 s_0 = P q_0, so its rounding
+ * errors fall differently. This restates the reference's choice operation for
+ * operation, to count on how many elements that matters.
+ *   mode 1: the input formula applied to the exact sum (what a host statement of
+ *           the modular product by the reference's own residue formula gives);
+ *   mode 2: the Metal kernel's order: reference representatives of the inputs,
+ *           partial reductions every 1008 k in float, final reduction in float.
+ * w16[l*M*N + i*N + j] in [-128, 128]. */
+static inline double ref_residue_f64(double x, int p) {
+    const double pd = (double)p, inv = 1.0 / pd;                  /* gpu_memory.mm:2576-2580 */
+    return x - pd * rint(x * inv);
+}
+static inline float ref_residue_f32(float v, float pf, float pinv) {
+    return v - pf * rintf(v * pinv);                              /* metal_softfloat.h:4063-4064 */
+}
+
+void oracle_ozaki_crt_products_refrep(const double* A, const double* B,
+                                      uint64_t M, uint64_t K, uint64_t N,
+                                      const int* mu, const int* nu, int num_moduli, int mode,
+                                      int16_t* w16) {
+    float* ar = (float*)malloc((size_t)M * K * sizeof(float));
+    float* br = (float*)malloc((size_t)N * K * sizeof(float));
+    for (int l = 0; l < num_moduli; l++) {
+        const int p = ORACLE_OZAKI_MODULI[l];
+        const float pf = (float)p, pinv = 1.0f / pf;
+        for (uint64_t i = 0; i < M; i++)
+            for (uint64_t k = 0; k < K; k++)
+                ar[i * K + k] = (float)ref_residue_f64(trunc(A[i * K + k] * ldexp(1.0, mu[i])), p);
+        for (uint64_t k = 0; k < K; k++)
+            for (uint64_t j = 0; j < N; j++)
+                br[j * K + k] = (float)ref_residue_f64(trunc(B[k * N + j] * ldexp(1.0, nu[j])), p);
+        #pragma omp parallel for schedule(static)
+        for (uint64_t i = 0; i < M; i++)
+            for (uint64_t j = 0; j < N; j++) {
+                const float* a = ar + i * K;
+                const float* b = br + j * K;
+                float w;
+                if (mode == 2) {
+                    float partial = 0.0f;
+                    for (uint64_t k0 = 0; k0 < K; k0 += 1008) {
+                        const uint64_t k1 = (k0 + 1008 < K) ? k0 + 1008 : K;
+                        int32_t v = 0;                            /* |v| <= 1008 * 128^2 < 2^24: exact in float too */
+                        for (uint64_t k = k0; k < k1; k++) v += (int32_t)a[k] * (int32_t)b[k];
+                        partial += ref_residue_f32((float)v, pf, pinv);
+                    }
+                    w = ref_residue_f32(partial, pf, pinv);
+                } else {
+                    int64_t v = 0;
+                    for (uint64_t k = 0; k < K; k++) v += (int64_t)a[k] * (int64_t)b[k];
+                    w = (float)ref_residue_f64((double)v, p);
+                }
+                w16[(uint64_t)l * M * N + i * N + j] = (int16_t)w;
+            }
+    }
+    free(ar); free(br);
+}
+
+/* The exact tier with the reference's representatives (mode as above); the
+ * accumulation is oracle_ozaki_crt_reconstruct's, operation for operation, on
+ * residues that may be +128. Also counts the elements whose residue modulo 256
+ * is the half-way class (n_half) and those among them that came out as +128
+ * (n_plus): only these can differ from oracle_matmul_ozaki_crt_f64. */
+int oracle_matmul_ozaki_crt_refrep_f64(const double* A, const double* B, double* C,
+                                       uint64_t M, uint64_t K, uint64_t N,
+                                       int num_moduli, int mode,
+                                       uint64_t* n_half, uint64_t* n_plus) {
+    if (!A || !B || !C || M == 0 || K == 0 || N == 0 || (mode != 1 && mode != 2)) return -1;
+    if (!all_finite(A, M * K) || !all_finite(B, K * N)) return -1;
+    if (num_moduli < 2) num_moduli = 2;
+    if (num_moduli > ORACLE_OZAKI_MAX_MODULI) num_moduli = ORACLE_OZAKI_MAX_MODULI;
+    OracleCRTConstants crt;
+    crt_constants(num_moduli, g_aligned_weights, &crt);
+    int* mu = (int*)malloc((size_t)M * sizeof(int));
+    int* nu = (int*)malloc((size_t)N * sizeof(int));
+    int16_t* w16 = (int16_t*)malloc((size_t)num_moduli * M * N * sizeof(int16_t));
+    oracle_ozaki_crt_scaling(A, B, M, K, N, &crt, mu, nu);
+    oracle_ozaki_crt_products_refrep(A, B, M, K, N, mu, nu, num_moduli, mode, w16);
+    const uint64_t tot = M * N;
+    uint64_t half = 0, plus = 0;
+    for (uint64_t i = 0; i < M; i++) {
+        const double mu_inv = ldexp(1.0, -mu[i]);
+        for (uint64_t j = 0; j < N; j++) {
+            const uint64_t idx = i * N + j;
+            if (w16[idx] == 128 || w16[idx] == -128) { half++; plus += w16[idx] == 128; }
+            double S1 = 0.0, S2 = 0.0;
+            for (int l = 0; l < crt.num_moduli; l++) {
+                const double w = (double)w16[(uint64_t)l * tot + idx];
+                S1 = fma(crt.sl1[l], w, S1);
+                S2 = fma(crt.sl2[l], w, S2);
+            }
+            const double s = S1 + S2;
+            const double Q = round(s * crt.Pinv);
+            const double c_prime = fma(-crt.P1, Q, S1) + fma(-crt.P2, Q, S2);
+            C[idx] = (c_prime * mu_inv) * ldexp(1.0, -nu[j]);
+        }
+    }
+    if (n_half) *n_half = half;
+    if (n_plus) *n_plus = plus;
+    free(mu); free(nu); free(w16);
+    return 0;
+}
+
 /* BASELINE config 5: one dense layer through the exact tier. The add is the
  * broadcast of b over rows (runtime_tensor_math.cpp:672-740), the activation is
  * std::tanh applied elementwise (lib/core/model_io.cpp:709). */

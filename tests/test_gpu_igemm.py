@@ -133,6 +133,27 @@ def test_slice_diagonal_sums(gpu, M, K, N, s, kernel):
     assert np.array_equal(got.astype(np.int64), exact(a, b, M, N, K, plan))
 
 
+@pytest.mark.parametrize("M,K,N", [(4096, 1024, 4096), (4096, 4096, 4096), (4096, 4096, 1024), (4096, 512, 4096)])
+def test_direct_kernel_on_the_mlp_shapes_and_the_shortest_tiles(gpu, M, K, N):
+    """The direct kernel's loads are issued from asm statements and waited for by count, so a
+    late operand would show as a wrong residue and nowhere else. The layer shapes of BASELINE
+    configuration 5 (16 planes, K = 1024 and 4096: 4096 or 1024 tiles on 256 CUs, the request
+    cursor crossing a tile boundary every 8 or 32 k-blocks) and the shortest tile there is
+    (K = 512: one ring of four k-blocks, so the cursor is in the next tile during every block):
+    all residues against the persistent kernel's, bit for bit, and sampled rows against exact
+    integer arithmetic."""
+    print("case: direct kernel %dx%dx%d, 16 planes" % (M, K, N), flush=True)
+    rng = np.random.default_rng(M + 3 * K + 7 * N)
+    a, b = planes(rng, 16, M, K), planes(rng, 16, N, K)
+    plan = [[(l, l)] for l in range(16)]
+    got = run(a, b, M, N, plan, 1, "direct")
+    assert np.array_equal(got, run(a, b, M, N, plan, 1, "persistent"))
+    rows = np.unique(np.concatenate([np.arange(0, M, 257), [63, 64, 255, 256, M - 1]]))
+    for l, p in enumerate(MODULI):
+        want = a[l][rows, :K].astype(np.float64) @ b[l][:N, :K].astype(np.float64).T
+        assert np.array_equal(got[l][rows].astype(np.int64), symmetric(want.astype(np.int64), p)), (l, p)
+
+
 def test_bad_arguments(gpu):
     lib = ea.load()
     g = ea.HipIgemmArgs()

@@ -214,3 +214,31 @@ def test_interleaved_contraction_config4_reduced_size(gpu):
             assert normwise(o[:64], ref, Ar[:64], Br) <= 1e-6
         if exact:
             assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0][:64], ref)
+
+
+def test_direct_kernel_batched_with_integer_operands(gpu):
+    """A batch through hip_hgemm_16_batched on interleaved operands (the direct kernel walks
+    all matrices' tiles in one persistent launch, the batch index as the operand plane) against
+    the row-major kernels on the same operands and against the exact integer product: small
+    integers are exact in bf16 and every fp32 sum of their products is exact, so all three
+    must agree bit for bit. K = 512 is the shortest tile the kernel has (one ring of four
+    k-blocks); 24 matrices of 4 x 4 tiles are more tiles than CUs."""
+    print("case: hip_hgemm_16_batched 24 x 1024x512x1024 integer operands", flush=True)
+    lib = ea.load()
+    batch, M, K, N = 24, 1024, 512, 1024
+    rng = np.random.default_rng(5)
+    A = rng.integers(-7, 8, (batch, M, K)).astype(np.float64)
+    B = rng.integers(-7, 8, (batch, K, N)).astype(np.float64)
+    dA, dB = ea.DeviceArray.from_host(A), ea.DeviceArray.from_host(B)
+    assert lib.hip_hgemm_plane_layout(M, N, batch) == 1
+    outs = []
+    for layout in (0, 1):
+        a16, b16 = ea.DeviceArray((batch, M, K), np.uint16), ea.DeviceArray((batch, N, K), np.uint16)
+        assert lib.hip_convert_f64_to_16_planes(dA.ptr, a16.ptr, batch, M, K, M, K, 1, 0, layout, stream()) == 0
+        assert lib.hip_convert_f64_to_16_planes(dB.ptr, b16.ptr, batch, N, K, N, K, 1, 1, layout, stream()) == 0
+        dC = ea.DeviceArray((batch, M, N), np.float32)
+        assert lib.hip_hgemm_16_batched(a16.ptr, b16.ptr, batch, M, K, N, M, N, K, 1, layout, dC.ptr, stream()) == 0
+        ea.synchronize()
+        outs.append(dC.download())
+    assert np.array_equal(outs[0], outs[1])
+    assert np.array_equal(outs[1].astype(np.float64), A @ B)

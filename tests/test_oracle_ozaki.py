@@ -364,3 +364,42 @@ def test_crt_exact_tier_guarantee_is_normwise_not_componentwise():
     num = sum((Fraction(float(Ca[i, j])) - exact[i][j]) ** 2 for i in range(4) for j in range(3))
     den = sum(Fraction(float(x)) ** 2 for x in A.ravel()) * sum(Fraction(float(x)) ** 2 for x in B.ravel())
     assert float(num) ** 0.5 / float(den) ** 0.5 < 1e-15
+
+
+@pytest.mark.parametrize("kind", ["normal", "wide"])
+def test_crt_half_way_class_of_modulus_256_reference_representative(kind):
+    """The one place where this oracle and the reference can return different bits for the
+    exact tier: when a product's residue modulo 256 is the half-way class, the oracle (and the
+    GPU) carry -128, the reference's floating-point residue formulas +128 or -128 by the parity
+    of a rounded quotient (gpu_memory.mm:2573-2583; metal_softfloat.h:3907-4100 with its partial
+    reductions every 1008 k). Modulo 256 that is the same number; the reference's weighted sum
+    is inexact, so the choice can move its rounding error. Counted here on N(0,1) and on
+    wide-range operands (BASELINE configuration 3's law), K = 2304 = three partial reductions:
+    about one element in 256 is in the class, about half of those come out as +128, and of
+    those a handful per 65536 elements change at all; the ones that do move by the
+    reference's own error quantum (far more than 2 ulp, far inside its 1e-9 gate). With
+    aligned weights the sum is exact and no element changes."""
+    M, K, N = 256, 2304, 256
+    if kind == "normal":
+        A, B = synth.normal(41, (M, K)), synth.normal(42, (K, N))
+    else:
+        A, B = synth.wide_range(43, (M, K), -30, 30), synth.wide_range(44, (K, N), -30, 30)
+    exact = A.astype(np.longdouble) @ B.astype(np.longdouble)
+    scale = np.abs(A).max(axis=1)[:, None] * np.abs(B).max(axis=0)[None, :] * K
+    for aligned in (False, True):
+        base = oracle.matmul_ozaki_crt(A, B, aligned=aligned)
+        for mode in (1, 2):
+            got, n_half, n_plus = oracle.matmul_ozaki_crt_refrep(A, B, mode, aligned=aligned)
+            changed = got != base
+            print(kind, "aligned" if aligned else "reference weights", "mode", mode, "half-way class", n_half,
+                  "as +128", n_plus, "elements that change", int(changed.sum()))
+            assert M * N / 400 < n_half < M * N / 170            # one element in 256
+            assert 0.35 * n_half < n_plus < 0.65 * n_half        # parity of a quotient: about half
+            if aligned:
+                assert not changed.any()
+            else:
+                assert changed.sum() <= 8                        # of 65536: at most about one in ten thousand
+                # where it changes, both values are the reference's arithmetic with its inexact sum:
+                # each within the reference's 1e-9 gate of the exact product, neither within 2 ulp of the other
+                for v in (got, base):
+                    assert float(np.max(np.abs(v[changed] - exact[changed]) / scale[changed], initial=0.0)) < 1e-9
