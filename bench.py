@@ -187,6 +187,11 @@ def main():
         rate = C.c_double()
         if probe.hip_probe_peak(kind, rnd, C.byref(rate), st) == 0:
             sustained[name] = rate.value / 1e12
+    t_m, t_v, t_b = C.c_double(), C.c_double(), C.c_double()
+    if probe.hip_probe_coissue(C.byref(t_m), C.byref(t_v), C.byref(t_b), st) == 0:
+        sustained["simd_shared_by_a_wave_of_mfma_and_a_wave_of_valu_ms"] = {
+            "mfma_alone": t_m.value, "valu_alone": t_v.value, "both": t_b.value,
+            "note": "both = max: side by side; both = sum: the SIMD runs one or the other"}
     log("device sustains (T/s):", json.dumps(sustained))
     fast = (M % 128 == 0 and N % 128 == 0 and K % 16 == 0)
     kernel = "dgemm_fast_kernel<NN>" if fast else "dgemm_mfma_kernel<128,128>"

@@ -59,7 +59,7 @@ COMMON = [
 # register the compiler spills while such a load is still in flight would be saved
 # before its data has arrived. They must therefore compile without any vector
 # spill; the compiler's resource remarks are checked after every build.
-NO_SPILL = {"igemm_i8.hip": ["igemm_i8_direct_kernel"], "hgemm_16.hip": ["hgemm_direct_kernel"]}
+NO_SPILL = {"igemm_i8.hip": ["igemm_i8_direct_kernel", "igemm_i8_direct_half_kernel"], "hgemm_16.hip": ["hgemm_direct_kernel"]}
 
 
 def _check_no_spill(src, remarks):

@@ -33,6 +33,7 @@
 #include "kernels.h"
 #include "gemm_pipe.h"
 #include "gemm_pipe2.h"
+#include "gemm_pipe3.h"
 
 typedef int v4i_t __attribute__((ext_vector_type(4)));
 typedef int v16i_t __attribute__((ext_vector_type(16)));
@@ -278,9 +279,11 @@ __device__ const ModulusTables MOD_TABLES = make_modulus_tables();
  * is private to a wave (no workgroup barrier): residues are packed four to a
  * word, parked in the wave's own 32 x 128-byte LDS stage and leave as 16-byte
  * stores, eight lanes to a 128-byte row segment. */
+template <int TN>
 __device__ __forceinline__ void epilogue_direct(const HipIgemmArgs& g, int o, int m0, int n0,
-                                                v16i_t (&acc)[pipe2::TM][pipe2::TN], int8_t* stage) {
-    constexpr int TM = pipe2::TM, TN = pipe2::TN;
+                                                v16i_t (&acc)[2][TN], int8_t* stage) {
+    constexpr int TM = 2, TILE_M = 256, TILE_N = 32 * TN;         /* the block tile: four waves of 64 rows */
+    static_assert(TN % 4 == 0, "whole 128-column halves");
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int li = lane & 31, lh = lane >> 5;
@@ -290,7 +293,7 @@ __device__ __forceinline__ void epilogue_direct(const HipIgemmArgs& g, int o, in
         const bool vec_ok = (g.N % 4 == 0);
         /* a tile inside the matrix: no bounds, no branches, one address per block (the same for every lane) */
         const bool interior0 = vec_ok && (((uintptr_t)out & 15) == 0) &&
-                               m0 + pipe2::BM <= (int)g.M && n0 + pipe2::BN <= (int)g.N;
+                               m0 + TILE_M <= (int)g.M && n0 + TILE_N <= (int)g.N;
 #pragma unroll
         for (int t = 0; t < TM; t++) {
             const int row = m0 + wave * 64 + t * 32 + li;
@@ -305,12 +308,17 @@ __device__ __forceinline__ void epilogue_direct(const HipIgemmArgs& g, int o, in
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 if (interior0) {
-                    v4i_t w[4];
-#pragma unroll
-                    for (int i = 0; i < 4; i++) w[i] = pipe2::parked_row16(stage, i);
+                    constexpr int AB = (TN >= 8) ? 4 : 2;        /* rows in flight: registers are short on the 128-column tile */
                     int32_t* p = out + (size_t)(row - li + (lane >> 3)) * g.N + (n0 + u * 32 + 4 * (lane & 7));
 #pragma unroll
-                    for (int i = 0; i < 4; i++) *(v4i_t*)(p + (size_t)(8 * i) * g.N) = w[i];
+                    for (int i0 = 0; i0 < 4; i0 += AB) {
+                        v4i_t w[AB];
+#pragma unroll
+                        for (int i = 0; i < AB; i++) w[i] = pipe2::parked_row16(stage, i0 + i);
+#pragma unroll
+                        for (int i = 0; i < AB; i++) *(v4i_t*)(p + (size_t)(8 * (i0 + i)) * g.N) = w[i];
+                        if (AB < 4) __builtin_amdgcn_sched_barrier(0);
+                    }
                 } else {
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
@@ -341,11 +349,11 @@ __device__ __forceinline__ void epilogue_direct(const HipIgemmArgs& g, int o, in
     constexpr int EP = pipe2::EPI_PITCH;
     int8_t* out = g.out_i8 + (size_t)o * g.M * g.N;
     const bool vec_ok = (g.N % 16 == 0) && (((uintptr_t)out & 15) == 0);
-    const bool interior = vec_ok && m0 + pipe2::BM <= (int)g.M && n0 + pipe2::BN <= (int)g.N;    /* the same for every lane */
+    const bool interior = vec_ok && m0 + TILE_M <= (int)g.M && n0 + TILE_N <= (int)g.N;    /* the same for every lane */
 #pragma unroll
     for (int t = 0; t < TM; t++) {
 #pragma unroll
-        for (int h = 0; h < 2; h++) {                     /* columns 128 h .. 128 h + 127 of the tile */
+        for (int h = 0; h < TN / 4; h++) {                /* columns 128 h .. 128 h + 127 of the tile */
 #pragma unroll
             for (int uu = 0; uu < 4; uu++) {
                 const int u = 4 * h + uu;
@@ -353,24 +361,26 @@ __device__ __forceinline__ void epilogue_direct(const HipIgemmArgs& g, int o, in
                 /* Eight elements abreast, one operation of the chain at a time: every
                  * instruction depends on the one eight back, not on its neighbour (a wave
                  * alone on its SIMD has nobody to fill the gaps a dependent chain leaves:
-                 * 9.3 -> 8.9 us per tile). */
+                 * 9.3 -> 8.9 us per tile). Four abreast where two waves share the SIMD and
+                 * registers are short (the 128-column tile). */
+                constexpr int VG = (TN >= 8) ? 2 : 1;             /* groups of four columns per pass */
 #pragma unroll
-                for (int vv = 0; vv < 4; vv += 2) {
-                    uint32_t a8[8];
-                    int x[8], r[8];
-                    float q[8];
+                for (int vv = 0; vv < 4; vv += VG) {
+                    uint32_t a8[4 * VG];
+                    int x[4 * VG], r[4 * VG];
+                    float q[4 * VG];
 #pragma unroll
-                    for (int e = 0; e < 8; e++) a8[e] = (uint32_t)acc[t][u][4 * vv + e] + lift;
+                    for (int e = 0; e < 4 * VG; e++) a8[e] = (uint32_t)acc[t][u][4 * vv + e] + lift;
 #pragma unroll
-                    for (int e = 0; e < 8; e++) x[e] = (int)__builtin_amdgcn_udot4(a8[e], wbytes, 0u, false);
+                    for (int e = 0; e < 4 * VG; e++) x[e] = (int)__builtin_amdgcn_udot4(a8[e], wbytes, 0u, false);
 #pragma unroll
-                    for (int e = 0; e < 8; e++) q[e] = (float)x[e];
+                    for (int e = 0; e < 4 * VG; e++) q[e] = (float)x[e];
 #pragma unroll
-                    for (int e = 0; e < 8; e++) q[e] = fmaf(q[e], pinv, 12582912.0f);
+                    for (int e = 0; e < 4 * VG; e++) q[e] = fmaf(q[e], pinv, 12582912.0f);
 #pragma unroll
-                    for (int e = 0; e < 8; e++) r[e] = __mul24(__float_as_int(q[e]), -p) + x[e];
+                    for (int e = 0; e < 4 * VG; e++) r[e] = __mul24(__float_as_int(q[e]), -p) + x[e];
 #pragma unroll
-                    for (int w = 0; w < 2; w++) {
+                    for (int w = 0; w < VG; w++) {
                         const uint32_t lo2 = __builtin_amdgcn_perm((uint32_t)r[4 * w + 1], (uint32_t)r[4 * w], 0x0c0c0400u);
                         const uint32_t hi2 = __builtin_amdgcn_perm((uint32_t)r[4 * w + 3], (uint32_t)r[4 * w + 2], 0x04000c0cu);
                         *(uint32_t*)(stage + li * EP + uu * 32 + 8 * (vv + w) + 4 * lh) = lo2 | hi2;
@@ -383,12 +393,18 @@ __device__ __forceinline__ void epilogue_direct(const HipIgemmArgs& g, int o, in
                 /* a tile inside the matrix: no bounds, no branches, one address per wave
                  * and row block (2.8 of this epilogue's 9 us per tile were the guarded
                  * stores below: a branch and a 64-bit product each) */
-                v4i_t val[4];
-#pragma unroll
-                for (int i = 0; i < 4; i++) val[i] = *(const v4i_t*)(stage + ((lane >> 3) + 8 * i) * EP + (lane & 7) * 16);
+                constexpr int AB = (TN >= 8) ? 4 : 2;            /* rows in flight, as above */
                 int8_t* dst = out + (size_t)(m0 + wave * 64 + t * 32 + (lane >> 3)) * g.N + (n0 + 128 * h + 16 * (lane & 7));
 #pragma unroll
-                for (int i = 0; i < 4; i++) *(v4i_t*)(dst + (size_t)(8 * i) * g.N) = val[i];
+                for (int i0 = 0; i0 < 4; i0 += AB) {
+                    v4i_t val[AB];
+#pragma unroll
+                    for (int i = 0; i < AB; i++)
+                        val[i] = *(const v4i_t*)(stage + ((lane >> 3) + 8 * (i0 + i)) * EP + (lane & 7) * 16);
+#pragma unroll
+                    for (int i = 0; i < AB; i++) *(v4i_t*)(dst + (size_t)(8 * (i0 + i)) * g.N) = val[i];
+                    if (AB < 4) __builtin_amdgcn_sched_barrier(0);
+                }
                 continue;
             }
 #pragma unroll
@@ -437,9 +453,41 @@ void igemm_i8_direct_kernel(HipIgemmArgs g, int tiles_m, int tiles_n, int chunk,
         return false;
     };
     auto epi = [&](v16i_t (&acc)[pipe2::TM][pipe2::TN], const pipe::Tile& t, int8_t* stage) {
-        epilogue_direct(g, t.tag, t.m0, t.n0, acc, stage);
+        epilogue_direct<pipe2::TN>(g, t.tag, t.m0, t.n0, acc, stage);
     };
     pipe2::run_tiles<I8Op>(smem_i8, cm, next_tile, epi);
+}
+
+/* The same on 256 x 128 tiles with 128 accumulators per wave, two workgroups per
+ * CU (gemm_pipe3.h): a second wave on every SIMD fills the first one's waits. For
+ * contractions whose K is short enough for the time between tiles to matter. */
+__global__ __launch_bounds__(256, 2)
+void igemm_i8_direct_half_kernel(HipIgemmArgs g, int tiles_m, int tiles_n, int chunk, int n_ids) {
+    extern __shared__ __align__(16) int8_t smem_i8[];
+    pipe::Source cm;
+    cm.a_planes = g.a_planes; cm.b_planes = g.b_planes;
+    cm.a_plane_stride = g.a_plane_stride; cm.b_plane_stride = g.b_plane_stride;
+    cm.ld = (int)g.ldk;
+
+    int next_id = (int)blockIdx.x;
+    auto next_tile = [&](pipe::Tile& t) -> bool {
+        while (next_id < n_ids) {
+            int o, tm, tn;
+            const bool real = map_workgroup(next_id, tiles_m, tiles_n, (int)g.n_out, chunk, &o, &tm, &tn);
+            next_id += (int)gridDim.x;
+            if (!real) continue;
+            const int pair_lo = pipe2::scalar_load(g.pair_first + o);
+            t.m0 = tm * pipe3::BM; t.n0 = tn * pipe3::BN; t.tag = o;
+            t.a_idx = g.pair_a + pair_lo; t.b_idx = g.pair_b + pair_lo;
+            t.npairs = pipe2::scalar_load(g.pair_first + o + 1) - pair_lo;
+            if (t.npairs > 0) return true;
+        }
+        return false;
+    };
+    auto epi = [&](v16i_t (&acc)[pipe3::TM][pipe3::TN], const pipe::Tile& t, int8_t* stage) {
+        epilogue_direct<pipe3::TN>(g, t.tag, t.m0, t.n0, acc, stage);
+    };
+    pipe3::run_tiles<I8Op>(smem_i8, cm, next_tile, epi);
 }
 
 /* ---- simple kernel --------------------------------------------------------- */
@@ -620,6 +668,28 @@ int launch_direct(const HipIgemmArgs& a, hipStream_t st) {
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 
+int launch_direct_half(const HipIgemmArgs& a, hipStream_t st) {
+    constexpr int SMEM = pipe3::SMEM_BYTES;
+    static bool attr_set = false;
+    static int num_cus = 0;
+    auto kern = igemm_i8_direct_half_kernel;
+    if (!attr_set) {
+        if (!ESHKOL_HIP_OK(hipFuncSetAttribute((const void*)kern,
+                hipFuncAttributeMaxDynamicSharedMemorySize, SMEM))) return -1;
+        num_cus = eshkol_hip_num_cus();
+        attr_set = true;
+    }
+    const int tiles_m = (int)((a.M + pipe3::BM - 1) / pipe3::BM), tiles_n = (int)((a.N + pipe3::BN - 1) / pipe3::BN);
+    const int chunk = (tiles_m * tiles_n + 7) / 8;
+    const long long n_ids = 8LL * chunk * a.n_out;
+    if (n_ids > 0x7fffffffLL || n_ids <= 0) return -1;
+    long long grid = 2LL * ((num_cus / 8) * 8);     /* two workgroups per CU, a multiple of the XCD count */
+    if (grid < 8) grid = 8;
+    if (grid > n_ids) grid = n_ids;
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), SMEM, st, a, tiles_m, tiles_n, chunk, (int)n_ids);
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
 int launch_simple(const HipIgemmArgs& a, hipStream_t st) {
     constexpr int BM = 128, BN = 128;
     constexpr int MAIN = 2 * (BM + BN) * SPITCH, EPI = BM * (BN + 16);
@@ -638,14 +708,14 @@ extern "C" void hip_igemm_set_persistent(int on) { EshkolHipLock lk; g_persisten
 
 /* Tuning hook: 0 keeps every launch on row-major planes and the register-staged
  * kernels. Same results. */
-extern "C" void hip_igemm_set_direct(int on) { EshkolHipLock lk; g_direct = on ? 1 : 0; }
+extern "C" void hip_igemm_set_direct(int on) { EshkolHipLock lk; g_direct = (on >= 0 && on <= 3) ? on : 1; }
 
 /* The plane layout the tiers should produce for a contraction of n_out output
  * planes of M x N: 1 (interleaved, for the direct-to-LDS kernel) when the launch
  * has enough 256 x 256 tiles to be worth a workgroup per CU, else 0. */
 extern "C" int hip_igemm_plane_layout(uint64_t M, uint64_t N, int n_out) {
     const uint64_t big = ((M + 255) / 256) * ((N + 255) / 256) * (uint64_t)(n_out > 0 ? n_out : 0);
-    return (g_direct && big >= 128) ? 1 : 0;
+    return (g_direct != 0 && big >= 128) ? 1 : 0;
 }
 
 extern "C" int hip_igemm_i8(const HipIgemmArgs* args, void* stream) {
@@ -666,7 +736,11 @@ extern "C" int hip_igemm_i8(const HipIgemmArgs* args, void* stream) {
          * every output plane with 1..64 products, row counts padded to 256 */
         if (a.ldk % 512 != 0 || a.max_pairs < 1) return -1;
         if ((a.a_plane_stride % (32ull * a.ldk)) || (a.b_plane_stride % (32ull * a.ldk))) return -1;
-        return launch_direct(a, st);
+        /* Products of at most 1024 bytes of k per row take the 256 x 128 kernel with
+         * two workgroups per CU (measured 5 ... 13 % faster there, slower from 2048 on);
+         * row counts of B padded to 256 cover its tiles too. g_direct 2 / 3: always / never. */
+        const bool half = g_direct == 2 || (g_direct == 1 && a.ldk <= 1024 && a.max_pairs == 1);
+        return half ? launch_direct_half(a, st) : launch_direct(a, st);
     }
     if (a.layout != 0) return -1;
     /* Operand planes are padded to multiples of 256 rows, so either tiling reads

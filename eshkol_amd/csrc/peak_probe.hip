@@ -116,7 +116,88 @@ void probe_copy(const v4i_t* __restrict__ src, v4i_t* __restrict__ dst, size_t n
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
 }
 
+/* Do a wave's vector ALU instructions run while another wave's MFMAs occupy the
+ * same SIMD? 512 threads = eight waves per workgroup, one workgroup per CU, two
+ * waves on every SIMD: waves 0-3 issue int8 MFMAs back to back, waves 4-7 the
+ * instruction mix of a residue epilogue (add, byte dot product, convert, fma,
+ * 24-bit multiply-add). Either half can be switched off with a count of 0. */
+__global__ __launch_bounds__(512, 1)
+void probe_coissue(int mfma_iters, int valu_iters, int* sink) {
+    const int wave = threadIdx.x >> 6;
+    if (wave < 4) {
+        v16i_t acc[4];
+        v4i_t a, b;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][r] = 0;
+#pragma unroll
+        for (int r = 0; r < 4; r++) { a[r] = 0x01010101 * (int)(threadIdx.x & 3); b[r] = 0x02020202; }
+        for (int it = 0; it < mfma_iters; it++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc[i], 0, 0, 0);
+        }
+        int s = 0;
+        for (int i = 0; i < 4; i++) for (int r = 0; r < 16; r++) s += acc[i][r];
+        if (s == 0x12345678) sink[0] = s;
+    } else {
+        unsigned x[8];
+        float q[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) x[e] = mix(threadIdx.x * 8 + e);
+        const unsigned wb = 0x01100401u;
+        const int p = 251;
+        const float pinv = 1.0f / 251.0f;
+        for (int it = 0; it < valu_iters; it++) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) x[e] = x[e] + 0x80000000u + (unsigned)it;
+#pragma unroll
+            for (int e = 0; e < 8; e++) x[e] = __builtin_amdgcn_udot4(x[e], wb, x[e] >> 24, false);
+#pragma unroll
+            for (int e = 0; e < 8; e++) q[e] = fmaf((float)(int)x[e], pinv, 12582912.0f);
+#pragma unroll
+            for (int e = 0; e < 8; e++) x[e] = (unsigned)(__mul24(__float_as_int(q[e]), -p) + (int)x[e]) ^ (x[e] << 13);
+        }
+        unsigned s = 0;
+        for (int e = 0; e < 8; e++) s += x[e];
+        if (s == 0x12345678u) sink[1] = (int)s;
+    }
+}
+
 }  // namespace
+
+/* Times (ms) of the MFMA waves alone, the vector ALU waves alone, and both together,
+ * each wave's work the same in all three. both = max of the two would mean the SIMD
+ * runs them side by side; both = their sum means it runs one or the other. */
+extern "C" int hip_probe_coissue(double* mfma_ms, double* valu_ms, double* both_ms, void* stream) {
+    if (!mfma_ms || !valu_ms || !both_ms) return -1;
+    hipStream_t st = (hipStream_t)stream;
+    int* sink = nullptr;
+    hipEvent_t e0, e1;
+    if (!ESHKOL_HIP_OK(hipMalloc((void**)&sink, 256))) return -1;
+    if (!ESHKOL_HIP_OK(hipEventCreate(&e0)) || !ESHKOL_HIP_OK(hipEventCreate(&e1))) { (void)hipFree(sink); return -1; }
+    const int M = 20000, V = 6000;
+    const int counts[3][2] = {{M, 0}, {0, V}, {M, V}};
+    double out[3] = {0.0, 0.0, 0.0};
+    int rc = 0;
+    for (int c = 0; c < 3 && rc == 0; c++) {
+        float best = 1e30f;
+        for (int rep = 0; rep < 3; rep++) {
+            (void)hipEventRecord(e0, st);
+            hipLaunchKernelGGL(probe_coissue, dim3(256), dim3(512), 0, st, counts[c][0], counts[c][1], sink);
+            (void)hipEventRecord(e1, st);
+            float ms = 0.0f;
+            if (!ESHKOL_HIP_OK(hipEventSynchronize(e1)) || !ESHKOL_HIP_OK(hipEventElapsedTime(&ms, e0, e1))) { rc = -1; break; }
+            if (rep > 0 && ms < best) best = ms;
+        }
+        out[c] = best;
+    }
+    *mfma_ms = out[0]; *valu_ms = out[1]; *both_ms = out[2];
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipFree(sink);
+    return rc;
+}
 
 /* kind 0: fp64 MFMA flop/s, 1: int8 MFMA op/s, 2: bf16 MFMA flop/s, 3: HBM copy
  * bytes/s (read + written). random_operands selects random operand bits for the

@@ -95,9 +95,12 @@ void hip_dgemm_set_prefetch_depth(int depth);
 void hip_igemm_set_prefetch(int pf);
 
 /* 1 (default): contractions with at least 128 tiles take interleaved operand
- * planes and the kernel that loads them straight into LDS and MFMA registers;
- * 0: row-major planes and the register-staged kernels everywhere. Same results;
- * the switch exists to compare them. */
+ * planes and the kernels that load them straight into LDS and MFMA registers
+ * (256 x 128 tiles and two workgroups per CU for products of at most 1024 bytes
+ * of k, 256 x 256 tiles and one otherwise); 2: the 256 x 128 kernel for all of
+ * them; 3: the 256 x 256 kernel for all of them; 0: row-major planes and the
+ * register-staged kernels everywhere. Same results; the switch exists to
+ * compare them. */
 void hip_igemm_set_direct(int on);
 
 /* The same switch for the 16-bit tier. */
@@ -125,6 +128,14 @@ void hip_ozaki_crt_set_host_pass(int on);
  * than seeded. Synchronises the stream; allocates and frees
  * its own buffers. */
 int hip_probe_peak(int kind, int random_operands, double* rate, void* stream);
+
+/* Whether a SIMD runs one wave's vector ALU instructions beside another wave's
+ * MFMAs: the time (ms) of four waves of back-to-back int8 MFMAs per CU, of four
+ * waves of a residue epilogue's instruction mix per CU, and of both sharing the
+ * SIMDs two waves each. both = the larger of the two: side by side; both = their
+ * sum: one or the other. What the choice of one or two workgroups per CU for the
+ * int8 contraction rests on. */
+int hip_probe_coissue(double* mfma_ms, double* valu_ms, double* both_ms, void* stream);
 
 #ifdef __cplusplus
 }

@@ -39,7 +39,7 @@ def test_library_exports_every_declared_symbol():
     assert not [n for n in declared if "_last_stages" in n or n.startswith("hip_probe_")]
     assert [n for n in declared if "_set_" in n] == ["eshkol_gpu_set_threshold", "hip_ozaki_crt_set_aligned_weights"]
     assert not hasattr(lib, "hip_probe_peak")
-    assert hasattr(ea.load_probe(), "hip_probe_peak")
+    assert hasattr(ea.load_probe(), "hip_probe_peak") and hasattr(ea.load_probe(), "hip_probe_coissue")
     assert C.c_size_t.in_dll(lib, "g_gpu_threshold").value in (100000, int(os.environ.get("ESHKOL_GPU_THRESHOLD", 100000)))
 
 

@@ -15,7 +15,9 @@ pytestmark = pytest.mark.gpu
 
 MODULI = [256, 255, 253, 251, 247, 241, 239, 233, 229, 227, 223, 217, 211, 199, 197, 193]
 KERNELS = {"simple": (0, 0), "pipelined": (2, 0), "persistent": (2, 1), "pipelined-1": (1, 0), "persistent-1": (1, 1),
-           "direct": (2, 1)}           # interleaved planes, operands loaded straight into LDS / MFMA registers
+           "direct": (2, 1),           # interleaved planes, operands loaded straight into LDS / MFMA registers
+           "direct-half": (2, 1)}      # the same on 256 x 128 tiles, two workgroups per CU
+DIRECT_MODE = {"direct": 3, "direct-half": 2}
 
 
 def pad(n, m):
@@ -44,7 +46,7 @@ def run(a, b, M, N, plan, mode, kernel):
     """plan: list of lists of (a_plane, b_plane) per output plane."""
     lib = ea.load()
     pf, pers = KERNELS[kernel]
-    if kernel == "direct":
+    if kernel in DIRECT_MODE:
         a, b = interleave(a), interleave(b)
     first = np.cumsum([0] + [len(p) for p in plan]).astype(np.int32)
     pa = np.array([t[0] for p in plan for t in p], np.int32)
@@ -60,19 +62,21 @@ def run(a, b, M, N, plan, mode, kernel):
     g.ldk, g.M, g.N, g.n_out = a.shape[2], M, N, n_out
     g.pair_first, g.pair_a, g.pair_b = dF.ptr, dPa.ptr, dPb.ptr
     g.mode, g.max_pairs, g.modulus = mode, max(len(p) for p in plan), dMod.ptr
-    g.layout = 1 if kernel == "direct" else 0
+    g.layout = 1 if kernel in DIRECT_MODE else 0
     if mode == 1:
         g.out_i8 = out.ptr
     else:
         g.out_i32 = out.ptr
     lib.hip_igemm_set_prefetch(pf)
     lib.hip_igemm_set_persistent(pers)
+    lib.hip_igemm_set_direct(DIRECT_MODE.get(kernel, 1))
     try:
         assert lib.hip_igemm_i8(C.byref(g), stream()) == 0
         ea.synchronize()
     finally:
         lib.hip_igemm_set_prefetch(2)
         lib.hip_igemm_set_persistent(1)
+        lib.hip_igemm_set_direct(1)
     return out.download()
 
 
@@ -148,6 +152,7 @@ def test_direct_kernel_on_the_mlp_shapes_and_the_shortest_tiles(gpu, M, K, N):
     plan = [[(l, l)] for l in range(16)]
     got = run(a, b, M, N, plan, 1, "direct")
     assert np.array_equal(got, run(a, b, M, N, plan, 1, "persistent"))
+    assert np.array_equal(got, run(a, b, M, N, plan, 1, "direct-half"))
     rows = np.unique(np.concatenate([np.arange(0, M, 257), [63, 64, 255, 256, M - 1]]))
     for l, p in enumerate(MODULI):
         want = a[l][rows, :K].astype(np.float64) @ b[l][:N, :K].astype(np.float64).T
