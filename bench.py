@@ -30,7 +30,7 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-PEAK = {"fp64_mfma": 78.6e12, "int8_mfma": 5.0e15, "bf16_mfma": 2.5e15, "hbm": 8.0e12}
+PEAK = {"fp64_mfma": 78.6e12, "fp32_mfma": 157.3e12, "int8_mfma": 5.0e15, "bf16_mfma": 2.5e15, "hbm": 8.0e12}
 
 
 def log(*a):
@@ -88,7 +88,7 @@ def main():
     flops = 2.0 * M * N * K
     steps, warm = args.steps, args.warmup
     timer = ea.Timer()
-    want = set(args.only.split(",")) if args.only else {"crt", "int8", "reduced", "mlp", "backward", "host", "sizes", "c1"}
+    want = set(args.only.split(",")) if args.only else {"crt", "int8", "reduced", "mlp", "backward", "host", "sizes", "c1", "f32"}
 
     if args.pmc_probe:
         # Short program for `rocprofv3 --pmc ...` runs: a 512 MiB device copy of known size
@@ -211,6 +211,24 @@ def main():
     tiers["native_fp64_%dx%dx%d" % (M, N2, K)] = {"ms": w2, "gflops": 2.0 * M * N2 * K / (w2 * 1e-3) / 1e9,
                                                    "frac_of_peak": 2.0 * M * N2 * K / (e2 * 1e-3) / PEAK["fp64_mfma"]}
     dB2.free(); dC2.free()
+
+    # ---- single precision entry (eshkol_gpu_matmul_f32) on the fp32 matrix cores ------
+    if "f32" in want:
+        A32, B32 = A.astype(np.float32), B.astype(np.float32)
+        dA32, dB32 = ea.DeviceArray.from_host(A32), ea.DeviceArray.from_host(B32)
+        dC32f = ea.DeviceArray((M, N), np.float32)
+        ef, wf32 = timed(lambda: lib.hip_sgemm_f32(dA32.ptr, dB32.ptr, dC32f.ptr, M, K, N, st), settle_ms=40.0)
+        rows32 = list(range(0, M, max(M // 4, 1)))[:4]
+        got32 = dC32f.download()[rows32].astype(np.float64)
+        ref32 = A32[rows32].astype(np.float64) @ B32.astype(np.float64)
+        err32 = float(np.linalg.norm(got32 - ref32) / (np.linalg.norm(A32[rows32].astype(np.float64)) * np.linalg.norm(B32.astype(np.float64))))
+        tiers["native_fp32_matrix_cores"] = {"ms": wf32, "gflops": flops / (wf32 * 1e-3) / 1e9,
+                                             "frac_of_fp32_peak": flops / (ef * 1e-3) / PEAK["fp32_mfma"],
+                                             "peak": "fp32 MFMA 157.3 TFLOP/s", "normwise_error_sampled_rows": err32}
+        log("native fp32: %.3f ms %.1f GFLOP/s" % (wf32, flops / (wf32 * 1e-3) / 1e9))
+        for d in (dA32, dB32, dC32f):
+            d.free()
+        del A32, B32
 
     # ---- Ozaki-II CRT exact tier: configuration 3 --------------------------------
     if "crt" in want:

@@ -149,6 +149,7 @@ SIGNATURES = {
     "hip_ozaki_fast_split_planes_f64": (C.c_int, [vp, u64, u64, vp, C.c_int, vp, u64, u64, C.c_int, C.c_int, vp]),
     "hip_ozaki_fast_reconstruct_f64": (C.c_int, [vp, u64, u64, u64, C.c_int, vp, vp, vp, vp]),
     "hip_igemm_set_direct": (None, [C.c_int]),
+    "hip_igemm_set_cu_limit": (None, [C.c_int]),
     "hip_hgemm_set_direct": (None, [C.c_int]),
     "hip_hgemm_plane_layout": (C.c_int, [u64, u64, u64]),
     "hip_hgemm_16_batched": (C.c_int, [vp, vp, u64, u64, u64, u64, u64, u64, u64, C.c_int, C.c_int, vp, vp]),

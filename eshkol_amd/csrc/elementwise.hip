@@ -1,7 +1,6 @@
 /*
  * Streaming (HBM-bound) kernels shared by the tiers: transpose, per-row
- * absolute maximum, the elementwise family, the dense-layer epilogue, and the
- * single-precision GEMM of eshkol_gpu_matmul_f32.
+ * absolute maximum, the elementwise family and the dense-layer epilogue.
  */
 #include "hip_common.h"
 #include <hip/hip_ext.h>
@@ -177,47 +176,6 @@ void bias_act_f64_kernel(double* __restrict__ Y, const double* __restrict__ bias
     }
 }
 
-/* Plain LDS-tiled fp32 GEMM (64x64 tile, 4x4 outputs per thread). This entry
- * has no caller on the language side; it is kept correct, not tuned. */
-__global__ __launch_bounds__(256)
-void sgemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C,
-                      int M, int N, int K) {
-    __shared__ float As[16][64 + 1];
-    __shared__ float Bs[16][64 + 1];
-    const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
-    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
-    float acc[4][4] = {};
-    for (int k0 = 0; k0 < K; k0 += 16) {
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const int idx = threadIdx.x + 256 * r;
-            const int am = idx >> 4, ak = idx & 15;
-            As[ak][am] = (m0 + am < M && k0 + ak < K) ? A[(size_t)(m0 + am) * K + k0 + ak] : 0.0f;
-            const int bk = idx >> 6, bn = idx & 63;
-            Bs[bk][bn] = (k0 + bk < K && n0 + bn < N) ? B[(size_t)(k0 + bk) * N + n0 + bn] : 0.0f;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int k = 0; k < 16; k++) {
-            float a[4], b[4];
-#pragma unroll
-            for (int i = 0; i < 4; i++) { a[i] = As[k][ty * 4 + i]; b[i] = Bs[k][tx * 4 + i]; }
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-                for (int j = 0; j < 4; j++) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
-        }
-        __syncthreads();
-    }
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int r = m0 + ty * 4 + i, c = n0 + tx * 4 + j;
-            if (r < M && c < N) C[(size_t)r * N + c] = acc[i][j];
-        }
-}
-
 inline unsigned grid_1d(uint64_t n, unsigned block, unsigned cap) {
     uint64_t g = (n + block - 1) / block;
     if (g > cap) g = cap;
@@ -291,13 +249,3 @@ extern "C" int hip_bias_act_f64(double* Y, const double* bias, uint64_t rows, ui
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 
-extern "C" int hip_sgemm_f32(const float* A, const float* B, float* C,
-                             uint64_t M, uint64_t K, uint64_t N, void* stream) {
-    if (!A || !B || !C || M == 0 || K == 0 || N == 0) return -1;
-    if (M > 0x7fffffffULL || K > 0x7fffffffULL || N > 0x7fffffffULL) return -1;
-    const uint64_t gx = (N + 63) / 64, gy = (M + 63) / 64;
-    if (gy > 65535) return -1;
-    hipLaunchKernelGGL(sgemm_f32_kernel, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0,
-                       (hipStream_t)stream, A, B, C, (int)M, (int)N, (int)K);
-    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
-}

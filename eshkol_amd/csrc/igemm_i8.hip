@@ -643,6 +643,8 @@ int launch_persistent(const HipIgemmArgs& a, hipStream_t st) {
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 
+int g_cu_limit = 0;      /* > 0: the persistent 256 x 256 kernel leaves the other CUs to whatever else runs */
+
 int launch_direct(const HipIgemmArgs& a, hipStream_t st) {
     constexpr int SMEM = pipe2::SMEM_BYTES;
     static bool attr_set = false;
@@ -662,6 +664,7 @@ int launch_direct(const HipIgemmArgs& a, hipStream_t st) {
     const long long n_ids = 8LL * chunk * a.n_out;
     if (n_ids > 0x7fffffffLL || n_ids <= 0) return -1;
     long long grid = (num_cus / 8) * 8;             /* one workgroup per CU, a multiple of the XCD count */
+    if (g_cu_limit > 0 && grid > g_cu_limit) grid = (g_cu_limit / 8) * 8;
     if (grid < 8) grid = 8;
     if (grid > n_ids) grid = n_ids;
     hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), SMEM, st, a, tiles_m, tiles_n, chunk, (int)n_ids);
@@ -709,6 +712,8 @@ extern "C" void hip_igemm_set_persistent(int on) { EshkolHipLock lk; g_persisten
 /* Tuning hook: 0 keeps every launch on row-major planes and the register-staged
  * kernels. Same results. */
 extern "C" void hip_igemm_set_direct(int on) { EshkolHipLock lk; g_direct = (on >= 0 && on <= 3) ? on : 1; }
+
+extern "C" void hip_igemm_set_cu_limit(int cus) { EshkolHipLock lk; g_cu_limit = cus > 0 ? cus : 0; }
 
 /* The plane layout the tiers should produce for a contraction of n_out output
  * planes of M x N: 1 (interleaved, for the direct-to-LDS kernel) when the launch

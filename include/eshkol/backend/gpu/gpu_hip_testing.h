@@ -103,6 +103,12 @@ void hip_igemm_set_prefetch(int pf);
  * compare them. */
 void hip_igemm_set_direct(int on);
 
+/* Workgroups of the persistent 256 x 256 int8 kernel: 0 (default) one per CU;
+ * n > 0 at most n (rounded down to a multiple of 8), which leaves the other CUs
+ * to kernels queued on other streams. For measuring what running the streaming
+ * stages beside the contraction would cost and gain. */
+void hip_igemm_set_cu_limit(int cus);
+
 /* The same switch for the 16-bit tier. */
 void hip_hgemm_set_direct(int on);
 
