@@ -71,7 +71,7 @@ def main():
     ap.add_argument("--no-stages", action="store_true")
     ap.add_argument("--only", default="", help="comma list of what to time besides native: crt,int8,reduced,mlp,backward,host,sizes,c1")
     ap.add_argument("--no-accuracy", action="store_true", help="skip the extended-precision check of sampled rows")
-    ap.add_argument("--pmc-probe", default="", choices=["", "dgemm", "crt", "fast", "int8", "reduced"],
+    ap.add_argument("--pmc-probe", default="", choices=["", "dgemm", "crt", "fast", "int8", "reduced", "crt-layer1", "sgemm"],
                     help="run a calibration copy and three launches of one tier, for rocprofv3 --pmc")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -93,6 +93,8 @@ def main():
     if args.pmc_probe:
         # Short program for `rocprofv3 --pmc ...` runs: a 512 MiB device copy of known size
         # (calibrates FETCH_SIZE / WRITE_SIZE), then three launches of one tier. No timing.
+        if args.pmc_probe == "crt-layer1":           # first layer of configuration 5: 4096 x 1024 x 4096
+            M, K, N = 4096, 1024, 4096
         src, dst, out = ea.DeviceArray((M, K)), ea.DeviceArray((K, N)), ea.DeviceArray((M, N))
         src.upload(synth.normal(11, (M, K)))
         hip.hipMemcpy(dst.ptr, src.ptr, min(src.nbytes, 512 << 20), ea.D2D)
@@ -100,13 +102,15 @@ def main():
         dst.upload(synth.normal(12, (K, N)))
         calls = {"dgemm": lambda: lib.hip_dgemm_f64(src.ptr, dst.ptr, out.ptr, M, K, N, st),
                  "crt": lambda: lib.hip_matmul_ozaki_crt_f64(src.ptr, dst.ptr, out.ptr, M, K, N, 16, 0, None, 0, st),
+                 "crt-layer1": lambda: lib.hip_matmul_ozaki_crt_f64(src.ptr, dst.ptr, out.ptr, M, K, N, 16, 0, None, 0, st),
+                 "sgemm": lambda: lib.hip_sgemm_f32(src.ptr, dst.ptr, out.ptr, M, K, N, st),
                  "fast": lambda: lib.hip_matmul_ozaki_fast_f64(src.ptr, dst.ptr, out.ptr, M, K, N, 11, st),
                  "int8": lambda: lib.hip_matmul_ozaki_int8_f64(src.ptr, dst.ptr, out.ptr, M, K, N, 6, st),
                  "reduced": lambda: lib.hip_matmul_reduced_f64(src.ptr, dst.ptr, out.ptr, M, K, N, 3, 0, st)}
         for _ in range(3):
             assert calls[args.pmc_probe]() == 0
         hip.hipDeviceSynchronize()
-        print(json.dumps({"pmc_probe": args.pmc_probe, "size": n}))
+        print(json.dumps({"pmc_probe": args.pmc_probe, "shape": [M, K, N]}))
         return
 
     def timed(fn, k=steps, w=warm, settle_ms=0.0):
