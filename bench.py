@@ -70,6 +70,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-stages", action="store_true")
     ap.add_argument("--only", default="", help="comma list of what to time besides native: crt,int8,reduced,mlp,backward,host,sizes,c1")
+    ap.add_argument("--igemm-direct", type=int, default=-1,
+                    help="hip_igemm_set_direct() for this run (1 default choice by K, 2 the 256x128 kernel, 3 the 256x256 kernel)")
     ap.add_argument("--no-accuracy", action="store_true", help="skip the extended-precision check of sampled rows")
     ap.add_argument("--pmc-probe", default="", choices=["", "dgemm", "crt", "fast", "int8", "reduced", "crt-layer1", "sgemm"],
                     help="run a calibration copy and three launches of one tier, for rocprofv3 --pmc")
@@ -90,6 +92,8 @@ def main():
     timer = ea.Timer()
     want = set(args.only.split(",")) if args.only else {"crt", "int8", "reduced", "mlp", "backward", "host", "sizes", "c1", "f32"}
 
+    if args.igemm_direct >= 0:
+        lib.hip_igemm_set_direct(args.igemm_direct)
     if args.pmc_probe:
         # Short program for `rocprofv3 --pmc ...` runs: a 512 MiB device copy of known size
         # (calibrates FETCH_SIZE / WRITE_SIZE), then three launches of one tier. No timing.
