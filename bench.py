@@ -195,11 +195,26 @@ def main():
         rate = C.c_double()
         if probe.hip_probe_peak(kind, rnd, C.byref(rate), st) == 0:
             sustained[name] = rate.value / 1e12
-    t_m, t_v, t_b = C.c_double(), C.c_double(), C.c_double()
-    if probe.hip_probe_coissue(C.byref(t_m), C.byref(t_v), C.byref(t_b), st) == 0:
-        sustained["simd_shared_by_a_wave_of_mfma_and_a_wave_of_valu_ms"] = {
-            "mfma_alone": t_m.value, "valu_alone": t_v.value, "both": t_b.value,
-            "note": "both = max: side by side; both = sum: the SIMD runs one or the other"}
+    # a SIMD shared by a wave of int8 MFMAs and a wave of vector ALU instructions of one kind (ms):
+    # short = vector ALU waves the shorter ones (hidden: share of them that ran beside the MFMAs),
+    # long = the longer ones (rate: their speed beside the MFMAs relative to alone)
+    shared = {}
+    for kname, kind in (("v_fma_f32", 0), ("v_dot4_u32_u8", 1), ("residue_epilogue_mix", 2),
+                        ("residue_epilogue_mix_without_dot4", 3)):
+        for rname, rnd in (("constant", 0), ("random", 1)):
+            row = {}
+            for vname, iters in (("short", 6000), ("long", 30000)):
+                t_m, t_v, t_b = C.c_double(), C.c_double(), C.c_double()
+                if probe.hip_probe_coissue(kind, rnd, iters, C.byref(t_m), C.byref(t_v), C.byref(t_b), st) != 0:
+                    continue
+                m, v, b = t_m.value, t_v.value, t_b.value
+                row[vname] = {"mfma": round(m, 3), "valu": round(v, 3), "both": round(b, 3)}
+                if vname == "short":
+                    row[vname]["hidden"] = round((m + v - b) / min(m, v), 2)
+                else:
+                    row[vname]["rate_beside_mfma"] = round((m + v - b) / m, 2)
+            shared["%s_%s_operands" % (kname, rname)] = row
+    sustained["simd_shared_by_a_wave_of_mfma_and_a_wave_of_valu_ms"] = shared
     log("device sustains (T/s):", json.dumps(sustained))
     fast = (M % 128 == 0 and N % 128 == 0 and K % 16 == 0)
     kernel = "dgemm_fast_kernel<NN>" if fast else "dgemm_mfma_kernel<128,128>"

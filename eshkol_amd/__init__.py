@@ -198,7 +198,7 @@ def load_probe():
     probe.hip_probe_peak.restype = C.c_int
     probe.hip_probe_peak.argtypes = [C.c_int, C.c_int, dp, vp]
     probe.hip_probe_coissue.restype = C.c_int
-    probe.hip_probe_coissue.argtypes = [dp, dp, dp, vp]
+    probe.hip_probe_coissue.argtypes = [C.c_int, C.c_int, C.c_int, dp, dp, dp, vp]
     return probe
 
 

@@ -6,13 +6,23 @@
  * Why. With 256 accumulators a wave owns its SIMD, and whenever it does not issue
  * MFMAs (the epilogue of a finished tile, the barrier of every k-block, a wait
  * for LDS) the SIMD's matrix pipe idles. The epilogue does not depend on K, so it
- * weighs most on short contractions (K = 1024: about half of a tile). A second
- * wave on the SIMD fills what of that is waiting: barrier and LDS waits, the
- * epilogue's trips through LDS and its stores. It does NOT fill the epilogue's
- * arithmetic: on this chip a SIMD runs either MFMA passes or vector ALU
- * instructions, whichever wave they come from (a wave of MFMAs and a wave of
- * VALU work sharing a SIMD take the sum of their times, measured), so staggering
- * the two workgroups of a CU by half a tile changed nothing and is not done.
+ * weighs most on short contractions (K = 1024: about half of a tile). With two
+ * workgroups per CU the pair settles by itself into opposite phases: while one
+ * is in its epilogue the other is in its main loop (time stamps per workgroup and
+ * CU, 4096 x 1024 x 1024, sixteen planes: epilogue 6 us, main loop 8 us, two tiles
+ * per 14.5 us and CU, where one workgroup alone would need 10 us per tile).
+ *
+ * What bounds it. A SIMD does run a wave's vector ALU instructions beside another
+ * wave's MFMAs, but at about half their speed alone (0.4 ... 0.7 measured per
+ * instruction with random operand bytes in the MFMAs), and v_dot4 not at all: it
+ * shares the matrix pipe. So the epilogue beside a main loop takes 6 us where it
+ * takes 3 alone, during those 6 us only one wave per SIMD issues MFMAs, and that
+ * wave alone does not fill the pipe (8 us per tile, against 5.9 per tile while
+ * both workgroups are in their main loops). Taking the byte dot product out of
+ * the epilogue (two 16-bit folds instead: 6.2 -> 5.0 us beside a main loop),
+ * raising either phase's wave priority, and reading the B fragments of a k-step
+ * earlier were each measured and change the kernel's time by less than the
+ * 2 per cent two runs differ by; none is in.
  * Measured on sixteen residue planes of 4096 x 4096: K = 512 -6 %, K = 1024 -5 %
  * (-8 % at 8192 x 8192), K = 2048 +2 %, K >= 4096 +7 ... +10 % against the
  * 256 x 256 kernel: this one is for K <= 1024.

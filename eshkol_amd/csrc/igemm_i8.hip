@@ -459,8 +459,8 @@ void igemm_i8_direct_kernel(HipIgemmArgs g, int tiles_m, int tiles_n, int chunk,
 }
 
 /* The same on 256 x 128 tiles with 128 accumulators per wave, two workgroups per
- * CU (gemm_pipe3.h): a second wave on every SIMD fills the first one's waits. For
- * contractions whose K is short enough for the time between tiles to matter. */
+ * CU (gemm_pipe3.h): while one workgroup is in its epilogue the other multiplies.
+ * For contractions whose K is short enough for the time between tiles to matter. */
 __global__ __launch_bounds__(256, 2)
 void igemm_i8_direct_half_kernel(HipIgemmArgs g, int tiles_m, int tiles_n, int chunk, int n_ids) {
     extern __shared__ __align__(16) int8_t smem_i8[];

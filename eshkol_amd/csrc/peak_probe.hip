@@ -116,13 +116,20 @@ void probe_copy(const v4i_t* __restrict__ src, v4i_t* __restrict__ dst, size_t n
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
 }
 
-/* Do a wave's vector ALU instructions run while another wave's MFMAs occupy the
- * same SIMD? 512 threads = eight waves per workgroup, one workgroup per CU, two
- * waves on every SIMD: waves 0-3 issue int8 MFMAs back to back, waves 4-7 the
- * instruction mix of a residue epilogue (add, byte dot product, convert, fma,
- * 24-bit multiply-add). Either half can be switched off with a count of 0. */
+/* Which of a wave's vector ALU instructions run while another wave's MFMAs occupy
+ * the same SIMD? 512 threads = eight waves per workgroup, one workgroup per CU, two
+ * waves on every SIMD: waves 0-3 issue int8 MFMAs back to back (constant or random
+ * operand bits), waves 4-7 forty instructions per iteration of one kind, eight
+ * independent chains:
+ *   KIND 0  v_fma_f32                 (stands for the plain vector ALU instructions)
+ *   KIND 1  v_dot4_u32_u8             (the byte dot product of a residue epilogue)
+ *   KIND 2  the epilogue's mix: add, byte dot product, convert, fma, 24-bit multiply-add
+ *   KIND 3  the same mix with the byte dot product replaced by a 16-bit fold
+ *           (shift, 24-bit multiply-add), which reduces modulo p as well
+ * Either half can be switched off with a count of 0. */
+template <int KIND>
 __global__ __launch_bounds__(512, 1)
-void probe_coissue(int mfma_iters, int valu_iters, int* sink) {
+void probe_coissue(int mfma_iters, int valu_iters, int random, int* sink) {
     const int wave = threadIdx.x >> 6;
     if (wave < 4) {
         v16i_t acc[4];
@@ -132,7 +139,11 @@ void probe_coissue(int mfma_iters, int valu_iters, int* sink) {
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][r] = 0;
 #pragma unroll
-        for (int r = 0; r < 4; r++) { a[r] = 0x01010101 * (int)(threadIdx.x & 3); b[r] = 0x02020202; }
+        for (int r = 0; r < 4; r++) {
+            const unsigned h1 = mix(threadIdx.x * 4 + r + blockIdx.x * 7919), h2 = mix(h1 + 12345);
+            a[r] = random ? (int)h1 : 0x01010101 * (int)(threadIdx.x & 3);
+            b[r] = random ? (int)h2 : 0x02020202;
+        }
         for (int it = 0; it < mfma_iters; it++) {
 #pragma unroll
             for (int i = 0; i < 4; i++) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc[i], 0, 0, 0);
@@ -142,21 +153,44 @@ void probe_coissue(int mfma_iters, int valu_iters, int* sink) {
         if (s == 0x12345678) sink[0] = s;
     } else {
         unsigned x[8];
-        float q[8];
 #pragma unroll
         for (int e = 0; e < 8; e++) x[e] = mix(threadIdx.x * 8 + e);
-        const unsigned wb = 0x01100401u;
-        const int p = 251;
-        const float pinv = 1.0f / 251.0f;
-        for (int it = 0; it < valu_iters; it++) {
+        if (KIND == 0) {
+            const unsigned c = 0x3f7fbe77u;     /* 0.999 */
+            for (int it = 0; it < valu_iters; it++) {
 #pragma unroll
-            for (int e = 0; e < 8; e++) x[e] = x[e] + 0x80000000u + (unsigned)it;
+                for (int r = 0; r < 5; r++)
 #pragma unroll
-            for (int e = 0; e < 8; e++) x[e] = __builtin_amdgcn_udot4(x[e], wb, x[e] >> 24, false);
+                    for (int e = 0; e < 8; e++) asm volatile("v_fma_f32 %0, %0, %1, %1" : "+v"(x[e]) : "v"(c));
+            }
+        } else if (KIND == 1) {
+            const unsigned wb = 0x01100401u;
+            for (int it = 0; it < valu_iters; it++) {
 #pragma unroll
-            for (int e = 0; e < 8; e++) q[e] = fmaf((float)(int)x[e], pinv, 12582912.0f);
+                for (int r = 0; r < 5; r++)
 #pragma unroll
-            for (int e = 0; e < 8; e++) x[e] = (unsigned)(__mul24(__float_as_int(q[e]), -p) + (int)x[e]) ^ (x[e] << 13);
+                    for (int e = 0; e < 8; e++) asm volatile("v_dot4_u32_u8 %0, %0, %1, %0" : "+v"(x[e]) : "v"(wb));
+            }
+        } else {
+            float q[8];
+            const unsigned wb = 0x01100401u;
+            const int p = 251;
+            const float pinv = 1.0f / 251.0f;
+            for (int it = 0; it < valu_iters; it++) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) x[e] = x[e] + 0x80000000u + (unsigned)it;
+                if (KIND == 2) {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) x[e] = __builtin_amdgcn_udot4(x[e], wb, x[e] >> 24, false);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) x[e] = (unsigned)(__mul24((int)(x[e] >> 16), 25 - 65536) + (int)x[e]);
+                }
+#pragma unroll
+                for (int e = 0; e < 8; e++) q[e] = fmaf((float)(int)x[e], pinv, 12582912.0f);
+#pragma unroll
+                for (int e = 0; e < 8; e++) x[e] = (unsigned)(__mul24(__float_as_int(q[e]), -p) + (int)x[e]) ^ (x[e] << 13);
+            }
         }
         unsigned s = 0;
         for (int e = 0; e < 8; e++) s += x[e];
@@ -166,17 +200,22 @@ void probe_coissue(int mfma_iters, int valu_iters, int* sink) {
 
 }  // namespace
 
-/* Times (ms) of the MFMA waves alone, the vector ALU waves alone, and both together,
- * each wave's work the same in all three. both = max of the two would mean the SIMD
- * runs them side by side; both = their sum means it runs one or the other. */
-extern "C" int hip_probe_coissue(double* mfma_ms, double* valu_ms, double* both_ms, void* stream) {
-    if (!mfma_ms || !valu_ms || !both_ms) return -1;
+/* Times (ms) of the MFMA waves alone (20000 iterations of four MFMAs), the vector
+ * ALU waves alone (valu_iters iterations) and both together, each wave's work the
+ * same in all three. With the vector ALU waves the shorter ones, both = the MFMA
+ * time means they ran entirely beside the MFMAs and both = the sum that they did
+ * not run beside them at all; with the vector ALU waves the longer ones,
+ * (mfma + valu - both) / mfma is the rate at which they advance beside the MFMAs,
+ * relative to their rate alone. */
+extern "C" int hip_probe_coissue(int kind, int random_operands, int valu_iters,
+                                 double* mfma_ms, double* valu_ms, double* both_ms, void* stream) {
+    if (!mfma_ms || !valu_ms || !both_ms || kind < 0 || kind > 3 || valu_iters <= 0) return -1;
     hipStream_t st = (hipStream_t)stream;
     int* sink = nullptr;
     hipEvent_t e0, e1;
     if (!ESHKOL_HIP_OK(hipMalloc((void**)&sink, 256))) return -1;
     if (!ESHKOL_HIP_OK(hipEventCreate(&e0)) || !ESHKOL_HIP_OK(hipEventCreate(&e1))) { (void)hipFree(sink); return -1; }
-    const int M = 20000, V = 6000;
+    const int M = 20000, V = valu_iters;
     const int counts[3][2] = {{M, 0}, {0, V}, {M, V}};
     double out[3] = {0.0, 0.0, 0.0};
     int rc = 0;
@@ -184,7 +223,10 @@ extern "C" int hip_probe_coissue(double* mfma_ms, double* valu_ms, double* both_
         float best = 1e30f;
         for (int rep = 0; rep < 3; rep++) {
             (void)hipEventRecord(e0, st);
-            hipLaunchKernelGGL(probe_coissue, dim3(256), dim3(512), 0, st, counts[c][0], counts[c][1], sink);
+            if (kind == 0) hipLaunchKernelGGL(probe_coissue<0>, dim3(256), dim3(512), 0, st, counts[c][0], counts[c][1], random_operands, sink);
+            else if (kind == 1) hipLaunchKernelGGL(probe_coissue<1>, dim3(256), dim3(512), 0, st, counts[c][0], counts[c][1], random_operands, sink);
+            else if (kind == 2) hipLaunchKernelGGL(probe_coissue<2>, dim3(256), dim3(512), 0, st, counts[c][0], counts[c][1], random_operands, sink);
+            else hipLaunchKernelGGL(probe_coissue<3>, dim3(256), dim3(512), 0, st, counts[c][0], counts[c][1], random_operands, sink);
             (void)hipEventRecord(e1, st);
             float ms = 0.0f;
             if (!ESHKOL_HIP_OK(hipEventSynchronize(e1)) || !ESHKOL_HIP_OK(hipEventElapsedTime(&ms, e0, e1))) { rc = -1; break; }

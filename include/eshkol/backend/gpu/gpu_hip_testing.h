@@ -135,13 +135,19 @@ void hip_ozaki_crt_set_host_pass(int on);
  * its own buffers. */
 int hip_probe_peak(int kind, int random_operands, double* rate, void* stream);
 
-/* Whether a SIMD runs one wave's vector ALU instructions beside another wave's
- * MFMAs: the time (ms) of four waves of back-to-back int8 MFMAs per CU, of four
- * waves of a residue epilogue's instruction mix per CU, and of both sharing the
- * SIMDs two waves each. both = the larger of the two: side by side; both = their
- * sum: one or the other. What the choice of one or two workgroups per CU for the
- * int8 contraction rests on. */
-int hip_probe_coissue(double* mfma_ms, double* valu_ms, double* both_ms, void* stream);
+/* Which vector ALU instructions a SIMD runs beside another wave's MFMAs: the time
+ * (ms) of four waves of back-to-back int8 MFMAs per CU (constant or random operand
+ * bits), of four waves of vector ALU instructions per CU (kind 0: v_fma_f32, 1:
+ * v_dot4_u32_u8, 2: the instruction mix of a residue epilogue, which holds one byte
+ * dot product in nine instructions, 3: that mix with a shift and a 24-bit
+ * multiply-add in the dot product's place; valu_iters iterations), and of both
+ * sharing the SIMDs two waves each. With the vector ALU waves the shorter ones,
+ * both = mfma: entirely beside the MFMAs; both = mfma + valu: not at all. With
+ * them the longer ones, (mfma + valu - both) / mfma is their rate beside the MFMAs
+ * relative to their rate alone. What the 256 x 128 int8 contraction with two
+ * workgroups per CU rests on. */
+int hip_probe_coissue(int kind, int random_operands, int valu_iters,
+                      double* mfma_ms, double* valu_ms, double* both_ms, void* stream);
 
 #ifdef __cplusplus
 }
