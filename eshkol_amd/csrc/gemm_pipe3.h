@@ -13,16 +13,18 @@
  * per 14.5 us and CU, where one workgroup alone would need 10 us per tile).
  *
  * What bounds it. A SIMD does run a wave's vector ALU instructions beside another
- * wave's MFMAs, but at about half their speed alone (0.4 ... 0.7 measured per
- * instruction with random operand bytes in the MFMAs), and v_dot4 not at all: it
- * shares the matrix pipe. So the epilogue beside a main loop takes 6 us where it
- * takes 3 alone, during those 6 us only one wave per SIMD issues MFMAs, and that
- * wave alone does not fill the pipe (8 us per tile, against 5.9 per tile while
- * both workgroups are in their main loops). Taking the byte dot product out of
- * the epilogue (two 16-bit folds instead: 6.2 -> 5.0 us beside a main loop),
- * raising either phase's wave priority, and reading the B fragments of a k-step
- * earlier were each measured and change the kernel's time by less than the
- * 2 per cent two runs differ by; none is in.
+ * wave's MFMAs, at about half their speed alone (v_dot4 not at all: the matrix pipe
+ * executes it), so the epilogue beside a main loop takes 6 us where it takes 3
+ * alone. Time stamps per k-block: the matrix pipe is busy 0.6 of the cycles while
+ * the sibling is in its epilogue and 0.96 while both multiply, at a clock of 1.65
+ * GHz; with the epilogue taken out it is busy 0.99 and the chip lowers the clock
+ * to 1.43 GHz. The kernel's time follows the energy it spends under the power
+ * limit rather than the cycles its pipe is busy: taking the byte dot product out
+ * of the epilogue (a 16-bit fold instead: 6.2 -> 5.0 us beside a main loop, one
+ * instruction more per element, clock 1.59 GHz), raising either phase's wave
+ * priority and reading the B fragments of a k-step earlier were each measured
+ * and change the kernel's time by less than the 2 per cent two runs differ by;
+ * none is in.
  * Measured on sixteen residue planes of 4096 x 4096: K = 512 -6 %, K = 1024 -5 %
  * (-8 % at 8192 x 8192), K = 2048 +2 %, K >= 4096 +7 ... +10 % against the
  * 256 x 256 kernel: this one is for K <= 1024.
