@@ -37,7 +37,7 @@ class HipIgemmArgs(C.Structure):
                 ("ldk", u32), ("M", u32), ("N", u32), ("n_out", u32),
                 ("pair_first", vp), ("pair_a", vp), ("pair_b", vp),
                 ("mode", i32), ("max_pairs", i32), ("modulus", vp), ("out_i32", vp), ("out_i8", vp),
-                ("layout", i32)]
+                ("layout", i32), ("ldn", u32), ("out_rows", u32)]
 
 
 class HipOzakiCrtStages(C.Structure):

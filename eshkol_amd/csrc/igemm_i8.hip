@@ -90,8 +90,8 @@ __device__ __forceinline__ void epilogue(const HipIgemmArgs& g, int o, int m0, i
     const int li = lane & 31, lh = lane >> 5;
 
     if (g.mode == 0) {
-        int32_t* out = g.out_i32 + (size_t)o * g.M * g.N;
-        const bool vec_ok = (g.N % 4 == 0);
+        int32_t* out = g.out_i32 + (size_t)o * g.out_rows * g.ldn;
+        const bool vec_ok = (g.ldn % 4 == 0);
 #pragma unroll
         for (int t = 0; t < TM; t++) {
             const int row = m0 + wm * TM * 32 + t * 32 + li;
@@ -101,16 +101,16 @@ __device__ __forceinline__ void epilogue(const HipIgemmArgs& g, int o, int m0, i
 #pragma unroll
                 for (int v = 0; v < 4; v++) {
                     const int col = n0 + wn * TN * 32 + u * 32 + 8 * v + 4 * lh;
-                    if (row < (int)g.M) {
-                        int32_t* p = out + (size_t)row * g.N + col;
-                        if (vec_ok && col + 3 < (int)g.N) {
+                    if (row < (int)g.out_rows) {
+                        int32_t* p = out + (size_t)row * g.ldn + col;
+                        if (vec_ok && col + 3 < (int)g.ldn) {
                             v4i_t w = {acc[t][u][4 * v], acc[t][u][4 * v + 1],
                                        acc[t][u][4 * v + 2], acc[t][u][4 * v + 3]};
                             *(v4i_t*)p = w;
                         } else {
 #pragma unroll
                             for (int e = 0; e < 4; e++)
-                                if (col + e < (int)g.N) p[e] = acc[t][u][4 * v + e];
+                                if (col + e < (int)g.ldn) p[e] = acc[t][u][4 * v + e];
                         }
                     }
                     /* one 4-register group at a time: without the fence the
@@ -167,20 +167,20 @@ __device__ __forceinline__ void epilogue(const HipIgemmArgs& g, int o, int m0, i
         }
     }
     __syncthreads();
-    int8_t* out = g.out_i8 + (size_t)o * g.M * g.N;
-    const bool vec_ok = (g.N % 16 == 0) && (((uintptr_t)out & 15) == 0);
+    int8_t* out = g.out_i8 + (size_t)o * g.out_rows * g.ldn;
+    const bool vec_ok = (g.ldn % 16 == 0) && (((uintptr_t)out & 15) == 0);
     constexpr int CHUNKS_PER_ROW = BN / 16;
     constexpr int TOTAL = BM * CHUNKS_PER_ROW;
     for (int c = tid; c < TOTAL; c += NT) {
         const int lrow = c / CHUNKS_PER_ROW, lc = (c % CHUNKS_PER_ROW) * 16;
         const int row = m0 + lrow, col = n0 + lc;
-        if (row >= (int)g.M || col >= (int)g.N) continue;
+        if (row >= (int)g.out_rows || col >= (int)g.ldn) continue;
         const int8_t* src = stage + lrow * EPITCH + lc;
-        int8_t* dst = out + (size_t)row * g.N + col;
-        if (vec_ok && col + 15 < (int)g.N) {
+        int8_t* dst = out + (size_t)row * g.ldn + col;
+        if (vec_ok && col + 15 < (int)g.ldn) {
             *(v4i_t*)dst = *(const v4i_t*)src;
         } else {
-            for (int e = 0; e < 16 && col + e < (int)g.N; e++) dst[e] = src[e];
+            for (int e = 0; e < 16 && col + e < (int)g.ldn; e++) dst[e] = src[e];
         }
     }
 }
@@ -289,11 +289,11 @@ __device__ __forceinline__ void epilogue_direct(const HipIgemmArgs& g, int o, in
     const int li = lane & 31, lh = lane >> 5;
 
     if (g.mode == 0) {
-        int32_t* out = g.out_i32 + (size_t)o * g.M * g.N;
-        const bool vec_ok = (g.N % 4 == 0);
+        int32_t* out = g.out_i32 + (size_t)o * g.out_rows * g.ldn;
+        const bool vec_ok = (g.ldn % 4 == 0);
         /* a tile inside the matrix: no bounds, no branches, one address per block (the same for every lane) */
         const bool interior0 = vec_ok && (((uintptr_t)out & 15) == 0) &&
-                               m0 + TILE_M <= (int)g.M && n0 + TILE_N <= (int)g.N;
+                               m0 + TILE_M <= (int)g.out_rows && n0 + TILE_N <= (int)g.ldn;
 #pragma unroll
         for (int t = 0; t < TM; t++) {
             const int row = m0 + wave * 64 + t * 32 + li;
@@ -309,14 +309,14 @@ __device__ __forceinline__ void epilogue_direct(const HipIgemmArgs& g, int o, in
                 }
                 if (interior0) {
                     constexpr int AB = (TN >= 8) ? 4 : 2;        /* rows in flight: registers are short on the 128-column tile */
-                    int32_t* p = out + (size_t)(row - li + (lane >> 3)) * g.N + (n0 + u * 32 + 4 * (lane & 7));
+                    int32_t* p = out + (size_t)(row - li + (lane >> 3)) * g.ldn + (n0 + u * 32 + 4 * (lane & 7));
 #pragma unroll
                     for (int i0 = 0; i0 < 4; i0 += AB) {
                         v4i_t w[AB];
 #pragma unroll
                         for (int i = 0; i < AB; i++) w[i] = pipe2::parked_row16(stage, i0 + i);
 #pragma unroll
-                        for (int i = 0; i < AB; i++) *(v4i_t*)(p + (size_t)(8 * (i0 + i)) * g.N) = w[i];
+                        for (int i = 0; i < AB; i++) *(v4i_t*)(p + (size_t)(8 * (i0 + i)) * g.ldn) = w[i];
                         if (AB < 4) __builtin_amdgcn_sched_barrier(0);
                     }
                 } else {
@@ -324,10 +324,10 @@ __device__ __forceinline__ void epilogue_direct(const HipIgemmArgs& g, int o, in
                     for (int i = 0; i < 4; i++) {
                         const v4i_t w = pipe2::parked_row16(stage, i);
                         const int orow = row - li + (lane >> 3) + 8 * i, col = n0 + u * 32 + 4 * (lane & 7);
-                        if (orow < (int)g.M && col < (int)g.N) {
-                            int32_t* p = out + (size_t)orow * g.N + col;
-                            if (vec_ok && col + 3 < (int)g.N) *(v4i_t*)p = w;
-                            else for (int e = 0; e < 4; e++) if (col + e < (int)g.N) p[e] = w[e];
+                        if (orow < (int)g.out_rows && col < (int)g.ldn) {
+                            int32_t* p = out + (size_t)orow * g.ldn + col;
+                            if (vec_ok && col + 3 < (int)g.ldn) *(v4i_t*)p = w;
+                            else for (int e = 0; e < 4; e++) if (col + e < (int)g.ldn) p[e] = w[e];
                         }
                     }
                 }
@@ -347,9 +347,9 @@ __device__ __forceinline__ void epilogue_direct(const HipIgemmArgs& g, int o, in
     const uint32_t lift = (uint32_t)pipe2::scalar_load((const int32_t*)&MOD_TABLES.start[p & 0x1ff]);
     const float pinv = 1.0f / (float)p;
     constexpr int EP = pipe2::EPI_PITCH;
-    int8_t* out = g.out_i8 + (size_t)o * g.M * g.N;
-    const bool vec_ok = (g.N % 16 == 0) && (((uintptr_t)out & 15) == 0);
-    const bool interior = vec_ok && m0 + TILE_M <= (int)g.M && n0 + TILE_N <= (int)g.N;    /* the same for every lane */
+    int8_t* out = g.out_i8 + (size_t)o * g.out_rows * g.ldn;
+    const bool vec_ok = (g.ldn % 16 == 0) && (((uintptr_t)out & 15) == 0);
+    const bool interior = vec_ok && m0 + TILE_M <= (int)g.out_rows && n0 + TILE_N <= (int)g.ldn;    /* the same for every lane */
 #pragma unroll
     for (int t = 0; t < TM; t++) {
 #pragma unroll
@@ -394,7 +394,7 @@ __device__ __forceinline__ void epilogue_direct(const HipIgemmArgs& g, int o, in
                  * and row block (2.8 of this epilogue's 9 us per tile were the guarded
                  * stores below: a branch and a 64-bit product each) */
                 constexpr int AB = (TN >= 8) ? 4 : 2;            /* rows in flight, as above */
-                int8_t* dst = out + (size_t)(m0 + wave * 64 + t * 32 + (lane >> 3)) * g.N + (n0 + 128 * h + 16 * (lane & 7));
+                int8_t* dst = out + (size_t)(m0 + wave * 64 + t * 32 + (lane >> 3)) * g.ldn + (n0 + 128 * h + 16 * (lane & 7));
 #pragma unroll
                 for (int i0 = 0; i0 < 4; i0 += AB) {
                     v4i_t val[AB];
@@ -402,7 +402,7 @@ __device__ __forceinline__ void epilogue_direct(const HipIgemmArgs& g, int o, in
                     for (int i = 0; i < AB; i++)
                         val[i] = *(const v4i_t*)(stage + ((lane >> 3) + 8 * (i0 + i)) * EP + (lane & 7) * 16);
 #pragma unroll
-                    for (int i = 0; i < AB; i++) *(v4i_t*)(dst + (size_t)(8 * (i0 + i)) * g.N) = val[i];
+                    for (int i = 0; i < AB; i++) *(v4i_t*)(dst + (size_t)(8 * (i0 + i)) * g.ldn) = val[i];
                     if (AB < 4) __builtin_amdgcn_sched_barrier(0);
                 }
                 continue;
@@ -413,13 +413,13 @@ __device__ __forceinline__ void epilogue_direct(const HipIgemmArgs& g, int o, in
                 const int lrow = c >> 3, ch = c & 7;
                 const int row = m0 + wave * 64 + t * 32 + lrow, col = n0 + 128 * h + 16 * ch;
                 const v4i_t val = *(const v4i_t*)(stage + lrow * EP + ch * 16);
-                if (row < (int)g.M && col < (int)g.N) {
-                    int8_t* dst = out + (size_t)row * g.N + col;
-                    if (vec_ok && col + 15 < (int)g.N) {
+                if (row < (int)g.out_rows && col < (int)g.ldn) {
+                    int8_t* dst = out + (size_t)row * g.ldn + col;
+                    if (vec_ok && col + 15 < (int)g.ldn) {
                         *(v4i_t*)dst = val;
                     } else {
                         const int8_t* src = stage + lrow * EP + ch * 16;
-                        for (int e = 0; e < 16 && col + e < (int)g.N; e++) dst[e] = src[e];
+                        for (int e = 0; e < 16 && col + e < (int)g.ldn; e++) dst[e] = src[e];
                     }
                 }
             }
@@ -727,9 +727,13 @@ extern "C" int hip_igemm_i8(const HipIgemmArgs* args, void* stream) {
     EshkolHipCall bracket(stream);
     if (!args || !args->a_planes || !args->b_planes || !args->pair_first || !args->pair_a || !args->pair_b)
         return -1;
-    const HipIgemmArgs& a = *args;
+    HipIgemmArgs a = *args;
     if (a.M == 0 || a.N == 0 || a.n_out == 0 || a.ldk == 0 || a.ldk % 128 != 0) return -1;
     if (a.M > 0x7fffffffu || a.N > 0x7fffffffu) return -1;
+    /* output planes of out_rows x ldn elements: dense unless the caller allocated them larger */
+    if (a.ldn == 0) a.ldn = a.N;
+    if (a.out_rows == 0) a.out_rows = a.M;
+    if (a.ldn < a.N || a.out_rows < a.M || a.ldn > 0x7fffffffu || a.out_rows > 0x7fffffffu) return -1;
     if (((uintptr_t)a.a_planes & 15) || ((uintptr_t)a.b_planes & 15) ||
         (a.a_plane_stride & 15) || (a.b_plane_stride & 15)) return -1;
     if (a.mode == 0) { if (!a.out_i32) return -1; }

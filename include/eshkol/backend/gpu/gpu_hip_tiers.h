@@ -123,9 +123,9 @@ typedef struct {
     const int32_t* pair_first;
     const int32_t* pair_a;
     const int32_t* pair_b;
-    /* mode 0: out_i32[o][M][N] = the int32 sums
-     * mode 1: out_i8[o][M][N]  = the sum modulo modulus[o], representative in
-     *         [-p/2, p/2); modulus[] in device memory                           */
+    /* mode 0: out_i32[o][out_rows][ldn] = the int32 sums
+     * mode 1: out_i8[o][out_rows][ldn]  = the sum modulo modulus[o], representative
+     *         in [-p/2, p/2); modulus[] in device memory                        */
     int32_t mode;
     int32_t max_pairs;        /* upper bound on products per output plane (host knows the plan) */
     const int32_t* modulus;
@@ -139,6 +139,13 @@ typedef struct {
      * 1 KiB of contiguous memory. Needs ldk % 512 == 0 and max_pairs >= 1 (every
      * output plane at least one product). */
     int32_t layout;
+    /* The output planes as allocated: out_rows rows of ldn elements each (0: M and
+     * N, dense planes). With ldn a multiple of 16 (4 for mode 0) every store is a
+     * 16-byte one whatever N is, and with out_rows and ldn multiples of 256 no tile
+     * has a bound to check. Elements outside M x N come from the operands' zero
+     * padding: they are written as zeros, or not at all where no tile covers them. */
+    uint32_t ldn;
+    uint32_t out_rows;
 } HipIgemmArgs;
 int hip_igemm_i8(const HipIgemmArgs* args, void* stream);
 

@@ -42,8 +42,9 @@ def interleave(x):
     return np.ascontiguousarray(y).reshape(n, rows, ldk)
 
 
-def run(a, b, M, N, plan, mode, kernel):
-    """plan: list of lists of (a_plane, b_plane) per output plane."""
+def run(a, b, M, N, plan, mode, kernel, out_rows=0, ldn=0):
+    """plan: list of lists of (a_plane, b_plane) per output plane. out_rows, ldn: the output planes as
+    allocated (0: M x N); the whole planes come back."""
     lib = ea.load()
     pf, pers = KERNELS[kernel]
     if kernel in DIRECT_MODE:
@@ -55,8 +56,9 @@ def run(a, b, M, N, plan, mode, kernel):
     dF, dPa, dPb = (ea.DeviceArray.from_host(x) for x in (first, pa, pb))
     dMod = ea.DeviceArray.from_host(np.array(MODULI[:len(plan)] if mode == 1 else [1], np.int32))
     n_out = len(plan)
-    out = ea.DeviceArray.from_host(np.full((n_out, M, N), 0x55, np.int8 if mode == 1 else np.int32))
+    out = ea.DeviceArray.from_host(np.full((n_out, out_rows or M, ldn or N), 0x55, np.int8 if mode == 1 else np.int32))
     g = ea.HipIgemmArgs()
+    g.out_rows, g.ldn = out_rows, ldn
     g.a_planes, g.b_planes = dA.ptr, dB.ptr
     g.a_plane_stride, g.b_plane_stride = a.shape[1] * a.shape[2], b.shape[1] * b.shape[2]
     g.ldk, g.M, g.N, g.n_out = a.shape[2], M, N, n_out
@@ -101,6 +103,27 @@ def test_residue_products(gpu, M, K, N, kernel):
     want = exact(a, b, M, N, K, plan)
     for l, p in enumerate(MODULI):
         assert np.array_equal(got[l].astype(np.int64), symmetric(want[l], p)), (l, p)
+
+
+@pytest.mark.parametrize("kernel", list(KERNELS))
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("M,K,N,out_rows,ldn", [(1000, 700, 1300, 1024, 1536), (1000, 700, 1300, 1000, 1312),
+                                                (2041, 512, 2051, 2048, 2304), (1023, 256, 1025, 1023, 1028)])
+def test_output_planes_larger_than_the_product(gpu, M, K, N, out_rows, ldn, mode, kernel):
+    """Output planes allocated with a row pitch and a row count of their own: the M x N corner holds what the
+    dense call gives, the rest zeros (products of the operands' zero padding) or what was there before."""
+    rng = np.random.default_rng(M + N + mode)
+    n = 16 if mode == 1 else 3
+    a, b = planes(rng, n, M, K), planes(rng, n, N, K)
+    plan = [[(l, l)] for l in range(n)] if mode == 1 else [[(0, 0)], [(1, 1), (2, 2)], [(0, 2), (1, 0), (2, 1)]]
+    dense = run(a, b, M, N, plan, mode, kernel)
+    got = run(a, b, M, N, plan, mode, kernel, out_rows, ldn)
+    assert got.shape == (len(plan), out_rows, ldn)
+    assert np.array_equal(got[:, :M, :N], dense)
+    rest = got.copy()
+    rest[:, :M, :N] = 0
+    fill = 0x55
+    assert np.all((rest == 0) | (rest == fill))
 
 
 @pytest.mark.parametrize("kernel", list(KERNELS))
