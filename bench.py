@@ -329,6 +329,7 @@ def main():
             ga.pair_first, ga.pair_a, ga.pair_b = dT.ptr, dT.ptr + 17 * 4, dT.ptr + 17 * 4
             ga.mode, ga.modulus, ga.out_i8 = 1, dT.ptr + 33 * 4, sg.w_planes
             ga.max_pairs, ga.layout = 1, lay
+            ga.out_rows, ga.ldn = sg.w_rows, sg.w_ld
             eg, _ = timed(lambda: lib.hip_igemm_i8(C.byref(ga), st), settle_ms=40.0)
             # reconstruct: nmod*M*N read + 8*M*N written
             ones = (C.c_double * 16)(*([1.0] * 16))

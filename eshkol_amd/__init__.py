@@ -43,20 +43,20 @@ class HipIgemmArgs(C.Structure):
 class HipOzakiCrtStages(C.Structure):
     _fields_ = [("a_planes", vp), ("b_planes", vp), ("w_planes", vp), ("mu", vp), ("nu", vp),
                 ("rows_a_padded", u64), ("rows_b_padded", u64), ("ldk", u64),
-                ("num_moduli", i32), ("E", i32), ("layout", i32)]
+                ("num_moduli", i32), ("E", i32), ("layout", i32), ("w_rows", u64), ("w_ld", u64)]
 
 
 class HipOzakiFastStages(C.Structure):
     _fields_ = [("a_planes", vp), ("b_planes", vp), ("w_planes", vp), ("shift_a", vp), ("shift_b", vp),
                 ("rows_a_padded", u64), ("rows_b_padded", u64), ("ldk", u64),
                 ("num_moduli", i32), ("E", i32), ("cap", i32), ("moduli", i32 * 16),
-                ("layout", i32)]
+                ("layout", i32), ("w_rows", u64), ("w_ld", u64)]
 
 
 class HipOzakiInt8Stages(C.Structure):
     _fields_ = [("a_slices", vp), ("b_slices", vp), ("products", vp), ("rmax", vp), ("cmax", vp),
                 ("rows_a_padded", u64), ("rows_b_padded", u64), ("ldk", u64),
-                ("s", i32), ("nbuf", i32), ("layout", i32)]
+                ("s", i32), ("nbuf", i32), ("layout", i32), ("g_rows", u64), ("g_ld", u64)]
 
 
 BUF = C.POINTER(EshkolGPUBuffer)

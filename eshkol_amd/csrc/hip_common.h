@@ -96,6 +96,14 @@ static inline int eshkol_hip_num_cus(void) {
 
 static inline size_t round_up_sz(size_t v, size_t m) { return (v + m - 1) / m * m; }
 
+/* Rows and row pitch of the product planes a tier puts between its contraction and
+ * its reconstruction (HipIgemmArgs.out_rows, ldn). A pitch of a multiple of 16
+ * elements keeps every store of the contraction and every load of the
+ * reconstruction a vector one whatever N is; from 1024 on both are rounded up to
+ * the contraction's 256 x 256 tile, which then has no bound to check anywhere. */
+static inline uint64_t eshkol_product_rows(uint64_t M) { return M >= 1024 ? round_up_sz(M, 256) : M; }
+static inline uint64_t eshkol_product_pitch(uint64_t N) { return N >= 1024 ? round_up_sz(N, 256) : round_up_sz(N, 16); }
+
 /* A store whose line nothing on the device reads again soon (operand planes on
  * their way to HBM: gigabytes written once, read by a later kernel): the
  * non-temporal form keeps such lines from displacing what the caches hold and

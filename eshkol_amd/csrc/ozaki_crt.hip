@@ -301,32 +301,38 @@ struct CrtConsts {
  * use: the kernel moves 24 bytes per element and has to keep HBM busy. So is
  * the tanh epilogue: its code would otherwise cost every launch three quarters
  * of its occupancy in registers. */
-/* VEC: N is a multiple of four and W and C are aligned for 4- and 16-byte
+/* W is [NMOD][wrows][ldw]: the product planes as the contraction left them.
+ * VEC 1: N is a multiple of four and W and C are aligned for 4- and 16-byte
  * accesses (the launcher checks): every thread then has four whole elements, and
  * the kernel carries none of the byte-wise path, whose address arithmetic the
  * compiler would otherwise place in front of both paths (a third of the
- * kernel's vector instructions: it is bound by them, not by HBM). */
-template <int NMOD, bool TANH, bool VEC>
+ * kernel's vector instructions: it is bound by them, not by HBM).
+ * VEC 2: W's pitch and base allow the 4-byte loads, but N is not a multiple of
+ * four or C's rows do not start on 16-byte boundaries: whole groups of four are
+ * stored as two 16-byte words at 8-byte alignment, the last group of a row
+ * element by element.
+ * VEC 0: nothing is known about W's alignment either (dense planes of any N). */
+typedef double d2u_t __attribute__((ext_vector_type(2), aligned(8)));
+template <int NMOD, bool TANH, int VEC>
 __global__ __launch_bounds__(256)
-void crt_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t N, CrtConsts cc,
+void crt_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t wrows, uint64_t ldw, uint64_t M, uint64_t N, CrtConsts cc,
                             const int32_t* __restrict__ mu, const int32_t* __restrict__ nu,
                             const double* __restrict__ bias, double* __restrict__ C) {
     const uint32_t cpr = (uint32_t)(((N + 3) / 4 + 255) / 256);   /* blocks per row */
     const uint64_t row = blockIdx.x / cpr;
     const uint64_t col = ((uint64_t)(blockIdx.x % cpr) * 256 + threadIdx.x) * 4;
     if (col >= N) return;
-    const uint64_t tot = M * N, idx = row * N + col;
-    const int nvalid = VEC ? 4 : ((N - col < 4) ? (int)(N - col) : 4);
-    const bool vec = VEC || ((nvalid == 4) && ((N & 3) == 0) && (((uintptr_t)W & 3) == 0));
+    const uint64_t tot = wrows * ldw, idx = row * N + col, widx = row * ldw + col;
+    const int nvalid = (VEC == 1) ? 4 : ((N - col < 4) ? (int)(N - col) : 4);
     uint32_t u[NMOD];
-    if (vec) {
-        const int8_t* p = W + idx;                 /* one address, then a step per plane */
+    if (VEC != 0) {
+        const int8_t* p = W + widx;                /* one address, then a step per plane */
 #pragma unroll
         for (int l = 0; l < NMOD; l++) { u[l] = *(const uint32_t*)p; p += tot; }
     } else {
 #pragma unroll
         for (int l = 0; l < NMOD; l++) {
-            const int8_t* w = W + (uint64_t)l * tot + idx;
+            const int8_t* w = W + (uint64_t)l * tot + widx;
             u[l] = 0;
 #pragma unroll
             for (int e = 0; e < 4; e++) if (e < nvalid) u[l] |= (uint32_t)(uint8_t)w[e] << (8 * e);
@@ -366,9 +372,14 @@ void crt_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t N
         if (TANH) v = eshkol_tanh_f64(v);
         out[e] = v;
     }
-    if (VEC || (vec && (((uintptr_t)C & 15) == 0))) {
+    if (VEC == 1) {
         d2_t* o = (d2_t*)(C + idx);
         d2_t lo, hi;
+        lo.x = out[0]; lo.y = out[1]; hi.x = out[2]; hi.y = out[3];
+        o[0] = lo; o[1] = hi;
+    } else if (VEC == 2 && nvalid == 4) {
+        d2u_t* o = (d2u_t*)(C + idx);
+        d2u_t lo, hi;
         lo.x = out[0]; lo.y = out[1]; hi.x = out[2]; hi.y = out[3];
         o[0] = lo; o[1] = hi;
     } else {
@@ -801,13 +812,12 @@ extern "C" int hip_ozaki_crt_split_planes_f64(const double* X, uint64_t rows, ui
     return crt_split_any(X, rows, K, shift, num_moduli, planes, rows_padded, ldk, kmajor != 0, layout, stream);
 }
 
-extern "C" int hip_ozaki_crt_reconstruct_f64(const int8_t* w_planes, uint64_t M, uint64_t N, int num_moduli,
-                                             const double* sl1, const double* sl2,
-                                             double P1, double P2, double Pinv,
-                                             const int32_t* mu, const int32_t* nu,
-                                             const double* bias, int act,
-                                             double* C, void* stream) {
-    if (!w_planes || !sl1 || !sl2 || !mu || !nu || !C || M == 0 || N == 0) return -1;
+/* Reconstruction from product planes of wrows rows of ldw bytes each. */
+static int crt_reconstruct(const int8_t* w_planes, uint64_t wrows, uint64_t ldw, uint64_t M, uint64_t N, int num_moduli,
+                           const double* sl1, const double* sl2, double P1, double P2, double Pinv,
+                           const int32_t* mu, const int32_t* nu, const double* bias, int act,
+                           double* C, void* stream) {
+    if (!w_planes || !sl1 || !sl2 || !mu || !nu || !C || M == 0 || N == 0 || wrows < M || ldw < N) return -1;
     if (num_moduli < 2 || num_moduli > MAX_MODULI || act < 0 || act > 1) return -1;
     if ((((N + 3) / 4 + 255) / 256) * M > 0x7fffffffULL) return -1;
     CrtConsts cc;
@@ -815,13 +825,15 @@ extern "C" int hip_ozaki_crt_reconstruct_f64(const int8_t* w_planes, uint64_t M,
     for (int l = 0; l < num_moduli; l++) { cc.sl1[l] = sl1[l]; cc.sl2[l] = sl2[l]; }
     cc.P1 = P1; cc.P2 = P2; cc.Pinv = Pinv; cc.n = num_moduli;
     dim3 grid((unsigned)((((N + 3) / 4 + 255) / 256) * M));
-    const bool vec = (N % 4 == 0) && (((uintptr_t)w_planes & 3) == 0) && (((uintptr_t)C & 15) == 0);
+    /* 4-byte loads of W: its base, pitch and plane size multiples of four (N itself, for dense planes) */
+    const bool wvec = (ldw % 4 == 0) && ((wrows * ldw) % 4 == 0) && (((uintptr_t)w_planes & 3) == 0);
+    const int vec = !wvec ? 0 : ((N % 4 == 0) && (((uintptr_t)C & 15) == 0)) ? 1 : 2;
     switch (num_moduli) {
 #define LAUNCH(n, tanh, v) hipLaunchKernelGGL((crt_reconstruct_kernel<n, tanh, v>), grid, dim3(256), 0,    \
-                                              (hipStream_t)stream, w_planes, M, N, cc, mu, nu, bias, C)
+                                              (hipStream_t)stream, w_planes, wrows, ldw, M, N, cc, mu, nu, bias, C)
 #define CASE(n) case n:                                                                                   \
-        if (act == 1) { if (vec) LAUNCH(n, true, true); else LAUNCH(n, true, false); }                     \
-        else { if (vec) LAUNCH(n, false, true); else LAUNCH(n, false, false); }                            \
+        if (act == 1) { if (vec == 1) LAUNCH(n, true, 1); else if (vec == 2) LAUNCH(n, true, 2); else LAUNCH(n, true, 0); } \
+        else { if (vec == 1) LAUNCH(n, false, 1); else if (vec == 2) LAUNCH(n, false, 2); else LAUNCH(n, false, 0); }       \
         break;
         CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8) CASE(9)
         CASE(10) CASE(11) CASE(12) CASE(13) CASE(14) CASE(15) CASE(16)
@@ -830,6 +842,15 @@ extern "C" int hip_ozaki_crt_reconstruct_f64(const int8_t* w_planes, uint64_t M,
         default: return -1;
     }
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
+extern "C" int hip_ozaki_crt_reconstruct_f64(const int8_t* w_planes, uint64_t M, uint64_t N, int num_moduli,
+                                             const double* sl1, const double* sl2,
+                                             double P1, double P2, double Pinv,
+                                             const int32_t* mu, const int32_t* nu,
+                                             const double* bias, int act,
+                                             double* C, void* stream) {
+    return crt_reconstruct(w_planes, M, N, M, N, num_moduli, sl1, sl2, P1, P2, Pinv, mu, nu, bias, act, C, stream);
 }
 
 void eshkol_hip_crt_release(void) {
@@ -962,7 +983,8 @@ static int crt_matmul_impl(const double* A, const double* B, double* C,
         const int32_t* nu = b_ready ? prepared->nu : dnu;
         int8_t* Ap = (int8_t*)eshkol_hip_workspace(WS_APLANES, (size_t)n_mod * Mp * ldk);
         int8_t* Bp = b_ready ? prepared->planes : (int8_t*)eshkol_hip_workspace(WS_BPLANES, (size_t)n_mod * Np * ldk);
-        int8_t* Wp = (int8_t*)eshkol_hip_workspace(WS_PRODUCTS, (size_t)n_mod * M * N);
+        const uint64_t Mw = eshkol_product_rows(M), Nw = eshkol_product_pitch(N);
+        int8_t* Wp = (int8_t*)eshkol_hip_workspace(WS_PRODUCTS, (size_t)n_mod * Mw * Nw);
         if (!Ap || !Bp || !Wp) return -1;
         if (crt_split_any(A, M, K, dmu, n_mod, Ap, Mp, ldk, a_kmajor, layout, st) != 0) return -1;
         if (!b_ready && crt_split_any(B, N, K, dnu, n_mod, Bp, Np, ldk, b_kmajor, layout, st) != 0) return -1;
@@ -974,10 +996,12 @@ static int crt_matmul_impl(const double* A, const double* B, double* C,
         ga.pair_first = g_tables; ga.pair_a = g_tables + 17; ga.pair_b = g_tables + 17;
         ga.mode = 1; ga.max_pairs = 1; ga.modulus = g_tables + 33; ga.out_i8 = Wp;
         ga.layout = layout;
+        ga.out_rows = (uint32_t)Mw; ga.ldn = (uint32_t)Nw;
         if (hip_igemm_i8(&ga, st) != 0) return -1;
-        if (hip_ozaki_crt_reconstruct_f64(Wp, M, N, n_mod, crt.sl1, crt.sl2, crt.P1, crt.P2, crt.Pinv,
-                                          dmu, nu, bias, act, C, st) != 0) return -1;
+        if (crt_reconstruct(Wp, Mw, Nw, M, N, n_mod, crt.sl1, crt.sl2, crt.P1, crt.P2, crt.Pinv,
+                            dmu, nu, bias, act, C, st) != 0) return -1;
         g_last.a_planes = Ap; g_last.b_planes = Bp; g_last.w_planes = Wp;
+        g_last.w_rows = Mw; g_last.w_ld = Nw;
         g_last.mu = dmu; g_last.nu = (int32_t*)nu;
         g_last.rows_a_padded = Mp; g_last.rows_b_padded = Np; g_last.ldk = ldk;
         g_last.num_moduli = n_mod; g_last.E = E; g_last.layout = layout;

@@ -227,12 +227,18 @@ void fast_split_kmajor_il_kernel(const double* __restrict__ X, uint64_t rows, ui
  * (the kernel moves 8 + n bytes per element and has to keep HBM busy). */
 struct FracLimbs { int32_t d[FAST_MAX_MODULI][4]; };
 
-/* VEC: N is a multiple of four and W and C are aligned for 4- and 16-byte
+/* W is [NMOD][wrows][ldw], the product planes as the contraction left them.
+ * VEC 1: N is a multiple of four and W and C are aligned for 4- and 16-byte
  * accesses (the launcher checks): the kernel then carries none of the byte-wise
- * path, whose address arithmetic would otherwise sit in front of both paths. */
-template <int NMOD, bool VEC>
+ * path, whose address arithmetic would otherwise sit in front of both paths.
+ * VEC 2: W allows the 4-byte loads, but N is not a multiple of four or C's rows
+ * do not start on 16-byte boundaries: whole groups of four leave as two 16-byte
+ * words at 8-byte alignment, a row's last group element by element.
+ * VEC 0: nothing is known about W either (dense planes of any N). */
+typedef double d2u_t __attribute__((ext_vector_type(2), aligned(8)));
+template <int NMOD, int VEC>
 __global__ __launch_bounds__(256)
-void fast_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t N,
+void fast_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t wrows, uint64_t ldw, uint64_t M, uint64_t N,
                              FracLimbs fl, double P_over_2_64,
                              const int32_t* __restrict__ sh_a, const int32_t* __restrict__ sh_b,
                              double* __restrict__ C) {
@@ -240,18 +246,17 @@ void fast_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t 
     const uint64_t row = blockIdx.x / cpr;
     const uint64_t col = ((uint64_t)(blockIdx.x % cpr) * 256 + threadIdx.x) * 4;
     if (col >= N) return;
-    const uint64_t tot = M * N, idx = row * N + col;
-    const int nvalid = VEC ? 4 : ((N - col < 4) ? (int)(N - col) : 4);
-    const bool vec = VEC || ((nvalid == 4) && ((N & 3) == 0) && (((uintptr_t)W & 3) == 0));
+    const uint64_t tot = wrows * ldw, idx = row * N + col, widx = row * ldw + col;
+    const int nvalid = (VEC == 1) ? 4 : ((N - col < 4) ? (int)(N - col) : 4);
     uint32_t u[NMOD];
-    if (vec) {
-        const int8_t* p = W + idx;                 /* one address, then a step per plane */
+    if (VEC != 0) {
+        const int8_t* p = W + widx;                /* one address, then a step per plane */
 #pragma unroll
         for (int l = 0; l < NMOD; l++) { u[l] = *(const uint32_t*)p; p += tot; }
     } else {
 #pragma unroll
         for (int l = 0; l < NMOD; l++) {
-            const int8_t* w = W + (uint64_t)l * tot + idx;
+            const int8_t* w = W + (uint64_t)l * tot + widx;
             u[l] = 0;
 #pragma unroll
             for (int e = 0; e < 4; e++) if (e < nvalid) u[l] |= (uint32_t)(uint8_t)w[e] << (8 * e);
@@ -284,10 +289,14 @@ void fast_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t M, uint64_t 
         const double f = fma((double)(int32_t)(S >> 32), 4294967296.0, (double)(uint32_t)S);
         out[e] = ldexp(f * P_over_2_64, -(sa + sb[e]));
     }
-    if (VEC || (vec && (((uintptr_t)C & 15) == 0))) {
+    if (VEC == 1) {
         d2_t lo, hi;
         lo.x = out[0]; lo.y = out[1]; hi.x = out[2]; hi.y = out[3];
         ((d2_t*)(C + idx))[0] = lo; ((d2_t*)(C + idx))[1] = hi;
+    } else if (VEC == 2 && nvalid == 4) {
+        d2u_t lo, hi;
+        lo.x = out[0]; lo.y = out[1]; hi.x = out[2]; hi.y = out[3];
+        ((d2u_t*)(C + idx))[0] = lo; ((d2u_t*)(C + idx))[1] = hi;
     } else {
 #pragma unroll
         for (int e = 0; e < 4; e++) if (e < nvalid) C[idx + e] = out[e];
@@ -444,28 +453,35 @@ extern "C" int hip_ozaki_fast_split_planes_f64(const double* X, uint64_t rows, u
     return split_any(X, rows, K, shift, f.table, planes, rows_padded, ldk, kmajor != 0, layout, (hipStream_t)stream);
 }
 
+/* Reconstruction from product planes of wrows rows of ldw bytes each. */
+static int fast_reconstruct(const int8_t* w_planes, uint64_t wrows, uint64_t ldw, uint64_t M, uint64_t N,
+                            const FastPlan& f, const int32_t* shift_a, const int32_t* shift_b, double* C, hipStream_t st) {
+    if (wrows < M || ldw < N) return -1;
+    const uint64_t nblk = (((N + 3) / 4 + 255) / 256) * M;
+    if (nblk > 0x7fffffffULL) return -1;
+    const bool wvec = (ldw % 4 == 0) && ((wrows * ldw) % 4 == 0) && (((uintptr_t)w_planes & 3) == 0);
+    const int vec = !wvec ? 0 : ((N % 4 == 0) && (((uintptr_t)C & 15) == 0)) ? 1 : 2;
+    switch (f.n) {
+#define LAUNCH(n, v) hipLaunchKernelGGL((fast_reconstruct_kernel<n, v>), dim3((unsigned)nblk), dim3(256), 0, st,  \
+                                        w_planes, wrows, ldw, M, N, f.limbs, ldexp(f.P, -64), shift_a, shift_b, C)
+#define CASE(n) case n:                                                                                          \
+        if (vec == 1) LAUNCH(n, 1); else if (vec == 2) LAUNCH(n, 2); else LAUNCH(n, 0);                           \
+        break;
+        CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8) CASE(9)
+        CASE(10) CASE(11) CASE(12) CASE(13) CASE(14) CASE(15) CASE(16)
+#undef CASE
+#undef LAUNCH
+        default: return -1;
+    }
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -3;
+}
+
 extern "C" int hip_ozaki_fast_reconstruct_f64(const int8_t* w_planes, uint64_t M, uint64_t N, uint64_t K, int num_moduli,
                                               const int32_t* shift_a, const int32_t* shift_b, double* C, void* stream) {
     if (!w_planes || !shift_a || !shift_b || !C || M == 0 || N == 0 || K == 0 || K > 131071) return -1;
     FastPlan f;
     if (make_plan(K, num_moduli, &f, true) != 0) return -1;
-    const uint64_t nblk = (((N + 3) / 4 + 255) / 256) * M;
-    if (nblk > 0x7fffffffULL) return -1;
-    hipStream_t st = (hipStream_t)stream;
-    const bool vec = (N % 4 == 0) && (((uintptr_t)w_planes & 3) == 0) && (((uintptr_t)C & 15) == 0);
-    switch (f.n) {
-#define CASE(n) case n:                                                                                          \
-        if (vec) hipLaunchKernelGGL((fast_reconstruct_kernel<n, true>), dim3((unsigned)nblk), dim3(256), 0, st,   \
-                                    w_planes, M, N, f.limbs, ldexp(f.P, -64), shift_a, shift_b, C);               \
-        else hipLaunchKernelGGL((fast_reconstruct_kernel<n, false>), dim3((unsigned)nblk), dim3(256), 0, st,      \
-                                w_planes, M, N, f.limbs, ldexp(f.P, -64), shift_a, shift_b, C);                   \
-        break;
-        CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8) CASE(9)
-        CASE(10) CASE(11) CASE(12) CASE(13) CASE(14) CASE(15) CASE(16)
-#undef CASE
-        default: return -1;
-    }
-    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+    return fast_reconstruct(w_planes, M, N, M, N, f, shift_a, shift_b, C, (hipStream_t)stream) == 0 ? 0 : -1;
 }
 
 void eshkol_hip_fast_release(void) {
@@ -505,7 +521,8 @@ extern "C" int hip_matmul_ozaki_fast_f64_ex(const double* A, const double* B, do
     int32_t* shb = (int32_t*)eshkol_hip_workspace(WS_COLSHIFT, N * sizeof(int32_t));
     int8_t* Ap = (int8_t*)eshkol_hip_workspace(WS_APLANES, (size_t)f.n * Mp * ldk);
     int8_t* Bp = (int8_t*)eshkol_hip_workspace(WS_BPLANES, (size_t)f.n * Np * ldk);
-    int8_t* Wp = (int8_t*)eshkol_hip_workspace(WS_PRODUCTS, (size_t)f.n * M * N);
+    const uint64_t Mw = eshkol_product_rows(M), Nw = eshkol_product_pitch(N);
+    int8_t* Wp = (int8_t*)eshkol_hip_workspace(WS_PRODUCTS, (size_t)f.n * Mw * Nw);
     if (!amax || !bmax || !sha || !shb || !Ap || !Bp || !Wp) return -2;
 
     /* frexp exponent e = floor(log2 max) + 1 (gpu_memory.mm:2886-2905); the split
@@ -533,29 +550,16 @@ extern "C" int hip_matmul_ozaki_fast_f64_ex(const double* A, const double* B, do
     ga.pair_first = g_tables; ga.pair_a = g_tables + 17; ga.pair_b = g_tables + 17;
     ga.mode = 1; ga.max_pairs = 1; ga.modulus = g_tables + 33; ga.out_i8 = Wp;
     ga.layout = layout;
+    ga.out_rows = (uint32_t)Mw; ga.ldn = (uint32_t)Nw;
     if (hip_igemm_i8(&ga, st) != 0) return -1;
 
-    const uint64_t nblk = (((N + 3) / 4 + 255) / 256) * M;
-    if (nblk > 0x7fffffffULL) return -1;
-    const bool vec = (N % 4 == 0) && (((uintptr_t)Wp & 3) == 0) && (((uintptr_t)C & 15) == 0);
-    switch (f.n) {
-#define CASE(n) case n:                                                                                          \
-        if (vec) hipLaunchKernelGGL((fast_reconstruct_kernel<n, true>), dim3((unsigned)nblk), dim3(256), 0, st,   \
-                                    Wp, M, N, f.limbs, ldexp(f.P, -64), sha, shb, C);                             \
-        else hipLaunchKernelGGL((fast_reconstruct_kernel<n, false>), dim3((unsigned)nblk), dim3(256), 0, st,      \
-                                Wp, M, N, f.limbs, ldexp(f.P, -64), sha, shb, C);                                 \
-        break;
-        CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8) CASE(9)
-        CASE(10) CASE(11) CASE(12) CASE(13) CASE(14) CASE(15) CASE(16)
-#undef CASE
-        default: return -1;
-    }
-    if (!ESHKOL_HIP_OK(hipGetLastError())) return -3;
+    { const int rc = fast_reconstruct(Wp, Mw, Nw, M, N, f, sha, shb, C, st); if (rc != 0) return rc; }
     CrtMaxima mx[2];
     if (eshkol_crt_scan_result(ticket, mx, st) != 0) return -1;
     if (mx[0].nonfinite || mx[1].nonfinite) return -1;                  /* NaN / Inf: not this tier's business; C holds no result */
 
     g_last.a_planes = Ap; g_last.b_planes = Bp; g_last.w_planes = Wp;
+    g_last.w_rows = Mw; g_last.w_ld = Nw;
     g_last.shift_a = sha; g_last.shift_b = shb;
     g_last.rows_a_padded = Mp; g_last.rows_b_padded = Np; g_last.ldk = ldk;
     g_last.num_moduli = f.n; g_last.E = f.E; g_last.cap = f.cap; g_last.layout = layout;

@@ -153,12 +153,18 @@ void slice_kmajor_il_kernel(const double* __restrict__ X, uint64_t rows, uint64_
     slice_group<16>(x, sc, s, planes + eshkol_plane_offset(1, row, k, ldk), rows_padded * ldk);
 }
 
-/* gpu_cuda_kernels.cu:728-741, COLS (2 or 4) consecutive columns per thread; the
- * wider form needs N to be a multiple of 4. The buffers of one element are read
- * four at a time so that a wave keeps several kilobytes of loads in flight. */
-template <int COLS>
+/* gpu_cuda_kernels.cu:728-741, COLS (2 or 4) consecutive columns per thread. The
+ * product buffers are [nbuf][grows][ldg] int32. PITCHED: their pitch, plane size
+ * and base are multiples of COLS words (the tier's own buffers: the pitch is
+ * rounded up beyond N), so every thread loads whole vectors whatever N is, and
+ * whole groups leave as 16-byte stores at 8-byte alignment; otherwise (dense
+ * buffers of any N) vectors only where N is a multiple of COLS. The buffers of one
+ * element are read four at a time so that a wave keeps several kilobytes of loads
+ * in flight. */
+typedef double d2u_t __attribute__((ext_vector_type(2), aligned(8)));
+template <int COLS, bool PITCHED>
 __global__ __launch_bounds__(256)
-void reconstruct_kernel(double* __restrict__ C, const int32_t* __restrict__ Gall,
+void reconstruct_kernel(double* __restrict__ C, const int32_t* __restrict__ Gall, uint64_t grows, uint64_t ldg,
                         const double* __restrict__ weights, int nbuf,
                         const double* __restrict__ rmax, const double* __restrict__ cmax,
                         uint64_t M, uint64_t N) {
@@ -167,15 +173,15 @@ void reconstruct_kernel(double* __restrict__ C, const int32_t* __restrict__ Gall
     const uint64_t row = blockIdx.x / cpr;
     const uint64_t col = ((uint64_t)(blockIdx.x % cpr) * 256 + threadIdx.x) * COLS;
     if (col >= N) return;
-    const uint64_t tot = M * N, idx = row * N + col;
+    const uint64_t tot = grows * ldg, idx = row * N + col, gidx = row * ldg + col;
     const int nvalid = (N - col < COLS) ? (int)(N - col) : COLS;
-    const bool vec = (nvalid == COLS) && (N % COLS == 0);
+    const bool vec = PITCHED || ((nvalid == COLS) && (N % COLS == 0));
     double acc[COLS];
 #pragma unroll
     for (int e = 0; e < COLS; e++) acc[e] = 0.0;
 #pragma unroll 4
     for (int b = 0; b < nbuf; b++) {
-        const int32_t* g = Gall + (uint64_t)b * tot + idx;
+        const int32_t* g = Gall + (uint64_t)b * tot + gidx;
         int32_t gv[COLS];
         if (vec) {
             const vec_t v = *(const vec_t*)g;
@@ -190,14 +196,14 @@ void reconstruct_kernel(double* __restrict__ C, const int32_t* __restrict__ Gall
         for (int e = 0; e < COLS; e++) acc[e] = acc[e] + w * (double)gv[e];
     }
     const double r = rmax[row];
-    if (vec && (((uintptr_t)C & 15) == 0)) {
+    if (PITCHED ? (nvalid == COLS) : (vec && (((uintptr_t)C & 15) == 0))) {
         /* the reference's operations in its order; the results leave two to a store */
 #pragma unroll
         for (int e = 0; e < COLS; e += 2) {
-            d2_t v;
+            d2u_t v;
             v.x = (acc[e] * r) * cmax[col + e];
             v.y = (acc[e + 1] * r) * cmax[col + e + 1];
-            *(d2_t*)(C + idx + e) = v;
+            *(d2u_t*)(C + idx + e) = v;
         }
         return;
     }
@@ -279,20 +285,30 @@ extern "C" int hip_ozaki_slice_planes_f64(const double* X, uint64_t rows, uint64
     return slice_any(X, rows, K, scale, s, planes, rows_padded, ldk, kmajor != 0, layout, stream);
 }
 
+/* Reconstruction from product buffers of grows rows of ldg words each. */
+static int slice_reconstruct(double* C, const int32_t* Gall, uint64_t grows, uint64_t ldg, const double* d_weights, int nbuf,
+                             const double* rmax, const double* cmax, uint64_t M, uint64_t N, hipStream_t st) {
+    if (!C || !Gall || !d_weights || !rmax || !cmax || nbuf < 1 || M == 0 || N == 0 || grows < M || ldg < N) return -1;
+    const bool pitched = (ldg % 4 == 0) && ((grows * ldg) % 4 == 0) && (((uintptr_t)Gall & 15) == 0) && ldg >= ((N + 3) & ~3ull);
+    const int cols = (pitched || (N % 4 == 0 && ((uintptr_t)Gall & 15) == 0)) ? 4 : 2;
+    const uint64_t nblk = (((N + cols - 1) / cols + 255) / 256) * M;
+    if (nblk > 0x7fffffffULL) return -1;
+    if (pitched)
+        hipLaunchKernelGGL((reconstruct_kernel<4, true>), dim3((unsigned)nblk), dim3(256), 0, st,
+                           C, Gall, grows, ldg, d_weights, nbuf, rmax, cmax, M, N);
+    else if (cols == 4)
+        hipLaunchKernelGGL((reconstruct_kernel<4, false>), dim3((unsigned)nblk), dim3(256), 0, st,
+                           C, Gall, grows, ldg, d_weights, nbuf, rmax, cmax, M, N);
+    else
+        hipLaunchKernelGGL((reconstruct_kernel<2, false>), dim3((unsigned)nblk), dim3(256), 0, st,
+                           C, Gall, grows, ldg, d_weights, nbuf, rmax, cmax, M, N);
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
 extern "C" int hip_ozaki_reconstruct_f64(double* C, const int32_t* Gall, const double* d_weights, int nbuf,
                                          const double* rmax, const double* cmax,
                                          uint64_t M, uint64_t N, void* stream) {
-    if (!C || !Gall || !d_weights || !rmax || !cmax || nbuf < 1 || M == 0 || N == 0) return -1;
-    const int cols = (N % 4 == 0 && ((uintptr_t)Gall & 15) == 0) ? 4 : 2;
-    const uint64_t nblk = (((N + cols - 1) / cols + 255) / 256) * M;
-    if (nblk > 0x7fffffffULL) return -1;
-    if (cols == 4)
-        hipLaunchKernelGGL(reconstruct_kernel<4>, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
-                           C, Gall, d_weights, nbuf, rmax, cmax, M, N);
-    else
-        hipLaunchKernelGGL(reconstruct_kernel<2>, dim3((unsigned)nblk), dim3(256), 0, (hipStream_t)stream,
-                           C, Gall, d_weights, nbuf, rmax, cmax, M, N);
-    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+    return slice_reconstruct(C, Gall, M, N, d_weights, nbuf, rmax, cmax, M, N, (hipStream_t)stream);
 }
 
 void eshkol_hip_int8_release(void) {
@@ -364,7 +380,8 @@ extern "C" int hip_matmul_ozaki_int8_f64_ex(const double* A, const double* B, do
     const Plan* dplan = plan_on_device(plan_host, st);
     int8_t* As   = (int8_t*)eshkol_hip_workspace(WS_APLANES, (size_t)s * Mp * ldk);
     int8_t* Bs   = (int8_t*)eshkol_hip_workspace(WS_BPLANES, (size_t)s * Np * ldk);
-    int32_t* G   = (int32_t*)eshkol_hip_workspace(WS_PRODUCTS, (size_t)nbuf * M * N * sizeof(int32_t));
+    const uint64_t Mw = eshkol_product_rows(M), Nw = eshkol_product_pitch(N);
+    int32_t* G   = (int32_t*)eshkol_hip_workspace(WS_PRODUCTS, (size_t)nbuf * Mw * Nw * sizeof(int32_t));
     if (!rmax || !cmax || !dplan || !As || !Bs || !G) return -1;
 
     if ((a_kmajor ? hip_colabsmax_f64(A, K, M, 1.0, rmax, st) : hip_rowabsmax_f64(A, M, K, 1.0, rmax, st)) != 0) return -1;
@@ -387,14 +404,16 @@ extern "C" int hip_matmul_ozaki_int8_f64_ex(const double* A, const double* B, do
     ga.ldk = (uint32_t)ldk; ga.M = (uint32_t)M; ga.N = (uint32_t)N; ga.n_out = (uint32_t)nbuf;
     ga.pair_first = dplan->first; ga.pair_a = dplan->pa; ga.pair_b = dplan->pb;
     ga.mode = 0; ga.max_pairs = s; ga.out_i32 = G; ga.layout = layout;
+    ga.out_rows = (uint32_t)Mw; ga.ldn = (uint32_t)Nw;
     if (hip_igemm_i8(&ga, st) != 0) return -1;
-    if (hip_ozaki_reconstruct_f64(C, G, dplan->w, nbuf, rmax, cmax, M, N, st) != 0) return -1;
+    if (slice_reconstruct(C, G, Mw, Nw, dplan->w, nbuf, rmax, cmax, M, N, st) != 0) return -1;
 
     CrtMaxima mx[2];
     if (eshkol_crt_scan_result(ticket, mx, st) != 0) return -1;
     if (mx[0].nonfinite || mx[1].nonfinite) return -1;
 
     g_last.a_slices = As; g_last.b_slices = Bs; g_last.products = G;
+    g_last.g_rows = Mw; g_last.g_ld = Nw;
     g_last.rmax = rmax; g_last.cmax = cmax;
     g_last.rows_a_padded = Mp; g_last.rows_b_padded = Np; g_last.ldk = ldk;
     g_last.s = s; g_last.nbuf = nbuf; g_last.layout = layout;

@@ -31,12 +31,13 @@ typedef struct {
     uint64_t rows_a_padded, rows_b_padded, ldk;
     int32_t num_moduli, E;
     int32_t layout;             /* of a_planes and b_planes: HipIgemmArgs.layout */
+    uint64_t w_rows, w_ld;      /* w_planes is [num_moduli][w_rows][w_ld]: the products' M x N corner counts */
 } HipOzakiCrtStages;
 int hip_ozaki_crt_last_stages(HipOzakiCrtStages* out);
 
 /* Device pointers to the stages of the last hip_matmul_ozaki_fast_f64 call (valid
  * until the next tier call): residue planes [l][row padded to 256][ldk] of A and
- * of B^T, product residues [l][M][N], the per-row and per-column shifts
+ * of B^T, product residues [l][w_rows][w_ld] (the M x N corner counts), the per-row and per-column shifts
  * E - frexp exponent (0 for an all-zero row), and the moduli. */
 typedef struct {
     const int8_t* a_planes;
@@ -48,6 +49,7 @@ typedef struct {
     int32_t num_moduli, E, cap;
     int32_t moduli[16];
     int32_t layout;             /* of a_planes and b_planes: HipIgemmArgs.layout */
+    uint64_t w_rows, w_ld;      /* w_planes is [num_moduli][w_rows][w_ld] */
 } HipOzakiFastStages;
 int hip_ozaki_fast_last_stages(HipOzakiFastStages* out);
 
@@ -58,6 +60,7 @@ typedef struct {
     uint64_t rows_a_padded, rows_b_padded, ldk;
     int32_t s, nbuf;
     int32_t layout;             /* of a_slices and b_slices: HipIgemmArgs.layout */
+    uint64_t g_rows, g_ld;      /* products is [nbuf][g_rows][g_ld] */
 } HipOzakiInt8Stages;
 int hip_ozaki_int8_last_stages(HipOzakiInt8Stages* out);
 

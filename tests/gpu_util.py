@@ -74,7 +74,7 @@ def run_crt(A, B, num_moduli=16, adaptive=False, bias=None, act=0, want_stages=T
               a_planes=ap[:, :M, :K], b_planes=bp[:, :N, :K],
               a_pad_clear=(not ap[:, M:, :].any()) and (not ap[:, :, K:].any()),
               b_pad_clear=(not bp[:, N:, :].any()) and (not bp[:, :, K:].any()),
-              w_planes=ea.download_raw(sg.w_planes, (n, M, N), np.int8))
+              w_planes=ea.download_raw(sg.w_planes, (n, sg.w_rows, sg.w_ld), np.int8)[:, :M, :N])
     return 0, Cg, st
 
 
@@ -94,7 +94,7 @@ def run_int8(A, B, T, want_stages=True):
     Bs = ea.deinterleave(ea.download_raw(sg.b_slices, (s, sg.rows_b_padded, sg.ldk), np.int8), sg.layout)
     st = dict(s=s, nbuf=sg.nbuf, a_slices=As[:, :M, :K], b_slices=Bs[:, :N, :K],
               pad_clear=not (As[:, M:, :].any() or As[:, :, K:].any() or Bs[:, N:, :].any() or Bs[:, :, K:].any()),
-              products=ea.download_raw(sg.products, (sg.nbuf, M, N), np.int32),
+              products=ea.download_raw(sg.products, (sg.nbuf, sg.g_rows, sg.g_ld), np.int32)[:, :M, :N],
               rmax=ea.download_raw(sg.rmax, (M,), np.float64), cmax=ea.download_raw(sg.cmax, (N,), np.float64))
     return 0, Cg, st
 
@@ -134,5 +134,5 @@ def run_fast(A, B, n_mod=11, want_stages=True, trans=None):
               a_planes=ap[:, :M, :K], b_planes=bp[:, :N, :K],
               a_pad_clear=(not ap[:, M:, :].any()) and (not ap[:, :, K:].any()),
               b_pad_clear=(not bp[:, N:, :].any()) and (not bp[:, :, K:].any()),
-              w_planes=ea.download_raw(sg.w_planes, (n, M, N), np.int8))
+              w_planes=ea.download_raw(sg.w_planes, (n, sg.w_rows, sg.w_ld), np.int8)[:, :M, :N])
     return 0, Cg, st
