@@ -480,15 +480,19 @@ void hgemm_pipe_kernel(const uint16_t* __restrict__ A, const uint16_t* __restric
  * the transposed 32 x 32 tile of rows m0 + 64 wave + 32 t + lane%32, columns
  * n0 + 32 u + 8 v + 4 (lane/32) + 0..3 in registers 4v .. 4v+3. A batch of
  * products is one launch: a tile's batch index is its operand plane. */
-/* INTERIOR: the tile lies inside the matrix and its rows can move as 16-byte pieces: the
- * stores then carry no bounds and no branches, and one address serves a block.
+/* INTERIOR: the tile lies inside the matrix: the stores then carry no bounds and no
+ * branches, and one address serves a block. Rows move as 16-byte pieces whatever N is:
+ * the vector types below promise the element's alignment only (global memory takes
+ * 16-byte accesses at any 4-byte boundary), so an odd N costs no more than lines
+ * written in two parts.
  * OM: the output mode where the caller has already branched on it (-1: read out_mode_arg). */
 template <bool BF16, bool INTERIOR, int OM = -1>
 __device__ __forceinline__ void store_tile_direct(v16f_t (&acc)[pipe2::TM][pipe2::TN], int m0, int n0, int M, int N,
                                                   int out_mode_arg, void* Cout, int8_t* stage) {
     const int out_mode = OM >= 0 ? OM : out_mode_arg;      /* OM >= 0: known when compiled, nothing decided per value */
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const bool vec_f32 = (N & 3) == 0, vec_f64 = (N & 1) == 0;
+    typedef int v4iu_t __attribute__((ext_vector_type(4), aligned(4)));
+    typedef double d2u_t __attribute__((ext_vector_type(2), aligned(8)));
 #pragma unroll
     for (int t = 0; t < pipe2::TM; t++) {
         const int row0 = m0 + wave * 64 + t * 32;
@@ -521,7 +525,7 @@ __device__ __forceinline__ void store_tile_direct(v16f_t (&acc)[pipe2::TM][pipe2
 #pragma unroll
                     /* streaming: 2 per cent of the 8192^3 product (0.818 -> 0.802 ms); the fp64
                      * form below gains nothing from it */
-                    for (int i = 0; i < 4; i++) eshkol_store_streaming((v4i_t*)(p + (size_t)(8 * i) * N), w[i]);
+                    for (int i = 0; i < 4; i++) __builtin_nontemporal_store((v4iu_t)w[i], (v4iu_t*)(p + (size_t)(8 * i) * N));
                 } else {
                     pipe2::v2i_t w[8];
 #pragma unroll
@@ -529,7 +533,7 @@ __device__ __forceinline__ void store_tile_direct(v16f_t (&acc)[pipe2::TM][pipe2
                     double* p = (double*)Cout + (size_t)(row0 + (lane >> 4)) * N + cb + 2 * (lane & 15);
 #pragma unroll
                     for (int i = 0; i < 8; i++)
-                        *(d2_t*)(p + (size_t)(4 * i) * N) = (d2_t){(double)__int_as_float(w[i][0]), (double)__int_as_float(w[i][1])};
+                        *(d2u_t*)(p + (size_t)(4 * i) * N) = (d2u_t){(double)__int_as_float(w[i][0]), (double)__int_as_float(w[i][1])};
                 }
             } else if (out_mode == 0) {
 #pragma unroll
@@ -538,7 +542,7 @@ __device__ __forceinline__ void store_tile_direct(v16f_t (&acc)[pipe2::TM][pipe2
                     const int row = row0 + (lane >> 3) + 8 * i, col = cb + 4 * (lane & 7);
                     if (row < M && col < N) {
                         float* p = (float*)Cout + (size_t)row * N + col;
-                        if (vec_f32 && col + 3 < N) *(v4i_t*)p = w;
+                        if (col + 3 < N) *(v4iu_t*)p = (v4iu_t)w;
                         else for (int e = 0; e < 4; e++) if (col + e < N) p[e] = __int_as_float(w[e]);
                     }
                 }
@@ -549,7 +553,7 @@ __device__ __forceinline__ void store_tile_direct(v16f_t (&acc)[pipe2::TM][pipe2
                     const int row = row0 + (lane >> 4) + 4 * i, col = cb + 2 * (lane & 15);
                     if (row < M && col < N) {
                         double* p = (double*)Cout + (size_t)row * N + col;
-                        if (vec_f64 && col + 1 < N) *(d2_t*)p = (d2_t){(double)__int_as_float(w[0]), (double)__int_as_float(w[1])};
+                        if (col + 1 < N) *(d2u_t*)p = (d2u_t){(double)__int_as_float(w[0]), (double)__int_as_float(w[1])};
                         else for (int e = 0; e < 2; e++) if (col + e < N) p[e] = (double)__int_as_float(w[e]);
                     }
                 }
@@ -597,7 +601,7 @@ void hgemm_direct_kernel(const uint16_t* __restrict__ A, const uint16_t* __restr
     const uint64_t c_bytes = (uint64_t)M * (uint64_t)N * (out_mode == 0 ? 4u : 8u);
     auto epi = [&](v16f_t (&acc)[pipe2::TM][pipe2::TN], const pipe::Tile& t, int8_t* stage) {
         void* Ct = (int8_t*)Cout + (uint64_t)t.tag * c_bytes;
-        const bool interior = t.m0 + pipe2::BM <= M && t.n0 + pipe2::BN <= N && (N & 3) == 0 && (((uintptr_t)Ct & 15) == 0);
+        const bool interior = t.m0 + pipe2::BM <= M && t.n0 + pipe2::BN <= N;
         if (!interior) store_tile_direct<BF16, false>(acc, t.m0, t.n0, M, N, out_mode, Ct, stage);
         else if (out_mode == 0) store_tile_direct<BF16, true, 0>(acc, t.m0, t.n0, M, N, 0, Ct, stage);
         else if (out_mode == 1) store_tile_direct<BF16, true, 1>(acc, t.m0, t.n0, M, N, 1, Ct, stage);

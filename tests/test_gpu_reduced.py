@@ -40,7 +40,7 @@ def test_reduced_matches_reference_statement(gpu, M, K, N, dtype):
 
 
 @pytest.mark.parametrize("dtype", [2, 3])
-@pytest.mark.parametrize("M,K,N", [(3072, 256, 3072), (3000, 200, 2900)])
+@pytest.mark.parametrize("M,K,N", [(3072, 256, 3072), (3000, 200, 2900), (3001, 200, 2901), (3072, 256, 3073)])
 def test_rounded_output_of_the_kernel_for_large_products(gpu, M, K, N, dtype):
     """From 128 tiles of 256 x 256 on, the tier's contraction is the kernel that loads its
     operands straight into LDS and MFMA registers, with an epilogue of its own for every
@@ -214,6 +214,33 @@ def test_interleaved_contraction_config4_reduced_size(gpu):
             assert normwise(o[:64], ref, Ar[:64], Br) <= 1e-6
         if exact:
             assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0][:64], ref)
+
+
+@pytest.mark.parametrize("M,N", [(3000, 2901), (3072, 3073), (3001, 3070)])
+def test_direct_kernel_fp32_rows_that_start_off_16_byte_boundaries(gpu, M, N):
+    """fp32 results whose rows do not start on 16-byte boundaries (N not a multiple of four) leave the
+    direct kernel as 16-byte stores all the same; integer operands make every sum exact, so the result
+    must equal the integer product bit for bit, ragged edges included, and nothing may be written
+    beyond the M x N values."""
+    print("case: hip_hgemm_16_batched fp32 out", M, N, flush=True)
+    lib = ea.load()
+    K = 512
+    rng = np.random.default_rng(M + N)
+    A = rng.integers(-7, 8, (M, K)).astype(np.float64)
+    B = rng.integers(-7, 8, (K, N)).astype(np.float64)
+    dA, dB = ea.DeviceArray.from_host(A), ea.DeviceArray.from_host(B)
+    Mp, Np = (M + 255) // 256 * 256, (N + 255) // 256 * 256
+    assert lib.hip_hgemm_plane_layout(M, N, 1) == 1
+    a16, b16 = ea.DeviceArray((Mp, K), np.uint16), ea.DeviceArray((Np, K), np.uint16)
+    assert lib.hip_convert_f64_to_16_planes(dA.ptr, a16.ptr, 1, M, K, Mp, K, 1, 0, 1, stream()) == 0
+    assert lib.hip_convert_f64_to_16_planes(dB.ptr, b16.ptr, 1, N, K, Np, K, 1, 1, 1, stream()) == 0
+    guard = 64
+    dC = ea.DeviceArray.from_host(np.full(M * N + guard, -1.5, np.float32))
+    assert lib.hip_hgemm_16_batched(a16.ptr, b16.ptr, 1, M, K, N, Mp, Np, K, 1, 1, dC.ptr, stream()) == 0
+    ea.synchronize()
+    out = dC.download()
+    assert np.all(out[M * N:] == -1.5)
+    assert np.array_equal(out[:M * N].reshape(M, N).astype(np.float64), A @ B)
 
 
 def test_direct_kernel_batched_with_integer_operands(gpu):
