@@ -282,7 +282,12 @@ __device__ __forceinline__ void lds_only_barrier() {
  * workgroups of such a launch compute the tiles at positions 0 .. whole - 1 of
  * the tile order whole, as an unsplit launch of `whole` workgroups would (small
  * tiles only; 0 for large ones). */
-struct SplitArgs { int first_tile, tail, kb_per_piece; double* partial; int whole; };
+struct SplitArgs { int first_tile, tail, kb_per_piece; double* partial; int whole; int lda, ldb; };
+/* lda, ldb: row pitches of the operands as stored, in doubles; 0 for the dense pitch
+ * the shape implies. Set (by dgemm_any, under the library lock every entry point
+ * holds) when an operand was copied to an even pitch first; the launchers below put
+ * them into every SplitArgs they build. */
+int g_lda = 0, g_ldb = 0;
 
 template <bool TA, bool TB, bool KTAIL, bool SPLIT, int TS = 128, int PF = 1>
 __global__ __launch_bounds__(256, TS == 128 ? 2 : 4)
@@ -331,6 +336,7 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
     /* This thread's four 16-byte chunks of each operand tile: global pointers
      * for k-block 0. Rows beyond the matrix (edge tiles) are clamped to its last
      * rows: they load valid memory and feed outputs that are never stored. */
+    const int lda = sp.lda ? sp.lda : (TA ? M : K), ldb = sp.ldb ? sp.ldb : (TB ? K : N);
     const double* pa[OpA::CHUNKS];
     const double* pb[OpB::CHUNKS];
     /* first k of chunk r inside a k-block (recomputed where the k-tail needs it: the few
@@ -342,12 +348,12 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
         const int c = tid + 256 * r;
         if (TA) {
             int m = m0 + 2 * (c % (BM / 2));
-            m = (m < M - 2) ? m : M - 2;
-            pa[r] = A + (size_t)ka_of(r) * M + m;
+            m = (m < lda - 2) ? m : lda - 2;         /* a pair may end in the pitch's padding, not beyond it */
+            pa[r] = A + (size_t)ka_of(r) * lda + m;
         } else {
             int m = m0 + (c >> 3);
             m = (m < M - 1) ? m : M - 1;
-            pa[r] = A + (size_t)m * K + ka_of(r);
+            pa[r] = A + (size_t)m * lda + ka_of(r);
         }
     }
 #pragma unroll
@@ -356,15 +362,15 @@ void dgemm_fast_kernel(const double* __restrict__ A, const double* __restrict__ 
         if (TB) {
             int n = n0 + (c >> 3);
             n = (n < N - 1) ? n : N - 1;
-            pb[r] = B + (size_t)n * K + kbo_of(r);
+            pb[r] = B + (size_t)n * ldb + kbo_of(r);
         } else {
             int n = n0 + 2 * (c % (BN / 2));
-            n = (n < N - 2) ? n : N - 2;
-            pb[r] = B + (size_t)kbo_of(r) * N + n;
+            n = (n < ldb - 2) ? n : ldb - 2;
+            pb[r] = B + (size_t)kbo_of(r) * ldb + n;
         }
     }
-    const size_t a_step = TA ? (size_t)BK * M : (size_t)BK;     /* doubles per k-block */
-    const size_t b_step = TB ? (size_t)BK : (size_t)BK * N;
+    const size_t a_step = TA ? (size_t)BK * lda : (size_t)BK;   /* doubles per k-block */
+    const size_t b_step = TB ? (size_t)BK : (size_t)BK * ldb;
 
     OpA a[PF];
     OpB b[PF];
@@ -705,7 +711,7 @@ int launch_fast_k(const double* A, const double* B, double* C, int M, int N, int
     const int tiles_m = (M + 127) / 128, tiles_n = (N + 127) / 128;
     const long long nwg = (long long)tiles_m * tiles_n;
     if (nwg > 0x7fffffffLL || batch < 1 || batch > 65535) return -1;
-    SplitArgs sp = {0, 1, 0, nullptr, 0};
+    SplitArgs sp = {0, 1, 0, nullptr, 0, g_lda, g_ldb};
 
     /* Two workgroups fit on a CU, so a launch runs in rounds of `slots` tiles, and
      * a last round of a few tiles takes as long as a full one. Its tiles are
@@ -772,7 +778,7 @@ int launch_fast64_k(const double* A, const double* B, double* C, int M, int N, i
     const int tiles_m = (M + 63) / 64, tiles_n = (N + 63) / 64;
     const long long nwg = (long long)tiles_m * tiles_n;
     if (nwg > 0x7fffffffLL || batch < 1 || batch > 65535) return -1;
-    SplitArgs sp = {0, 1, 0, nullptr, 0};
+    SplitArgs sp = {0, 1, 0, nullptr, 0, g_lda, g_ldb};
     /* leftover tiles cut along k, in one launch with the whole ones (small_tile_tail_pieces) */
     const int nkb = (K + BK - 1) / BK;
     const int p = small_tile_tail_pieces(nwg, nkb, g_tail_split && batch == 1);
@@ -827,15 +833,12 @@ int launch(const double* A, const double* B, double* C, int M, int N, int K, int
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 
-template <bool TA, bool TB>
-int launch_shape(const double* A, const double* B, double* C, int m, int n, int k, int batch, bool vec,
-                 hipStream_t st) {
+enum class Kernel { Fast64, Fast128, General128, General64 };
+
+/* Which kernel a shape takes. */
+Kernel choose_kernel(int m, int n, int k, int batch, bool vec) {
     /* Small outputs cannot fill 256 CUs with 128x128 tiles: use 64x64 there. */
     const long long big_tiles = (long long)((m + 127) / 128) * (long long)((n + 127) / 128) * batch;
-    /* Row-major A next to a k-major B: writing A's tile k-major into LDS (so both
-     * operands are read the same way) measured 1 % faster than keeping A's rows
-     * at 8192^3; with both operands row-major the natural forms are faster. */
-    constexpr bool ALK = TA || !TB;
     /* 16-byte operand chunks (even pitches, aligned bases) and at least one whole k-block */
     const int nkb = (k + BK - 1) / BK;
     const bool may_cut = g_tail_split && batch == 1;
@@ -854,15 +857,39 @@ int launch_shape(const double* A, const double* B, double* C, int m, int n, int 
     if (straight && (g_small_tile == 2 ||
                      (g_small_tile == 1 && big_tiles < 4LL * eshkol_hip_num_cus() &&
                       small_tile_us(small_tiles, nkb, may_cut) < large_tile_us(big_tiles, nkb, may_cut))))
-        return launch_fast64<TA, TB>(A, B, C, m, n, k, batch, st);
-    if (g_fast_path && (big_tiles >= 192 || cut) && vec && m >= 2 && n >= 2 && k >= BK)
-        return launch_fast<TA, TB>(A, B, C, m, n, k, batch, st);
-    if (big_tiles >= 256) {
-        return vec ? launch<128, 128, true, TA, TB, ALK, !TB>(A, B, C, m, n, k, batch, st)
-                   : launch<128, 128, false, TA, TB, TA, !TB>(A, B, C, m, n, k, batch, st);
+        return Kernel::Fast64;
+    if (straight && (big_tiles >= 192 || cut)) return Kernel::Fast128;
+    return big_tiles >= 256 ? Kernel::General128 : Kernel::General64;
+}
+
+template <bool TA, bool TB>
+int launch_shape(const double* A, const double* B, double* C, int m, int n, int k, int batch, bool vec,
+                 hipStream_t st) {
+    /* Row-major A next to a k-major B: writing A's tile k-major into LDS (so both
+     * operands are read the same way) measured 1 % faster than keeping A's rows
+     * at 8192^3; with both operands row-major the natural forms are faster. */
+    constexpr bool ALK = TA || !TB;
+    switch (choose_kernel(m, n, k, batch, vec)) {
+        case Kernel::Fast64: return launch_fast64<TA, TB>(A, B, C, m, n, k, batch, st);
+        case Kernel::Fast128: return launch_fast<TA, TB>(A, B, C, m, n, k, batch, st);
+        case Kernel::General128:
+            return vec ? launch<128, 128, true, TA, TB, ALK, !TB>(A, B, C, m, n, k, batch, st)
+                       : launch<128, 128, false, TA, TB, TA, !TB>(A, B, C, m, n, k, batch, st);
+        default:
+            return vec ? launch<64, 64, true, TA, TB, TA, !TB>(A, B, C, m, n, k, batch, st)
+                       : launch<64, 64, false, TA, TB, TA, !TB>(A, B, C, m, n, k, batch, st);
     }
-    return vec ? launch<64, 64, true, TA, TB, TA, !TB>(A, B, C, m, n, k, batch, st)
-               : launch<64, 64, false, TA, TB, TA, !TB>(A, B, C, m, n, k, batch, st);
+}
+
+/* dst[r][c] = src[r][c] for c < cols, 0 for cols <= c < ld: an operand whose rows do
+ * not start on 16-byte boundaries (odd cols, or a base that is not aligned) copied
+ * to an even pitch. */
+__global__ __launch_bounds__(256)
+void dgemm_pad_copy_kernel(const double* __restrict__ src, double* __restrict__ dst, int rows, int cols, int ld) {
+    const int c = (int)(blockIdx.x * 256 + threadIdx.x);
+    if (c >= ld) return;
+    for (int r = (int)blockIdx.y; r < rows; r += (int)gridDim.y)
+        dst[(size_t)r * ld + c] = (c < cols) ? src[(size_t)r * cols + c] : 0.0;
 }
 
 }  // namespace
@@ -881,6 +908,52 @@ int dgemm_any(const double* A, const double* B, double* C, uint64_t M, uint64_t 
                      ((uintptr_t)A % 16 == 0) && ((uintptr_t)B % 16 == 0) &&
                      (batch == 1 || ((M * K) % 2 == 0 && (K * N) % 2 == 0));
     const int m = (int)M, n = (int)N, k = (int)K;
+    /* Operands whose rows do not start on 16-byte boundaries (an odd pitch, a base that
+     * is not aligned) would take the kernel of 8-byte loads, at two thirds of the rate
+     * (4096 x 4096 x 4097: 3.0 ms against 2.1). Where the shape would otherwise run the
+     * straight-line kernel and is large enough for two passes over an operand not to
+     * matter, the operand is copied to an even pitch first and the kernel told the
+     * pitch; the k-tail and edge logic work on the logical sizes as before, and a pair
+     * of values that straddles the end of a row ends in the copy's zero. C needs no
+     * copy: the kernel stores it value by value. */
+    if (!vec && batch == 1 && 2.0 * (double)M * (double)N * (double)K >= 4.0e9) {
+        const Kernel would = choose_kernel(m, n, k, 1, true);
+        if (would == Kernel::Fast64 || would == Kernel::Fast128) {
+            const int rows_a = trans_a ? k : m, rows_b = trans_b ? n : k;
+            const bool copy_a = (pitch_a % 2 != 0) || ((uintptr_t)A % 16 != 0);
+            const bool copy_b = (pitch_b % 2 != 0) || ((uintptr_t)B % 16 != 0);
+            const int lda = (int)(pitch_a + (pitch_a & 1)), ldb = (int)(pitch_b + (pitch_b & 1));
+            const double* a2 = A;
+            const double* b2 = B;
+            bool ok = pitch_a < 0x7fffffffULL && pitch_b < 0x7fffffffULL;
+            if (ok && copy_a) {
+                double* w = (double*)eshkol_hip_workspace(WS_DGEMM_PAD_A, (size_t)rows_a * lda * sizeof(double));
+                if (w) {
+                    hipLaunchKernelGGL(dgemm_pad_copy_kernel, dim3((unsigned)((lda + 255) / 256), (unsigned)(rows_a < 65535 ? rows_a : 65535)),
+                                       dim3(256), 0, st, A, w, rows_a, (int)pitch_a, lda);
+                    a2 = w;
+                } else ok = false;
+            }
+            if (ok && copy_b) {
+                double* w = (double*)eshkol_hip_workspace(WS_DGEMM_PAD_B, (size_t)rows_b * ldb * sizeof(double));
+                if (w) {
+                    hipLaunchKernelGGL(dgemm_pad_copy_kernel, dim3((unsigned)((ldb + 255) / 256), (unsigned)(rows_b < 65535 ? rows_b : 65535)),
+                                       dim3(256), 0, st, B, w, rows_b, (int)pitch_b, ldb);
+                    b2 = w;
+                } else ok = false;
+            }
+            if (ok) {
+                g_lda = copy_a ? lda : 0;
+                g_ldb = copy_b ? ldb : 0;
+                int rc;
+                if (trans_a) rc = launch_shape<true, false>(a2, b2, C, m, n, k, 1, true, st);
+                else if (trans_b) rc = launch_shape<false, true>(a2, b2, C, m, n, k, 1, true, st);
+                else rc = launch_shape<false, false>(a2, b2, C, m, n, k, 1, true, st);
+                g_lda = 0; g_ldb = 0;
+                return rc;
+            }
+        }
+    }
     /* the grid's y extent is limited to 65535 */
     for (uint64_t done = 0; done < batch; ) {
         const int nb = (int)((batch - done < 65535) ? batch - done : 65535);

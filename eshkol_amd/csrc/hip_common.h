@@ -36,6 +36,8 @@ enum {
     WS_F32_C,
     WS_COLPARTIAL,  /* per-slice partial column maxima                       */
     WS_DGEMM_PARTIAL, /* partial tiles of a k-split last round of the fp64 GEMM */
+    WS_DGEMM_PAD_A, /* copies of fp64 operands whose rows do not start on 16-byte  */
+    WS_DGEMM_PAD_B, /* boundaries, at an even pitch                                */
     WS_MISC,
     WS_COUNT
 };

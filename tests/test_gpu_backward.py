@@ -185,3 +185,38 @@ def test_full_size_backward_properties(gpu):
     assert np.array_equal(gA[rows], G[rows] @ B.T)
     cols = [0, 1, 127, 128, 777, N - 1]
     assert np.array_equal(gB[:, cols], A.T @ G[:, cols])
+
+
+@pytest.mark.parametrize("M,K,N", [(1537, 1601, 1409), (2049, 1024, 2047), (2048, 1025, 2048), (1409, 2001, 1538)])
+def test_native_large_operands_with_rows_off_16_byte_boundaries(gpu, M, K, N):
+    """Large products whose operands have an odd pitch are copied to an even one and run the straight-line
+    kernel with that pitch. Small integers make every sum exact, so all three operand forms must give the
+    integer product bit for bit, edges included; random operands must stay within the tier's tolerance."""
+    print("dgemm_ex, odd pitches", M, K, N, flush=True)
+    rng = np.random.default_rng(M + K + N)
+    A = rng.integers(-9, 10, (M, K)).astype(np.float64)
+    B = rng.integers(-9, 10, (K, N)).astype(np.float64)
+    ref = A @ B
+    At, Bt = np.ascontiguousarray(A.T), np.ascontiguousarray(B.T)
+    assert np.array_equal(dgemm_ex(A, B, M, K, N, 0, 0), ref)
+    assert np.array_equal(dgemm_ex(A, Bt, M, K, N, 0, 1), ref)
+    assert np.array_equal(dgemm_ex(At, B, M, K, N, 1, 0), ref)
+    A, B = synth.uniform(100 + M, (M, K)), synth.uniform(200 + N, (K, N))
+    rows = np.array([0, 1, M // 2, M - 2, M - 1])
+    got = dgemm_ex(A, B, M, K, N, 0, 0)
+    assert normwise(got[rows], oracle.matmul_f64(A[rows], B), A[rows], B) <= TOL
+    assert normwise(got, A @ B, A, B) <= TOL
+
+
+def test_native_large_operands_with_a_base_off_16_byte_boundaries(gpu):
+    """Even pitches, but the operands start 8 bytes into their buffers."""
+    M, K, N = 1536, 1600, 1408
+    rng = np.random.default_rng(3)
+    A = rng.integers(-9, 10, (M, K)).astype(np.float64)
+    B = rng.integers(-9, 10, (K, N)).astype(np.float64)
+    bufA = ea.DeviceArray.from_host(np.concatenate([[777.0], A.ravel()]))
+    bufB = ea.DeviceArray.from_host(np.concatenate([[777.0], B.ravel()]))
+    dC = ea.DeviceArray((M, N))
+    assert ea.load().hip_dgemm_f64_ex(bufA.ptr + 8, bufB.ptr + 8, dC.ptr, M, K, N, 0, 0, stream()) == 0
+    ea.synchronize()
+    assert np.array_equal(dC.download(), A @ B)
