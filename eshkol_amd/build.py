@@ -24,6 +24,7 @@ SOURCES = [
     "gpu_memory_hip.cpp",
     "host_copy.cpp",
     "dgemm_f64.hip",
+    "dgemv_f64.hip",
     "sgemm_f32.hip",
     "igemm_i8.hip",
     "hgemm_16.hip",

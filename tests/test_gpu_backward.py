@@ -220,3 +220,45 @@ def test_native_large_operands_with_a_base_off_16_byte_boundaries(gpu):
     assert ea.load().hip_dgemm_f64_ex(bufA.ptr + 8, bufB.ptr + 8, dC.ptr, M, K, N, 0, 0, stream()) == 0
     ea.synchronize()
     assert np.array_equal(dC.download(), A @ B)
+
+
+@pytest.mark.parametrize("thin", [1, 2, 3, 5, 8, 9, 16])
+@pytest.mark.parametrize("wide,K", [(1024, 1024), (1025, 1031), (4096, 100), (3001, 2050), (2, 1 << 19)])
+def test_native_products_with_one_thin_side(gpu, thin, wide, K):
+    """A vector or a few against a matrix (M or N at most 16) take kernels of their own, bound by HBM, in all
+    three operand forms and with either side thin. Integer operands make every sum exact, so the result must
+    be the integer product bit for bit; random operands must stay within the tier's tolerance."""
+    if wide < 1024 and thin > 2:
+        pytest.skip("the wide side here only serves as a shape the thin kernels must leave alone")
+    print("dgemm_ex, thin side", thin, wide, K, flush=True)
+    rng = np.random.default_rng(thin * 7 + wide + K)
+    for (M, N) in ((thin, wide), (wide, thin)):
+        A = rng.integers(-9, 10, (M, K)).astype(np.float64)
+        B = rng.integers(-9, 10, (K, N)).astype(np.float64)
+        ref = A @ B
+        At, Bt = np.ascontiguousarray(A.T), np.ascontiguousarray(B.T)
+        assert np.array_equal(dgemm_ex(A, B, M, K, N, 0, 0), ref)
+        assert np.array_equal(dgemm_ex(A, Bt, M, K, N, 0, 1), ref)
+        assert np.array_equal(dgemm_ex(At, B, M, K, N, 1, 0), ref)
+        A, B = synth.uniform(100 + M, (M, K)), synth.uniform(200 + N, (K, N))
+        ref = oracle.matmul_f64(A, B) if M * N * K <= (1 << 27) else A @ B
+        At, Bt = np.ascontiguousarray(A.T), np.ascontiguousarray(B.T)
+        assert normwise(dgemm_ex(A, B, M, K, N, 0, 0), ref, A, B) <= TOL
+        assert normwise(dgemm_ex(A, Bt, M, K, N, 0, 1), ref, A, B) <= TOL
+        assert normwise(dgemm_ex(At, B, M, K, N, 1, 0), ref, A, B) <= TOL
+
+
+def test_native_thin_products_write_nothing_else(gpu):
+    """The result of a thin product lies in a buffer with guard values around it."""
+    lib = ea.load()
+    for (M, K, N) in ((3, 777, 2049), (2049, 777, 3), (1, 4096, 4097), (4097, 4096, 1)):
+        rng = np.random.default_rng(M + N)
+        A = rng.integers(-9, 10, (M, K)).astype(np.float64)
+        B = rng.integers(-9, 10, (K, N)).astype(np.float64)
+        dA, dB = dev(A), dev(B)
+        buf = ea.DeviceArray.from_host(np.full(M * N + 128, -7.25))
+        assert lib.hip_dgemm_f64(dA.ptr, dB.ptr, buf.ptr + 64 * 8, M, K, N, stream()) == 0
+        ea.synchronize()
+        out = buf.download()
+        assert np.all(out[:64] == -7.25) and np.all(out[64 + M * N:] == -7.25)
+        assert np.array_equal(out[64:64 + M * N].reshape(M, N), A @ B)
