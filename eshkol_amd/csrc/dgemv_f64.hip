@@ -1,6 +1,7 @@
 /*
  * fp64 products with one thin side: C[M x N] = A[M x K] * B[K x N] where M or N is
- * at most 8 (a vector or a handful of vectors against a matrix). Behind the same
+ * small (a vector or a handful of vectors against a matrix: up to 8, or up to 32 where
+ * the big operand has the output index contiguous). Behind the same
  * entry points as the matrix-core GEMM (hip_dgemm_f64 / hip_dgemm_f64_ex), which
  * replace cublasDgemm (lib/backend/gpu/gpu_memory_cuda.cpp:611-650) for every shape.
  *
@@ -15,8 +16,8 @@
  *   big[K][O], the output index contiguous (B as given with M thin; A held transposed
  *   with N thin). A lane owns two adjacent outputs o and reads 16 bytes of every row k;
  *   the thin operand's value for (s, k) is the same for the whole wave: a scalar load.
- *   The four waves of a workgroup take every fourth k of the workgroup's k-range and
- *   add up through LDS; workgroups split K further where O alone cannot fill the
+ *   The four waves of a workgroup take groups of four k of the workgroup's k-range in
+ *   turn and add up through LDS; workgroups split K further where O alone cannot fill the
  *   device, each leaving a partial result that a second kernel adds in a fixed order.
  *
  *   big[O][K], k contiguous (A as given with N thin; B held transposed with M thin). A
@@ -50,7 +51,8 @@ __global__ __launch_bounds__(256)
 void skinny_kfirst_kernel(const double* __restrict__ big, long ldb, int K, int O,
                           const double* __restrict__ thin, long ts, long tk, int S,
                           double* __restrict__ C, long cs, long co, double* __restrict__ part, int kchunk) {
-    __shared__ double red[3][SP][COLS_PER_WG];
+    constexpr int RB = SP < 16 ? SP : 16;
+    __shared__ double red[3][RB][COLS_PER_WG];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int o = (int)blockIdx.x * COLS_PER_WG + 2 * lane;
@@ -78,34 +80,41 @@ void skinny_kfirst_kernel(const double* __restrict__ big, long ldb, int K, int O
             if (O >= 2) { const d2u_t v = *(const d2u_t*)(bp + (long)(k + i) * ldb); b0[i] = v.x; b1[i] = v.y; }
             else { b0[i] = big[(long)(k + i) * ldb]; b1[i] = 0.0; }
         }
-        double a[SP][4];                        /* the same for every lane: scalar loads */
-        if (CONTIG == 1) {
+        /* the thin operand's values are the same for every lane: scalar loads, eight s at a
+         * time (more than 64 scalar registers of them at once and the compiler spills) */
+        constexpr int SB = SP < 8 ? SP : 8;
 #pragma unroll
-            for (int s = 0; s < SP; s++) {
-                const double* t = thin + (long)(s < S ? s : 0) * ts + k;
+        for (int s0 = 0; s0 < SP; s0 += SB) {
+            double a[SB][4];
+            if (CONTIG == 1) {
 #pragma unroll
-                for (int i = 0; i < 4; i++) a[s][i] = (s < S) ? t[i] : 0.0;
+                for (int s = 0; s < SB; s++) {
+                    const double* t = thin + (long)(s0 + s < S ? s0 + s : 0) * ts + k;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) a[s][i] = (s0 + s < S) ? t[i] : 0.0;
+                }
+            } else if (CONTIG == 2) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const double* t = thin + (long)(k + i) * tk + s0;
+#pragma unroll
+                    for (int s = 0; s < SB; s++) a[s][i] = t[s];
+                }
+            } else {
+#pragma unroll
+                for (int s = 0; s < SB; s++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) a[s][i] = (s0 + s < S) ? thin[(long)(s0 + s) * ts + (long)(k + i) * tk] : 0.0;
             }
-        } else if (CONTIG == 2) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const double* t = thin + (long)(k + i) * tk;
+            for (int i = 0; i < 4; i++)
 #pragma unroll
-                for (int s = 0; s < SP; s++) a[s][i] = t[s];
-            }
-        } else {
-#pragma unroll
-            for (int s = 0; s < SP; s++)
-#pragma unroll
-                for (int i = 0; i < 4; i++) a[s][i] = (s < S) ? thin[(long)s * ts + (long)(k + i) * tk] : 0.0;
+                for (int s = 0; s < SB; s++) {
+                    acc0[s0 + s] = fma(a[s][i], b0[i], acc0[s0 + s]);
+                    acc1[s0 + s] = fma(a[s][i], b1[i], acc1[s0 + s]);
+                }
+            if (SP > SB) __builtin_amdgcn_sched_barrier(0);
         }
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-#pragma unroll
-            for (int s = 0; s < SP; s++) {
-                acc0[s] = fma(a[s][i], b0[i], acc0[s]);
-                acc1[s] = fma(a[s][i], b1[i], acc1[s]);
-            }
     }
     /* what is left of a k-range that is not a multiple of four: its owner is the wave whose turn it is */
     if (k < k_hi) {
@@ -123,29 +132,42 @@ void skinny_kfirst_kernel(const double* __restrict__ big, long ldb, int K, int O
     }
     /* a lane clamped to the last pair holds that pair's sums: only o == O - 1 of an odd O
      * is a real output among them, and it is the pair's second value */
-    if (wave > 0) {
-#pragma unroll
-        for (int s = 0; s < SP; s++) { red[wave - 1][s][2 * lane] = acc0[s]; red[wave - 1][s][2 * lane + 1] = acc1[s]; }
-    }
-    __syncthreads();
-    if (wave != 0 || !one) return;
     const bool shifted = !two && O >= 2;          /* this lane's o is O - 1, held as the second value of the clamped pair */
 #pragma unroll
-    for (int s = 0; s < SP; s++) {
-        if (s >= S) break;
-        double r0 = acc0[s], r1 = acc1[s];
+    for (int s0 = 0; s0 < SP; s0 += RB) {         /* through LDS, at most sixteen s at a time */
+        if (s0 > 0) __syncthreads();
+        if (wave > 0) {
 #pragma unroll
-        for (int w = 0; w < 3; w++) { r0 += red[w][s][2 * lane]; r1 += red[w][s][2 * lane + 1]; }
-        if (shifted) r0 = r1;
-        if (gridDim.y == 1) {
-            C[(long)s * cs + (long)o * co] = r0;
-            if (two) C[(long)s * cs + (long)(o + 1) * co] = r1;
-        } else {
-            double* p = part + ((size_t)blockIdx.y * S + s) * (size_t)O + o;
-            p[0] = r0;
-            if (two) p[1] = r1;
+            for (int s = 0; s < RB; s++) { red[wave - 1][s][2 * lane] = acc0[s0 + s]; red[wave - 1][s][2 * lane + 1] = acc1[s0 + s]; }
+        }
+        __syncthreads();
+        if (wave == 0 && one) {
+#pragma unroll
+            for (int s = 0; s < RB; s++) {
+                if (s0 + s >= S) break;
+                double r0 = acc0[s0 + s], r1 = acc1[s0 + s];
+#pragma unroll
+                for (int w = 0; w < 3; w++) { r0 += red[w][s][2 * lane]; r1 += red[w][s][2 * lane + 1]; }
+                if (shifted) r0 = r1;
+                if (gridDim.y == 1) {
+                    C[(long)(s0 + s) * cs + (long)o * co] = r0;
+                    if (two) C[(long)(s0 + s) * cs + (long)(o + 1) * co] = r1;
+                } else {
+                    double* p = part + ((size_t)blockIdx.y * S + s0 + s) * (size_t)O + o;
+                    p[0] = r0;
+                    if (two) p[1] = r1;
+                }
+            }
         }
     }
+}
+
+/* dst[k][s] = src[s * ts + k]: the thin operand from rows of k to dense [K][S] */
+__global__ __launch_bounds__(256)
+void skinny_thin_to_dense_kernel(const double* __restrict__ src, long ts, int S, int K, double* __restrict__ dst) {
+    const int k = (int)(blockIdx.x * 256 + threadIdx.x);
+    if (k >= K) return;
+    for (int s = 0; s < S; s++) dst[(size_t)k * S + s] = src[(long)s * ts + k];
 }
 
 /* C(s, o) = sum over pieces y of part[(y * S + s) * O + o], y ascending */
@@ -295,11 +317,12 @@ int launch_klast(const double* big, long ldb, int O, int K, const double* thin, 
 bool eshkol_hip_dgemm_is_skinny(uint64_t M, uint64_t K, uint64_t N, int trans_a, int trans_b) {
     const uint64_t thin = M < N ? M : N, wide = M < N ? N : M;
     if (thin == 0 || wide < 1024 || K < 64 || K > 0x7fffffffULL || wide > 0x7fffffffULL) return false;
-    (void)trans_a; (void)trans_b;
-    /* up to eight thin rows or columns: from nine on the scalar loads of the first kernel and
-     * the registers of the second fall behind the tiled kernel (16 x 8192 x 8192: 0.31 ms
-     * against 0.27) */
-    return thin <= 8 && wide * K >= (1ull << 20);
+    /* The kernel for k-contiguous big operands holds R x S sums per lane and is out of
+     * registers after eight thin columns; the other one carries up to thirty-two thin rows
+     * (3 TB/s at 32 x 8192 x 8192, where the tiled kernel reaches 2), from seventeen on only
+     * where the big operand is large enough for the difference to show. */
+    const uint64_t limit = !kfirst ? 8u : (wide * K >= (1ull << 24)) ? 32u : 16u;
+    return thin <= limit && wide * K >= (1ull << 20);
 }
 
 /* C = op(A) op(B) for a product eshkol_hip_dgemm_is_skinny() accepts. */
@@ -315,13 +338,24 @@ int eshkol_hip_dgemm_skinny(const double* A, const double* B, double* C, uint64_
     else        { ts = trans_b ? (long)K : 1; tk = trans_b ? 1 : (long)N; cs = 1; co = (long)N; }
     const bool kfirst = thin_m ? !trans_b : (trans_a != 0);
     const long ldb = kfirst ? (long)O : (long)K;
-    const int sp = S <= 1 ? 1 : S <= 2 ? 2 : S <= 4 ? 4 : 8;
+    const int sp = S <= 1 ? 1 : S <= 2 ? 2 : S <= 4 ? 4 : S <= 8 ? 8 : S <= 16 ? 16 : 32;
+    if (kfirst && sp >= 16 && tk == 1) {
+        /* From nine thin rows of k on: sixteen streams of scalar loads, one per row, run at
+         * less than half the rate of the same values held densely as [K][S] (16 x 8192 x 8192:
+         * 0.29 ms against 0.12): a megabyte, transposed first. */
+        double* dense = (double*)eshkol_hip_workspace(WS_DGEMM_PAD_A, (size_t)K * S * sizeof(double));
+        if (!dense) return -1;
+        hipLaunchKernelGGL(skinny_thin_to_dense_kernel, dim3((unsigned)((k + 255) / 256)), dim3(256), 0, st, thin, ts, S, k, dense);
+        thin = dense; ts = 1; tk = S;
+    }
     if (kfirst) {
         switch (sp) {
             case 1: return launch_kfirst<1>(big, ldb, k, O, thin, ts, tk, S, C, cs, co, st);
             case 2: return launch_kfirst<2>(big, ldb, k, O, thin, ts, tk, S, C, cs, co, st);
             case 4: return launch_kfirst<4>(big, ldb, k, O, thin, ts, tk, S, C, cs, co, st);
-            default: return launch_kfirst<8>(big, ldb, k, O, thin, ts, tk, S, C, cs, co, st);
+            case 8: return launch_kfirst<8>(big, ldb, k, O, thin, ts, tk, S, C, cs, co, st);
+            case 16: return launch_kfirst<16>(big, ldb, k, O, thin, ts, tk, S, C, cs, co, st);
+            default: return launch_kfirst<32>(big, ldb, k, O, thin, ts, tk, S, C, cs, co, st);
         }
     }
     /* the thin operand with k last: k contiguous (tk == 1), or dense [K][S] (ts == 1, tk == S) */

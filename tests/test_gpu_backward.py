@@ -222,8 +222,8 @@ def test_native_large_operands_with_a_base_off_16_byte_boundaries(gpu):
     assert np.array_equal(dC.download(), A @ B)
 
 
-@pytest.mark.parametrize("thin", [1, 2, 3, 5, 8, 9, 16])
-@pytest.mark.parametrize("wide,K", [(1024, 1024), (1025, 1031), (4096, 100), (3001, 2050), (2, 1 << 19)])
+@pytest.mark.parametrize("thin", [1, 2, 3, 5, 8, 9, 16, 17, 32])
+@pytest.mark.parametrize("wide,K", [(1024, 1024), (1025, 1031), (4096, 100), (3001, 2050), (4097, 4100), (2, 1 << 19)])
 def test_native_products_with_one_thin_side(gpu, thin, wide, K):
     """A vector or a few against a matrix (M or N at most 16) take kernels of their own, bound by HBM, in all
     three operand forms and with either side thin. Integer operands make every sum exact, so the result must
