@@ -223,13 +223,11 @@ def test_native_large_operands_with_a_base_off_16_byte_boundaries(gpu):
 
 
 @pytest.mark.parametrize("thin", [1, 2, 3, 5, 8, 9, 16, 17, 32])
-@pytest.mark.parametrize("wide,K", [(1024, 1024), (1025, 1031), (4096, 100), (3001, 2050), (4097, 4100), (2, 1 << 19)])
+@pytest.mark.parametrize("wide,K", [(1024, 1024), (1025, 1031), (4096, 100), (3001, 2050), (4097, 4100)])
 def test_native_products_with_one_thin_side(gpu, thin, wide, K):
     """A vector or a few against a matrix (M or N at most 16) take kernels of their own, bound by HBM, in all
     three operand forms and with either side thin. Integer operands make every sum exact, so the result must
     be the integer product bit for bit; random operands must stay within the tier's tolerance."""
-    if wide < 1024 and thin > 2:
-        pytest.skip("the wide side here only serves as a shape the thin kernels must leave alone")
     print("dgemm_ex, thin side", thin, wide, K, flush=True)
     rng = np.random.default_rng(thin * 7 + wide + K)
     for (M, N) in ((thin, wide), (wide, thin)):
@@ -246,6 +244,17 @@ def test_native_products_with_one_thin_side(gpu, thin, wide, K):
         assert normwise(dgemm_ex(A, B, M, K, N, 0, 0), ref, A, B) <= TOL
         assert normwise(dgemm_ex(A, Bt, M, K, N, 0, 1), ref, A, B) <= TOL
         assert normwise(dgemm_ex(At, B, M, K, N, 1, 0), ref, A, B) <= TOL
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 1 << 19, 2), (2, 1 << 19, 2), (2, 1 << 19, 1), (3, 70000, 900)])
+def test_native_products_thin_on_both_sides_keep_the_tiled_kernel(gpu, M, K, N):
+    """Neither side is wide: not a shape for the thin kernels; the result must not care."""
+    rng = np.random.default_rng(M + N)
+    A = rng.integers(-9, 10, (M, K)).astype(np.float64)
+    B = rng.integers(-9, 10, (K, N)).astype(np.float64)
+    assert np.array_equal(dgemm_ex(A, B, M, K, N, 0, 0), A @ B)
+    assert np.array_equal(dgemm_ex(A, np.ascontiguousarray(B.T), M, K, N, 0, 1), A @ B)
+    assert np.array_equal(dgemm_ex(np.ascontiguousarray(A.T), B, M, K, N, 1, 0), A @ B)
 
 
 def test_native_thin_products_write_nothing_else(gpu):
