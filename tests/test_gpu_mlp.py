@@ -25,9 +25,11 @@ def forward(X, layers):
     return outs
 
 
-def test_mlp_reduced_size(gpu):
-    dims = [64, 256, 256, 64]
-    X = synth.normal(1, (128, dims[0]))
+@pytest.mark.parametrize("batch,dims", [(128, [64, 256, 256, 64]), (130, [63, 255, 129, 65]), (37, [100, 1030, 77, 3])])
+def test_mlp_reduced_size(gpu, batch, dims):
+    """Layer sizes that are multiples of four, and sizes that are multiples of nothing (rows of the
+    activations off 16-byte boundaries, a last group of columns that is not whole)."""
+    X = synth.normal(1, (batch, dims[0]))
     layers = [(synth.xavier_uniform(10 + i, dims[i], dims[i + 1]), synth.uniform(20 + i, (dims[i + 1],), -0.05, 0.05))
               for i in range(3)]
     outs = forward(X, layers)
