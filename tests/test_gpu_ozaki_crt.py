@@ -140,6 +140,45 @@ def test_full_size_config3_sampled(gpu):
     assert st["a_pad_clear"] and st["b_pad_clear"]
 
 
+@pytest.mark.parametrize("M,K,N", [(3001, 1030, 3005), (4095, 515, 4097), (2303, 2049, 2561)])
+def test_large_sizes_that_are_multiples_of_nothing_sampled(gpu, M, K, N):
+    """Products large enough for the kernels that load straight into LDS and MFMA registers, with
+    sizes that end inside a tile in every dimension and an N that puts C's rows off 16-byte
+    boundaries: the product planes then have a pitch of their own. Sampled rows and columns, the
+    edges among them, against the oracle run on those rows and columns; every residue product
+    recomputed from the device's own planes with exact integers."""
+    print("crt ragged", M, K, N, flush=True)
+    A = synth.wide_range(41 + M, (M, K)); B = synth.wide_range(42 + N, (K, N))
+    rc, Cg, st = run_crt(A, B)
+    assert rc == 0 and st["num_moduli"] == 16
+    rows = [0, 1, 255, 256, M // 2 + 1, M - 257, M - 2, M - 1]
+    cols = [0, 3, 255, 256, N // 2, N - 256, N - 2, N - 1]
+    so = oracle.ozaki_crt_stages(A[rows], B[:, cols])
+    assert so["E"] == st["E"]
+    assert np.array_equal(st["mu"][rows], so["mu"]) and np.array_equal(st["nu"][cols], so["nu"])
+    assert np.array_equal(st["a_planes"][:, rows, :], so["a_planes"])
+    assert np.array_equal(st["b_planes"][:, cols, :], so["b_planes"])
+    assert st["a_pad_clear"] and st["b_pad_clear"]
+    assert np.array_equal(st["w_planes"][:, rows][:, :, cols], so["w_planes"])
+    assert ulp_distance(Cg[rows][:, cols], so["C"]).max() <= MAX_ULP
+    for l, p in enumerate(oracle.MODULI):            # every element of every plane, exactly
+        acc = st["a_planes"][l].astype(np.float64) @ st["b_planes"][l].astype(np.float64).T
+        w = st["w_planes"][l].astype(np.int64)
+        assert np.all((acc.astype(np.int64) - w) % p == 0) and w.min() >= -(p // 2) and w.max() <= (p - 1) // 2
+    # The whole result against the oracle's own product is too slow here. With the aligned weights
+    # (the reference's own lose low bits in the weighted sum) the tier is exact on small integers,
+    # which checks every element of C, edges included.
+    import eshkol_amd as ea
+    rng = np.random.default_rng(M)
+    Ai = rng.integers(-50, 51, (M, K)).astype(np.float64); Bi = rng.integers(-50, 51, (K, N)).astype(np.float64)
+    was = ea.load().hip_ozaki_crt_set_aligned_weights(1)
+    try:
+        rc, Ci, _ = run_crt(Ai, Bi, want_stages=False)
+    finally:
+        ea.load().hip_ozaki_crt_set_aligned_weights(was)
+    assert rc == 0 and np.array_equal(Ci, Ai @ Bi)
+
+
 def both_bookkeeping_paths(A, B, **kw):
     """The device scan with a handful of host log2 calls, and the host pass over every
     maximum, must give the same E, shifts, planes and result; returns the first."""
