@@ -143,3 +143,25 @@ def test_error_stays_inside_the_tolerance_the_budget_selector_assumes(gpu, n_mod
         err = np.abs((Cg - ref).astype(np.float64))
         scale = np.linalg.norm(A, axis=1)[:, None] * np.linalg.norm(B, axis=0)[None, :]
         assert (err / scale).max() <= tol, (n_mod, E.value, float((err / scale).max()), tol)
+
+
+@pytest.mark.parametrize("M,K,N", [(3001, 1030, 3005), (4095, 515, 4097)])
+def test_large_sizes_that_are_multiples_of_nothing_sampled(gpu, M, K, N):
+    """Sizes that end inside a tile in every dimension, with an N that puts C's rows off 16-byte
+    boundaries (the product planes then have a pitch of their own): every residue product recomputed
+    from the device's own planes with exact integers, and sampled rows and columns against the oracle."""
+    print("fast ragged", M, K, N, flush=True)
+    A = synth.wide_range(45 + M, (M, K)); B = synth.wide_range(46 + N, (K, N))
+    rc, Cg, st = run_fast(A, B, 11)
+    assert rc == 0
+    for l, p in enumerate(st["moduli"]):
+        acc = st["a_planes"][l].astype(np.float64) @ st["b_planes"][l].astype(np.float64).T
+        w = st["w_planes"][l].astype(np.int64)
+        assert np.all((acc.astype(np.int64) - w) % p == 0) and np.abs(w).max() <= p // 2 + (p % 2 == 0), l
+    rows = [0, 1, 255, 256, M // 2 + 1, M - 257, M - 2, M - 1]
+    cols = [0, 3, 255, 256, N // 2, N - 256, N - 2, N - 1]
+    rc, Cs, _ = run_fast(A[rows], B[:, cols], 11)
+    assert rc == 0
+    # every stage is local to a row of A or a column of B once E is fixed by K and the moduli count
+    assert np.array_equal(Cg[rows][:, cols], Cs)
+    check_all_stages(np.ascontiguousarray(A[rows]), np.ascontiguousarray(B[:, cols]))

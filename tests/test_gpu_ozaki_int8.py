@@ -80,3 +80,30 @@ def test_full_size_sampled(gpu):
     assert np.array_equal(st["products"][:, rows][:, :, cols], so["products"])
     assert ulp_distance(Cg[rows][:, cols], so["C"]).max() <= 2
     assert st["pad_clear"]
+
+
+@pytest.mark.parametrize("M,K,N,T", [(3001, 1030, 3005, 6), (4095, 515, 4097, 4)])
+def test_large_sizes_that_are_multiples_of_nothing_sampled(gpu, M, K, N, T):
+    """Sizes that end inside a tile in every dimension, with an N that puts C's rows off 16-byte
+    boundaries (the int32 product buffers then have a pitch of their own): sampled rows and columns,
+    the edges among them, against the oracle run on those rows and columns."""
+    print("int8 ragged", M, K, N, T, flush=True)
+    A, B = synth.normal(43 + M, (M, K)), synth.normal(44 + N, (K, N))
+    rc, Cg, st = run_int8(A, B, T)
+    assert rc == 0
+    rows = [0, 1, 255, 256, M // 2 + 1, M - 257, M - 2, M - 1]
+    cols = [0, 3, 255, 256, N // 2, N - 256, N - 2, N - 1]
+    so = oracle.ozaki_int8_stages(A[rows], B[:, cols], T)
+    assert np.array_equal(st["rmax"][rows], so["rmax"]) and np.array_equal(st["cmax"][cols], so["cmax"])
+    assert np.array_equal(st["a_slices"][:, rows, :], so["a_slices"])
+    assert np.array_equal(st["b_slices"][:, cols, :], so["b_slices"])
+    assert np.array_equal(st["products"][:, rows][:, :, cols], so["products"])
+    assert ulp_distance(Cg[rows][:, cols], so["C"]).max() <= 2
+    assert st["pad_clear"]
+    # every element: the same slices multiplied in float64 (exact: the sums stay far below 2^53)
+    plan = so["plan"]
+    for b in range(st["nbuf"]):
+        lo, hi = plan["first"][b], plan["first"][b + 1]
+        acc = sum(st["a_slices"][plan["pair_p"][t]].astype(np.float64) @ st["b_slices"][plan["pair_q"][t]].astype(np.float64).T
+                  for t in range(lo, hi))
+        assert np.array_equal(acc.astype(np.int64), st["products"][b].astype(np.int64)), b
