@@ -25,6 +25,7 @@ SOURCES = [
     "host_copy.cpp",
     "dgemm_f64.hip",
     "dgemv_f64.hip",
+    "dgemm_small_f64.hip",
     "sgemm_f32.hip",
     "igemm_i8.hip",
     "hgemm_16.hip",

@@ -908,6 +908,9 @@ int dgemm_any(const double* A, const double* B, double* C, uint64_t M, uint64_t 
                      ((uintptr_t)A % 16 == 0) && ((uintptr_t)B % 16 == 0) &&
                      (batch == 1 || ((M * K) % 2 == 0 && (K * N) % 2 == 0));
     const int m = (int)M, n = (int)N, k = (int)K;
+    /* matrices far smaller than a tile, one or many: several to a workgroup (dgemm_small_f64.hip) */
+    if (g_fast_path && eshkol_hip_dgemm_is_small(M, K, N))
+        return eshkol_hip_dgemm_small(A, B, C, M, K, N, trans_a, trans_b, batch, st);
     /* a vector or a few against a matrix: bound by HBM, not by the matrix cores (dgemv_f64.hip) */
     if (g_fast_path && batch == 1 && eshkol_hip_dgemm_is_skinny(M, K, N, trans_a, trans_b))
         return eshkol_hip_dgemm_skinny(A, B, C, M, K, N, trans_a, trans_b, st);

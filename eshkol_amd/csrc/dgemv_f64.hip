@@ -321,6 +321,8 @@ bool eshkol_hip_dgemm_is_skinny(uint64_t M, uint64_t K, uint64_t N, int trans_a,
      * registers after eight thin columns; the other one carries up to thirty-two thin rows
      * (3 TB/s at 32 x 8192 x 8192, where the tiled kernel reaches 2), from seventeen on only
      * where the big operand is large enough for the difference to show. */
+    const bool thin_m = M <= N;
+    const bool kfirst = thin_m ? !trans_b : (trans_a != 0);     /* the big operand has the output index contiguous */
     const uint64_t limit = !kfirst ? 8u : (wide * K >= (1ull << 24)) ? 32u : 16u;
     return thin <= limit && wide * K >= (1ull << 20);
 }

@@ -114,6 +114,11 @@ static inline uint64_t eshkol_product_pitch(uint64_t N) { return N >= 1024 ? rou
  * themselves or with their neighbours in the wave: 8-byte pieces of a line sent
  * this way are not merged on the way out (the slice tier's reconstruction ran
  * twice as long with them). */
+/* fp64 products of matrices far smaller than a tile, one or a batch (dgemm_small_f64.hip) */
+bool eshkol_hip_dgemm_is_small(uint64_t M, uint64_t K, uint64_t N);
+int eshkol_hip_dgemm_small(const double* A, const double* B, double* C, uint64_t M, uint64_t K, uint64_t N,
+                           int trans_a, int trans_b, uint64_t batch, hipStream_t st);
+
 /* fp64 products with one thin side (dgemv_f64.hip): whether the shape is one, and the
  * product itself. hip_dgemm_f64 and hip_dgemm_f64_ex send such shapes there. */
 bool eshkol_hip_dgemm_is_skinny(uint64_t M, uint64_t K, uint64_t N, int trans_a, int trans_b);

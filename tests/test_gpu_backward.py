@@ -271,3 +271,37 @@ def test_native_thin_products_write_nothing_else(gpu):
         out = buf.download()
         assert np.all(out[:64] == -7.25) and np.all(out[64 + M * N:] == -7.25)
         assert np.array_equal(out[64:64 + M * N].reshape(M, N), A @ B)
+
+
+@pytest.mark.parametrize("batch,M,K,N", [(1, 1, 1, 1), (1, 3, 3, 3), (7, 3, 3, 3), (4096, 8, 8, 8), (1000, 5, 7, 6), (513, 16, 16, 16),
+                                         (300, 32, 32, 32), (33, 32, 31, 1), (65, 1, 64, 32), (100, 2, 500, 2), (2, 32, 32, 32),
+                                         (70001, 4, 4, 4), (1000, 33, 17, 29), (40, 64, 5, 16), (40, 16, 9, 64)])
+def test_native_batches_of_matrices_far_smaller_than_a_tile(gpu, batch, M, K, N):
+    """Matrices of a few kilobytes, several to a workgroup: small integers make every sum exact, so
+    the batch must equal the integer products bit for bit, the buffer's guard values untouched;
+    random operands within the tier's tolerance of the oracle's batch loop."""
+    print("dgemm small batched", batch, M, K, N, flush=True)
+    lib = ea.load()
+    rng = np.random.default_rng(batch + M + K + N)
+    A = rng.integers(-9, 10, (batch, M, K)).astype(np.float64)
+    B = rng.integers(-9, 10, (batch, K, N)).astype(np.float64)
+    dA, dB = dev(A), dev(B)
+    buf = ea.DeviceArray.from_host(np.full(batch * M * N + 128, -7.25))
+    assert lib.hip_dgemm_f64_batched(dA.ptr, dB.ptr, buf.ptr + 64 * 8, batch, M, K, N, stream()) == 0
+    ea.synchronize()
+    out = buf.download()
+    assert np.all(out[:64] == -7.25) and np.all(out[64 + batch * M * N:] == -7.25)
+    assert np.array_equal(out[64:64 + batch * M * N].reshape(batch, M, N), A @ B)
+    nb = min(batch, 50)
+    A, B = synth.uniform(1 + M, (nb, M, K)), synth.uniform(2 + N, (nb, K, N))
+    dA, dB, dC = dev(A), dev(B), ea.DeviceArray((nb, M, N))
+    assert lib.hip_dgemm_f64_batched(dA.ptr, dB.ptr, dC.ptr, nb, M, K, N, stream()) == 0
+    ea.synchronize()
+    got = dC.download()
+    for b in range(nb):
+        assert normwise(got[b], oracle.matmul_f64(A[b], B[b]), A[b], B[b]) <= TOL
+        # one matrix on its own, in every operand form, gives the batch's bits
+        if b < 3:
+            assert np.array_equal(dgemm_ex(A[b], B[b], M, K, N, 0, 0), got[b])
+            assert np.array_equal(dgemm_ex(A[b], np.ascontiguousarray(B[b].T), M, K, N, 0, 1), got[b])
+            assert np.array_equal(dgemm_ex(np.ascontiguousarray(A[b].T), B[b], M, K, N, 1, 0), got[b])
