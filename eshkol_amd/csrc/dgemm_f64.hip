@@ -917,12 +917,12 @@ int dgemm_any(const double* A, const double* B, double* C, uint64_t M, uint64_t 
     /* Operands whose rows do not start on 16-byte boundaries (an odd pitch, a base that
      * is not aligned) would take the kernel of 8-byte loads, at two thirds of the rate
      * (4096 x 4096 x 4097: 3.0 ms against 2.1). Where the shape would otherwise run the
-     * straight-line kernel and is large enough for two passes over an operand not to
-     * matter, the operand is copied to an even pitch first and the kernel told the
+     * straight-line kernel and is large enough (0.2 GFLOP: some ten microseconds) for
+     * another launch and two passes over an operand not to matter, the operand is copied to an even pitch first and the kernel told the
      * pitch; the k-tail and edge logic work on the logical sizes as before, and a pair
      * of values that straddles the end of a row ends in the copy's zero. C needs no
      * copy: the kernel stores it value by value. */
-    if (!vec && batch == 1 && 2.0 * (double)M * (double)N * (double)K >= 4.0e9) {
+    if (!vec && batch == 1 && 2.0 * (double)M * (double)N * (double)K >= 2.0e8) {
         const Kernel would = choose_kernel(m, n, k, 1, true);
         if (would == Kernel::Fast64 || would == Kernel::Fast128) {
             const int rows_a = trans_a ? k : m, rows_b = trans_b ? n : k;

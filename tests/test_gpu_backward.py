@@ -187,7 +187,8 @@ def test_full_size_backward_properties(gpu):
     assert np.array_equal(gB[:, cols], A.T @ G[:, cols])
 
 
-@pytest.mark.parametrize("M,K,N", [(1537, 1601, 1409), (2049, 1024, 2047), (2048, 1025, 2048), (1409, 2001, 1538)])
+@pytest.mark.parametrize("M,K,N", [(1537, 1601, 1409), (2049, 1024, 2047), (2048, 1025, 2048), (1409, 2001, 1538),
+                                   (513, 515, 517), (301, 1999, 303), (33, 2048, 2048)])
 def test_native_large_operands_with_rows_off_16_byte_boundaries(gpu, M, K, N):
     """Large products whose operands have an odd pitch are copied to an even one and run the straight-line
     kernel with that pitch. Small integers make every sum exact, so all three operand forms must give the
