@@ -911,18 +911,21 @@ int dgemm_any(const double* A, const double* B, double* C, uint64_t M, uint64_t 
     /* matrices far smaller than a tile, one or many: several to a workgroup (dgemm_small_f64.hip) */
     if (g_fast_path && eshkol_hip_dgemm_is_small(M, K, N))
         return eshkol_hip_dgemm_small(A, B, C, M, K, N, trans_a, trans_b, batch, st);
+    if (g_fast_path && batch == 1 && eshkol_hip_dgemm_is_small_long_k(M, K, N))
+        return eshkol_hip_dgemm_small_long_k(A, B, C, M, K, N, trans_a, trans_b, st);
     /* a vector or a few against a matrix: bound by HBM, not by the matrix cores (dgemv_f64.hip) */
     if (g_fast_path && batch == 1 && eshkol_hip_dgemm_is_skinny(M, K, N, trans_a, trans_b))
         return eshkol_hip_dgemm_skinny(A, B, C, M, K, N, trans_a, trans_b, st);
     /* Operands whose rows do not start on 16-byte boundaries (an odd pitch, a base that
      * is not aligned) would take the kernel of 8-byte loads, at two thirds of the rate
      * (4096 x 4096 x 4097: 3.0 ms against 2.1). Where the shape would otherwise run the
-     * straight-line kernel and is large enough (0.2 GFLOP: some ten microseconds) for
-     * another launch and two passes over an operand not to matter, the operand is copied to an even pitch first and the kernel told the
+     * straight-line kernel and is large enough (20 MFLOP: some ten microseconds in the other kernel) for
+     * another launch and two passes over an operand not to matter, or has a k long enough
+     * to want cutting (only that kernel's launches are cut along k), the operand is copied to an even pitch first and the kernel told the
      * pitch; the k-tail and edge logic work on the logical sizes as before, and a pair
      * of values that straddles the end of a row ends in the copy's zero. C needs no
      * copy: the kernel stores it value by value. */
-    if (!vec && batch == 1 && 2.0 * (double)M * (double)N * (double)K >= 2.0e8) {
+    if (!vec && batch == 1 && (2.0 * (double)M * (double)N * (double)K >= 2.0e7 || K >= 512)) {
         const Kernel would = choose_kernel(m, n, k, 1, true);
         if (would == Kernel::Fast64 || would == Kernel::Fast128) {
             const int rows_a = trans_a ? k : m, rows_b = trans_b ? n : k;

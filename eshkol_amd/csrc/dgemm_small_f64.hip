@@ -48,7 +48,85 @@ void dgemm_small_batched_kernel(const double* __restrict__ A, const double* __re
     }
 }
 
+/* One product with few outputs and a long k (1 x 6699 x 139, 13 x 6701 x 11): a single tile
+ * would walk all of K in one workgroup (0.38 ms for the first of the two). Here workgroup
+ * p takes k in [p kc, (p + 1) kc), copies its slices of both operands into LDS (op(A) as
+ * sA[i][kk], op(B) as sB[kk][j], whatever form the caller holds them in), sums one output
+ * per thread over its slice, and leaves part[p][i][j]; dgemm_small_sum_kernel adds the
+ * pieces, p ascending. */
+__global__ __launch_bounds__(256)
+void dgemm_small_splitk_kernel(const double* __restrict__ A, const double* __restrict__ B,
+                               int M, int K, int N, int ta, int tb, int kc, double* __restrict__ part) {
+    extern __shared__ __align__(16) double small_smem[];
+    const int k0 = (int)blockIdx.x * kc;
+    const int nk = (K - k0 < kc) ? K - k0 : kc;
+    const int pa = kc + 1;                        /* pitch of sA: rows of one k-slice land in different banks */
+    double* sA = small_smem;
+    double* sB = small_smem + (size_t)M * pa;
+    const int tid = (int)threadIdx.x;
+    if (ta) {                                     /* A is [K][M]: i contiguous */
+        for (int e = tid; e < nk * M; e += 256) { const int kk = e / M, i = e - kk * M; sA[i * pa + kk] = A[(size_t)(k0 + kk) * M + i]; }
+    } else {                                      /* A is [M][K]: k contiguous */
+        for (int e = tid; e < M * nk; e += 256) { const int i = e / nk, kk = e - i * nk; sA[i * pa + kk] = A[(size_t)i * K + k0 + kk]; }
+    }
+    if (tb) {                                     /* B is [N][K]: k contiguous */
+        for (int e = tid; e < N * nk; e += 256) { const int j = e / nk, kk = e - j * nk; sB[kk * N + j] = B[(size_t)j * K + k0 + kk]; }
+    } else {                                      /* B is [K][N]: j contiguous */
+        for (int e = tid; e < nk * N; e += 256) sB[e] = B[(size_t)k0 * N + e];
+    }
+    __syncthreads();
+    double* out = part + (size_t)blockIdx.x * M * N;
+    for (int e = tid; e < M * N; e += 256) {
+        const int i = e / N, j = e - i * N;
+        const double* a = sA + i * pa;
+        const double* b = sB + j;
+        double acc = 0.0;
+        for (int kk = 0; kk < nk; kk++) acc = fma(a[kk], b[kk * N], acc);
+        out[e] = acc;
+    }
+}
+
+__global__ __launch_bounds__(256)
+void dgemm_small_sum_kernel(const double* __restrict__ part, int pieces, int outputs, double* __restrict__ C) {
+    const int e = (int)(blockIdx.x * 256 + threadIdx.x);
+    if (e >= outputs) return;
+    double r = 0.0;
+    int p = 0;
+    for (; p + 8 <= pieces; p += 8) {             /* eight loads in flight, added in order */
+        double v[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) v[q] = part[(size_t)(p + q) * outputs + e];
+#pragma unroll
+        for (int q = 0; q < 8; q++) r += v[q];
+    }
+    for (; p < pieces; p++) r += part[(size_t)p * outputs + e];
+    C[e] = r;
+}
+
 }  // namespace
+
+/* One product of few outputs and a long k: eshkol_hip_dgemm_small_long_k takes it. */
+bool eshkol_hip_dgemm_is_small_long_k(uint64_t M, uint64_t K, uint64_t N) {
+    return M * N <= 1024 && M + N <= 256 && K >= 256 && K <= 0x7fffffffULL;
+}
+
+int eshkol_hip_dgemm_small_long_k(const double* A, const double* B, double* C, uint64_t M, uint64_t K, uint64_t N,
+                                  int trans_a, int trans_b, hipStream_t st) {
+    const int m = (int)M, k = (int)K, n = (int)N;
+    /* slices of k: as long as 32 KiB of LDS hold (at least 16), at most 512, and enough of them for every CU */
+    int kc = (int)(4096 / (m + n)) - 1;
+    if (kc > 512) kc = 512;
+    const int per_cu = (k + eshkol_hip_num_cus() - 1) / eshkol_hip_num_cus();
+    if (kc > per_cu) kc = per_cu < 16 ? 16 : per_cu;
+    if (kc < 15) return -1;
+    const int pieces = (k + kc - 1) / kc;
+    double* part = (double*)eshkol_hip_workspace(WS_DGEMM_PARTIAL, (size_t)pieces * m * n * sizeof(double));
+    if (!part) return -1;
+    const size_t lds = ((size_t)m * (kc + 1) + (size_t)kc * n) * sizeof(double);
+    hipLaunchKernelGGL(dgemm_small_splitk_kernel, dim3((unsigned)pieces), dim3(256), lds, st, A, B, m, k, n, trans_a, trans_b, kc, part);
+    hipLaunchKernelGGL(dgemm_small_sum_kernel, dim3((unsigned)((m * n + 255) / 256)), dim3(256), 0, st, part, pieces, m * n, C);
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
 
 /* Shapes eshkol_hip_dgemm_small takes. */
 bool eshkol_hip_dgemm_is_small(uint64_t M, uint64_t K, uint64_t N) {

@@ -316,7 +316,7 @@ int launch_klast(const double* big, long ldb, int O, int K, const double* thin, 
  * enough to give every CU work, and the big operand worth a pass of its own. */
 bool eshkol_hip_dgemm_is_skinny(uint64_t M, uint64_t K, uint64_t N, int trans_a, int trans_b) {
     const uint64_t thin = M < N ? M : N, wide = M < N ? N : M;
-    if (thin == 0 || wide < 1024 || K < 64 || K > 0x7fffffffULL || wide > 0x7fffffffULL) return false;
+    if (thin == 0 || wide < 128 || K < 64 || K > 0x7fffffffULL || wide > 0x7fffffffULL) return false;
     /* The kernel for k-contiguous big operands holds R x S sums per lane and is out of
      * registers after eight thin columns; the other one carries up to thirty-two thin rows
      * (3 TB/s at 32 x 8192 x 8192, where the tiled kernel reaches 2), from seventeen on only
@@ -324,7 +324,7 @@ bool eshkol_hip_dgemm_is_skinny(uint64_t M, uint64_t K, uint64_t N, int trans_a,
     const bool thin_m = M <= N;
     const bool kfirst = thin_m ? !trans_b : (trans_a != 0);     /* the big operand has the output index contiguous */
     const uint64_t limit = !kfirst ? 8u : (wide * K >= (1ull << 24)) ? 32u : 16u;
-    return thin <= limit && wide * K >= (1ull << 20);
+    return thin <= limit && wide * K >= (1ull << 17);
 }
 
 /* C = op(A) op(B) for a product eshkol_hip_dgemm_is_skinny() accepts. */

@@ -119,6 +119,10 @@ bool eshkol_hip_dgemm_is_small(uint64_t M, uint64_t K, uint64_t N);
 int eshkol_hip_dgemm_small(const double* A, const double* B, double* C, uint64_t M, uint64_t K, uint64_t N,
                            int trans_a, int trans_b, uint64_t batch, hipStream_t st);
 
+bool eshkol_hip_dgemm_is_small_long_k(uint64_t M, uint64_t K, uint64_t N);
+int eshkol_hip_dgemm_small_long_k(const double* A, const double* B, double* C, uint64_t M, uint64_t K, uint64_t N,
+                                  int trans_a, int trans_b, hipStream_t st);
+
 /* fp64 products with one thin side (dgemv_f64.hip): whether the shape is one, and the
  * product itself. hip_dgemm_f64 and hip_dgemm_f64_ex send such shapes there. */
 bool eshkol_hip_dgemm_is_skinny(uint64_t M, uint64_t K, uint64_t N, int trans_a, int trans_b);

@@ -306,3 +306,26 @@ def test_native_batches_of_matrices_far_smaller_than_a_tile(gpu, batch, M, K, N)
             assert np.array_equal(dgemm_ex(A[b], B[b], M, K, N, 0, 0), got[b])
             assert np.array_equal(dgemm_ex(A[b], np.ascontiguousarray(B[b].T), M, K, N, 0, 1), got[b])
             assert np.array_equal(dgemm_ex(np.ascontiguousarray(A[b].T), B[b], M, K, N, 1, 0), got[b])
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 6699, 139), (13, 6701, 11), (108, 5980, 3), (6, 3945, 1), (1, 1919, 1), (27, 3215, 6),
+                                   (31, 300, 33), (16, 100000, 16), (255, 257, 1), (64, 256, 16), (1, 256, 255), (32, 4097, 32)])
+def test_native_products_of_few_outputs_and_a_long_k(gpu, M, K, N):
+    """Few outputs, long k: the contraction is cut into slices over the workgroups and the pieces are
+    added in a fixed order. Integer operands: exact, bit for bit, in every operand form; random
+    operands within the tier's tolerance; the same call twice gives the same bits."""
+    print("dgemm small long k", M, K, N, flush=True)
+    rng = np.random.default_rng(M + K + N)
+    A = rng.integers(-9, 10, (M, K)).astype(np.float64)
+    B = rng.integers(-9, 10, (K, N)).astype(np.float64)
+    ref = A @ B
+    At, Bt = np.ascontiguousarray(A.T), np.ascontiguousarray(B.T)
+    assert np.array_equal(dgemm_ex(A, B, M, K, N, 0, 0), ref)
+    assert np.array_equal(dgemm_ex(A, Bt, M, K, N, 0, 1), ref)
+    assert np.array_equal(dgemm_ex(At, B, M, K, N, 1, 0), ref)
+    A, B = synth.uniform(100 + M, (M, K)), synth.uniform(200 + N, (K, N))
+    got = dgemm_ex(A, B, M, K, N, 0, 0)
+    assert normwise(got, oracle.matmul_f64(A, B), A, B) <= TOL
+    assert np.array_equal(got, dgemm_ex(A, B, M, K, N, 0, 0))
+    assert normwise(dgemm_ex(np.ascontiguousarray(A.T), B, M, K, N, 1, 0), oracle.matmul_f64(A, B), A, B) <= TOL
+    assert normwise(dgemm_ex(A, np.ascontiguousarray(B.T), M, K, N, 0, 1), oracle.matmul_f64(A, B), A, B) <= TOL
