@@ -329,3 +329,20 @@ def test_native_products_of_few_outputs_and_a_long_k(gpu, M, K, N):
     assert np.array_equal(got, dgemm_ex(A, B, M, K, N, 0, 0))
     assert normwise(dgemm_ex(np.ascontiguousarray(A.T), B, M, K, N, 1, 0), oracle.matmul_f64(A, B), A, B) <= TOL
     assert normwise(dgemm_ex(A, np.ascontiguousarray(B.T), M, K, N, 0, 1), oracle.matmul_f64(A, B), A, B) <= TOL
+
+
+def test_native_random_shapes_take_whichever_kernel_and_agree_with_integers(gpu):
+    """Eighty shapes drawn log-uniformly (1 ... 3000 per dimension), random operand form: whichever of
+    the fp64 kernels a shape is routed to (tiles with or without a cut k, copies to an even pitch, the
+    thin-side kernels, the kernels for matrices smaller than a tile), small integers must come out as
+    the exact integer product."""
+    rng = np.random.default_rng(20240)
+    for case in range(80):
+        M, K, N = (max(1, int(2 ** rng.uniform(0, 11.55))) for _ in range(3))
+        ta, tb = [(0, 0), (0, 1), (1, 0)][rng.integers(0, 3)]
+        print("dgemm_ex random", case, M, K, N, ta, tb, flush=True)
+        A = rng.integers(-9, 10, (M, K)).astype(np.float64)
+        B = rng.integers(-9, 10, (K, N)).astype(np.float64)
+        X = np.ascontiguousarray(A.T) if ta else A
+        Y = np.ascontiguousarray(B.T) if tb else B
+        assert np.array_equal(dgemm_ex(X, Y, M, K, N, ta, tb), A @ B), (M, K, N, ta, tb)
