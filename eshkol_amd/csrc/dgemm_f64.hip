@@ -883,13 +883,16 @@ int launch_shape(const double* A, const double* B, double* C, int m, int n, int 
 
 /* dst[r][c] = src[r][c] for c < cols, 0 for cols <= c < ld: an operand whose rows do
  * not start on 16-byte boundaries (odd cols, or a base that is not aligned) copied
- * to an even pitch. */
+ * to an even pitch. One launch copies both operands of a product (blockIdx.z says
+ * which); an operand that needs no copy comes with rows == 0. */
+struct PadCopy { const double* src; double* dst; int rows, cols, ld; };
 __global__ __launch_bounds__(256)
-void dgemm_pad_copy_kernel(const double* __restrict__ src, double* __restrict__ dst, int rows, int cols, int ld) {
+void dgemm_pad_copy_kernel(PadCopy a, PadCopy b) {
+    const PadCopy& p = blockIdx.z == 0 ? a : b;
     const int c = (int)(blockIdx.x * 256 + threadIdx.x);
-    if (c >= ld) return;
-    for (int r = (int)blockIdx.y; r < rows; r += (int)gridDim.y)
-        dst[(size_t)r * ld + c] = (c < cols) ? src[(size_t)r * cols + c] : 0.0;
+    if (c >= p.ld) return;
+    for (int r = (int)blockIdx.y; r < p.rows; r += (int)gridDim.y)
+        p.dst[(size_t)r * p.ld + c] = (c < p.cols) ? p.src[(size_t)r * p.cols + c] : 0.0;
 }
 
 }  // namespace
@@ -935,21 +938,22 @@ int dgemm_any(const double* A, const double* B, double* C, uint64_t M, uint64_t 
             const double* a2 = A;
             const double* b2 = B;
             bool ok = pitch_a < 0x7fffffffULL && pitch_b < 0x7fffffffULL;
+            PadCopy ca = {A, nullptr, 0, (int)pitch_a, lda}, cb = {B, nullptr, 0, (int)pitch_b, ldb};
             if (ok && copy_a) {
-                double* w = (double*)eshkol_hip_workspace(WS_DGEMM_PAD_A, (size_t)rows_a * lda * sizeof(double));
-                if (w) {
-                    hipLaunchKernelGGL(dgemm_pad_copy_kernel, dim3((unsigned)((lda + 255) / 256), (unsigned)(rows_a < 65535 ? rows_a : 65535)),
-                                       dim3(256), 0, st, A, w, rows_a, (int)pitch_a, lda);
-                    a2 = w;
-                } else ok = false;
+                ca.dst = (double*)eshkol_hip_workspace(WS_DGEMM_PAD_A, (size_t)rows_a * lda * sizeof(double));
+                ca.rows = rows_a;
+                if (ca.dst) a2 = ca.dst; else ok = false;
             }
             if (ok && copy_b) {
-                double* w = (double*)eshkol_hip_workspace(WS_DGEMM_PAD_B, (size_t)rows_b * ldb * sizeof(double));
-                if (w) {
-                    hipLaunchKernelGGL(dgemm_pad_copy_kernel, dim3((unsigned)((ldb + 255) / 256), (unsigned)(rows_b < 65535 ? rows_b : 65535)),
-                                       dim3(256), 0, st, B, w, rows_b, (int)pitch_b, ldb);
-                    b2 = w;
-                } else ok = false;
+                cb.dst = (double*)eshkol_hip_workspace(WS_DGEMM_PAD_B, (size_t)rows_b * ldb * sizeof(double));
+                cb.rows = rows_b;
+                if (cb.dst) b2 = cb.dst; else ok = false;
+            }
+            if (ok) {
+                const int wide = (copy_a && (!copy_b || lda > ldb)) ? lda : ldb;
+                const int tall = (ca.rows > cb.rows) ? ca.rows : cb.rows;
+                hipLaunchKernelGGL(dgemm_pad_copy_kernel, dim3((unsigned)((wide + 255) / 256), (unsigned)(tall < 65535 ? tall : 65535), 2),
+                                   dim3(256), 0, st, ca, cb);
             }
             if (ok) {
                 g_lda = copy_a ? lda : 0;
