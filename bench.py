@@ -507,42 +507,22 @@ def main():
                     return rc
                 src = acts[i]
             return 0
-        # ... and with every layer handing the next one the row maxima of its activations
-        rowmax = [ea.DeviceArray((batch,)) for i in range(3)]
-
-        def mlp_forward_chained():
-            src, known = X, None
-            for i in range(3):
-                rc = lib.hip_matmul_ozaki_crt_prepared_chain_f64(src.ptr, known, handles[i], acts[i].ptr, rowmax[i].ptr,
-                                                                 batch, dims[i], dims[i + 1], 16, bs[i].ptr, 1, st)
-                if rc != 0:
-                    return rc
-                src, known = acts[i], rowmax[i].ptr
-            return 0
         os.dup2(devnull, 2)
         try:
             mlp_forward(); hip.hipDeviceSynchronize()
             plain = acts[2].download()
             e7p, w7p = timed(mlp_forward_prepared, settle_ms=40.0)
-            same = bool(np.array_equal(plain, acts[2].download()))
-            e7c, w7c = timed(mlp_forward_chained, settle_ms=40.0)
         finally:
             os.dup2(saved, 2)
-        same_chained = bool(np.array_equal(plain, acts[2].download()))
+        same = bool(np.array_equal(plain, acts[2].download()))
         for h in handles:
             lib.hip_ozaki_crt_release_prepared(h)
         tiers["mlp_forward_exact_tier_batch4096_1024_4096_4096_1024"] = {
             "ms": w7, "gflops_fp64_equiv": mlp_flops / (w7 * 1e-3) / 1e9,
             "with_prepared_weights_ms": w7p, "with_prepared_weights_gflops_fp64_equiv": mlp_flops / (w7p * 1e-3) / 1e9,
             "prepared_output_bit_identical": same,
-            "with_prepared_weights_and_chained_row_maxima_ms": w7c,
-            "with_prepared_weights_and_chained_row_maxima_gflops_fp64_equiv": mlp_flops / (w7c * 1e-3) / 1e9,
-            "chained_output_bit_identical": same_chained,
             "note": "three GEMMs, bias add + tanh fused in the reconstruct epilogue; prepared = the weights' column "
-                    "maxima and residue planes computed once instead of on every forward pass; chained = each layer's "
-                    "reconstruction also leaves the row maxima of its activations, which the next layer takes instead "
-                    "of reading the activations for them (hip_matmul_ozaki_crt_prepared_chain_f64)"}
-        log("mlp forward, prepared weights and chained row maxima: %.3f ms (same bits: %s)" % (w7c, same_chained))
+                    "maxima and residue planes computed once instead of on every forward pass"}
         log("mlp forward (exact tier): %.3f ms %.1f GFLOP/s-eq; with prepared weights %.3f ms (same bits: %s)"
             % (w7, mlp_flops / (w7 * 1e-3) / 1e9, w7p, same))
         for d in [X] + Ws + bs + acts:

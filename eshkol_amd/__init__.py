@@ -145,7 +145,6 @@ SIGNATURES = {
     "hip_igemm_set_persistent": (None, [C.c_int]),
     "hip_ozaki_crt_prepare_operand_b": (C.c_int, [vp, u64, u64, C.c_int, C.c_int, u64, C.POINTER(vp), vp]),
     "hip_matmul_ozaki_crt_prepared_f64": (C.c_int, [vp, vp, vp, u64, u64, u64, C.c_int, C.c_int, C.c_int, vp, C.c_int, vp]),
-    "hip_matmul_ozaki_crt_prepared_chain_f64": (C.c_int, [vp, vp, vp, vp, vp, u64, u64, u64, C.c_int, vp, C.c_int, vp]),
     "hip_ozaki_crt_release_prepared": (None, [vp]),
     "hip_ozaki_fast_split_planes_f64": (C.c_int, [vp, u64, u64, vp, C.c_int, vp, u64, u64, C.c_int, C.c_int, vp]),
     "hip_ozaki_fast_reconstruct_f64": (C.c_int, [vp, u64, u64, u64, C.c_int, vp, vp, vp, vp]),

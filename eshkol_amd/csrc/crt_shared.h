@@ -62,10 +62,6 @@ int eshkol_rowabsmax_shift_f64(const double* A, uint64_t M, uint64_t K, double z
                                double* rmax, int32_t* shift, int E, hipStream_t stream, hipEvent_t done = nullptr);
 int eshkol_colabsmax_shift_f64(const double* X, uint64_t K, uint64_t R, double zero_value,
                                double* cmax, int32_t* shift, int E, hipStream_t stream, hipEvent_t done = nullptr);
-/* The same outputs from maxima that are known already (n doubles on the device). */
-int eshkol_maxima_shift_f64(const double* maxima, uint64_t n, double zero_value,
-                            double* out, int32_t* shift, int E, hipStream_t stream, hipEvent_t done = nullptr,
-                            double* clear = nullptr);
 /* done, when given, becomes the completion event of the launch's last kernel
  * (the kernel's own completion signal: no marker is queued behind it, which
  * would hold the next kernel of the stream back by 6-7 us). */

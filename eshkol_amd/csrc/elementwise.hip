@@ -83,22 +83,6 @@ void rowabsmax_f64_kernel(const double* __restrict__ A, uint64_t M, uint64_t K,
     }
 }
 
-/* Maxima that are known already (a previous product left them beside its result): the
- * same outputs as rowabsmax_f64_kernel without reading the matrix. clear, when given, is
- * an array of n doubles set to zero on the way (where the product about to be queued will
- * collect the maxima of its own result). */
-__global__ __launch_bounds__(256)
-void maxima_shift_kernel(const double* __restrict__ in, uint64_t n, double zero_value,
-                         double* __restrict__ out, int32_t* __restrict__ shift, int E, double* __restrict__ clear) {
-    const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
-    if (clear) clear[i] = 0.0;
-    double m = in[i];
-    if (!(m <= 1.7976931348623157e308)) m = __builtin_inf();
-    out[i] = (m > 0.0) ? m : zero_value;
-    if (shift) shift[i] = shift_of_maximum(m, E);
-}
-
 /* Column maxima of a row-major X[K][R] in two steps: a block takes 64 columns
  * by one slice of the rows (a wave reads 512 contiguous bytes per row) and
  * writes its partial maxima; the second kernel folds the slices. */
@@ -217,16 +201,6 @@ int eshkol_rowabsmax_shift_f64(const double* A, uint64_t M, uint64_t K, double z
     if (g > 0x7fffffffULL) return -1;
     hipExtLaunchKernelGGL(rowabsmax_f64_kernel, dim3((unsigned)g), dim3(256), 0, stream, nullptr, done, 0,
                           A, M, K, zero_value, rmax, shift, E);
-    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
-}
-
-int eshkol_maxima_shift_f64(const double* maxima, uint64_t n, double zero_value,
-                            double* out, int32_t* shift, int E, hipStream_t stream, hipEvent_t done, double* clear) {
-    if (!maxima || !out || n == 0) return -1;
-    const uint64_t g = (n + 255) / 256;
-    if (g > 0x7fffffffULL) return -1;
-    hipExtLaunchKernelGGL(maxima_shift_kernel, dim3((unsigned)g), dim3(256), 0, stream, nullptr, done, 0,
-                          maxima, n, zero_value, out, shift, E, clear);
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 

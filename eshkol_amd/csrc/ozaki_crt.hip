@@ -313,40 +313,15 @@ struct CrtConsts {
  * element by element.
  * VEC 0: nothing is known about W's alignment either (dense planes of any N). */
 typedef double d2u_t __attribute__((ext_vector_type(2), aligned(8)));
-
-/* Largest v over the 64 lanes of a wave, all of them active; the same value in every lane. */
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ uint32_t wave_max_step(uint32_t v) {
-    /* lanes without a source, or outside ROW_MASK, take 0: the identity of an unsigned max */
-    const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, ROW_MASK, 0xf, false);
-    return o > v ? o : v;
-}
-__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
-    v = wave_max_step<0x111, 0xf>(v);       /* row_shr:1 */
-    v = wave_max_step<0x112, 0xf>(v);       /* row_shr:2 */
-    v = wave_max_step<0x114, 0xf>(v);       /* row_shr:4 */
-    v = wave_max_step<0x118, 0xf>(v);       /* row_shr:8: lane 15 of every row of 16 holds the row's maximum */
-    v = wave_max_step<0x142, 0xa>(v);       /* row_bcast:15 into rows 1 and 3 */
-    v = wave_max_step<0x143, 0xc>(v);       /* row_bcast:31 into rows 2 and 3: lane 63 holds the wave's maximum */
-    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
-}
-
 template <int NMOD, bool TANH, int VEC>
 __global__ __launch_bounds__(256)
 void crt_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t wrows, uint64_t ldw, uint64_t M, uint64_t N, CrtConsts cc,
                             const int32_t* __restrict__ mu, const int32_t* __restrict__ nu,
-                            const double* __restrict__ bias, double* __restrict__ C,
-                            unsigned long long* __restrict__ rowmax) {
+                            const double* __restrict__ bias, double* __restrict__ C) {
     const uint32_t cpr = (uint32_t)(((N + 3) / 4 + 255) / 256);   /* blocks per row */
     const uint64_t row = blockIdx.x / cpr;
     const uint64_t col = ((uint64_t)(blockIdx.x % cpr) * 256 + threadIdx.x) * 4;
-    /* rowmax, when given (the same for the whole launch), receives the largest |C[row][j]| as
-     * the bits of a double (of +inf if a value is not finite), so that the next product of a
-     * chain of layers need not read C for it */
-    const bool live = col < N;
-    if (!live && !rowmax) return;                 /* with rowmax every lane stays for the wave's maximum */
-    unsigned long long mine = 0;
-    if (live) {
+    if (col >= N) return;
     const uint64_t tot = wrows * ldw, idx = row * N + col, widx = row * ldw + col;
     const int nvalid = (VEC == 1) ? 4 : ((N - col < 4) ? (int)(N - col) : 4);
     uint32_t u[NMOD];
@@ -410,29 +385,6 @@ void crt_reconstruct_kernel(const int8_t* __restrict__ W, uint64_t wrows, uint64
     } else {
 #pragma unroll
         for (int e = 0; e < 4; e++) if (e < nvalid) C[idx + e] = out[e];
-    }
-    if (rowmax) {
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            if (e < nvalid) {
-                const double a = fabs(out[e]);
-                const unsigned long long bits = (a <= 1.7976931348623157e308) ? (unsigned long long)__double_as_longlong(a)
-                                                                             : 0x7ff0000000000000ull;
-                if (bits > mine) mine = bits;
-            }
-        }
-    }
-    }
-    /* The wave's maximum with data-parallel-primitive moves (six v_max_u32 per 32-bit half;
-     * through LDS shuffles the kernel, which is bound by its vector instructions, was 15 per
-     * cent slower, with every thread looking at the row's maximum in memory first 55), then
-     * one atomic per wave: all of a workgroup's waves are in the same row. */
-    if (rowmax) {
-        const uint32_t hi = (uint32_t)(mine >> 32);
-        const uint32_t top = wave_max_u32(hi);
-        const uint32_t low = wave_max_u32(hi == top ? (uint32_t)mine : 0u);
-        const unsigned long long m = (unsigned long long)top << 32 | low;
-        if ((threadIdx.x & 63) == 0 && m) atomicMax(rowmax + row, m);
     }
 }
 
@@ -864,7 +816,7 @@ extern "C" int hip_ozaki_crt_split_planes_f64(const double* X, uint64_t rows, ui
 static int crt_reconstruct(const int8_t* w_planes, uint64_t wrows, uint64_t ldw, uint64_t M, uint64_t N, int num_moduli,
                            const double* sl1, const double* sl2, double P1, double P2, double Pinv,
                            const int32_t* mu, const int32_t* nu, const double* bias, int act,
-                           double* C, void* stream, double* c_rowmax = nullptr) {
+                           double* C, void* stream) {
     if (!w_planes || !sl1 || !sl2 || !mu || !nu || !C || M == 0 || N == 0 || wrows < M || ldw < N) return -1;
     if (num_moduli < 2 || num_moduli > MAX_MODULI || act < 0 || act > 1) return -1;
     if ((((N + 3) / 4 + 255) / 256) * M > 0x7fffffffULL) return -1;
@@ -878,8 +830,7 @@ static int crt_reconstruct(const int8_t* w_planes, uint64_t wrows, uint64_t ldw,
     const int vec = !wvec ? 0 : ((N % 4 == 0) && (((uintptr_t)C & 15) == 0)) ? 1 : 2;
     switch (num_moduli) {
 #define LAUNCH(n, tanh, v) hipLaunchKernelGGL((crt_reconstruct_kernel<n, tanh, v>), grid, dim3(256), 0,    \
-                                              (hipStream_t)stream, w_planes, wrows, ldw, M, N, cc, mu, nu, bias, C,  \
-                                              (unsigned long long*)c_rowmax)
+                                              (hipStream_t)stream, w_planes, wrows, ldw, M, N, cc, mu, nu, bias, C)
 #define CASE(n) case n:                                                                                   \
         if (act == 1) { if (vec == 1) LAUNCH(n, true, 1); else if (vec == 2) LAUNCH(n, true, 2); else LAUNCH(n, true, 0); } \
         else { if (vec == 1) LAUNCH(n, false, 1); else if (vec == 2) LAUNCH(n, false, 2); else LAUNCH(n, false, 0); }       \
@@ -949,20 +900,11 @@ struct CrtPreparedB {
 constexpr uint32_t PREPARED_MAGIC = 0x43525442u;
 }  // namespace
 
-__global__ __launch_bounds__(256)
-void crt_clear_u64_kernel(unsigned long long* p, uint64_t n) {
-    const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < n) p[i] = 0;
-}
-
-/* a_rowmax (device, M doubles, or NULL): the row maxima of |A|, known already; A is then
- * not read for them. c_rowmax (device, M doubles, or NULL): receives the row maxima of |C|. */
 static int crt_matmul_impl(const double* A, const double* B, double* C,
                            uint64_t M, uint64_t K, uint64_t N,
                            int trans_a, int trans_b,
                            int num_moduli, int adaptive,
-                           const double* bias, int act, void* stream, const CrtPreparedB* prepared,
-                           const double* a_rowmax = nullptr, double* c_rowmax = nullptr) {
+                           const double* bias, int act, void* stream, const CrtPreparedB* prepared) {
     EshkolHipCall bracket(stream);
     if (!A || !B || !C || M == 0 || K == 0 || N == 0) return -1;
     if (M > 0x7fffffffULL || N > 0x7fffffffULL) return -1;
@@ -1027,14 +969,8 @@ static int crt_matmul_impl(const double* A, const double* B, double* C,
     /* the last kernel that writes maxima carries the event the scan's stream waits for */
     const hipEvent_t fork = fixed_E ? scan_event(M * K + K * N) : nullptr;
     const hipEvent_t fork_a = use_prepared ? fork : nullptr, fork_b = use_prepared ? nullptr : fork;
-    /* c_rowmax starts at zero: the kernel that turns known maxima into shifts clears it on
-     * its way, otherwise a launch of its own does */
-    bool c_cleared = false;
-    if (a_rowmax && !a_kmajor) {
-        if (eshkol_maxima_shift_f64(a_rowmax, M, 0.0, amax, mu_out, 52, st, fork_a, c_rowmax) != 0) return -1;
-        c_cleared = c_rowmax != nullptr;
-    } else if ((a_kmajor ? eshkol_colabsmax_shift_f64(A, K, M, 0.0, amax, mu_out, 52, st, fork_a)
-                         : eshkol_rowabsmax_shift_f64(A, M, K, 0.0, amax, mu_out, 52, st, fork_a)) != 0) return -1;
+    if ((a_kmajor ? eshkol_colabsmax_shift_f64(A, K, M, 0.0, amax, mu_out, 52, st, fork_a)
+                  : eshkol_rowabsmax_shift_f64(A, M, K, 0.0, amax, mu_out, 52, st, fork_a)) != 0) return -1;
     if (!use_prepared &&
         (b_kmajor ? eshkol_colabsmax_shift_f64(B, K, N, 0.0, bmax, nu_out, 52, st, fork_b)
                   : eshkol_rowabsmax_shift_f64(B, N, K, 0.0, bmax, nu_out, 52, st, fork_b)) != 0) return -1;
@@ -1050,10 +986,6 @@ static int crt_matmul_impl(const double* A, const double* B, double* C,
         const uint64_t Mw = eshkol_product_rows(M), Nw = eshkol_product_pitch(N);
         int8_t* Wp = (int8_t*)eshkol_hip_workspace(WS_PRODUCTS, (size_t)n_mod * Mw * Nw);
         if (!Ap || !Bp || !Wp) return -1;
-        if (c_rowmax && !c_cleared)               /* the reconstruction takes maxima over what is there */
-            hipLaunchKernelGGL(crt_clear_u64_kernel, dim3((unsigned)((M + 255) / 256)), dim3(256), 0, st,
-                               (unsigned long long*)c_rowmax, M);
-        c_cleared = false;                        /* a second round of products (after a host pass) clears again */
         if (crt_split_any(A, M, K, dmu, n_mod, Ap, Mp, ldk, a_kmajor, layout, st) != 0) return -1;
         if (!b_ready && crt_split_any(B, N, K, dnu, n_mod, Bp, Np, ldk, b_kmajor, layout, st) != 0) return -1;
         HipIgemmArgs ga;
@@ -1067,7 +999,7 @@ static int crt_matmul_impl(const double* A, const double* B, double* C,
         ga.out_rows = (uint32_t)Mw; ga.ldn = (uint32_t)Nw;
         if (hip_igemm_i8(&ga, st) != 0) return -1;
         if (crt_reconstruct(Wp, Mw, Nw, M, N, n_mod, crt.sl1, crt.sl2, crt.P1, crt.P2, crt.Pinv,
-                            dmu, nu, bias, act, C, st, c_rowmax) != 0) return -1;
+                            dmu, nu, bias, act, C, st) != 0) return -1;
         g_last.a_planes = Ap; g_last.b_planes = Bp; g_last.w_planes = Wp;
         g_last.w_rows = Mw; g_last.w_ld = Nw;
         g_last.mu = dmu; g_last.nu = (int32_t*)nu;
@@ -1244,16 +1176,6 @@ extern "C" int hip_matmul_ozaki_crt_prepared_f64(const double* A, const void* pr
     const CrtPreparedB* pb = (const CrtPreparedB*)prepared_b;
     if (!pb || pb->magic != PREPARED_MAGIC || pb->K != K || pb->N != N) return -1;
     return crt_matmul_impl(A, pb->src, C, M, K, N, trans_a, pb->trans_b, num_moduli, adaptive, bias, act, stream, pb);
-}
-
-extern "C" int hip_matmul_ozaki_crt_prepared_chain_f64(const double* A, const double* a_rowmax, const void* prepared_b,
-                                                       double* C, double* c_rowmax,
-                                                       uint64_t M, uint64_t K, uint64_t N, int num_moduli,
-                                                       const double* bias, int act, void* stream) {
-    const CrtPreparedB* pb = (const CrtPreparedB*)prepared_b;
-    if (!pb || pb->magic != PREPARED_MAGIC || pb->K != K || pb->N != N) return -1;
-    if (a_rowmax == c_rowmax && a_rowmax) return -1;
-    return crt_matmul_impl(A, pb->src, C, M, K, N, 0, pb->trans_b, num_moduli, 0, bias, act, stream, pb, a_rowmax, c_rowmax);
 }
 
 extern "C" int hip_matmul_ozaki_crt_f64(const double* A, const double* B, double* C,

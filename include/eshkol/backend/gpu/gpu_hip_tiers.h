@@ -221,21 +221,6 @@ int hip_matmul_ozaki_crt_prepared_f64(const double* A, const void* prepared_b, d
                                       uint64_t M, uint64_t K, uint64_t N, int trans_a,
                                       int num_moduli, int adaptive,
                                       const double* bias, int act, void* stream);
-
-/* The prepared product as a link in a chain of layers, each layer's result the next
- * one's first operand. The tier needs the row maxima max_k |A[i][k]| of its first
- * operand before anything else, a pass over A of its own (28 us for 4096 x 4096 at
- * what HBM delivers); here the reconstruction of one product leaves the row maxima
- * of its result (after bias and activation) in c_rowmax (device, M doubles; NULL:
- * not wanted), and the next call takes them as a_rowmax (NULL: not known, A is read
- * for them as usual). The caller vouches that a_rowmax holds the maxima of A as it
- * is now. Results are those of hip_matmul_ozaki_crt_prepared_f64 bit for bit. No
- * counterpart in the reference, whose layers are separate matmul calls
- * (lib/core/model_io.cpp:690-712). */
-int hip_matmul_ozaki_crt_prepared_chain_f64(const double* A, const double* a_rowmax, const void* prepared_b,
-                                            double* C, double* c_rowmax,
-                                            uint64_t M, uint64_t K, uint64_t N, int num_moduli,
-                                            const double* bias, int act, void* stream);
 void hip_ozaki_crt_release_prepared(void* handle);
 
 /* How the CRT weights s_l = (P / p_l) q_l are split into the two doubles the

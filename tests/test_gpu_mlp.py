@@ -3,8 +3,6 @@ every GEMM through the exact tier and the bias add and tanh fused into its
 epilogue. Checked against the oracle layer by layer; tanh is glibc's on the CPU
 and the device library's on the GPU, so the bar on the activations is 4 ulp of
 1.0 (|tanh| <= 1), while the pre-activation GEMM keeps the exact tier's 2 ulp."""
-import ctypes as C
-
 import numpy as np
 import pytest
 
@@ -110,50 +108,3 @@ def test_prepared_weights_give_the_same_bits(gpu, batch, dims):
     bad = layers[0][0].copy(); bad[3, 4] = np.inf
     assert lib.hip_ozaki_crt_prepare_operand_b(ea.DeviceArray.from_host(bad).ptr, dims[0], dims[1], 0, 16, batch,
                                                C.byref(h), st) == -1
-
-
-@pytest.mark.parametrize("batch,dims", [(130, [63, 255, 129, 65]), (512, [256, 1024, 1024, 256]), (2048, [1024, 2048, 1024])])
-def test_layers_chained_through_their_row_maxima_give_the_same_bits(gpu, batch, dims):
-    """hip_matmul_ozaki_crt_prepared_chain_f64: every layer leaves the row maxima of its activations, the next
-    takes them instead of reading the activations for them. Same bits as the unchained calls; the maxima are
-    the maxima."""
-    lib = ea.load()
-    st = lib.eshkol_hip_get_stream()
-    n = len(dims) - 1
-    X = ea.DeviceArray.from_host(synth.normal(1, (batch, dims[0])))
-    Ws = [ea.DeviceArray.from_host(synth.xavier_uniform(10 + i, dims[i], dims[i + 1])) for i in range(n)]
-    bs = [ea.DeviceArray.from_host(synth.uniform(20 + i, (dims[i + 1],), -0.05, 0.05)) for i in range(n)]
-    handles = []
-    for i in range(n):
-        h = C.c_void_p()
-        assert lib.hip_ozaki_crt_prepare_operand_b(Ws[i].ptr, dims[i], dims[i + 1], 0, 16, batch, C.byref(h), st) == 0
-        handles.append(h)
-    plain = [ea.DeviceArray((batch, dims[i + 1])) for i in range(n)]
-    chained = [ea.DeviceArray((batch, dims[i + 1])) for i in range(n)]
-    maxima = [ea.DeviceArray.from_host(np.full(batch, -3.0)) for i in range(n)]
-    src = X
-    for i in range(n):
-        assert lib.hip_matmul_ozaki_crt_prepared_f64(src.ptr, handles[i], plain[i].ptr, batch, dims[i], dims[i + 1],
-                                                     0, 16, 0, bs[i].ptr, 1, st) == 0
-        src = plain[i]
-    src, known = X, None
-    for i in range(n):
-        assert lib.hip_matmul_ozaki_crt_prepared_chain_f64(src.ptr, known, handles[i], chained[i].ptr, maxima[i].ptr,
-                                                           batch, dims[i], dims[i + 1], 16, bs[i].ptr, 1, st) == 0
-        src, known = chained[i], maxima[i].ptr
-    ea.synchronize()
-    for i in range(n):
-        got = chained[i].download()
-        assert np.array_equal(got, plain[i].download()), i
-        assert np.array_equal(maxima[i].download(), np.abs(got).max(axis=1)), i
-    # maxima that are wrong on purpose change the result: they really are what the call uses
-    wrong = ea.DeviceArray.from_host(np.abs(chained[0].download()).max(axis=1) * 4.0)
-    out = ea.DeviceArray((batch, dims[2]))
-    assert lib.hip_matmul_ozaki_crt_prepared_chain_f64(chained[0].ptr, wrong.ptr, handles[1], out.ptr, None,
-                                                       batch, dims[1], dims[2], 16, bs[1].ptr, 1, st) == 0
-    ea.synchronize()
-    other = out.download()
-    assert not np.array_equal(other, plain[1].download())             # the shifts moved by two bits: other residues
-    assert np.abs(other - plain[1].download()).max() <= 1e-6           # of the same product
-    for h in handles:
-        lib.hip_ozaki_crt_release_prepared(h)
