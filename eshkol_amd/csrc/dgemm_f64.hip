@@ -911,14 +911,17 @@ int dgemm_any(const double* A, const double* B, double* C, uint64_t M, uint64_t 
                      ((uintptr_t)A % 16 == 0) && ((uintptr_t)B % 16 == 0) &&
                      (batch == 1 || ((M * K) % 2 == 0 && (K * N) % 2 == 0));
     const int m = (int)M, n = (int)N, k = (int)K;
+    /* Shapes with kernels of their own; one that cannot run (no workspace to be had) leaves the
+     * product to the tiled kernels below. */
     /* matrices far smaller than a tile, one or many: several to a workgroup (dgemm_small_f64.hip) */
-    if (g_fast_path && eshkol_hip_dgemm_is_small(M, K, N))
-        return eshkol_hip_dgemm_small(A, B, C, M, K, N, trans_a, trans_b, batch, st);
-    if (g_fast_path && batch == 1 && eshkol_hip_dgemm_is_small_long_k(M, K, N))
-        return eshkol_hip_dgemm_small_long_k(A, B, C, M, K, N, trans_a, trans_b, st);
+    if (g_fast_path && eshkol_hip_dgemm_is_small(M, K, N) &&
+        eshkol_hip_dgemm_small(A, B, C, M, K, N, trans_a, trans_b, batch, st) == 0) return 0;
+    /* few outputs, a long k: slices of k over the workgroups */
+    if (g_fast_path && batch == 1 && eshkol_hip_dgemm_is_small_long_k(M, K, N) &&
+        eshkol_hip_dgemm_small_long_k(A, B, C, M, K, N, trans_a, trans_b, st) == 0) return 0;
     /* a vector or a few against a matrix: bound by HBM, not by the matrix cores (dgemv_f64.hip) */
-    if (g_fast_path && batch == 1 && eshkol_hip_dgemm_is_skinny(M, K, N, trans_a, trans_b))
-        return eshkol_hip_dgemm_skinny(A, B, C, M, K, N, trans_a, trans_b, st);
+    if (g_fast_path && batch == 1 && eshkol_hip_dgemm_is_skinny(M, K, N, trans_a, trans_b) &&
+        eshkol_hip_dgemm_skinny(A, B, C, M, K, N, trans_a, trans_b, st) == 0) return 0;
     /* Operands whose rows do not start on 16-byte boundaries (an odd pitch, a base that
      * is not aligned) would take the kernel of 8-byte loads, at two thirds of the rate
      * (4096 x 4096 x 4097: 3.0 ms against 2.1). Where the shape would otherwise run the
