@@ -28,6 +28,7 @@ SOURCES = [
     "dgemm_small_f64.hip",
     "sgemm_f32.hip",
     "igemm_i8.hip",
+    "igemm_thin_i8.hip",
     "hgemm_16.hip",
     "ozaki_crt.hip",
     "ozaki_int8.hip",

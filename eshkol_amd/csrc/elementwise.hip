@@ -83,6 +83,52 @@ void rowabsmax_f64_kernel(const double* __restrict__ A, uint64_t M, uint64_t K,
     }
 }
 
+/* The same for a few long rows (a handful of activation rows in front of a layer): a wave
+ * per row walks 4096 elements from one memory latency to the next (12 us for one row).
+ * Here a workgroup takes a row, every thread with four loads in flight. */
+__global__ __launch_bounds__(256)
+void rowabsmax_few_rows_f64_kernel(const double* __restrict__ A, uint64_t K,
+                                   double zero_value, double* __restrict__ rmax, int32_t* __restrict__ shift, int E) {
+    __shared__ double red[4];
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint64_t row = blockIdx.x;
+    const double* p = A + row * K;
+    double m = 0.0;
+    const bool vec = ((K & 1) == 0) && (((uintptr_t)A & 15) == 0);
+    if (vec) {
+        typedef double d2_t __attribute__((ext_vector_type(2)));
+        const d2_t* p2 = (const d2_t*)p;
+        const uint64_t n2 = K >> 1;
+        for (uint64_t k = tid; k < n2; k += 1024) {
+            d2_t v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) v[u] = (k + 256 * u < n2) ? p2[k + 256 * u] : (d2_t){0.0, 0.0};
+#pragma unroll
+            for (int u = 0; u < 4; u++) { absmax_step(v[u].x, &m); absmax_step(v[u].y, &m); }
+        }
+    } else {
+        for (uint64_t k = tid; k < K; k += 1024) {
+            double v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) v[u] = (k + 256 * u < K) ? p[k + 256 * u] : 0.0;
+#pragma unroll
+            for (int u = 0; u < 4; u++) absmax_step(v[u], &m);
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        double o = __shfl_xor(m, off, 64);
+        if (o > m) m = o;
+    }
+    if (lane == 0) red[wave] = m;
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 1; w < 4; w++) if (red[w] > m) m = red[w];
+        rmax[row] = (m > 0.0) ? m : zero_value;
+        if (shift) shift[row] = shift_of_maximum(m, E);
+    }
+}
+
 /* Column maxima of a row-major X[K][R] in two steps: a block takes 64 columns
  * by one slice of the rows (a wave reads 512 contiguous bytes per row) and
  * writes its partial maxima; the second kernel folds the slices. */
@@ -199,6 +245,11 @@ int eshkol_rowabsmax_shift_f64(const double* A, uint64_t M, uint64_t K, double z
     if (!A || !rmax || M == 0 || K == 0) return -1;
     const uint64_t g = (M + 3) / 4;
     if (g > 0x7fffffffULL) return -1;
+    if (M <= 256 && K >= 1024) {        /* fewer waves than SIMDs, rows long enough to feel it */
+        hipExtLaunchKernelGGL(rowabsmax_few_rows_f64_kernel, dim3((unsigned)M), dim3(256), 0, stream, nullptr, done, 0,
+                              A, K, zero_value, rmax, shift, E);
+        return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+    }
     hipExtLaunchKernelGGL(rowabsmax_f64_kernel, dim3((unsigned)g), dim3(256), 0, stream, nullptr, done, 0,
                           A, M, K, zero_value, rmax, shift, E);
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;

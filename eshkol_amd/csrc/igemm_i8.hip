@@ -38,6 +38,9 @@
 typedef int v4i_t __attribute__((ext_vector_type(4)));
 typedef int v16i_t __attribute__((ext_vector_type(16)));
 
+/* igemm_thin_i8.hip: a first operand of a few rows, interleaved planes */
+int eshkol_hip_igemm_thin(const HipIgemmArgs& a, hipStream_t st);
+
 namespace {
 
 struct I8Op {
@@ -715,11 +718,14 @@ extern "C" void hip_igemm_set_direct(int on) { EshkolHipLock lk; g_direct = (on 
 
 extern "C" void hip_igemm_set_cu_limit(int cus) { EshkolHipLock lk; g_cu_limit = cus > 0 ? cus : 0; }
 
+int eshkol_hip_igemm_direct_mode(void) { return g_direct; }
+
 /* The plane layout the tiers should produce for a contraction of n_out output
  * planes of M x N: 1 (interleaved, for the direct-to-LDS kernel) when the launch
  * has enough 256 x 256 tiles to be worth a workgroup per CU, else 0. */
 extern "C" int hip_igemm_plane_layout(uint64_t M, uint64_t N, int n_out) {
     const uint64_t big = ((M + 255) / 256) * ((N + 255) / 256) * (uint64_t)(n_out > 0 ? n_out : 0);
+    if (eshkol_hip_igemm_is_thin(M)) return 1;     /* streams the second operand's planes */
     return (g_direct != 0 && big >= 128) ? 1 : 0;
 }
 
@@ -745,6 +751,8 @@ extern "C" int hip_igemm_i8(const HipIgemmArgs* args, void* stream) {
          * every output plane with 1..64 products, row counts padded to 256 */
         if (a.ldk % 512 != 0 || a.max_pairs < 1) return -1;
         if ((a.a_plane_stride % (32ull * a.ldk)) || (a.b_plane_stride % (32ull * a.ldk))) return -1;
+        /* a few rows against the second operand's planes: bound by reading those once */
+        if (eshkol_hip_igemm_is_thin(a.M)) return eshkol_hip_igemm_thin(a, st);
         /* Products of at most 1024 bytes of k per row take the 256 x 128 kernel with
          * two workgroups per CU (measured 5 ... 13 % faster there, slower from 2048 on);
          * row counts of B padded to 256 cover its tiles too. g_direct 2 / 3: always / never. */

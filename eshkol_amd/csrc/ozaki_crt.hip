@@ -930,7 +930,10 @@ static int crt_matmul_impl(const double* A, const double* B, double* C,
     /* planes interleaved (and the k pitch padded to whole groups of four 128-byte
      * blocks) when the contraction will take the kernel that wants them so */
     const int layout = hip_igemm_plane_layout(M, N, num_moduli);
-    const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ldk = round_up_sz(K, layout ? 512 : 256);
+    /* a first operand of a few rows goes to the kernel that streams the second operand's
+     * planes: its own planes then need whole blocks of 32 rows only */
+    const bool thin = layout == 1 && eshkol_hip_igemm_is_thin(M);
+    const uint64_t Mp = round_up_sz(M, thin ? 32 : 256), Np = round_up_sz(N, 256), ldk = round_up_sz(K, layout ? 512 : 256);
     /* Both operands come out as planes [row][k]. An operand stored with k
      * contiguous (A as given, B when the caller holds B^T) is read row by row;
      * one stored k-major (B as given, A when the caller holds A^T) is read

@@ -18,15 +18,17 @@ KERNELS = {"simple": (0, 0), "pipelined": (2, 0), "persistent": (2, 1), "pipelin
            "direct": (2, 1),           # interleaved planes, operands loaded straight into LDS / MFMA registers
            "direct-half": (2, 1)}      # the same on 256 x 128 tiles, two workgroups per CU
 DIRECT_MODE = {"direct": 3, "direct-half": 2}
+# interleaved planes; "thin": what the entry point picks by itself for at most 64 rows of A
+INTERLEAVED = set(DIRECT_MODE) | {"thin"}
 
 
 def pad(n, m):
     return (n + m - 1) // m * m
 
 
-def planes(rng, n_planes, rows, K, lo=-128, hi=128):
+def planes(rng, n_planes, rows, K, lo=-128, hi=128, row_pad=256):
     """[n_planes][rows padded to 256][K padded to 256] int8, padding zero."""
-    out = np.zeros((n_planes, pad(rows, 256), pad(K, 256)), np.int8)
+    out = np.zeros((n_planes, pad(rows, row_pad), pad(K, 256)), np.int8)
     out[:, :rows, :K] = rng.integers(lo, hi, (n_planes, rows, K), dtype=np.int8)
     return out
 
@@ -46,8 +48,8 @@ def run(a, b, M, N, plan, mode, kernel, out_rows=0, ldn=0):
     """plan: list of lists of (a_plane, b_plane) per output plane. out_rows, ldn: the output planes as
     allocated (0: M x N); the whole planes come back."""
     lib = ea.load()
-    pf, pers = KERNELS[kernel]
-    if kernel in DIRECT_MODE:
+    pf, pers = KERNELS.get(kernel, (2, 1))
+    if kernel in INTERLEAVED:
         a, b = interleave(a), interleave(b)
     first = np.cumsum([0] + [len(p) for p in plan]).astype(np.int32)
     pa = np.array([t[0] for p in plan for t in p], np.int32)
@@ -64,7 +66,7 @@ def run(a, b, M, N, plan, mode, kernel, out_rows=0, ldn=0):
     g.ldk, g.M, g.N, g.n_out = a.shape[2], M, N, n_out
     g.pair_first, g.pair_a, g.pair_b = dF.ptr, dPa.ptr, dPb.ptr
     g.mode, g.max_pairs, g.modulus = mode, max(len(p) for p in plan), dMod.ptr
-    g.layout = 1 if kernel in DIRECT_MODE else 0
+    g.layout = 1 if kernel in INTERLEAVED else 0
     if mode == 1:
         g.out_i8 = out.ptr
     else:
@@ -124,6 +126,59 @@ def test_output_planes_larger_than_the_product(gpu, M, K, N, out_rows, ldn, mode
     rest[:, :M, :N] = 0
     fill = 0x55
     assert np.all((rest == 0) | (rest == fill))
+
+
+THIN_SHAPES = [(1, 512, 32), (5, 700, 100), (32, 4096, 1024), (33, 1000, 1300), (64, 2049, 257), (17, 130, 4096)]
+
+
+@pytest.mark.parametrize("M,K,N", THIN_SHAPES)
+def test_thin_first_operand_residues(gpu, M, K, N):
+    """At most 64 rows of A, planes padded to whole blocks of 32 rows only: the kernel that streams B's planes."""
+    rng = np.random.default_rng(M + K + N)
+    a, b = planes(rng, 16, M, K, row_pad=32), planes(rng, 16, N, K)
+    plan = [[(l, l)] for l in range(16)]
+    got = run(a, b, M, N, plan, 1, "thin")
+    want = exact(a, b, M, N, K, plan)
+    for l, p in enumerate(MODULI):
+        assert np.array_equal(got[l].astype(np.int64), symmetric(want[l], p)), (l, p)
+    # the tiled kernel on the same operands (rows padded to its 256): the same bytes
+    a256 = np.zeros((16, 256, a.shape[2]), np.int8)
+    a256[:, :a.shape[1]] = a
+    assert np.array_equal(run(a256, b, M, N, plan, 1, "direct"), got)
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("M,K,N,out_rows,ldn", [(7, 700, 100, 7, 112), (40, 512, 1030, 40, 1280), (64, 300, 33, 64, 33),
+                                                (3, 1024, 95, 5, 95), (32, 520, 64, 32, 66)])
+def test_thin_first_operand_plans_and_output_pitches(gpu, M, K, N, out_rows, ldn, mode):
+    """Several products per output plane (the slice tier's plans), int32 sums and residues, output planes with
+    a pitch of their own, also one that keeps no store aligned."""
+    rng = np.random.default_rng(M + N + mode)
+    a, b = planes(rng, 3, M, K, row_pad=32), planes(rng, 3, N, K)
+    plan = [[(0, 0)], [(1, 1), (2, 2)], [(0, 2), (1, 0), (2, 1)]]
+    got = run(a, b, M, N, plan, mode, "thin", out_rows, ldn)
+    want = exact(a, b, M, N, K, plan)
+    if mode == 1:
+        want = np.stack([symmetric(want[l], MODULI[l]) for l in range(3)])
+    assert np.array_equal(got[:, :M, :N].astype(np.int64), want)
+    rest = got.copy()
+    rest[:, :M, :N] = 0
+    assert np.all((rest == 0) | (rest == 0x55))
+
+
+def test_thin_first_operand_extremes_of_the_accumulator(gpu):
+    """All -128 against -128 and against 127 at the largest K: both ends of the int32 range."""
+    M, N, K = 9, 96, 131072 - 256
+    a = np.full((16, 32, K), -128, np.int8)
+    a[:, M:] = 0
+    b = np.full((16, 256, K), -128, np.int8)
+    b[:, 1::2, :] = 127
+    b[:, N:] = 0
+    plan = [[(l, l)] for l in range(16)]
+    got = run(a, b, M, N, plan, 1, "thin")
+    want = exact(a, b, M, N, K, plan)
+    for l, p in enumerate(MODULI):
+        assert np.array_equal(got[l].astype(np.int64), symmetric(want[l], p)), (l, p)
 
 
 @pytest.mark.parametrize("kernel", list(KERNELS))

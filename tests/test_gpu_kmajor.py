@@ -43,6 +43,27 @@ def test_column_maxima(gpu, K, R):
         assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("rows,K", [(1, 1024), (5, 4096), (64, 4097), (256, 1031), (3, 131071), (7, 5002)])
+def test_row_maxima_of_a_few_long_rows(gpu, rows, K):
+    """A handful of rows in front of a layer: a workgroup per row. Also from a base that is
+    not a multiple of 16 bytes, with a zero row and a row that holds a NaN."""
+    lib = ea.load()
+    X = synth.wide_range(rows * 7 + K, (rows, K))
+    if rows > 2:
+        X[1, :] = 0.0
+        X[2, K - 1] = np.nan
+    flat = dev(np.concatenate([[0.0], X.ravel()]))
+    for base, zero_value in ((dev(X).ptr, 0.0), (flat.ptr + 8, 1.0)):
+        out = ea.DeviceArray((rows,))
+        assert lib.hip_rowabsmax_f64(base, rows, K, zero_value, out.ptr, stream()) == 0
+        ea.synchronize()
+        got = out.download()
+        want = np.abs(X).max(axis=1)
+        want[want == 0.0] = zero_value
+        want[np.isnan(want)] = np.inf
+        assert np.array_equal(got, want)
+
+
 def test_column_maxima_flag_non_finite_input(gpu):
     lib = ea.load()
     X = synth.normal(3, (200, 70))

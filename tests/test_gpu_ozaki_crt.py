@@ -30,7 +30,8 @@ def check_all_stages(A, B, num_moduli=16, adaptive=False):
 SHAPES = [(1, 1, 1), (5, 3, 4), (64, 128, 64), (100, 200, 90), (257, 129, 255), (300, 1000, 17),
           (512, 512, 512), (33, 2049, 65), (768, 640, 1024),
           (3, 131071, 2),                      # the largest K the tier accepts
-          (3001, 2, 2), (2, 2, 3001), (1, 1031, 513)]
+          (3001, 2, 2), (2, 2, 3001), (1, 1031, 513),
+          (8, 4096, 1024), (32, 1024, 2048), (64, 1000, 777), (65, 1000, 777)]      # a few rows against a layer
 
 
 @pytest.mark.parametrize("M,K,N", SHAPES)
