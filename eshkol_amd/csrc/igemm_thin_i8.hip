@@ -12,7 +12,12 @@
  *     pieces of 8 KiB, every lane with eight 16-byte loads in flight, so that the launch
  *     has thousands of waves and tens of megabytes on their way at any time;
  *   - the first operand (32 or 64 rows, read by every workgroup of the plane) comes from
- *     the L2;
+ *     the L2, every wave fetching the fragments it needs for itself. That is what bounds
+ *     the row count: the L2 delivered about 11 TB/s to the CUs whatever the split, so with
+ *     R blocks of 32 rows and C column blocks per workgroup the stream gets 1 / (1 + R / C)
+ *     of it (5.7 TB/s at R 1 C 2, 4.5 at R 2 C 2, 3.2 at R 4 C 2: no better than the
+ *     tiled kernels, which is why this stops at 64 rows). Two column blocks per workgroup
+ *     where that still leaves a couple of thousand workgroups, else one;
  *   - the four partial sums meet in LDS; every thread then owns four consecutive columns
  *     of one row, reduces them modulo p (mode 1, the arithmetic of the tiled kernels'
  *     epilogue) and stores one word, or the four int32 sums (mode 0).
@@ -26,7 +31,6 @@ typedef int v4i_t __attribute__((ext_vector_type(4)));
 typedef int v16i_t __attribute__((ext_vector_type(16)));
 
 namespace {
-
 
 /* Four consecutive columns of one output row: the int32 sums (mode 0) or their residues
  * modulo p packed into one word (mode 1). col is a multiple of 4.

@@ -649,10 +649,10 @@ bool ensure_mailbox() {
     g_mailbox = (CrtScan*)h; g_mailbox_dev = (CrtScan*)d;
     return true;
 }
-/* 0 when both halves carry `ticket` */
-int await_mailbox(uint32_t ticket, hipStream_t st) {
+/* 0 when both halves carry `ticket` (halves == 1: the first, the only one that scan wrote) */
+int await_mailbox(uint32_t ticket, hipStream_t st, int halves) {
     volatile uint32_t* r0 = &g_mailbox[0].ready;
-    volatile uint32_t* r1 = &g_mailbox[1].ready;
+    volatile uint32_t* r1 = &g_mailbox[halves == 2 ? 1 : 0].ready;
     const auto t0 = std::chrono::steady_clock::now();
     for (unsigned spin = 0; *r0 != ticket || *r1 != ticket; spin++) {
         if ((spin & 1023) == 1023 &&
@@ -669,12 +669,14 @@ int await_mailbox(uint32_t ticket, hipStream_t st) {
 /* Queues the scan of the two vectors of maxima; 0 on failure, else the ticket its
  * summary will carry. */
 hipStream_t g_scan_ran_on = nullptr;  /* the stream the last scan was queued on: what a wait drains if the ticket does not show */
+int g_scan_halves = 2;                /* 1: the last scan looked at A's maxima only (B's summary was kept when B was prepared) */
 uint32_t scan_launch(const double* amax, uint64_t M, const double* bmax, uint64_t N,
-                     int32_t* fl_a, int32_t* fl_b, hipStream_t st) {
+                     int32_t* fl_a, int32_t* fl_b, hipStream_t st, int halves = 2) {
     if (!ensure_mailbox()) return 0;
     g_scan_ran_on = st;
+    g_scan_halves = halves;
     const uint32_t ticket = ++g_ticket ? g_ticket : ++g_ticket;            /* never 0: the mailbox starts zeroed */
-    hipLaunchKernelGGL(crt_scan_kernel, dim3(2), dim3(SCAN_THREADS), 0, st, amax, M, bmax, N, fl_a, fl_b,
+    hipLaunchKernelGGL(crt_scan_kernel, dim3(halves), dim3(SCAN_THREADS), 0, st, amax, M, bmax, N, fl_a, fl_b,
                        g_mailbox_dev, ticket);
     return ESHKOL_HIP_OK(hipGetLastError()) ? ticket : 0;
 }
@@ -690,15 +692,16 @@ hipEvent_t scan_event(uint64_t operand_elems) {
 /* event_attached: the caller made scan_event() the completion event of the last
  * kernel the scan depends on, so no marker needs to be queued behind st. */
 uint32_t scan_launch_aside(const double* amax, uint64_t M, const double* bmax, uint64_t N, hipStream_t st,
-                           uint64_t operand_elems, bool event_attached) {
+                           uint64_t operand_elems, bool event_attached, int halves = 2) {
     if (!ensure_mailbox()) return 0;
-    if (operand_elems < ASIDE_FROM) return scan_launch(amax, M, bmax, N, nullptr, nullptr, st);
+    if (operand_elems < ASIDE_FROM) return scan_launch(amax, M, bmax, N, nullptr, nullptr, st, halves);
     if ((!event_attached && !ESHKOL_HIP_OK(hipEventRecord(g_scan_event, st))) ||
         !ESHKOL_HIP_OK(hipStreamWaitEvent(g_scan_stream, g_scan_event, 0))) return 0;
-    return scan_launch(amax, M, bmax, N, nullptr, nullptr, g_scan_stream);
+    return scan_launch(amax, M, bmax, N, nullptr, nullptr, g_scan_stream, halves);
 }
+/* the mailbox once the scan that carries `ticket` has written it (its second half is that scan's only if it had two) */
 const CrtScan* scan_await(uint32_t ticket) {
-    return (ticket != 0 && await_mailbox(ticket, g_scan_ran_on) == 0) ? g_mailbox : nullptr;
+    return (ticket != 0 && await_mailbox(ticket, g_scan_ran_on, g_scan_halves) == 0) ? g_mailbox : nullptr;
 }
 
 /* device-resident constant tables for the contraction: identity pair lists and moduli */
@@ -896,6 +899,7 @@ struct CrtPreparedB {
     double* bmax;               /* [N] column maxima, device */
     int32_t* nu;                /* [N] shifts 52 - floor(log2 max), device */
     int8_t* planes;             /* [n_mod][rows_padded][ldk], device */
+    CrtScan scan;               /* the scan's summary of bmax: it does not change either */
 };
 constexpr uint32_t PREPARED_MAGIC = 0x43525442u;
 }  // namespace
@@ -977,9 +981,18 @@ static int crt_matmul_impl(const double* A, const double* B, double* C,
     if (!use_prepared &&
         (b_kmajor ? eshkol_colabsmax_shift_f64(B, K, N, 0.0, bmax, nu_out, 52, st, fork_b)
                   : eshkol_rowabsmax_shift_f64(B, N, K, 0.0, bmax, nu_out, 52, st, fork_b)) != 0) return -1;
-    const uint32_t ticket = fixed_E ? scan_launch_aside(amax, M, bmax, N, st, M * K + K * N, fork != nullptr)
+    /* prepared planes: the scan looks at A's maxima only, B's summary was kept with the planes */
+    const uint32_t ticket = fixed_E ? scan_launch_aside(amax, M, bmax, N, st, M * K + K * N, fork != nullptr, use_prepared ? 1 : 2)
                                     : scan_launch(amax, M, bmax, N, dmu, dnu, st);
     if (!ticket) return -1;
+    CrtScan merged[2];
+    auto await_scan = [&]() -> const CrtScan* {
+        const CrtScan* h = scan_await(ticket);
+        if (!h || !use_prepared) return h;
+        merged[0] = h[0];
+        merged[1] = prepared->scan;
+        return merged;
+    };
 
     /* Everything after the shifts, queued in one go. */
     auto enqueue_products = [&](int n_mod, const HostCrt& crt, int E, bool b_ready) -> int {
@@ -1031,7 +1044,7 @@ static int crt_matmul_impl(const double* A, const double* B, double* C,
         if (enqueue_products(num_moduli, crt, E, use_prepared) != 0) return -1;
         announce(num_moduli, crt);
         announced = true;
-        h_scan = scan_await(ticket);
+        h_scan = await_scan();
         if (!h_scan) return -1;
         if (h_scan[0].nonfinite || h_scan[1].nonfinite) return -1;  /* NaN/Inf input */
         if (!h_scan[0].extreme && !h_scan[1].extreme) {
@@ -1040,7 +1053,7 @@ static int crt_matmul_impl(const double* A, const double* B, double* C,
             return 0;
         }
     }
-    if (!h_scan) h_scan = scan_await(ticket);
+    if (!h_scan) h_scan = await_scan();
     if (!h_scan) return -1;
     if (h_scan[0].nonfinite || h_scan[1].nonfinite) return -1;          /* NaN/Inf input */
 
@@ -1154,6 +1167,7 @@ extern "C" int hip_ozaki_crt_prepare_operand_b(const double* B, uint64_t K, uint
     const CrtScan* h = scan_await(scan_launch(pb->bmax, N, pb->bmax, N, nullptr, nullptr, st));
     if (!h || h[1].nonfinite || h[1].extreme) return fail();     /* such a B takes the full pass on every call */
     if (h[1].nonzero && !(52 - h[1].e_min <= 1023 && 52 - h[1].e_max >= -1022)) return fail();
+    pb->scan = h[1];
     if (crt_split_any(B, N, K, pb->nu, num_moduli, pb->planes, Np, ldk, b_kmajor, layout, st) != 0) return fail();
     if (!ESHKOL_HIP_OK(hipStreamSynchronize(st))) return fail();
     *handle = pb;
