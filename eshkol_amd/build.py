@@ -25,6 +25,7 @@ SOURCES = [
     "host_copy.cpp",
     "dgemm_f64.hip",
     "dgemv_f64.hip",
+    "dgemm_thin_f64.hip",
     "dgemm_small_f64.hip",
     "sgemm_f32.hip",
     "igemm_i8.hip",
@@ -46,6 +47,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # AGPR half of the register file (measured: 36 vs 78 TFLOP/s on a register-only
 # loop); the int8 and 16-bit MFMAs do not care. Keep fp64 accumulators in VGPRs.
 EXTRA = {"dgemm_f64.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+         "dgemm_thin_f64.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
          "peak_probe.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 # -ffp-contract=off: every fused multiply-add the arithmetic relies on is

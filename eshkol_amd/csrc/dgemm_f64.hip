@@ -916,10 +916,13 @@ int dgemm_any(const double* A, const double* B, double* C, uint64_t M, uint64_t 
     /* matrices far smaller than a tile, one or many: several to a workgroup (dgemm_small_f64.hip) */
     if (g_fast_path && eshkol_hip_dgemm_is_small(M, K, N) &&
         eshkol_hip_dgemm_small(A, B, C, M, K, N, trans_a, trans_b, batch, st) == 0) return 0;
+    /* up to 64 rows (or columns) against a matrix: streamed through the matrix cores (dgemm_thin_f64.hip) */
+    if (g_fast_path && batch == 1 && eshkol_hip_dgemm_is_thin_rows(M, K, N, trans_a, trans_b) &&
+        eshkol_hip_dgemm_thin_rows(A, B, C, M, K, N, trans_a, trans_b, st) == 0) return 0;
     /* few outputs, a long k: slices of k over the workgroups */
     if (g_fast_path && batch == 1 && eshkol_hip_dgemm_is_small_long_k(M, K, N) &&
         eshkol_hip_dgemm_small_long_k(A, B, C, M, K, N, trans_a, trans_b, st) == 0) return 0;
-    /* a vector or a few against a matrix: bound by HBM, not by the matrix cores (dgemv_f64.hip) */
+    /* a vector against a matrix with k contiguous: plain fma loops at the rate of HBM (dgemv_f64.hip) */
     if (g_fast_path && batch == 1 && eshkol_hip_dgemm_is_skinny(M, K, N, trans_a, trans_b) &&
         eshkol_hip_dgemm_skinny(A, B, C, M, K, N, trans_a, trans_b, st) == 0) return 0;
     /* Operands whose rows do not start on 16-byte boundaries (an odd pitch, a base that

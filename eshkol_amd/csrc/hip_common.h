@@ -129,11 +129,17 @@ bool eshkol_hip_dgemm_is_small_long_k(uint64_t M, uint64_t K, uint64_t N);
 int eshkol_hip_dgemm_small_long_k(const double* A, const double* B, double* C, uint64_t M, uint64_t K, uint64_t N,
                                   int trans_a, int trans_b, hipStream_t st);
 
-/* fp64 products with one thin side (dgemv_f64.hip): whether the shape is one, and the
- * product itself. hip_dgemm_f64 and hip_dgemm_f64_ex send such shapes there. */
+/* One vector against a matrix held with k contiguous (dgemv_f64.hip): whether the shape is
+ * one, and the product itself. hip_dgemm_f64 and hip_dgemm_f64_ex send such shapes there. */
 bool eshkol_hip_dgemm_is_skinny(uint64_t M, uint64_t K, uint64_t N, int trans_a, int trans_b);
 int eshkol_hip_dgemm_skinny(const double* A, const double* B, double* C, uint64_t M, uint64_t K, uint64_t N,
                             int trans_a, int trans_b, hipStream_t st);
+
+/* fp64 products with up to 64 rows on the thin side: the big operand streamed through the
+ * matrix cores (dgemm_thin_f64.hip) */
+bool eshkol_hip_dgemm_is_thin_rows(uint64_t M, uint64_t K, uint64_t N, int trans_a, int trans_b);
+int eshkol_hip_dgemm_thin_rows(const double* A, const double* B, double* C, uint64_t M, uint64_t K, uint64_t N,
+                               int trans_a, int trans_b, hipStream_t st);
 
 #ifdef __HIPCC__
 template <class T>

@@ -223,11 +223,12 @@ def test_native_large_operands_with_a_base_off_16_byte_boundaries(gpu):
     assert np.array_equal(dC.download(), A @ B)
 
 
-@pytest.mark.parametrize("thin", [1, 2, 3, 5, 8, 9, 16, 17, 32])
+@pytest.mark.parametrize("thin", [1, 2, 3, 5, 8, 9, 16, 17, 32, 33, 48, 64, 65])
 @pytest.mark.parametrize("wide,K", [(1024, 1024), (1025, 1031), (4096, 100), (3001, 2050), (4097, 4100)])
 def test_native_products_with_one_thin_side(gpu, thin, wide, K):
-    """A vector or a few against a matrix (M or N at most 16) take kernels of their own, bound by HBM, in all
-    three operand forms and with either side thin. Integer operands make every sum exact, so the result must
+    """A vector or a few against a matrix take kernels of their own, bound by HBM (up to 64 rows where the big
+    operand has the output index contiguous: the matrix cores stream it), in all three operand forms and with
+    either side thin. Integer operands make every sum exact, so the result must
     be the integer product bit for bit; random operands must stay within the tier's tolerance."""
     print("dgemm_ex, thin side", thin, wide, K, flush=True)
     rng = np.random.default_rng(thin * 7 + wide + K)
@@ -261,7 +262,7 @@ def test_native_products_thin_on_both_sides_keep_the_tiled_kernel(gpu, M, K, N):
 def test_native_thin_products_write_nothing_else(gpu):
     """The result of a thin product lies in a buffer with guard values around it."""
     lib = ea.load()
-    for (M, K, N) in ((3, 777, 2049), (2049, 777, 3), (1, 4096, 4097), (4097, 4096, 1)):
+    for (M, K, N) in ((3, 777, 2049), (2049, 777, 3), (1, 4096, 4097), (4097, 4096, 1), (33, 1031, 2049), (2049, 1031, 48)):
         rng = np.random.default_rng(M + N)
         A = rng.integers(-9, 10, (M, K)).astype(np.float64)
         B = rng.integers(-9, 10, (K, N)).astype(np.float64)
@@ -272,6 +273,33 @@ def test_native_thin_products_write_nothing_else(gpu):
         out = buf.download()
         assert np.all(out[:64] == -7.25) and np.all(out[64 + M * N:] == -7.25)
         assert np.array_equal(out[64:64 + M * N].reshape(M, N), A @ B)
+
+
+def test_native_batch_of_rows_against_a_matrix_with_infinities_and_an_odd_base(gpu):
+    """9 ... 64 rows against a matrix read through the matrix cores: an infinity in the big operand shows in its
+    own column only (the zeros that pad the last round of k must not meet it), also when k is not a multiple of
+    the round and the strip of columns is cut; operands whose base is 8 bytes off a 16-byte boundary."""
+    lib = ea.load()
+    M, K, N = 20, 1031, 1100
+    rng = np.random.default_rng(5)
+    A = rng.integers(-9, 10, (M, K)).astype(np.float64)
+    B = rng.integers(-9, 10, (K, N)).astype(np.float64)
+    A[:, K - 1] = np.abs(A[:, K - 1]) + 1.0
+    B[K - 1, 7] = np.inf
+    B[3, N - 1] = -np.inf
+    A[:, 3] = np.abs(A[:, 3]) + 1.0
+    bufA = ea.DeviceArray.from_host(np.concatenate([[0.0], A.ravel()]))
+    bufB = ea.DeviceArray.from_host(np.concatenate([[0.0], B.ravel()]))
+    out = ea.DeviceArray.from_host(np.zeros(M * N + 1))
+    assert lib.hip_dgemm_f64(bufA.ptr + 8, bufB.ptr + 8, out.ptr + 8, M, K, N, stream()) == 0
+    ea.synchronize()
+    got = out.download()[1:].reshape(M, N)
+    with np.errstate(invalid="ignore"):
+        want = A @ B
+    assert np.all(got[:, 7] == np.inf) and np.all(got[:, N - 1] == -np.inf)
+    keep = np.ones(N, bool)
+    keep[[7, N - 1]] = False
+    assert np.array_equal(got[:, keep], want[:, keep])
 
 
 @pytest.mark.parametrize("batch,M,K,N", [(1, 1, 1, 1), (1, 3, 3, 3), (7, 3, 3, 3), (4096, 8, 8, 8), (1000, 5, 7, 6), (513, 16, 16, 16),
