@@ -525,7 +525,53 @@ def main():
                     "maxima and residue planes computed once instead of on every forward pass"}
         log("mlp forward (exact tier): %.3f ms %.1f GFLOP/s-eq; with prepared weights %.3f ms (same bits: %s)"
             % (w7, mlp_flops / (w7 * 1e-3) / 1e9, w7p, same))
-        for d in [X] + Ws + bs + acts:
+        # the same layers in front of a batch of 32 rows: bound by reading the weights once (their
+        # sixteen residue planes in the exact tier, the fp64 values in the native one)
+        small = 32
+        Xs = ea.DeviceArray.from_host(synth.normal(73, (small, dims[0])))
+        acts_s = [ea.DeviceArray((small, dims[i + 1])) for i in range(3)]
+        handles = []
+        for i in range(3):
+            h = C.c_void_p()
+            assert lib.hip_ozaki_crt_prepare_operand_b(Ws[i].ptr, dims[i], dims[i + 1], 0, 16, small, C.byref(h), st) == 0
+            handles.append(h)
+
+        def small_prepared():
+            src = Xs
+            for i in range(3):
+                rc = lib.hip_matmul_ozaki_crt_prepared_f64(src.ptr, handles[i], acts_s[i].ptr, small, dims[i], dims[i + 1],
+                                                           0, 16, 0, bs[i].ptr, 1, st)
+                if rc != 0:
+                    return rc
+                src = acts_s[i]
+            return 0
+
+        def small_native():
+            src = Xs
+            for i in range(3):
+                rc = lib.hip_dgemm_f64(src.ptr, Ws[i].ptr, acts_s[i].ptr, small, dims[i], dims[i + 1], st)
+                rc = rc or lib.hip_bias_act_f64(acts_s[i].ptr, bs[i].ptr, small, dims[i + 1], 1, st)
+                if rc != 0:
+                    return rc
+                src = acts_s[i]
+            return 0
+        os.dup2(devnull, 2)
+        try:
+            _, ws_p = timed(small_prepared, k=20, w=5)
+            _, ws_n = timed(small_native, k=20, w=5)
+        finally:
+            os.dup2(saved, 2)
+        for h in handles:
+            lib.hip_ozaki_crt_release_prepared(h)
+        weight_elems = float(sum(dims[i] * dims[i + 1] for i in range(3)))
+        tiers["mlp_forward_batch32_1024_4096_4096_1024"] = {
+            "exact_tier_prepared_weights_ms": ws_p, "native_fp64_ms": ws_n,
+            "exact_tier_weight_planes_GBps": 16.0 * weight_elems / (ws_p * 1e-3) / 1e9,
+            "native_weights_GBps": 8.0 * weight_elems / (ws_n * 1e-3) / 1e9,
+            "note": "whole forward passes (max, split, contraction, reconstruct per layer; GEMM and bias + tanh per layer); "
+                    "the rates count the weights' bytes once over the whole pass"}
+        log("mlp forward, batch 32: exact tier with prepared weights %.3f ms, native fp64 %.3f ms" % (ws_p, ws_n))
+        for d in [X, Xs] + Ws + bs + acts + acts_s:
             d.free()
 
     # ---- smaller cubes: where each tier starts to pay (the crossover the reference documents at
