@@ -278,26 +278,32 @@ void launch_rows(bool klast, const double* T, long t_r, long t_k, int R, const d
 }
 
 int g_thin_rows = 1;        /* fewest rows sent here; 0: none (tuning) */
-int g_thin_rows_klast = 1;  /* 0: only big operands with the output index contiguous (tuning) */
+int g_thin_rows_klast = 1;
+int g_thin_min_kc = 0;       /* fewest k per slice, 0: by the shape (tuning) */
+int g_thin_min_wide = 16;    /* narrowest big operand (tuning) */
+int g_thin_min_log2 = 13;    /* smallest big operand, log2 of its elements (tuning) */
 
 }  // namespace
 
 extern "C" void hip_dgemm_set_thin_rows(int from) { EshkolHipLock lk; g_thin_rows = from > 0 ? from : 0; }
+extern "C" void hip_dgemm_set_thin_tuning(int min_kc, int min_wide, int min_log2) { EshkolHipLock lk; g_thin_min_kc = min_kc; g_thin_min_wide = min_wide; g_thin_min_log2 = min_log2; }
 extern "C" void hip_dgemm_set_thin_rows_klast(int on) { EshkolHipLock lk; g_thin_rows_klast = on ? 1 : 0; }
 
-/* Up to 64 rows on the thin side and a big operand that is worth streaming; one vector
- * against a matrix with k contiguous is left to dgemv_f64.hip, and the widest thin sides
- * on a short k to the tiled kernels (64 x 300 x 4000: 17 us here, 13 there). */
+/* Up to 64 rows on the thin side. The other side may be narrow too where k is long
+ * (32 x 4109 x 36: 34 us on the tiled kernels, which have one tile to cut along k, 10
+ * here); what the tiled kernels keep is the widest thin sides on a short k
+ * (64 x 300 x 4000: 17 us here, 13 there) and operands of a few thousand elements. One
+ * vector against a matrix with k contiguous is left to dgemv_f64.hip. */
 bool eshkol_hip_dgemm_is_thin_rows(uint64_t M, uint64_t K, uint64_t N, int trans_a, int trans_b) {
     if (!g_thin_rows) return false;
     const bool thin_m = M <= N;
     const uint64_t thin = thin_m ? M : N, wide = thin_m ? N : M;
     const bool kfirst = thin_m ? !trans_b : (trans_a != 0);
     if (!kfirst && (!g_thin_rows_klast || thin < 2)) return false;
-    if (thin < (uint64_t)g_thin_rows || thin > 64 || wide < 128 || K < 64) return false;
+    if (thin < (uint64_t)g_thin_rows || thin > 64 || wide < (uint64_t)g_thin_min_wide || K < 64) return false;
     if (thin > 48 && K < 512) return false;
     if (K > 0x7fffffffULL || wide > 0x7fffffffULL) return false;
-    return wide * K >= (1ull << 17);
+    return wide * K >= (1ull << g_thin_min_log2);
 }
 
 int eshkol_hip_dgemm_thin_rows(const double* A, const double* B, double* C, uint64_t M, uint64_t K, uint64_t N,
@@ -315,7 +321,10 @@ int eshkol_hip_dgemm_thin_rows(const double* A, const double* B, double* C, uint
      * at least four rounds of 64 k per workgroup */
     const int strips = (O + 63) / 64;
     int slices = (3 * eshkol_hip_num_cus()) / strips;
-    if (slices > k / 256) slices = k / 256;
+    /* a slice of at least 256 k, shorter where the strips are few or k is short (more slices
+     * are all the parallelism such a launch has) */
+    const int min_kc = g_thin_min_kc ? g_thin_min_kc : strips <= 2 ? 64 : (strips <= 4 || k < 2048) ? 128 : 256;
+    if (slices > k / min_kc) slices = k / min_kc;
     if (slices > 128) slices = 128;                 /* the sum walks them one thread per output */
     if (slices < 1) slices = 1;
     int kc = (k + slices - 1) / slices;
