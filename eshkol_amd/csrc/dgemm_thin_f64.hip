@@ -54,6 +54,10 @@ void dgemm_thin_rows_kernel(const double* __restrict__ T, long t_r, long t_k, in
     const int ks = (int)blockIdx.y * kc;
     const int ke = (ks + kc < K) ? ks + kc : K;
     const bool cols_in = o + 3 < O;
+    /* more than 64 thin rows: a chunk of 64 per blockIdx.z */
+    T += (long)blockIdx.z * 64 * t_r;
+    out += (long)blockIdx.z * 64 * c_r;
+    R = (R - 64 * (int)blockIdx.z < 64) ? R - 64 * (int)blockIdx.z : 64;
     v4d_t acc[RB][4];
 #pragma unroll
     for (int rb = 0; rb < RB; rb++)
@@ -166,6 +170,9 @@ void dgemm_thin_rows_klast_kernel(const double* __restrict__ T, long t_r, long t
     const int ob = (int)blockIdx.x * 64;
     const int ks = (int)blockIdx.y * kc;
     const int ke = (ks + kc < K) ? ks + kc : K;
+    T += (long)blockIdx.z * 64 * t_r;
+    out += (long)blockIdx.z * 64 * c_r;
+    R = (R - 64 * (int)blockIdx.z < 64) ? R - 64 * (int)blockIdx.z : 64;
     v4d_t acc[RB][4];
 #pragma unroll
     for (int rb = 0; rb < RB; rb++)
@@ -265,7 +272,7 @@ void dgemm_thin_rows_sum_kernel(const double* __restrict__ part, int slices, int
 template <int RB>
 void launch_rows(bool klast, const double* T, long t_r, long t_k, int R, const double* G, long ldg, int K, int O, int kc,
                  int slices, double* out, long c_r, long c_o, long slice_stride, hipStream_t st) {
-    const dim3 grid((unsigned)((O + 63) / 64), (unsigned)slices);
+    const dim3 grid((unsigned)((O + 63) / 64), (unsigned)slices, (unsigned)((R + 63) / 64));
     if (!klast)
         hipLaunchKernelGGL(dgemm_thin_rows_kernel<RB>, grid, dim3(256), 0, st,
                            T, t_r, t_k, R, G, ldg, K, O, kc, out, c_r, c_o, slice_stride);
@@ -281,12 +288,14 @@ int g_thin_rows = 1;        /* fewest rows sent here; 0: none (tuning) */
 int g_thin_rows_klast = 1;
 int g_thin_min_kc = 0;       /* fewest k per slice, 0: by the shape (tuning) */
 int g_thin_min_wide = 16;    /* narrowest big operand (tuning) */
+int g_thin_chunks = 1;       /* 0: no more than 64 thin rows (tuning) */
 int g_thin_min_log2 = 13;    /* smallest big operand, log2 of its elements (tuning) */
 
 }  // namespace
 
 extern "C" void hip_dgemm_set_thin_rows(int from) { EshkolHipLock lk; g_thin_rows = from > 0 ? from : 0; }
 extern "C" void hip_dgemm_set_thin_tuning(int min_kc, int min_wide, int min_log2) { EshkolHipLock lk; g_thin_min_kc = min_kc; g_thin_min_wide = min_wide; g_thin_min_log2 = min_log2; }
+extern "C" void hip_dgemm_set_thin_chunks(int on) { EshkolHipLock lk; g_thin_chunks = on ? 1 : 0; }
 extern "C" void hip_dgemm_set_thin_rows_klast(int on) { EshkolHipLock lk; g_thin_rows_klast = on ? 1 : 0; }
 
 /* Up to 64 rows on the thin side. The other side may be narrow too where k is long
@@ -300,8 +309,17 @@ bool eshkol_hip_dgemm_is_thin_rows(uint64_t M, uint64_t K, uint64_t N, int trans
     const uint64_t thin = thin_m ? M : N, wide = thin_m ? N : M;
     const bool kfirst = thin_m ? !trans_b : (trans_a != 0);
     if (!kfirst && (!g_thin_rows_klast || thin < 2)) return false;
-    if (thin < (uint64_t)g_thin_rows || thin > 64 || wide < (uint64_t)g_thin_min_wide || K < 64) return false;
+    if (thin < (uint64_t)g_thin_rows || wide < (uint64_t)g_thin_min_wide || K < 64) return false;
     if (thin > 48 && K < 512) return false;
+    if (thin > 64) {
+        /* chunks of 64 rows, each reading the big operand again: where the tiled kernels would
+         * have a few dozen tiles and a long k to walk, and the big operand stays in the caches
+         * (135 x 2559 x 349: 50 -> 23 us, 70 x 32768 x 128: 71 -> 38; 250 x 4096 x 700 would
+         * go from 43 to 54) */
+        if (!g_thin_chunks || thin > 256 || K < 1024) return false;
+        const uint64_t blocks = ((thin + 63) / 64) * ((wide + 63) / 64);
+        if (blocks > 48 || (wide * K > (2ull << 20) && blocks > 8)) return false;
+    }
     if (K > 0x7fffffffULL || wide > 0x7fffffffULL) return false;
     return wide * K >= (1ull << g_thin_min_log2);
 }
@@ -320,7 +338,8 @@ int eshkol_hip_dgemm_thin_rows(const double* A, const double* B, double* C, uint
     /* slices of k where the strips alone leave CUs idle: about three workgroups per CU,
      * at least four rounds of 64 k per workgroup */
     const int strips = (O + 63) / 64;
-    int slices = (3 * eshkol_hip_num_cus()) / strips;
+    const int chunks = (R + 63) / 64;
+    int slices = (3 * eshkol_hip_num_cus()) / (strips * chunks);
     /* a slice of at least 256 k, shorter where the strips are few or k is short (more slices
      * are all the parallelism such a launch has) */
     const int min_kc = g_thin_min_kc ? g_thin_min_kc : strips <= 2 ? 64 : (strips <= 4 || k < 2048) ? 128 : 256;

@@ -262,7 +262,8 @@ def test_native_products_thin_on_both_sides_keep_the_tiled_kernel(gpu, M, K, N):
 def test_native_thin_products_write_nothing_else(gpu):
     """The result of a thin product lies in a buffer with guard values around it."""
     lib = ea.load()
-    for (M, K, N) in ((3, 777, 2049), (2049, 777, 3), (1, 4096, 4097), (4097, 4096, 1), (33, 1031, 2049), (2049, 1031, 48)):
+    for (M, K, N) in ((3, 777, 2049), (2049, 777, 3), (1, 4096, 4097), (4097, 4096, 1), (33, 1031, 2049), (2049, 1031, 48),
+                      (135, 2559, 349), (20, 3000, 18)):
         rng = np.random.default_rng(M + N)
         A = rng.integers(-9, 10, (M, K)).astype(np.float64)
         B = rng.integers(-9, 10, (K, N)).astype(np.float64)
@@ -273,6 +274,25 @@ def test_native_thin_products_write_nothing_else(gpu):
         out = buf.download()
         assert np.all(out[:64] == -7.25) and np.all(out[64 + M * N:] == -7.25)
         assert np.array_equal(out[64:64 + M * N].reshape(M, N), A @ B)
+
+
+@pytest.mark.parametrize("M,K,N", [(135, 2559, 349), (100, 8192, 100), (256, 4096, 256), (65, 1500, 300), (70, 32768, 128),
+                                   (32, 4109, 36), (51, 7755, 52), (12, 215, 60), (49, 5536, 2), (129, 1024, 1024)])
+def test_native_small_outputs_with_a_long_k(gpu, M, K, N):
+    """Up to 256 rows against a narrow operand with a long k: chunks of 64 rows through the kernel that streams the
+    big operand, all operand forms and either side as the thin one; integers exact, random operands within tolerance."""
+    print("dgemm_ex, small outputs, long k", M, K, N, flush=True)
+    rng = np.random.default_rng(M + K + N)
+    for (m, n) in ((M, N), (N, M)):
+        A = rng.integers(-9, 10, (m, K)).astype(np.float64)
+        B = rng.integers(-9, 10, (K, n)).astype(np.float64)
+        ref = A @ B
+        At, Bt = np.ascontiguousarray(A.T), np.ascontiguousarray(B.T)
+        assert np.array_equal(dgemm_ex(A, B, m, K, n, 0, 0), ref)
+        assert np.array_equal(dgemm_ex(A, Bt, m, K, n, 0, 1), ref)
+        assert np.array_equal(dgemm_ex(At, B, m, K, n, 1, 0), ref)
+        A, B = synth.uniform(100 + m, (m, K)), synth.uniform(200 + n, (K, n))
+        assert normwise(dgemm_ex(A, B, m, K, n, 0, 0), A @ B, A, B) <= TOL
 
 
 def test_native_batch_of_rows_against_a_matrix_with_infinities_and_an_odd_base(gpu):

@@ -14,6 +14,17 @@ from gpu_util import normwise, run_dgemm
 pytestmark = pytest.mark.gpu
 TOL = 1e-14
 
+
+@pytest.fixture
+def tiled(gpu):
+    """For the tests of the tiled kernels' own variants (tile sizes, cuts along k): shapes with a
+    thin side or a small output would otherwise take the kernels of dgemm_thin_f64.hip."""
+    import eshkol_amd as ea
+    lib = ea.load()
+    lib.hip_dgemm_set_thin_rows(0)
+    yield
+    lib.hip_dgemm_set_thin_rows(1)
+
 SHAPES = [(1, 1, 1), (2, 2, 2), (1, 100, 1), (3, 5, 4), (5, 7, 3), (16, 16, 16), (64, 64, 64),
           (65, 67, 66), (37, 130, 9), (128, 128, 128), (129, 257, 131), (256, 256, 256),
           (300, 17, 500), (512, 1000, 64), (1000, 33, 1000), (1024, 1024, 1024),
@@ -90,7 +101,7 @@ def test_full_size_properties(gpu, M, K, N):
 @pytest.mark.parametrize("M,K,N", [(2048, 16, 2048), (2048, 48, 2048), (2048, 1024, 2048), (4096, 2064, 1024),
                                    (1024, 512, 4096), (2050, 130, 2046), (2049, 1000, 2050), (3000, 72, 1500),
                                    (1922, 4098, 2174), (2048, 18, 2048), (2176, 30, 1930)])
-def test_straight_line_kernel_matches_bounds_checked_kernel_bitwise(gpu, M, K, N):
+def test_straight_line_kernel_matches_bounds_checked_kernel_bitwise(gpu, tiled, M, K, N):
     """Large launches take a kernel without bounds checks (edge rows clamped,
     k-tail zeroed): same tiles, same summation order, so the same bits as the
     bounds-checked kernel, for all three operand forms. The output buffer is
@@ -140,7 +151,7 @@ def test_straight_line_kernel_in_a_batch(gpu):
 
 @pytest.mark.parametrize("M,K,N", [(3072, 256, 3072), (3072, 1000, 3072), (3000, 520, 3100), (3200, 160, 3072),
                                    (2944, 4100, 3060)])
-def test_k_split_last_round(gpu, M, K, N):
+def test_k_split_last_round(gpu, tiled, M, K, N):
     """More than one round of tiles with a nearly empty last round: those tiles are cut
     along k and the pieces added in a fixed order. Same result on every run, the tiles
     of the full rounds bit-identical to an unsplit launch, everything within the tier's
@@ -183,7 +194,7 @@ def test_k_split_last_round(gpu, M, K, N):
 
 @pytest.mark.parametrize("M,K,N", [(512, 2048, 512), (128, 8192, 128), (400, 1000, 400), (300, 1002, 1100),
                                    (1536, 1024, 1536), (130, 4098, 258), (1152, 1152, 1152)])
-def test_k_split_of_a_launch_that_does_not_fill_the_device(gpu, M, K, N):
+def test_k_split_of_a_launch_that_does_not_fill_the_device(gpu, tiled, M, K, N):
     """Fewer 128 x 128 tiles than CUs: every tile is cut along k and the pieces are added in
     a fixed order. Same bits on every run, within the tier's bound (against the whole launch
     too), nothing stored outside C; for all three operand forms."""
@@ -219,7 +230,7 @@ def test_k_split_of_a_launch_that_does_not_fill_the_device(gpu, M, K, N):
 
 @pytest.mark.parametrize("M,K,N", [(1024, 1024, 1024), (1000, 700, 1300), (130, 4098, 258), (64, 16, 64), (2, 16, 2),
                                    (900, 1001 * 2, 1100), (2048, 512, 2048)])
-def test_small_tile_kernel_gives_the_bits_of_the_large_one(gpu, M, K, N):
+def test_small_tile_kernel_gives_the_bits_of_the_large_one(gpu, tiled, M, K, N):
     """The straight-line kernel with 64 x 64 tiles (launches that would otherwise be cut along k)
     sums every output element in the same order as the 128 x 128 one: with whole tiles the two
     must agree bit for bit, for all three operand forms, edge tiles and k-tails included, and
@@ -252,7 +263,7 @@ def test_small_tile_kernel_gives_the_bits_of_the_large_one(gpu, M, K, N):
 
 
 @pytest.mark.parametrize("M,K,N", [(1536, 1024, 1536), (1280, 1288, 1280), (1300, 2000, 1250), (1792, 1024, 1800)])
-def test_k_split_of_the_small_tiles_left_over(gpu, M, K, N):
+def test_k_split_of_the_small_tiles_left_over(gpu, tiled, M, K, N):
     """64 x 64 tiles beyond the last multiple of the CU count are cut along k, in the same
     launch behind the whole ones, and their pieces added in a fixed order. Same result on
     every run, the whole tiles bit-identical to an uncut launch, everything within the
@@ -294,7 +305,7 @@ def test_k_split_of_the_small_tiles_left_over(gpu, M, K, N):
 
 @pytest.mark.parametrize("M,K,N", [(1024, 1024, 1024), (2304, 512, 2304), (3072, 640, 3072), (520, 4096, 500), (2048, 2048, 2048),
                                    (4096, 256, 4100), (300, 1002, 1100)])
-def test_the_tile_size_chosen_by_itself_changes_no_bits_of_whole_tiles(gpu, M, K, N):
+def test_the_tile_size_chosen_by_itself_changes_no_bits_of_whole_tiles(gpu, tiled, M, K, N):
     """The library picks the tile size of the straight-line kernel from the launch's shape.
     With every tile whole (no cuts along k) all choices sum in the same order: the default
     must give the bits of both forced sizes, and with cuts allowed stay within the tier's bound."""
