@@ -161,6 +161,10 @@ SIGNATURES = {
     "hip_dgemm_set_tail_split": (None, [C.c_int]),
     "hip_dgemm_set_small_tile": (None, [C.c_int]),
     "hip_dgemm_set_prefetch_depth": (None, [C.c_int]),
+    "hip_dgemm_set_thin_rows": (None, [C.c_int]),
+    "hip_dgemm_set_thin_rows_klast": (None, [C.c_int]),
+    "hip_dgemm_set_thin_chunks": (None, [C.c_int]),
+    "hip_igemm_set_thin_variant": (None, [C.c_int]),
     "hip_ozaki_crt_set_host_pass": (None, [C.c_int]),
     "hip_igemm_set_prefetch": (None, [C.c_int]),
 }

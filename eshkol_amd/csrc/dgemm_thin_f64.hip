@@ -286,15 +286,13 @@ void launch_rows(bool klast, const double* T, long t_r, long t_k, int R, const d
 
 int g_thin_rows = 1;        /* fewest rows sent here; 0: none (tuning) */
 int g_thin_rows_klast = 1;
-int g_thin_min_kc = 0;       /* fewest k per slice, 0: by the shape (tuning) */
-int g_thin_min_wide = 16;    /* narrowest big operand (tuning) */
+constexpr int THIN_MIN_WIDE = 16;      /* narrowest big operand */
 int g_thin_chunks = 1;       /* 0: no more than 64 thin rows (tuning) */
-int g_thin_min_log2 = 13;    /* smallest big operand, log2 of its elements (tuning) */
+constexpr int THIN_MIN_LOG2 = 13;      /* smallest big operand, log2 of its elements */
 
 }  // namespace
 
 extern "C" void hip_dgemm_set_thin_rows(int from) { EshkolHipLock lk; g_thin_rows = from > 0 ? from : 0; }
-extern "C" void hip_dgemm_set_thin_tuning(int min_kc, int min_wide, int min_log2) { EshkolHipLock lk; g_thin_min_kc = min_kc; g_thin_min_wide = min_wide; g_thin_min_log2 = min_log2; }
 extern "C" void hip_dgemm_set_thin_chunks(int on) { EshkolHipLock lk; g_thin_chunks = on ? 1 : 0; }
 extern "C" void hip_dgemm_set_thin_rows_klast(int on) { EshkolHipLock lk; g_thin_rows_klast = on ? 1 : 0; }
 
@@ -309,7 +307,7 @@ bool eshkol_hip_dgemm_is_thin_rows(uint64_t M, uint64_t K, uint64_t N, int trans
     const uint64_t thin = thin_m ? M : N, wide = thin_m ? N : M;
     const bool kfirst = thin_m ? !trans_b : (trans_a != 0);
     if (!kfirst && (!g_thin_rows_klast || thin < 2)) return false;
-    if (thin < (uint64_t)g_thin_rows || wide < (uint64_t)g_thin_min_wide || K < 64) return false;
+    if (thin < (uint64_t)g_thin_rows || wide < (uint64_t)THIN_MIN_WIDE || K < 64) return false;
     if (thin > 48 && K < 512) return false;
     if (thin > 64) {
         /* chunks of 64 rows, each reading the big operand again: where the tiled kernels would
@@ -321,7 +319,7 @@ bool eshkol_hip_dgemm_is_thin_rows(uint64_t M, uint64_t K, uint64_t N, int trans
         if (blocks > 48 || (wide * K > (2ull << 20) && blocks > 8)) return false;
     }
     if (K > 0x7fffffffULL || wide > 0x7fffffffULL) return false;
-    return wide * K >= (1ull << g_thin_min_log2);
+    return wide * K >= (1ull << THIN_MIN_LOG2);
 }
 
 int eshkol_hip_dgemm_thin_rows(const double* A, const double* B, double* C, uint64_t M, uint64_t K, uint64_t N,
@@ -342,7 +340,7 @@ int eshkol_hip_dgemm_thin_rows(const double* A, const double* B, double* C, uint
     int slices = (3 * eshkol_hip_num_cus()) / (strips * chunks);
     /* a slice of at least 256 k, shorter where the strips are few or k is short (more slices
      * are all the parallelism such a launch has) */
-    const int min_kc = g_thin_min_kc ? g_thin_min_kc : strips <= 2 ? 64 : (strips <= 4 || k < 2048) ? 128 : 256;
+    const int min_kc = strips <= 2 ? 64 : (strips <= 4 || k < 2048) ? 128 : 256;
     if (slices > k / min_kc) slices = k / min_kc;
     if (slices > 128) slices = 128;                 /* the sum walks them one thread per output */
     if (slices < 1) slices = 1;

@@ -94,6 +94,20 @@ void hip_dgemm_set_small_tile(int mode);
  * registers; 1: one. Same bits; the switch exists to compare them. */
 void hip_dgemm_set_prefetch_depth(int depth);
 
+/* Fewest rows on the thin side that take the kernels which stream the big operand
+ * through the matrix cores without tiles (1, the default: every product with up to 64
+ * thin rows that qualifies; 0: none, such shapes then take the tiled kernels). The
+ * summation order differs between the two, the tolerance is the tier's. */
+void hip_dgemm_set_thin_rows(int from);
+/* The same for the two refinements of that path, for measurements: big operands with k
+ * contiguous (1 default), and more than 64 thin rows in chunks of 64 (1 default). */
+void hip_dgemm_set_thin_rows_klast(int on);
+void hip_dgemm_set_thin_chunks(int on);
+
+/* Column blocks per workgroup of the int8 kernel for a first operand of at most 64 rows:
+ * 0 (default) by the shape, 1 or 2 forced. Same results. */
+void hip_igemm_set_thin_variant(int column_blocks);
+
 /* k-blocks kept in flight by the pipelined int8 kernel (1..3; 0 = simple kernel only). */
 void hip_igemm_set_prefetch(int pf);
 
@@ -102,7 +116,9 @@ void hip_igemm_set_prefetch(int pf);
  * (256 x 128 tiles and two workgroups per CU for products of at most 1024 bytes
  * of k, 256 x 256 tiles and one otherwise); 2: the 256 x 128 kernel for all of
  * them; 3: the 256 x 256 kernel for all of them; 0: row-major planes and the
- * register-staged kernels everywhere. Same results; the switch exists to
+ * register-staged kernels everywhere. With 1, a first operand of at most 64 rows
+ * takes the kernel that streams the second operand's planes (any other value
+ * keeps such products on the kernels named). Same results; the switch exists to
  * compare them. */
 void hip_igemm_set_direct(int on);
 
