@@ -407,16 +407,19 @@ void resident_release_all(void) {
 /* The prepared form of the resident tensor at device address dB as the K x N second
  * operand of the exact tier, made on first use; NULL if dB is not resident, the
  * tier declines or the byte cap is reached (then the call prepares nothing and
- * splits B as always, which a verbose run says once per tensor). Planes made for
- * the other plane layout (a product whose row count puts it on the other side of
- * hip_igemm_plane_layout) are made again for this one: keeping them would mean
- * splitting B on every such call while they sit in device memory unused. A
+ * splits B as always, which a verbose run says once per tensor). Row-major planes
+ * are made again, interleaved, for the first product that wants interleaved ones (a
+ * row count on the other side of hip_igemm_plane_layout): keeping them would mean
+ * splitting B on every such call while they sit in device memory unused.
+ * Interleaved planes then stay, whatever the row counts that follow. A
  * failed allocation is not remembered; a refusal that depends on the contents
  * is, until pin or refresh bring new contents. */
 void* resident_prepared_b(const double* dB, uint64_t M, uint64_t K, uint64_t N, int moduli) {
     Resident* r = resident_find_device(dB);
     if (!r || r->bytes != K * N * sizeof(double)) return nullptr;
-    const int layout = hip_igemm_plane_layout(M, N, moduli);
+    /* interleaved planes serve every row count; row-major ones only products that want them */
+    const bool keep = r->prepared && r->prep_layout == 1 && r->prep_K == K && r->prep_N == N && r->prep_moduli == moduli;
+    const int layout = keep ? 1 : hip_igemm_plane_layout(M, N, moduli);
     if (r->prepared && (r->prep_K != K || r->prep_N != N || r->prep_moduli != moduli || r->prep_layout != layout)) {
         if (r->prep_K == K && r->prep_N == N && r->prep_moduli == moduli)
             GPU_LOG("resident operand %p: residue planes are in the %s layout, this product wants the other: "

@@ -890,6 +890,7 @@ extern "C" int hip_ozaki_crt_last_stages(HipOzakiCrtStages* out) {
  * multiplies fresh activations by the same weights need only split the
  * activations. The planes are the bytes the tier would compute itself, so the
  * result is the same bit for bit. */
+int eshkol_hip_igemm_direct_mode(void);     /* igemm_i8.hip: 1 unless a test forces a kernel */
 namespace {
 struct CrtPreparedB {
     uint32_t magic;
@@ -933,7 +934,12 @@ static int crt_matmul_impl(const double* A, const double* B, double* C,
 
     /* planes interleaved (and the k pitch padded to whole groups of four 128-byte
      * blocks) when the contraction will take the kernel that wants them so */
-    const int layout = hip_igemm_plane_layout(M, N, num_moduli);
+    /* Interleaved planes serve every row count (the kernels that take them run with any
+     * number of tiles), so a second operand prepared in that layout keeps it; row-major
+     * planes serve only the products that would make row-major planes themselves. */
+    const bool keep_interleaved = prepared && prepared->layout == 1 && !adaptive && !g_force_host_pass &&
+                                  prepared->n_mod == num_moduli && eshkol_hip_igemm_direct_mode() == 1;
+    const int layout = keep_interleaved ? 1 : hip_igemm_plane_layout(M, N, num_moduli);
     /* a first operand of a few rows goes to the kernel that streams the second operand's
      * planes: its own planes then need whole blocks of 32 rows only */
     const bool thin = layout == 1 && eshkol_hip_igemm_is_thin(M);

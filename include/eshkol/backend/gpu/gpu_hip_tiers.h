@@ -213,8 +213,10 @@ int hip_matmul_ozaki_crt_f64(const double* A, const double* B, double* C,
  * does not depend on the operands (sixteen moduli at every K the tier accepts;
  * -1 otherwise, and for a B with non-finite entries or a column maximum within
  * 2^-40 of a power of two; -2 when device memory for the planes cannot be had). M_expected is the row count of the products to
- * come: it selects the plane layout (hip_igemm_plane_layout); a call whose
- * shape wants the other layout, or adaptive != 0, simply splits B again. B
+ * come: it selects the plane layout (hip_igemm_plane_layout). Interleaved planes
+ * (layout 1) then serve products of every row count; row-major planes serve the
+ * products that would make row-major planes themselves, and a call whose shape
+ * wants interleaved ones, or adaptive != 0, simply splits B again. B
  * must stay valid and unchanged while the handle lives; eshkol_gpu_resident_pin
  * tensors get this treatment by themselves when the dispatcher routes a product
  * to this tier. */

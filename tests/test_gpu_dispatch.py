@@ -578,24 +578,24 @@ assert np.array_equal(ea.matmul_dispatch(X, W), oracle.matmul_ozaki_crt(X, W))
 
 
 def test_resident_planes_follow_the_plane_layout_and_the_byte_cap(gpu):
-    """Planes prepared for one plane layout are made again when a product wants the other
-    (512 rows: 64 tiles, row-major planes; 1024 rows: 128 tiles, interleaved), with a line in
-    the verbose log, instead of staying in memory unused while B is split on every call; and
-    ESHKOL_GPU_PREPARED_BYTES bounds what they may take (0: none). Results are the unpinned
-    path's either way."""
+    """Row-major planes (512 rows: 64 tiles) are made again, interleaved, when a product wants
+    interleaved ones (1024 rows: 128 tiles), with a line in the verbose log, instead of staying
+    in memory unused while B is split on every call; interleaved planes then serve every row
+    count that follows (512 again, 700). ESHKOL_GPU_PREPARED_BYTES
+    bounds what they may take (0: none). Results are the unpinned path's either way."""
     body = r"""
 K, N = 1024, 512
 W = synth.xavier_uniform(5, K, N)
 assert lib.eshkol_gpu_resident_pin(W.ctypes.data, W.nbytes) == 0
-for M in (512, 1024, 1024, 512):
+for M in (512, 1024, 1024, 512, 700):
     X = synth.normal(M, (M, K))
     assert np.array_equal(ea.matmul_dispatch(X, W), oracle.matmul_ozaki_crt(X, W)), M
 lib.eshkol_gpu_resident_unpin(W.ctypes.data)
 """
     env = {"ESHKOL_HIP_F64_KERNEL": "ozaki-crt", "ESHKOL_GPU_THRESHOLD": "1", "ESHKOL_GPU_VERBOSE": "1"}
     r = run_child(body, env)
-    assert r.stderr.count("residue planes of the exact tier prepared") == 3
-    assert r.stderr.count("this product wants the other: preparing them again") == 2
+    assert r.stderr.count("residue planes of the exact tier prepared") == 2
+    assert r.stderr.count("this product wants the other: preparing them again") == 1
     r = run_child(body, dict(env, ESHKOL_GPU_PREPARED_BYTES="0"))
     assert "residue planes of the exact tier prepared" not in r.stderr
     assert r.stderr.count("would exceed ESHKOL_GPU_PREPARED_BYTES=0") == 1       # said once, then remembered
