@@ -923,8 +923,8 @@ int dgemm_any(const double* A, const double* B, double* C, uint64_t M, uint64_t 
     if (g_fast_path && batch == 1 && eshkol_hip_dgemm_is_small_long_k(M, K, N) &&
         eshkol_hip_dgemm_small_long_k(A, B, C, M, K, N, trans_a, trans_b, st) == 0) return 0;
     /* a vector against a matrix with k contiguous: plain fma loops at the rate of HBM (dgemv_f64.hip) */
-    if (g_fast_path && batch == 1 && eshkol_hip_dgemm_is_skinny(M, K, N, trans_a, trans_b) &&
-        eshkol_hip_dgemm_skinny(A, B, C, M, K, N, trans_a, trans_b, st) == 0) return 0;
+    if (g_fast_path && batch == 1 && eshkol_hip_dgemm_is_matvec(M, K, N, trans_a, trans_b) &&
+        eshkol_hip_dgemm_matvec(A, B, C, M, K, N, trans_a, trans_b, st) == 0) return 0;
     /* Operands whose rows do not start on 16-byte boundaries (an odd pitch, a base that
      * is not aligned) would take the kernel of 8-byte loads, at two thirds of the rate
      * (4096 x 4096 x 4097: 3.0 ms against 2.1). Where the shape would otherwise run the

@@ -76,9 +76,9 @@ void dgemv_klast_kernel(const double* __restrict__ big, long ldb, int O, int K,
 
 }  // namespace
 
-/* Whether eshkol_hip_dgemm_skinny takes the product: one vector against a matrix held with
+/* Whether eshkol_hip_dgemm_matvec takes the product: one vector against a matrix held with
  * k contiguous, long enough in both directions for the launch to matter. */
-bool eshkol_hip_dgemm_is_skinny(uint64_t M, uint64_t K, uint64_t N, int trans_a, int trans_b) {
+bool eshkol_hip_dgemm_is_matvec(uint64_t M, uint64_t K, uint64_t N, int trans_a, int trans_b) {
     const uint64_t thin = M < N ? M : N, wide = M < N ? N : M;
     if (thin != 1 || wide < 128 || K < 64 || K > 0x7fffffffULL || wide > 0x7fffffffULL) return false;
     const bool thin_m = M <= N;
@@ -86,8 +86,8 @@ bool eshkol_hip_dgemm_is_skinny(uint64_t M, uint64_t K, uint64_t N, int trans_a,
     return klast && wide * K >= (1ull << 17);
 }
 
-/* C = op(A) op(B) for a product eshkol_hip_dgemm_is_skinny() accepts. */
-int eshkol_hip_dgemm_skinny(const double* A, const double* B, double* C, uint64_t M, uint64_t K, uint64_t N,
+/* C = op(A) op(B) for a product eshkol_hip_dgemm_is_matvec() accepts. */
+int eshkol_hip_dgemm_matvec(const double* A, const double* B, double* C, uint64_t M, uint64_t K, uint64_t N,
                             int trans_a, int trans_b, hipStream_t st) {
     (void)trans_a; (void)trans_b;
     const bool thin_m = M <= N;

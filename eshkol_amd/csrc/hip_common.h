@@ -131,8 +131,8 @@ int eshkol_hip_dgemm_small_long_k(const double* A, const double* B, double* C, u
 
 /* One vector against a matrix held with k contiguous (dgemv_f64.hip): whether the shape is
  * one, and the product itself. hip_dgemm_f64 and hip_dgemm_f64_ex send such shapes there. */
-bool eshkol_hip_dgemm_is_skinny(uint64_t M, uint64_t K, uint64_t N, int trans_a, int trans_b);
-int eshkol_hip_dgemm_skinny(const double* A, const double* B, double* C, uint64_t M, uint64_t K, uint64_t N,
+bool eshkol_hip_dgemm_is_matvec(uint64_t M, uint64_t K, uint64_t N, int trans_a, int trans_b);
+int eshkol_hip_dgemm_matvec(const double* A, const double* B, double* C, uint64_t M, uint64_t K, uint64_t N,
                             int trans_a, int trans_b, hipStream_t st);
 
 /* fp64 products with up to 64 rows on the thin side: the big operand streamed through the
