@@ -277,7 +277,9 @@ def test_native_thin_products_write_nothing_else(gpu):
 
 
 @pytest.mark.parametrize("M,K,N", [(135, 2559, 349), (100, 8192, 100), (256, 4096, 256), (65, 1500, 300), (70, 32768, 128),
-                                   (32, 4109, 36), (51, 7755, 52), (12, 215, 60), (49, 5536, 2), (129, 1024, 1024)])
+                                   (32, 4109, 36), (51, 7755, 52), (12, 215, 60), (49, 5536, 2), (129, 1024, 1024),
+                                   (64, 512, 16), (16, 64, 2048), (2, 65, 128), (256, 1024, 64), (65, 1024, 17), (48, 511, 4000),
+                                   (49, 511, 4000), (64, 16384, 33)])
 def test_native_small_outputs_with_a_long_k(gpu, M, K, N):
     """Up to 256 rows against a narrow operand with a long k: chunks of 64 rows through the kernel that streams the
     big operand, all operand forms and either side as the thin one; integers exact, random operands within tolerance."""

@@ -128,7 +128,8 @@ def test_output_planes_larger_than_the_product(gpu, M, K, N, out_rows, ldn, mode
     assert np.all((rest == 0) | (rest == fill))
 
 
-THIN_SHAPES = [(1, 512, 32), (5, 700, 100), (32, 4096, 1024), (33, 1000, 1300), (64, 2049, 257), (17, 130, 4096)]
+THIN_SHAPES = [(1, 512, 32), (5, 700, 100), (32, 4096, 1024), (33, 1000, 1300), (64, 2049, 257), (17, 130, 4096),
+               (64, 512, 4100), (32, 1, 1), (2, 513, 33)]
 
 
 @pytest.mark.parametrize("M,K,N", THIN_SHAPES)
