@@ -114,7 +114,8 @@ void hip_igemm_set_prefetch(int pf);
 /* 1 (default): contractions with at least 128 tiles take interleaved operand
  * planes and the kernels that load them straight into LDS and MFMA registers
  * (256 x 128 tiles and two workgroups per CU for products of at most 1024 bytes
- * of k, 256 x 256 tiles and one otherwise); 2: the 256 x 128 kernel for all of
+ * of k and for launches with fewer 256 x 256 tiles than CUs, 256 x 256 tiles and
+ * one otherwise); 2: the 256 x 128 kernel for all of
  * them; 3: the 256 x 256 kernel for all of them; 0: row-major planes and the
  * register-staged kernels everywhere. With 1, a first operand of at most 64 rows
  * takes the kernel that streams the second operand's planes (any other value
