@@ -166,6 +166,7 @@ SIGNATURES = {
     "hip_dgemm_set_thin_chunks": (None, [C.c_int]),
     "hip_igemm_set_thin_variant": (None, [C.c_int]),
     "hip_ozaki_crt_set_host_pass": (None, [C.c_int]),
+    "hip_ozaki_crt_set_fused_scan": (None, [C.c_int]),
     "hip_igemm_set_prefetch": (None, [C.c_int]),
 }
 

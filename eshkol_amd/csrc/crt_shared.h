@@ -54,6 +54,25 @@ constexpr ByteWeights byte_weights(int modulus) {
     return { c[0] | c[1] << 8 | c[2] << 16 | c[3] << 24, c[4] | c[5] << 8 | c[6] << 16 | c[7] << 24 };
 }
 
+/* One step of a maximum of magnitudes. A NaN or an infinity anywhere makes the result
+ * +inf, which the tiers read as "not representable, use the native GEMM". */
+__device__ __forceinline__ void eshkol_absmax_step(double v, double* m) {
+    const double a = fabs(v);
+    if (!(a <= 1.7976931348623157e308)) *m = __builtin_inf();
+    else if (a > *m) *m = a;
+}
+
+/* E - floor(log2 m) for a maximum m > 0 (exponent field; subnormals by their
+ * leading bit), 0 for m = 0: the per-row shift of the CRT tiers when E does not
+ * depend on the operands (gpu_memory.mm:2524-2532). */
+__device__ __forceinline__ int32_t eshkol_shift_of_maximum(double m, int E) {
+    if (!(m > 0.0)) return 0;
+    const unsigned long long bits = (unsigned long long)__double_as_longlong(m);
+    const int ef = (int)(bits >> 52);
+    const int e = ef ? ef - 1023 : (63 - __clzll((long long)(bits & 0xfffffffffffffull))) - 1074;
+    return E - e;
+}
+
 /* ---- maxima with the shifts beside them (implemented in elementwise.hip) ------------
  * hip_rowabsmax_f64 / hip_colabsmax_f64 that also write, when shift is not null,
  * shift[i] = E - floor(log2 max_i) (0 for a maximum of zero): what the split of a

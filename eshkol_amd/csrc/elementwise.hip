@@ -34,23 +34,6 @@ void transpose_f64_kernel(const double* __restrict__ in, double* __restrict__ ou
 /* One wave per row: lanes stride the row 16 bytes at a time, then a butterfly
  * max across the wave. A NaN or infinity anywhere in the row makes the result
  * +inf, which the tiers read as "not representable, use the native GEMM". */
-__device__ __forceinline__ void absmax_step(double v, double* m) {
-    const double a = fabs(v);
-    if (!(a <= 1.7976931348623157e308)) *m = __builtin_inf();
-    else if (a > *m) *m = a;
-}
-
-/* E - floor(log2 m) for a maximum m > 0 (exponent field; subnormals by their
- * leading bit), 0 for m = 0: the per-row shift of the CRT tiers when E does not
- * depend on the operands (gpu_memory.mm:2524-2532). */
-__device__ __forceinline__ int32_t shift_of_maximum(double m, int E) {
-    if (!(m > 0.0)) return 0;
-    const unsigned long long bits = (unsigned long long)__double_as_longlong(m);
-    const int ef = (int)(bits >> 52);
-    const int e = ef ? ef - 1023 : (63 - __clzll((long long)(bits & 0xfffffffffffffull))) - 1074;
-    return E - e;
-}
-
 __global__ __launch_bounds__(256)
 void rowabsmax_f64_kernel(const double* __restrict__ A, uint64_t M, uint64_t K,
                           double zero_value, double* __restrict__ rmax, int32_t* __restrict__ shift, int E) {
@@ -66,11 +49,11 @@ void rowabsmax_f64_kernel(const double* __restrict__ A, uint64_t M, uint64_t K,
         const uint64_t n2 = K >> 1;
         for (uint64_t k = lane; k < n2; k += 64) {
             d2_t v = p2[k];
-            absmax_step(v.x, &m);
-            absmax_step(v.y, &m);
+            eshkol_absmax_step(v.x, &m);
+            eshkol_absmax_step(v.y, &m);
         }
     } else {
-        for (uint64_t k = lane; k < K; k += 64) absmax_step(p[k], &m);
+        for (uint64_t k = lane; k < K; k += 64) eshkol_absmax_step(p[k], &m);
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
@@ -79,7 +62,7 @@ void rowabsmax_f64_kernel(const double* __restrict__ A, uint64_t M, uint64_t K,
     }
     if (lane == 0) {
         rmax[row] = (m > 0.0) ? m : zero_value;
-        if (shift) shift[row] = shift_of_maximum(m, E);
+        if (shift) shift[row] = eshkol_shift_of_maximum(m, E);
     }
 }
 
@@ -104,7 +87,7 @@ void rowabsmax_few_rows_f64_kernel(const double* __restrict__ A, uint64_t K,
 #pragma unroll
             for (int u = 0; u < 4; u++) v[u] = (k + 256 * u < n2) ? p2[k + 256 * u] : (d2_t){0.0, 0.0};
 #pragma unroll
-            for (int u = 0; u < 4; u++) { absmax_step(v[u].x, &m); absmax_step(v[u].y, &m); }
+            for (int u = 0; u < 4; u++) { eshkol_absmax_step(v[u].x, &m); eshkol_absmax_step(v[u].y, &m); }
         }
     } else {
         for (uint64_t k = tid; k < K; k += 1024) {
@@ -112,7 +95,7 @@ void rowabsmax_few_rows_f64_kernel(const double* __restrict__ A, uint64_t K,
 #pragma unroll
             for (int u = 0; u < 4; u++) v[u] = (k + 256 * u < K) ? p[k + 256 * u] : 0.0;
 #pragma unroll
-            for (int u = 0; u < 4; u++) absmax_step(v[u], &m);
+            for (int u = 0; u < 4; u++) eshkol_absmax_step(v[u], &m);
         }
     }
 #pragma unroll
@@ -125,7 +108,7 @@ void rowabsmax_few_rows_f64_kernel(const double* __restrict__ A, uint64_t K,
     if (tid == 0) {
         for (int w = 1; w < 4; w++) if (red[w] > m) m = red[w];
         rmax[row] = (m > 0.0) ? m : zero_value;
-        if (shift) shift[row] = shift_of_maximum(m, E);
+        if (shift) shift[row] = eshkol_shift_of_maximum(m, E);
     }
 }
 
@@ -150,9 +133,9 @@ void colabsmax_partial_kernel(const double* __restrict__ X, uint64_t K, uint64_t
 #pragma unroll
             for (int u = 0; u < 8; u++) v[u] = X[(k + 4 * u) * R + col];
 #pragma unroll
-            for (int u = 0; u < 8; u++) absmax_step(v[u], &m);
+            for (int u = 0; u < 8; u++) eshkol_absmax_step(v[u], &m);
         }
-        for (; k < k1; k += 4) absmax_step(X[k * R + col], &m);
+        for (; k < k1; k += 4) eshkol_absmax_step(X[k * R + col], &m);
     }
     red[part][c] = m;
     __syncthreads();
@@ -178,7 +161,7 @@ void colabsmax_fold_kernel(const double* __restrict__ partial, uint64_t R, int s
     }
     for (; s < slices; s++) { const double o = partial[(uint64_t)s * R + col]; if (o > m) m = o; }
     out[col] = (m > 0.0) ? m : zero_value;
-    if (shift) shift[col] = shift_of_maximum(m, E);
+    if (shift) shift[col] = eshkol_shift_of_maximum(m, E);
 }
 
 __device__ __forceinline__ double apply_op(int op, double a, double b, bool has_b) {

@@ -424,16 +424,13 @@ __device__ __forceinline__ void decode_positive(double m, int* e, unsigned long 
     else { const int p = 63 - __clzll((long long)mant); *e = p - 1074; *n = mant << (52 - p); }
 }
 
-/* block 0: the M row maxima of A; block 1: the N maxima of B */
-__global__ __launch_bounds__(SCAN_THREADS)
-void crt_scan_kernel(const double* __restrict__ amax, uint64_t M, const double* __restrict__ bmax, uint64_t N,
-                     int32_t* __restrict__ fl_a, int32_t* __restrict__ fl_b, CrtScan* out, uint32_t ticket) {
+/* One workgroup of THREADS threads scans the n_rows maxima x[] (global or LDS memory) and
+ * leaves their summary in *o, the ticket last. */
+template <int THREADS>
+__device__ __forceinline__ void scan_block(const double* x, uint64_t n_rows, int32_t* fl, CrtScan* o, uint32_t ticket) {
+    constexpr int SCAN_THREADS = THREADS;
     __shared__ unsigned long long s_max, keys[256];
     __shared__ int s_nonfinite, s_extreme, s_nonzero, s_emin, s_emax, s_ncand;
-    const double* x = blockIdx.x ? bmax : amax;
-    const uint64_t n_rows = blockIdx.x ? N : M;
-    int32_t* fl = blockIdx.x ? fl_b : fl_a;
-    CrtScan* o = out + blockIdx.x;
     const int tid = threadIdx.x;
     if (tid == 0) { s_max = 0; s_nonfinite = 0; s_extreme = 0; s_nonzero = 0; s_emin = INT32_MAX; s_emax = INT32_MIN; s_ncand = 0; }
     if (tid < 256) keys[tid] = 0;
@@ -531,6 +528,74 @@ void crt_scan_kernel(const double* __restrict__ amax, uint64_t M, const double* 
         __threadfence_system();
         *(volatile uint32_t*)&o->ready = ticket;
     }
+}
+
+/* block 0: the M row maxima of A; block 1: the N maxima of B */
+__global__ __launch_bounds__(SCAN_THREADS)
+void crt_scan_kernel(const double* __restrict__ amax, uint64_t M, const double* __restrict__ bmax, uint64_t N,
+                     int32_t* __restrict__ fl_a, int32_t* __restrict__ fl_b, CrtScan* out, uint32_t ticket) {
+    scan_block<SCAN_THREADS>(blockIdx.x ? bmax : amax, blockIdx.x ? N : M, blockIdx.x ? fl_b : fl_a,
+                             out + blockIdx.x, ticket);
+}
+
+/* A few long rows in front of prepared planes: their maxima, their shifts and the scan of
+ * the maxima in one launch (three launch-sized kernels otherwise, 8 us of the 50 a layer
+ * takes). A workgroup per row, every thread with four loads in flight; the workgroup
+ * that finishes last (a counter in device memory, left at zero again) scans the M <= 256
+ * maxima, which it reads with atomic loads into LDS: no cache of its CU has seen them. */
+constexpr int FUSED_MAX_ROWS = 256;
+__global__ __launch_bounds__(256)
+void crt_rowmax_scan_kernel(const double* __restrict__ A, uint64_t M, uint64_t K, double* rmax, int32_t* __restrict__ shift,
+                            int E, unsigned* counter, CrtScan* out, uint32_t ticket) {
+    __shared__ double red[4];
+    __shared__ double maxima[FUSED_MAX_ROWS];
+    __shared__ int s_last;
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint64_t row = blockIdx.x;
+    const double* p = A + row * K;
+    double m = 0.0;
+    if (((K & 1) == 0) && (((uintptr_t)A & 15) == 0)) {
+        typedef double d2_t __attribute__((ext_vector_type(2)));
+        const d2_t* p2 = (const d2_t*)p;
+        const uint64_t n2 = K >> 1;
+        for (uint64_t k = tid; k < n2; k += 1024) {
+            d2_t v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) v[u] = (k + 256 * u < n2) ? p2[k + 256 * u] : (d2_t){0.0, 0.0};
+#pragma unroll
+            for (int u = 0; u < 4; u++) { eshkol_absmax_step(v[u].x, &m); eshkol_absmax_step(v[u].y, &m); }
+        }
+    } else {
+        for (uint64_t k = tid; k < K; k += 1024) {
+            double v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) v[u] = (k + 256 * u < K) ? p[k + 256 * u] : 0.0;
+#pragma unroll
+            for (int u = 0; u < 4; u++) eshkol_absmax_step(v[u], &m);
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const double o = __shfl_xor(m, off, 64);
+        if (o > m) m = o;
+    }
+    if (lane == 0) red[wave] = m;
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 1; w < 4; w++) if (red[w] > m) m = red[w];
+        __hip_atomic_store(&rmax[row], m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        shift[row] = eshkol_shift_of_maximum(m, E);
+        __threadfence();
+        s_last = atomicAdd(counter, 1u) == gridDim.x - 1 ? 1 : 0;
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();
+    if (tid == 0) *counter = 0;                       /* the next launch on the stream starts from zero */
+    for (uint64_t i = tid; i < M; i += 256)
+        maxima[i] = __hip_atomic_load(&rmax[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    scan_block<256>(maxima, M, nullptr, out, ticket);
 }
 
 /* shift = E - floor(log2 max), 0 for a maximum of zero (gpu_memory.mm:2524-2532), in place */
@@ -705,10 +770,11 @@ const CrtScan* scan_await(uint32_t ticket) {
 }
 
 /* device-resident constant tables for the contraction: identity pair lists and moduli */
-int32_t* g_tables = nullptr;   /* [0..16] pair_first, [17..32] pair index, [33..48] moduli */
+int32_t* g_tables = nullptr;   /* [0..16] pair_first, [17..32] pair index, [33..48] moduli, [49] the fused scan's counter */
 int ensure_tables(hipStream_t st) {
     if (g_tables) return 0;
-    int32_t h[17 + 16 + 16];
+    int32_t h[17 + 16 + 16 + 1];
+    h[49] = 0;
     for (int i = 0; i <= 16; i++) h[i] = i;
     for (int i = 0; i < 16; i++) { h[17 + i] = i; h[33 + i] = H_MODULI[i]; }
     if (!ESHKOL_HIP_OK(hipMalloc((void**)&g_tables, sizeof h))) { g_tables = nullptr; return -1; }
@@ -717,8 +783,21 @@ int ensure_tables(hipStream_t st) {
     return 0;
 }
 
+/* Row maxima, shifts (E fixed) and the scan of A's maxima alone in one launch on st, for a
+ * few long rows in front of prepared planes; the ticket, 0 on failure. */
+uint32_t rowmax_scan_launch(const double* A, uint64_t M, uint64_t K, double* amax, int32_t* mu, int E, hipStream_t st) {
+    if (!ensure_mailbox() || !g_tables || M == 0 || M > (uint64_t)FUSED_MAX_ROWS) return 0;
+    g_scan_ran_on = st;
+    g_scan_halves = 1;
+    const uint32_t ticket = ++g_ticket ? g_ticket : ++g_ticket;
+    hipLaunchKernelGGL(crt_rowmax_scan_kernel, dim3((unsigned)M), dim3(256), 0, st, A, M, K, amax, mu, E,
+                       (unsigned*)(g_tables + 49), g_mailbox_dev, ticket);
+    return ESHKOL_HIP_OK(hipGetLastError()) ? ticket : 0;
+}
+
 HipOzakiCrtStages g_last = {};
 bool g_force_host_pass = false;
+bool g_fused_scan = true;      /* tuning: false keeps the three kernels apart */
 
 template <int NMOD>
 void launch_split(const double* X, uint64_t rows, uint64_t K, const int32_t* shift, int8_t* planes,
@@ -868,6 +947,7 @@ void eshkol_hip_crt_release(void) {
 }
 
 extern "C" void hip_ozaki_crt_set_host_pass(int on) { EshkolHipLock lk; g_force_host_pass = on != 0; }
+extern "C" void hip_ozaki_crt_set_fused_scan(int on) { EshkolHipLock lk; g_fused_scan = on != 0; }
 
 extern "C" int hip_ozaki_crt_set_aligned_weights(int on) {
     EshkolHipLock lk;
@@ -979,17 +1059,24 @@ static int crt_matmul_impl(const double* A, const double* B, double* C,
                          floor((crt_constants(num_moduli).log2P - 3.0 - log2K) / 2.0) >= 52.0;
     int32_t* const mu_out = fixed_E ? dmu : nullptr;
     int32_t* const nu_out = fixed_E ? dnu : nullptr;
-    /* the last kernel that writes maxima carries the event the scan's stream waits for */
-    const hipEvent_t fork = fixed_E ? scan_event(M * K + K * N) : nullptr;
-    const hipEvent_t fork_a = use_prepared ? fork : nullptr, fork_b = use_prepared ? nullptr : fork;
-    if ((a_kmajor ? eshkol_colabsmax_shift_f64(A, K, M, 0.0, amax, mu_out, 52, st, fork_a)
-                  : eshkol_rowabsmax_shift_f64(A, M, K, 0.0, amax, mu_out, 52, st, fork_a)) != 0) return -1;
-    if (!use_prepared &&
-        (b_kmajor ? eshkol_colabsmax_shift_f64(B, K, N, 0.0, bmax, nu_out, 52, st, fork_b)
-                  : eshkol_rowabsmax_shift_f64(B, N, K, 0.0, bmax, nu_out, 52, st, fork_b)) != 0) return -1;
-    /* prepared planes: the scan looks at A's maxima only, B's summary was kept with the planes */
-    const uint32_t ticket = fixed_E ? scan_launch_aside(amax, M, bmax, N, st, M * K + K * N, fork != nullptr, use_prepared ? 1 : 2)
-                                    : scan_launch(amax, M, bmax, N, dmu, dnu, st);
+    /* a few long rows in front of prepared planes: maxima, shifts and scan in one launch */
+    const bool fused_scan = use_prepared && !a_kmajor && M <= (uint64_t)FUSED_MAX_ROWS && K >= 1024 && g_fused_scan;
+    uint32_t ticket = 0;
+    if (fused_scan) {
+        ticket = rowmax_scan_launch(A, M, K, amax, dmu, 52, st);
+    } else {
+        /* the last kernel that writes maxima carries the event the scan's stream waits for */
+        const hipEvent_t fork = fixed_E ? scan_event(M * K + K * N) : nullptr;
+        const hipEvent_t fork_a = use_prepared ? fork : nullptr, fork_b = use_prepared ? nullptr : fork;
+        if ((a_kmajor ? eshkol_colabsmax_shift_f64(A, K, M, 0.0, amax, mu_out, 52, st, fork_a)
+                      : eshkol_rowabsmax_shift_f64(A, M, K, 0.0, amax, mu_out, 52, st, fork_a)) != 0) return -1;
+        if (!use_prepared &&
+            (b_kmajor ? eshkol_colabsmax_shift_f64(B, K, N, 0.0, bmax, nu_out, 52, st, fork_b)
+                      : eshkol_rowabsmax_shift_f64(B, N, K, 0.0, bmax, nu_out, 52, st, fork_b)) != 0) return -1;
+        /* prepared planes: the scan looks at A's maxima only, B's summary was kept with the planes */
+        ticket = fixed_E ? scan_launch_aside(amax, M, bmax, N, st, M * K + K * N, fork != nullptr, use_prepared ? 1 : 2)
+                         : scan_launch(amax, M, bmax, N, dmu, dnu, st);
+    }
     if (!ticket) return -1;
     CrtScan merged[2];
     auto await_scan = [&]() -> const CrtScan* {

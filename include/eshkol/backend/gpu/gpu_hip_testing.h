@@ -137,6 +137,11 @@ void hip_hgemm_set_direct(int on);
  * workgroup per tile. Same results; the switch exists to compare them. */
 void hip_igemm_set_persistent(int on);
 
+/* 1 (default): a few long rows (at most 256, k from 1024 on) in front of a prepared second
+ * operand get their maxima, their shifts and the scan of the maxima from one launch; 0:
+ * from the three kernels every other shape uses. Same results. */
+void hip_ozaki_crt_set_fused_scan(int on);
+
 /* 0 (default): the CRT tier finds floor(log2) of the row and column maxima and
  * the few maxima that can carry the largest fractional part of log2 on the
  * device, and the host calls log2 on those few only; 1: the host takes log2 of

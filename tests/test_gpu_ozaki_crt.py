@@ -235,6 +235,57 @@ def test_shift_bookkeeping_mantissas_next_to_a_power_of_two(gpu):
         both_bookkeeping_paths(A, Bx)
 
 
+@pytest.mark.parametrize("M,K,N", [(1, 1024, 512), (8, 4096, 300), (64, 1031, 1000), (200, 2048, 256), (256, 1024, 64)])
+def test_few_rows_in_front_of_prepared_planes(gpu, M, K, N):
+    """A few long rows against a prepared second operand: row maxima, shifts and the scan of the maxima are one
+    launch there (the workgroup that finishes last scans). Results are the plain entry point's bit for bit and the
+    oracle's within the tier's bar, also with zero rows, tiny and huge rows, a maximum next to a power of two (the
+    scan hands such operands to the host pass), and a NaN or an infinity is refused; with the three kernels kept
+    apart the same again."""
+    import ctypes as C
+    import eshkol_amd as ea
+    lib = ea.load()
+    st = lib.eshkol_hip_get_stream()
+    B = synth.normal(50 + N, (K, N))
+    dB = ea.DeviceArray.from_host(B)
+    h = C.c_void_p()
+    assert lib.hip_ozaki_crt_prepare_operand_b(dB.ptr, K, N, 0, 16, M, C.byref(h), st) == 0
+
+    def run(A, prepared):
+        dA, dC = ea.DeviceArray.from_host(A), ea.DeviceArray((M, N))
+        if prepared:
+            rc = lib.hip_matmul_ozaki_crt_prepared_f64(dA.ptr, h, dC.ptr, M, K, N, 0, 16, 0, None, 0, st)
+        else:
+            rc = lib.hip_matmul_ozaki_crt_f64(dA.ptr, dB.ptr, dC.ptr, M, K, N, 16, 0, None, 0, st)
+        ea.synchronize()
+        return rc, dC.download()
+
+    base = synth.normal(60 + M, (M, K))
+    cases = [base]
+    A = base.copy(); A[0, :] = 0.0; cases.append(A)
+    A = base.copy(); A[M - 1, :] *= 2.0 ** -600; A[M // 2, :] *= 2.0 ** 500; cases.append(A)
+    A = base / np.abs(base).max() * 0.9; A[0, K - 1] = 4.0 - 2.0 ** -45; cases.append(A)     # an extreme mantissa
+    A = base / np.abs(base).max(axis=1, keepdims=True) * 1.75; cases.append(A)              # every maximum the same
+    try:
+        for fused in (1, 0):
+            lib.hip_ozaki_crt_set_fused_scan(fused)
+            for i in range(2):                      # twice: the counter the last workgroup leaves must be zero again
+                for A in cases:
+                    rc, got = run(A, True)
+                    assert rc == 0
+                    rc, want = run(A, False)
+                    assert rc == 0 and np.array_equal(got, want)
+                    assert ulp_distance(got, oracle.matmul_ozaki_crt(A, B)).max() <= MAX_ULP
+            for bad in (np.nan, np.inf, -np.inf):
+                A = base.copy(); A[M - 1, 7] = bad
+                assert run(A, True)[0] == -1
+            rc, got = run(base, True)               # and the call after a refusal is whole again
+            assert rc == 0 and np.array_equal(got, run(base, False)[1])
+    finally:
+        lib.hip_ozaki_crt_set_fused_scan(1)
+        lib.hip_ozaki_crt_release_prepared(h)
+
+
 def test_aligned_weight_split_matches_the_oracle_and_is_accurate(gpu):
     """hip_ozaki_crt_set_aligned_weights(1): the CRT weights split at a common bit.
     Residues and products are those of the default mode, the result equals the
