@@ -318,7 +318,7 @@ bool eshkol_hip_dgemm_is_thin_rows(uint64_t M, uint64_t K, uint64_t N, int trans
         const uint64_t blocks = ((thin + 63) / 64) * ((wide + 63) / 64);
         if (blocks > 48 || (wide * K > (2ull << 20) && blocks > 8)) return false;
     }
-    if (K > 0x7fffffffULL || wide > 0x7fffffffULL) return false;
+    if (K > 0x7fffff00ULL || wide > 0x7fffff00ULL) return false;      /* strip and round indices are ints */
     return wide * K >= (1ull << THIN_MIN_LOG2);
 }
 
