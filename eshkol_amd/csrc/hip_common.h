@@ -115,10 +115,10 @@ static inline uint64_t eshkol_product_pitch(uint64_t N) { return N >= 1024 ? rou
  * this way are not merged on the way out (the slice tier's reconstruction ran
  * twice as long with them). */
 /* The int8 contraction for a first operand of a few rows (igemm_thin_i8.hip): whether a
- * first operand of M rows is one (at most 64); hip_igemm_i8 sends interleaved planes of
- * such a product there, and the tiers then pad the first operand's planes to whole blocks
- * of 32 rows instead of 256. */
-bool eshkol_hip_igemm_is_thin(uint64_t M);
+ * product of M x N output planes is one (up to 128 rows, up to 160 against 4096 columns or
+ * more); hip_igemm_i8 sends interleaved planes of such a product there, and the tiers then
+ * pad the first operand's planes to whole blocks of 32 rows instead of 256. */
+bool eshkol_hip_igemm_is_thin(uint64_t M, uint64_t N);
 
 /* fp64 products of matrices far smaller than a tile, one or a batch (dgemm_small_f64.hip) */
 bool eshkol_hip_dgemm_is_small(uint64_t M, uint64_t K, uint64_t N);

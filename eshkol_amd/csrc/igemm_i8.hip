@@ -725,7 +725,7 @@ int eshkol_hip_igemm_direct_mode(void) { return g_direct; }
  * has enough 256 x 256 tiles to be worth a workgroup per CU, else 0. */
 extern "C" int hip_igemm_plane_layout(uint64_t M, uint64_t N, int n_out) {
     const uint64_t big = ((M + 255) / 256) * ((N + 255) / 256) * (uint64_t)(n_out > 0 ? n_out : 0);
-    if (eshkol_hip_igemm_is_thin(M)) return 1;     /* streams the second operand's planes */
+    if (eshkol_hip_igemm_is_thin(M, N)) return 1;     /* streams the second operand's planes */
     return (g_direct != 0 && big >= 128) ? 1 : 0;
 }
 
@@ -752,7 +752,7 @@ extern "C" int hip_igemm_i8(const HipIgemmArgs* args, void* stream) {
         if (a.ldk % 512 != 0 || a.max_pairs < 1) return -1;
         if ((a.a_plane_stride % (32ull * a.ldk)) || (a.b_plane_stride % (32ull * a.ldk))) return -1;
         /* a few rows against the second operand's planes: bound by reading those once */
-        if (eshkol_hip_igemm_is_thin(a.M)) return eshkol_hip_igemm_thin(a, st);
+        if (eshkol_hip_igemm_is_thin(a.M, a.N)) return eshkol_hip_igemm_thin(a, st);
         /* Products of at most 1024 bytes of k per row take the 256 x 128 kernel with
          * two workgroups per CU (measured 5 ... 13 % faster there, slower from 2048 on), and
          * so do launches with fewer 256 x 256 tiles than CUs, whatever their k: twice the

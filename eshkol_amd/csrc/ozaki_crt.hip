@@ -1022,7 +1022,7 @@ static int crt_matmul_impl(const double* A, const double* B, double* C,
     const int layout = keep_interleaved ? 1 : hip_igemm_plane_layout(M, N, num_moduli);
     /* a first operand of a few rows goes to the kernel that streams the second operand's
      * planes: its own planes then need whole blocks of 32 rows only */
-    const bool thin = layout == 1 && eshkol_hip_igemm_is_thin(M);
+    const bool thin = layout == 1 && eshkol_hip_igemm_is_thin(M, N);
     const uint64_t Mp = round_up_sz(M, thin ? 32 : 256), Np = round_up_sz(N, 256), ldk = round_up_sz(K, layout ? 512 : 256);
     /* Both operands come out as planes [row][k]. An operand stored with k
      * contiguous (A as given, B when the caller holds B^T) is read row by row;

@@ -104,8 +104,9 @@ void hip_dgemm_set_thin_rows(int from);
 void hip_dgemm_set_thin_rows_klast(int on);
 void hip_dgemm_set_thin_chunks(int on);
 
-/* Column blocks per workgroup of the int8 kernel for a first operand of at most 64 rows:
- * 0 (default) by the shape, 1 or 2 forced. Same results. */
+/* Which of the int8 kernels for a first operand of a few rows runs: 0 (default) by the
+ * shape; 1 or 2: the kernel for up to 64 rows with that many column blocks per workgroup;
+ * 3: the kernel that shares the rows through LDS. Same results. */
 void hip_igemm_set_thin_variant(int column_blocks);
 
 /* k-blocks kept in flight by the pipelined int8 kernel (1..3; 0 = simple kernel only). */
@@ -117,8 +118,8 @@ void hip_igemm_set_prefetch(int pf);
  * of k and for launches with fewer 256 x 256 tiles than CUs, 256 x 256 tiles and
  * one otherwise); 2: the 256 x 128 kernel for all of
  * them; 3: the 256 x 256 kernel for all of them; 0: row-major planes and the
- * register-staged kernels everywhere. With 1, a first operand of at most 64 rows
- * takes the kernel that streams the second operand's planes (any other value
+ * register-staged kernels everywhere. With 1, a first operand of a few rows
+ * takes the kernels that stream the second operand's planes (any other value
  * keeps such products on the kernels named). Same results; the switch exists to
  * compare them. */
 void hip_igemm_set_direct(int on);

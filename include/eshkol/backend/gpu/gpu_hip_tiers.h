@@ -106,8 +106,8 @@ int hip_bias_act_f64(double* Y, const double* bias, uint64_t rows, uint64_t cols
  * (metal_softfloat.h:3907-4100). Operand planes are K-contiguous int8 with a
  * row pitch of ldk bytes (multiple of 128, zero padded beyond K) and row counts
  * padded with zero rows to multiples of 256 (interleaved planes of a first operand
- * of at most 64 rows: to multiples of 32; such products take a kernel of their own
- * that streams the second operand's planes once). The pipelined kernel needs ldk to
+ * of at most 128 rows, or 160 where N >= 4096: to multiples of 32; such products take
+ * kernels of their own that stream the second operand's planes once). The pipelined kernel needs ldk to
  * be a multiple of 256, 1 <= max_pairs <= 64 and every output plane to have at
  * least one product (pair_first strictly increasing); pass max_pairs = 0 for
  * plans with empty planes: they take the simple kernel, which writes zeros. */
@@ -154,8 +154,8 @@ int hip_igemm_i8(const HipIgemmArgs* args, void* stream);
 /* The layout (HipIgemmArgs.layout) the tiers give their operand planes for a
  * contraction of n_out output planes of M x N: 1 when the launch has at least
  * 128 tiles of 256 x 256 and so takes the direct-to-LDS kernel, or when M is at
- * most 64 (the kernel for thin products), else 0. With 1 the k pitch is padded to
- * a multiple of 512. */
+ * most 128 (160 where N >= 4096: the kernels for a few rows), else 0. With 1 the k
+ * pitch is padded to a multiple of 512. */
 int hip_igemm_plane_layout(uint64_t M, uint64_t N, int n_out);
 
 /* ---- Ozaki-II CRT exact tier ------------------------------------------------

@@ -297,9 +297,11 @@ def test_plane_layout_decisions_are_host_arithmetic():
     assert lib.hip_igemm_plane_layout(1024, 1024, 7) == 0           # 112 tiles: too few
     assert lib.hip_igemm_plane_layout(512, 512, 16) == 0
     assert lib.hip_igemm_plane_layout(40, 4096, 16) == 1            # 16 tile columns x 16 planes
-    assert lib.hip_igemm_plane_layout(40, 512, 16) == 1             # at most 64 rows: the kernel that streams B's planes
-    assert lib.hip_igemm_plane_layout(64, 100, 2) == 1
-    assert lib.hip_igemm_plane_layout(65, 512, 16) == 0             # 32 tiles
+    assert lib.hip_igemm_plane_layout(40, 512, 16) == 1             # a few rows: the kernels that stream B's planes
+    assert lib.hip_igemm_plane_layout(128, 100, 2) == 1
+    assert lib.hip_igemm_plane_layout(129, 512, 16) == 0            # 32 tiles
+    assert lib.hip_igemm_plane_layout(160, 4096, 2) == 1            # up to 160 rows against 4096 columns
+    assert lib.hip_igemm_plane_layout(161, 4096, 2) == 0
     assert lib.hip_hgemm_plane_layout(8192, 8192, 1) == 1
     assert lib.hip_hgemm_plane_layout(1024, 1024, 1) == 0
     assert lib.hip_hgemm_plane_layout(1024, 1024, 8) == 1           # a batch fills the device

@@ -129,12 +129,16 @@ def test_output_planes_larger_than_the_product(gpu, M, K, N, out_rows, ldn, mode
 
 
 THIN_SHAPES = [(1, 512, 32), (5, 700, 100), (32, 4096, 1024), (33, 1000, 1300), (64, 2049, 257), (17, 130, 4096),
-               (64, 512, 4100), (32, 1, 1), (2, 513, 33)]
+               (64, 512, 4100), (32, 1, 1), (2, 513, 33),
+               # 33 ... 160 rows: rows shared through LDS (two row blocks only against many column blocks)
+               (40, 512, 4100), (65, 700, 100), (96, 4096, 1024), (128, 513, 300), (100, 1, 1), (129, 512, 4096),
+               (160, 1000, 4100), (97, 2049, 129)]
 
 
 @pytest.mark.parametrize("M,K,N", THIN_SHAPES)
 def test_thin_first_operand_residues(gpu, M, K, N):
-    """At most 64 rows of A, planes padded to whole blocks of 32 rows only: the kernel that streams B's planes."""
+    """A few rows of A (up to 128, up to 160 against 4096 columns or more), planes padded to whole blocks of 32
+    rows only: the kernels that stream B's planes."""
     rng = np.random.default_rng(M + K + N)
     a, b = planes(rng, 16, M, K, row_pad=32), planes(rng, 16, N, K)
     plan = [[(l, l)] for l in range(16)]
@@ -150,7 +154,8 @@ def test_thin_first_operand_residues(gpu, M, K, N):
 
 @pytest.mark.parametrize("mode", [0, 1])
 @pytest.mark.parametrize("M,K,N,out_rows,ldn", [(7, 700, 100, 7, 112), (40, 512, 1030, 40, 1280), (64, 300, 33, 64, 33),
-                                                (3, 1024, 95, 5, 95), (32, 520, 64, 32, 66)])
+                                                (3, 1024, 95, 5, 95), (32, 520, 64, 32, 66), (100, 700, 90, 101, 96),
+                                                (128, 512, 257, 128, 259), (50, 600, 4100, 64, 4112)])
 def test_thin_first_operand_plans_and_output_pitches(gpu, M, K, N, out_rows, ldn, mode):
     """Several products per output plane (the slice tier's plans), int32 sums and residues, output planes with
     a pitch of their own, also one that keeps no store aligned."""
