@@ -151,6 +151,7 @@ SIGNATURES = {
     "hip_igemm_set_direct": (None, [C.c_int]),
     "hip_igemm_set_cu_limit": (None, [C.c_int]),
     "hip_hgemm_set_direct": (None, [C.c_int]),
+    "hip_reduced_set_thin": (None, [C.c_int]),
     "hip_hgemm_plane_layout": (C.c_int, [u64, u64, u64]),
     "hip_hgemm_16_batched": (C.c_int, [vp, vp, u64, u64, u64, u64, u64, u64, u64, C.c_int, C.c_int, vp, vp]),
     "hip_convert_f64_to_16_planes": (C.c_int, [vp, vp, u64, u64, u64, u64, u64, C.c_int, C.c_int, C.c_int, vp]),

@@ -754,6 +754,175 @@ int convert_any(const double* in, uint16_t* out, uint64_t batch, uint64_t rows, 
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 
+/* ---- a few rows against a big second operand held as fp64 [K][N] ------------------------
+ * The tier on such a product spends its time on the second operand: read once as fp64 to
+ * narrow it, written as 16 bits, read again by a contraction that has a handful of tiles
+ * (32 x 4096 x 4096: 92 us, of which the operand read once is 27). Here it is read once:
+ * a workgroup takes a strip of 128 columns and a slice of k, its four waves deal the
+ * slice out sixteen k at a time; a lane loads four consecutive columns of eight rows of k
+ * (the 32 lanes of a half-wave 1 KiB of each row), narrows them in registers and has, for
+ * each of its four columns, the eight consecutive k of one matrix-core operand: four
+ * instructions per block of 32 rows, column j of instruction c being column 4 j + c of
+ * the strip. The first operand is narrowed beforehand (it is small) and its fragments come
+ * from L2. Same arithmetic as the tier's other kernels (16-bit operands, fp32 sums); the
+ * sums of the four waves meet in LDS, slices of k leave fp32 partial results that a second
+ * kernel adds in ascending order, rounds if asked and stores. */
+typedef double d4u_t __attribute__((ext_vector_type(4), aligned(8)));
+
+template <bool BF16>
+__device__ __forceinline__ void store_reduced(void* Cout, int out_mode, size_t idx, float x) {
+    if (out_mode == 2) x = round16<BF16>(x);
+    if (out_mode == 0) ((float*)Cout)[idx] = x;
+    else ((double*)Cout)[idx] = (double)x;
+}
+
+template <bool BF16, int RB>
+__global__ __launch_bounds__(256)
+void reduced_thin_kernel(const uint16_t* __restrict__ A16, int lda, int M,
+                         const double* __restrict__ B, int K, int N, int kc,
+                         float* __restrict__ part, long slice_stride, void* Cout, int out_mode) {
+    __shared__ v4f_t red[4][4][64];
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int li = lane & 31, lh = lane >> 5;
+    const int n0 = (int)blockIdx.x * 128, col = n0 + 4 * li;
+    const int ks = (int)blockIdx.y * kc;
+    const int ke = (ks + kc < K) ? ks + kc : K;
+    const bool edge = n0 + 128 > N;                              /* the same for the whole workgroup */
+    int oc[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) oc[c] = (col + c < N) ? col + c : N - 1;
+    v16f_t acc[RB][4];
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[rb][c][r] = 0.0f;
+
+    for (int k0 = ks + 16 * wave; k0 < ke; k0 += 64) {
+        const int kk = k0 + 8 * lh;
+        double v[8][4];
+        if (k0 + 16 <= ke && !edge) {                           /* the same for the whole wave */
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const d4u_t x = *(const d4u_t*)(B + (size_t)(kk + j) * N + col);
+                v[j][0] = x[0]; v[j][1] = x[1]; v[j][2] = x[2]; v[j][3] = x[3];
+            }
+        } else {
+            /* the last, partial round of the slice and the last strip: clamped addresses,
+             * zeros beyond the slice (the first operand is not zero there) */
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const bool in = kk + j < ke;
+                const size_t kr = (size_t)(in ? kk + j : ke - 1);
+#pragma unroll
+                for (int c = 0; c < 4; c++) { const double x = B[kr * N + oc[c]]; v[j][c] = in ? x : 0.0; }
+            }
+        }
+        v4i_t op[4];
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) op[c][q] = (int)narrow_pair<BF16>(v[2 * q][c], v[2 * q + 1][c]);
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++) {
+            const v4i_t a = *(const v4i_t*)(A16 + (size_t)(rb * 32 + li) * lda + kk);
+#pragma unroll
+            for (int c = 0; c < 4; c++) H16Op<BF16>::mfma(op[c], a, acc[rb][c]);
+        }
+    }
+    /* acc[rb][c]: lane%32 is the output row, registers 4v .. 4v+3 are columns j = 8v + 4 (lane/32) + 0..3
+     * of instruction c, i.e. columns n0 + 4 j + c. One (rb, c) at a time through LDS. */
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            if (rb + c) __syncthreads();
+#pragma unroll
+            for (int vv = 0; vv < 4; vv++)
+                red[wave][vv][lane] = (v4f_t){acc[rb][c][4 * vv], acc[rb][c][4 * vv + 1], acc[rb][c][4 * vv + 2], acc[rb][c][4 * vv + 3]};
+            __syncthreads();
+            const int row = rb * 32 + li;
+            if (row >= M) continue;                              /* the barriers sit above */
+            v4f_t s = red[0][wave][lane];
+#pragma unroll
+            for (int w = 1; w < 4; w++) s += red[w][wave][lane];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int cx = n0 + 4 * (8 * wave + 4 * lh + e) + c;
+                if (cx >= N) continue;
+                if (part) part[(size_t)blockIdx.y * slice_stride + (size_t)row * N + cx] = s[e];
+                else store_reduced<BF16>(Cout, out_mode, (size_t)row * N + cx, s[e]);
+            }
+        }
+    }
+}
+
+template <bool BF16>
+__global__ __launch_bounds__(256)
+void reduced_thin_sum_kernel(const float* __restrict__ part, int slices, long n, void* Cout, int out_mode) {
+    const long e = (long)blockIdx.x * 256 + threadIdx.x;
+    if (e >= n) return;
+    float s = 0.0f;
+    int y = 0;
+    for (; y + 8 <= slices; y += 8) {                            /* eight loads in flight, added in ascending order */
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = part[(size_t)(y + u) * n + e];
+#pragma unroll
+        for (int u = 0; u < 8; u++) s += v[u];
+    }
+    for (; y < slices; y++) s += part[(size_t)y * n + e];
+    store_reduced<BF16>(Cout, out_mode, (size_t)e, s);
+}
+
+int g_reduced_thin = 1;
+
+/* Slices of k for the kernel above: about three workgroups per CU, at least 256 k each
+ * (128 where the strips are few), at most 64 slices. By the shape alone. */
+struct ThinPlan { int slices, kc; size_t part_bytes; };
+ThinPlan reduced_thin_plan(uint64_t M, uint64_t K, uint64_t N) {
+    const int strips = (int)((N + 127) / 128);
+    const int min_kc = strips <= 4 ? 128 : 256;
+    int slices = (3 * eshkol_hip_num_cus()) / strips;
+    if (slices > (int)(K / min_kc)) slices = (int)(K / min_kc);
+    if (slices > 64) slices = 64;
+    if (slices < 1) slices = 1;
+    int kc = (int)((K + slices - 1) / slices);
+    kc = (kc + 63) / 64 * 64;
+    slices = (int)((K + kc - 1) / kc);
+    return { slices, kc, slices > 1 ? (size_t)slices * M * N * sizeof(float) : 0 };
+}
+
+/* up to 64 rows against a second operand as the runtime stores it (B [K][N]) that is worth
+ * streaming; everything else keeps the narrowing kernels and the tiled contraction */
+bool reduced_is_thin(uint64_t batch, uint64_t M, uint64_t K, uint64_t N, int trans_b) {
+    return g_reduced_thin && batch == 1 && !trans_b && M <= 64 && N >= 128 && K >= 64 && N * K >= (1ull << 21) &&
+           K <= 0x3fffff00ULL && N <= 0x7fffff00ULL;
+}
+
+/* A16: M rows (padded to 64) of ld elements, written here; part: reduced_thin_plan().part_bytes. */
+int reduced_thin(const double* A, const double* B, double* C, uint64_t M, uint64_t K, uint64_t N, int trans_a,
+                 int is_bf16, int round_output, uint16_t* A16, uint64_t ld, float* part, hipStream_t st) {
+    if (convert_any(A, A16, 1, M, K, 64, ld, is_bf16, trans_a != 0, 0, st) != 0) return -1;
+    const ThinPlan pl = reduced_thin_plan(M, K, N);
+    const dim3 grid((unsigned)((N + 127) / 128), (unsigned)pl.slices);
+    const int out_mode = round_output ? 2 : 1;
+    float* p = pl.slices > 1 ? part : nullptr;
+    const long stride = (long)(M * N);
+#define THIN(BF, RB) hipLaunchKernelGGL((reduced_thin_kernel<BF, RB>), grid, dim3(256), 0, st, A16, (int)ld, (int)M, B, (int)K, \
+                                        (int)N, pl.kc, p, stride, (void*)C, out_mode)
+    if (is_bf16) { if (M <= 32) THIN(true, 1); else THIN(true, 2); }
+    else         { if (M <= 32) THIN(false, 1); else THIN(false, 2); }
+#undef THIN
+    if (p) {
+        const long n = (long)(M * N);
+        if (is_bf16) hipLaunchKernelGGL(reduced_thin_sum_kernel<true>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, p, pl.slices, n, (void*)C, out_mode);
+        else         hipLaunchKernelGGL(reduced_thin_sum_kernel<false>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, p, pl.slices, n, (void*)C, out_mode);
+    }
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
 /* Padded operand shape and plane layout of the reduced tier for a batch of
  * M x K x N products: interleaved 16-bit operands (and a k pitch of whole
  * 512-byte groups) when the launch has enough 256 x 256 tiles for the
@@ -783,6 +952,9 @@ int reduced_pipeline(const double* A, const double* B, double* C, uint64_t batch
 /* Tuning hook: 0 keeps the 16-bit tier on row-major operands and the
  * register-staged kernels. Same results. */
 extern "C" void hip_hgemm_set_direct(int on) { EshkolHipLock lk; g_direct16 = on ? 1 : 0; }
+/* Tuning hook: 0 keeps a few rows against a big second operand on the narrowing kernels
+ * and the tiled contraction. Same arithmetic, another order of the fp32 sums. */
+extern "C" void hip_reduced_set_thin(int on) { EshkolHipLock lk; g_reduced_thin = on ? 1 : 0; }
 
 extern "C" int hip_hgemm_plane_layout(uint64_t M, uint64_t N, uint64_t batch) {
     const uint64_t tiles = ((M + 255) / 256) * ((N + 255) / 256) * batch;
@@ -829,6 +1001,14 @@ extern "C" int hip_matmul_reduced_f64_batched_ex(const double* A, const double* 
     if (M > 0x7fffffffULL || K > 0x3fffffffULL || N > 0x7fffffffULL || batch > 0x7fffffffULL) return -1;
     hipStream_t st = (hipStream_t)stream;
     const ReducedShape sh = reduced_shape(batch, M, K, N);
+    if (reduced_is_thin(batch, M, K, N, trans_b)) {
+        /* a few rows: the second operand is read once, as fp64, and never copied */
+        const ThinPlan pl = reduced_thin_plan(M, K, N);
+        uint16_t* A16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_A, 64 * sh.ld * 2);
+        float* part = pl.part_bytes ? (float*)eshkol_hip_workspace(WS_DGEMM_PARTIAL, pl.part_bytes) : nullptr;
+        if (A16 && (part || !pl.part_bytes))
+            return reduced_thin(A, B, C, M, K, N, trans_a, dtype == 3, round_output, A16, sh.ld, part, st);
+    }
     uint16_t* A16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_A, batch * sh.Mp * sh.ld * 2);
     uint16_t* B16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_B, batch * sh.Np * sh.ld * 2);
     if (!A16 || !B16) return -1;
@@ -914,6 +1094,21 @@ extern "C" int hip_matmul_reduced_f64_noalloc(const double* A, const double* B, 
     }
     unsigned char* base = noalloc_scratch();
     if (!base) return -1;
+    if (reduced_is_thin(1, M, K, N, 0)) {
+        /* the same kernel and slices as the workspace entry point: the first operand's 64
+         * rows of 16-bit values and the fp32 partial sums take the place of the copies */
+        const ThinPlan pl = reduced_thin_plan(M, K, N);
+        const uint64_t a16 = round_up_sz(64 * sh.ld * 2, 256);
+        if (a16 + pl.part_bytes > NOALLOC_SCRATCH_BYTES) {
+            fprintf(stderr, "[GPU] hip_matmul_reduced_f64_noalloc: %llux%llux%llu needs %llu bytes of partial sums, "
+                            "the static scratch holds %llu; use hip_matmul_reduced_f64\n",
+                    (unsigned long long)M, (unsigned long long)K, (unsigned long long)N,
+                    (unsigned long long)(a16 + pl.part_bytes), (unsigned long long)NOALLOC_SCRATCH_BYTES);
+            return -3;
+        }
+        return reduced_thin(A, B, C, M, K, N, 0, dtype == 3, round_output, (uint16_t*)base, sh.ld,
+                            (float*)(base + a16), (hipStream_t)stream);
+    }
     return reduced_pipeline(A, B, C, 1, M, K, N, 0, 0, dtype == 3, round_output,
                             (uint16_t*)base, (uint16_t*)(base + a_bytes), sh, (hipStream_t)stream);
 }

@@ -9,7 +9,7 @@ import pytest
 import eshkol_amd as ea
 import oracle
 from eshkol_amd import synth
-from gpu_util import normwise, run_reduced, stream
+from gpu_util import Operands, normwise, run_reduced, stream
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-2
@@ -37,6 +37,50 @@ def test_reduced_matches_reference_statement(gpu, M, K, N, dtype):
     if dtype == 3:
         # fp32 accumulation order is unspecified; the sum is close to a k-ascending one
         assert normwise(wide, oracle.matmul_reduced_f32acc(A, B, dtype, False), Ar, Br) <= 1e-6
+
+
+@pytest.mark.parametrize("dtype", [2, 3])
+@pytest.mark.parametrize("M,K,N", [(1, 8192, 256), (5, 7000, 300), (32, 4096, 1024), (33, 2049, 1030), (64, 520, 4099),
+                                   (17, 512, 4100), (40, 16400, 130)])
+def test_a_few_rows_against_a_big_second_operand(gpu, M, K, N, dtype):
+    """Up to 64 rows against B as the runtime stores it: B is read once as fp64 and narrowed in registers on
+    its way to the matrix cores. Same arithmetic as the tier's other kernels (16-bit operands, fp32 sums), so:
+    the reference statement within the fp32 bar, the rounded output the unrounded one rounded, the tiled path
+    within the scatter of fp32 summation orders, an infinity in B in its own column only, the entry point that
+    allocates nothing the same bits."""
+    print("reduced, few rows", M, K, N, dtype, flush=True)
+    lib = ea.load()
+    A = oracle.reduce_precision(synth.normal(700 + M, (M, K), 1.0 / np.sqrt(K)), dtype)
+    B = oracle.reduce_precision(synth.normal(800 + N, (K, N), 1.0 / np.sqrt(K)), dtype)
+    ref = oracle.matmul_f64(A, B)
+    wide = run_reduced(A, B, dtype, round_output=False)
+    assert normwise(wide, ref, A, B) <= 1e-6
+    narrow = run_reduced(A, B, dtype, round_output=True)
+    ok = (np.abs(wide) >= 2.0 ** -14) | (wide == 0)
+    assert np.array_equal(narrow[ok], oracle.reduce_precision(wide, dtype)[ok])
+    lib.hip_reduced_set_thin(0)
+    try:
+        tiled = run_reduced(A, B, dtype, round_output=False)
+    finally:
+        lib.hip_reduced_set_thin(1)
+    assert normwise(wide, tiled, A, B) <= 1e-6 and not np.array_equal(wide, tiled) or M * N < 64
+    # operands that are not 16-bit values yet are narrowed on the way, as by the narrowing kernels
+    A2, B2 = synth.normal(1 + M, (M, K)), synth.normal(2 + N, (K, N))
+    got = run_reduced(A2, B2, dtype, round_output=False)
+    want = oracle.matmul_f64(oracle.reduce_precision(A2, dtype), oracle.reduce_precision(B2, dtype))
+    assert normwise(got, want, A2, B2) <= 1e-6
+    # an infinity in the last row of k and in the last column shows in its own column only
+    B3 = B.copy(); B3[K - 1, 3] = np.inf; B3[0, N - 1] = -np.inf
+    A3 = A.copy(); A3[:, K - 1] = np.abs(A3[:, K - 1]) + 2.0 ** -6; A3[:, 0] = np.abs(A3[:, 0]) + 2.0 ** -6
+    A3 = oracle.reduce_precision(A3, dtype)
+    got = run_reduced(A3, B3, dtype, round_output=False)
+    assert np.all(got[:, 3] == np.inf) and np.all(got[:, N - 1] == -np.inf)
+    keep = np.ones(N, bool); keep[[3, N - 1]] = False
+    assert np.isfinite(got[:, keep]).all()
+    if M * K <= (1 << 20) and K * N <= (4 << 20):
+        ops = Operands(A, B)
+        assert lib.hip_matmul_reduced_f64_noalloc(ops.dA.ptr, ops.dB.ptr, ops.dC.ptr, M, K, N, dtype, 0, stream()) == 0
+        assert np.array_equal(ops.result(), wide)
 
 
 @pytest.mark.parametrize("dtype", [2, 3])
