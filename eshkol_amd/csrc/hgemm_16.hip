@@ -780,7 +780,7 @@ template <bool BF16, int RB>
 __global__ __launch_bounds__(256)
 void reduced_thin_kernel(const uint16_t* __restrict__ A16, int lda, int M,
                          const double* __restrict__ B, int K, int N, int kc,
-                         float* __restrict__ part, long slice_stride, void* Cout, int out_mode) {
+                         float* __restrict__ part, long slice_stride, void* Cout, int out_mode, long c_r, long c_o) {
     __shared__ v4f_t red[4][4][64];
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 31, lh = lane >> 5;
@@ -852,15 +852,103 @@ void reduced_thin_kernel(const uint16_t* __restrict__ A16, int lda, int M,
                 const int cx = n0 + 4 * (8 * wave + 4 * lh + e) + c;
                 if (cx >= N) continue;
                 if (part) part[(size_t)blockIdx.y * slice_stride + (size_t)row * N + cx] = s[e];
-                else store_reduced<BF16>(Cout, out_mode, (size_t)row * N + cx, s[e]);
+                else store_reduced<BF16>(Cout, out_mode, (size_t)((long)row * c_r + (long)cx * c_o), s[e]);
             }
         }
     }
 }
 
+/* The same against a big operand with k contiguous, G[O][K] (the second operand held
+ * transposed, or a matrix against a few columns): a lane loads eight consecutive k of one
+ * output's row (64 bytes; the two halves of a wave the sixteen k of a round) and narrows
+ * them into one matrix-core operand; a workgroup's strip is four blocks of 32 outputs. */
+template <bool BF16, int RB>
+__global__ __launch_bounds__(256)
+void reduced_thin_klast_kernel(const uint16_t* __restrict__ T16, int ldt, int R,
+                               const double* __restrict__ G, int K, int O, int kc,
+                               float* __restrict__ part, long slice_stride, void* Cout, int out_mode, long c_r, long c_o) {
+    __shared__ v4f_t red[4][4][64];
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int li = lane & 31, lh = lane >> 5;
+    const int o0 = (int)blockIdx.x * 128;
+    const int ks = (int)blockIdx.y * kc;
+    const int ke = (ks + kc < K) ? ks + kc : K;
+    size_t g_off[4];
+#pragma unroll
+    for (int cb = 0; cb < 4; cb++) {
+        const int o = o0 + 32 * cb + li;
+        g_off[cb] = (size_t)(o < O ? o : O - 1) * K;            /* rows beyond the operand repeat the last: never stored */
+    }
+    v16f_t acc[RB][4];
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+        for (int cb = 0; cb < 4; cb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[rb][cb][r] = 0.0f;
+
+    for (int k0 = ks + 16 * wave; k0 < ke; k0 += 64) {
+        const int kk = k0 + 8 * lh;
+        v4i_t op[4];
+        if (k0 + 16 <= ke) {                                    /* the same for the whole wave */
+#pragma unroll
+            for (int cb = 0; cb < 4; cb++) {
+                const d4u_t x0 = *(const d4u_t*)(G + g_off[cb] + kk), x1 = *(const d4u_t*)(G + g_off[cb] + kk + 4);
+                op[cb] = (v4i_t){(int)narrow_pair<BF16>(x0[0], x0[1]), (int)narrow_pair<BF16>(x0[2], x0[3]),
+                                 (int)narrow_pair<BF16>(x1[0], x1[1]), (int)narrow_pair<BF16>(x1[2], x1[3])};
+            }
+        } else {
+#pragma unroll
+            for (int cb = 0; cb < 4; cb++) {
+                double x[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const bool in = kk + j < ke;
+                    const double g = G[g_off[cb] + (in ? kk + j : ke - 1)];
+                    x[j] = in ? g : 0.0;
+                }
+                op[cb] = (v4i_t){(int)narrow_pair<BF16>(x[0], x[1]), (int)narrow_pair<BF16>(x[2], x[3]),
+                                 (int)narrow_pair<BF16>(x[4], x[5]), (int)narrow_pair<BF16>(x[6], x[7])};
+            }
+        }
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++) {
+            const v4i_t a = *(const v4i_t*)(T16 + (size_t)(rb * 32 + li) * ldt + kk);
+#pragma unroll
+            for (int cb = 0; cb < 4; cb++) H16Op<BF16>::mfma(op[cb], a, acc[rb][cb]);
+        }
+    }
+    /* acc[rb][cb]: lane%32 is the thin row, registers 4v .. 4v+3 are outputs o0 + 32 cb + 8v + 4 (lane/32) + 0..3 */
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++) {
+#pragma unroll
+        for (int cb = 0; cb < 4; cb++) {
+            if (rb + cb) __syncthreads();
+#pragma unroll
+            for (int vv = 0; vv < 4; vv++)
+                red[wave][vv][lane] = (v4f_t){acc[rb][cb][4 * vv], acc[rb][cb][4 * vv + 1], acc[rb][cb][4 * vv + 2], acc[rb][cb][4 * vv + 3]};
+            __syncthreads();
+            const int row = rb * 32 + li;
+            if (row >= R) continue;                              /* the barriers sit above */
+            v4f_t s = red[0][wave][lane];
+#pragma unroll
+            for (int w = 1; w < 4; w++) s += red[w][wave][lane];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int o = o0 + 32 * cb + 8 * wave + 4 * lh + e;
+                if (o >= O) continue;
+                if (part) part[(size_t)blockIdx.y * slice_stride + (size_t)row * O + o] = s[e];
+                else store_reduced<BF16>(Cout, out_mode, (size_t)((long)row * c_r + (long)o * c_o), s[e]);
+            }
+        }
+    }
+}
+
+/* C(r, o) = the slices' partial sums [slice][r][o] added in ascending order, rounded if asked */
 template <bool BF16>
 __global__ __launch_bounds__(256)
-void reduced_thin_sum_kernel(const float* __restrict__ part, int slices, long n, void* Cout, int out_mode) {
+void reduced_thin_sum_kernel(const float* __restrict__ part, int slices, long n, int O, void* Cout, int out_mode,
+                             long c_r, long c_o) {
     const long e = (long)blockIdx.x * 256 + threadIdx.x;
     if (e >= n) return;
     float s = 0.0f;
@@ -873,16 +961,18 @@ void reduced_thin_sum_kernel(const float* __restrict__ part, int slices, long n,
         for (int u = 0; u < 8; u++) s += v[u];
     }
     for (; y < slices; y++) s += part[(size_t)y * n + e];
-    store_reduced<BF16>(Cout, out_mode, (size_t)e, s);
+    const long r = e / O, o = e - r * O;
+    store_reduced<BF16>(Cout, out_mode, (size_t)(r * c_r + o * c_o), s);
 }
 
 int g_reduced_thin = 1;
 
-/* Slices of k for the kernel above: about three workgroups per CU, at least 256 k each
- * (128 where the strips are few), at most 64 slices. By the shape alone. */
+/* Slices of k for the kernels above: about three workgroups per CU, at least 256 k each
+ * (128 where the strips are few), at most 64 slices. By the shape alone. R: rows on the
+ * thin side, O: outputs on the wide one. */
 struct ThinPlan { int slices, kc; size_t part_bytes; };
-ThinPlan reduced_thin_plan(uint64_t M, uint64_t K, uint64_t N) {
-    const int strips = (int)((N + 127) / 128);
+ThinPlan reduced_thin_plan(uint64_t R, uint64_t K, uint64_t O) {
+    const int strips = (int)((O + 127) / 128);
     const int min_kc = strips <= 4 ? 128 : 256;
     int slices = (3 * eshkol_hip_num_cus()) / strips;
     if (slices > (int)(K / min_kc)) slices = (int)(K / min_kc);
@@ -891,34 +981,54 @@ ThinPlan reduced_thin_plan(uint64_t M, uint64_t K, uint64_t N) {
     int kc = (int)((K + slices - 1) / slices);
     kc = (kc + 63) / 64 * 64;
     slices = (int)((K + kc - 1) / kc);
-    return { slices, kc, slices > 1 ? (size_t)slices * M * N * sizeof(float) : 0 };
+    return { slices, kc, slices > 1 ? (size_t)slices * R * O * sizeof(float) : 0 };
 }
 
-/* up to 64 rows against a second operand as the runtime stores it (B [K][N]) that is worth
- * streaming; everything else keeps the narrowing kernels and the tiled contraction */
-bool reduced_is_thin(uint64_t batch, uint64_t M, uint64_t K, uint64_t N, int trans_b) {
-    return g_reduced_thin && batch == 1 && !trans_b && M <= 64 && N >= 128 && K >= 64 && N * K >= (1ull << 21) &&
-           K <= 0x3fffff00ULL && N <= 0x7fffff00ULL;
+/* up to 64 rows (or columns) against a big operand that is worth streaming, every operand
+ * form; everything else keeps the narrowing kernels and the tiled contraction */
+bool reduced_is_thin(uint64_t batch, uint64_t M, uint64_t K, uint64_t N) {
+    const uint64_t thin = M <= N ? M : N, wide = M <= N ? N : M;
+    return g_reduced_thin && batch == 1 && thin <= 64 && wide >= 128 && K >= 64 && wide * K >= (1ull << 21) &&
+           K <= 0x3fffff00ULL && wide <= 0x7fffff00ULL;
+}
+ThinPlan reduced_thin_plan_for(uint64_t M, uint64_t K, uint64_t N) {
+    return M <= N ? reduced_thin_plan(M, K, N) : reduced_thin_plan(N, K, M);
 }
 
-/* A16: M rows (padded to 64) of ld elements, written here; part: reduced_thin_plan().part_bytes. */
-int reduced_thin(const double* A, const double* B, double* C, uint64_t M, uint64_t K, uint64_t N, int trans_a,
-                 int is_bf16, int round_output, uint16_t* A16, uint64_t ld, float* part, hipStream_t st) {
-    if (convert_any(A, A16, 1, M, K, 64, ld, is_bf16, trans_a != 0, 0, st) != 0) return -1;
-    const ThinPlan pl = reduced_thin_plan(M, K, N);
-    const dim3 grid((unsigned)((N + 127) / 128), (unsigned)pl.slices);
+/* T16: 64 rows of ld elements for the thin operand's 16-bit copy, written here; part:
+ * reduced_thin_plan_for().part_bytes. */
+int reduced_thin(const double* A, const double* B, double* C, uint64_t M, uint64_t K, uint64_t N, int trans_a, int trans_b,
+                 int is_bf16, int round_output, uint16_t* T16, uint64_t ld, float* part, hipStream_t st) {
+    const bool thin_m = M <= N;
+    const uint64_t R = thin_m ? M : N, O = thin_m ? N : M;
+    /* the thin operand as rows of k: A (k-major when the caller holds A^T), or B's columns
+     * (k-major as the runtime stores B, rows of k when the caller holds B^T) */
+    const double* T = thin_m ? A : B;
+    const bool t_kmajor = thin_m ? trans_a != 0 : trans_b == 0;
+    if (convert_any(T, T16, 1, R, K, 64, ld, is_bf16, t_kmajor, 0, st) != 0) return -1;
+    const double* G = thin_m ? B : A;
+    const bool kfirst = thin_m ? trans_b == 0 : trans_a != 0;    /* the big operand has the output index contiguous */
+    const long c_r = thin_m ? (long)N : 1, c_o = thin_m ? 1 : (long)N;
+    const ThinPlan pl = reduced_thin_plan(R, K, O);
+    const dim3 grid((unsigned)((O + 127) / 128), (unsigned)pl.slices);
     const int out_mode = round_output ? 2 : 1;
     float* p = pl.slices > 1 ? part : nullptr;
-    const long stride = (long)(M * N);
-#define THIN(BF, RB) hipLaunchKernelGGL((reduced_thin_kernel<BF, RB>), grid, dim3(256), 0, st, A16, (int)ld, (int)M, B, (int)K, \
-                                        (int)N, pl.kc, p, stride, (void*)C, out_mode)
-    if (is_bf16) { if (M <= 32) THIN(true, 1); else THIN(true, 2); }
-    else         { if (M <= 32) THIN(false, 1); else THIN(false, 2); }
+    const long stride = (long)(R * O);
+#define THIN(KERN, BF, RB) hipLaunchKernelGGL((KERN<BF, RB>), grid, dim3(256), 0, st, T16, (int)ld, (int)R, G, (int)K, \
+                                              (int)O, pl.kc, p, stride, (void*)C, out_mode, c_r, c_o)
+    if (kfirst) {
+        if (is_bf16) { if (R <= 32) THIN(reduced_thin_kernel, true, 1); else THIN(reduced_thin_kernel, true, 2); }
+        else         { if (R <= 32) THIN(reduced_thin_kernel, false, 1); else THIN(reduced_thin_kernel, false, 2); }
+    } else {
+        if (is_bf16) { if (R <= 32) THIN(reduced_thin_klast_kernel, true, 1); else THIN(reduced_thin_klast_kernel, true, 2); }
+        else         { if (R <= 32) THIN(reduced_thin_klast_kernel, false, 1); else THIN(reduced_thin_klast_kernel, false, 2); }
+    }
 #undef THIN
     if (p) {
-        const long n = (long)(M * N);
-        if (is_bf16) hipLaunchKernelGGL(reduced_thin_sum_kernel<true>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, p, pl.slices, n, (void*)C, out_mode);
-        else         hipLaunchKernelGGL(reduced_thin_sum_kernel<false>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, p, pl.slices, n, (void*)C, out_mode);
+        const long n = (long)(R * O);
+        const dim3 sgrid((unsigned)((n + 255) / 256));
+        if (is_bf16) hipLaunchKernelGGL(reduced_thin_sum_kernel<true>, sgrid, dim3(256), 0, st, p, pl.slices, n, (int)O, (void*)C, out_mode, c_r, c_o);
+        else         hipLaunchKernelGGL(reduced_thin_sum_kernel<false>, sgrid, dim3(256), 0, st, p, pl.slices, n, (int)O, (void*)C, out_mode, c_r, c_o);
     }
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
@@ -1001,13 +1111,13 @@ extern "C" int hip_matmul_reduced_f64_batched_ex(const double* A, const double* 
     if (M > 0x7fffffffULL || K > 0x3fffffffULL || N > 0x7fffffffULL || batch > 0x7fffffffULL) return -1;
     hipStream_t st = (hipStream_t)stream;
     const ReducedShape sh = reduced_shape(batch, M, K, N);
-    if (reduced_is_thin(batch, M, K, N, trans_b)) {
-        /* a few rows: the second operand is read once, as fp64, and never copied */
-        const ThinPlan pl = reduced_thin_plan(M, K, N);
+    if (reduced_is_thin(batch, M, K, N)) {
+        /* a few rows or columns: the big operand is read once, as fp64, and never copied */
+        const ThinPlan pl = reduced_thin_plan_for(M, K, N);
         uint16_t* A16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_A, 64 * sh.ld * 2);
         float* part = pl.part_bytes ? (float*)eshkol_hip_workspace(WS_DGEMM_PARTIAL, pl.part_bytes) : nullptr;
         if (A16 && (part || !pl.part_bytes))
-            return reduced_thin(A, B, C, M, K, N, trans_a, dtype == 3, round_output, A16, sh.ld, part, st);
+            return reduced_thin(A, B, C, M, K, N, trans_a, trans_b, dtype == 3, round_output, A16, sh.ld, part, st);
     }
     uint16_t* A16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_A, batch * sh.Mp * sh.ld * 2);
     uint16_t* B16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_B, batch * sh.Np * sh.ld * 2);
@@ -1094,10 +1204,10 @@ extern "C" int hip_matmul_reduced_f64_noalloc(const double* A, const double* B, 
     }
     unsigned char* base = noalloc_scratch();
     if (!base) return -1;
-    if (reduced_is_thin(1, M, K, N, 0)) {
+    if (reduced_is_thin(1, M, K, N)) {
         /* the same kernel and slices as the workspace entry point: the first operand's 64
          * rows of 16-bit values and the fp32 partial sums take the place of the copies */
-        const ThinPlan pl = reduced_thin_plan(M, K, N);
+        const ThinPlan pl = reduced_thin_plan_for(M, K, N);
         const uint64_t a16 = round_up_sz(64 * sh.ld * 2, 256);
         if (a16 + pl.part_bytes > NOALLOC_SCRATCH_BYTES) {
             fprintf(stderr, "[GPU] hip_matmul_reduced_f64_noalloc: %llux%llux%llu needs %llu bytes of partial sums, "
@@ -1106,7 +1216,7 @@ extern "C" int hip_matmul_reduced_f64_noalloc(const double* A, const double* B, 
                     (unsigned long long)(a16 + pl.part_bytes), (unsigned long long)NOALLOC_SCRATCH_BYTES);
             return -3;
         }
-        return reduced_thin(A, B, C, M, K, N, 0, dtype == 3, round_output, (uint16_t*)base, sh.ld,
+        return reduced_thin(A, B, C, M, K, N, 0, 0, dtype == 3, round_output, (uint16_t*)base, sh.ld,
                             (float*)(base + a16), (hipStream_t)stream);
     }
     return reduced_pipeline(A, B, C, 1, M, K, N, 0, 0, dtype == 3, round_output,

@@ -84,6 +84,40 @@ def test_a_few_rows_against_a_big_second_operand(gpu, M, K, N, dtype):
 
 
 @pytest.mark.parametrize("dtype", [2, 3])
+@pytest.mark.parametrize("thin,K,wide", [(1, 8192, 300), (7, 2049, 1030), (33, 4100, 520), (64, 515, 4099)])
+def test_a_few_rows_or_columns_in_every_operand_form(gpu, thin, K, wide, dtype):
+    """The thin side may be M or N, and either operand may be held transposed: two kernels (the big operand
+    with the output index contiguous, or with k contiguous) serve all of them. Against the reference statement
+    within the fp32 bar, and the tiled path within the scatter of fp32 summation orders."""
+    print("reduced, thin side, forms", thin, K, wide, dtype, flush=True)
+    lib = ea.load()
+    for (M, N) in ((thin, wide), (wide, thin)):
+        A = oracle.reduce_precision(synth.normal(70 + M, (M, K), 1.0 / np.sqrt(K)), dtype)
+        B = oracle.reduce_precision(synth.normal(80 + N, (K, N), 1.0 / np.sqrt(K)), dtype)
+        ref = oracle.matmul_f64(A, B)
+        for ta, tb in ((0, 0), (0, 1), (1, 0)):
+            X = np.ascontiguousarray(A.T) if ta else A
+            Y = np.ascontiguousarray(B.T) if tb else B
+            dX, dY, dC = ea.DeviceArray.from_host(X), ea.DeviceArray.from_host(Y), ea.DeviceArray((M, N))
+            outs = []
+            for on in (1, 0):
+                lib.hip_reduced_set_thin(on)
+                try:
+                    assert lib.hip_matmul_reduced_f64_ex(dX.ptr, dY.ptr, dC.ptr, M, K, N, ta, tb, dtype, 0, stream()) == 0
+                    ea.synchronize()
+                finally:
+                    lib.hip_reduced_set_thin(1)
+                outs.append(dC.download())
+            assert normwise(outs[0], ref, A, B) <= 1e-6, (M, N, ta, tb)
+            assert normwise(outs[0], outs[1], A, B) <= 1e-6
+            assert lib.hip_matmul_reduced_f64_ex(dX.ptr, dY.ptr, dC.ptr, M, K, N, ta, tb, dtype, 1, stream()) == 0
+            ea.synchronize()
+            narrow = dC.download()
+            ok = (np.abs(outs[0]) >= 2.0 ** -14) | (outs[0] == 0)
+            assert np.array_equal(narrow[ok], oracle.reduce_precision(outs[0], dtype)[ok])
+
+
+@pytest.mark.parametrize("dtype", [2, 3])
 @pytest.mark.parametrize("M,K,N", [(3072, 256, 3072), (3000, 200, 2900), (3001, 200, 2901), (3072, 256, 3073)])
 def test_rounded_output_of_the_kernel_for_large_products(gpu, M, K, N, dtype):
     """From 128 tiles of 256 x 256 on, the tier's contraction is the kernel that loads its
