@@ -463,6 +463,18 @@ def main():
         log("batched reduced tier, 64 experts: %.3f ms in one launch per stage, %.3f ms as a loop" % (wo, wl))
         for d in (xa, xb, xc):
             d.free()
+        # a few rows against a layer's weights held as the runtime holds them (f64 storage, [K][N]): the tier
+        # reads them once and narrows them in registers; the floor is that one read
+        tm, tk, tn = 32, 4096, 4096
+        ta_ = ea.DeviceArray.from_host(synth.normal(65, (tm, tk), 1.0 / np.sqrt(tk)))
+        tb_ = ea.DeviceArray.from_host(synth.normal(66, (tk, tn), 1.0 / np.sqrt(tk)))
+        tc_ = ea.DeviceArray((tm, tn))
+        _, wt = timed(lambda: lib.hip_matmul_reduced_f64(ta_.ptr, tb_.ptr, tc_.ptr, tm, tk, tn, 3, 1, st), k=20, w=5)
+        tiers["reduced_bf16_32x4096x4096"] = {"ms": wt, "weights_GBps": 8.0 * tk * tn / (wt * 1e-3) / 1e9,
+                                             "frac_of_hbm": 8.0 * tk * tn / (wt * 1e-3) / 8e12}
+        log("reduced bf16, 32 rows against 4096 x 4096: %.3f ms (%.0f GB/s of weights)" % (wt, 8.0 * tk * tn / (wt * 1e-3) / 1e9))
+        for d in (ta_, tb_, tc_):
+            d.free()
         del Ar, Br
 
     # ---- batched MLP forward through the exact tier: configuration 5 ---------------------------
