@@ -758,12 +758,14 @@ int convert_any(const double* in, uint16_t* out, uint64_t batch, uint64_t rows, 
  * The tier on such a product spends its time on the second operand: read once as fp64 to
  * narrow it, written as 16 bits, read again by a contraction that has a handful of tiles
  * (32 x 4096 x 4096: 92 us, of which the operand read once is 27). Here it is read once:
- * a workgroup takes a strip of 128 columns and a slice of k, its four waves deal the
- * slice out sixteen k at a time; a lane loads four consecutive columns of eight rows of k
- * (the 32 lanes of a half-wave 1 KiB of each row), narrows them in registers and has, for
- * each of its four columns, the eight consecutive k of one matrix-core operand: four
- * instructions per block of 32 rows, column j of instruction c being column 4 j + c of
- * the strip. The first operand is narrowed beforehand (it is small) and its fragments come
+ * a workgroup takes a strip of 32 CW columns and a slice of k, its four waves deal the
+ * slice out sixteen k at a time; a lane loads CW consecutive columns of eight rows of k
+ * (the 32 lanes of a half-wave 256 CW contiguous bytes of each row), narrows them in
+ * registers and has, for each of its columns, the eight consecutive k of one matrix-core
+ * operand: CW instructions per block of 32 rows, column j of instruction c being column
+ * CW j + c of the strip. CW = 2: strips of 64 columns measured faster than of 128 at every
+ * row count (32 rows: 38 -> 31 us, 64 rows: 48 -> 36), and leave registers for the sums of
+ * 128 rows. The first operand is narrowed beforehand (it is small) and its fragments come
  * from L2. Same arithmetic as the tier's other kernels (16-bit operands, fp32 sums); the
  * sums of the four waves meet in LDS, slices of k leave fp32 partial results that a second
  * kernel adds in ascending order, rounds if asked and stores. */
@@ -776,7 +778,7 @@ __device__ __forceinline__ void store_reduced(void* Cout, int out_mode, size_t i
     else ((double*)Cout)[idx] = (double)x;
 }
 
-template <bool BF16, int RB>
+template <bool BF16, int RB, int CW>
 __global__ __launch_bounds__(256)
 void reduced_thin_kernel(const uint16_t* __restrict__ A16, int lda, int M,
                          const double* __restrict__ B, int K, int N, int kc,
@@ -784,29 +786,31 @@ void reduced_thin_kernel(const uint16_t* __restrict__ A16, int lda, int M,
     __shared__ v4f_t red[4][4][64];
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 31, lh = lane >> 5;
-    const int n0 = (int)blockIdx.x * 128, col = n0 + 4 * li;
+    typedef double dcu_t __attribute__((ext_vector_type(CW), aligned(8)));
+    const int n0 = (int)blockIdx.x * (32 * CW), col = n0 + CW * li;
     const int ks = (int)blockIdx.y * kc;
     const int ke = (ks + kc < K) ? ks + kc : K;
-    const bool edge = n0 + 128 > N;                              /* the same for the whole workgroup */
-    int oc[4];
+    const bool edge = n0 + 32 * CW > N;                              /* the same for the whole workgroup */
+    int oc[CW];
 #pragma unroll
-    for (int c = 0; c < 4; c++) oc[c] = (col + c < N) ? col + c : N - 1;
-    v16f_t acc[RB][4];
+    for (int c = 0; c < CW; c++) oc[c] = (col + c < N) ? col + c : N - 1;
+    v16f_t acc[RB][CW];
 #pragma unroll
     for (int rb = 0; rb < RB; rb++)
 #pragma unroll
-        for (int c = 0; c < 4; c++)
+        for (int c = 0; c < CW; c++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[rb][c][r] = 0.0f;
 
     for (int k0 = ks + 16 * wave; k0 < ke; k0 += 64) {
         const int kk = k0 + 8 * lh;
-        double v[8][4];
+        double v[8][CW];
         if (k0 + 16 <= ke && !edge) {                           /* the same for the whole wave */
 #pragma unroll
             for (int j = 0; j < 8; j++) {
-                const d4u_t x = *(const d4u_t*)(B + (size_t)(kk + j) * N + col);
-                v[j][0] = x[0]; v[j][1] = x[1]; v[j][2] = x[2]; v[j][3] = x[3];
+                const dcu_t x = *(const dcu_t*)(B + (size_t)(kk + j) * N + col);
+#pragma unroll
+                for (int c = 0; c < CW; c++) v[j][c] = x[c];
             }
         } else {
             /* the last, partial round of the slice and the last strip: clamped addresses,
@@ -816,27 +820,27 @@ void reduced_thin_kernel(const uint16_t* __restrict__ A16, int lda, int M,
                 const bool in = kk + j < ke;
                 const size_t kr = (size_t)(in ? kk + j : ke - 1);
 #pragma unroll
-                for (int c = 0; c < 4; c++) { const double x = B[kr * N + oc[c]]; v[j][c] = in ? x : 0.0; }
+                for (int c = 0; c < CW; c++) { const double x = B[kr * N + oc[c]]; v[j][c] = in ? x : 0.0; }
             }
         }
-        v4i_t op[4];
+        v4i_t op[CW];
 #pragma unroll
-        for (int c = 0; c < 4; c++)
+        for (int c = 0; c < CW; c++)
 #pragma unroll
             for (int q = 0; q < 4; q++) op[c][q] = (int)narrow_pair<BF16>(v[2 * q][c], v[2 * q + 1][c]);
 #pragma unroll
         for (int rb = 0; rb < RB; rb++) {
             const v4i_t a = *(const v4i_t*)(A16 + (size_t)(rb * 32 + li) * lda + kk);
 #pragma unroll
-            for (int c = 0; c < 4; c++) H16Op<BF16>::mfma(op[c], a, acc[rb][c]);
+            for (int c = 0; c < CW; c++) H16Op<BF16>::mfma(op[c], a, acc[rb][c]);
         }
     }
     /* acc[rb][c]: lane%32 is the output row, registers 4v .. 4v+3 are columns j = 8v + 4 (lane/32) + 0..3
-     * of instruction c, i.e. columns n0 + 4 j + c. One (rb, c) at a time through LDS. */
+     * of instruction c, i.e. columns n0 + CW j + c. One (rb, c) at a time through LDS. */
 #pragma unroll
     for (int rb = 0; rb < RB; rb++) {
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
+        for (int c = 0; c < CW; c++) {
             if (rb + c) __syncthreads();
 #pragma unroll
             for (int vv = 0; vv < 4; vv++)
@@ -849,7 +853,7 @@ void reduced_thin_kernel(const uint16_t* __restrict__ A16, int lda, int M,
             for (int w = 1; w < 4; w++) s += red[w][wave][lane];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                const int cx = n0 + 4 * (8 * wave + 4 * lh + e) + c;
+                const int cx = n0 + CW * (8 * wave + 4 * lh + e) + c;
                 if (cx >= N) continue;
                 if (part) part[(size_t)blockIdx.y * slice_stride + (size_t)row * N + cx] = s[e];
                 else store_reduced<BF16>(Cout, out_mode, (size_t)((long)row * c_r + (long)cx * c_o), s[e]);
@@ -861,8 +865,8 @@ void reduced_thin_kernel(const uint16_t* __restrict__ A16, int lda, int M,
 /* The same against a big operand with k contiguous, G[O][K] (the second operand held
  * transposed, or a matrix against a few columns): a lane loads eight consecutive k of one
  * output's row (64 bytes; the two halves of a wave the sixteen k of a round) and narrows
- * them into one matrix-core operand; a workgroup's strip is four blocks of 32 outputs. */
-template <bool BF16, int RB>
+ * them into one matrix-core operand; a workgroup's strip is NB blocks of 32 outputs. */
+template <bool BF16, int RB, int NB>
 __global__ __launch_bounds__(256)
 void reduced_thin_klast_kernel(const uint16_t* __restrict__ T16, int ldt, int R,
                                const double* __restrict__ G, int K, int O, int kc,
@@ -870,36 +874,36 @@ void reduced_thin_klast_kernel(const uint16_t* __restrict__ T16, int ldt, int R,
     __shared__ v4f_t red[4][4][64];
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane & 31, lh = lane >> 5;
-    const int o0 = (int)blockIdx.x * 128;
+    const int o0 = (int)blockIdx.x * (32 * NB);
     const int ks = (int)blockIdx.y * kc;
     const int ke = (ks + kc < K) ? ks + kc : K;
-    size_t g_off[4];
+    size_t g_off[NB];
 #pragma unroll
-    for (int cb = 0; cb < 4; cb++) {
+    for (int cb = 0; cb < NB; cb++) {
         const int o = o0 + 32 * cb + li;
         g_off[cb] = (size_t)(o < O ? o : O - 1) * K;            /* rows beyond the operand repeat the last: never stored */
     }
-    v16f_t acc[RB][4];
+    v16f_t acc[RB][NB];
 #pragma unroll
     for (int rb = 0; rb < RB; rb++)
 #pragma unroll
-        for (int cb = 0; cb < 4; cb++)
+        for (int cb = 0; cb < NB; cb++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[rb][cb][r] = 0.0f;
 
     for (int k0 = ks + 16 * wave; k0 < ke; k0 += 64) {
         const int kk = k0 + 8 * lh;
-        v4i_t op[4];
+        v4i_t op[NB];
         if (k0 + 16 <= ke) {                                    /* the same for the whole wave */
 #pragma unroll
-            for (int cb = 0; cb < 4; cb++) {
+            for (int cb = 0; cb < NB; cb++) {
                 const d4u_t x0 = *(const d4u_t*)(G + g_off[cb] + kk), x1 = *(const d4u_t*)(G + g_off[cb] + kk + 4);
                 op[cb] = (v4i_t){(int)narrow_pair<BF16>(x0[0], x0[1]), (int)narrow_pair<BF16>(x0[2], x0[3]),
                                  (int)narrow_pair<BF16>(x1[0], x1[1]), (int)narrow_pair<BF16>(x1[2], x1[3])};
             }
         } else {
 #pragma unroll
-            for (int cb = 0; cb < 4; cb++) {
+            for (int cb = 0; cb < NB; cb++) {
                 double x[8];
 #pragma unroll
                 for (int j = 0; j < 8; j++) {
@@ -915,14 +919,14 @@ void reduced_thin_klast_kernel(const uint16_t* __restrict__ T16, int ldt, int R,
         for (int rb = 0; rb < RB; rb++) {
             const v4i_t a = *(const v4i_t*)(T16 + (size_t)(rb * 32 + li) * ldt + kk);
 #pragma unroll
-            for (int cb = 0; cb < 4; cb++) H16Op<BF16>::mfma(op[cb], a, acc[rb][cb]);
+            for (int cb = 0; cb < NB; cb++) H16Op<BF16>::mfma(op[cb], a, acc[rb][cb]);
         }
     }
     /* acc[rb][cb]: lane%32 is the thin row, registers 4v .. 4v+3 are outputs o0 + 32 cb + 8v + 4 (lane/32) + 0..3 */
 #pragma unroll
     for (int rb = 0; rb < RB; rb++) {
 #pragma unroll
-        for (int cb = 0; cb < 4; cb++) {
+        for (int cb = 0; cb < NB; cb++) {
             if (rb + cb) __syncthreads();
 #pragma unroll
             for (int vv = 0; vv < 4; vv++)
@@ -972,7 +976,8 @@ int g_reduced_thin = 1;
  * thin side, O: outputs on the wide one. */
 struct ThinPlan { int slices, kc; size_t part_bytes; };
 ThinPlan reduced_thin_plan(uint64_t R, uint64_t K, uint64_t O) {
-    const int strips = (int)((O + 127) / 128);
+    const int width = 64;           /* outputs per strip */
+    const int strips = (int)((O + width - 1) / width);
     const int min_kc = strips <= 4 ? 128 : 256;
     int slices = (3 * eshkol_hip_num_cus()) / strips;
     if (slices > (int)(K / min_kc)) slices = (int)(K / min_kc);
@@ -984,18 +989,18 @@ ThinPlan reduced_thin_plan(uint64_t R, uint64_t K, uint64_t O) {
     return { slices, kc, slices > 1 ? (size_t)slices * R * O * sizeof(float) : 0 };
 }
 
-/* up to 64 rows (or columns) against a big operand that is worth streaming, every operand
+/* up to 128 rows (or columns) against a big operand that is worth streaming, every operand
  * form; everything else keeps the narrowing kernels and the tiled contraction */
 bool reduced_is_thin(uint64_t batch, uint64_t M, uint64_t K, uint64_t N) {
     const uint64_t thin = M <= N ? M : N, wide = M <= N ? N : M;
-    return g_reduced_thin && batch == 1 && thin <= 64 && wide >= 128 && K >= 64 && wide * K >= (1ull << 21) &&
+    return g_reduced_thin && batch == 1 && thin <= 128 && wide >= 128 && K >= 64 && wide * K >= (1ull << 21) &&
            K <= 0x3fffff00ULL && wide <= 0x7fffff00ULL;
 }
 ThinPlan reduced_thin_plan_for(uint64_t M, uint64_t K, uint64_t N) {
     return M <= N ? reduced_thin_plan(M, K, N) : reduced_thin_plan(N, K, M);
 }
 
-/* T16: 64 rows of ld elements for the thin operand's 16-bit copy, written here; part:
+/* T16: 128 rows of ld elements for the thin operand's 16-bit copy, written here; part:
  * reduced_thin_plan_for().part_bytes. */
 int reduced_thin(const double* A, const double* B, double* C, uint64_t M, uint64_t K, uint64_t N, int trans_a, int trans_b,
                  int is_bf16, int round_output, uint16_t* T16, uint64_t ld, float* part, hipStream_t st) {
@@ -1005,24 +1010,23 @@ int reduced_thin(const double* A, const double* B, double* C, uint64_t M, uint64
      * (k-major as the runtime stores B, rows of k when the caller holds B^T) */
     const double* T = thin_m ? A : B;
     const bool t_kmajor = thin_m ? trans_a != 0 : trans_b == 0;
-    if (convert_any(T, T16, 1, R, K, 64, ld, is_bf16, t_kmajor, 0, st) != 0) return -1;
+    if (convert_any(T, T16, 1, R, K, 128, ld, is_bf16, t_kmajor, 0, st) != 0) return -1;
     const double* G = thin_m ? B : A;
     const bool kfirst = thin_m ? trans_b == 0 : trans_a != 0;    /* the big operand has the output index contiguous */
     const long c_r = thin_m ? (long)N : 1, c_o = thin_m ? 1 : (long)N;
     const ThinPlan pl = reduced_thin_plan(R, K, O);
-    const dim3 grid((unsigned)((O + 127) / 128), (unsigned)pl.slices);
+    const int width = 64;
+    const dim3 grid((unsigned)((O + width - 1) / width), (unsigned)pl.slices);
     const int out_mode = round_output ? 2 : 1;
     float* p = pl.slices > 1 ? part : nullptr;
     const long stride = (long)(R * O);
-#define THIN(KERN, BF, RB) hipLaunchKernelGGL((KERN<BF, RB>), grid, dim3(256), 0, st, T16, (int)ld, (int)R, G, (int)K, \
-                                              (int)O, pl.kc, p, stride, (void*)C, out_mode, c_r, c_o)
-    if (kfirst) {
-        if (is_bf16) { if (R <= 32) THIN(reduced_thin_kernel, true, 1); else THIN(reduced_thin_kernel, true, 2); }
-        else         { if (R <= 32) THIN(reduced_thin_kernel, false, 1); else THIN(reduced_thin_kernel, false, 2); }
-    } else {
-        if (is_bf16) { if (R <= 32) THIN(reduced_thin_klast_kernel, true, 1); else THIN(reduced_thin_klast_kernel, true, 2); }
-        else         { if (R <= 32) THIN(reduced_thin_klast_kernel, false, 1); else THIN(reduced_thin_klast_kernel, false, 2); }
-    }
+#define THIN(KERN, BF, RB, W) hipLaunchKernelGGL((KERN<BF, RB, W>), grid, dim3(256), 0, st, T16, (int)ld, (int)R, G, (int)K, \
+                                                 (int)O, pl.kc, p, stride, (void*)C, out_mode, c_r, c_o)
+#define THIN_BY_ROWS(KERN, BF) do { if (R <= 32) THIN(KERN, BF, 1, 2); else if (R <= 64) THIN(KERN, BF, 2, 2); \
+                                    else if (R <= 96) THIN(KERN, BF, 3, 2); else THIN(KERN, BF, 4, 2); } while (0)
+    if (kfirst) { if (is_bf16) THIN_BY_ROWS(reduced_thin_kernel, true); else THIN_BY_ROWS(reduced_thin_kernel, false); }
+    else        { if (is_bf16) THIN_BY_ROWS(reduced_thin_klast_kernel, true); else THIN_BY_ROWS(reduced_thin_klast_kernel, false); }
+#undef THIN_BY_ROWS
 #undef THIN
     if (p) {
         const long n = (long)(R * O);
@@ -1114,7 +1118,7 @@ extern "C" int hip_matmul_reduced_f64_batched_ex(const double* A, const double* 
     if (reduced_is_thin(batch, M, K, N)) {
         /* a few rows or columns: the big operand is read once, as fp64, and never copied */
         const ThinPlan pl = reduced_thin_plan_for(M, K, N);
-        uint16_t* A16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_A, 64 * sh.ld * 2);
+        uint16_t* A16 = (uint16_t*)eshkol_hip_workspace(WS_HALF_A, 128 * sh.ld * 2);
         float* part = pl.part_bytes ? (float*)eshkol_hip_workspace(WS_DGEMM_PARTIAL, pl.part_bytes) : nullptr;
         if (A16 && (part || !pl.part_bytes))
             return reduced_thin(A, B, C, M, K, N, trans_a, trans_b, dtype == 3, round_output, A16, sh.ld, part, st);
@@ -1205,10 +1209,10 @@ extern "C" int hip_matmul_reduced_f64_noalloc(const double* A, const double* B, 
     unsigned char* base = noalloc_scratch();
     if (!base) return -1;
     if (reduced_is_thin(1, M, K, N)) {
-        /* the same kernel and slices as the workspace entry point: the first operand's 64
+        /* the same kernel and slices as the workspace entry point: the thin operand's 128
          * rows of 16-bit values and the fp32 partial sums take the place of the copies */
         const ThinPlan pl = reduced_thin_plan_for(M, K, N);
-        const uint64_t a16 = round_up_sz(64 * sh.ld * 2, 256);
+        const uint64_t a16 = round_up_sz(128 * sh.ld * 2, 256);
         if (a16 + pl.part_bytes > NOALLOC_SCRATCH_BYTES) {
             fprintf(stderr, "[GPU] hip_matmul_reduced_f64_noalloc: %llux%llux%llu needs %llu bytes of partial sums, "
                             "the static scratch holds %llu; use hip_matmul_reduced_f64\n",

@@ -133,7 +133,7 @@ void hip_igemm_set_cu_limit(int cus);
 /* The same switch for the 16-bit tier. */
 void hip_hgemm_set_direct(int on);
 
-/* 1 (default): the reduced tier on up to 64 rows or columns against a big operand reads
+/* 1 (default): the reduced tier on up to 128 rows or columns against a big operand reads
  * that operand once, as fp64, and narrows it in registers on its way to the matrix cores;
  * 0: narrowing kernels and the tiled contraction, as for every other shape. Same
  * arithmetic, another order of the fp32 sums. */

@@ -337,7 +337,7 @@ int hip_matmul_reduced_f64_batched(const double* A, const double* B, double* C,
  * process ends) instead of the grow-only workspace, and the call reaches no
  * hipMalloc, hipFree or allocating library routine. Returns -3 with a message
  * on stderr when 2 * (roundup(M,256) + roundup(N,256)) * roundup(K,256) bytes
- * exceed that limit (for up to 64 rows or columns against an operand of two million
+ * exceed that limit (for up to 128 rows or columns against an operand of two million
  * elements or more, which both entry points multiply without a 16-bit copy of it: also when
  * the fp32 partial sums of that kernel, at most 25 MiB, do not fit beside the
  * first operand's copy), otherwise what hip_matmul_reduced_f64 returns, and the

@@ -41,9 +41,9 @@ def test_reduced_matches_reference_statement(gpu, M, K, N, dtype):
 
 @pytest.mark.parametrize("dtype", [2, 3])
 @pytest.mark.parametrize("M,K,N", [(1, 8192, 256), (5, 7000, 300), (32, 4096, 1024), (33, 2049, 1030), (64, 520, 4099),
-                                   (17, 512, 4100), (40, 16400, 130)])
+                                   (17, 512, 4100), (40, 16400, 130), (100, 4096, 1024), (128, 1031, 2050)])
 def test_a_few_rows_against_a_big_second_operand(gpu, M, K, N, dtype):
-    """Up to 64 rows against B as the runtime stores it: B is read once as fp64 and narrowed in registers on
+    """Up to 128 rows against B as the runtime stores it: B is read once as fp64 and narrowed in registers on
     its way to the matrix cores. Same arithmetic as the tier's other kernels (16-bit operands, fp32 sums), so:
     the reference statement within the fp32 bar, the rounded output the unrounded one rounded, the tiled path
     within the scatter of fp32 summation orders, an infinity in B in its own column only, the entry point that
@@ -84,7 +84,8 @@ def test_a_few_rows_against_a_big_second_operand(gpu, M, K, N, dtype):
 
 
 @pytest.mark.parametrize("dtype", [2, 3])
-@pytest.mark.parametrize("thin,K,wide", [(1, 8192, 300), (7, 2049, 1030), (33, 4100, 520), (64, 515, 4099)])
+@pytest.mark.parametrize("thin,K,wide", [(1, 8192, 300), (7, 2049, 1030), (33, 4100, 520), (64, 515, 4099), (65, 2049, 1030),
+                                         (96, 4100, 520), (128, 515, 4099)])
 def test_a_few_rows_or_columns_in_every_operand_form(gpu, thin, K, wide, dtype):
     """The thin side may be M or N, and either operand may be held transposed: two kernels (the big operand
     with the output index contiguous, or with k contiguous) serve all of them. Against the reference statement
