@@ -118,6 +118,39 @@ def test_a_few_rows_or_columns_in_every_operand_form(gpu, thin, K, wide, dtype):
             assert np.array_equal(narrow[ok], oracle.reduce_precision(outs[0], dtype)[ok])
 
 
+def test_random_shapes_with_a_thin_side_take_whichever_kernel_and_agree(gpu):
+    """Sixty random shapes with one side of at most 140 and a random operand form: whichever kernel the tier picks
+    (the ones that read the big operand once, or narrowing and tiles), the result is the reference statement's within
+    the fp32 bar. Small integers that are 16-bit values make the sums exact in fp32 whatever their order: those
+    must come out bit for bit."""
+    lib = ea.load()
+    rng = np.random.default_rng(77)
+    for it in range(60):
+        thin = int(rng.integers(1, 141))
+        wide = int(2 ** rng.uniform(7, 12.3))
+        K = int(2 ** rng.uniform(6, 13))
+        M, N = (thin, wide) if rng.integers(0, 2) else (wide, thin)
+        ta, tb = [(0, 0), (0, 0), (0, 1), (1, 0)][int(rng.integers(0, 4))]
+        dtype = 2 + int(rng.integers(0, 2))
+        print("reduced, random", M, K, N, ta, tb, dtype, flush=True)
+        A = rng.integers(-3, 4, (M, K)).astype(np.float64)
+        B = rng.integers(-3, 4, (K, N)).astype(np.float64)
+        X = np.ascontiguousarray(A.T) if ta else A
+        Y = np.ascontiguousarray(B.T) if tb else B
+        dX, dY, dC = ea.DeviceArray.from_host(X), ea.DeviceArray.from_host(Y), ea.DeviceArray((M, N))
+        assert lib.hip_matmul_reduced_f64_ex(dX.ptr, dY.ptr, dC.ptr, M, K, N, ta, tb, dtype, 0, stream()) == 0
+        ea.synchronize()
+        assert np.array_equal(dC.download(), A @ B), (M, K, N, ta, tb, dtype)
+        A = oracle.reduce_precision(rng.standard_normal((M, K)) / np.sqrt(K), dtype)
+        B = oracle.reduce_precision(rng.standard_normal((K, N)) / np.sqrt(K), dtype)
+        X = np.ascontiguousarray(A.T) if ta else A
+        Y = np.ascontiguousarray(B.T) if tb else B
+        dX, dY = ea.DeviceArray.from_host(X), ea.DeviceArray.from_host(Y)
+        assert lib.hip_matmul_reduced_f64_ex(dX.ptr, dY.ptr, dC.ptr, M, K, N, ta, tb, dtype, 0, stream()) == 0
+        ea.synchronize()
+        assert normwise(dC.download(), A @ B, A, B) <= 1e-6, (M, K, N, ta, tb, dtype)
+
+
 @pytest.mark.parametrize("dtype", [2, 3])
 @pytest.mark.parametrize("M,K,N", [(3072, 256, 3072), (3000, 200, 2900), (3001, 200, 2901), (3072, 256, 3073)])
 def test_rounded_output_of_the_kernel_for_large_products(gpu, M, K, N, dtype):
