@@ -286,6 +286,22 @@ def test_few_rows_in_front_of_prepared_planes(gpu, M, K, N):
         lib.hip_ozaki_crt_release_prepared(h)
 
 
+def test_random_shapes_with_a_few_rows_match_the_oracle(gpu):
+    """Thirty random products with up to 170 rows: whichever contraction kernel the row count and the width pick
+    (the two for a few rows, or tiles), residue products and results are the oracle's."""
+    rng = np.random.default_rng(2024)
+    done = 0
+    while done < 30:
+        M = int(rng.integers(1, 171)); K = int(2 ** rng.uniform(6, 11.5)); N = int(2 ** rng.uniform(4, 12.3))
+        if M * K * N > 1.5e8:
+            continue
+        done += 1
+        print("crt, random", M, K, N, flush=True)
+        A = synth.wide_range(1000 + done, (M, K))
+        B = synth.wide_range(2000 + done, (K, N))
+        check_all_stages(A, B)
+
+
 def test_aligned_weight_split_matches_the_oracle_and_is_accurate(gpu):
     """hip_ozaki_crt_set_aligned_weights(1): the CRT weights split at a common bit.
     Residues and products are those of the default mode, the result equals the
