@@ -55,6 +55,21 @@ def test_wide_range_inputs_all_stages(gpu, M, K, N):
     check_all_stages(A, B)
 
 
+def test_random_shapes_with_a_few_rows_all_stages(gpu):
+    """Twenty random products with up to 170 rows: whichever contraction kernel the shape picks, every stage is the
+    oracle's."""
+    rng = np.random.default_rng(31)
+    done = 0
+    while done < 20:
+        M = int(rng.integers(1, 171)); K = int(2 ** rng.uniform(6, 11.5)); N = int(2 ** rng.uniform(4, 12.3))
+        if M * K * N > 1.0e8:
+            continue
+        done += 1
+        print("fast, random", M, K, N, flush=True)
+        check_all_stages(synth.wide_range(3000 + done, (M, K)), synth.wide_range(4000 + done, (K, N)),
+                         n_mod=int(rng.integers(2, 17)))
+
+
 @pytest.mark.parametrize("n", [2, 5, 8, 11, 16])
 def test_moduli_counts(gpu, n):
     A, B = synth.normal(13, (96, 160)), synth.normal(14, (160, 80))

@@ -36,6 +36,21 @@ def test_all_stages(gpu, M, K, N, T):
     check_all_stages(A, B, T)
 
 
+def test_random_shapes_with_a_few_rows_all_stages(gpu):
+    """Twenty random products with up to 170 rows and a random slice count: whichever contraction kernel the shape
+    picks (its plans sum several products per output plane), every stage is the oracle's."""
+    rng = np.random.default_rng(32)
+    done = 0
+    while done < 20:
+        M = int(rng.integers(1, 171)); K = int(2 ** rng.uniform(6, 11.5)); N = int(2 ** rng.uniform(4, 12.3))
+        if M * K * N > 1.0e8:
+            continue
+        done += 1
+        T = int(rng.integers(1, 9))
+        print("int8, random", M, K, N, T, flush=True)
+        check_all_stages(synth.normal(5000 + done, (M, K)), synth.normal(6000 + done, (K, N)), T)
+
+
 def test_wide_range_and_zero_rows(gpu):
     A = synth.wide_range(1, (80, 120), -12, 12); B = synth.wide_range(2, (120, 60), -12, 12)
     A[4, :] = 0.0; B[:, 11] = 0.0
