@@ -688,9 +688,12 @@ int launch(const uint16_t* A, const uint16_t* Bt, int M, int N, int ld_bytes, in
 
 /* batch products stored back to back: A [batch][rows_a][ld], Bt [batch][rows_b][ld]
  * (rows_a, rows_b the padded row counts), C [batch][M][N]. */
+int hgemm_thin16(const uint16_t* A, const uint16_t* Bt, uint64_t M, uint64_t N, uint64_t ld,
+                 int is_bf16, int out_mode, void* C, hipStream_t st);
+
 int hgemm_any(const uint16_t* A, const uint16_t* Bt, uint64_t batch, uint64_t M, uint64_t K, uint64_t N,
               uint64_t rows_a, uint64_t rows_b, uint64_t ld,
-              int is_bf16, int layout, int out_mode, void* C, hipStream_t st) {
+              int is_bf16, int layout, int out_mode, void* C, hipStream_t st, bool may_use_workspace = false) {
     if (!A || !Bt || !C || M == 0 || K == 0 || N == 0 || batch == 0) return -1;
     if (M > 0x7fffffffULL || N > 0x7fffffffULL || batch > 0x7fffffffULL) return -1;
     if (ld < K || ld % 64 != 0 || ld * 2 > 0x7fffffffULL) return -1;
@@ -705,6 +708,11 @@ int hgemm_any(const uint16_t* A, const uint16_t* Bt, uint64_t batch, uint64_t M,
                        : launch_direct<false>(A, Bt, m, n, ldb, out_mode, C, nb, a_stride, b_stride, st);
     }
     if (layout != 0) return -1;
+    /* up to 128 rows against a big second operand: stream it once (callers that may use the
+     * library workspace, i.e. the entry points for 16-bit operands; the f64 pipelines have
+     * the kernels that read fp64 directly) */
+    if (may_use_workspace && batch == 1 && M <= 128 && N >= 128 && N * ld >= (1ull << 21) &&
+        hgemm_thin16(A, Bt, M, N, ld, is_bf16, out_mode, C, st) == 0) return 0;
     const long long big = (long long)((M + 255) / 256) * ((N + 255) / 256);
     /* the pipelined kernel wants whole pairs of 128-byte k-blocks and more than two per tile */
     if (batch == 1 && big >= 128 && ldb % 256 == 0 && ldb >= 512)
@@ -866,10 +874,12 @@ void reduced_thin_kernel(const uint16_t* __restrict__ A16, int lda, int M,
  * transposed, or a matrix against a few columns): a lane loads eight consecutive k of one
  * output's row (64 bytes; the two halves of a wave the sixteen k of a round) and narrows
  * them into one matrix-core operand; a workgroup's strip is NB blocks of 32 outputs. */
-template <bool BF16, int RB, int NB>
+/* G16: the big operand is 16-bit already (rows of ldg elements, zero padded in k and in rows,
+ * as hip_hgemm_16 takes its operands): loaded as it is, K counts the padded k. */
+template <bool BF16, int RB, int NB, bool G16 = false>
 __global__ __launch_bounds__(256)
 void reduced_thin_klast_kernel(const uint16_t* __restrict__ T16, int ldt, int R,
-                               const double* __restrict__ G, int K, int O, int kc,
+                               const void* __restrict__ Gv, int K, int O, int kc,
                                float* __restrict__ part, long slice_stride, void* Cout, int out_mode, long c_r, long c_o) {
     __shared__ v4f_t red[4][4][64];
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -883,6 +893,8 @@ void reduced_thin_klast_kernel(const uint16_t* __restrict__ T16, int ldt, int R,
         const int o = o0 + 32 * cb + li;
         g_off[cb] = (size_t)(o < O ? o : O - 1) * K;            /* rows beyond the operand repeat the last: never stored */
     }
+    const double* G = (const double*)Gv;
+    const uint16_t* Gh = (const uint16_t*)Gv;
     v16f_t acc[RB][NB];
 #pragma unroll
     for (int rb = 0; rb < RB; rb++)
@@ -894,7 +906,10 @@ void reduced_thin_klast_kernel(const uint16_t* __restrict__ T16, int ldt, int R,
     for (int k0 = ks + 16 * wave; k0 < ke; k0 += 64) {
         const int kk = k0 + 8 * lh;
         v4i_t op[NB];
-        if (k0 + 16 <= ke) {                                    /* the same for the whole wave */
+        if (G16) {
+#pragma unroll
+            for (int cb = 0; cb < NB; cb++) op[cb] = *(const v4i_t*)(Gh + g_off[cb] + kk);
+        } else if (k0 + 16 <= ke) {                             /* the same for the whole wave */
 #pragma unroll
             for (int cb = 0; cb < NB; cb++) {
                 const d4u_t x0 = *(const d4u_t*)(G + g_off[cb] + kk), x1 = *(const d4u_t*)(G + g_off[cb] + kk + 4);
@@ -1037,6 +1052,34 @@ int reduced_thin(const double* A, const double* B, double* C, uint64_t M, uint64
     return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
 }
 
+/* hip_hgemm_16 on up to 128 rows: A [rows padded][ld] and Bt [rows padded][ld] 16-bit, zero
+ * padded; the big operand streamed once by the kernel for k-contiguous operands. */
+int hgemm_thin16(const uint16_t* A, const uint16_t* Bt, uint64_t M, uint64_t N, uint64_t ld,
+                 int is_bf16, int out_mode, void* C, hipStream_t st) {
+    if (!g_reduced_thin) return -1;
+    const ThinPlan pl = reduced_thin_plan(M, ld, N);
+    float* p = nullptr;
+    if (pl.slices > 1) {
+        p = (float*)eshkol_hip_workspace(WS_DGEMM_PARTIAL, pl.part_bytes);
+        if (!p) return -1;
+    }
+    const dim3 grid((unsigned)((N + 63) / 64), (unsigned)pl.slices);
+    const long stride = (long)(M * N), c_r = (long)N, c_o = 1;
+#define THIN16(BF, RB) hipLaunchKernelGGL((reduced_thin_klast_kernel<BF, RB, 2, true>), grid, dim3(256), 0, st, A, (int)ld, (int)M, \
+                                          (const void*)Bt, (int)ld, (int)N, pl.kc, p, stride, C, out_mode, c_r, c_o)
+#define THIN16_BY_ROWS(BF) do { if (M <= 32) THIN16(BF, 1); else if (M <= 64) THIN16(BF, 2); else if (M <= 96) THIN16(BF, 3); else THIN16(BF, 4); } while (0)
+    if (is_bf16) THIN16_BY_ROWS(true); else THIN16_BY_ROWS(false);
+#undef THIN16_BY_ROWS
+#undef THIN16
+    if (p) {
+        const long n = (long)(M * N);
+        const dim3 sgrid((unsigned)((n + 255) / 256));
+        if (is_bf16) hipLaunchKernelGGL(reduced_thin_sum_kernel<true>, sgrid, dim3(256), 0, st, p, pl.slices, n, (int)N, C, out_mode, c_r, c_o);
+        else         hipLaunchKernelGGL(reduced_thin_sum_kernel<false>, sgrid, dim3(256), 0, st, p, pl.slices, n, (int)N, C, out_mode, c_r, c_o);
+    }
+    return ESHKOL_HIP_OK(hipGetLastError()) ? 0 : -1;
+}
+
 /* Padded operand shape and plane layout of the reduced tier for a batch of
  * M x K x N products: interleaved 16-bit operands (and a k pitch of whole
  * 512-byte groups) when the launch has enough 256 x 256 tiles for the
@@ -1094,7 +1137,7 @@ extern "C" int hip_convert_f64_to_16_planes(const double* in, uint16_t* out, uin
 extern "C" int hip_hgemm_16(const uint16_t* A, const uint16_t* Bt, uint64_t M, uint64_t K, uint64_t N,
                             uint64_t ld, int is_bf16, float* C, void* stream) {
     EshkolHipCall bracket(stream);
-    return hgemm_any(A, Bt, 1, M, K, N, round_up_sz(M, 256), round_up_sz(N, 256), ld, is_bf16, 0, 0, C, (hipStream_t)stream);
+    return hgemm_any(A, Bt, 1, M, K, N, round_up_sz(M, 256), round_up_sz(N, 256), ld, is_bf16, 0, 0, C, (hipStream_t)stream, true);
 }
 
 extern "C" int hip_hgemm_16_batched(const uint16_t* A, const uint16_t* Bt, uint64_t batch,
@@ -1102,7 +1145,7 @@ extern "C" int hip_hgemm_16_batched(const uint16_t* A, const uint16_t* Bt, uint6
                                     uint64_t rows_a_padded, uint64_t rows_b_padded, uint64_t ld,
                                     int is_bf16, int layout, float* C, void* stream) {
     EshkolHipCall bracket(stream);
-    return hgemm_any(A, Bt, batch, M, K, N, rows_a_padded, rows_b_padded, ld, is_bf16, layout, 0, C, (hipStream_t)stream);
+    return hgemm_any(A, Bt, batch, M, K, N, rows_a_padded, rows_b_padded, ld, is_bf16, layout, 0, C, (hipStream_t)stream, true);
 }
 
 extern "C" int hip_matmul_reduced_f64_batched_ex(const double* A, const double* B, double* C,

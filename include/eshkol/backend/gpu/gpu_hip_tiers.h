@@ -350,7 +350,10 @@ size_t hip_matmul_reduced_f64_noalloc_limit(void);
 
 /* 16-bit operands already in device memory (A [M][K], Bt [N][K], pitch ld
  * elements, multiple of 64, rows padded to multiples of 256 with zeros), fp32
- * result C[M][N]: the contraction alone (BASELINE configuration 4). */
+ * result C[M][N]: the contraction alone (BASELINE configuration 4). Up to 128
+ * rows against a second operand of two million elements or more read that
+ * operand once, in slices of k whose fp32 partial sums (in the library's
+ * workspace) a second kernel adds in ascending order. */
 int hip_hgemm_16(const uint16_t* A, const uint16_t* Bt, uint64_t M, uint64_t K, uint64_t N,
                  uint64_t ld, int is_bf16, float* C, void* stream);
 

@@ -218,6 +218,47 @@ def test_hgemm_fp32_output_config4_reduced_size(gpu):
     assert normwise(Cg, oracle.matmul_f64(Ar, Br), Ar, Br) <= 1e-6
 
 
+@pytest.mark.parametrize("is_bf16", [0, 1])
+@pytest.mark.parametrize("M,K,N", [(1, 8192, 256), (7, 2050, 1030), (32, 4096, 4096), (33, 1000, 2100), (100, 520, 4099),
+                                   (128, 4096, 1024)])
+def test_a_few_rows_of_16_bit_operands_stream_the_second_operand(gpu, M, K, N, is_bf16):
+    """hip_hgemm_16 on up to 128 rows against a big second operand reads that operand once
+    instead of tiling it: against the oracle on the narrowed operands, and, on small
+    integers (exact in fp32 whatever the order of the sums), equal to the tiled kernel."""
+    print("hgemm16 thin", M, K, N, is_bf16, flush=True)
+    lib = ea.load()
+    dtype = 3 if is_bf16 else 2
+    rp = lambda r: -(-r // 256) * 256
+    ld = -(-K // 64) * 64
+
+    def run(A, Bt):
+        dA, dBt = ea.DeviceArray.from_host(A), ea.DeviceArray.from_host(Bt)
+        a16 = ea.DeviceArray.from_host(np.full((rp(M), ld), 0x7777, np.uint16))
+        b16 = ea.DeviceArray.from_host(np.full((rp(N), ld), 0x7777, np.uint16))
+        assert lib.hip_convert_f64_to_16(dA.ptr, a16.ptr, M, K, rp(M), ld, is_bf16, stream()) == 0
+        assert lib.hip_convert_f64_to_16(dBt.ptr, b16.ptr, N, K, rp(N), ld, is_bf16, stream()) == 0
+        dC = ea.DeviceArray.from_host(np.full((M, N), np.nan, np.float32))
+        assert lib.hip_hgemm_16(a16.ptr, b16.ptr, M, K, N, ld, is_bf16, dC.ptr, stream()) == 0
+        ea.synchronize()
+        return dC.download().astype(np.float64)
+
+    A = synth.normal(70 + M, (M, K), 1.0 / np.sqrt(K)); Bt = synth.normal(71 + N, (N, K), 1.0 / np.sqrt(K))
+    if is_bf16:
+        Ar, Br = oracle.reduce_precision(A, dtype), oracle.reduce_precision(Bt, dtype).T
+    else:       # IEEE narrowing, subnormals included (the device's; the reference's f16 narrowing differs below 2^-14)
+        Ar, Br = A.astype(np.float16).astype(np.float64), Bt.astype(np.float16).astype(np.float64).T
+    assert normwise(run(A, Bt), oracle.matmul_f64(Ar, Br), Ar, Br) <= 1e-6
+    i = np.arange(M * K, dtype=np.int64).reshape(M, K); j = np.arange(N * K, dtype=np.int64).reshape(N, K)
+    Ai = ((i * 7 + i // K) % 7 - 3).astype(np.float64); Bi = ((j * 5 + j // K) % 5 - 2).astype(np.float64)
+    want = Ai @ Bi.T
+    assert np.array_equal(run(Ai, Bi), want)
+    lib.hip_reduced_set_thin(0)
+    try:
+        assert np.array_equal(run(Ai, Bi), want)
+    finally:
+        lib.hip_reduced_set_thin(1)
+
+
 def test_full_size_config4_sampled(gpu):
     n = 8192
     print("reduced full", n, flush=True)
