@@ -469,11 +469,20 @@ def main():
         ta_ = ea.DeviceArray.from_host(synth.normal(65, (tm, tk), 1.0 / np.sqrt(tk)))
         tb_ = ea.DeviceArray.from_host(synth.normal(66, (tk, tn), 1.0 / np.sqrt(tk)))
         tc_ = ea.DeviceArray((tm, tn))
-        _, wt = timed(lambda: lib.hip_matmul_reduced_f64(ta_.ptr, tb_.ptr, tc_.ptr, tm, tk, tn, 3, 1, st), k=20, w=5)
+        _, wt = timed(lambda: lib.hip_matmul_reduced_f64(ta_.ptr, tb_.ptr, tc_.ptr, tm, tk, tn, 3, 1, st), k=20, w=5, settle_ms=20.0)
         tiers["reduced_bf16_32x4096x4096"] = {"ms": wt, "weights_GBps": 8.0 * tk * tn / (wt * 1e-3) / 1e9,
                                              "frac_of_hbm": 8.0 * tk * tn / (wt * 1e-3) / 8e12}
         log("reduced bf16, 32 rows against 4096 x 4096: %.3f ms (%.0f GB/s of weights)" % (wt, 8.0 * tk * tn / (wt * 1e-3) / 1e9))
-        for d in (ta_, tb_, tc_):
+        # the same with both operands already bf16 and resident (weights narrowed once, held transposed)
+        ta16 = ea.DeviceArray.from_host(np.zeros((256, tk), np.uint16)); tb16 = ea.DeviceArray.from_host(np.zeros((tn, tk), np.uint16))
+        tbt_ = ea.DeviceArray.from_host(np.ascontiguousarray(synth.normal(66, (tk, tn), 1.0 / np.sqrt(tk)).T))
+        assert lib.hip_convert_f64_to_16(ta_.ptr, ta16.ptr, tm, tk, 256, tk, 1, st) == 0
+        assert lib.hip_convert_f64_to_16(tbt_.ptr, tb16.ptr, tn, tk, tn, tk, 1, st) == 0
+        tc32 = ea.DeviceArray((tm, tn), np.float32)
+        _, wt16 = timed(lambda: lib.hip_hgemm_16(ta16.ptr, tb16.ptr, tm, tk, tn, tk, 1, tc32.ptr, st), k=20, w=5, settle_ms=20.0)
+        tiers["reduced_bf16_32x4096x4096"]["bf16_operands_resident_ms"] = wt16
+        log("the same with bf16 operands resident: %.3f ms" % wt16)
+        for d in (ta_, tb_, tc_, ta16, tb16, tbt_, tc32):
             d.free()
         del Ar, Br
 
@@ -569,8 +578,8 @@ def main():
             return 0
         os.dup2(devnull, 2)
         try:
-            _, ws_p = timed(small_prepared, k=20, w=5)
-            _, ws_n = timed(small_native, k=20, w=5)
+            _, ws_p = timed(small_prepared, k=20, w=5, settle_ms=10.0)
+            _, ws_n = timed(small_native, k=20, w=5, settle_ms=10.0)
         finally:
             os.dup2(saved, 2)
         for h in handles:
