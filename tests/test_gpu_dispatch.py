@@ -357,7 +357,8 @@ def test_concurrent_callers_serialise_on_the_library(gpu):
     assert lib.eshkol_gpu_init() == 1
     old = lib.eshkol_gpu_get_threshold()
     lib.eshkol_gpu_set_threshold(1)
-    shapes = [(4100, 2048, 2056), (300, 200, 260), (1024, 1024, 1024), (4096, 2048, 2048), (64, 4096, 96), (700, 50, 900)]
+    shapes = [(4100, 2048, 2056), (300, 200, 260), (1024, 1024, 1024), (4096, 2048, 2048), (64, 4096, 96), (700, 50, 900),
+              (32, 2048, 4096), (1, 8192, 1024), (2048, 4096, 3)]
     ops = [(synth.normal(20 + i, (m, k)), synth.normal(40 + i, (k, n))) for i, (m, k, n) in enumerate(shapes)]
     want = [ea.matmul_dispatch(a, b) for a, b in ops]            # one at a time
     got = [[None] * len(ops) for _ in range(2)]
