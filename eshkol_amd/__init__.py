@@ -157,6 +157,7 @@ SIGNATURES = {
     "hip_convert_f64_to_16_planes": (C.c_int, [vp, vp, u64, u64, u64, u64, u64, C.c_int, C.c_int, C.c_int, vp]),
     "hip_matmul_reduced_f64_batched": (C.c_int, [vp, vp, vp, u64, u64, u64, u64, C.c_int, C.c_int, vp]),
     "hip_igemm_plane_layout": (C.c_int, [u64, u64, C.c_int]),
+    "hip_igemm_plane_layout_single": (C.c_int, [u64, u64, u64, C.c_int]),
     "hip_ozaki_crt_split_planes_f64": (C.c_int, [vp, u64, u64, vp, C.c_int, vp, u64, u64, C.c_int, C.c_int, vp]),
     "hip_ozaki_slice_planes_f64": (C.c_int, [vp, u64, u64, vp, C.c_int, vp, u64, u64, C.c_int, C.c_int, vp]),
     "hip_dgemm_set_tail_split": (None, [C.c_int]),

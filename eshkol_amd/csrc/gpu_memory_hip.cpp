@@ -409,7 +409,7 @@ void resident_release_all(void) {
  * tier declines or the byte cap is reached (then the call prepares nothing and
  * splits B as always, which a verbose run says once per tensor). Row-major planes
  * are made again, interleaved, for the first product that wants interleaved ones (a
- * row count on the other side of hip_igemm_plane_layout): keeping them would mean
+ * row count on the other side of hip_igemm_plane_layout_single): keeping them would mean
  * splitting B on every such call while they sit in device memory unused.
  * Interleaved planes then stay, whatever the row counts that follow. A
  * failed allocation is not remembered; a refusal that depends on the contents
@@ -419,7 +419,7 @@ void* resident_prepared_b(const double* dB, uint64_t M, uint64_t K, uint64_t N, 
     if (!r || r->bytes != K * N * sizeof(double)) return nullptr;
     /* interleaved planes serve every row count; row-major ones only products that want them */
     const bool keep = r->prepared && r->prep_layout == 1 && r->prep_K == K && r->prep_N == N && r->prep_moduli == moduli;
-    const int layout = keep ? 1 : hip_igemm_plane_layout(M, N, moduli);
+    const int layout = keep ? 1 : hip_igemm_plane_layout_single(M, K, N, moduli);
     if (r->prepared && (r->prep_K != K || r->prep_N != N || r->prep_moduli != moduli || r->prep_layout != layout)) {
         if (r->prep_K == K && r->prep_N == N && r->prep_moduli == moduli)
             GPU_LOG("resident operand %p: residue planes are in the %s layout, this product wants the other: "

@@ -729,6 +729,17 @@ extern "C" int hip_igemm_plane_layout(uint64_t M, uint64_t N, int n_out) {
     return (g_direct != 0 && big >= 128) ? 1 : 0;
 }
 
+/* The same for contractions of one product per output plane over K of k (the two CRT
+ * tiers), which the 256 x 128 kernel may take: from sixteen tiles of 256 x 256 and 1024 of
+ * k on, that kernel on interleaved planes is at least as fast as the kernels for row-major
+ * planes (256 x 1024 x 256, sixteen planes: 12.7 us against 13.2; 256 x 4096 x 1024: 38.7
+ * against 47.3; 256 x 16384 x 256: 102 against 152), so such launches are interleaved too. */
+extern "C" int hip_igemm_plane_layout_single(uint64_t M, uint64_t K, uint64_t N, int n_out) {
+    if (hip_igemm_plane_layout(M, N, n_out)) return 1;
+    const uint64_t big = ((M + 255) / 256) * ((N + 255) / 256) * (uint64_t)(n_out > 0 ? n_out : 0);
+    return ((g_direct == 1 || g_direct == 2) && K >= 1024 && big >= 16) ? 1 : 0;
+}
+
 extern "C" int hip_igemm_i8(const HipIgemmArgs* args, void* stream) {
     EshkolHipCall bracket(stream);
     if (!args || !args->a_planes || !args->b_planes || !args->pair_first || !args->pair_a || !args->pair_b)

@@ -1019,7 +1019,7 @@ static int crt_matmul_impl(const double* A, const double* B, double* C,
      * planes serve only the products that would make row-major planes themselves. */
     const bool keep_interleaved = prepared && prepared->layout == 1 && !adaptive && !g_force_host_pass &&
                                   prepared->n_mod == num_moduli && eshkol_hip_igemm_direct_mode() == 1;
-    const int layout = keep_interleaved ? 1 : hip_igemm_plane_layout(M, N, num_moduli);
+    const int layout = keep_interleaved ? 1 : hip_igemm_plane_layout_single(M, K, N, num_moduli);
     /* a first operand of a few rows goes to the kernel that streams the second operand's
      * planes: its own planes then need whole blocks of 32 rows only */
     const bool thin = layout == 1 && eshkol_hip_igemm_is_thin(M, N);
@@ -1236,7 +1236,7 @@ extern "C" int hip_ozaki_crt_prepare_operand_b(const double* B, uint64_t K, uint
     const HostCrt& crt = crt_constants(num_moduli);
     /* only where E does not depend on the operands (gpu_memory.mm:2510-2512) */
     if (!(floor((crt.log2P - 3.0 - log2((double)K)) / 2.0) >= 52.0)) return -1;
-    const int layout = hip_igemm_plane_layout(M_expected ? M_expected : 1, N, num_moduli);
+    const int layout = hip_igemm_plane_layout_single(M_expected ? M_expected : 1, K, N, num_moduli);
     const uint64_t Np = round_up_sz(N, 256), ldk = round_up_sz(K, layout ? 512 : 256);
     const bool b_kmajor = trans_b == 0;
     CrtPreparedB* pb = new CrtPreparedB();

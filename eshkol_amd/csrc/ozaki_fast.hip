@@ -512,7 +512,7 @@ extern "C" int hip_matmul_ozaki_fast_f64_ex(const double* A, const double* B, do
     if (!eshkol_crt_quiet()) fprintf(stderr, "[GPU] Ozaki-II FAST: n_mod=%d E=%d cap=%d log2(P)=%.1f (int8 MFMA GEMMs)\n",
             f.n, f.E, f.cap, f.log2P);                                  /* gpu_memory.mm:2859 */
 
-    const int layout = hip_igemm_plane_layout(M, N, f.n);
+    const int layout = hip_igemm_plane_layout_single(M, K, N, f.n);
     const uint64_t Mp = round_up_sz(M, 256), Np = round_up_sz(N, 256), ldk = round_up_sz(K, layout ? 512 : 256);
     const bool a_kmajor = trans_a != 0, b_kmajor = trans_b == 0;
     double* amax = (double*)eshkol_hip_workspace(WS_ROWSCALE, M * sizeof(double));

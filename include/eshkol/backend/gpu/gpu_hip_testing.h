@@ -112,7 +112,8 @@ void hip_igemm_set_thin_variant(int column_blocks);
 /* k-blocks kept in flight by the pipelined int8 kernel (1..3; 0 = simple kernel only). */
 void hip_igemm_set_prefetch(int pf);
 
-/* 1 (default): contractions with at least 128 tiles take interleaved operand
+/* 1 (default): contractions with at least 128 tiles (the CRT tiers: 16 tiles and
+ * 1024 of k) take interleaved operand
  * planes and the kernels that load them straight into LDS and MFMA registers
  * (256 x 128 tiles and two workgroups per CU for products of at most 1024 bytes
  * of k and for launches with fewer 256 x 256 tiles than CUs, 256 x 256 tiles and

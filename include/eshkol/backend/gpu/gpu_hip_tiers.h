@@ -157,6 +157,11 @@ int hip_igemm_i8(const HipIgemmArgs* args, void* stream);
  * most 128 (160 where N >= 4096: the kernels for a few rows), else 0. With 1 the k
  * pitch is padded to a multiple of 512. */
 int hip_igemm_plane_layout(uint64_t M, uint64_t N, int n_out);
+/* The rule of the two CRT tiers, whose contractions are one product per output plane over
+ * K of k: 1 as above, and also from sixteen tiles of 256 x 256 and K >= 1024 on (such
+ * launches take a kernel on 256 x 128 tiles that the plans of several products per plane
+ * cannot use). */
+int hip_igemm_plane_layout_single(uint64_t M, uint64_t K, uint64_t N, int n_out);
 
 /* ---- Ozaki-II CRT exact tier ------------------------------------------------
  * Residue planes of trunc(X[i,k] * 2^shift[i]) modulo the first num_moduli

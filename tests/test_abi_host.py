@@ -302,6 +302,12 @@ def test_plane_layout_decisions_are_host_arithmetic():
     assert lib.hip_igemm_plane_layout(129, 512, 16) == 0            # 32 tiles
     assert lib.hip_igemm_plane_layout(160, 4096, 2) == 1            # up to 160 rows against 4096 columns
     assert lib.hip_igemm_plane_layout(161, 4096, 2) == 0
+    # one product per output plane (the CRT tiers): also from sixteen tiles and 1024 of k on
+    assert lib.hip_igemm_plane_layout_single(512, 1024, 512, 16) == 1
+    assert lib.hip_igemm_plane_layout_single(512, 1023, 512, 16) == 0
+    assert lib.hip_igemm_plane_layout_single(256, 4096, 256, 15) == 0
+    assert lib.hip_igemm_plane_layout_single(161, 4096, 1024, 16) == 1
+    assert lib.hip_igemm_plane_layout_single(8192, 512, 8192, 16) == 1
     assert lib.hip_hgemm_plane_layout(8192, 8192, 1) == 1
     assert lib.hip_hgemm_plane_layout(1024, 1024, 1) == 0
     assert lib.hip_hgemm_plane_layout(1024, 1024, 8) == 1           # a batch fills the device

@@ -579,13 +579,14 @@ assert np.array_equal(ea.matmul_dispatch(X, W), oracle.matmul_ozaki_crt(X, W))
 
 
 def test_resident_planes_follow_the_plane_layout_and_the_byte_cap(gpu):
-    """Row-major planes (512 rows: 64 tiles) are made again, interleaved, when a product wants
+    """Row-major planes (512 rows: 64 tiles, and k too short for the kernel that would take
+    interleaved planes on so few) are made again, interleaved, when a product wants
     interleaved ones (1024 rows: 128 tiles), with a line in the verbose log, instead of staying
     in memory unused while B is split on every call; interleaved planes then serve every row
     count that follows (512 again, 700). ESHKOL_GPU_PREPARED_BYTES
     bounds what they may take (0: none). Results are the unpinned path's either way."""
     body = r"""
-K, N = 1024, 512
+K, N = 512, 512
 W = synth.xavier_uniform(5, K, N)
 assert lib.eshkol_gpu_resident_pin(W.ctypes.data, W.nbytes) == 0
 for M in (512, 1024, 1024, 512, 700):
