@@ -31,7 +31,9 @@ SHAPES = [(1, 1, 1), (5, 3, 4), (64, 128, 64), (100, 200, 90), (257, 129, 255), 
           (512, 512, 512), (33, 2049, 65), (768, 640, 1024),
           (3, 131071, 2),                      # the largest K the tier accepts
           (3001, 2, 2), (2, 2, 3001), (1, 1031, 513),
-          (8, 4096, 1024), (32, 1024, 2048), (64, 1000, 777), (65, 1000, 777)]      # a few rows against a layer
+          (8, 4096, 1024), (32, 1024, 2048), (64, 1000, 777), (65, 1000, 777),      # a few rows against a layer
+          # fewer tiles than CUs and k from 1024 on: interleaved planes on the 256 x 128 kernel
+          (200, 1024, 300), (161, 1100, 1000), (300, 2048, 257), (256, 4100, 256)]
 
 
 @pytest.mark.parametrize("M,K,N", SHAPES)

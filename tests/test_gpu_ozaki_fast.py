@@ -45,7 +45,9 @@ def check_all_stages(A, B, n_mod=11, trans=None):
 
 
 SHAPES = [(1, 1, 1), (5, 3, 4), (64, 128, 64), (100, 200, 90), (257, 129, 255), (33, 2049, 65), (512, 640, 384),
-          (3, 131071, 2), (3001, 2, 2), (2, 2, 3001), (1, 1031, 513)]
+          (3, 131071, 2), (3001, 2, 2), (2, 2, 3001), (1, 1031, 513),
+          # fewer tiles than CUs and k from 1024 on: interleaved planes on the 256 x 128 kernel (not yet at 11 tiles)
+          (200, 1024, 300), (300, 2048, 257), (256, 1024, 256)]
 
 
 @pytest.mark.parametrize("M,K,N", SHAPES)
