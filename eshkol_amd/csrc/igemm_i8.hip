@@ -766,12 +766,13 @@ extern "C" int hip_igemm_i8(const HipIgemmArgs* args, void* stream) {
         if (eshkol_hip_igemm_is_thin(a.M, a.N)) return eshkol_hip_igemm_thin(a, st);
         /* Products of at most 1024 bytes of k per row take the 256 x 128 kernel with
          * two workgroups per CU (measured 5 ... 13 % faster there, slower from 2048 on), and
-         * so do launches with fewer 256 x 256 tiles than CUs, whatever their k: twice the
-         * workgroups (64 tiles of k = 4096: 50 -> 39 us, 32 of k = 8192: 86 -> 53). Row counts
+         * so do launches with no more 256 x 256 tiles than CUs, whatever their k: twice the
+         * workgroups (64 tiles of k = 4096: 50 -> 39 us, 32 of k = 8192: 86 -> 53, 256 of
+         * k = 4096: 100 -> 92, of k = 2048: 48 -> 44). Row counts
          * of B padded to 256 cover its tiles too. g_direct 2 / 3: always / never. */
         const uint64_t tiles256 = (uint64_t)((a.M + 255) / 256) * ((a.N + 255) / 256) * a.n_out;
         const bool half = g_direct == 2 || (g_direct == 1 && a.max_pairs == 1 &&
-                                            (a.ldk <= 1024 || tiles256 < (uint64_t)eshkol_hip_num_cus()));
+                                            (a.ldk <= 1024 || tiles256 <= (uint64_t)eshkol_hip_num_cus()));
         return half ? launch_direct_half(a, st) : launch_direct(a, st);
     }
     if (a.layout != 0) return -1;

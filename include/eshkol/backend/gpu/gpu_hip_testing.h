@@ -116,7 +116,7 @@ void hip_igemm_set_prefetch(int pf);
  * 1024 of k) take interleaved operand
  * planes and the kernels that load them straight into LDS and MFMA registers
  * (256 x 128 tiles and two workgroups per CU for products of at most 1024 bytes
- * of k and for launches with fewer 256 x 256 tiles than CUs, 256 x 256 tiles and
+ * of k and for launches with no more 256 x 256 tiles than CUs, 256 x 256 tiles and
  * one otherwise); 2: the 256 x 128 kernel for all of
  * them; 3: the 256 x 256 kernel for all of them; 0: row-major planes and the
  * register-staged kernels everywhere. With 1, a first operand of a few rows
