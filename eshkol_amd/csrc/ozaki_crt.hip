@@ -518,16 +518,16 @@ __device__ __forceinline__ void scan_block(const double* x, uint64_t n_rows, int
             }
         }
     }
-    /* `out` is host memory the CPU is polling: every thread's stores (the candidates, the
-     * summary) must be out before the ticket that announces them; one fence for both */
+    /* `out` is host memory the CPU is polling: every thread's candidate stores must
+     * be out before the ticket that announces them */
+    __threadfence_system();
     __syncthreads();
     if (tid == 0) {
         o->mant_max = s_max; o->nonfinite = s_nonfinite; o->extreme = s_extreme; o->nonzero = s_nonzero;
         o->e_min = s_emin; o->e_max = s_emax; o->ncand = s_ncand;
+        __threadfence_system();
+        *(volatile uint32_t*)&o->ready = ticket;
     }
-    __threadfence_system();
-    __syncthreads();
-    if (tid == 0) *(volatile uint32_t*)&o->ready = ticket;
 }
 
 /* block 0: the M row maxima of A; block 1: the N maxima of B */
