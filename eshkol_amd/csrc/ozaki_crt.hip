@@ -558,12 +558,12 @@ void crt_rowmax_scan_kernel(const double* __restrict__ A, uint64_t M, uint64_t K
         typedef double d2_t __attribute__((ext_vector_type(2)));
         const d2_t* p2 = (const d2_t*)p;
         const uint64_t n2 = K >> 1;
-        for (uint64_t k = tid; k < n2; k += 1024) {
-            d2_t v[4];
+        for (uint64_t k = tid; k < n2; k += 2048) {
+            d2_t v[8];
 #pragma unroll
-            for (int u = 0; u < 4; u++) v[u] = (k + 256 * u < n2) ? p2[k + 256 * u] : (d2_t){0.0, 0.0};
+            for (int u = 0; u < 8; u++) v[u] = (k + 256 * u < n2) ? p2[k + 256 * u] : (d2_t){0.0, 0.0};
 #pragma unroll
-            for (int u = 0; u < 4; u++) { eshkol_absmax_step(v[u].x, &m); eshkol_absmax_step(v[u].y, &m); }
+            for (int u = 0; u < 8; u++) { eshkol_absmax_step(v[u].x, &m); eshkol_absmax_step(v[u].y, &m); }
         }
     } else {
         for (uint64_t k = tid; k < K; k += 1024) {
