@@ -215,7 +215,7 @@ int g_thin_variant = 0;      /* tuning: 1, 2: column blocks per workgroup of the
 
 }  // namespace
 
-extern "C" void hip_igemm_set_thin_variant(int v) { g_thin_variant = (v >= 1 && v <= 3) ? v : 0; }
+extern "C" void hip_igemm_set_thin_variant(int v) { EshkolHipLock lk; g_thin_variant = (v >= 1 && v <= 3) ? v : 0; }
 
 /* Whether hip_igemm_i8 sends interleaved planes of an M x N product here (not while a test
  * forces a tiled kernel). By M and N alone, so that a tier that pads its planes for these
