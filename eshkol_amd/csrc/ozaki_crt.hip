@@ -1060,7 +1060,8 @@ static int crt_matmul_impl(const double* A, const double* B, double* C,
     int32_t* const mu_out = fixed_E ? dmu : nullptr;
     int32_t* const nu_out = fixed_E ? dnu : nullptr;
     /* a few long rows in front of prepared planes: maxima, shifts and scan in one launch */
-    const bool fused_scan = use_prepared && !a_kmajor && M <= (uint64_t)FUSED_MAX_ROWS && K >= 1024 && g_fused_scan;
+    /* (up to 160 rows: beyond, the workgroups' fences and their additions to the one counter cost what the launches saved) */
+    const bool fused_scan = use_prepared && !a_kmajor && M <= 160 && K >= 1024 && g_fused_scan;
     uint32_t ticket = 0;
     if (fused_scan) {
         ticket = rowmax_scan_launch(A, M, K, amax, dmu, 52, st);

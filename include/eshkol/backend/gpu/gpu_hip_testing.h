@@ -145,7 +145,7 @@ void hip_reduced_set_thin(int on);
  * workgroup per tile. Same results; the switch exists to compare them. */
 void hip_igemm_set_persistent(int on);
 
-/* 1 (default): a few long rows (at most 256, k from 1024 on) in front of a prepared second
+/* 1 (default): a few long rows (at most 160, k from 1024 on) in front of a prepared second
  * operand get their maxima, their shifts and the scan of the maxima from one launch; 0:
  * from the three kernels every other shape uses. Same results. */
 void hip_ozaki_crt_set_fused_scan(int on);

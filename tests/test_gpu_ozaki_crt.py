@@ -237,7 +237,8 @@ def test_shift_bookkeeping_mantissas_next_to_a_power_of_two(gpu):
         both_bookkeeping_paths(A, Bx)
 
 
-@pytest.mark.parametrize("M,K,N", [(1, 1024, 512), (8, 4096, 300), (64, 1031, 1000), (200, 2048, 256), (256, 1024, 64)])
+@pytest.mark.parametrize("M,K,N", [(1, 1024, 512), (8, 4096, 300), (64, 1031, 1000), (160, 1500, 300), (161, 1500, 300), (200, 2048, 256),
+                                   (256, 1024, 64)])
 def test_few_rows_in_front_of_prepared_planes(gpu, M, K, N):
     """A few long rows against a prepared second operand: row maxima, shifts and the scan of the maxima are one
     launch there (the workgroup that finishes last scans). Results are the plain entry point's bit for bit and the
